@@ -1,0 +1,931 @@
+// fm_api.hip — the C ABI of libfinchhip.so (include/finch_hip.h): context,
+// HBM-resident weight stores, argument validation and kernel submission.
+// Host logic only; kernels live in fm_decode / fm_dense / fm_dequant / fm_gguf /
+// fm_prefill.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <string>
+#include <vector>
+
+#include "fm_common.h"
+
+// ---- launchers implemented in the kernel files ------------------------------
+struct FmDenseSpec {
+    const uint8_t *W, *S, *B;
+    float *out;
+    int out_dim;
+    int first_item;
+};
+extern "C" {
+int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs, const FmExpertGeom *g,
+                            int layer0, int layer_stride, int n_layers, const float *d_x,
+                            const int32_t *d_idx, const float *d_w, int K, float *d_act,
+                            float *d_expert_out, float *d_out, unsigned int *d_counters,
+                            int flags, int n_cu, hipStream_t st);
+int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
+                    const float *d_x, int M, int n_cu, hipStream_t st);
+int fm_launch_dequant_affine(const void *W, const void *S, const void *B, int out_dim,
+                             int in_dim, int group_size, int bits, int scale_fp16,
+                             uint8_t *codes, float *w32, uint16_t *w16, hipStream_t st);
+int fm_launch_dequant_gguf(const void *W, int out_dim, int in_dim, int ggml_type, float *w32,
+                           hipStream_t st);
+int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t *const *d_up,
+                          const uint8_t *const *d_down, const FmGgufGeom *g, int layer0,
+                          int layer_stride, int n_layers, const float *d_x,
+                          const int32_t *d_idx, const float *d_w, int K, float *d_act,
+                          float *d_expert_out, float *d_out, unsigned int *d_counters,
+                          int flags, int n_cu, hipStream_t st);
+int fm_launch_gguf_matvec(const uint8_t *d_W, int ggml_type, const float *d_x, float *d_out,
+                          int out_dim, int in_dim, int n_cu, hipStream_t st);
+int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGeom *g, const float *d_X,
+                             const int32_t *d_idx, const float *d_w, int M, int K,
+                             float *d_out, void *d_ws, size_t ws_bytes, int flags, int n_cu,
+                             hipStream_t st);
+size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K);
+}
+
+namespace {
+
+struct Tensor {
+    bool used = false, owned = false;
+    void *W = nullptr, *S = nullptr, *B = nullptr;
+    int out_dim = 0, in_dim = 0, group_size = 0, bits = 0, scale_fp16 = 0;
+};
+
+struct LayerBuf {
+    void *ptr = nullptr;
+    bool owned = false;
+};
+
+}  // namespace
+
+struct fm_ctx {
+    int device = 0;
+    int n_cu = 256;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    std::string err;
+
+    // affine expert store
+    bool aff_cfg = false;
+    FmExpertGeom geom{};
+    int n_layers = 0;
+    std::vector<LayerBuf> layers;
+    uint8_t **d_layer_ptrs = nullptr;
+
+    // GGUF expert store
+    bool gguf_cfg = false;
+    FmGgufGeom ggeom{};
+    int g_layers = 0;
+    std::vector<LayerBuf> g_gate, g_up, g_down;
+    uint8_t **d_gg_ptrs = nullptr;   // [3][g_layers]
+
+    // scratch shared by both stores, sized for `cap_groups` groups of FM_MAX_K slots
+    int cap_groups = 0, cap_hidden = 0, cap_inter = 0;
+    float *d_act = nullptr, *d_eo = nullptr;
+    unsigned int *d_counters = nullptr;
+    // staging for the host-pointer entry points
+    void *d_stage = nullptr;
+    size_t stage_bytes = 0;
+    void *d_ws = nullptr;
+    size_t ws_bytes = 0;
+
+    std::vector<Tensor> tensors;
+};
+
+namespace {
+
+int fail(fm_ctx *c, int code, const char *fmt, ...) {
+    if (c) {
+        char buf[512];
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(buf, sizeof buf, fmt, ap);
+        va_end(ap);
+        c->err = buf;
+    }
+    return code;
+}
+
+#define HIPCHK(c, call)                                                              \
+    do {                                                                             \
+        hipError_t e_ = (call);                                                      \
+        if (e_ != hipSuccess)                                                        \
+            return fail((c), FM_ERR_HIP, "%s: %s", #call, hipGetErrorString(e_));    \
+    } while (0)
+
+struct DeviceGuard {
+    int prev = -1;
+    explicit DeviceGuard(int dev) {
+        (void)hipGetDevice(&prev);
+        if (prev != dev) (void)hipSetDevice(dev);
+        else prev = -1;
+    }
+    ~DeviceGuard() {
+        if (prev >= 0) (void)hipSetDevice(prev);
+    }
+};
+
+int ensure_stage(fm_ctx *c, size_t bytes) {
+    if (c->stage_bytes >= bytes) return FM_OK;
+    if (c->d_stage) HIPCHK(c, hipFree(c->d_stage));
+    c->d_stage = nullptr;
+    c->stage_bytes = 0;
+    HIPCHK(c, hipMalloc(&c->d_stage, bytes));
+    c->stage_bytes = bytes;
+    return FM_OK;
+}
+
+int ensure_ws(fm_ctx *c, size_t bytes) {
+    if (c->ws_bytes >= bytes) return FM_OK;
+    if (c->d_ws) HIPCHK(c, hipFree(c->d_ws));
+    c->d_ws = nullptr;
+    c->ws_bytes = 0;
+    HIPCHK(c, hipMalloc(&c->d_ws, bytes));
+    c->ws_bytes = bytes;
+    return FM_OK;
+}
+
+// scratch for `groups` groups (layers of a step, or positions of a chunk)
+int ensure_scratch(fm_ctx *c, int groups, int hidden, int inter) {
+    if (groups <= c->cap_groups && hidden <= c->cap_hidden && inter <= c->cap_inter)
+        return FM_OK;
+    int g = groups > c->cap_groups ? groups : c->cap_groups;
+    int h = hidden > c->cap_hidden ? hidden : c->cap_hidden;
+    int in = inter > c->cap_inter ? inter : c->cap_inter;
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    if (c->d_act) (void)hipFree(c->d_act);
+    if (c->d_eo) (void)hipFree(c->d_eo);
+    if (c->d_counters) (void)hipFree(c->d_counters);
+    c->d_act = c->d_eo = nullptr;
+    c->d_counters = nullptr;
+    c->cap_groups = 0;
+    HIPCHK(c, hipMalloc((void **)&c->d_act, (size_t)g * FM_MAX_K * in * sizeof(float)));
+    HIPCHK(c, hipMalloc((void **)&c->d_eo, (size_t)g * FM_MAX_K * h * sizeof(float)));
+    HIPCHK(c, hipMalloc((void **)&c->d_counters, (size_t)g * sizeof(unsigned int)));
+    HIPCHK(c, hipMemsetAsync(c->d_counters, 0, (size_t)g * sizeof(unsigned int), c->stream));
+    c->cap_groups = g;
+    c->cap_hidden = h;
+    c->cap_inter = in;
+    return FM_OK;
+}
+
+void free_layers(std::vector<LayerBuf> &v) {
+    for (auto &l : v)
+        if (l.owned && l.ptr) (void)hipFree(l.ptr);
+    v.clear();
+}
+
+int set_layer(fm_ctx *c, std::vector<LayerBuf> &v, int layer, const void *src, size_t nbytes,
+              bool adopt) {
+    LayerBuf &lb = v[layer];
+    if (adopt) {
+        if (lb.owned && lb.ptr) HIPCHK(c, hipFree(lb.ptr));
+        lb.ptr = const_cast<void *>(src);
+        lb.owned = false;
+        return FM_OK;
+    }
+    if (!lb.owned || !lb.ptr) {
+        lb.ptr = nullptr;
+        lb.owned = false;
+        HIPCHK(c, hipMalloc(&lb.ptr, nbytes));
+        lb.owned = true;
+    }
+    HIPCHK(c, hipMemcpy(lb.ptr, src, nbytes, hipMemcpyHostToDevice));
+    return FM_OK;
+}
+
+bool pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+
+size_t gguf_row_bytes(int in_dim, int type) {
+    return (size_t)(in_dim / 256) * (type == FM_GGML_Q4_K ? 144u : 210u);
+}
+
+}  // namespace
+
+// ============================================================================
+// context
+// ============================================================================
+extern "C" int fm_ctx_create(int device, fm_ctx **out) {
+    if (!out) return FM_ERR_ARG;
+    *out = nullptr;
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || device < 0 || device >= ndev)
+        return FM_ERR_HIP;   // no GPU: there is no CPU fallback
+    fm_ctx *c = new (std::nothrow) fm_ctx;
+    if (!c) return FM_ERR_NOMEM;
+    c->device = device;
+    DeviceGuard dg(device);
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0)
+        c->n_cu = prop.multiProcessorCount;
+    if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreate(&c->ev0) != hipSuccess || hipEventCreate(&c->ev1) != hipSuccess) {
+        delete c;
+        return FM_ERR_HIP;
+    }
+    *out = c;
+    return FM_OK;
+}
+
+extern "C" int fm_ctx_destroy(fm_ctx *c) {
+    if (!c) return FM_ERR_ARG;
+    DeviceGuard dg(c->device);
+    (void)hipStreamSynchronize(c->stream);
+    free_layers(c->layers);
+    free_layers(c->g_gate);
+    free_layers(c->g_up);
+    free_layers(c->g_down);
+    for (auto &t : c->tensors)
+        if (t.used && t.owned) {
+            (void)hipFree(t.W);
+            (void)hipFree(t.S);
+            (void)hipFree(t.B);
+        }
+    void *ptrs[] = {c->d_layer_ptrs, c->d_gg_ptrs, c->d_act, c->d_eo, c->d_counters,
+                    c->d_stage, c->d_ws};
+    for (void *p : ptrs)
+        if (p) (void)hipFree(p);
+    (void)hipEventDestroy(c->ev0);
+    (void)hipEventDestroy(c->ev1);
+    (void)hipStreamDestroy(c->stream);
+    delete c;
+    return FM_OK;
+}
+
+extern "C" int fm_sync(fm_ctx *c) {
+    if (!c) return FM_ERR_ARG;
+    DeviceGuard dg(c->device);
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    return FM_OK;
+}
+
+extern "C" void *fm_stream(fm_ctx *c) { return c ? (void *)c->stream : nullptr; }
+
+extern "C" const char *fm_last_error(fm_ctx *c) { return c ? c->err.c_str() : "null context"; }
+
+extern "C" const char *fm_status_string(int s) {
+    switch (s) {
+        case FM_OK: return "ok";
+        case FM_ERR_ARG: return "bad argument";
+        case FM_ERR_HIP: return "HIP runtime error";
+        case FM_ERR_STATE: return "store not configured or layer not resident";
+        case FM_ERR_UNSUPPORTED: return "unsupported format or shape";
+        case FM_ERR_NOMEM: return "out of memory";
+        default: return "unknown status";
+    }
+}
+
+extern "C" int fm_timer_start(fm_ctx *c) {
+    if (!c) return FM_ERR_ARG;
+    DeviceGuard dg(c->device);
+    HIPCHK(c, hipEventRecord(c->ev0, c->stream));
+    return FM_OK;
+}
+
+extern "C" int fm_timer_stop(fm_ctx *c, float *ms) {
+    if (!c || !ms) return FM_ERR_ARG;
+    DeviceGuard dg(c->device);
+    HIPCHK(c, hipEventRecord(c->ev1, c->stream));
+    HIPCHK(c, hipEventSynchronize(c->ev1));
+    HIPCHK(c, hipEventElapsedTime(ms, c->ev0, c->ev1));
+    return FM_OK;
+}
+
+// ============================================================================
+// affine expert store
+// ============================================================================
+extern "C" int fm_experts_config(fm_ctx *c, int n_layers, int n_experts, int hidden, int inter,
+                                 int group_size, int bits, int scale_dtype) {
+    if (!c) return FM_ERR_ARG;
+    if (n_layers < 1 || n_experts < 1 || hidden < 1 || inter < 1)
+        return fail(c, FM_ERR_ARG, "experts_config: non-positive dimension");
+    if (group_size != 64) return fail(c, FM_ERR_UNSUPPORTED, "group_size %d (only 64)", group_size);
+    if (bits != 3 && bits != 4) return fail(c, FM_ERR_UNSUPPORTED, "expert bits %d (3 or 4)", bits);
+    if (scale_dtype != FM_SCALE_BF16 && scale_dtype != FM_SCALE_FP16)
+        return fail(c, FM_ERR_ARG, "scale_dtype %d", scale_dtype);
+    // a lane owns 128 columns; 4..32 lanes per gate/up row, 1..16 per down row
+    int lu = hidden / 128, ld = inter / 128;
+    if (hidden % 128 || inter % 128 || !pow2(lu) || !pow2(ld) || lu < 4 || lu > 32 || ld > 16 ||
+        inter % (4 * (64 / lu)) || hidden % (4 * (64 / ld)))
+        return fail(c, FM_ERR_UNSUPPORTED, "hidden %d / inter %d: need 128*2^j columns", hidden,
+                    inter);
+    DeviceGuard dg(c->device);
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    free_layers(c->layers);
+    if (c->d_layer_ptrs) HIPCHK(c, hipFree(c->d_layer_ptrs));
+    c->d_layer_ptrs = nullptr;
+    c->aff_cfg = false;
+
+    FmExpertGeom &g = c->geom;
+    g.hidden = hidden;
+    g.inter = inter;
+    g.group_size = group_size;
+    g.bits = bits;
+    g.scale_fp16 = scale_dtype == FM_SCALE_FP16;
+    g.n_experts = n_experts;
+    // finchmoe/repack_experts.py:76-87, 141-151: W, scales, biases of gate, up, down
+    uint64_t gu_w = (uint64_t)inter * hidden * bits / 8, gu_s = (uint64_t)inter * (hidden / 64) * 2;
+    uint64_t d_w = (uint64_t)hidden * inter * bits / 8, d_s = (uint64_t)hidden * (inter / 64) * 2;
+    uint64_t o = 0;
+    g.gate_w = (uint32_t)o; o += gu_w; g.gate_s = (uint32_t)o; o += gu_s; g.gate_b = (uint32_t)o; o += gu_s;
+    g.up_w = (uint32_t)o;   o += gu_w; g.up_s = (uint32_t)o;   o += gu_s; g.up_b = (uint32_t)o;   o += gu_s;
+    g.down_w = (uint32_t)o; o += d_w;  g.down_s = (uint32_t)o; o += d_s;  g.down_b = (uint32_t)o; o += d_s;
+    g.expert_size = o;
+    c->n_layers = n_layers;
+    c->layers.assign(n_layers, LayerBuf());
+    HIPCHK(c, hipMalloc((void **)&c->d_layer_ptrs, (size_t)n_layers * sizeof(uint8_t *)));
+    HIPCHK(c, hipMemset(c->d_layer_ptrs, 0, (size_t)n_layers * sizeof(uint8_t *)));
+    c->aff_cfg = true;
+    return FM_OK;
+}
+
+extern "C" size_t fm_experts_expert_size(fm_ctx *c) {
+    return (c && c->aff_cfg) ? (size_t)c->geom.expert_size : 0;
+}
+
+static int experts_set_layer(fm_ctx *c, int layer, const void *blob, size_t nbytes, bool adopt) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
+    if (!blob || layer < 0 || layer >= c->n_layers) return fail(c, FM_ERR_ARG, "layer %d", layer);
+    size_t want = (size_t)c->geom.n_experts * c->geom.expert_size;
+    if (nbytes != want)
+        return fail(c, FM_ERR_ARG, "layer blob is %zu bytes, expected %zu", nbytes, want);
+    if (adopt && ((uintptr_t)blob & 15)) return fail(c, FM_ERR_ARG, "device blob not 16-byte aligned");
+    DeviceGuard dg(c->device);
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    int rc = set_layer(c, c->layers, layer, blob, nbytes, adopt);
+    if (rc) return rc;
+    HIPCHK(c, hipMemcpy(c->d_layer_ptrs + layer, &c->layers[layer].ptr, sizeof(void *),
+                        hipMemcpyHostToDevice));
+    return FM_OK;
+}
+
+extern "C" int fm_experts_upload_layer(fm_ctx *c, int layer, const void *blob, size_t nbytes) {
+    return experts_set_layer(c, layer, blob, nbytes, false);
+}
+extern "C" int fm_experts_adopt_layer(fm_ctx *c, int layer, const void *blob, size_t nbytes) {
+    return experts_set_layer(c, layer, blob, nbytes, true);
+}
+
+// ============================================================================
+// routed experts, decode
+// ============================================================================
+static int check_layers(fm_ctx *c, const std::vector<LayerBuf> &v, int layer0, int n) {
+    if (layer0 < 0 || n < 1 || layer0 + n > (int)v.size())
+        return fail(c, FM_ERR_ARG, "layers %d..%d out of range", layer0, layer0 + n - 1);
+    for (int l = layer0; l < layer0 + n; l++)
+        if (!v[l].ptr) return fail(c, FM_ERR_STATE, "layer %d not resident", l);
+    return FM_OK;
+}
+
+extern "C" int fm_moe_decode_step_dev(fm_ctx *c, int layer0, int n_layers, const float *d_x,
+                                      const int32_t *d_idx, const float *d_w, int K,
+                                      float *d_out, float *d_expert_out, int flags) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
+    if (!d_x || !d_idx || !d_w || !d_out) return fail(c, FM_ERR_ARG, "null pointer");
+    if (K < 1 || K > FM_MAX_K) return fail(c, FM_ERR_ARG, "K %d outside 1..%d", K, FM_MAX_K);
+    int rc = check_layers(c, c->layers, layer0, n_layers);
+    if (rc) return rc;
+    DeviceGuard dg(c->device);
+    rc = ensure_scratch(c, n_layers, c->geom.hidden, c->geom.inter);
+    if (rc) return rc;
+    rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer0, 1, n_layers, d_x, d_idx, d_w,
+                                 K, c->d_act, d_expert_out ? d_expert_out : c->d_eo, d_out,
+                                 c->d_counters, flags, c->n_cu, c->stream);
+    if (rc) return fail(c, rc, "decode launch failed: %s", hipGetErrorString(hipGetLastError()));
+    return FM_OK;
+}
+
+extern "C" int fm_moe_decode_dev(fm_ctx *c, int layer, const float *d_x, const int32_t *d_idx,
+                                 const float *d_w, int K, float *d_out, float *d_expert_out,
+                                 int flags) {
+    return fm_moe_decode_step_dev(c, layer, 1, d_x, d_idx, d_w, K, d_out, d_expert_out, flags);
+}
+
+// host-pointer wrapper shared by the affine and GGUF stores and by decode
+// (M = 1) and prefill (M positions)
+typedef int (*moe_dev_fn)(fm_ctx *, int, const float *, const int32_t *, const float *, int, int,
+                          float *, float *, int);
+
+static int moe_host_call(fm_ctx *c, moe_dev_fn fn, int hidden, int layer, const float *x,
+                         const int32_t *idx, const float *w, int M, int K, float *out,
+                         float *expert_out, int flags) {
+    if (!x || !idx || !w || !out) return fail(c, FM_ERR_ARG, "null pointer");
+    if (M < 1) return fail(c, FM_ERR_ARG, "M %d", M);
+    if (K < 1 || K > FM_MAX_K) return fail(c, FM_ERR_ARG, "K %d outside 1..%d", K, FM_MAX_K);
+    DeviceGuard dg(c->device);
+    size_t nx = (size_t)M * hidden * 4, ni = (size_t)M * K * 4, ne = (size_t)M * K * hidden * 4;
+    size_t off_x = 0, off_i = off_x + nx, off_w = off_i + ((ni + 255) & ~(size_t)255);
+    size_t off_o = off_w + ((ni + 255) & ~(size_t)255), off_e = off_o + nx;
+    int rc = ensure_stage(c, off_e + (expert_out ? ne : 0));
+    if (rc) return rc;
+    char *st = (char *)c->d_stage;
+    HIPCHK(c, hipMemcpyAsync(st + off_x, x, nx, hipMemcpyHostToDevice, c->stream));
+    HIPCHK(c, hipMemcpyAsync(st + off_i, idx, ni, hipMemcpyHostToDevice, c->stream));
+    HIPCHK(c, hipMemcpyAsync(st + off_w, w, ni, hipMemcpyHostToDevice, c->stream));
+    if (flags & FM_ACCUMULATE)
+        HIPCHK(c, hipMemcpyAsync(st + off_o, out, nx, hipMemcpyHostToDevice, c->stream));
+    rc = fn(c, layer, (const float *)(st + off_x), (const int32_t *)(st + off_i),
+            (const float *)(st + off_w), M, K, (float *)(st + off_o),
+            expert_out ? (float *)(st + off_e) : nullptr, flags);
+    if (rc) return rc;
+    HIPCHK(c, hipMemcpyAsync(out, st + off_o, nx, hipMemcpyDeviceToHost, c->stream));
+    if (expert_out)
+        HIPCHK(c, hipMemcpyAsync(expert_out, st + off_e, ne, hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    return FM_OK;
+}
+
+static int aff_decode_fn(fm_ctx *c, int layer, const float *x, const int32_t *idx, const float *w,
+                         int, int K, float *out, float *eo, int flags) {
+    return fm_moe_decode_step_dev(c, layer, 1, x, idx, w, K, out, eo, flags);
+}
+
+extern "C" int fm_moe_decode(fm_ctx *c, int layer, const float *x, const int32_t *idx,
+                             const float *w, int K, float *out, float *expert_out, int flags) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
+    return moe_host_call(c, aff_decode_fn, c->geom.hidden, layer, x, idx, w, 1, K, out,
+                         expert_out, flags);
+}
+
+// ============================================================================
+// routed experts, chunked prefill
+// ============================================================================
+// Chunks below this many positions run the decode kernels once per position
+// (grid-batched); larger chunks are grouped by expert for the MFMA GEMM.
+#define FM_PREFILL_GEMM_MIN_M 32
+
+extern "C" int fm_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, const int32_t *d_idx,
+                                  const float *d_w, int M, int K, float *d_out, int flags) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
+    if (!d_X || !d_idx || !d_w || !d_out) return fail(c, FM_ERR_ARG, "null pointer");
+    if (M < 1) return fail(c, FM_ERR_ARG, "M %d", M);
+    if (K < 1 || K > FM_MAX_K) return fail(c, FM_ERR_ARG, "K %d outside 1..%d", K, FM_MAX_K);
+    int rc = check_layers(c, c->layers, layer, 1);
+    if (rc) return rc;
+    DeviceGuard dg(c->device);
+    if (M >= FM_PREFILL_GEMM_MIN_M && !(flags & FM_GUARD)) {
+        size_t ws = fm_prefill_affine_ws_bytes(&c->geom, M, K);
+        if (ws) {
+            rc = ensure_ws(c, ws);
+            if (rc) return rc;
+            rc = fm_launch_prefill_affine((const uint8_t *)c->layers[layer].ptr, &c->geom, d_X,
+                                          d_idx, d_w, M, K, d_out, c->d_ws, c->ws_bytes, flags,
+                                          c->n_cu, c->stream);
+            if (rc != FM_ERR_UNSUPPORTED) {
+                if (rc) return fail(c, rc, "prefill launch failed: %s",
+                                    hipGetErrorString(hipGetLastError()));
+                return FM_OK;
+            }
+        }
+    }
+    rc = ensure_scratch(c, M, c->geom.hidden, c->geom.inter);
+    if (rc) return rc;
+    rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer, 0, M, d_X, d_idx, d_w, K,
+                                 c->d_act, c->d_eo, d_out, c->d_counters, flags, c->n_cu,
+                                 c->stream);
+    if (rc) return fail(c, rc, "prefill launch failed: %s", hipGetErrorString(hipGetLastError()));
+    return FM_OK;
+}
+
+static int aff_prefill_fn(fm_ctx *c, int layer, const float *x, const int32_t *idx,
+                          const float *w, int M, int K, float *out, float *, int flags) {
+    return fm_moe_prefill_dev(c, layer, x, idx, w, M, K, out, flags);
+}
+
+extern "C" int fm_moe_prefill(fm_ctx *c, int layer, const float *X, const int32_t *idx,
+                              const float *w, int M, int K, float *out, int flags) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
+    return moe_host_call(c, aff_prefill_fn, c->geom.hidden, layer, X, idx, w, M, K, out, nullptr,
+                         flags);
+}
+
+// ============================================================================
+// dense affine tensors
+// ============================================================================
+static int tensor_add(fm_ctx *c, const void *W, const void *S, const void *B, int out_dim,
+                      int in_dim, int group_size, int bits, int scale_dtype, bool adopt,
+                      fm_tensor *out) {
+    if (!c) return FM_ERR_ARG;
+    if (!W || !S || !B || !out) return fail(c, FM_ERR_ARG, "null pointer");
+    if (out_dim < 1 || in_dim < 1) return fail(c, FM_ERR_ARG, "non-positive dimension");
+    if (group_size != 64) return fail(c, FM_ERR_UNSUPPORTED, "group_size %d (only 64)", group_size);
+    if (bits != 3 && bits != 4 && bits != 8)
+        return fail(c, FM_ERR_UNSUPPORTED, "tensor bits %d (3, 4 or 8)", bits);
+    if (scale_dtype != FM_SCALE_BF16 && scale_dtype != FM_SCALE_FP16)
+        return fail(c, FM_ERR_ARG, "scale_dtype %d", scale_dtype);
+    int lpr = in_dim / 128;
+    if (in_dim % 128 || !pow2(lpr) || lpr > 64)
+        return fail(c, FM_ERR_UNSUPPORTED, "in_dim %d: need 128*2^j, j<=6", in_dim);
+    DeviceGuard dg(c->device);
+    Tensor t;
+    t.used = true;
+    t.out_dim = out_dim;
+    t.in_dim = in_dim;
+    t.group_size = group_size;
+    t.bits = bits;
+    t.scale_fp16 = scale_dtype == FM_SCALE_FP16;
+    size_t wb = (size_t)out_dim * in_dim * bits / 8, sb = (size_t)out_dim * (in_dim / 64) * 2;
+    if (adopt) {
+        if (((uintptr_t)W & 15) || ((uintptr_t)S & 3) || ((uintptr_t)B & 3))
+            return fail(c, FM_ERR_ARG, "device tensor not aligned (W 16, S/B 4 bytes)");
+        t.W = const_cast<void *>(W);
+        t.S = const_cast<void *>(S);
+        t.B = const_cast<void *>(B);
+    } else {
+        t.owned = true;
+        HIPCHK(c, hipMalloc(&t.W, wb));
+        HIPCHK(c, hipMalloc(&t.S, sb));
+        HIPCHK(c, hipMalloc(&t.B, sb));
+        HIPCHK(c, hipMemcpy(t.W, W, wb, hipMemcpyHostToDevice));
+        HIPCHK(c, hipMemcpy(t.S, S, sb, hipMemcpyHostToDevice));
+        HIPCHK(c, hipMemcpy(t.B, B, sb, hipMemcpyHostToDevice));
+    }
+    for (size_t i = 0; i < c->tensors.size(); i++)
+        if (!c->tensors[i].used) {
+            c->tensors[i] = t;
+            *out = (fm_tensor)i;
+            return FM_OK;
+        }
+    c->tensors.push_back(t);
+    *out = (fm_tensor)(c->tensors.size() - 1);
+    return FM_OK;
+}
+
+extern "C" int fm_tensor_register(fm_ctx *c, const void *W, const void *S, const void *B,
+                                  int out_dim, int in_dim, int group_size, int bits,
+                                  int scale_dtype, fm_tensor *out) {
+    return tensor_add(c, W, S, B, out_dim, in_dim, group_size, bits, scale_dtype, false, out);
+}
+extern "C" int fm_tensor_adopt(fm_ctx *c, const void *W, const void *S, const void *B,
+                               int out_dim, int in_dim, int group_size, int bits,
+                               int scale_dtype, fm_tensor *out) {
+    return tensor_add(c, W, S, B, out_dim, in_dim, group_size, bits, scale_dtype, true, out);
+}
+
+static Tensor *get_tensor(fm_ctx *c, fm_tensor t) {
+    if (t < 0 || (size_t)t >= c->tensors.size() || !c->tensors[t].used) return nullptr;
+    return &c->tensors[t];
+}
+
+extern "C" int fm_tensor_release(fm_ctx *c, fm_tensor t) {
+    if (!c) return FM_ERR_ARG;
+    Tensor *p = get_tensor(c, t);
+    if (!p) return fail(c, FM_ERR_ARG, "bad tensor handle %d", t);
+    DeviceGuard dg(c->device);
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    if (p->owned) {
+        (void)hipFree(p->W);
+        (void)hipFree(p->S);
+        (void)hipFree(p->B);
+    }
+    *p = Tensor();
+    return FM_OK;
+}
+
+static int matvec_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
+                      float *const *d_outs, int M) {
+    if (!ts || !d_x || !d_outs) return fail(c, FM_ERR_ARG, "null pointer");
+    if (n < 1) return fail(c, FM_ERR_ARG, "n %d", n);
+    DeviceGuard dg(c->device);
+    // batches of up to 8 tensors with equal in_dim / bits / scale type
+    int i = 0;
+    while (i < n) {
+        Tensor *t0 = get_tensor(c, ts[i]);
+        if (!t0) return fail(c, FM_ERR_ARG, "bad tensor handle %d", ts[i]);
+        FmDenseSpec specs[8];
+        int m = 0;
+        while (i < n && m < 8) {
+            Tensor *t = get_tensor(c, ts[i]);
+            if (!t) return fail(c, FM_ERR_ARG, "bad tensor handle %d", ts[i]);
+            if (t->in_dim != t0->in_dim)
+                return fail(c, FM_ERR_ARG, "tensors of one batch must share in_dim (%d vs %d)",
+                            t->in_dim, t0->in_dim);
+            if (t->bits != t0->bits || t->scale_fp16 != t0->scale_fp16) break;
+            if (!d_outs[i]) return fail(c, FM_ERR_ARG, "null output %d", i);
+            specs[m].W = (const uint8_t *)t->W;
+            specs[m].S = (const uint8_t *)t->S;
+            specs[m].B = (const uint8_t *)t->B;
+            specs[m].out = d_outs[i];
+            specs[m].out_dim = t->out_dim;
+            specs[m].first_item = 0;
+            m++;
+            i++;
+        }
+        int rc = fm_launch_dense(specs, m, t0->in_dim, t0->bits, t0->scale_fp16, d_x, M, c->n_cu,
+                                 c->stream);
+        if (rc) return fail(c, rc, "matvec launch failed: %s", hipGetErrorString(hipGetLastError()));
+    }
+    return FM_OK;
+}
+
+extern "C" int fm_matvec_batch_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
+                                   float *const *d_outs) {
+    if (!c) return FM_ERR_ARG;
+    return matvec_dev(c, ts, n, d_x, d_outs, 1);
+}
+
+extern "C" int fm_matvec_prefill_dev(fm_ctx *c, fm_tensor t, const float *d_X, float *d_out,
+                                     int M) {
+    if (!c) return FM_ERR_ARG;
+    if (M < 1 || M > 65535) return fail(c, FM_ERR_ARG, "M %d outside 1..65535", M);
+    float *outs[1] = {d_out};
+    return matvec_dev(c, &t, 1, d_X, outs, M);
+}
+
+static int matvec_host(fm_ctx *c, const fm_tensor *ts, int n, const float *x, float *const *outs,
+                       int M) {
+    if (!ts || !x || !outs) return fail(c, FM_ERR_ARG, "null pointer");
+    if (n < 1 || n > 64) return fail(c, FM_ERR_ARG, "n %d outside 1..64", n);
+    Tensor *t0 = get_tensor(c, ts[0]);
+    if (!t0) return fail(c, FM_ERR_ARG, "bad tensor handle %d", ts[0]);
+    DeviceGuard dg(c->device);
+    size_t nx = (size_t)M * t0->in_dim * 4, total = nx;
+    std::vector<size_t> offs(n);
+    for (int i = 0; i < n; i++) {
+        Tensor *t = get_tensor(c, ts[i]);
+        if (!t) return fail(c, FM_ERR_ARG, "bad tensor handle %d", ts[i]);
+        if (!outs[i]) return fail(c, FM_ERR_ARG, "null output %d", i);
+        offs[i] = total;
+        total += ((size_t)M * t->out_dim * 4 + 255) & ~(size_t)255;
+    }
+    int rc = ensure_stage(c, total);
+    if (rc) return rc;
+    char *st = (char *)c->d_stage;
+    HIPCHK(c, hipMemcpyAsync(st, x, nx, hipMemcpyHostToDevice, c->stream));
+    std::vector<float *> d_outs(n);
+    for (int i = 0; i < n; i++) d_outs[i] = (float *)(st + offs[i]);
+    rc = matvec_dev(c, ts, n, (const float *)st, d_outs.data(), M);
+    if (rc) return rc;
+    for (int i = 0; i < n; i++)
+        HIPCHK(c, hipMemcpyAsync(outs[i], d_outs[i], (size_t)M * get_tensor(c, ts[i])->out_dim * 4,
+                                 hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    return FM_OK;
+}
+
+extern "C" int fm_matvec_batch(fm_ctx *c, const fm_tensor *ts, int n, const float *x,
+                               float *const *outs) {
+    if (!c) return FM_ERR_ARG;
+    return matvec_host(c, ts, n, x, outs, 1);
+}
+
+extern "C" int fm_matvec_prefill(fm_ctx *c, fm_tensor t, const float *X, float *out, int M) {
+    if (!c) return FM_ERR_ARG;
+    if (M < 1 || M > 65535) return fail(c, FM_ERR_ARG, "M %d outside 1..65535", M);
+    float *outs[1] = {out};
+    return matvec_host(c, &t, 1, X, outs, M);
+}
+
+// ============================================================================
+// GGUF expert store
+// ============================================================================
+extern "C" int fm_gguf_config(fm_ctx *c, int n_layers, int n_experts, int hidden, int inter,
+                              int gate_type, int up_type, int down_type) {
+    if (!c) return FM_ERR_ARG;
+    if (n_layers < 1 || n_experts < 1) return fail(c, FM_ERR_ARG, "non-positive dimension");
+    // finchmoe/infer.m:3166: the fused gate+up kernel is Q4_K only
+    if (gate_type != FM_GGML_Q4_K || up_type != FM_GGML_Q4_K)
+        return fail(c, FM_ERR_UNSUPPORTED, "gate/up must be Q4_K (12), got %d/%d", gate_type, up_type);
+    if (down_type != FM_GGML_Q4_K && down_type != FM_GGML_Q6_K)
+        return fail(c, FM_ERR_UNSUPPORTED, "down must be Q4_K (12) or Q6_K (14), got %d", down_type);
+    if (hidden % 256 || inter % 256 || hidden < 256 || inter < 256 || hidden > 16384 || inter > 16384)
+        return fail(c, FM_ERR_UNSUPPORTED, "hidden %d / inter %d: need multiples of 256", hidden, inter);
+    DeviceGuard dg(c->device);
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    free_layers(c->g_gate);
+    free_layers(c->g_up);
+    free_layers(c->g_down);
+    if (c->d_gg_ptrs) HIPCHK(c, hipFree(c->d_gg_ptrs));
+    c->d_gg_ptrs = nullptr;
+    c->gguf_cfg = false;
+    FmGgufGeom &g = c->ggeom;
+    g.hidden = hidden;
+    g.inter = inter;
+    g.n_experts = n_experts;
+    g.gate_type = gate_type;
+    g.up_type = up_type;
+    g.down_type = down_type;
+    g.gu_row_bytes = (uint32_t)gguf_row_bytes(hidden, gate_type);
+    g.down_row_bytes = (uint32_t)gguf_row_bytes(inter, down_type);
+    // finchmoe/infer.m:1141-1146: slab = out rows x row bytes
+    g.gate_slab = (uint64_t)inter * g.gu_row_bytes;
+    g.up_slab = g.gate_slab;
+    g.down_slab = (uint64_t)hidden * g.down_row_bytes;
+    c->g_layers = n_layers;
+    c->g_gate.assign(n_layers, LayerBuf());
+    c->g_up.assign(n_layers, LayerBuf());
+    c->g_down.assign(n_layers, LayerBuf());
+    HIPCHK(c, hipMalloc((void **)&c->d_gg_ptrs, (size_t)3 * n_layers * sizeof(uint8_t *)));
+    HIPCHK(c, hipMemset(c->d_gg_ptrs, 0, (size_t)3 * n_layers * sizeof(uint8_t *)));
+    c->gguf_cfg = true;
+    return FM_OK;
+}
+
+static int gguf_set_layer(fm_ctx *c, int layer, const void *gate, const void *up,
+                          const void *down, bool adopt) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->gguf_cfg) return fail(c, FM_ERR_STATE, "GGUF store not configured");
+    if (!gate || !up || !down || layer < 0 || layer >= c->g_layers)
+        return fail(c, FM_ERR_ARG, "layer %d", layer);
+    if (adopt && (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)down) & 15))
+        return fail(c, FM_ERR_ARG, "device slab not 16-byte aligned");
+    DeviceGuard dg(c->device);
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    const FmGgufGeom &g = c->ggeom;
+    int rc = set_layer(c, c->g_gate, layer, gate, (size_t)g.n_experts * g.gate_slab, adopt);
+    if (!rc) rc = set_layer(c, c->g_up, layer, up, (size_t)g.n_experts * g.up_slab, adopt);
+    if (!rc) rc = set_layer(c, c->g_down, layer, down, (size_t)g.n_experts * g.down_slab, adopt);
+    if (rc) return rc;
+    void *p[3] = {c->g_gate[layer].ptr, c->g_up[layer].ptr, c->g_down[layer].ptr};
+    for (int i = 0; i < 3; i++)
+        HIPCHK(c, hipMemcpy(c->d_gg_ptrs + (size_t)i * c->g_layers + layer, &p[i], sizeof(void *),
+                            hipMemcpyHostToDevice));
+    return FM_OK;
+}
+
+extern "C" int fm_gguf_upload_layer(fm_ctx *c, int layer, const void *gate, const void *up,
+                                    const void *down) {
+    return gguf_set_layer(c, layer, gate, up, down, false);
+}
+extern "C" int fm_gguf_adopt_layer(fm_ctx *c, int layer, const void *gate, const void *up,
+                                   const void *down) {
+    return gguf_set_layer(c, layer, gate, up, down, true);
+}
+
+static int gguf_decode_groups(fm_ctx *c, int layer0, int layer_stride, int groups,
+                              const float *d_x, const int32_t *d_idx, const float *d_w, int K,
+                              float *d_out, float *d_expert_out, int flags) {
+    if (!c->gguf_cfg) return fail(c, FM_ERR_STATE, "GGUF store not configured");
+    if (!d_x || !d_idx || !d_w || !d_out) return fail(c, FM_ERR_ARG, "null pointer");
+    if (K < 1 || K > FM_MAX_K) return fail(c, FM_ERR_ARG, "K %d outside 1..%d", K, FM_MAX_K);
+    int rc = check_layers(c, c->g_gate, layer0, layer_stride ? groups : 1);
+    if (rc) return rc;
+    DeviceGuard dg(c->device);
+    rc = ensure_scratch(c, groups, c->ggeom.hidden, c->ggeom.inter);
+    if (rc) return rc;
+    rc = fm_launch_decode_gguf(c->d_gg_ptrs, c->d_gg_ptrs + c->g_layers,
+                               c->d_gg_ptrs + 2 * (size_t)c->g_layers, &c->ggeom, layer0,
+                               layer_stride, groups, d_x, d_idx, d_w, K, c->d_act,
+                               d_expert_out ? d_expert_out : c->d_eo, d_out, c->d_counters, flags,
+                               c->n_cu, c->stream);
+    if (rc) return fail(c, rc, "GGUF decode launch failed: %s", hipGetErrorString(hipGetLastError()));
+    return FM_OK;
+}
+
+extern "C" int fm_gguf_moe_decode_step_dev(fm_ctx *c, int layer0, int n_layers, const float *d_x,
+                                           const int32_t *d_idx, const float *d_w, int K,
+                                           float *d_out, float *d_expert_out, int flags) {
+    if (!c) return FM_ERR_ARG;
+    if (n_layers < 1) return fail(c, FM_ERR_ARG, "n_layers %d", n_layers);
+    return gguf_decode_groups(c, layer0, 1, n_layers, d_x, d_idx, d_w, K, d_out, d_expert_out, flags);
+}
+
+extern "C" int fm_gguf_moe_decode_dev(fm_ctx *c, int layer, const float *d_x, const int32_t *d_idx,
+                                      const float *d_w, int K, float *d_out, float *d_expert_out,
+                                      int flags) {
+    if (!c) return FM_ERR_ARG;
+    return gguf_decode_groups(c, layer, 1, 1, d_x, d_idx, d_w, K, d_out, d_expert_out, flags);
+}
+
+extern "C" int fm_gguf_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, const int32_t *d_idx,
+                                       const float *d_w, int M, int K, float *d_out, int flags) {
+    if (!c) return FM_ERR_ARG;
+    if (M < 1) return fail(c, FM_ERR_ARG, "M %d", M);
+    return gguf_decode_groups(c, layer, 0, M, d_X, d_idx, d_w, K, d_out, nullptr, flags);
+}
+
+static int gguf_decode_fn(fm_ctx *c, int layer, const float *x, const int32_t *idx, const float *w,
+                          int, int K, float *out, float *eo, int flags) {
+    return gguf_decode_groups(c, layer, 1, 1, x, idx, w, K, out, eo, flags);
+}
+static int gguf_prefill_fn(fm_ctx *c, int layer, const float *x, const int32_t *idx,
+                           const float *w, int M, int K, float *out, float *, int flags) {
+    return gguf_decode_groups(c, layer, 0, M, x, idx, w, K, out, nullptr, flags);
+}
+
+extern "C" int fm_gguf_moe_decode(fm_ctx *c, int layer, const float *x, const int32_t *idx,
+                                  const float *w, int K, float *out, float *expert_out, int flags) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->gguf_cfg) return fail(c, FM_ERR_STATE, "GGUF store not configured");
+    return moe_host_call(c, gguf_decode_fn, c->ggeom.hidden, layer, x, idx, w, 1, K, out,
+                         expert_out, flags);
+}
+
+extern "C" int fm_gguf_moe_prefill(fm_ctx *c, int layer, const float *X, const int32_t *idx,
+                                   const float *w, int M, int K, float *out, int flags) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->gguf_cfg) return fail(c, FM_ERR_STATE, "GGUF store not configured");
+    return moe_host_call(c, gguf_prefill_fn, c->ggeom.hidden, layer, X, idx, w, M, K, out, nullptr,
+                         flags);
+}
+
+extern "C" int fm_gguf_matvec(fm_ctx *c, const void *W, int ggml_type, const float *x, float *out,
+                              int out_dim, int in_dim) {
+    if (!c) return FM_ERR_ARG;
+    if (!W || !x || !out) return fail(c, FM_ERR_ARG, "null pointer");
+    if (ggml_type != FM_GGML_Q4_K && ggml_type != FM_GGML_Q6_K)
+        return fail(c, FM_ERR_UNSUPPORTED, "ggml type %d", ggml_type);
+    if (out_dim < 1 || in_dim < 256 || in_dim % 256 || in_dim > 16384)
+        return fail(c, FM_ERR_UNSUPPORTED, "in_dim %d: need a multiple of 256 up to 16384", in_dim);
+    DeviceGuard dg(c->device);
+    size_t wb = (size_t)out_dim * gguf_row_bytes(in_dim, ggml_type);
+    size_t off_x = (wb + 255) & ~(size_t)255, off_o = off_x + (((size_t)in_dim * 4 + 255) & ~(size_t)255);
+    int rc = ensure_stage(c, off_o + (size_t)out_dim * 4);
+    if (rc) return rc;
+    char *st = (char *)c->d_stage;
+    HIPCHK(c, hipMemcpyAsync(st, W, wb, hipMemcpyHostToDevice, c->stream));
+    HIPCHK(c, hipMemcpyAsync(st + off_x, x, (size_t)in_dim * 4, hipMemcpyHostToDevice, c->stream));
+    rc = fm_launch_gguf_matvec((const uint8_t *)st, ggml_type, (const float *)(st + off_x),
+                               (float *)(st + off_o), out_dim, in_dim, c->n_cu, c->stream);
+    if (rc) return fail(c, rc, "GGUF matvec launch failed");
+    HIPCHK(c, hipMemcpyAsync(out, st + off_o, (size_t)out_dim * 4, hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    return FM_OK;
+}
+
+// ============================================================================
+// dequant (bit-exact checks)
+// ============================================================================
+static int dequant_common(fm_ctx *c, const void *dW, const void *dS, const void *dB, int rows,
+                          int cols, int bits, int scale_fp16, int ggml_type, uint8_t *codes,
+                          float *w_f32, uint16_t *w_f16) {
+    size_t n = (size_t)rows * cols;
+    size_t off32 = (n + 255) & ~(size_t)255, off16 = off32 + n * 4;
+    int rc = ensure_stage(c, off16 + n * 2);
+    if (rc) return rc;
+    char *st = (char *)c->d_stage;
+    if (ggml_type) {
+        rc = fm_launch_dequant_gguf(dW, rows, cols, ggml_type, (float *)(st + off32), c->stream);
+    } else {
+        rc = fm_launch_dequant_affine(dW, dS, dB, rows, cols, 64, bits, scale_fp16,
+                                      (uint8_t *)st, (float *)(st + off32),
+                                      (uint16_t *)(st + off16), c->stream);
+    }
+    if (rc) return fail(c, rc, "dequant launch failed");
+    if (codes) HIPCHK(c, hipMemcpyAsync(codes, st, n, hipMemcpyDeviceToHost, c->stream));
+    if (w_f32) HIPCHK(c, hipMemcpyAsync(w_f32, st + off32, n * 4, hipMemcpyDeviceToHost, c->stream));
+    if (w_f16) HIPCHK(c, hipMemcpyAsync(w_f16, st + off16, n * 2, hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    return FM_OK;
+}
+
+extern "C" int fm_dequant_expert(fm_ctx *c, int layer, int expert, int which, uint8_t *codes,
+                                 float *w_f32, uint16_t *w_f16) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
+    int rc = check_layers(c, c->layers, layer, 1);
+    if (rc) return rc;
+    const FmExpertGeom &g = c->geom;
+    if (expert < 0 || expert >= g.n_experts) return fail(c, FM_ERR_ARG, "expert %d", expert);
+    if (which < FM_MAT_GATE || which > FM_MAT_DOWN) return fail(c, FM_ERR_ARG, "which %d", which);
+    DeviceGuard dg(c->device);
+    const uint8_t *e = (const uint8_t *)c->layers[layer].ptr + (size_t)expert * g.expert_size;
+    uint32_t wo[3] = {g.gate_w, g.up_w, g.down_w}, so[3] = {g.gate_s, g.up_s, g.down_s},
+             bo[3] = {g.gate_b, g.up_b, g.down_b};
+    int rows = which == FM_MAT_DOWN ? g.hidden : g.inter, cols = which == FM_MAT_DOWN ? g.inter : g.hidden;
+    return dequant_common(c, e + wo[which], e + so[which], e + bo[which], rows, cols, g.bits,
+                          g.scale_fp16, 0, codes, w_f32, w_f16);
+}
+
+extern "C" int fm_dequant_tensor(fm_ctx *c, fm_tensor t, uint8_t *codes, float *w_f32,
+                                 uint16_t *w_f16) {
+    if (!c) return FM_ERR_ARG;
+    Tensor *p = get_tensor(c, t);
+    if (!p) return fail(c, FM_ERR_ARG, "bad tensor handle %d", t);
+    DeviceGuard dg(c->device);
+    return dequant_common(c, p->W, p->S, p->B, p->out_dim, p->in_dim, p->bits, p->scale_fp16, 0,
+                          codes, w_f32, w_f16);
+}
+
+extern "C" int fm_gguf_dequant_expert(fm_ctx *c, int layer, int expert, int which, float *w_f32) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->gguf_cfg) return fail(c, FM_ERR_STATE, "GGUF store not configured");
+    if (!w_f32) return fail(c, FM_ERR_ARG, "null pointer");
+    int rc = check_layers(c, c->g_gate, layer, 1);
+    if (rc) return rc;
+    const FmGgufGeom &g = c->ggeom;
+    if (expert < 0 || expert >= g.n_experts) return fail(c, FM_ERR_ARG, "expert %d", expert);
+    if (which < FM_MAT_GATE || which > FM_MAT_DOWN) return fail(c, FM_ERR_ARG, "which %d", which);
+    DeviceGuard dg(c->device);
+    const uint8_t *base;
+    int rows, cols, type;
+    if (which == FM_MAT_GATE) {
+        base = (const uint8_t *)c->g_gate[layer].ptr + (size_t)expert * g.gate_slab;
+        rows = g.inter; cols = g.hidden; type = g.gate_type;
+    } else if (which == FM_MAT_UP) {
+        base = (const uint8_t *)c->g_up[layer].ptr + (size_t)expert * g.up_slab;
+        rows = g.inter; cols = g.hidden; type = g.up_type;
+    } else {
+        base = (const uint8_t *)c->g_down[layer].ptr + (size_t)expert * g.down_slab;
+        rows = g.hidden; cols = g.inter; type = g.down_type;
+    }
+    return dequant_common(c, base, nullptr, nullptr, rows, cols, 0, 0, type, nullptr, w_f32, nullptr);
+}

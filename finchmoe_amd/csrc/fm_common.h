@@ -1,0 +1,75 @@
+// fm_common.h — shared declarations of libfinchhip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "../../include/finch_hip.h"
+
+#define FM_MAX_K 8
+#define FM_WAVE 64
+
+// Geometry of one affine expert blob, passed to kernels by value.
+// Layout: finchmoe/repack_experts.py:76-163, finchmoe/infer.m:174-234.
+struct FmExpertGeom {
+    int hidden, inter, group_size, bits, scale_fp16, n_experts;
+    uint32_t gate_w, gate_s, gate_b, up_w, up_s, up_b, down_w, down_s, down_b;
+    uint64_t expert_size;
+};
+
+// Geometry of the GGUF slabs of one layer (finchmoe/infer.m:1017-1022).
+struct FmGgufGeom {
+    int hidden, inter, n_experts;
+    int gate_type, up_type, down_type;
+    uint64_t gate_slab, up_slab, down_slab;   // bytes per expert
+    uint32_t gu_row_bytes, down_row_bytes;
+};
+
+// ---------------------------------------------------------------- device helpers
+#if defined(__HIPCC__)
+
+// 16-bit scale / bias widening.  BF16: finchmoe/infer.m:690-695.
+// FP16: IEEE half -> float (finchmoe/infer.m:1579-1593 computes the same value).
+__device__ __forceinline__ float fm_bf16_lo(uint32_t pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float fm_bf16_hi(uint32_t pair) { return __uint_as_float(pair & 0xFFFF0000u); }
+__device__ __forceinline__ float fm_fp16_bits(uint32_t h) {
+    _Float16 v = __builtin_bit_cast(_Float16, (unsigned short)h);
+    return (float)v;
+}
+template <bool FP16>
+__device__ __forceinline__ float fm_widen_lo(uint32_t pair) {
+    if constexpr (FP16) return fm_fp16_bits(pair & 0xFFFFu);
+    else return fm_bf16_lo(pair);
+}
+template <bool FP16>
+__device__ __forceinline__ float fm_widen_hi(uint32_t pair) {
+    if constexpr (FP16) return fm_fp16_bits(pair >> 16);
+    else return fm_bf16_hi(pair);
+}
+
+// Sum over aligned groups of N lanes (N a power of two <= 64); every lane of
+// the group receives the sum.  N <= 16 stays inside a DPP row.
+template <int CTRL>
+__device__ __forceinline__ float fm_dpp(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+template <int N>
+__device__ __forceinline__ float fm_group_sum(float v) {
+    if constexpr (N >= 2) v += fm_dpp<0xB1>(v);    // quad_perm [1,0,3,2]
+    if constexpr (N >= 4) v += fm_dpp<0x4E>(v);    // quad_perm [2,3,0,1]
+    // once every lane of a quad holds the quad's sum, mirroring within 8 (then
+    // 16) lanes fetches the neighbouring quad's (half row's) sum
+    if constexpr (N >= 8) v += fm_dpp<0x141>(v);   // row_half_mirror
+    if constexpr (N >= 16) v += fm_dpp<0x140>(v);  // row_mirror
+    if constexpr (N >= 32) v += __shfl_xor(v, 16);
+    if constexpr (N >= 64) v += __shfl_xor(v, 32);
+    return v;
+}
+
+__device__ __forceinline__ float fm_silu_mul(float g, float u) {
+    return (g / (1.0f + expf(-g))) * u;   // finchmoe/infer.m:1780-1786
+}
+
+#endif  // __HIPCC__

@@ -1,0 +1,290 @@
+// fm_decode.hip — routed-expert decode for affine-packed experts:
+//   kernel 1  gate GEMV + up GEMV + SwiGLU for every (layer, slot) pair
+//   kernel 2  down GEMV per pair, then the router-weighted sum in slot order
+// Replaces the four dispatches per expert of gpu_encode_experts_batched
+// (finchmoe/infer.m:4337-4378: dequant_matvec_3bit x3 + swiglu_fused) and the
+// weighted sum of moe_combine_residual (finchmoe/shaders.metal:2213-2228).
+//
+// Work decomposition.  A pair p = (layer l, slot k) selects expert idx[l][k].
+// A 256-thread workgroup (4 waves) takes `rows_per_item` consecutive output
+// rows of one pair.  Inside a wave, LPR = in_dim/128 adjacent lanes share a
+// row (each owns 128 columns, see fm_unpack.h), so one wave step covers
+// 64/LPR rows, read as one contiguous run of memory:
+//   gate/up (in 2048): 16 lanes x 48 B = one 768-byte row, 4 rows per step
+//   down    (in 512):   4 lanes x 48 B = one 192-byte row, 16 rows per step
+// The scales (and biases) of those rows are contiguous too — [rows][groups]
+// 16-bit, two groups per lane = one dword per lane.
+#include "fm_unpack.h"
+
+namespace {
+
+struct DecodeArgs {
+    const uint8_t *const *layer_ptrs;   // [n_layers] device pointers to layer blobs
+    FmExpertGeom g;
+    int layer0;
+    int layer_stride;   // 1: pair group l is layer layer0+l; 0: all groups use layer0 (positions of a chunk)
+    int K;
+    const float *x;          // [nl][hidden]
+    const int32_t *idx;      // [nl][K]
+    const float *w;          // [nl][K]
+    float *act;              // [nl][K][inter]   scratch
+    float *expert_out;       // [nl][K][hidden]
+    float *out;              // [nl][hidden]
+    unsigned int *counters;  // [nl] arrival counters, zero between launches
+    int rows_per_item;
+    int items_per_pair;
+    int flags;
+};
+
+// ---------------------------------------------------------------- kernel 1
+template <int BITS, int LPR, bool FP16>
+__global__ __launch_bounds__(256) void fm_gate_up_swiglu(DecodeArgs a) {
+    constexpr int RPS = FM_WAVE / LPR;   // rows per wave step
+    constexpr int BPL = FmLaneBytes<BITS>::value;
+    const int item = blockIdx.x;
+    const int pair = item / a.items_per_pair;
+    const int chunk = item - pair * a.items_per_pair;
+    const int l = pair / a.K;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int c = lane % LPR, r = lane / LPR;
+    const int rows_per_wave = a.rows_per_item >> 2;
+    const int row0 = chunk * a.rows_per_item + wave * rows_per_wave;
+    float *act = a.act + (size_t)pair * a.g.inter;
+
+    const int e = a.idx[pair];
+    if ((unsigned)e >= (unsigned)a.g.n_experts) {   // treated as weight 0
+        for (int i = lane; i < rows_per_wave; i += FM_WAVE) act[row0 + i] = 0.0f;
+        return;
+    }
+    const uint8_t *blob = a.layer_ptrs[a.layer0 + l * a.layer_stride] + (size_t)e * a.g.expert_size;
+    const int row_bytes = a.g.hidden * BITS / 8;
+    const int sb_row_bytes = (a.g.hidden / 64) * 2;
+
+    // issue the first weight loads before the activation loads
+    size_t woff = (size_t)(row0 + r) * row_bytes + (size_t)c * BPL;
+    size_t soff = (size_t)(row0 + r) * sb_row_bytes + (size_t)c * 4;
+    const size_t wstep = (size_t)RPS * row_bytes, sstep = (size_t)RPS * sb_row_bytes;
+    FmRowSlice<BITS> gcur, ucur, gnext, unext;
+    fm_load_slice<BITS>(gcur, blob + a.g.gate_w + woff, blob + a.g.gate_s + soff,
+                        blob + a.g.gate_b + soff);
+    fm_load_slice<BITS>(ucur, blob + a.g.up_w + woff, blob + a.g.up_s + soff,
+                        blob + a.g.up_b + soff);
+
+    float xs[FM_CPL], xsum0, xsum1;
+    fm_load_x<BITS>(a.x + (size_t)l * a.g.hidden + c * FM_CPL, xs, xsum0, xsum1);
+
+    const int steps = rows_per_wave / RPS;
+    for (int it = 0; it < steps; it++) {
+        if (it + 1 < steps) {
+            woff += wstep;
+            soff += sstep;
+            fm_load_slice<BITS>(gnext, blob + a.g.gate_w + woff, blob + a.g.gate_s + soff,
+                                blob + a.g.gate_b + soff);
+            fm_load_slice<BITS>(unext, blob + a.g.up_w + woff, blob + a.g.up_s + soff,
+                                blob + a.g.up_b + soff);
+        }
+        float gv = fm_group_sum<LPR>(fm_lane_dot<BITS, FP16>(gcur, xs, xsum0, xsum1));
+        float uv = fm_group_sum<LPR>(fm_lane_dot<BITS, FP16>(ucur, xs, xsum0, xsum1));
+        if (c == 0) act[row0 + it * RPS + r] = fm_silu_mul(gv, uv);
+        gcur = gnext;
+        ucur = unext;
+    }
+}
+
+// ---------------------------------------------------------------- kernel 2
+// The last workgroup of a layer to finish its down rows (arrival counter) sums
+// the K per-expert vectors in slot order, so the result does not depend on
+// which workgroup that is.
+template <bool GUARD>
+__device__ void fm_combine_layer(const DecodeArgs &a, int l, float *red) {
+    const int H = a.g.hidden, K = a.K;
+    const float *eo = a.expert_out + (size_t)l * K * H;
+    float wk[FM_MAX_K];
+    float total = 0.0f;
+    for (int k = 0; k < K; k++) {
+        float w = a.w[l * K + k];
+        if ((unsigned)a.idx[l * K + k] >= (unsigned)a.g.n_experts) w = 0.0f;
+        if constexpr (GUARD) {
+            // finchmoe/infer.m:10190-10196: keep the expert iff sum(out^2) is
+            // finite and < 1e20
+            float part = 0.0f;
+            for (int j = threadIdx.x; j < H; j += blockDim.x) {
+                float v = eo[(size_t)k * H + j];
+                part = fmaf(v, v, part);
+            }
+            part = fm_group_sum<64>(part);
+            __syncthreads();
+            if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
+            __syncthreads();
+            float er = red[0] + red[1] + red[2] + red[3];
+            bool keep = isfinite(er) && er < 1e20f;
+            if (keep) total += w; else w = 0.0f;
+        }
+        wk[k] = w;
+    }
+    float rn = 1.0f;
+    if constexpr (GUARD) {
+        if (total > 0.0f && total < 0.99f) rn = 1.0f / total;   // infer.m:10200-10204
+    }
+    float *out = a.out + (size_t)l * H;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) {
+        float acc = 0.0f;
+        for (int k = 0; k < K; k++)
+            if (wk[k] != 0.0f) acc += wk[k] * eo[(size_t)k * H + j];
+        if constexpr (GUARD) acc *= rn;
+        out[j] = (a.flags & FM_ACCUMULATE) ? out[j] + acc : acc;
+    }
+}
+
+template <int BITS, int LPR, bool FP16>
+__global__ __launch_bounds__(256) void fm_down_combine(DecodeArgs a) {
+    constexpr int RPS = FM_WAVE / LPR;
+    constexpr int BPL = FmLaneBytes<BITS>::value;
+    __shared__ float red[4];
+    __shared__ int s_last;
+    const int item = blockIdx.x;
+    const int pair = item / a.items_per_pair;
+    const int chunk = item - pair * a.items_per_pair;
+    const int l = pair / a.K;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int c = lane % LPR, r = lane / LPR;
+    const int rows_per_wave = a.rows_per_item >> 2;
+    const int row0 = chunk * a.rows_per_item + wave * rows_per_wave;
+    float *eo = a.expert_out + (size_t)pair * a.g.hidden;
+
+    const int e = a.idx[pair];
+    if ((unsigned)e >= (unsigned)a.g.n_experts) {
+        for (int i = lane; i < rows_per_wave; i += FM_WAVE) eo[row0 + i] = 0.0f;
+    } else {
+        const uint8_t *blob = a.layer_ptrs[a.layer0 + l * a.layer_stride] + (size_t)e * a.g.expert_size;
+        const int row_bytes = a.g.inter * BITS / 8;
+        const int sb_row_bytes = (a.g.inter / 64) * 2;
+        size_t woff = (size_t)(row0 + r) * row_bytes + (size_t)c * BPL;
+        size_t soff = (size_t)(row0 + r) * sb_row_bytes + (size_t)c * 4;
+        const size_t wstep = (size_t)RPS * row_bytes, sstep = (size_t)RPS * sb_row_bytes;
+        FmRowSlice<BITS> cur, next;
+        fm_load_slice<BITS>(cur, blob + a.g.down_w + woff, blob + a.g.down_s + soff,
+                            blob + a.g.down_b + soff);
+        float xs[FM_CPL], xsum0, xsum1;
+        fm_load_x<BITS>(a.act + (size_t)pair * a.g.inter + c * FM_CPL, xs, xsum0, xsum1);
+        const int steps = rows_per_wave / RPS;
+        for (int it = 0; it < steps; it++) {
+            if (it + 1 < steps) {
+                woff += wstep;
+                soff += sstep;
+                fm_load_slice<BITS>(next, blob + a.g.down_w + woff, blob + a.g.down_s + soff,
+                                    blob + a.g.down_b + soff);
+            }
+            float v = fm_group_sum<LPR>(fm_lane_dot<BITS, FP16>(cur, xs, xsum0, xsum1));
+            if (c == 0) eo[row0 + it * RPS + r] = v;
+            cur = next;
+        }
+    }
+
+    // arrival: make this workgroup's rows visible device-wide, then count
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned total = (unsigned)(a.K * a.items_per_pair);
+        unsigned old = atomicAdd(&a.counters[l], 1u);
+        s_last = (old == total - 1u);
+    }
+    __syncthreads();
+    if (s_last) {
+        __threadfence();
+        if (a.flags & FM_GUARD) fm_combine_layer<true>(a, l, red);
+        else fm_combine_layer<false>(a, l, red);
+        if (threadIdx.x == 0) a.counters[l] = 0u;
+    }
+}
+
+template <int BITS, bool FP16>
+int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down,
+                    hipStream_t st) {
+    DecodeArgs a1 = a, a2 = a;
+    a1.rows_per_item = rpi_up;
+    a1.items_per_pair = a.g.inter / rpi_up;
+    a2.rows_per_item = rpi_down;
+    a2.items_per_pair = a.g.hidden / rpi_down;
+    dim3 b(256);
+    const int lpr_up = a.g.hidden / FM_CPL, lpr_down = a.g.inter / FM_CPL;
+#define FM_UP(L) \
+    hipLaunchKernelGGL((fm_gate_up_swiglu<BITS, L, FP16>), dim3(n_pairs * a1.items_per_pair), b, 0, st, a1)
+#define FM_DOWN(L) \
+    hipLaunchKernelGGL((fm_down_combine<BITS, L, FP16>), dim3(n_pairs * a2.items_per_pair), b, 0, st, a2)
+    switch (lpr_up) {
+        case 4: FM_UP(4); break;
+        case 8: FM_UP(8); break;
+        case 16: FM_UP(16); break;
+        case 32: FM_UP(32); break;
+        default: return FM_ERR_UNSUPPORTED;
+    }
+    switch (lpr_down) {
+        case 1: FM_DOWN(1); break;
+        case 2: FM_DOWN(2); break;
+        case 4: FM_DOWN(4); break;
+        case 8: FM_DOWN(8); break;
+        case 16: FM_DOWN(16); break;
+        default: return FM_ERR_UNSUPPORTED;
+    }
+#undef FM_UP
+#undef FM_DOWN
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
+
+// rows per workgroup: min_rows * 2^j dividing `rows`, as large as possible (at
+// most `cap`) while the launch still has at least `want` workgroups
+int pick_rows_per_item(int rows, int n_pairs, int min_rows, int cap, int want) {
+    int rpi = min_rows;
+    while (rpi * 2 <= cap && rows % (rpi * 2) == 0 && (rows / (rpi * 2)) * n_pairs >= want)
+        rpi *= 2;
+    return rpi;
+}
+
+}  // namespace
+
+// Enqueue both kernels for n_layers x K pairs (n_layers groups of K slots: the
+// layers of a decode step, or with layer_stride 0 the positions of a chunk).  Shapes are validated by the
+// caller (fm_api.cpp): hidden, inter multiples of 128 with a supported
+// lanes-per-row, every layer resident.
+extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
+                                       const FmExpertGeom *g, int layer0, int layer_stride,
+                                       int n_layers, const float *d_x, const int32_t *d_idx,
+                                       const float *d_w, int K, float *d_act,
+                                       float *d_expert_out, float *d_out,
+                                       unsigned int *d_counters, int flags, int n_cu,
+                                       hipStream_t st) {
+    DecodeArgs a;
+    a.layer_ptrs = d_layer_ptrs;
+    a.g = *g;
+    a.layer0 = layer0;
+    a.layer_stride = layer_stride;
+    a.K = K;
+    a.x = d_x;
+    a.idx = d_idx;
+    a.w = d_w;
+    a.act = d_act;
+    a.expert_out = d_expert_out;
+    a.out = d_out;
+    a.counters = d_counters;
+    a.flags = flags;
+    a.rows_per_item = a.items_per_pair = 0;
+    const int n_pairs = n_layers * K;
+    const int lpr_up = g->hidden / FM_CPL, lpr_down = g->inter / FM_CPL;
+    if (lpr_up < 1 || lpr_down < 1) return FM_ERR_UNSUPPORTED;
+    // a wave step covers 64/LPR rows and a workgroup has 4 waves
+    const int min_up = 4 * (FM_WAVE / lpr_up), min_down = 4 * (FM_WAVE / lpr_down);
+    if (g->inter % min_up || g->hidden % min_down) return FM_ERR_UNSUPPORTED;
+    const int want = 4 * n_cu;
+    const int rpi_up = pick_rows_per_item(g->inter, n_pairs, min_up, 64, want);
+    const int rpi_down = pick_rows_per_item(g->hidden, n_pairs, min_down, 256, want);
+    if (g->bits == 3) {
+        return g->scale_fp16 ? launch_decode_t<3, true>(a, n_pairs, rpi_up, rpi_down, st)
+                             : launch_decode_t<3, false>(a, n_pairs, rpi_up, rpi_down, st);
+    }
+    if (g->bits == 4) {
+        return g->scale_fp16 ? launch_decode_t<4, true>(a, n_pairs, rpi_up, rpi_down, st)
+                             : launch_decode_t<4, false>(a, n_pairs, rpi_up, rpi_down, st);
+    }
+    return FM_ERR_UNSUPPORTED;
+}

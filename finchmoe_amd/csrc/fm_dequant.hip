@@ -1,0 +1,112 @@
+// fm_dequant.hip — materialise what the GEMV/GEMM kernels decode on the fly, for
+// bit-exact checks: integer codes and fp32 weights of an affine tensor
+// (finchmoe/infer.m:1720-1725, 1751-1757) or of GGUF Q4_K / Q6_K rows
+// (finchmoe/infer.m:1604-1657).  One thread per weight; not a hot path.
+#include "fm_common.h"
+
+namespace {
+
+__global__ void fm_dequant_affine_k(const uint8_t *W, const uint16_t *S, const uint16_t *B,
+                                    int out_dim, int in_dim, int group_size, int bits,
+                                    int scale_fp16, uint8_t *codes, float *w32,
+                                    uint16_t *w16) {
+    size_t n = (size_t)out_dim * in_dim;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (size_t)gridDim.x * blockDim.x) {
+        int r = (int)(i / in_dim), col = (int)(i % in_dim);
+        uint32_t q;
+        if (bits == 3) {
+            // 8 codes per 24-bit little-endian field (repack_experts.py:250-257)
+            const uint8_t *p = W + (size_t)r * (in_dim * 3 / 8) + 3 * (col >> 3);
+            uint32_t v = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
+            q = (v >> (3 * (col & 7))) & 7u;
+        } else {
+            // LSB-first fields of a little-endian u32 (quantize_model.py:35-43)
+            int vpu = 32 / bits;
+            const uint32_t *p = reinterpret_cast<const uint32_t *>(W) + (size_t)r * (in_dim / vpu);
+            q = (p[col / vpu] >> ((col % vpu) * bits)) & ((1u << bits) - 1u);
+        }
+        int ng = in_dim / group_size;
+        uint32_t sbits = S[(size_t)r * ng + col / group_size];
+        uint32_t bbits = B[(size_t)r * ng + col / group_size];
+        float s = scale_fp16 ? fm_fp16_bits(sbits) : fm_bf16_lo(sbits);
+        float b = scale_fp16 ? fm_fp16_bits(bbits) : fm_bf16_lo(bbits);
+        // code * scale is exact in fp32 (<= 8 + 11 significant bits), so the sum
+        // is rounded once whether or not the compiler contracts it into an FMA
+        float w = (float)q * s + b;
+        if (codes) codes[i] = (uint8_t)q;
+        if (w32) w32[i] = w;
+        if (w16) {
+            _Float16 h = (_Float16)w;   // round-to-nearest-even
+            w16[i] = __builtin_bit_cast(unsigned short, h);
+        }
+    }
+}
+
+// finchmoe/infer.m:1595-1603
+__device__ __forceinline__ void scale_min_k4(int j, const uint8_t *s, int &sc, int &m) {
+    if (j < 4) {
+        sc = s[j] & 63;
+        m = s[j + 4] & 63;
+    } else {
+        sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4);
+        m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+    }
+}
+
+__global__ void fm_dequant_gguf_k(const uint8_t *W, int out_dim, int in_dim, int ggml_type,
+                                  float *w32) {
+    size_t n = (size_t)out_dim * in_dim;
+    const int bsz = ggml_type == FM_GGML_Q4_K ? 144 : 210;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (size_t)gridDim.x * blockDim.x) {
+        int r = (int)(i / in_dim), col = (int)(i % in_dim);
+        const uint8_t *blk = W + ((size_t)r * (in_dim / 256) + (col >> 8)) * bsz;
+        int e = col & 255;
+        float w;
+        if (ggml_type == FM_GGML_Q4_K) {
+            float d = fm_fp16_bits(blk[0] | (blk[1] << 8));
+            float dmin = fm_fp16_bits(blk[2] | (blk[3] << 8));
+            int chunk = e >> 6, high = (e >> 5) & 1, l = e & 31;
+            int sc, m;
+            scale_min_k4(2 * chunk + high, blk + 4, sc, m);
+            int nib = (blk[16 + 32 * chunk + l] >> (4 * high)) & 0xF;
+            float d1 = d * (float)sc, m1 = dmin * (float)m;
+            w = d1 * (float)nib - m1;
+        } else {
+            float d = fm_fp16_bits(blk[208] | (blk[209] << 8));
+            int half = e >> 7, vi = e & 127;
+            int nib = (blk[64 * half + (vi & 63)] >> (4 * (vi >> 6))) & 0xF;
+            int hi2 = (blk[128 + 32 * half + (vi & 31)] >> (2 * ((vi >> 5) & 3))) & 3;
+            int sc = (int)(int8_t)blk[192 + 8 * half + (vi >> 4)];
+            int q = (nib | (hi2 << 4)) - 32;
+            w = d * (float)sc * (float)q;
+        }
+        w32[i] = w;
+    }
+}
+
+}  // namespace
+
+extern "C" int fm_launch_dequant_affine(const void *W, const void *S, const void *B,
+                                        int out_dim, int in_dim, int group_size, int bits,
+                                        int scale_fp16, uint8_t *codes, float *w32,
+                                        uint16_t *w16, hipStream_t st) {
+    size_t n = (size_t)out_dim * in_dim;
+    int blocks = (int)((n + 255) / 256);
+    if (blocks > 65535) blocks = 65535;
+    hipLaunchKernelGGL(fm_dequant_affine_k, dim3(blocks), dim3(256), 0, st,
+                       (const uint8_t *)W, (const uint16_t *)S, (const uint16_t *)B, out_dim,
+                       in_dim, group_size, bits, scale_fp16, codes, w32, w16);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
+
+extern "C" int fm_launch_dequant_gguf(const void *W, int out_dim, int in_dim, int ggml_type,
+                                      float *w32, hipStream_t st) {
+    size_t n = (size_t)out_dim * in_dim;
+    int blocks = (int)((n + 255) / 256);
+    if (blocks > 65535) blocks = 65535;
+    hipLaunchKernelGGL(fm_dequant_gguf_k, dim3(blocks), dim3(256), 0, st, (const uint8_t *)W,
+                       out_dim, in_dim, ggml_type, w32);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}

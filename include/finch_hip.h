@@ -1,0 +1,200 @@
+/*
+ * finch_hip.h — C ABI of libfinchhip.so: FinchMoE's quantized-expert operator
+ * path (dequant fused with the matrix products) on one MI355X (gfx950).
+ *
+ * The reference has no header or FFI for this path: its "operator API" is a set
+ * of static C functions in finchmoe/infer.m driving Metal kernels.  Each entry
+ * point below names the reference function whose operand contract it keeps
+ * (paths relative to the reference tree).  Packed weights are accepted in the
+ * reference's own layouts, byte for byte:
+ *   - affine expert blobs  packed_experts_{N}bit/layer_XX.bin
+ *                          (finchmoe/repack_experts.py:76-163, 336-392;
+ *                           finchmoe/infer.m:174-234)
+ *   - dense affine tensors .weight U32 / .scales / .biases
+ *                          (finchmoe/quantize_non_experts.py:294, 365-386;
+ *                           finchmoe/quantize_model.py:19-47)
+ *   - GGUF expert slabs    Q4_K / Q6_K stacked tensors
+ *                          (finchmoe/infer.m:1017-1022, 1120-1148, 1604-1657)
+ *
+ * Conventions
+ *   - every function returns an fm_status (0 = ok, negative = error); nothing
+ *     aborts; fm_last_error() gives a message for the last failure on a context
+ *   - *_dev entry points take DEVICE pointers, enqueue on the context's stream
+ *     and return without waiting; host-pointer entry points (no suffix) copy
+ *     in, run, copy out and wait, like the reference's synchronous calls
+ *   - a context is not re-entrant: one caller thread at a time, one stream
+ *     (the reference's compute path is single-threaded, infer.m:13874)
+ *   - weights are immutable after upload; host copies may be freed afterwards
+ *   - there is no CPU fallback: without a GPU every compute call fails
+ */
+#ifndef FINCH_HIP_H
+#define FINCH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FM_API __attribute__((visibility("default")))
+
+typedef struct fm_ctx fm_ctx;
+
+typedef enum {
+    FM_OK = 0,
+    FM_ERR_ARG = -1,          /* bad argument (null, range, shape, alignment)  */
+    FM_ERR_HIP = -2,          /* a HIP runtime call failed                     */
+    FM_ERR_STATE = -3,        /* store not configured / layer not resident     */
+    FM_ERR_UNSUPPORTED = -4,  /* format or shape this build has no kernel for  */
+    FM_ERR_NOMEM = -5
+} fm_status;
+
+/* 16-bit type of the per-group scale and bias.  The reference stores BF16
+ * (finchmoe/repack_experts.py:232-234, finchmoe/infer.m:690-695). */
+enum { FM_SCALE_BF16 = 0, FM_SCALE_FP16 = 1 };
+
+/* ggml tensor types accepted for GGUF slabs (finchmoe/infer.m:1606, 1631) */
+enum { FM_GGML_Q4_K = 12, FM_GGML_Q6_K = 14 };
+
+/* flags of the routed-expert calls */
+enum {
+    FM_ACCUMULATE = 1,  /* out += result (gpu_gguf_experts_forward adds into
+                           moe_out, infer.m:3340); default overwrites          */
+    FM_GUARD = 2        /* CPU-path combine: skip an expert whose output has a
+                           non-finite or >=1e20 sum of squares, renormalise
+                           when 0 < sum of kept weights < 0.99
+                           (infer.m:10190-10204).  Default is the GPU path's
+                           plain slot-order sum (shaders.metal:2213-2228).    */
+};
+
+/* which matrix of an expert (dequant entry points) */
+enum { FM_MAT_GATE = 0, FM_MAT_UP = 1, FM_MAT_DOWN = 2 };
+
+/* ---------------------------------------------------------------- context
+ * Replaces MetalCtx + metal_setup (finchmoe/infer.m:2190-2811). */
+FM_API int fm_ctx_create(int device, fm_ctx **out);
+FM_API int fm_ctx_destroy(fm_ctx *ctx);
+FM_API int fm_sync(fm_ctx *ctx);
+FM_API void *fm_stream(fm_ctx *ctx);                 /* the hipStream_t of the context */
+FM_API const char *fm_last_error(fm_ctx *ctx);
+FM_API const char *fm_status_string(int status);
+/* event pair on the context's stream around whatever is enqueued in between */
+FM_API int fm_timer_start(fm_ctx *ctx);
+FM_API int fm_timer_stop(fm_ctx *ctx, float *elapsed_ms);   /* waits for the stop event */
+
+/* ---------------------------------------------------------------- expert store, affine
+ * Replaces the packed-expert files + pread/LRU machinery
+ * (finchmoe/infer.m:5816-6575, 15421-15425) by HBM residency.
+ * bits: 3 or 4.  hidden, inter multiples of 128.  group_size 64. */
+FM_API int fm_experts_config(fm_ctx *ctx, int n_layers, int n_experts, int hidden, int inter,
+                      int group_size, int bits, int scale_dtype);
+FM_API size_t fm_experts_expert_size(fm_ctx *ctx);   /* bytes of one expert, 0 if unconfigured */
+/* verbatim bytes of layer_XX.bin: n_experts * expert_size */
+FM_API int fm_experts_upload_layer(fm_ctx *ctx, int layer, const void *host_blob, size_t nbytes);
+/* same layout already in device memory owned by the caller (16-byte aligned);
+ * must stay valid until the context is destroyed or the layer is replaced */
+FM_API int fm_experts_adopt_layer(fm_ctx *ctx, int layer, const void *dev_blob, size_t nbytes);
+
+/* ---------------------------------------------------------------- routed experts, decode
+ * Replaces gpu_encode_experts_batched + moe_combine_residual's weighted sum
+ * (finchmoe/infer.m:4065-4383, finchmoe/shaders.metal:2196-2231) and the CPU
+ * twin (infer.m:10109-10204).
+ *   x[hidden] fp32, idx[K] int32 (distinct experts, any order), w[K] fp32
+ *   out[hidden] = sum_k w[k] * down_k(SiLU(gate_k x) * up_k x), k in slot order
+ *   expert_out (may be NULL) receives the K per-expert vectors [K][hidden]
+ *   K in 1..8.  w[k] == 0 keeps the slot but adds nothing (valid[k]=0,
+ *   infer.m:9672).  An index outside 0..n_experts-1 is treated as w[k] = 0. */
+FM_API int fm_moe_decode_dev(fm_ctx *ctx, int layer, const float *d_x, const int32_t *d_idx,
+                      const float *d_w, int K, float *d_out, float *d_expert_out, int flags);
+FM_API int fm_moe_decode(fm_ctx *ctx, int layer, const float *x, const int32_t *idx,
+                  const float *w, int K, float *out, float *expert_out, int flags);
+/* n_layers consecutive layers in one submission, each with its own x, idx, w:
+ * x[n_layers][hidden], idx[n_layers][K], w[n_layers][K], out[n_layers][hidden],
+ * expert_out[n_layers][K][hidden] or NULL.  (The per-token loop over layers,
+ * infer.m:15771, with the expert blocks of all layers batched.) */
+FM_API int fm_moe_decode_step_dev(fm_ctx *ctx, int layer0, int n_layers, const float *d_x,
+                           const int32_t *d_idx, const float *d_w, int K, float *d_out,
+                           float *d_expert_out, int flags);
+
+/* ---------------------------------------------------------------- routed experts, chunked prefill
+ * Replaces prefill_chunk_cmd3_encode / prefill_chunk_cmd3_batch_general
+ * (finchmoe/infer.m:10704-11059): M positions, each with its own top-K.
+ *   X[M][hidden] fp32, idx[M][K], w[M][K], out[M][hidden] fp32.
+ * Result contract: the same as fm_moe_decode per position. */
+FM_API int fm_moe_prefill_dev(fm_ctx *ctx, int layer, const float *d_X, const int32_t *d_idx,
+                       const float *d_w, int M, int K, float *d_out, int flags);
+FM_API int fm_moe_prefill(fm_ctx *ctx, int layer, const float *X, const int32_t *idx,
+                   const float *w, int M, int K, float *out, int flags);
+
+/* ---------------------------------------------------------------- dense affine tensors
+ * Replaces fast_dequant_matvec / BatchMatvecSpec + fast_batch_matvec /
+ * gpu_encode_prefill_matvec (finchmoe/infer.m:3369, 3401-3411, 4477, 3672;
+ * kernels dequant_matvec_4bit_v3 and _prefill, shaders.metal:374-463, 2460-2529).
+ * W: u32 [out_dim][in_dim*bits/32] (bits 4 or 8) or bytes [out_dim][in_dim*3/8]
+ * (bits 3); S, B: 16-bit [out_dim][in_dim/group_size]. */
+typedef int fm_tensor;   /* handle >= 0 */
+FM_API int fm_tensor_register(fm_ctx *ctx, const void *W, const void *S, const void *B,
+                       int out_dim, int in_dim, int group_size, int bits,
+                       int scale_dtype, fm_tensor *out);
+/* device-resident W, S, B owned by the caller (16-byte aligned) */
+FM_API int fm_tensor_adopt(fm_ctx *ctx, const void *d_W, const void *d_S, const void *d_B,
+                    int out_dim, int in_dim, int group_size, int bits,
+                    int scale_dtype, fm_tensor *out);
+FM_API int fm_tensor_release(fm_ctx *ctx, fm_tensor t);
+/* n matvecs sharing one input vector (all tensors must have the same in_dim) */
+FM_API int fm_matvec_batch_dev(fm_ctx *ctx, const fm_tensor *tensors, int n, const float *d_x,
+                        float *const *d_outs);
+FM_API int fm_matvec_batch(fm_ctx *ctx, const fm_tensor *tensors, int n, const float *x,
+                    float *const *outs);
+/* M positions: X[M][in_dim] -> out[M][out_dim] */
+FM_API int fm_matvec_prefill_dev(fm_ctx *ctx, fm_tensor t, const float *d_X, float *d_out, int M);
+FM_API int fm_matvec_prefill(fm_ctx *ctx, fm_tensor t, const float *X, float *out, int M);
+
+/* ---------------------------------------------------------------- GGUF expert store
+ * Replaces GgufExpertInfo + the slab copies of gpu_gguf_experts_forward
+ * (finchmoe/infer.m:1017-1022, 3239-3290).  gate/up/down are the stacked
+ * per-layer tensors, expert e at e*slab; gate and up must be Q4_K, down Q4_K or
+ * Q6_K (infer.m:3166). */
+FM_API int fm_gguf_config(fm_ctx *ctx, int n_layers, int n_experts, int hidden, int inter,
+                   int gate_type, int up_type, int down_type);
+FM_API int fm_gguf_upload_layer(fm_ctx *ctx, int layer, const void *gate, const void *up,
+                         const void *down);
+FM_API int fm_gguf_adopt_layer(fm_ctx *ctx, int layer, const void *d_gate, const void *d_up,
+                        const void *d_down);
+/* gpu_gguf_experts_forward (finchmoe/infer.m:3153-3366) */
+FM_API int fm_gguf_moe_decode_dev(fm_ctx *ctx, int layer, const float *d_x, const int32_t *d_idx,
+                           const float *d_w, int K, float *d_out, float *d_expert_out,
+                           int flags);
+FM_API int fm_gguf_moe_decode(fm_ctx *ctx, int layer, const float *x, const int32_t *idx,
+                       const float *w, int K, float *out, float *expert_out, int flags);
+FM_API int fm_gguf_moe_decode_step_dev(fm_ctx *ctx, int layer0, int n_layers, const float *d_x,
+                                const int32_t *d_idx, const float *d_w, int K,
+                                float *d_out, float *d_expert_out, int flags);
+/* prefill_chunk_cmd3_batch_general in GGUF mode (finchmoe/infer.m:10958-11059) */
+FM_API int fm_gguf_moe_prefill_dev(fm_ctx *ctx, int layer, const float *d_X, const int32_t *d_idx,
+                            const float *d_w, int M, int K, float *d_out, int flags);
+FM_API int fm_gguf_moe_prefill(fm_ctx *ctx, int layer, const float *X, const int32_t *idx,
+                        const float *w, int M, int K, float *out, int flags);
+/* single Q4_K / Q6_K matvec (gpu_gguf_dequant_matvec, finchmoe/infer.m:3050;
+ * kernel dequant_matvec_qk, shaders.metal:3216-3299); host pointers */
+FM_API int fm_gguf_matvec(fm_ctx *ctx, const void *W, int ggml_type, const float *x, float *out,
+                   int out_dim, int in_dim);
+
+/* ---------------------------------------------------------------- dequant (bit-exact checks)
+ * The reference has no such call; these expose what its kernels compute on the
+ * fly — code = field of the packed word, w = (float)code * scale + bias in fp32
+ * (finchmoe/infer.m:1725, 1757; shaders.metal:598-605) — so tests can compare
+ * codes and weights bit for bit.  Host output buffers, any may be NULL:
+ * codes u8 [rows][cols], w_f32 [rows][cols], w_f16 = RNE(w_f32) as IEEE half. */
+FM_API int fm_dequant_expert(fm_ctx *ctx, int layer, int expert, int which, uint8_t *codes,
+                      float *w_f32, uint16_t *w_f16);
+FM_API int fm_dequant_tensor(fm_ctx *ctx, fm_tensor t, uint8_t *codes, float *w_f32,
+                      uint16_t *w_f16);
+/* GGUF: w_f32 = the block formula (finchmoe/infer.m:1604-1657) */
+FM_API int fm_gguf_dequant_expert(fm_ctx *ctx, int layer, int expert, int which, float *w_f32);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FINCH_HIP_H */

@@ -1,0 +1,93 @@
+"""GPU parity of the dense affine GEMV (GatedDeltaNet projections) against the CPU oracle."""
+import numpy as np
+import pytest
+
+from finchmoe_amd import binding as fb
+from finchmoe_amd import formats as F
+from .conftest import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def _tensor(hip, rng, out_dim, in_dim, bits, dtype="bf16"):
+    codes, W, S, B = F.synth_affine_tensor(rng, out_dim, in_dim, bits, dtype)
+    sd = fb.SCALE_BF16 if dtype == "bf16" else fb.SCALE_FP16
+    t = hip.tensor_register(W, S, B, out_dim, in_dim, bits, 64, sd)
+    return t, (codes, W, S, B, sd)
+
+
+def test_gdn_projections_4bit(hip, orc):
+    """in_proj_qkv [8192,2048] + in_proj_z [4096,2048] from one x, then out_proj
+    [2048,4096] (infer.m:8119-8122, 8500-8502)."""
+    rng = np.random.default_rng(1)
+    tq, q = _tensor(hip, rng, 8192, 2048, 4)
+    tz, z = _tensor(hip, rng, 4096, 2048, 4)
+    to, o = _tensor(hip, rng, 2048, 4096, 4)
+    x = rng.standard_normal(2048).astype(np.float32)
+    oq, oz = hip.matvec_batch([tq, tz], x, [8192, 4096])
+    assert_parity(oq, orc.dequant_matvec(q[1], q[2], q[3], x, 8192, 2048, 4, nthreads=8), "qkv")
+    assert_parity(oz, orc.dequant_matvec(z[1], z[2], z[3], x, 4096, 2048, 4, nthreads=8), "z")
+    y = rng.standard_normal(4096).astype(np.float32)
+    (oo,) = hip.matvec_batch([to], y, [2048])
+    r, _ = assert_parity(oo, orc.dequant_matvec(o[1], o[2], o[3], y, 2048, 4096, 4, nthreads=8), "out_proj")
+    assert r < 2e-5
+    for t in (tq, tz, to):
+        hip.tensor_release(t)
+
+
+@pytest.mark.parametrize("bits,dtype,out_dim,in_dim", [
+    (4, "bf16", 32, 2048), (4, "fp16", 100, 512), (8, "bf16", 256, 2048), (3, "bf16", 77, 1024),
+    (4, "bf16", 5, 128), (8, "fp16", 33, 256), (4, "bf16", 64, 8192)])
+def test_matvec_shapes_and_widths(hip, orc, bits, dtype, out_dim, in_dim):
+    """Ragged out_dim, small and large in_dim, every packing width, both scale types;
+    codes and weights bit-exact, outputs within tolerance."""
+    rng = np.random.default_rng(out_dim * 31 + in_dim + bits)
+    t, (codes, W, S, B, sd) = _tensor(hip, rng, out_dim, in_dim, bits, dtype)
+    gc, gw, gh = hip.dequant_tensor(t, out_dim, in_dim)
+    rc, rw = orc.dequant_affine(W, S, B, out_dim, in_dim, bits, scale_dtype=sd)
+    assert np.array_equal(gc, codes) and np.array_equal(gc, rc)
+    assert np.array_equal(gw.view(np.uint32), rw.view(np.uint32))
+    assert np.array_equal(gh, rw.astype(np.float16).view(np.uint16))
+    x = rng.standard_normal(in_dim).astype(np.float32)
+    (got,) = hip.matvec_batch([t], x, [out_dim])
+    assert_parity(got, orc.dequant_matvec(W, S, B, x, out_dim, in_dim, bits, scale_dtype=sd), "matvec")
+    # one-hot input returns a dequantized column
+    e = np.zeros(in_dim, np.float32)
+    e[in_dim // 2 + 3] = 1.0
+    (col,) = hip.matvec_batch([t], e, [out_dim])
+    assert np.allclose(col, rw[:, in_dim // 2 + 3], rtol=1e-6, atol=1e-9)
+    hip.tensor_release(t)
+
+
+def test_matvec_prefill_positions(hip, orc):
+    """M-position clone (dequant_matvec_4bit_prefill): every position equals the single call."""
+    rng = np.random.default_rng(3)
+    t, (codes, W, S, B, sd) = _tensor(hip, rng, 512, 2048, 4)
+    X = rng.standard_normal((8, 2048)).astype(np.float32)
+    out = hip.matvec_prefill(t, X, 512)
+    for m in range(8):
+        (single,) = hip.matvec_batch([t], X[m], [512])
+        assert np.array_equal(out[m], single)
+        assert_parity(out[m], orc.dequant_matvec(W, S, B, X[m], 512, 2048, 4), "pos %d" % m)
+    hip.tensor_release(t)
+
+
+def test_mixed_batch_and_errors(hip, orc):
+    rng = np.random.default_rng(4)
+    t4, a = _tensor(hip, rng, 64, 2048, 4)
+    t8, b = _tensor(hip, rng, 32, 2048, 8)
+    x = rng.standard_normal(2048).astype(np.float32)
+    o4, o8 = hip.matvec_batch([t4, t8], x, [64, 32])    # mixed widths: split into two launches
+    assert_parity(o4, orc.dequant_matvec(a[1], a[2], a[3], x, 64, 2048, 4), "4-bit")
+    assert_parity(o8, orc.dequant_matvec(b[1], b[2], b[3], x, 32, 2048, 8), "8-bit")
+    from finchmoe_amd import FinchError
+    t5, _ = _tensor(hip, rng, 16, 512, 4)
+    with pytest.raises(FinchError):
+        hip.matvec_batch([t4, t5], x, [64, 16])           # in_dim mismatch
+    with pytest.raises(FinchError):
+        hip.matvec_batch([12345], x, [64])
+    with pytest.raises(FinchError) as e:
+        hip.tensor_register(a[1], a[2], a[3], 64, 2000, 4)
+    assert e.value.status == fb.ERR_UNSUPPORTED
+    for t in (t4, t8, t5):
+        hip.tensor_release(t)
