@@ -40,6 +40,14 @@ def load():
     path = lib_path()
     if not os.path.exists(path):
         raise FinchError(ERR_STATE, "libfinchhip.so not built: run python -m finchmoe_amd.build")
+    # One HIP runtime per process.  PyTorch ships its own libamdhip64 (same SONAME as the
+    # system one); if it is loaded first, this library's libamdhip64.so.7 dependency binds to
+    # it.  Loaded in the other order the process ends up with two runtimes and the second one
+    # finds no device.  So when torch is installed, load it first.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = C.CDLL(path)
     vp, i, sz = C.c_void_p, C.c_int, C.c_size_t
     sig = {
