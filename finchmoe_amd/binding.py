@@ -59,6 +59,8 @@ def load():
         "fm_status_string": (C.c_char_p, [i]),
         "fm_timer_start": (i, [vp]),
         "fm_timer_stop": (i, [vp, C.POINTER(C.c_float)]),
+        "fm_kernel_timing": (i, [vp, i]),
+        "fm_kernel_timing_read": (i, [vp, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i)]),
         "fm_experts_config": (i, [vp, i, i, i, i, i, i, i]),
         "fm_experts_expert_size": (sz, [vp]),
         "fm_experts_upload_layer": (i, [vp, i, vp, sz]),
@@ -146,6 +148,14 @@ class FinchHip:
         ms = C.c_float()
         self._chk(self.L.fm_timer_stop(self.h, C.byref(ms)))
         return ms.value
+
+    def kernel_timing(self, enable):
+        self._chk(self.L.fm_kernel_timing(self.h, int(enable)))
+
+    def kernel_timing_read(self):
+        a, b, n = C.c_double(), C.c_double(), C.c_int()
+        self._chk(self.L.fm_kernel_timing_read(self.h, C.byref(a), C.byref(b), C.byref(n)))
+        return a.value, b.value, n.value
 
     # ---- affine expert store
     def experts_config(self, n_layers, n_experts, hidden=2048, inter=512, group_size=64, bits=3,

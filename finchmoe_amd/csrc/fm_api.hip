@@ -23,7 +23,7 @@ int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs, const FmExpertGe
                             int layer0, int layer_stride, int n_layers, const float *d_x,
                             const int32_t *d_idx, const float *d_w, int K, float *d_act,
                             float *d_expert_out, float *d_out, unsigned int *d_counters,
-                            int flags, int n_cu, hipStream_t st);
+                            int flags, int n_cu, hipStream_t st, hipEvent_t *kev);
 int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
                     const float *d_x, int M, int n_cu, hipStream_t st);
 int fm_launch_dequant_affine(const void *W, const void *S, const void *B, int out_dim,
@@ -36,7 +36,7 @@ int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t *const *d_
                           int layer_stride, int n_layers, const float *d_x,
                           const int32_t *d_idx, const float *d_w, int K, float *d_act,
                           float *d_expert_out, float *d_out, unsigned int *d_counters,
-                          int flags, int n_cu, hipStream_t st);
+                          int flags, int n_cu, hipStream_t st, hipEvent_t *kev);
 int fm_launch_gguf_matvec(const uint8_t *d_W, int ggml_type, const float *d_x, float *d_out,
                           int out_dim, int in_dim, int n_cu, hipStream_t st);
 int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGeom *g, const float *d_X,
@@ -66,6 +66,10 @@ struct fm_ctx {
     int n_cu = 256;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    hipEvent_t kev[3] = {nullptr, nullptr, nullptr};
+    bool ktiming = false;
+    double k1_ms = 0.0, k2_ms = 0.0;
+    int kcalls = 0;
     std::string err;
 
     // affine expert store
@@ -226,6 +230,11 @@ extern "C" int fm_ctx_create(int device, fm_ctx **out) {
         delete c;
         return FM_ERR_HIP;
     }
+    for (auto &e : c->kev)
+        if (hipEventCreate(&e) != hipSuccess) {
+            delete c;
+            return FM_ERR_HIP;
+        }
     *out = c;
     return FM_OK;
 }
@@ -250,6 +259,7 @@ extern "C" int fm_ctx_destroy(fm_ctx *c) {
         if (p) (void)hipFree(p);
     (void)hipEventDestroy(c->ev0);
     (void)hipEventDestroy(c->ev1);
+    for (auto &e : c->kev) (void)hipEventDestroy(e);
     (void)hipStreamDestroy(c->stream);
     delete c;
     return FM_OK;
@@ -291,6 +301,36 @@ extern "C" int fm_timer_stop(fm_ctx *c, float *ms) {
     HIPCHK(c, hipEventRecord(c->ev1, c->stream));
     HIPCHK(c, hipEventSynchronize(c->ev1));
     HIPCHK(c, hipEventElapsedTime(ms, c->ev0, c->ev1));
+    return FM_OK;
+}
+
+extern "C" int fm_kernel_timing(fm_ctx *c, int enable) {
+    if (!c) return FM_ERR_ARG;
+    c->ktiming = enable != 0;
+    c->k1_ms = c->k2_ms = 0.0;
+    c->kcalls = 0;
+    return FM_OK;
+}
+
+extern "C" int fm_kernel_timing_read(fm_ctx *c, double *k1, double *k2, int *calls) {
+    if (!c) return FM_ERR_ARG;
+    if (k1) *k1 = c->k1_ms;
+    if (k2) *k2 = c->k2_ms;
+    if (calls) *calls = c->kcalls;
+    c->k1_ms = c->k2_ms = 0.0;
+    c->kcalls = 0;
+    return FM_OK;
+}
+
+// after a decode launch with the three timing events recorded
+static int ktiming_collect(fm_ctx *c) {
+    HIPCHK(c, hipEventSynchronize(c->kev[2]));
+    float a = 0.0f, b = 0.0f;
+    HIPCHK(c, hipEventElapsedTime(&a, c->kev[0], c->kev[1]));
+    HIPCHK(c, hipEventElapsedTime(&b, c->kev[1], c->kev[2]));
+    c->k1_ms += a;
+    c->k2_ms += b;
+    c->kcalls++;
     return FM_OK;
 }
 
@@ -395,8 +435,10 @@ extern "C" int fm_moe_decode_step_dev(fm_ctx *c, int layer0, int n_layers, const
     if (rc) return rc;
     rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer0, 1, n_layers, d_x, d_idx, d_w,
                                  K, c->d_act, d_expert_out ? d_expert_out : c->d_eo, d_out,
-                                 c->d_counters, flags, c->n_cu, c->stream);
+                                 c->d_counters, flags, c->n_cu, c->stream,
+                                 c->ktiming ? c->kev : nullptr);
     if (rc) return fail(c, rc, "decode launch failed: %s", hipGetErrorString(hipGetLastError()));
+    if (c->ktiming) return ktiming_collect(c);
     return FM_OK;
 }
 
@@ -489,7 +531,7 @@ extern "C" int fm_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, const 
     if (rc) return rc;
     rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer, 0, M, d_X, d_idx, d_w, K,
                                  c->d_act, c->d_eo, d_out, c->d_counters, flags, c->n_cu,
-                                 c->stream);
+                                 c->stream, nullptr);
     if (rc) return fail(c, rc, "prefill launch failed: %s", hipGetErrorString(hipGetLastError()));
     return FM_OK;
 }
@@ -775,8 +817,9 @@ static int gguf_decode_groups(fm_ctx *c, int layer0, int layer_stride, int group
                                c->d_gg_ptrs + 2 * (size_t)c->g_layers, &c->ggeom, layer0,
                                layer_stride, groups, d_x, d_idx, d_w, K, c->d_act,
                                d_expert_out ? d_expert_out : c->d_eo, d_out, c->d_counters, flags,
-                               c->n_cu, c->stream);
+                               c->n_cu, c->stream, c->ktiming ? c->kev : nullptr);
     if (rc) return fail(c, rc, "GGUF decode launch failed: %s", hipGetErrorString(hipGetLastError()));
+    if (c->ktiming) return ktiming_collect(c);
     return FM_OK;
 }
 

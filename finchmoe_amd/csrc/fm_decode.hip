@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256) void fm_down_combine(DecodeArgs a) {
 
 template <int BITS, bool FP16>
 int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down,
-                    hipStream_t st) {
+                    hipStream_t st, hipEvent_t *kev) {
     DecodeArgs a1 = a, a2 = a;
     a1.rows_per_item = rpi_up;
     a1.items_per_pair = a.g.inter / rpi_up;
@@ -212,6 +212,7 @@ int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down,
     hipLaunchKernelGGL((fm_gate_up_swiglu<BITS, L, FP16>), dim3(n_pairs * a1.items_per_pair), b, 0, st, a1)
 #define FM_DOWN(L) \
     hipLaunchKernelGGL((fm_down_combine<BITS, L, FP16>), dim3(n_pairs * a2.items_per_pair), b, 0, st, a2)
+    if (kev) (void)hipEventRecord(kev[0], st);
     switch (lpr_up) {
         case 4: FM_UP(4); break;
         case 8: FM_UP(8); break;
@@ -219,6 +220,7 @@ int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down,
         case 32: FM_UP(32); break;
         default: return FM_ERR_UNSUPPORTED;
     }
+    if (kev) (void)hipEventRecord(kev[1], st);
     switch (lpr_down) {
         case 1: FM_DOWN(1); break;
         case 2: FM_DOWN(2); break;
@@ -229,6 +231,7 @@ int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down,
     }
 #undef FM_UP
 #undef FM_DOWN
+    if (kev) (void)hipEventRecord(kev[2], st);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 
@@ -253,7 +256,7 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
                                        const float *d_w, int K, float *d_act,
                                        float *d_expert_out, float *d_out,
                                        unsigned int *d_counters, int flags, int n_cu,
-                                       hipStream_t st) {
+                                       hipStream_t st, hipEvent_t *kev) {
     DecodeArgs a;
     a.layer_ptrs = d_layer_ptrs;
     a.g = *g;
@@ -279,12 +282,12 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     const int rpi_up = pick_rows_per_item(g->inter, n_pairs, min_up, 64, want);
     const int rpi_down = pick_rows_per_item(g->hidden, n_pairs, min_down, 256, want);
     if (g->bits == 3) {
-        return g->scale_fp16 ? launch_decode_t<3, true>(a, n_pairs, rpi_up, rpi_down, st)
-                             : launch_decode_t<3, false>(a, n_pairs, rpi_up, rpi_down, st);
+        return g->scale_fp16 ? launch_decode_t<3, true>(a, n_pairs, rpi_up, rpi_down, st, kev)
+                             : launch_decode_t<3, false>(a, n_pairs, rpi_up, rpi_down, st, kev);
     }
     if (g->bits == 4) {
-        return g->scale_fp16 ? launch_decode_t<4, true>(a, n_pairs, rpi_up, rpi_down, st)
-                             : launch_decode_t<4, false>(a, n_pairs, rpi_up, rpi_down, st);
+        return g->scale_fp16 ? launch_decode_t<4, true>(a, n_pairs, rpi_up, rpi_down, st, kev)
+                             : launch_decode_t<4, false>(a, n_pairs, rpi_up, rpi_down, st, kev);
     }
     return FM_ERR_UNSUPPORTED;
 }

@@ -5,7 +5,8 @@
 extern "C" int fm_launch_decode_gguf(const uint8_t *const *, const uint8_t *const *,
                                      const uint8_t *const *, const FmGgufGeom *, int, int, int,
                                      const float *, const int32_t *, const float *, int, float *,
-                                     float *, float *, unsigned int *, int, int, hipStream_t) {
+                                     float *, float *, unsigned int *, int, int, hipStream_t,
+                                     hipEvent_t *) {
     return FM_ERR_UNSUPPORTED;
 }
 extern "C" int fm_launch_gguf_matvec(const uint8_t *, int, const float *, float *, int, int, int,
