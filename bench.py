@@ -194,12 +194,12 @@ def run_decode_step(args):
         "token_latency_us": {"mean": round(float(lat.mean()), 1), "p50": round(float(np.median(lat)), 1),
                              "p99": round(float(np.percentile(lat, 99)), 1)},
         "unique_experts_touched_in_256_tokens": uniq,
-        "kernels_us": {"fm_gate_up_swiglu": round(k1_us, 2), "fm_down_combine": round(k2_us, 2)},
+        "kernels_us": {"fm_gate_up_swiglu": round(k1_us, 2), "fm_down+fm_combine": round(k2_us, 2)},
         "roofline": {"bound": "hbm", "kernel": "fm_gate_up_swiglu<3,16>",
                      "achieved": round(k1_bytes / (k1_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(k1_bytes / (k1_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                      "traffic": None, "bytes_per_launch": k1_bytes},
-        "roofline_down": {"bound": "hbm", "kernel": "fm_down_combine<3,4>",
+        "roofline_down": {"bound": "hbm", "kernel": "fm_down<3,4> + fm_combine",
                           "achieved": round((bytes_step - k1_bytes) / (k2_us * 1e-6) / 1e9, 1),
                           "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": round((bytes_step - k1_bytes) / (k2_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)},

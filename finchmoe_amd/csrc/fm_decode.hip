@@ -1,6 +1,7 @@
 // fm_decode.hip — routed-expert decode for affine-packed experts:
 //   kernel 1  gate GEMV + up GEMV + SwiGLU for every (layer, slot) pair
-//   kernel 2  down GEMV per pair, then the router-weighted sum in slot order
+//   kernel 2  down GEMV per pair -> per-expert output vectors
+//   kernel 3  router-weighted sum of the K vectors of a layer, in slot order
 // Replaces the four dispatches per expert of gpu_encode_experts_batched
 // (finchmoe/infer.m:4337-4378: dequant_matvec_3bit x3 + swiglu_fused) and the
 // weighted sum of moe_combine_residual (finchmoe/shaders.metal:2213-2228).
@@ -30,7 +31,6 @@ struct DecodeArgs {
     float *act;              // [nl][K][inter]   scratch
     float *expert_out;       // [nl][K][hidden]
     float *out;              // [nl][hidden]
-    unsigned int *counters;  // [nl] arrival counters, zero between launches
     int rows_per_item;
     int items_per_pair;
     int flags;
@@ -91,57 +91,64 @@ __global__ __launch_bounds__(256) void fm_gate_up_swiglu(DecodeArgs a) {
     }
 }
 
-// ---------------------------------------------------------------- kernel 2
-// The last workgroup of a layer to finish its down rows (arrival counter) sums
-// the K per-expert vectors in slot order, so the result does not depend on
-// which workgroup that is.
+// ---------------------------------------------------------------- kernel 3
+// out[l][j] = sum_k w[l][k] * expert_out[l][k][j], k in slot order
+// (finchmoe/shaders.metal:2213-2228).  GUARD adds the CPU path's finite check
+// and renormalisation (finchmoe/infer.m:10190-10204); it needs the whole
+// vector of each expert, so one workgroup covers a layer.
 template <bool GUARD>
-__device__ void fm_combine_layer(const DecodeArgs &a, int l, float *red) {
+__global__ __launch_bounds__(256) void fm_combine(DecodeArgs a) {
+    __shared__ float red[4];
+    const int l = blockIdx.x;
     const int H = a.g.hidden, K = a.K;
     const float *eo = a.expert_out + (size_t)l * K * H;
     float wk[FM_MAX_K];
     float total = 0.0f;
-    for (int k = 0; k < K; k++) {
-        float w = a.w[l * K + k];
-        if ((unsigned)a.idx[l * K + k] >= (unsigned)a.g.n_experts) w = 0.0f;
-        if constexpr (GUARD) {
-            // finchmoe/infer.m:10190-10196: keep the expert iff sum(out^2) is
-            // finite and < 1e20
-            float part = 0.0f;
-            for (int j = threadIdx.x; j < H; j += blockDim.x) {
-                float v = eo[(size_t)k * H + j];
-                part = fmaf(v, v, part);
+#pragma unroll
+    for (int k = 0; k < FM_MAX_K; k++) {
+        float w = 0.0f;
+        if (k < K) {
+            w = a.w[l * K + k];
+            if ((unsigned)a.idx[l * K + k] >= (unsigned)a.g.n_experts) w = 0.0f;
+            if constexpr (GUARD) {
+                float part = 0.0f;
+                for (int j = threadIdx.x; j < H; j += blockDim.x) {
+                    float v = eo[(size_t)k * H + j];
+                    part = fmaf(v, v, part);
+                }
+                part = fm_group_sum<64>(part);
+                __syncthreads();
+                if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
+                __syncthreads();
+                float er = red[0] + red[1] + red[2] + red[3];
+                bool keep = isfinite(er) && er < 1e20f;
+                if (keep) total += w; else w = 0.0f;
             }
-            part = fm_group_sum<64>(part);
-            __syncthreads();
-            if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
-            __syncthreads();
-            float er = red[0] + red[1] + red[2] + red[3];
-            bool keep = isfinite(er) && er < 1e20f;
-            if (keep) total += w; else w = 0.0f;
         }
         wk[k] = w;
     }
     float rn = 1.0f;
     if constexpr (GUARD) {
-        if (total > 0.0f && total < 0.99f) rn = 1.0f / total;   // infer.m:10200-10204
+        if (total > 0.0f && total < 0.99f) rn = 1.0f / total;
     }
     float *out = a.out + (size_t)l * H;
-    for (int j = threadIdx.x; j < H; j += blockDim.x) {
+    const int j0 = GUARD ? 0 : blockIdx.y * blockDim.x;
+    const int j1 = GUARD ? H : min(H, j0 + (int)blockDim.x);
+    for (int j = j0 + threadIdx.x; j < j1; j += blockDim.x) {
         float acc = 0.0f;
-        for (int k = 0; k < K; k++)
-            if (wk[k] != 0.0f) acc += wk[k] * eo[(size_t)k * H + j];
+#pragma unroll
+        for (int k = 0; k < FM_MAX_K; k++)
+            if (k < K && wk[k] != 0.0f) acc += wk[k] * eo[(size_t)k * H + j];
         if constexpr (GUARD) acc *= rn;
         out[j] = (a.flags & FM_ACCUMULATE) ? out[j] + acc : acc;
     }
 }
 
+// ---------------------------------------------------------------- kernel 2
 template <int BITS, int LPR, bool FP16>
-__global__ __launch_bounds__(256) void fm_down_combine(DecodeArgs a) {
+__global__ __launch_bounds__(256) void fm_down(DecodeArgs a) {
     constexpr int RPS = FM_WAVE / LPR;
     constexpr int BPL = FmLaneBytes<BITS>::value;
-    __shared__ float red[4];
-    __shared__ int s_last;
     const int item = blockIdx.x;
     const int pair = item / a.items_per_pair;
     const int chunk = item - pair * a.items_per_pair;
@@ -181,21 +188,6 @@ __global__ __launch_bounds__(256) void fm_down_combine(DecodeArgs a) {
         }
     }
 
-    // arrival: make this workgroup's rows visible device-wide, then count
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned total = (unsigned)(a.K * a.items_per_pair);
-        unsigned old = atomicAdd(&a.counters[l], 1u);
-        s_last = (old == total - 1u);
-    }
-    __syncthreads();
-    if (s_last) {
-        __threadfence();
-        if (a.flags & FM_GUARD) fm_combine_layer<true>(a, l, red);
-        else fm_combine_layer<false>(a, l, red);
-        if (threadIdx.x == 0) a.counters[l] = 0u;
-    }
 }
 
 template <int BITS, bool FP16>
@@ -211,7 +203,7 @@ int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down,
 #define FM_UP(L) \
     hipLaunchKernelGGL((fm_gate_up_swiglu<BITS, L, FP16>), dim3(n_pairs * a1.items_per_pair), b, 0, st, a1)
 #define FM_DOWN(L) \
-    hipLaunchKernelGGL((fm_down_combine<BITS, L, FP16>), dim3(n_pairs * a2.items_per_pair), b, 0, st, a2)
+    hipLaunchKernelGGL((fm_down<BITS, L, FP16>), dim3(n_pairs * a2.items_per_pair), b, 0, st, a2)
     if (kev) (void)hipEventRecord(kev[0], st);
     switch (lpr_up) {
         case 4: FM_UP(4); break;
@@ -231,6 +223,11 @@ int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down,
     }
 #undef FM_UP
 #undef FM_DOWN
+    const int n_groups = n_pairs / a.K;
+    if (a.flags & FM_GUARD)
+        hipLaunchKernelGGL(fm_combine<true>, dim3(n_groups), b, 0, st, a);
+    else
+        hipLaunchKernelGGL(fm_combine<false>, dim3(n_groups, (a.g.hidden + 255) / 256), b, 0, st, a);
     if (kev) (void)hipEventRecord(kev[2], st);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
@@ -269,7 +266,7 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     a.act = d_act;
     a.expert_out = d_expert_out;
     a.out = d_out;
-    a.counters = d_counters;
+    (void)d_counters;
     a.flags = flags;
     a.rows_per_item = a.items_per_pair = 0;
     const int n_pairs = n_layers * K;
