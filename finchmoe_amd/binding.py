@@ -26,7 +26,8 @@ class FinchError(RuntimeError):
 
 
 def lib_path():
-    return os.path.join(_HERE, "libfinchhip.so")
+    """In-tree library; FINCH_HIP_LIB overrides the path (alternative builds)."""
+    return os.environ.get("FINCH_HIP_LIB") or os.path.join(_HERE, "libfinchhip.so")
 
 
 _LIB = None

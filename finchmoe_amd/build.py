@@ -27,7 +27,11 @@ def _stale(target, deps):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def build(force=False, verbose=False):
+def build(force=False, verbose=False, extra_flags=(), lib=None):
+    """extra_flags / lib: alternative builds (experiments) into another file."""
+    global LIB
+    if lib:
+        LIB, force = lib, True
     deps = [os.path.join(CSRC, f) for f in os.listdir(CSRC)]
     deps.append(os.path.join(HERE, "..", "include", "finch_hip.h"))
     if force or _stale(LIB, deps):
@@ -35,9 +39,9 @@ def build(force=False, verbose=False):
         procs = []
         os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
         for src in SOURCES:
-            obj = os.path.join(HERE, "build", src.replace(".hip", ".o"))
+            obj = os.path.join(HERE, "build", ("alt_" if lib else "") + src.replace(".hip", ".o"))
             objs.append(obj)
-            cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+            cmd = [HIPCC] + FLAGS + list(extra_flags) + ["-c", os.path.join(CSRC, src), "-o", obj]
             if verbose:
                 print(" ".join(cmd))
             procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE,
@@ -53,7 +57,7 @@ def build(force=False, verbose=False):
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
         subprocess.check_call(cmd)
     host_src = os.path.join(HERE, "host", "finch_ops.c")
-    if os.path.exists(host_src) and (force or _stale(HOSTLIB, [host_src, os.path.join(HERE, "host", "finch_ops.h")])):
+    if not lib and os.path.exists(host_src) and (force or _stale(HOSTLIB, [host_src, os.path.join(HERE, "host", "finch_ops.h")])):
         subprocess.check_call(["gcc", "-O2", "-std=c99", "-fPIC", "-shared", "-Wall",
                                "-I", os.path.join(HERE, "..", "include"),
                                "-o", HOSTLIB, host_src, "-L", HERE, "-lfinchhip",

@@ -15,7 +15,7 @@
 //   down    (in 512):   4 lanes x 48 B = one 192-byte row, 16 rows per step
 // The scales (and biases) of those rows are contiguous too — [rows][groups]
 // 16-bit, two groups per lane = one dword per lane.
-#include "fm_unpack.h"
+#include "fm_mfma.h"
 
 namespace {
 
@@ -190,8 +190,168 @@ __global__ __launch_bounds__(256) void fm_down(DecodeArgs a) {
 
 }
 
+// ======================================================================
+// Matrix-core path (fm_mfma.h): persistent waves over a static partition.
+//
+// All row steps of all pairs form one sequence of "units" (a unit = one wave
+// step = 64/LPR rows of one pair).  The launch has a fixed number of waves;
+// wave w takes the contiguous unit range [U*w/W, U*(w+1)/W) and streams
+// through it with the next unit's loads in flight, so a wave reads tens of
+// kilobytes back to back instead of a few rows, and every wave ends after its
+// own range (no queue, no spinning).  The activation registers are rebuilt
+// only when the range crosses into another layer (gate/up) or pair (down).
+// ======================================================================
+template <int BITS>
+struct FmUnitPtrs {
+    const uint8_t *w, *s, *b;
+};
+
+template <int BITS, int LPR>
+__device__ __forceinline__ void fm_unit_lane_offsets(int lane, int row_bytes, int sb_row_bytes,
+                                                     size_t &woff, size_t &soff, int &row_in_step,
+                                                     int &ch) {
+    const int j = lane & 3;
+    ch = (lane >> 2) % LPR;
+    const int rq = lane / (4 * LPR);
+    row_in_step = 4 * rq + j;
+    woff = (size_t)row_in_step * row_bytes + (size_t)ch * FmLaneBytes<BITS>::value;
+    soff = (size_t)row_in_step * sb_row_bytes + (size_t)ch * 4;
+}
+
+// gate + up + SwiGLU
+template <int BITS, int LPR, bool FP16>
+__global__ __launch_bounds__(256) void fm_gate_up_swiglu_mfma(DecodeArgs a) {
+    constexpr int RPS = FM_WAVE / LPR;
+    const int lane = threadIdx.x & 63;
+    const int wid = blockIdx.x * 4 + (threadIdx.x >> 6), nw = gridDim.x * 4;
+    const int n_pairs = a.items_per_pair;            // reused field: number of pairs
+    const int upp = a.g.inter / RPS;                 // units per pair
+    const long total = (long)n_pairs * upp;
+    long u = total * wid / nw;
+    const long u_end = total * (wid + 1) / nw;
+    if (u >= u_end) return;
+    const int row_bytes = a.g.hidden * BITS / 8, sb_row_bytes = (a.g.hidden / 64) * 2;
+    size_t woff, soff;
+    int ris, ch;
+    fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff, soff, ris, ch);
+    const size_t wstep = (size_t)RPS * row_bytes, sstep = (size_t)RPS * sb_row_bytes;
+
+    int pair = (int)(u / upp), rstep = (int)(u - (long)pair * upp);
+    // state of the unit being loaded ("n") and of the unit being computed ("c")
+    auto blob_of = [&](int p) -> const uint8_t * {
+        int e = a.idx[p];
+        if ((unsigned)e >= (unsigned)a.g.n_experts) return nullptr;
+        return a.layer_ptrs[a.layer0 + (p / a.K) * a.layer_stride] + (size_t)e * a.g.expert_size;
+    };
+    const uint8_t *blob_n = blob_of(pair);
+    FmRowSlice<BITS> gcur, ucur, gnext, unext;
+    auto load_unit = [&](const uint8_t *blob, int rs, FmRowSlice<BITS> &gs, FmRowSlice<BITS> &us) {
+        if (blob) {
+            size_t wo = woff + (size_t)rs * wstep, so = soff + (size_t)rs * sstep;
+            fm_load_slice<BITS>(gs, blob + a.g.gate_w + wo, blob + a.g.gate_s + so,
+                                blob + a.g.gate_b + so);
+            fm_load_slice<BITS>(us, blob + a.g.up_w + wo, blob + a.g.up_s + so,
+                                blob + a.g.up_b + so);
+        }
+    };
+    load_unit(blob_n, rstep, gcur, ucur);
+    int pair_c = pair, rstep_c = rstep;
+    const uint8_t *blob_c = blob_n;
+    FmActRegs ar;
+    int layer_c = -1;
+    for (; u < u_end; u++) {
+        // advance the loader one unit ahead
+        rstep++;
+        if (rstep == upp) {
+            rstep = 0;
+            pair++;
+            if (u + 1 < u_end) blob_n = blob_of(pair);
+        }
+        if (u + 1 < u_end) load_unit(blob_n, rstep, gnext, unext);
+        const int l = pair_c / a.K;
+        if (l != layer_c) {
+            fm_build_act<BITS>(a.x + (size_t)l * a.g.hidden + ch * FM_CPL, lane & 3, ar);
+            layer_c = l;
+        }
+        float v = 0.0f;
+        if (blob_c) {
+            float gv = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(gcur, ar));
+            float uv = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(ucur, ar));
+            v = fm_silu_mul(gv, uv);
+        }
+        if (ch == 0) a.act[(size_t)pair_c * a.g.inter + rstep_c * RPS + ris] = v;
+        gcur = gnext;
+        ucur = unext;
+        pair_c = pair;
+        rstep_c = rstep;
+        blob_c = blob_n;
+    }
+}
+
+// down projection -> per-expert output vectors
+template <int BITS, int LPR, bool FP16>
+__global__ __launch_bounds__(256) void fm_down_mfma(DecodeArgs a) {
+    constexpr int RPS = FM_WAVE / LPR;
+    const int lane = threadIdx.x & 63;
+    const int wid = blockIdx.x * 4 + (threadIdx.x >> 6), nw = gridDim.x * 4;
+    const int n_pairs = a.items_per_pair;
+    const int upp = a.g.hidden / RPS;
+    const long total = (long)n_pairs * upp;
+    long u = total * wid / nw;
+    const long u_end = total * (wid + 1) / nw;
+    if (u >= u_end) return;
+    const int row_bytes = a.g.inter * BITS / 8, sb_row_bytes = (a.g.inter / 64) * 2;
+    size_t woff, soff;
+    int ris, ch;
+    fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff, soff, ris, ch);
+    const size_t wstep = (size_t)RPS * row_bytes, sstep = (size_t)RPS * sb_row_bytes;
+
+    int pair = (int)(u / upp), rstep = (int)(u - (long)pair * upp);
+    auto blob_of = [&](int p) -> const uint8_t * {
+        int e = a.idx[p];
+        if ((unsigned)e >= (unsigned)a.g.n_experts) return nullptr;
+        return a.layer_ptrs[a.layer0 + (p / a.K) * a.layer_stride] + (size_t)e * a.g.expert_size;
+    };
+    const uint8_t *blob_n = blob_of(pair);
+    FmRowSlice<BITS> cur, next;
+    auto load_unit = [&](const uint8_t *blob, int rs, FmRowSlice<BITS> &ds) {
+        if (blob) {
+            size_t wo = woff + (size_t)rs * wstep, so = soff + (size_t)rs * sstep;
+            fm_load_slice<BITS>(ds, blob + a.g.down_w + wo, blob + a.g.down_s + so,
+                                blob + a.g.down_b + so);
+        }
+    };
+    load_unit(blob_n, rstep, cur);
+    int pair_c = pair, rstep_c = rstep;
+    const uint8_t *blob_c = blob_n;
+    FmActRegs ar;
+    int pair_x = -1;
+    for (; u < u_end; u++) {
+        rstep++;
+        if (rstep == upp) {
+            rstep = 0;
+            pair++;
+            if (u + 1 < u_end) blob_n = blob_of(pair);
+        }
+        if (u + 1 < u_end) load_unit(blob_n, rstep, next);
+        float v = 0.0f;
+        if (blob_c) {
+            if (pair_c != pair_x) {
+                fm_build_act<BITS>(a.act + (size_t)pair_c * a.g.inter + ch * FM_CPL, lane & 3, ar);
+                pair_x = pair_c;
+            }
+            v = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(cur, ar));
+        }
+        if (ch == 0) a.expert_out[(size_t)pair_c * a.g.hidden + rstep_c * RPS + ris] = v;
+        cur = next;
+        pair_c = pair;
+        rstep_c = rstep;
+        blob_c = blob_n;
+    }
+}
+
 template <int BITS, bool FP16>
-int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down,
+int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down, int n_cu,
                     hipStream_t st, hipEvent_t *kev) {
     DecodeArgs a1 = a, a2 = a;
     a1.rows_per_item = rpi_up;
@@ -200,29 +360,54 @@ int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down,
     a2.items_per_pair = a.g.hidden / rpi_down;
     dim3 b(256);
     const int lpr_up = a.g.hidden / FM_CPL, lpr_down = a.g.inter / FM_CPL;
+    // matrix-core path: one wave per SIMD slot that the register budget allows,
+    // fewer when there are not enough units to give every wave two
+    const bool mfma_up = lpr_up >= 4 && lpr_up <= 16, mfma_down = lpr_down <= 16;
+    auto stream_grid = [&](long units) {
+        long waves = (long)n_cu * 4 * 2;
+        if (units < 2 * waves) waves = (units + 1) / 2;
+        if (waves < 1) waves = 1;
+        return dim3((unsigned)((waves + 3) / 4));
+    };
+    if (kev) (void)hipEventRecord(kev[0], st);
+    if (mfma_up) {
+        DecodeArgs am = a;
+        am.items_per_pair = n_pairs;
+        dim3 g = stream_grid((long)n_pairs * (a.g.inter / (FM_WAVE / lpr_up)));
+#define FM_UPM(L) hipLaunchKernelGGL((fm_gate_up_swiglu_mfma<BITS, L, FP16>), g, b, 0, st, am)
+        switch (lpr_up) {
+            case 4: FM_UPM(4); break;
+            case 8: FM_UPM(8); break;
+            default: FM_UPM(16); break;
+        }
+#undef FM_UPM
+    } else {
 #define FM_UP(L) \
     hipLaunchKernelGGL((fm_gate_up_swiglu<BITS, L, FP16>), dim3(n_pairs * a1.items_per_pair), b, 0, st, a1)
-#define FM_DOWN(L) \
-    hipLaunchKernelGGL((fm_down<BITS, L, FP16>), dim3(n_pairs * a2.items_per_pair), b, 0, st, a2)
-    if (kev) (void)hipEventRecord(kev[0], st);
-    switch (lpr_up) {
-        case 4: FM_UP(4); break;
-        case 8: FM_UP(8); break;
-        case 16: FM_UP(16); break;
-        case 32: FM_UP(32); break;
-        default: return FM_ERR_UNSUPPORTED;
+        switch (lpr_up) {
+            case 32: FM_UP(32); break;
+            default: return FM_ERR_UNSUPPORTED;
+        }
+#undef FM_UP
     }
     if (kev) (void)hipEventRecord(kev[1], st);
-    switch (lpr_down) {
-        case 1: FM_DOWN(1); break;
-        case 2: FM_DOWN(2); break;
-        case 4: FM_DOWN(4); break;
-        case 8: FM_DOWN(8); break;
-        case 16: FM_DOWN(16); break;
-        default: return FM_ERR_UNSUPPORTED;
+    if (mfma_down) {
+        DecodeArgs am = a;
+        am.items_per_pair = n_pairs;
+        dim3 g = stream_grid((long)n_pairs * (a.g.hidden / (FM_WAVE / lpr_down)));
+#define FM_DOWNM(L) hipLaunchKernelGGL((fm_down_mfma<BITS, L, FP16>), g, b, 0, st, am)
+        switch (lpr_down) {
+            case 1: FM_DOWNM(1); break;
+            case 2: FM_DOWNM(2); break;
+            case 4: FM_DOWNM(4); break;
+            case 8: FM_DOWNM(8); break;
+            default: FM_DOWNM(16); break;
+        }
+#undef FM_DOWNM
+    } else {
+        return FM_ERR_UNSUPPORTED;
     }
-#undef FM_UP
-#undef FM_DOWN
+    (void)a2;
     const int n_groups = n_pairs / a.K;
     if (a.flags & FM_GUARD)
         hipLaunchKernelGGL(fm_combine<true>, dim3(n_groups), b, 0, st, a);
@@ -279,12 +464,12 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     const int rpi_up = pick_rows_per_item(g->inter, n_pairs, min_up, 64, want);
     const int rpi_down = pick_rows_per_item(g->hidden, n_pairs, min_down, 256, want);
     if (g->bits == 3) {
-        return g->scale_fp16 ? launch_decode_t<3, true>(a, n_pairs, rpi_up, rpi_down, st, kev)
-                             : launch_decode_t<3, false>(a, n_pairs, rpi_up, rpi_down, st, kev);
+        return g->scale_fp16 ? launch_decode_t<3, true>(a, n_pairs, rpi_up, rpi_down, n_cu, st, kev)
+                             : launch_decode_t<3, false>(a, n_pairs, rpi_up, rpi_down, n_cu, st, kev);
     }
     if (g->bits == 4) {
-        return g->scale_fp16 ? launch_decode_t<4, true>(a, n_pairs, rpi_up, rpi_down, st, kev)
-                             : launch_decode_t<4, false>(a, n_pairs, rpi_up, rpi_down, st, kev);
+        return g->scale_fp16 ? launch_decode_t<4, true>(a, n_pairs, rpi_up, rpi_down, n_cu, st, kev)
+                             : launch_decode_t<4, false>(a, n_pairs, rpi_up, rpi_down, n_cu, st, kev);
     }
     return FM_ERR_UNSUPPORTED;
 }
