@@ -191,21 +191,18 @@ __global__ __launch_bounds__(256) void fm_down(DecodeArgs a) {
 }
 
 // ======================================================================
-// Matrix-core path (fm_mfma.h): persistent waves over a static partition.
+// Matrix-core path (fm_mfma.h): persistent workgroups over a static partition.
 //
 // All row steps of all pairs form one sequence of "units" (a unit = one wave
-// step = 64/LPR rows of one pair).  The launch has a fixed number of waves;
-// wave w takes the contiguous unit range [U*w/W, U*(w+1)/W) and streams
-// through it with the next unit's loads in flight, so a wave reads tens of
-// kilobytes back to back instead of a few rows, and every wave ends after its
-// own range (no queue, no spinning).  The activation registers are rebuilt
-// only when the range crosses into another layer (gate/up) or pair (down).
+// step = 64/LPR rows of one pair).  The launch has a fixed number of
+// workgroups; workgroup g takes the contiguous unit range [U*g/G, U*(g+1)/G),
+// its four waves interleave over it, each with the next unit's loads in
+// flight — so a wave streams tens of kilobytes back to back instead of a few
+// rows, and every wave ends after its own share (no queue, no spinning).
+// A range is cut into segments that share an input vector (a layer for
+// gate/up, a pair for down); per segment the workgroup builds the activation
+// registers once in LDS (fm_build_act_lds) and every wave copies its own.
 // ======================================================================
-template <int BITS>
-struct FmUnitPtrs {
-    const uint8_t *w, *s, *b;
-};
-
 template <int BITS, int LPR>
 __device__ __forceinline__ void fm_unit_lane_offsets(int lane, int row_bytes, int sb_row_bytes,
                                                      size_t &woff, size_t &soff, int &row_in_step,
@@ -218,33 +215,31 @@ __device__ __forceinline__ void fm_unit_lane_offsets(int lane, int row_bytes, in
     soff = (size_t)row_in_step * sb_row_bytes + (size_t)ch * 4;
 }
 
-// gate + up + SwiGLU
+__device__ __forceinline__ const uint8_t *fm_pair_blob(const DecodeArgs &a, int p) {
+    int e = a.idx[p];
+    if ((unsigned)e >= (unsigned)a.g.n_experts) return nullptr;   // treated as weight 0
+    return a.layer_ptrs[a.layer0 + (p / a.K) * a.layer_stride] + (size_t)e * a.g.expert_size;
+}
+
+// gate + up + SwiGLU.  a.items_per_pair carries the number of pairs.
 template <int BITS, int LPR, bool FP16>
 __global__ __launch_bounds__(256) void fm_gate_up_swiglu_mfma(DecodeArgs a) {
     constexpr int RPS = FM_WAVE / LPR;
+    __shared__ FmActLds<LPR> lds;
+    __shared__ const uint8_t *lds_blob[FM_MAX_K];
     const int lane = threadIdx.x & 63;
-    const int wid = blockIdx.x * 4 + (threadIdx.x >> 6), nw = gridDim.x * 4;
-    const int n_pairs = a.items_per_pair;            // reused field: number of pairs
-    const int upp = a.g.inter / RPS;                 // units per pair
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_pairs = a.items_per_pair;
+    const int upp = a.g.inter / RPS;        // units per pair (>= 4)
+    const long upl = (long)upp * a.K;       // units per layer
     const long total = (long)n_pairs * upp;
-    long u = total * wid / nw;
-    const long u_end = total * (wid + 1) / nw;
-    if (u >= u_end) return;
+    const long wg0 = total * blockIdx.x / gridDim.x, wg1 = total * (blockIdx.x + 1) / gridDim.x;
     const int row_bytes = a.g.hidden * BITS / 8, sb_row_bytes = (a.g.hidden / 64) * 2;
     size_t woff, soff;
     int ris, ch;
     fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff, soff, ris, ch);
     const size_t wstep = (size_t)RPS * row_bytes, sstep = (size_t)RPS * sb_row_bytes;
 
-    int pair = (int)(u / upp), rstep = (int)(u - (long)pair * upp);
-    // state of the unit being loaded ("n") and of the unit being computed ("c")
-    auto blob_of = [&](int p) -> const uint8_t * {
-        int e = a.idx[p];
-        if ((unsigned)e >= (unsigned)a.g.n_experts) return nullptr;
-        return a.layer_ptrs[a.layer0 + (p / a.K) * a.layer_stride] + (size_t)e * a.g.expert_size;
-    };
-    const uint8_t *blob_n = blob_of(pair);
-    FmRowSlice<BITS> gcur, ucur, gnext, unext;
     auto load_unit = [&](const uint8_t *blob, int rs, FmRowSlice<BITS> &gs, FmRowSlice<BITS> &us) {
         if (blob) {
             size_t wo = woff + (size_t)rs * wstep, so = soff + (size_t)rs * sstep;
@@ -254,37 +249,49 @@ __global__ __launch_bounds__(256) void fm_gate_up_swiglu_mfma(DecodeArgs a) {
                                 blob + a.g.up_b + so);
         }
     };
-    load_unit(blob_n, rstep, gcur, ucur);
-    int pair_c = pair, rstep_c = rstep;
-    const uint8_t *blob_c = blob_n;
-    FmActRegs ar;
-    int layer_c = -1;
-    for (; u < u_end; u++) {
-        // advance the loader one unit ahead
-        rstep++;
-        if (rstep == upp) {
-            rstep = 0;
-            pair++;
-            if (u + 1 < u_end) blob_n = blob_of(pair);
+
+    for (long seg0 = wg0; seg0 < wg1;) {
+        const int l = (int)(seg0 / upl);
+        long seg1 = (long)(l + 1) * upl;
+        if (seg1 > wg1) seg1 = wg1;
+        __syncthreads();                          // previous segment's readers are done
+        fm_stage_x_lds<LPR>(a.x + (size_t)l * a.g.hidden, lds);
+        if (threadIdx.x < a.K) lds_blob[threadIdx.x] = fm_pair_blob(a, l * a.K + threadIdx.x);
+        __syncthreads();
+        // loader state: unit un = (pair pn, row step rsn) of this wave, one step ahead
+        long u = seg0 + wave;
+        int pn = (int)(u / upp) - l * a.K, rsn = (int)(u % upp);
+        const uint8_t *blob_n = u < seg1 ? lds_blob[pn] : nullptr;
+        FmRowSlice<BITS> gcur, ucur, gnext, unext;
+        if (u < seg1) load_unit(blob_n, rsn, gcur, ucur);   // in flight during the build
+        fm_build_act_lds<BITS, LPR>(lds);
+        __syncthreads();
+        FmActRegs ar;
+        fm_read_act_lds<LPR>(lds, lane, ar);
+        const uint8_t *blob_c = blob_n;
+        for (; u < seg1; u += 4) {
+            if (u + 4 < seg1) {
+                rsn += 4;
+                if (rsn >= upp) {
+                    rsn -= upp;
+                    pn++;
+                    blob_n = lds_blob[pn];
+                }
+                load_unit(blob_n, rsn, gnext, unext);
+            }
+            float v = 0.0f;
+            if (blob_c) {
+                float gv = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(gcur, ar));
+                float uv = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(ucur, ar));
+                v = fm_silu_mul(gv, uv);
+            }
+            // unit u = (pair, row step): act is [pair][inter], rows are contiguous
+            if (ch == 0) a.act[(size_t)u * RPS + ris] = v;
+            gcur = gnext;
+            ucur = unext;
+            blob_c = blob_n;
         }
-        if (u + 1 < u_end) load_unit(blob_n, rstep, gnext, unext);
-        const int l = pair_c / a.K;
-        if (l != layer_c) {
-            fm_build_act<BITS>(a.x + (size_t)l * a.g.hidden + ch * FM_CPL, lane & 3, ar);
-            layer_c = l;
-        }
-        float v = 0.0f;
-        if (blob_c) {
-            float gv = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(gcur, ar));
-            float uv = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(ucur, ar));
-            v = fm_silu_mul(gv, uv);
-        }
-        if (ch == 0) a.act[(size_t)pair_c * a.g.inter + rstep_c * RPS + ris] = v;
-        gcur = gnext;
-        ucur = unext;
-        pair_c = pair;
-        rstep_c = rstep;
-        blob_c = blob_n;
+        seg0 = seg1;
     }
 }
 
@@ -292,61 +299,53 @@ __global__ __launch_bounds__(256) void fm_gate_up_swiglu_mfma(DecodeArgs a) {
 template <int BITS, int LPR, bool FP16>
 __global__ __launch_bounds__(256) void fm_down_mfma(DecodeArgs a) {
     constexpr int RPS = FM_WAVE / LPR;
+    __shared__ FmActLds<LPR> lds;
     const int lane = threadIdx.x & 63;
-    const int wid = blockIdx.x * 4 + (threadIdx.x >> 6), nw = gridDim.x * 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_pairs = a.items_per_pair;
     const int upp = a.g.hidden / RPS;
     const long total = (long)n_pairs * upp;
-    long u = total * wid / nw;
-    const long u_end = total * (wid + 1) / nw;
-    if (u >= u_end) return;
+    const long wg0 = total * blockIdx.x / gridDim.x, wg1 = total * (blockIdx.x + 1) / gridDim.x;
     const int row_bytes = a.g.inter * BITS / 8, sb_row_bytes = (a.g.inter / 64) * 2;
     size_t woff, soff;
     int ris, ch;
     fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff, soff, ris, ch);
     const size_t wstep = (size_t)RPS * row_bytes, sstep = (size_t)RPS * sb_row_bytes;
 
-    int pair = (int)(u / upp), rstep = (int)(u - (long)pair * upp);
-    auto blob_of = [&](int p) -> const uint8_t * {
-        int e = a.idx[p];
-        if ((unsigned)e >= (unsigned)a.g.n_experts) return nullptr;
-        return a.layer_ptrs[a.layer0 + (p / a.K) * a.layer_stride] + (size_t)e * a.g.expert_size;
-    };
-    const uint8_t *blob_n = blob_of(pair);
-    FmRowSlice<BITS> cur, next;
-    auto load_unit = [&](const uint8_t *blob, int rs, FmRowSlice<BITS> &ds) {
-        if (blob) {
-            size_t wo = woff + (size_t)rs * wstep, so = soff + (size_t)rs * sstep;
+    for (long seg0 = wg0; seg0 < wg1;) {
+        const int p = (int)(seg0 / upp);
+        long seg1 = (long)(p + 1) * upp;
+        if (seg1 > wg1) seg1 = wg1;
+        const uint8_t *blob = fm_pair_blob(a, p);
+        long u = seg0 + wave;
+        int rs = (int)(u - (long)p * upp);
+        auto load_unit = [&](int r, FmRowSlice<BITS> &ds) {
+            size_t wo = woff + (size_t)r * wstep, so = soff + (size_t)r * sstep;
             fm_load_slice<BITS>(ds, blob + a.g.down_w + wo, blob + a.g.down_s + so,
                                 blob + a.g.down_b + so);
-        }
-    };
-    load_unit(blob_n, rstep, cur);
-    int pair_c = pair, rstep_c = rstep;
-    const uint8_t *blob_c = blob_n;
-    FmActRegs ar;
-    int pair_x = -1;
-    for (; u < u_end; u++) {
-        rstep++;
-        if (rstep == upp) {
-            rstep = 0;
-            pair++;
-            if (u + 1 < u_end) blob_n = blob_of(pair);
-        }
-        if (u + 1 < u_end) load_unit(blob_n, rstep, next);
-        float v = 0.0f;
-        if (blob_c) {
-            if (pair_c != pair_x) {
-                fm_build_act<BITS>(a.act + (size_t)pair_c * a.g.inter + ch * FM_CPL, lane & 3, ar);
-                pair_x = pair_c;
+        };
+        __syncthreads();
+        if (blob) {
+            fm_stage_x_lds<LPR>(a.act + (size_t)p * a.g.inter, lds);
+            FmRowSlice<BITS> cur, next;
+            if (u < seg1) load_unit(rs, cur);
+            __syncthreads();
+            fm_build_act_lds<BITS, LPR>(lds);
+            __syncthreads();
+            FmActRegs ar;
+            fm_read_act_lds<LPR>(lds, lane, ar);
+            for (; u < seg1; u += 4) {
+                rs += 4;
+                if (u + 4 < seg1) load_unit(rs, next);
+                float v = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(cur, ar));
+                if (ch == 0) a.expert_out[(size_t)u * RPS + ris] = v;
+                cur = next;
             }
-            v = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(cur, ar));
+        } else {
+            for (; u < seg1; u += 4)
+                if (ch == 0) a.expert_out[(size_t)u * RPS + ris] = 0.0f;
         }
-        if (ch == 0) a.expert_out[(size_t)pair_c * a.g.hidden + rstep_c * RPS + ris] = v;
-        cur = next;
-        pair_c = pair;
-        rstep_c = rstep;
-        blob_c = blob_n;
+        seg0 = seg1;
     }
 }
 
@@ -363,11 +362,13 @@ int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down, 
     // matrix-core path: one wave per SIMD slot that the register budget allows,
     // fewer when there are not enough units to give every wave two
     const bool mfma_up = lpr_up >= 4 && lpr_up <= 16, mfma_down = lpr_down <= 16;
+    // two workgroups per CU (register budget); fewer when the launch has too few
+    // units to give every wave two
     auto stream_grid = [&](long units) {
-        long waves = (long)n_cu * 4 * 2;
-        if (units < 2 * waves) waves = (units + 1) / 2;
-        if (waves < 1) waves = 1;
-        return dim3((unsigned)((waves + 3) / 4));
+        long wgs = (long)n_cu * 2;
+        if (units < 8 * wgs) wgs = (units + 7) / 8;
+        if (wgs < 1) wgs = 1;
+        return dim3((unsigned)wgs);
     };
     if (kev) (void)hipEventRecord(kev[0], st);
     if (mfma_up) {

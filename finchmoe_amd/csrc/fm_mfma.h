@@ -104,32 +104,35 @@ __device__ __forceinline__ uint32_t fm_window(const uint32_t *g) {
 }
 
 // pair P of a group as two bf16 values 1 + q * 2^t / 128
+// `ones` = 0x3F803F80 held in a vector register: V_AND_OR_B32 has no room for
+// two literals, with the constant in a register the mask can come from an SGPR
 template <int BITS, int P>
-__device__ __forceinline__ uint32_t fm_pair(const uint32_t *g) {
+__device__ __forceinline__ uint32_t fm_pair(const uint32_t *g, uint32_t ones) {
     using T = FmPairs<BITS>;
     uint32_t w = fm_window<T::start(P), T::GROUP_DWORDS>(g);
-    return (w & T::mask(P)) | 0x3F803F80u;   // v_and_or_b32
+    return (w & T::mask(P)) | ones;   // v_and_or_b32
 }
 
 // One group (64 codes) of one row against the lane's activation registers:
 // 16 MFMAs, each taking two pairs.  acc register i accumulates piece i.
 template <int BITS, int M>
 __device__ __forceinline__ void fm_group_mfma_steps(const uint32_t *g, const uint32_t *a,
-                                                    fm_f4 &acc) {
+                                                    uint32_t ones, fm_f4 &acc) {
     if constexpr (M < 16) {
-        uint32_t b0 = fm_pair<BITS, 2 * M>(g), b1 = fm_pair<BITS, 2 * M + 1>(g);
+        uint32_t b0 = fm_pair<BITS, 2 * M>(g, ones), b1 = fm_pair<BITS, 2 * M + 1>(g, ones);
         fm_s4 bv = __builtin_bit_cast(fm_s4, make_uint2(b0, b1));
         fm_s4 av = __builtin_bit_cast(fm_s4, make_uint2(a[2 * M], a[2 * M + 1]));
         acc = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av, bv, acc, 0, 0, 0);
-        fm_group_mfma_steps<BITS, M + 1>(g, a, acc);
+        fm_group_mfma_steps<BITS, M + 1>(g, a, ones, acc);
     }
 }
 
 // Per-lane activation state for one 128-column chunk.
 struct FmActRegs {
-    uint32_t a[2][32];   // [group][2 * mfma + half]: bf16 pairs of this lane's piece
-    float xsum[2];       // plain sum of x over each group
-    float xoff[2];       // sum of scale_k * x_k over each group (what the "1 +" adds)
+    uint32_t a[64];   // [32 * group + pair]: bf16 pairs of this lane's piece
+    float xsum[2];    // plain sum of x over each group
+    float xoff[2];    // sum of scale_k * x_k over each group (what the "1 +" adds)
+    uint32_t ones;    // bf16 pair (1.0, 1.0), kept in a register for V_AND_OR_B32
 };
 
 // bf16 piece `piece` (0, 1, 2; 3 -> zero) of v: truncations of the running remainder
@@ -143,25 +146,91 @@ __device__ __forceinline__ uint32_t fm_bf16_piece(float v, int piece) {
     return piece >= 3 ? 0u : bits;
 }
 
-template <int BITS, int G, int P>
-__device__ __forceinline__ void fm_build_act_pairs(const float *x, int piece, FmActRegs &ar) {
-    if constexpr (P < 32) {
-        using T = FmPairs<BITS>;
-        float xl = x[64 * G + T::lo(P)], xh = x[64 * G + T::hi(P)];
-        float sl = xl * fm_pair_scale_lo<BITS>(P), sh = xh * fm_pair_scale_hi<BITS>(P);
-        ar.xsum[G] += xl + xh;
-        ar.xoff[G] += sl + sh;
-        ar.a[G][P] = fm_bf16_piece(sl, piece) | (fm_bf16_piece(sh, piece) << 16);
-        fm_build_act_pairs<BITS, G, P + 1>(x, piece, ar);
+// LDS image of the activation registers of every (chunk, piece) of one input
+// vector, built once per workgroup and read by all its waves.
+//   x   [128*LPR] float   : the input vector, staged with coalesced loads
+//   a   [16][4*LPR] uint4 : register quad q of entry e = 4*chunk + piece (lane-major,
+//                           so a wave's read of one quad is conflict free)
+//   sum [LPR] float4      : xsum0, xsum1, xoff0, xoff1 of each chunk
+template <int LPR>
+struct FmActLds {
+    float x[FM_CPL * LPR];
+    uint4 a[16][4 * LPR];
+    float4 sum[LPR];
+};
+
+// step 1 (all 256 threads): global x -> LDS; caller barriers afterwards
+template <int LPR>
+__device__ __forceinline__ void fm_stage_x_lds(const float *x, FmActLds<LPR> &L) {
+    const float4 *src = reinterpret_cast<const float4 *>(x);
+    float4 *dst = reinterpret_cast<float4 *>(L.x);
+#pragma unroll
+    for (int i = 0; i < (FM_CPL * LPR / 4 + 255) / 256; i++) {
+        int k = threadIdx.x + 256 * i;
+        if (k < FM_CPL * LPR / 4) dst[k] = src[k];
     }
 }
 
-// x points at the lane's 128 activations (fp32, global or LDS)
-template <int BITS>
-__device__ __forceinline__ void fm_build_act(const float *x, int piece, FmActRegs &ar) {
-    ar.xsum[0] = ar.xsum[1] = ar.xoff[0] = ar.xoff[1] = 0.0f;
-    fm_build_act_pairs<BITS, 0, 0>(x, piece, ar);
-    fm_build_act_pairs<BITS, 1, 0>(x, piece, ar);
+// step 2 (all 256 threads, after the barrier): LDS x -> register image + sums;
+// caller barriers afterwards
+template <int BITS, int LPR>
+__device__ __forceinline__ void fm_build_act_lds(FmActLds<LPR> &L) {
+    using T = FmPairs<BITS>;
+    constexpr int NE = 4 * LPR;
+    uint32_t *flat = reinterpret_cast<uint32_t *>(L.a);
+#pragma unroll 4
+    for (int d = threadIdx.x; d < NE * 64; d += 256) {
+        const int e = d >> 6, w = d & 63;
+        const int ch = e >> 2, piece = e & 3, G = w >> 5, P = w & 31;
+        const float *xc = L.x + ch * FM_CPL + 64 * G;
+        float sl = xc[T::lo(P)] * fm_pair_scale_lo<BITS>(P);
+        float sh = xc[T::hi(P)] * fm_pair_scale_hi<BITS>(P);
+        flat[((w >> 2) * NE + e) * 4 + (w & 3)] =
+            fm_bf16_piece(sl, piece) | (fm_bf16_piece(sh, piece) << 16);
+    }
+    // sums: 8 threads per (chunk, group), 4 pairs each
+    {
+        const int combo = threadIdx.x >> 3, sub = threadIdx.x & 7;
+        float xs = 0.0f, xo = 0.0f;
+        if (combo < 2 * LPR) {
+            const float *xc = L.x + (combo >> 1) * FM_CPL + 64 * (combo & 1);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int P = 4 * sub + i;
+                float xl = xc[T::lo(P)], xh = xc[T::hi(P)];
+                xs += xl + xh;
+                xo += xl * fm_pair_scale_lo<BITS>(P) + xh * fm_pair_scale_hi<BITS>(P);
+            }
+        }
+        xs = fm_group_sum<8>(xs);
+        xo = fm_group_sum<8>(xo);
+        if (combo < 2 * LPR && sub == 0) {
+            float *sp = reinterpret_cast<float *>(&L.sum[combo >> 1]);
+            sp[combo & 1] = xs;
+            sp[2 + (combo & 1)] = xo;
+        }
+    }
+}
+
+// lane = lane id in the wave; its entry is (lane % (4*LPR))
+template <int LPR>
+__device__ __forceinline__ void fm_read_act_lds(const FmActLds<LPR> &L, int lane, FmActRegs &ar) {
+    constexpr int NE = 4 * LPR;
+    const int e = lane % NE;
+#pragma unroll
+    for (int q = 0; q < 16; q++) {
+        uint4 v = L.a[q][e];
+        ar.a[4 * q + 0] = v.x;
+        ar.a[4 * q + 1] = v.y;
+        ar.a[4 * q + 2] = v.z;
+        ar.a[4 * q + 3] = v.w;
+    }
+    float4 sm = L.sum[e >> 2];
+    ar.xsum[0] = sm.x;
+    ar.xsum[1] = sm.y;
+    ar.xoff[0] = sm.z;
+    ar.xoff[1] = sm.w;
+    ar.ones = fm_opaque(0x3F803F80u);
 }
 
 // dot product of the lane's 128 codes of one row with the activation, scale and
@@ -173,8 +242,8 @@ __device__ __forceinline__ float fm_lane_dot_mfma(const FmRowSlice<BITS> &rs,
     const uint32_t *d = reinterpret_cast<const uint32_t *>(rs.q);
     fm_f4 acc0 = {-ar.xoff[0], 0.0f, 0.0f, 0.0f};
     fm_f4 acc1 = {-ar.xoff[1], 0.0f, 0.0f, 0.0f};
-    fm_group_mfma_steps<BITS, 0>(d, ar.a[0], acc0);
-    fm_group_mfma_steps<BITS, 0>(d + GD, ar.a[1], acc1);
+    fm_group_mfma_steps<BITS, 0>(d, ar.a, ar.ones, acc0);
+    fm_group_mfma_steps<BITS, 0>(d + GD, ar.a + 32, ar.ones, acc1);
     float d0 = (acc0[0] + acc0[1]) + acc0[2];
     float d1 = (acc1[0] + acc1[1]) + acc1[2];
     float r = fm_widen_lo<FP16>(rs.s) * d0;

@@ -61,6 +61,8 @@ __host__ __device__ constexpr int fm_col_shift(int j) {
     return (j & 1) ? 4 : 0;
 }
 
+typedef uint32_t fm_u4 __attribute__((ext_vector_type(4)));
+
 template <int BITS> struct FmLaneBytes;
 template <> struct FmLaneBytes<3> { static constexpr int value = 48; };
 template <> struct FmLaneBytes<4> { static constexpr int value = 64; };
@@ -71,18 +73,23 @@ template <> struct FmLaneBytes<8> { static constexpr int value = 128; };
 template <int BITS>
 struct FmRowSlice {
     static constexpr int NQ = FmLaneBytes<BITS>::value / 16;
-    uint4 q[NQ];
+    fm_u4 q[NQ];
     uint32_t s, b;
 };
 
 template <int BITS>
 __device__ __forceinline__ void fm_load_slice(FmRowSlice<BITS> &rs, const uint8_t *w,
                                               const uint8_t *s, const uint8_t *b) {
-    const uint4 *wp = reinterpret_cast<const uint4 *>(w);
+    // weights always live in device memory: say so, or a pointer that passed
+    // through LDS is loaded with FLAT instructions, which also count as LDS
+    // traffic and stall the compute on the prefetch
+    typedef const __attribute__((address_space(1))) fm_u4 *gq_t;
+    typedef const __attribute__((address_space(1))) uint32_t *gd_t;
+    gq_t wp = (gq_t)(uintptr_t)w;
 #pragma unroll
     for (int i = 0; i < FmRowSlice<BITS>::NQ; i++) rs.q[i] = wp[i];
-    rs.s = *reinterpret_cast<const uint32_t *>(s);
-    rs.b = *reinterpret_cast<const uint32_t *>(b);
+    rs.s = *(gd_t)(uintptr_t)s;
+    rs.b = *(gd_t)(uintptr_t)b;
 }
 
 // float of byte BYTE of v (v_cvt_f32_ubyteN).  The callers hide their masked
