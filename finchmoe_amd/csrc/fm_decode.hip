@@ -221,9 +221,25 @@ __device__ __forceinline__ const uint8_t *fm_pair_blob(const DecodeArgs &a, int 
     return a.layer_ptrs[a.layer0 + (p / a.K) * a.layer_stride] + (size_t)e * a.g.expert_size;
 }
 
+// A pointer every lane of the wave agrees on, moved to scalar registers so the
+// loads can use the scalar-base + 32-bit lane offset addressing form.
+__device__ __forceinline__ const uint8_t *fm_uniform(const uint8_t *p) {
+    uintptr_t v = (uintptr_t)p;
+    uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const uint8_t *)(((uintptr_t)hi << 32) | lo);
+}
+
 // gate + up + SwiGLU.  a.items_per_pair carries the number of pairs.
+//
+// Pipeline: the wave walks "half steps" — gate rows of a unit, then up rows of
+// the same unit — through a ring of three register slices: while slice k is
+// being multiplied, the loads of the next two half steps are in flight (a full
+// unit, ~6.6 KB per wave).  The loop is unrolled by three units so the ring
+// rotates without register copies.
 template <int BITS, int LPR, bool FP16>
-__global__ __launch_bounds__(256) void fm_gate_up_swiglu_mfma(DecodeArgs a) {
+__global__ __launch_bounds__(256)
+void fm_gate_up_swiglu_mfma(DecodeArgs a) {
     constexpr int RPS = FM_WAVE / LPR;
     __shared__ FmActLds<LPR> lds;
     __shared__ const uint8_t *lds_blob[FM_MAX_K];
@@ -235,69 +251,99 @@ __global__ __launch_bounds__(256) void fm_gate_up_swiglu_mfma(DecodeArgs a) {
     const long total = (long)n_pairs * upp;
     const long wg0 = total * blockIdx.x / gridDim.x, wg1 = total * (blockIdx.x + 1) / gridDim.x;
     const int row_bytes = a.g.hidden * BITS / 8, sb_row_bytes = (a.g.hidden / 64) * 2;
-    size_t woff, soff;
+    size_t woff_, soff_;
     int ris, ch;
-    fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff, soff, ris, ch);
-    const size_t wstep = (size_t)RPS * row_bytes, sstep = (size_t)RPS * sb_row_bytes;
-
-    auto load_unit = [&](const uint8_t *blob, int rs, FmRowSlice<BITS> &gs, FmRowSlice<BITS> &us) {
-        if (blob) {
-            size_t wo = woff + (size_t)rs * wstep, so = soff + (size_t)rs * sstep;
-            fm_load_slice<BITS>(gs, blob + a.g.gate_w + wo, blob + a.g.gate_s + so,
-                                blob + a.g.gate_b + so);
-            fm_load_slice<BITS>(us, blob + a.g.up_w + wo, blob + a.g.up_s + so,
-                                blob + a.g.up_b + so);
-        }
-    };
+    fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff_, soff_, ris, ch);
+    const uint32_t woff = (uint32_t)woff_, soff = (uint32_t)soff_;
+    const uint32_t wstep = (uint32_t)(RPS * row_bytes), sstep = (uint32_t)(RPS * sb_row_bytes);
+    FmBuildSlot<BITS> bslot;
+    bslot.init();
 
     for (long seg0 = wg0; seg0 < wg1;) {
         const int l = (int)(seg0 / upl);
         long seg1 = (long)(l + 1) * upl;
         if (seg1 > wg1) seg1 = wg1;
         __syncthreads();                          // previous segment's readers are done
-        fm_stage_x_lds<LPR>(a.x + (size_t)l * a.g.hidden, lds);
         if (threadIdx.x < a.K) lds_blob[threadIdx.x] = fm_pair_blob(a, l * a.K + threadIdx.x);
         __syncthreads();
-        // loader state: unit un = (pair pn, row step rsn) of this wave, one step ahead
-        long u = seg0 + wave;
-        int pn = (int)(u / upp) - l * a.K, rsn = (int)(u % upp);
-        const uint8_t *blob_n = u < seg1 ? lds_blob[pn] : nullptr;
-        FmRowSlice<BITS> gcur, ucur, gnext, unext;
-        if (u < seg1) load_unit(blob_n, rsn, gcur, ucur);   // in flight during the build
-        fm_build_act_lds<BITS, LPR>(lds);
+        // loader: half step (pair pn, row step rsn, matrix hn) of this wave
+        long u = seg0 + wave;          // unit being computed
+        long un = u;                   // unit being loaded
+        int pn = (int)(u / upp) - l * a.K, rsn = (int)(u % upp), hn = 0;
+        const uint8_t *blob_n = un < seg1 ? fm_uniform(lds_blob[pn]) : nullptr;
+        const uint8_t *blob_c = blob_n;            // blob of the unit being computed
+        const uint8_t *blob_q[2] = {blob_n, blob_n};   // blobs of the units in flight
+        auto load_half = [&](FmRowSlice<BITS> &t) {
+            if (un < seg1) {
+                if (blob_n) {
+                    const uint8_t *b = blob_n + (size_t)rsn * wstep;
+                    const uint8_t *sb = blob_n + (size_t)rsn * sstep;
+                    if (hn == 0)
+                        fm_load_slice<BITS>(t, b + a.g.gate_w + woff, sb + a.g.gate_s + soff,
+                                            sb + a.g.gate_b + soff);
+                    else
+                        fm_load_slice<BITS>(t, b + a.g.up_w + woff, sb + a.g.up_s + soff,
+                                            sb + a.g.up_b + soff);
+                }
+                if (hn == 1) {
+                    un += 4;
+                    rsn += 4;
+                    if (rsn >= upp) {
+                        rsn -= upp;
+                        pn++;
+                        if (un < seg1) blob_n = fm_uniform(lds_blob[pn]);
+                    }
+                }
+                hn ^= 1;
+            }
+        };
+        FmRowSlice<BITS> r0, r1, r2;
+        load_half(r0);                            // one unit in flight during the build
+        load_half(r1);
+        blob_q[0] = blob_n;                       // blob of unit u+4 (after the two loads)
+        fm_build_act_lds<BITS, LPR>(a.x + (size_t)l * a.g.hidden, bslot, lds);
         __syncthreads();
         FmActRegs ar;
         fm_read_act_lds<LPR>(lds, lane, ar);
-        const uint8_t *blob_c = blob_n;
-        for (; u < seg1; u += 4) {
-            if (u + 4 < seg1) {
-                rsn += 4;
-                if (rsn >= upp) {
-                    rsn -= upp;
-                    pn++;
-                    blob_n = lds_blob[pn];
-                }
-                load_unit(blob_n, rsn, gnext, unext);
-            }
+        float gv = 0.0f;
+        // one half step: start the load two half steps ahead, multiply the current slice
+        auto gate_step = [&](FmRowSlice<BITS> &cur, FmRowSlice<BITS> &tgt) {
+            load_half(tgt);
+            if (blob_c) gv = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(cur, ar));
+        };
+        auto up_step = [&](FmRowSlice<BITS> &cur, FmRowSlice<BITS> &tgt) {
+            // the load issued here is the up half of unit u+4... its blob is blob_q[0]
+            load_half(tgt);
             float v = 0.0f;
             if (blob_c) {
-                float gv = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(gcur, ar));
-                float uv = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(ucur, ar));
+                float uv = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(cur, ar));
                 v = fm_silu_mul(gv, uv);
             }
             // unit u = (pair, row step): act is [pair][inter], rows are contiguous
             if (ch == 0) a.act[(size_t)u * RPS + ris] = v;
-            gcur = gnext;
-            ucur = unext;
-            blob_c = blob_n;
+            u += 4;
+            blob_c = blob_q[0];
+            blob_q[0] = blob_n;
+        };
+        while (u < seg1) {
+            gate_step(r0, r2);
+            up_step(r1, r0);
+            if (u >= seg1) break;
+            gate_step(r2, r1);
+            up_step(r0, r2);
+            if (u >= seg1) break;
+            gate_step(r1, r0);
+            up_step(r2, r1);
         }
         seg0 = seg1;
     }
 }
 
-// down projection -> per-expert output vectors
+// down projection -> per-expert output vectors.  Ring of three slices: two units
+// of loads in flight ahead of the one being multiplied.
 template <int BITS, int LPR, bool FP16>
-__global__ __launch_bounds__(256) void fm_down_mfma(DecodeArgs a) {
+__global__ __launch_bounds__(256)
+void fm_down_mfma(DecodeArgs a) {
     constexpr int RPS = FM_WAVE / LPR;
     __shared__ FmActLds<LPR> lds;
     const int lane = threadIdx.x & 63;
@@ -307,10 +353,13 @@ __global__ __launch_bounds__(256) void fm_down_mfma(DecodeArgs a) {
     const long total = (long)n_pairs * upp;
     const long wg0 = total * blockIdx.x / gridDim.x, wg1 = total * (blockIdx.x + 1) / gridDim.x;
     const int row_bytes = a.g.inter * BITS / 8, sb_row_bytes = (a.g.inter / 64) * 2;
-    size_t woff, soff;
+    size_t woff_, soff_;
     int ris, ch;
-    fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff, soff, ris, ch);
-    const size_t wstep = (size_t)RPS * row_bytes, sstep = (size_t)RPS * sb_row_bytes;
+    fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff_, soff_, ris, ch);
+    const uint32_t woff = (uint32_t)woff_, soff = (uint32_t)soff_;
+    const uint32_t wstep = (uint32_t)(RPS * row_bytes), sstep = (uint32_t)(RPS * sb_row_bytes);
+    FmBuildSlot<BITS> bslot;
+    bslot.init();
 
     for (long seg0 = wg0; seg0 < wg1;) {
         const int p = (int)(seg0 / upp);
@@ -318,28 +367,39 @@ __global__ __launch_bounds__(256) void fm_down_mfma(DecodeArgs a) {
         if (seg1 > wg1) seg1 = wg1;
         const uint8_t *blob = fm_pair_blob(a, p);
         long u = seg0 + wave;
-        int rs = (int)(u - (long)p * upp);
-        auto load_unit = [&](int r, FmRowSlice<BITS> &ds) {
-            size_t wo = woff + (size_t)r * wstep, so = soff + (size_t)r * sstep;
-            fm_load_slice<BITS>(ds, blob + a.g.down_w + wo, blob + a.g.down_s + so,
-                                blob + a.g.down_b + so);
+        int rsn = (int)(u - (long)p * upp);
+        long un = u;
+        auto load_next = [&](FmRowSlice<BITS> &ds) {
+            if (un < seg1) {
+                const uint8_t *b = blob + (size_t)rsn * wstep;
+                const uint8_t *sb = blob + (size_t)rsn * sstep;
+                fm_load_slice<BITS>(ds, b + a.g.down_w + woff, sb + a.g.down_s + soff,
+                                    sb + a.g.down_b + soff);
+                un += 4;
+                rsn += 4;
+            }
         };
         __syncthreads();
         if (blob) {
-            fm_stage_x_lds<LPR>(a.act + (size_t)p * a.g.inter, lds);
-            FmRowSlice<BITS> cur, next;
-            if (u < seg1) load_unit(rs, cur);
-            __syncthreads();
-            fm_build_act_lds<BITS, LPR>(lds);
+            FmRowSlice<BITS> r0, r1, r2;
+            load_next(r0);
+            load_next(r1);
+            fm_build_act_lds<BITS, LPR>(a.act + (size_t)p * a.g.inter, bslot, lds);
             __syncthreads();
             FmActRegs ar;
             fm_read_act_lds<LPR>(lds, lane, ar);
-            for (; u < seg1; u += 4) {
-                rs += 4;
-                if (u + 4 < seg1) load_unit(rs, next);
+            auto step = [&](FmRowSlice<BITS> &cur, FmRowSlice<BITS> &tgt) {
+                load_next(tgt);
                 float v = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(cur, ar));
                 if (ch == 0) a.expert_out[(size_t)u * RPS + ris] = v;
-                cur = next;
+                u += 4;
+            };
+            while (u < seg1) {
+                step(r0, r2);
+                if (u >= seg1) break;
+                step(r1, r0);
+                if (u >= seg1) break;
+                step(r2, r1);
             }
         } else {
             for (; u < seg1; u += 4)

@@ -148,66 +148,75 @@ __device__ __forceinline__ uint32_t fm_bf16_piece(float v, int piece) {
 
 // LDS image of the activation registers of every (chunk, piece) of one input
 // vector, built once per workgroup and read by all its waves.
-//   x   [128*LPR] float   : the input vector, staged with coalesced loads
 //   a   [16][4*LPR] uint4 : register quad q of entry e = 4*chunk + piece (lane-major,
 //                           so a wave's read of one quad is conflict free)
 //   sum [LPR] float4      : xsum0, xsum1, xoff0, xoff1 of each chunk
 template <int LPR>
 struct FmActLds {
-    float x[FM_CPL * LPR];
     uint4 a[16][4 * LPR];
     float4 sum[LPR];
 };
 
-// step 1 (all 256 threads): global x -> LDS; caller barriers afterwards
-template <int LPR>
-__device__ __forceinline__ void fm_stage_x_lds(const float *x, FmActLds<LPR> &L) {
-    const float4 *src = reinterpret_cast<const float4 *>(x);
-    float4 *dst = reinterpret_cast<float4 *>(L.x);
-#pragma unroll
-    for (int i = 0; i < (FM_CPL * LPR / 4 + 255) / 256; i++) {
-        int k = threadIdx.x + 256 * i;
-        if (k < FM_CPL * LPR / 4) dst[k] = src[k];
+// What one thread contributes to the image: register slot w = tid % 64 (group
+// w/32, pair w%32) of chunks tid/64, tid/64 + 4, ...  The slot's two columns
+// and their scales depend on w only, so they are computed once per kernel.
+template <int BITS>
+struct FmBuildSlot {
+    int lo, hi;          // column offsets inside the 128-column chunk
+    float slo, shi;      // 128 / 2^t of the two codes
+    __device__ __forceinline__ void init() {
+        using T = FmPairs<BITS>;
+        const int w = threadIdx.x & 63, G = w >> 5, P = w & 31;
+        lo = 64 * G + T::lo(P);
+        hi = 64 * G + T::hi(P);
+        slo = fm_pair_scale_lo<BITS>(P);
+        shi = fm_pair_scale_hi<BITS>(P);
     }
-}
+};
 
-// step 2 (all 256 threads, after the barrier): LDS x -> register image + sums;
-// caller barriers afterwards
+// All 256 threads.  x = the 128*LPR activations in global memory.  The caller
+// puts a barrier before (previous readers done) and after (image complete).
 template <int BITS, int LPR>
-__device__ __forceinline__ void fm_build_act_lds(FmActLds<LPR> &L) {
-    using T = FmPairs<BITS>;
+__device__ __forceinline__ void fm_build_act_lds(const float *x, const FmBuildSlot<BITS> &bs,
+                                                 FmActLds<LPR> &L) {
     constexpr int NE = 4 * LPR;
-    uint32_t *flat = reinterpret_cast<uint32_t *>(L.a);
-#pragma unroll 4
-    for (int d = threadIdx.x; d < NE * 64; d += 256) {
-        const int e = d >> 6, w = d & 63;
-        const int ch = e >> 2, piece = e & 3, G = w >> 5, P = w & 31;
-        const float *xc = L.x + ch * FM_CPL + 64 * G;
-        float sl = xc[T::lo(P)] * fm_pair_scale_lo<BITS>(P);
-        float sh = xc[T::hi(P)] * fm_pair_scale_hi<BITS>(P);
-        flat[((w >> 2) * NE + e) * 4 + (w & 3)] =
-            fm_bf16_piece(sl, piece) | (fm_bf16_piece(sh, piece) << 16);
-    }
-    // sums: 8 threads per (chunk, group), 4 pairs each
-    {
-        const int combo = threadIdx.x >> 3, sub = threadIdx.x & 7;
-        float xs = 0.0f, xo = 0.0f;
-        if (combo < 2 * LPR) {
-            const float *xc = L.x + (combo >> 1) * FM_CPL + 64 * (combo & 1);
+    constexpr int NIT = (LPR + 3) / 4;     // chunks per thread
+    const int w = threadIdx.x & 63;
+    float xl[NIT], xh[NIT];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int P = 4 * sub + i;
-                float xl = xc[T::lo(P)], xh = xc[T::hi(P)];
-                xs += xl + xh;
-                xo += xl * fm_pair_scale_lo<BITS>(P) + xh * fm_pair_scale_hi<BITS>(P);
-            }
+    for (int i = 0; i < NIT; i++) {
+        const int ch = (threadIdx.x >> 6) + 4 * i;
+        const bool on = ch < LPR;
+        xl[i] = on ? x[ch * FM_CPL + bs.lo] : 0.0f;
+        xh[i] = on ? x[ch * FM_CPL + bs.hi] : 0.0f;
+    }
+    uint32_t *flat = reinterpret_cast<uint32_t *>(L.a);
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+        const int ch = (threadIdx.x >> 6) + 4 * i;
+        // exact three-way split of scale*x into bf16 pieces (truncations of the
+        // running remainder); the two columns share a register: low | high << 16
+        float vl = xl[i] * bs.slo, vh = xh[i] * bs.shi;
+        uint32_t l0 = __float_as_uint(vl) & 0xFFFF0000u, h0 = __float_as_uint(vh) & 0xFFFF0000u;
+        float rl = vl - __uint_as_float(l0), rh = vh - __uint_as_float(h0);
+        uint32_t l1 = __float_as_uint(rl) & 0xFFFF0000u, h1 = __float_as_uint(rh) & 0xFFFF0000u;
+        rl -= __uint_as_float(l1);
+        rh -= __uint_as_float(h1);
+        uint32_t l2 = __float_as_uint(rl), h2 = __float_as_uint(rh) & 0xFFFF0000u;
+        if (ch < LPR) {
+            uint32_t *dst = flat + ((w >> 2) * NE + 4 * ch) * 4 + (w & 3);
+            dst[0] = (l0 >> 16) | h0;
+            dst[4] = (l1 >> 16) | h1;
+            dst[8] = (l2 >> 16) | h2;
+            dst[12] = 0u;
         }
-        xs = fm_group_sum<8>(xs);
-        xo = fm_group_sum<8>(xo);
-        if (combo < 2 * LPR && sub == 0) {
-            float *sp = reinterpret_cast<float *>(&L.sum[combo >> 1]);
-            sp[combo & 1] = xs;
-            sp[2 + (combo & 1)] = xo;
+        // sums over the 32 slots of a group: lanes 0..31 / 32..63 of the wave
+        float xs = fm_group_sum<32>(xl[i] + xh[i]);
+        float xo = fm_group_sum<32>(vl + vh);
+        if (ch < LPR && (w & 31) == 0) {
+            float *sp = reinterpret_cast<float *>(&L.sum[ch]);
+            sp[w >> 5] = xs;
+            sp[2 + (w >> 5)] = xo;
         }
     }
 }
