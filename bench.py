@@ -210,6 +210,224 @@ def run_decode_step(args):
     return res
 
 
+def _finish(res, metric, workload, bytes_step, ms_per_step, args, extra_cfg=None):
+    out = {
+        "metric": metric, "value": round(bytes_step / (ms_per_step * 1e-3) / 1e9, 2), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic", "config": {"workload": workload, "bytes_per_step": bytes_step},
+        "us_per_step": round(ms_per_step * 1e3, 2),
+        "frac_of_hbm_peak": round(bytes_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+    }
+    if extra_cfg:
+        out["config"].update(extra_cfg)
+    out.update(res)
+    return out
+
+
+def _timed(ctx, step, args):
+    import torch
+    for t in range(args.warmup):
+        step(t)
+    ctx.sync()
+    torch.cuda.synchronize()
+    ctx.timer_start()
+    t0 = time.perf_counter()
+    for t in range(args.steps):
+        step(args.warmup + t)
+    ev_ms = ctx.timer_stop()
+    ctx.sync()
+    wall = time.perf_counter() - t0
+    return wall * 1e3 / args.steps, ev_ms / args.steps
+
+
+def run_decode_layer(args):
+    """config 0: one MoE layer per call, batch 1; calls cycle through 40 distinct layers
+    (440 MB > L2, so a call never finds its weights cached by the previous one)."""
+    import torch
+    from finchmoe_amd import FinchHip, formats
+    dev = torch.device("cuda:0")
+    lo = formats.expert_layout(H, I, 3)
+    es = lo["expert_size"]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+    blob = torch.empty(L, E, es, dtype=torch.uint8, device=dev)
+    for l in range(L):
+        fill_affine_layer(blob[l], lo, 3, gen)
+    ctx = FinchHip(0)
+    ctx.experts_config(L, E, H, I, 64, 3, 0)
+    for l in range(L):
+        ctx.experts_adopt_layer(l, blob[l].data_ptr(), E * es)
+    rng = np.random.default_rng(7)
+    tokens = 64
+    idx, w = zipf_routing(rng, tokens, L, E, K)
+    d_idx, d_w = torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)
+    d_x = torch.randn(L, H, device=dev)
+    d_out = torch.empty(L, H, device=dev)
+    torch.cuda.synchronize()
+
+    def step(t):
+        l, tok = t % L, (t // L) % tokens
+        o = (tok * L + l) * K * 4
+        ctx.moe_decode_dev(l, d_x.data_ptr() + l * H * 4, d_idx.data_ptr() + o, d_w.data_ptr() + o, K,
+                           d_out.data_ptr() + l * H * 4)
+
+    ms, ev = _timed(ctx, step, args)
+    ctx.kernel_timing(True)
+    for t in range(args.steps):
+        step(t)
+    k1, k2, n = ctx.kernel_timing_read()
+    ctx.kernel_timing(False)
+    res = {"kernels_us": {"fm_gate_up_swiglu_mfma": round(k1 / n * 1e3, 2),
+                          "fm_down_mfma+fm_combine": round(k2 / n * 1e3, 2)},
+           "event_ms_per_step": round(ev, 5)}
+    ctx.close()
+    return _finish(res, "3-bit expert GEMV HBM GB/s, one MoE layer per call", "config 0: single MoE layer, decode "
+                   "batch 1, hidden 2048, 256 experts, top-8, 3-bit g64; calls cycle over 40 layers",
+                   K * es, ms, args)
+
+
+def run_gdn(args):
+    """config 1: dense 4-bit GatedDeltaNet projections, batch 1, 40 independent weight sets."""
+    import torch
+    from finchmoe_amd import FinchHip
+    dev = torch.device("cuda:0")
+    ctx = FinchHip(0)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(99)
+    sets = []
+    keep = []
+
+    def tensor(out_dim, in_dim):
+        W = torch.empty(out_dim * in_dim // 2, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
+        s = torch.randn(out_dim * (in_dim // 64), device=dev, generator=gen).abs_() * (0.02 / 3.5)
+        b = s * -3.5
+        S, B = _bf16_trunc_bits(s), _bf16_trunc_bits(b)
+        keep.extend([W, S, B])
+        return ctx.tensor_adopt(W.data_ptr(), S.data_ptr(), B.data_ptr(), out_dim, in_dim, 4)
+
+    nsets = 40
+    for _ in range(nsets):
+        sets.append((tensor(8192, 2048), tensor(4096, 2048), tensor(2048, 4096)))
+    d_x = torch.randn(2048, device=dev)
+    d_y = torch.randn(4096, device=dev)
+    oq, oz, oo = (torch.empty(n, device=dev) for n in (8192, 4096, 2048))
+    torch.cuda.synchronize()
+
+    def step(t):
+        q, z, o = sets[t % nsets]
+        ctx.matvec_batch_dev([q, z], d_x.data_ptr(), [oq.data_ptr(), oz.data_ptr()])
+        ctx.matvec_batch_dev([o], d_y.data_ptr(), [oo.data_ptr()])
+
+    ms, ev = _timed(ctx, step, args)
+    bytes_set = 12288 * 1152 + 2048 * (2048 + 256)
+    res = {"event_ms_per_step": round(ev, 5)}
+    ctx.close()
+    return _finish(res, "dense 4-bit GatedDeltaNet projection GEMV HBM GB/s", "config 1: in_proj_qkv+z "
+                   "2048->12288 and out_proj 4096->2048, 4-bit g64, batch 1, 40 weight sets cycled",
+                   bytes_set, ms, args)
+
+
+def run_gguf(args):
+    """config 4: GGUF experts (Q4_K gate/up, Q6_K down), 40-layer decode step, batch 1."""
+    import torch
+    from finchmoe_amd import FinchHip
+    dev = torch.device("cuda:0")
+    n_layers = args.layers
+    gsl, dsl = I * (H // 256) * 144, H * (I // 256) * 210
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(5)
+    ctx = FinchHip(0)
+    ctx.gguf_config(n_layers, E, H, I)
+    keep = []
+
+    def slab(nblocks, bsz, d_off, n_d):
+        t = torch.empty(nblocks, bsz, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
+        d = (torch.randn(nblocks, n_d, device=dev, generator=gen).abs_() * 0.002).to(torch.float16)
+        t[:, d_off:d_off + 2 * n_d] = d.view(torch.uint8)
+        return t
+
+    for l in range(n_layers):
+        g = slab(E * I * (H // 256), 144, 0, 2)
+        u = slab(E * I * (H // 256), 144, 0, 2)
+        d = slab(E * H * (I // 256), 210, 208, 1)
+        keep.extend([g, u, d])
+        ctx.gguf_adopt_layer(l, g.data_ptr(), u.data_ptr(), d.data_ptr())
+    rng = np.random.default_rng(7)
+    tokens = 64
+    idx, w = zipf_routing(rng, tokens, n_layers, E, K)
+    d_idx, d_w = torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)
+    d_x = torch.randn(n_layers, H, device=dev)
+    d_out = torch.empty(n_layers, H, device=dev)
+    torch.cuda.synchronize()
+    isz = n_layers * K * 4
+
+    def step(t):
+        t %= tokens
+        ctx.gguf_moe_decode_step_dev(0, n_layers, d_x.data_ptr(), d_idx.data_ptr() + t * isz,
+                                     d_w.data_ptr() + t * isz, K, d_out.data_ptr())
+
+    ms, ev = _timed(ctx, step, args)
+    ctx.kernel_timing(True)
+    for t in range(args.steps):
+        step(t)
+    k1, k2, n = ctx.kernel_timing_read()
+    ctx.kernel_timing(False)
+    assert torch.isfinite(d_out).all()
+    res = {"kernels_us": {"fm_gguf_gate_up": round(k1 / n * 1e3, 2),
+                          "fm_gguf_down+combine": round(k2 / n * 1e3, 2)},
+           "event_ms_per_step": round(ev, 5)}
+    ctx.close()
+    return _finish(res, "GGUF Q4_K/Q6_K expert GEMV HBM GB/s over the %d-layer decode step" % n_layers,
+                   "config 4: %dx%d GGUF experts (Q4_K gate/up, Q6_K down) resident, top-8 Zipf(1.1), batch 1"
+                   % (n_layers, E), n_layers * K * (2 * gsl + dsl), ms, args)
+
+
+def run_prefill(args):
+    """config 3: chunked prefill of M positions on one layer (M = --chunk)."""
+    import torch
+    from finchmoe_amd import FinchHip, formats
+    dev = torch.device("cuda:0")
+    M = args.chunk
+    lo = formats.expert_layout(H, I, 3)
+    es = lo["expert_size"]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+    nl = 8
+    blob = torch.empty(nl, E, es, dtype=torch.uint8, device=dev)
+    for l in range(nl):
+        fill_affine_layer(blob[l], lo, 3, gen)
+    ctx = FinchHip(0)
+    ctx.experts_config(nl, E, H, I, 64, 3, 0)
+    for l in range(nl):
+        ctx.experts_adopt_layer(l, blob[l].data_ptr(), E * es)
+    rng = np.random.default_rng(7)
+    idx, w = zipf_routing(rng, M, nl, E, K)          # [M, nl, K]
+    idx = np.ascontiguousarray(idx.transpose(1, 0, 2))
+    w = np.ascontiguousarray(w.transpose(1, 0, 2))
+    d_idx, d_w = torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)
+    d_X = torch.randn(M, H, device=dev).to(torch.bfloat16).to(torch.float32)   # x ~ N(0,1) bf16
+    d_out = torch.empty(M, H, device=dev)
+    torch.cuda.synchronize()
+
+    def step(t):
+        l = t % nl
+        ctx.moe_prefill_dev(l, d_X.data_ptr(), d_idx.data_ptr() + l * M * K * 4,
+                            d_w.data_ptr() + l * M * K * 4, M, K, d_out.data_ptr())
+
+    ms, ev = _timed(ctx, step, args)
+    flops = M * K * 3 * 2 * H * I
+    uniq = float(np.mean([len(set(idx[l].reshape(-1).tolist())) for l in range(nl)]))
+    res = {"tflops": round(flops / (ms * 1e-3) / 1e12, 2),
+           "frac_of_bf16_mfma_peak": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+           "unique_experts_per_chunk": uniq, "event_ms_per_step": round(ev, 5)}
+    ctx.close()
+    out = _finish(res, "chunked-prefill expert product, %d-position chunk" % M,
+                  "config 3: %d-token chunk, top-8 Zipf(1.1), 3-bit g64 experts, x~N(0,1) bf16 values in fp32"
+                  % M, int(uniq * es), ms, args, {"flops_per_step": flops})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -217,6 +435,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="decode_step")
     ap.add_argument("--layers", type=int, default=L)
+    ap.add_argument("--chunk", type=int, default=512, help="positions per chunk (prefill workload)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
@@ -228,7 +447,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; there is no CPU fallback", file=sys.stderr)
         sys.exit(3)
-    runners = {"decode_step": run_decode_step}
+    runners = {"decode_step": run_decode_step, "decode_layer": run_decode_layer, "gdn": run_gdn,
+               "gguf": run_gguf, "prefill": run_prefill}
     if args.workload not in runners:
         print("bench.py: unknown workload %r (have: %s)" % (args.workload, ", ".join(runners)),
               file=sys.stderr)
