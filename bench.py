@@ -28,6 +28,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 peak
+# HBM bytes per launch of the gate+up kernel on the default workload, from rocprofv3 --pmc
+# FETCH_SIZE (x2: calibrated against a 1 GiB copy) + WRITE_SIZE, see
+# profiles/decode_step_3bit_hbm_traffic.md.  Offline measurement; null for other sizes.
+GATE_UP_TRAFFIC_BYTES_40L = 289838 * 1024 + 676 * 1024
 
 H, I, E, K, L = 2048, 512, 256, 8, 40
 
@@ -198,7 +202,8 @@ def run_decode_step(args):
         "roofline": {"bound": "hbm", "kernel": "fm_gate_up_swiglu<3,16>",
                      "achieved": round(k1_bytes / (k1_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(k1_bytes / (k1_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": None, "bytes_per_launch": k1_bytes},
+                     "traffic": GATE_UP_TRAFFIC_BYTES_40L if (n_layers, E, K) == (40, 256, 8) else None,
+                     "bytes_per_launch": k1_bytes},
         "roofline_down": {"bound": "hbm", "kernel": "fm_down<3,4> + fm_combine",
                           "achieved": round((bytes_step - k1_bytes) / (k2_us * 1e-6) / 1e9, 1),
                           "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -428,6 +433,27 @@ def run_prefill(args):
     return out
 
 
+def run_copy_probe(args):
+    """Plain device copy of known size (1 GiB read + 1 GiB written per step): the
+    calibration run for the FETCH_SIZE / WRITE_SIZE counters."""
+    import torch
+    dev = torch.device("cuda:0")
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device=dev).random_(0, 256)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    return _finish({}, "device copy GB/s (read + write)", "copy probe: 1 GiB uint8 torch copy_ per step",
+                   2 * n, ms, args)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -448,7 +474,7 @@ def main():
         print("bench.py: no GPU visible; there is no CPU fallback", file=sys.stderr)
         sys.exit(3)
     runners = {"decode_step": run_decode_step, "decode_layer": run_decode_layer, "gdn": run_gdn,
-               "gguf": run_gguf, "prefill": run_prefill}
+               "gguf": run_gguf, "prefill": run_prefill, "copy_probe": run_copy_probe}
     if args.workload not in runners:
         print("bench.py: unknown workload %r (have: %s)" % (args.workload, ", ".join(runners)),
               file=sys.stderr)
