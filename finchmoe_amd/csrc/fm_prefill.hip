@@ -38,7 +38,6 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 typedef const __attribute__((address_space(1))) uint8_t *gptr;
 
 #define PF_TM 16          // positions per item
-#define PF_THREADS 512
 #define PF_MAX_EXPERTS 1024
 
 struct PfItem { int expert, start, count, pad; };
@@ -93,71 +92,82 @@ struct PfLds {
 
 __device__ __forceinline__ uint32_t bf16_trunc(float v) { return __float_as_uint(v) >> 16; }
 
-// Build the operand images for `count` positions whose activation rows are
-// xrow(j) (fp32, NG*64 columns).
-template <int NG, class RowFn>
-__device__ void pf_stage(PfLds<NG> &L, int count, RowFn xrow) {
-    // main image: task = (position j, group g, half h, k step s) -> two 16-byte entries
-    for (int t = threadIdx.x; t < PF_TM * NG * 8; t += PF_THREADS) {
-        const int s = t & 3, h = (t >> 2) & 1, g = (t >> 3) % NG, j = t / (8 * NG);
-        uint32_t hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
-        if (j < count) {
-            const float *x = xrow(j) + 64 * g + 32 * h;
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int p = 4 * s + q;
-                // runtime forms of pf_lo / pf_hi / scales
-                const int far = p >= 10;
-                const int lc = far ? 20 + (p - 10) : 10 * (p / 5) + p % 5;
-                const int hc = lc + (far ? 6 : 5);
-                float vl = x[lc] * (far ? 32.0f : 8.0f), vh = x[hc] * (far ? 8.0f : 16.0f);
-                uint32_t l0 = __float_as_uint(vl) & 0xFFFF0000u, h0 = __float_as_uint(vh) & 0xFFFF0000u;
-                float rl = vl - __uint_as_float(l0), rh = vh - __uint_as_float(h0);
-                hi[q] = (l0 >> 16) | h0;
-                lo[q] = bf16_trunc(rl) | (__float_as_uint(rh) & 0xFFFF0000u);
-            }
-        }
-        const int base = ((g * 4 + s) * 2 + h) * 32;
+template <int S, int Q>
+__device__ __forceinline__ void pf_stage_pair(const float *x, uint32_t *hi, uint32_t *lo, float &xs,
+                                              float &xo) {
+    constexpr int p = 4 * S + Q;
+    constexpr float cl = (float)(128 >> pf_tl(p)), ch = (float)(128 >> pf_th(p));
+    float vl = x[pf_lo(p)] * cl, vh = x[pf_hi(p)] * ch;
+    // exact split into bf16 pieces; hi + lo = the value truncated to 16 significant bits
+    uint32_t l0 = __float_as_uint(vl) & 0xFFFF0000u, h0 = __float_as_uint(vh) & 0xFFFF0000u;
+    float rl = vl - __uint_as_float(l0), rh = vh - __uint_as_float(h0);
+    uint32_t l1 = __float_as_uint(rl) & 0xFFFF0000u, h1 = __float_as_uint(rh) & 0xFFFF0000u;
+    hi[Q] = (l0 >> 16) | h0;
+    lo[Q] = (l1 >> 16) | h1;
+    float tl = __uint_as_float(l0) + __uint_as_float(l1), th = __uint_as_float(h0) + __uint_as_float(h1);
+    xo += tl + th;
+    xs += tl * (1.0f / cl) + th * (1.0f / ch);
+}
+
+template <int NG, int S>
+__device__ __forceinline__ void pf_stage_steps(PfLds<NG> &L, const float *x, int g, int h, int j,
+                                               float &xs, float &xo) {
+    if constexpr (S < 4) {
+        uint32_t hi[4], lo[4];
+        pf_stage_pair<S, 0>(x, hi, lo, xs, xo);
+        pf_stage_pair<S, 1>(x, hi, lo, xs, xo);
+        pf_stage_pair<S, 2>(x, hi, lo, xs, xo);
+        pf_stage_pair<S, 3>(x, hi, lo, xs, xo);
+        const int base = ((g * 4 + S) * 2 + h) * 32;
         L.act[base + j] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
         L.act[base + 16 + j] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        pf_stage_steps<NG, S + 1>(L, x, g, h, j, xs, xo);
     }
-    // side image: per (position, group) the sums of the 16-bit activations
-    // x16 = hi + lo pieces divided by their scale, and of the scaled pieces
-    for (int t = threadIdx.x; t < 2 * 3 * 2 * 2 * 32 * 4; t += PF_THREADS)
+}
+
+// Build the operand images for `count` positions whose activation rows are
+// xrow(j) (fp32, NG*64 columns).  A task = (position, group, half): 32 activations
+// read with eight 128-bit loads, all k steps of that half built from registers.
+// The caller has a barrier before (previous readers done) and after.
+template <int NG, class RowFn>
+__device__ void pf_stage(PfLds<NG> &L, int count, RowFn xrow) {
+    for (int t = threadIdx.x; t < 2 * 3 * 2 * 2 * 32 * 4; t += blockDim.x)
         reinterpret_cast<uint32_t *>(L.side)[t] = 0u;
     __syncthreads();
-    for (int t = threadIdx.x; t < PF_TM * NG; t += PF_THREADS) {
-        const int g = t % NG, j = t / NG;
-        if (j >= count) continue;
-        const float *x = xrow(j) + 64 * g;
-        float xs = 0.0f, xo = 0.0f;
-        for (int hh = 0; hh < 2; hh++)
-            for (int p = 0; p < 16; p++) {
-                const int far = p >= 10;
-                const int lc = far ? 20 + (p - 10) : 10 * (p / 5) + p % 5;
-                const int hc = lc + (far ? 6 : 5);
-                const float cl = far ? 32.0f : 8.0f, chh = far ? 8.0f : 16.0f;
-                float vl = x[32 * hh + lc] * cl, vh = x[32 * hh + hc] * chh;
-                // value the two pieces represent: v truncated to 16 significant bits
-                float l0 = __uint_as_float(__float_as_uint(vl) & 0xFFFF0000u);
-                float h0 = __uint_as_float(__float_as_uint(vh) & 0xFFFF0000u);
-                float l1 = __uint_as_float(__float_as_uint(vl - l0) & 0xFFFF0000u);
-                float h1 = __uint_as_float(__float_as_uint(vh - h0) & 0xFFFF0000u);
-                float tl = l0 + l1, th = h0 + h1;
-                xo += tl + th;
-                xs += tl / cl + th / chh;
+    for (int t = threadIdx.x; t < PF_TM * NG * 2; t += blockDim.x) {
+        const int h = t & 1, g = (t >> 1) % NG, j = t / (2 * NG);
+        float x[32];
+        if (j < count) {
+            const float4 *xp = reinterpret_cast<const float4 *>(xrow(j) + 64 * g + 32 * h);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float4 v = xp[i];
+                x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
             }
-        // three bf16 pieces of xs and of -xo, stored on the hi row (mrow j) of the position
-        float vals[2] = {xs, -xo};
-        const int m2 = g >> 4, hh = (g >> 3) & 1, i = g & 7;
-        for (int term = 0; term < 2; term++) {
-            float r = vals[term];
-            for (int piece = 0; piece < 3; piece++) {
-                uint32_t b = __float_as_uint(r) & 0xFFFF0000u;
-                r -= __uint_as_float(b);
-                uint16_t *e = reinterpret_cast<uint16_t *>(
-                    &L.side[(((term * 3 + piece) * 2 + m2) * 2 + hh) * 32 + j]);
-                e[i] = (uint16_t)(b >> 16);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 32; i++) x[i] = 0.0f;
+        }
+        float xs = 0.0f, xo = 0.0f;
+        pf_stage_steps<NG, 0>(L, x, g, h, j, xs, xo);
+        // the two halves of a group sit in adjacent lanes
+        xs += fm_dpp<0xB1>(xs);
+        xo += fm_dpp<0xB1>(xo);
+        if (h == 0 && j < count) {
+            // three bf16 pieces of xsum and of -xoff, on the hi row (M row j) of the position
+            float vals[2] = {xs, -xo};
+            const int m2 = g >> 4, hh = (g >> 3) & 1, i = g & 7;
+#pragma unroll
+            for (int term = 0; term < 2; term++) {
+                float r = vals[term];
+#pragma unroll
+                for (int piece = 0; piece < 3; piece++) {
+                    uint32_t b = __float_as_uint(r) & 0xFFFF0000u;
+                    r -= __uint_as_float(b);
+                    uint16_t *e = reinterpret_cast<uint16_t *>(
+                        &L.side[(((term * 3 + piece) * 2 + m2) * 2 + hh) * 32 + j]);
+                    e[i] = (uint16_t)(b >> 16);
+                }
             }
         }
     }
@@ -192,27 +202,27 @@ __device__ __forceinline__ void pf_tile_pass(const PfLds<NG> &L, gptr wrow, gptr
             acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, sb, acc, 0, 0, 0);
         }
     }
-    // main product, two groups (48 bytes of the row) per iteration
-    fm_u4 cur[3], nxt[3];
+    // main product, two groups per iteration; the lane reads its own half (12 bytes) of each
+    typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+    typedef const __attribute__((address_space(1))) u32x3 *g3_t;
+    gptr wmine = wrow + 12 * h;
+    u32x3 cur0, cur1, nxt0, nxt1;
     uint32_t scur, snxt;
-    {
-        gq_t p = (gq_t)wrow;
-        cur[0] = p[0]; cur[1] = p[1]; cur[2] = p[2];
-        scur = *(const __attribute__((address_space(1))) uint32_t *)srow;
-    }
+    cur0 = *(g3_t)wmine;
+    cur1 = *(g3_t)(wmine + 24);
+    scur = *(const __attribute__((address_space(1))) uint32_t *)srow;
     for (int g2 = 0; g2 < NG / 2; g2++) {
         if (g2 + 1 < NG / 2) {
-            gq_t p = (gq_t)(wrow + 48 * (g2 + 1));
-            nxt[0] = p[0]; nxt[1] = p[1]; nxt[2] = p[2];
+            nxt0 = *(g3_t)(wmine + 48 * (g2 + 1));
+            nxt1 = *(g3_t)(wmine + 48 * (g2 + 1) + 24);
             snxt = *(const __attribute__((address_space(1))) uint32_t *)(srow + 4 * (g2 + 1));
         }
-        const uint32_t *d = reinterpret_cast<const uint32_t *>(cur);
 #pragma unroll
         for (int gg = 0; gg < 2; gg++) {
-            // this lane's half of group 2*g2+gg: dwords 6*gg + 3*h .. +2
             uint32_t my[3];
-#pragma unroll
-            for (int k = 0; k < 3; k++) my[k] = h ? d[6 * gg + 3 + k] : d[6 * gg + k];
+            my[0] = gg ? cur1.x : cur0.x;
+            my[1] = gg ? cur1.y : cur0.y;
+            my[2] = gg ? cur1.z : cur0.z;
             uint32_t v[16];
             pf_unpack<0>(my, ones, v);
             f16v dg;
@@ -229,49 +239,59 @@ __device__ __forceinline__ void pf_tile_pass(const PfLds<NG> &L, gptr wrow, gptr
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[i] = fmaf(sc, dg[i], acc[i]);
         }
-        cur[0] = nxt[0]; cur[1] = nxt[1]; cur[2] = nxt[2];
+        cur0 = nxt0;
+        cur1 = nxt1;
         scur = snxt;
     }
 }
 
 // ---------------------------------------------------------------- kernels
-// pairs -> grouped by expert, cut into items of <= PF_TM positions.  One workgroup.
+// pairs -> grouped by expert, cut into items of <= PF_TM positions.  One workgroup of
+// 1024 threads, one expert per thread for the two prefix sums.
 __global__ __launch_bounds__(1024) void fm_pf_sort(PfArgs a) {
-    __shared__ int hist[PF_MAX_EXPERTS], cursor[PF_MAX_EXPERTS];
-    const int E = a.g.n_experts, n = a.M * a.K;
-    for (int e = threadIdx.x; e < E; e += blockDim.x) hist[e] = 0;
+    __shared__ int hist[PF_MAX_EXPERTS], cursor[PF_MAX_EXPERTS], scan_a[PF_MAX_EXPERTS],
+        scan_b[PF_MAX_EXPERTS];
+    const int E = a.g.n_experts, n = a.M * a.K, e = threadIdx.x;
+    hist[e] = 0;
     __syncthreads();
     for (int p = threadIdx.x; p < n; p += blockDim.x) {
-        int e = a.idx[p];
-        if ((unsigned)e < (unsigned)E) atomicAdd(&hist[e], 1);
+        int x = a.idx[p];
+        if ((unsigned)x < (unsigned)E) atomicAdd(&hist[x], 1);
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int off = 0, ni = 0;
-        for (int e = 0; e < E; e++) {
-            cursor[e] = off;
-            for (int s = 0; s < hist[e]; s += PF_TM) {
-                PfItem it;
-                it.expert = e;
-                it.start = off + s;
-                it.count = hist[e] - s < PF_TM ? hist[e] - s : PF_TM;
-                it.pad = 0;
-                a.items[ni++] = it;
-            }
-            off += hist[e];
-        }
-        *a.n_items = ni;
+    const int cnt = e < E ? hist[e] : 0, nit = (cnt + PF_TM - 1) / PF_TM;
+    // inclusive scans of the pair counts and the item counts (Hillis-Steele)
+    scan_a[e] = cnt;
+    scan_b[e] = nit;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {
+        int va = e >= d ? scan_a[e - d] : 0, vb = e >= d ? scan_b[e - d] : 0;
+        __syncthreads();
+        scan_a[e] += va;
+        scan_b[e] += vb;
+        __syncthreads();
     }
+    const int off = scan_a[e] - cnt, ioff = scan_b[e] - nit;
+    cursor[e] = off;
+    for (int s = 0; s < nit; s++) {
+        PfItem it;
+        it.expert = e;
+        it.start = off + s * PF_TM;
+        it.count = cnt - s * PF_TM < PF_TM ? cnt - s * PF_TM : PF_TM;
+        it.pad = 0;
+        a.items[ioff + s] = it;
+    }
+    if (e == 1023) *a.n_items = scan_b[1023];
     __syncthreads();
     for (int p = threadIdx.x; p < n; p += blockDim.x) {
-        int e = a.idx[p];
-        if ((unsigned)e < (unsigned)E) a.sorted[atomicAdd(&cursor[e], 1)] = p;
+        int x = a.idx[p];
+        if ((unsigned)x < (unsigned)E) a.sorted[atomicAdd(&cursor[x], 1)] = p;
     }
 }
 
 // gate + up + SwiGLU for every item -> act[sorted position][inter]
 template <int NG>
-__global__ __launch_bounds__(PF_THREADS) void fm_pf_gate_up(PfArgs a) {
+__global__ __launch_bounds__(512) void fm_pf_gate_up(PfArgs a) {
     extern __shared__ uint4 pf_smem[];
     PfLds<NG> &L = *reinterpret_cast<PfLds<NG> *>(pf_smem);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -287,7 +307,7 @@ __global__ __launch_bounds__(PF_THREADS) void fm_pf_gate_up(PfArgs a) {
         __syncthreads();
         const uint8_t *blob = a.layer + (size_t)item.expert * a.g.expert_size;
         const int n = lane & 31, h = lane >> 5;
-        for (int rt = wave; rt < a.g.inter / 32; rt += PF_THREADS / 64) {
+        for (int rt = wave; rt < a.g.inter / 32; rt += blockDim.x / 64) {
             const int row = rt * 32 + n;
             f16v accg, accu;
             pf_tile_pass<NG>(L, (gptr)(uintptr_t)(blob + a.g.gate_w + (size_t)row * row_bytes),
@@ -310,7 +330,7 @@ __global__ __launch_bounds__(PF_THREADS) void fm_pf_gate_up(PfArgs a) {
 
 // down for every item -> eo[pair][hidden]
 template <int NG>
-__global__ __launch_bounds__(PF_THREADS) void fm_pf_down(PfArgs a) {
+__global__ __launch_bounds__(512) void fm_pf_down(PfArgs a) {
     extern __shared__ uint4 pf_smem[];
     PfLds<NG> &L = *reinterpret_cast<PfLds<NG> *>(pf_smem);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -324,7 +344,7 @@ __global__ __launch_bounds__(PF_THREADS) void fm_pf_down(PfArgs a) {
         __syncthreads();
         const uint8_t *blob = a.layer + (size_t)item.expert * a.g.expert_size;
         const int n = lane & 31, h = lane >> 5;
-        for (int rt = wave; rt < a.g.hidden / 32; rt += PF_THREADS / 64) {
+        for (int rt = wave; rt < a.g.hidden / 32; rt += blockDim.x / 64) {
             const int row = rt * 32 + n;
             f16v acc;
             pf_tile_pass<NG>(L, (gptr)(uintptr_t)(blob + a.g.down_w + (size_t)row * row_bytes),
@@ -407,8 +427,7 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
     a.eo = (float *)ws;
     hipLaunchKernelGGL(fm_pf_sort, dim3(1), dim3(1024), 0, st, a);
     const int max_items = g->n_experts + (int)(n / PF_TM);
-    const int grid = max_items < n_cu ? max_items : n_cu;
-#define PF_LAUNCH(KERN, NG)                                                                        \
+#define PF_LAUNCH(KERN, NG, GRID, NT)                                                              \
     do {                                                                                           \
         static bool attr_set = false;                                                              \
         if (!attr_set) {                                                                           \
@@ -417,11 +436,15 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
                 return FM_ERR_HIP;                                                                 \
             attr_set = true;                                                                       \
         }                                                                                          \
-        hipLaunchKernelGGL(KERN<NG>, dim3(grid), dim3(PF_THREADS), sizeof(PfLds<NG>), st, a);      \
+        hipLaunchKernelGGL(KERN<NG>, dim3(GRID), dim3(NT), sizeof(PfLds<NG>), st, a);              \
     } while (0)
-    if (g->hidden == 2048) PF_LAUNCH(fm_pf_gate_up, 32);
-    else PF_LAUNCH(fm_pf_gate_up, 16);
-    PF_LAUNCH(fm_pf_down, 8);
+    // one 8-wave workgroup per CU: the kernels need ~200 registers per lane (two accumulator
+    // tiles, a group tile, 16 operand registers, loads in flight), which caps a SIMD at two
+    // waves; capping the registers instead made them spill and run 2-5x slower
+    const int grid = max_items < n_cu ? max_items : n_cu;
+    if (g->hidden == 2048) PF_LAUNCH(fm_pf_gate_up, 32, grid, 512);
+    else PF_LAUNCH(fm_pf_gate_up, 16, grid, 512);
+    PF_LAUNCH(fm_pf_down, 8, grid, 512);
 #undef PF_LAUNCH
     hipLaunchKernelGGL(fm_pf_combine, dim3(M, (g->hidden + 1023) / 1024), dim3(256), 0, st, a, d_out, flags);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
