@@ -188,6 +188,28 @@ def test_other_shape_397b_class(orc):
         ctx.close()
 
 
+@pytest.mark.parametrize("h,i,bits", [(1024, 256, 3), (512, 128, 3), (1024, 512, 4), (512, 256, 4)])
+def test_small_shapes_cover_every_lane_map(orc, h, i, bits):
+    """hidden/inter combinations that exercise 8/4 lanes per gate row and 2/1/4 lanes per
+    down row (the kernels are specialised on lanes-per-row)."""
+    from finchmoe_amd import FinchHip
+    rng = np.random.default_rng(h + i + bits)
+    blob = F.synth_expert_layer(rng, 5, h, i, bits)
+    ctx = FinchHip(0)
+    try:
+        ctx.experts_config(1, 5, h, i, 64, bits, fb.SCALE_BF16)
+        ctx.experts_upload_layer(0, blob)
+        x = rng.standard_normal(h).astype(np.float32)
+        idx = np.array([4, 0, 2], np.int32)
+        w = np.array([0.5, 0.2, 0.3], np.float32)
+        ref, ref_eo = orc.moe_experts_forward(blob, x, idx, w, h, i, bits)
+        out, eo = ctx.moe_decode(0, x, idx, w)
+        assert_parity(eo, ref_eo, "expert_out %d/%d" % (h, i))
+        assert_parity(out, ref, "moe_out %d/%d" % (h, i))
+    finally:
+        ctx.close()
+
+
 def test_prefill_small_chunk_equals_per_position(hip, orc, store3):
     """Chunk of 8 positions (the reference default, infer.m:455): identical to running the
     decode call per position — bitwise, as the reference's bench_prefill.sh demands."""
