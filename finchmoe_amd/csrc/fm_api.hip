@@ -22,8 +22,9 @@ extern "C" {
 int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs, const FmExpertGeom *g,
                             int layer0, int layer_stride, int n_layers, const float *d_x,
                             const int32_t *d_idx, const float *d_w, int K, float *d_act,
-                            float *d_expert_out, float *d_out, unsigned int *d_counters,
-                            int flags, int n_cu, hipStream_t st, hipEvent_t *kev);
+                            float *d_expert_out, float *d_out, unsigned int *d_sync,
+                            unsigned int *epoch, unsigned int spin_limit, int flags, int n_cu,
+                            hipStream_t st, hipEvent_t *kev);
 int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
                     const float *d_x, int M, int n_cu, hipStream_t st);
 int fm_launch_dequant_affine(const void *W, const void *S, const void *B, int out_dim,
@@ -67,7 +68,14 @@ struct fm_ctx {
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     hipEvent_t kev[3] = {nullptr, nullptr, nullptr};
-    bool ktiming = false;
+    int ktiming = 0;   // 0 off, 1 whole operator, 2 phases as separate kernels
+    // grid barrier of the fused decode kernel: [0] arrival counter (only grows; the
+    // host tracks its value in sync_epoch), [1] error flag raised by a timed-out wait
+    unsigned int *d_sync = nullptr;
+    unsigned int sync_epoch = 0;
+    unsigned int spin_limit = 1u << 20;
+    bool split_phases = false;     // run the phases as separate kernels
+    bool sync_unchecked = false;   // a fused launch has not had its error flag read yet
     double k1_ms = 0.0, k2_ms = 0.0;
     int kcalls = 0;
     std::string err;
@@ -235,6 +243,12 @@ extern "C" int fm_ctx_create(int device, fm_ctx **out) {
             delete c;
             return FM_ERR_HIP;
         }
+    if (hipMalloc((void **)&c->d_sync, 2 * sizeof(unsigned int)) != hipSuccess ||
+        hipMemset(c->d_sync, 0, 2 * sizeof(unsigned int)) != hipSuccess) {
+        delete c;
+        return FM_ERR_NOMEM;
+    }
+    if (const char *e = getenv("FINCH_DECODE_SPLIT")) c->split_phases = e[0] == '1';
     *out = c;
     return FM_OK;
 }
@@ -253,7 +267,7 @@ extern "C" int fm_ctx_destroy(fm_ctx *c) {
             (void)hipFree(t.S);
             (void)hipFree(t.B);
         }
-    void *ptrs[] = {c->d_layer_ptrs, c->d_gg_ptrs, c->d_act, c->d_eo, c->d_counters,
+    void *ptrs[] = {c->d_layer_ptrs, c->d_gg_ptrs, c->d_act, c->d_eo, c->d_counters, c->d_sync,
                     c->d_stage, c->d_ws};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
@@ -265,11 +279,22 @@ extern "C" int fm_ctx_destroy(fm_ctx *c) {
     return FM_OK;
 }
 
+// After the stream has drained: did a fused decode launch give up on its grid barrier?
+static int check_grid_error(fm_ctx *c) {
+    if (!c->sync_unchecked) return FM_OK;
+    c->sync_unchecked = false;
+    unsigned int flag = 0;
+    HIPCHK(c, hipMemcpy(&flag, c->d_sync + 1, sizeof flag, hipMemcpyDeviceToHost));
+    if (!flag) return FM_OK;
+    HIPCHK(c, hipMemset(c->d_sync + 1, 0, sizeof flag));
+    return fail(c, FM_ERR_HIP, "decode kernel: grid barrier timed out, results are invalid");
+}
+
 extern "C" int fm_sync(fm_ctx *c) {
     if (!c) return FM_ERR_ARG;
     DeviceGuard dg(c->device);
     HIPCHK(c, hipStreamSynchronize(c->stream));
-    return FM_OK;
+    return check_grid_error(c);
 }
 
 extern "C" void *fm_stream(fm_ctx *c) { return c ? (void *)c->stream : nullptr; }
@@ -306,7 +331,7 @@ extern "C" int fm_timer_stop(fm_ctx *c, float *ms) {
 
 extern "C" int fm_kernel_timing(fm_ctx *c, int enable) {
     if (!c) return FM_ERR_ARG;
-    c->ktiming = enable != 0;
+    c->ktiming = enable < 0 ? 0 : (enable > 2 ? 2 : enable);
     c->k1_ms = c->k2_ms = 0.0;
     c->kcalls = 0;
     return FM_OK;
@@ -331,7 +356,7 @@ static int ktiming_collect(fm_ctx *c) {
     c->k1_ms += a;
     c->k2_ms += b;
     c->kcalls++;
-    return FM_OK;
+    return check_grid_error(c);
 }
 
 // ============================================================================
@@ -433,11 +458,13 @@ extern "C" int fm_moe_decode_step_dev(fm_ctx *c, int layer0, int n_layers, const
     DeviceGuard dg(c->device);
     rc = ensure_scratch(c, n_layers, c->geom.hidden, c->geom.inter);
     if (rc) return rc;
+    const bool split = c->split_phases || c->ktiming == 2;
     rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer0, 1, n_layers, d_x, d_idx, d_w,
                                  K, c->d_act, d_expert_out ? d_expert_out : c->d_eo, d_out,
-                                 c->d_counters, flags, c->n_cu, c->stream,
-                                 c->ktiming ? c->kev : nullptr);
+                                 split ? nullptr : c->d_sync, &c->sync_epoch, c->spin_limit,
+                                 flags, c->n_cu, c->stream, c->ktiming ? c->kev : nullptr);
     if (rc) return fail(c, rc, "decode launch failed: %s", hipGetErrorString(hipGetLastError()));
+    if (!split) c->sync_unchecked = true;
     if (c->ktiming) return ktiming_collect(c);
     return FM_OK;
 }
@@ -479,7 +506,7 @@ static int moe_host_call(fm_ctx *c, moe_dev_fn fn, int hidden, int layer, const 
     if (expert_out)
         HIPCHK(c, hipMemcpyAsync(expert_out, st + off_e, ne, hipMemcpyDeviceToHost, c->stream));
     HIPCHK(c, hipStreamSynchronize(c->stream));
-    return FM_OK;
+    return check_grid_error(c);
 }
 
 static int aff_decode_fn(fm_ctx *c, int layer, const float *x, const int32_t *idx, const float *w,
@@ -530,9 +557,11 @@ extern "C" int fm_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, const 
     rc = ensure_scratch(c, M, c->geom.hidden, c->geom.inter);
     if (rc) return rc;
     rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer, 0, M, d_X, d_idx, d_w, K,
-                                 c->d_act, c->d_eo, d_out, c->d_counters, flags, c->n_cu,
-                                 c->stream, nullptr);
+                                 c->d_act, c->d_eo, d_out, c->split_phases ? nullptr : c->d_sync,
+                                 &c->sync_epoch, c->spin_limit, flags, c->n_cu, c->stream,
+                                 nullptr);
     if (rc) return fail(c, rc, "prefill launch failed: %s", hipGetErrorString(hipGetLastError()));
+    if (!c->split_phases) c->sync_unchecked = true;
     return FM_OK;
 }
 

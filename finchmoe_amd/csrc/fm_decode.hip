@@ -19,6 +19,9 @@
 
 namespace {
 
+// waves per workgroup of the streaming kernels: one workgroup per CU, two waves per SIMD
+constexpr int FM_NW = 8;
+
 struct DecodeArgs {
     const uint8_t *const *layer_ptrs;   // [n_layers] device pointers to layer blobs
     FmExpertGeom g;
@@ -35,6 +38,18 @@ struct DecodeArgs {
     int items_per_pair;
     int flags;
 };
+
+// The intermediate vectors (act, expert_out) are written by one phase and read
+// by the next, possibly inside one launch and from a CU behind another L2.
+// They are stored and loaded as device-scope relaxed atomics: such accesses are
+// performed at the level all CUs share, so a consumer that starts after the
+// producer's stores have completed sees them without any cache maintenance.
+__device__ __forceinline__ void fm_st_shared(float *p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float fm_ld_shared(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 // ---------------------------------------------------------------- kernel 1
 template <int BITS, int LPR, bool FP16>
@@ -97,9 +112,8 @@ __global__ __launch_bounds__(256) void fm_gate_up_swiglu(DecodeArgs a) {
 // and renormalisation (finchmoe/infer.m:10190-10204); it needs the whole
 // vector of each expert, so one workgroup covers a layer.
 template <bool GUARD>
-__global__ __launch_bounds__(256) void fm_combine(DecodeArgs a) {
-    __shared__ float red[4];
-    const int l = blockIdx.x;
+__device__ __forceinline__ void fm_combine_rows(const DecodeArgs &a, int l, int j0, int j1,
+                                                float *red) {
     const int H = a.g.hidden, K = a.K;
     const float *eo = a.expert_out + (size_t)l * K * H;
     float wk[FM_MAX_K];
@@ -113,14 +127,15 @@ __global__ __launch_bounds__(256) void fm_combine(DecodeArgs a) {
             if constexpr (GUARD) {
                 float part = 0.0f;
                 for (int j = threadIdx.x; j < H; j += blockDim.x) {
-                    float v = eo[(size_t)k * H + j];
+                    float v = fm_ld_shared(eo + (size_t)k * H + j);
                     part = fmaf(v, v, part);
                 }
                 part = fm_group_sum<64>(part);
                 __syncthreads();
                 if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
                 __syncthreads();
-                float er = red[0] + red[1] + red[2] + red[3];
+                float er = 0.0f;
+                for (int i = 0; i < (int)(blockDim.x >> 6); i++) er += red[i];
                 bool keep = isfinite(er) && er < 1e20f;
                 if (keep) total += w; else w = 0.0f;
             }
@@ -132,16 +147,24 @@ __global__ __launch_bounds__(256) void fm_combine(DecodeArgs a) {
         if (total > 0.0f && total < 0.99f) rn = 1.0f / total;
     }
     float *out = a.out + (size_t)l * H;
-    const int j0 = GUARD ? 0 : blockIdx.y * blockDim.x;
-    const int j1 = GUARD ? H : min(H, j0 + (int)blockDim.x);
     for (int j = j0 + threadIdx.x; j < j1; j += blockDim.x) {
         float acc = 0.0f;
 #pragma unroll
         for (int k = 0; k < FM_MAX_K; k++)
-            if (k < K && wk[k] != 0.0f) acc += wk[k] * eo[(size_t)k * H + j];
+            if (k < K && wk[k] != 0.0f) acc += wk[k] * fm_ld_shared(eo + (size_t)k * H + j);
         if constexpr (GUARD) acc *= rn;
         out[j] = (a.flags & FM_ACCUMULATE) ? out[j] + acc : acc;
     }
+}
+
+// grid: GUARD (n_groups), otherwise (n_groups, ceil(hidden / 256))
+template <bool GUARD>
+__global__ __launch_bounds__(256) void fm_combine(DecodeArgs a) {
+    __shared__ float red[FM_NW];
+    const int H = a.g.hidden;
+    const int j0 = GUARD ? 0 : blockIdx.y * blockDim.x;
+    const int j1 = GUARD ? H : min(H, j0 + (int)blockDim.x);
+    fm_combine_rows<GUARD>(a, blockIdx.x, j0, j1, red);
 }
 
 // ---------------------------------------------------------------- kernel 2
@@ -191,28 +214,61 @@ __global__ __launch_bounds__(256) void fm_down(DecodeArgs a) {
 }
 
 // ======================================================================
-// Matrix-core path (fm_mfma.h): persistent workgroups over a static partition.
+// Matrix-core path (fm_mfma.h): persistent workgroups over a static partition,
+// weight ring in LDS.
 //
 // All row steps of all pairs form one sequence of "units" (a unit = one wave
 // step = 64/LPR rows of one pair).  The launch has a fixed number of
-// workgroups; workgroup g takes the contiguous unit range [U*g/G, U*(g+1)/G),
-// its four waves interleave over it, each with the next unit's loads in
-// flight — so a wave streams tens of kilobytes back to back instead of a few
-// rows, and every wave ends after its own share (no queue, no spinning).
-// A range is cut into segments that share an input vector (a layer for
-// gate/up, a pair for down); per segment the workgroup builds the activation
-// registers once in LDS (fm_build_act_lds) and every wave copies its own.
+// workgroups; workgroup g takes the contiguous unit range [U*g/G, U*(g+1)/G)
+// and its four waves interleave over it — so a wave streams tens of kilobytes
+// back to back instead of a few rows, and every wave ends after its own share
+// (no queue).  A range is cut into segments that share an input vector (a
+// layer for gate/up, a pair for down); per segment the workgroup builds the
+// activation registers once in LDS (fm_build_act_lds) and every wave copies
+// its own.
+//
+// Weight ring.  The rows of one wave step are consecutive rows of one matrix,
+// so a slice is three contiguous byte runs: 64 lanes' worth of codes (3072 or
+// 4096 B), 256 B of scales and 256 B of biases.  The wave copies them with
+// LDS-direct loads (global_load_lds: 64 lanes x 16 B or 4 B land back to back
+// at the address in M0).  They need no destination registers, so several
+// slices per wave are in flight while the multiply keeps the registers, and
+// every load instruction covers whole cache lines.  Each lane then reads its
+// own 48/64 bytes and its scale/bias words back from the slot.
+//
+// Ordering.  LDS-direct loads complete in issue order and count in vmcnt.  A
+// slice is consumed when RING-1 younger slices have been issued, so waiting
+// until at most LOADS*(RING-1) vector-memory operations are outstanding
+// guarantees that it has landed (stores only make the wait stricter); once the
+// loader has run out of work the wait is for zero.  The compiler does not see
+// the dependence between a load into LDS and the consumer's LDS read, so both
+// the wait and the read are explicit.
 // ======================================================================
+template <int BITS>
+struct FmDma {
+    static constexpr int NQ = FmLaneBytes<BITS>::value / 16;
+    static constexpr int WBYTES = FM_WAVE * FmLaneBytes<BITS>::value;
+    static constexpr int TAG = WBYTES + 512;        // trailer: which unit the slice belongs to
+    static constexpr int BYTES = WBYTES + 512 + 16; // codes + scales + biases + trailer
+    static constexpr int LOADS = NQ + 2;
+    // the workgroup's rings must fit in 160 KB of LDS next to the activation image
+    static constexpr int RING = BITS == 3 ? 4 : 3;
+    static constexpr int WG_BYTES = FM_NW * RING * BYTES;
+};
+
+typedef const __attribute__((address_space(1))) void *fm_gptr;
+typedef __attribute__((address_space(3))) void *fm_lptr;
+
 template <int BITS, int LPR>
 __device__ __forceinline__ void fm_unit_lane_offsets(int lane, int row_bytes, int sb_row_bytes,
-                                                     size_t &woff, size_t &soff, int &row_in_step,
-                                                     int &ch) {
+                                                     uint32_t &woff, uint32_t &soff,
+                                                     int &row_in_step, int &ch) {
     const int j = lane & 3;
     ch = (lane >> 2) % LPR;
     const int rq = lane / (4 * LPR);
     row_in_step = 4 * rq + j;
-    woff = (size_t)row_in_step * row_bytes + (size_t)ch * FmLaneBytes<BITS>::value;
-    soff = (size_t)row_in_step * sb_row_bytes + (size_t)ch * 4;
+    woff = (uint32_t)(row_in_step * row_bytes + ch * FmLaneBytes<BITS>::value);
+    soff = (uint32_t)(row_in_step * sb_row_bytes + ch * 4);
 }
 
 __device__ __forceinline__ const uint8_t *fm_pair_blob(const DecodeArgs &a, int p) {
@@ -221,8 +277,7 @@ __device__ __forceinline__ const uint8_t *fm_pair_blob(const DecodeArgs &a, int 
     return a.layer_ptrs[a.layer0 + (p / a.K) * a.layer_stride] + (size_t)e * a.g.expert_size;
 }
 
-// A pointer every lane of the wave agrees on, moved to scalar registers so the
-// loads can use the scalar-base + 32-bit lane offset addressing form.
+// A pointer every lane of the wave agrees on, moved to scalar registers.
 __device__ __forceinline__ const uint8_t *fm_uniform(const uint8_t *p) {
     uintptr_t v = (uintptr_t)p;
     uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
@@ -230,245 +285,502 @@ __device__ __forceinline__ const uint8_t *fm_uniform(const uint8_t *p) {
     return (const uint8_t *)(((uintptr_t)hi << 32) | lo);
 }
 
-// gate + up + SwiGLU.  a.items_per_pair carries the number of pairs.
-//
-// Pipeline: the wave walks "half steps" — gate rows of a unit, then up rows of
-// the same unit — through a ring of three register slices: while slice k is
-// being multiplied, the loads of the next two half steps are in flight (a full
-// unit, ~6.6 KB per wave).  The loop is unrolled by three units so the ring
-// rotates without register copies.
-template <int BITS, int LPR, bool FP16>
-__global__ __launch_bounds__(256)
-void fm_gate_up_swiglu_mfma(DecodeArgs a) {
-    constexpr int RPS = FM_WAVE / LPR;
-    __shared__ FmActLds<LPR> lds;
-    __shared__ const uint8_t *lds_blob[FM_MAX_K];
+template <int BITS, int I>
+__device__ __forceinline__ void fm_dma_codes(uint32_t slot, fm_gptr w) {
+    if constexpr (I < FmDma<BITS>::NQ) {
+        // the instruction offset moves the global and the LDS address alike
+        __builtin_amdgcn_global_load_lds(w, (fm_lptr)(uintptr_t)slot, 16, 1024 * I, 0);
+        fm_dma_codes<BITS, I + 1>(slot, w);
+    }
+}
+
+// w, s, b: first byte of the unit's rows in the weight, scale and bias regions
+template <int BITS>
+__device__ __forceinline__ void fm_dma_issue(uint32_t slot, const uint8_t *w, const uint8_t *s,
+                                             const uint8_t *b, int lane) {
+    fm_dma_codes<BITS, 0>(slot, (fm_gptr)(uintptr_t)(w + lane * 16));
+    __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(s + lane * 4),
+                                     (fm_lptr)(uintptr_t)(slot + FmDma<BITS>::WBYTES), 4, 0, 0);
+    __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(b + lane * 4),
+                                     (fm_lptr)(uintptr_t)(slot + FmDma<BITS>::WBYTES + 256), 4, 0, 0);
+}
+
+template <int N>
+__device__ __forceinline__ void fm_dma_wait(bool drain) {
+    if (drain) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// this lane's codes and scale/bias words out of a landed slot
+// (returns the slot's tag)
+template <int BITS>
+__device__ __forceinline__ uint32_t fm_dma_read(uint32_t slot, uint32_t woff, uint32_t soff,
+                                                FmRowSlice<BITS> &t) {
+    const uint32_t aw = slot + woff, as = slot + FmDma<BITS>::WBYTES + soff;
+    const uint32_t at = slot + FmDma<BITS>::TAG;
+    uint32_t tag;
+    if constexpr (BITS == 3) {
+        asm volatile("ds_read_b128 %0, %6\n\tds_read_b128 %1, %6 offset:16\n\t"
+                     "ds_read_b128 %2, %6 offset:32\n\tds_read_b32 %3, %7\n\t"
+                     "ds_read_b32 %4, %7 offset:256\n\tds_read_b32 %5, %8\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&v"(t.q[0]), "=&v"(t.q[1]), "=&v"(t.q[2]), "=&v"(t.s), "=&v"(t.b),
+                       "=&v"(tag)
+                     : "v"(aw), "v"(as), "v"(at)
+                     : "memory");
+    } else {
+        asm volatile("ds_read_b128 %0, %7\n\tds_read_b128 %1, %7 offset:16\n\t"
+                     "ds_read_b128 %2, %7 offset:32\n\tds_read_b128 %3, %7 offset:48\n\t"
+                     "ds_read_b32 %4, %8\n\tds_read_b32 %5, %8 offset:256\n\t"
+                     "ds_read_b32 %6, %9\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(t.q[0]), "=&v"(t.q[1]), "=&v"(t.q[2]), "=&v"(t.q[3]), "=&v"(t.s),
+                       "=&v"(t.b), "=&v"(tag)
+                     : "v"(aw), "v"(as), "v"(at)
+                     : "memory");
+    }
+    return __builtin_amdgcn_readfirstlane(tag);
+}
+
+// Dynamic LDS of the streaming kernels: ring [FM_NW][RING] slots, then the
+// activation image, then (gate/up only) the layer's blob table and valid mask.
+extern __shared__ __attribute__((aligned(16))) uint8_t fm_dyn_lds[];
+
+template <int BITS, int LPR_UP>
+constexpr size_t fm_stream_lds_bytes() {
+    return FmDma<BITS>::WG_BYTES + sizeof(FmActLds<LPR_UP>) + FM_MAX_K * sizeof(void *) + 16;
+}
+
+struct FmNoSync {
+    __device__ __forceinline__ void operator()() const {}
+};
+
+// Units of a segment are handed out one at a time from a counter in LDS: the
+// hardware favours the older of two waves that share a SIMD, so with a fixed
+// share per wave the favoured half finishes early and the CU runs the rest of
+// the kernel half empty.  With a shared counter every wave of the workgroup
+// ends within one unit of the others.
+// (Written as an instruction: the compiler would make an LDS atomic wait for
+// every outstanding LDS-direct load, which empties the ring.)
+__device__ __forceinline__ uint32_t fm_claim_unit(unsigned int *next, int lane) {
+    uint32_t v = 0;
+    if (lane == 0) {
+        const uint32_t addr = (uint32_t)(uintptr_t)(fm_lptr)next, one = 1u;
+        asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(v)
+                     : "v"(addr), "v"(one)
+                     : "memory");
+    }
+    return __builtin_amdgcn_readfirstlane(v);
+}
+
+// tag of the slice in a slot (which unit it belongs to), kept in the slot's
+// trailer so that the consumer needs no queue in registers
+__device__ __forceinline__ void fm_slot_tag(uint32_t slot_tag_addr, uint32_t tag) {
+    asm volatile("ds_write_b32 %0, %1" ::"v"(slot_tag_addr), "v"(tag) : "memory");
+}
+
+// gate + up + SwiGLU over this workgroup's share of the n_pairs * inter/RPS units.
+// An invalid expert index streams expert 0 and contributes zero.  `before_build`
+// runs once, after the first segment's loads are in flight and before the first
+// read of a.x.
+template <int BITS, int LPR, bool FP16, class Sync>
+__device__ __forceinline__ void fm_gate_up_phase(const DecodeArgs &a, int n_pairs,
+                                                 unsigned int *next_unit, Sync before_build) {
+    using D = FmDma<BITS>;
+    constexpr int RPS = FM_WAVE / LPR, RING = D::RING;
+    FmActLds<LPR> &lds = *reinterpret_cast<FmActLds<LPR> *>(fm_dyn_lds + D::WG_BYTES);
+    const uint8_t **lds_blob =
+        reinterpret_cast<const uint8_t **>(fm_dyn_lds + D::WG_BYTES + sizeof(FmActLds<LPR>));
+    uint32_t *lds_valid = reinterpret_cast<uint32_t *>(lds_blob + FM_MAX_K);
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int n_pairs = a.items_per_pair;
-    const int upp = a.g.inter / RPS;        // units per pair (>= 4)
+    const uint32_t ring0 =
+        (uint32_t)(uintptr_t)(fm_lptr)fm_dyn_lds + (uint32_t)wave * (RING * D::BYTES);
+    const int upp = a.g.inter / RPS;        // units per pair
     const long upl = (long)upp * a.K;       // units per layer
     const long total = (long)n_pairs * upp;
     const long wg0 = total * blockIdx.x / gridDim.x, wg1 = total * (blockIdx.x + 1) / gridDim.x;
     const int row_bytes = a.g.hidden * BITS / 8, sb_row_bytes = (a.g.hidden / 64) * 2;
-    size_t woff_, soff_;
+    uint32_t woff, soff;
     int ris, ch;
-    fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff_, soff_, ris, ch);
-    const uint32_t woff = (uint32_t)woff_, soff = (uint32_t)soff_;
+    fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff, soff, ris, ch);
     const uint32_t wstep = (uint32_t)(RPS * row_bytes), sstep = (uint32_t)(RPS * sb_row_bytes);
+    // region offsets as scalars (selected per half step with a scalar select)
+    const auto gw = a.g.gate_w, gs = a.g.gate_s, gb = a.g.gate_b;
+    const auto uw = a.g.up_w, us = a.g.up_s, ub = a.g.up_b;
     FmBuildSlot<BITS> bslot;
     bslot.init();
+    bool first = true;
 
     for (long seg0 = wg0; seg0 < wg1;) {
         const int l = (int)(seg0 / upl);
         long seg1 = (long)(l + 1) * upl;
         if (seg1 > wg1) seg1 = wg1;
+        const uint32_t seg_n = (uint32_t)(seg1 - seg0);
+        const uint32_t u_first = (uint32_t)(seg0 - (long)l * upl);   // first unit, in the layer
         __syncthreads();                          // previous segment's readers are done
-        if (threadIdx.x < a.K) lds_blob[threadIdx.x] = fm_pair_blob(a, l * a.K + threadIdx.x);
-        __syncthreads();
-        // loader: half step (pair pn, row step rsn, matrix hn) of this wave
-        long u = seg0 + wave;          // unit being computed
-        long un = u;                   // unit being loaded
-        int pn = (int)(u / upp) - l * a.K, rsn = (int)(u % upp), hn = 0;
-        const uint8_t *blob_n = un < seg1 ? fm_uniform(lds_blob[pn]) : nullptr;
-        const uint8_t *blob_c = blob_n;            // blob of the unit being computed
-        const uint8_t *blob_q[2] = {blob_n, blob_n};   // blobs of the units in flight
-        auto load_half = [&](FmRowSlice<BITS> &t) {
-            if (un < seg1) {
-                if (blob_n) {
-                    const uint8_t *b = blob_n + (size_t)rsn * wstep;
-                    const uint8_t *sb = blob_n + (size_t)rsn * sstep;
-                    if (hn == 0)
-                        fm_load_slice<BITS>(t, b + a.g.gate_w + woff, sb + a.g.gate_s + soff,
-                                            sb + a.g.gate_b + soff);
-                    else
-                        fm_load_slice<BITS>(t, b + a.g.up_w + woff, sb + a.g.up_s + soff,
-                                            sb + a.g.up_b + soff);
-                }
-                if (hn == 1) {
-                    un += 4;
-                    rsn += 4;
-                    if (rsn >= upp) {
-                        rsn -= upp;
-                        pn++;
-                        if (un < seg1) blob_n = fm_uniform(lds_blob[pn]);
-                    }
-                }
-                hn ^= 1;
+        if (threadIdx.x < 64) {
+            bool ok = false;
+            if (lane < a.K) {
+                const int e = a.idx[l * a.K + lane];
+                ok = (unsigned)e < (unsigned)a.g.n_experts;
+                lds_blob[lane] = a.layer_ptrs[a.layer0 + l * a.layer_stride] +
+                                 (size_t)(ok ? e : 0) * a.g.expert_size;
             }
+            const uint64_t m = __ballot(ok);
+            if (lane == 0) {
+                lds_valid[0] = (uint32_t)m;
+                *next_unit = 0u;
+            }
+        }
+        __syncthreads();
+        const uint32_t valid = __builtin_amdgcn_readfirstlane(lds_valid[0]);
+        // loader: the next half step (gate rows, then up rows of the same unit)
+        int hn = 0;
+        uint32_t tag_n = 0, rsn = 0, issued = 0, consumed = 0;
+        const uint8_t *blob_n = nullptr;
+        bool drain = false;
+        auto issue = [&](int slot_idx) {
+            if (drain) return;
+            if (hn == 0) {
+                const uint32_t ul = fm_claim_unit(next_unit, lane);
+                if (ul >= seg_n) {
+                    drain = true;
+                    return;
+                }
+                const uint32_t uq = u_first + ul;            // unit inside the layer
+                const uint32_t pn = uq / (uint32_t)upp;
+                rsn = uq - pn * (uint32_t)upp;
+                tag_n = (pn << 28) | ul;
+                blob_n = fm_uniform(lds_blob[pn]);
+            }
+            const uint32_t slot = ring0 + (uint32_t)slot_idx * D::BYTES;
+            fm_slot_tag(slot + D::TAG, tag_n);
+            const uint8_t *b = blob_n + (size_t)rsn * wstep;
+            const uint8_t *sb = blob_n + (size_t)rsn * sstep;
+            fm_dma_issue<BITS>(slot, b + (hn ? uw : gw), sb + (hn ? us : gs),
+                               sb + (hn ? ub : gb), lane);
+            hn ^= 1;
+            issued++;
         };
-        FmRowSlice<BITS> r0, r1, r2;
-        load_half(r0);                            // one unit in flight during the build
-        load_half(r1);
-        blob_q[0] = blob_n;                       // blob of unit u+4 (after the two loads)
-        fm_build_act_lds<BITS, LPR>(a.x + (size_t)l * a.g.hidden, bslot, lds);
+#pragma unroll
+        for (int k = 0; k < RING; k++) issue(k);
+        if (first) {
+            before_build();
+            first = false;
+        }
+        if (threadIdx.x < 256)
+            fm_build_act_lds<BITS, LPR, false>(a.x + (size_t)l * a.g.hidden, bslot, lds);
         __syncthreads();
         FmActRegs ar;
         fm_read_act_lds<LPR>(lds, lane, ar);
-        float gv = 0.0f;
-        // one half step: start the load two half steps ahead, multiply the current slice
-        auto gate_step = [&](FmRowSlice<BITS> &cur, FmRowSlice<BITS> &tgt) {
-            load_half(tgt);
-            if (blob_c) gv = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(cur, ar));
+        int c = 0;
+        uint32_t tag = 0;
+        auto half = [&]() {
+            FmRowSlice<BITS> t;
+            fm_dma_wait<D::LOADS *(RING - 1)>(drain);
+            tag = fm_dma_read<BITS>(ring0 + (uint32_t)c * D::BYTES, woff, soff, t);
+            consumed++;
+            issue(c);
+            c = c + 1 == RING ? 0 : c + 1;
+            return fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(t, ar));
         };
-        auto up_step = [&](FmRowSlice<BITS> &cur, FmRowSlice<BITS> &tgt) {
-            // the load issued here is the up half of unit u+4... its blob is blob_q[0]
-            load_half(tgt);
-            float v = 0.0f;
-            if (blob_c) {
-                float uv = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(cur, ar));
-                v = fm_silu_mul(gv, uv);
-            }
-            // unit u = (pair, row step): act is [pair][inter], rows are contiguous
-            if (ch == 0) a.act[(size_t)u * RPS + ris] = v;
-            u += 4;
-            blob_c = blob_q[0];
-            blob_q[0] = blob_n;
-        };
-        while (u < seg1) {
-            gate_step(r0, r2);
-            up_step(r1, r0);
-            if (u >= seg1) break;
-            gate_step(r2, r1);
-            up_step(r0, r2);
-            if (u >= seg1) break;
-            gate_step(r1, r0);
-            up_step(r2, r1);
+        while (consumed < issued) {
+            const float gv = half();
+            const float uv = half();
+            const uint32_t pc = tag >> 28, ul = tag & 0x0FFFFFFFu;
+            const float v = ((valid >> pc) & 1u) ? fm_silu_mul(gv, uv) : 0.0f;
+            // unit (pair, row step): act is [pair][inter], rows are contiguous
+            if (ch == 0) fm_st_shared(a.act + (size_t)(seg0 + ul) * RPS + ris, v);
         }
         seg0 = seg1;
     }
+    if (first) before_build();
 }
 
-// down projection -> per-expert output vectors.  Ring of three slices: two units
-// of loads in flight ahead of the one being multiplied.
-template <int BITS, int LPR, bool FP16>
-__global__ __launch_bounds__(256)
-void fm_down_mfma(DecodeArgs a) {
-    constexpr int RPS = FM_WAVE / LPR;
-    __shared__ FmActLds<LPR> lds;
+// down projection -> per-expert output vectors over this workgroup's share of
+// the n_pairs * hidden/RPS units.  `before_build` as above (first read of a.act).
+template <int BITS, int LPR, bool FP16, class Sync>
+__device__ __forceinline__ void fm_down_phase(const DecodeArgs &a, int n_pairs,
+                                              unsigned int *next_unit, Sync before_build) {
+    using D = FmDma<BITS>;
+    constexpr int RPS = FM_WAVE / LPR, RING = D::RING;
+    FmActLds<LPR> &lds = *reinterpret_cast<FmActLds<LPR> *>(fm_dyn_lds + D::WG_BYTES);
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int n_pairs = a.items_per_pair;
+    const uint32_t ring0 =
+        (uint32_t)(uintptr_t)(fm_lptr)fm_dyn_lds + (uint32_t)wave * (RING * D::BYTES);
     const int upp = a.g.hidden / RPS;
     const long total = (long)n_pairs * upp;
     const long wg0 = total * blockIdx.x / gridDim.x, wg1 = total * (blockIdx.x + 1) / gridDim.x;
     const int row_bytes = a.g.inter * BITS / 8, sb_row_bytes = (a.g.inter / 64) * 2;
-    size_t woff_, soff_;
+    uint32_t woff, soff;
     int ris, ch;
-    fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff_, soff_, ris, ch);
-    const uint32_t woff = (uint32_t)woff_, soff = (uint32_t)soff_;
+    fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff, soff, ris, ch);
     const uint32_t wstep = (uint32_t)(RPS * row_bytes), sstep = (uint32_t)(RPS * sb_row_bytes);
     FmBuildSlot<BITS> bslot;
     bslot.init();
+    bool first = true;
 
     for (long seg0 = wg0; seg0 < wg1;) {
         const int p = (int)(seg0 / upp);
         long seg1 = (long)(p + 1) * upp;
         if (seg1 > wg1) seg1 = wg1;
+        const uint32_t seg_n = (uint32_t)(seg1 - seg0);
+        const uint32_t rs_first = (uint32_t)(seg0 - (long)p * upp);
         const uint8_t *blob = fm_pair_blob(a, p);
-        long u = seg0 + wave;
-        int rsn = (int)(u - (long)p * upp);
-        long un = u;
-        auto load_next = [&](FmRowSlice<BITS> &ds) {
-            if (un < seg1) {
-                const uint8_t *b = blob + (size_t)rsn * wstep;
-                const uint8_t *sb = blob + (size_t)rsn * sstep;
-                fm_load_slice<BITS>(ds, b + a.g.down_w + woff, sb + a.g.down_s + soff,
-                                    sb + a.g.down_b + soff);
-                un += 4;
-                rsn += 4;
+        uint32_t issued = 0, consumed = 0;
+        bool drain = false;
+        auto issue = [&](int slot_idx) {
+            if (drain) return;
+            const uint32_t ul = fm_claim_unit(next_unit, lane);
+            if (ul >= seg_n) {
+                drain = true;
+                return;
             }
+            const uint32_t slot = ring0 + (uint32_t)slot_idx * D::BYTES;
+            fm_slot_tag(slot + D::TAG, ul);
+            const uint8_t *b = blob + (size_t)(rs_first + ul) * wstep;
+            const uint8_t *sb = blob + (size_t)(rs_first + ul) * sstep;
+            fm_dma_issue<BITS>(slot, b + a.g.down_w, sb + a.g.down_s, sb + a.g.down_b, lane);
+            issued++;
         };
+        __syncthreads();                          // previous segment's readers are done
+        if (threadIdx.x == 0) *next_unit = 0u;
         __syncthreads();
         if (blob) {
-            FmRowSlice<BITS> r0, r1, r2;
-            load_next(r0);
-            load_next(r1);
-            fm_build_act_lds<BITS, LPR>(a.act + (size_t)p * a.g.inter, bslot, lds);
+#pragma unroll
+            for (int k = 0; k < RING; k++) issue(k);
+        }
+        if (first) {
+            before_build();
+            first = false;
+        }
+        if (blob) {
+            if (threadIdx.x < 256)
+                fm_build_act_lds<BITS, LPR, true>(a.act + (size_t)p * a.g.inter, bslot, lds);
             __syncthreads();
             FmActRegs ar;
             fm_read_act_lds<LPR>(lds, lane, ar);
-            auto step = [&](FmRowSlice<BITS> &cur, FmRowSlice<BITS> &tgt) {
-                load_next(tgt);
-                float v = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(cur, ar));
-                if (ch == 0) a.expert_out[(size_t)u * RPS + ris] = v;
-                u += 4;
-            };
-            while (u < seg1) {
-                step(r0, r2);
-                if (u >= seg1) break;
-                step(r1, r0);
-                if (u >= seg1) break;
-                step(r2, r1);
+            int c = 0;
+            while (consumed < issued) {
+                FmRowSlice<BITS> t;
+                fm_dma_wait<D::LOADS *(RING - 1)>(drain);
+                const uint32_t ul = fm_dma_read<BITS>(ring0 + (uint32_t)c * D::BYTES, woff, soff, t);
+                consumed++;
+                issue(c);
+                c = c + 1 == RING ? 0 : c + 1;
+                const float v = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(t, ar));
+                if (ch == 0) fm_st_shared(a.expert_out + (size_t)(seg0 + ul) * RPS + ris, v);
             }
         } else {
-            for (; u < seg1; u += 4)
-                if (ch == 0) a.expert_out[(size_t)u * RPS + ris] = 0.0f;
+            for (long u = seg0 + (threadIdx.x >> 6); u < seg1; u += FM_NW)
+                if (ch == 0) fm_st_shared(a.expert_out + (size_t)u * RPS + ris, 0.0f);
         }
         seg0 = seg1;
     }
+    if (first) before_build();
+}
+
+template <int BITS, int LPR, bool FP16>
+__global__ __launch_bounds__(FM_NW * 64) void fm_gate_up_swiglu_lds(DecodeArgs a, int n_pairs) {
+    __shared__ unsigned int next_unit;
+    fm_gate_up_phase<BITS, LPR, FP16>(a, n_pairs, &next_unit, FmNoSync());
+}
+
+template <int BITS, int LPR, bool FP16>
+__global__ __launch_bounds__(FM_NW * 64) void fm_down_lds(DecodeArgs a, int n_pairs) {
+    __shared__ unsigned int next_unit;
+    fm_down_phase<BITS, LPR, FP16>(a, n_pairs, &next_unit, FmNoSync());
+}
+
+// ======================================================================
+// One launch for the whole operator: gate/up, down and combine as three phases
+// of one persistent grid, separated by grid-wide barriers.
+//
+// What the barrier buys: a phase's weights do not depend on the previous
+// phase, so every wave issues the first RING slices of its next share before
+// it waits — the memory pipeline stays full across the phase change, where
+// separate kernels drain it, relaunch and refill it.
+//
+// The barrier is an arrival counter in device memory that only ever grows: the
+// host hands each launch the value the counter had before it (`base`) and adds
+// two arrivals per workgroup afterwards, so nothing is reset between launches.
+// What crosses the barrier (act, expert_out) is stored and loaded at device
+// scope (fm_st_shared / fm_ld_shared), so a workgroup arrives once its waves'
+// stores have completed and no cache is written back or invalidated — device-
+// scope fences cost more here than the barrier saves.  Every workgroup of the grid must be resident at once — the
+// launcher sizes the grid from the occupancy query — and the wait is bounded:
+// past `spin_limit` polls a workgroup raises `*err` and goes on (results are
+// then wrong, the host reports the error, and the counter stays consistent
+// because every workgroup still arrives exactly twice).
+// ======================================================================
+struct FmGridSync {
+    unsigned int *counter;
+    unsigned int *err;
+    unsigned int base;
+    unsigned int spin_limit;
+};
+
+__device__ __forceinline__ void fm_grid_arrive(const FmGridSync &s) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's stores have completed
+    __syncthreads();
+    if (threadIdx.x == 0)
+        __hip_atomic_fetch_add(s.counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void fm_grid_wait(const FmGridSync &s, unsigned int target) {
+    if (threadIdx.x == 0) {
+        unsigned int polls = 0;
+        while ((int)(__hip_atomic_load(s.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) -
+                     target) < 0) {
+            if (++polls > s.spin_limit) {
+                __hip_atomic_store(s.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(8);
+        }
+    }
+    __syncthreads();
+}
+
+template <int BITS, int LPR_UP, bool FP16>
+__global__ __launch_bounds__(FM_NW * 64)
+void fm_moe_fused(DecodeArgs a, int n_pairs, FmGridSync sy) {
+    constexpr int LPR_DOWN = LPR_UP / 4;
+    __shared__ float red[FM_NW];
+    __shared__ unsigned int next_unit;
+    const unsigned int G = gridDim.x;
+    fm_gate_up_phase<BITS, LPR_UP, FP16>(a, n_pairs, &next_unit, FmNoSync());
+    fm_grid_arrive(sy);
+    fm_down_phase<BITS, LPR_DOWN, FP16>(a, n_pairs, &next_unit,
+                                        [&]() { fm_grid_wait(sy, sy.base + G); });
+    fm_grid_arrive(sy);
+    fm_grid_wait(sy, sy.base + 2 * G);
+    const int n_groups = n_pairs / a.K, H = a.g.hidden;
+    if (a.flags & FM_GUARD) {
+        for (int l = blockIdx.x; l < n_groups; l += G) fm_combine_rows<true>(a, l, 0, H, red);
+    } else {
+        const int cols = FM_NW * 64, per = (H + cols - 1) / cols;
+        for (int it = blockIdx.x; it < n_groups * per; it += G) {
+            const int l = it / per, j0 = (it - l * per) * cols;
+            fm_combine_rows<false>(a, l, j0, min(H, j0 + cols), red);
+        }
+    }
+}
+
+// Raise a kernel's dynamic LDS limit (the default stops at 64 KB).  Called on
+// every launch: the attribute belongs to the current device's copy of the kernel.
+bool fm_dyn_lds_ok(const void *fn, size_t bytes) {
+    return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) ==
+           hipSuccess;
+}
+
+// workgroups of a streaming launch: one per CU (LDS budget), fewer when there
+// are not enough units to give every wave `per_wave` of them
+dim3 fm_stream_grid(long units, int n_cu, int per_wave) {
+    long wgs = (long)n_cu;
+    const long need = (long)FM_NW * per_wave;
+    if (units < need * wgs) wgs = (units + need - 1) / need;
+    if (wgs < 1) wgs = 1;
+    return dim3((unsigned)wgs);
+}
+
+// One fused launch.  Returns FM_ERR_UNSUPPORTED when the grid cannot be made
+// fully resident (the caller then uses separate kernels).
+template <int BITS, int LPR_UP, bool FP16>
+int launch_fused(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st, FmGridSync sy,
+                 unsigned int *epoch) {
+    auto kfn = fm_moe_fused<BITS, LPR_UP, FP16>;
+    const size_t sh = fm_stream_lds_bytes<BITS, LPR_UP>();
+    if (!fm_dyn_lds_ok((const void *)kfn, sh)) return FM_ERR_HIP;
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kfn, FM_NW * 64, sh) !=
+            hipSuccess ||
+        per_cu < 1)
+        return FM_ERR_UNSUPPORTED;
+    per_cu = 1;
+    const long up_units = (long)n_pairs * (a.g.inter / (FM_WAVE / LPR_UP));
+    const long down_units = (long)n_pairs * (a.g.hidden / (FM_WAVE / (LPR_UP / 4)));
+    long wgs = (long)n_cu * per_cu;
+    const long small = up_units < down_units ? up_units : down_units;
+    if (small < FM_NW * wgs) wgs = (small + FM_NW - 1) / FM_NW;
+    if (wgs < 1) wgs = 1;
+    sy.base = *epoch;
+    *epoch += 2u * (unsigned)wgs;
+    hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(FM_NW * 64), sh, st, a, n_pairs, sy);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 
 template <int BITS, bool FP16>
 int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down, int n_cu,
-                    hipStream_t st, hipEvent_t *kev) {
-    DecodeArgs a1 = a, a2 = a;
-    a1.rows_per_item = rpi_up;
-    a1.items_per_pair = a.g.inter / rpi_up;
-    a2.rows_per_item = rpi_down;
-    a2.items_per_pair = a.g.hidden / rpi_down;
+                    hipStream_t st, hipEvent_t *kev, const FmGridSync *sy, unsigned int *epoch) {
     dim3 b(256);
     const int lpr_up = a.g.hidden / FM_CPL, lpr_down = a.g.inter / FM_CPL;
-    // matrix-core path: one wave per SIMD slot that the register budget allows,
-    // fewer when there are not enough units to give every wave two
-    const bool mfma_up = lpr_up >= 4 && lpr_up <= 16, mfma_down = lpr_down <= 16;
-    // two workgroups per CU (register budget); fewer when the launch has too few
-    // units to give every wave two
-    auto stream_grid = [&](long units) {
-        long wgs = (long)n_cu * 2;
-        if (units < 8 * wgs) wgs = (units + 7) / 8;
-        if (wgs < 1) wgs = 1;
-        return dim3((unsigned)wgs);
-    };
+    const bool lds_up = lpr_up >= 4 && lpr_up <= 16, lds_down = lpr_down <= 16;
+    if (!lds_down) return FM_ERR_UNSUPPORTED;
     if (kev) (void)hipEventRecord(kev[0], st);
-    if (mfma_up) {
-        DecodeArgs am = a;
-        am.items_per_pair = n_pairs;
-        dim3 g = stream_grid((long)n_pairs * (a.g.inter / (FM_WAVE / lpr_up)));
-#define FM_UPM(L) hipLaunchKernelGGL((fm_gate_up_swiglu_mfma<BITS, L, FP16>), g, b, 0, st, am)
+    if (sy && epoch && lds_up && lpr_down * 4 == lpr_up) {
+        int rc = FM_ERR_UNSUPPORTED;
         switch (lpr_up) {
-            case 4: FM_UPM(4); break;
-            case 8: FM_UPM(8); break;
-            default: FM_UPM(16); break;
+            case 4: rc = launch_fused<BITS, 4, FP16>(a, n_pairs, n_cu, st, *sy, epoch); break;
+            case 8: rc = launch_fused<BITS, 8, FP16>(a, n_pairs, n_cu, st, *sy, epoch); break;
+            case 16: rc = launch_fused<BITS, 16, FP16>(a, n_pairs, n_cu, st, *sy, epoch); break;
         }
-#undef FM_UPM
-    } else {
-#define FM_UP(L) \
-    hipLaunchKernelGGL((fm_gate_up_swiglu<BITS, L, FP16>), dim3(n_pairs * a1.items_per_pair), b, 0, st, a1)
+        if (rc != FM_ERR_UNSUPPORTED) {
+            if (kev) {
+                (void)hipEventRecord(kev[1], st);
+                (void)hipEventRecord(kev[2], st);
+            }
+            return rc;
+        }
+    }
+    if (lds_up) {
+        const long units = (long)n_pairs * (a.g.inter / (FM_WAVE / lpr_up));
+        const dim3 g = fm_stream_grid(units, n_cu, 2);
+#define FM_UP(L)                                                                   \
+    do {                                                                           \
+        auto kfn = fm_gate_up_swiglu_lds<BITS, L, FP16>;                           \
+        const size_t sh = fm_stream_lds_bytes<BITS, L>();                          \
+        if (!fm_dyn_lds_ok((const void *)kfn, sh)) return FM_ERR_HIP;              \
+        hipLaunchKernelGGL(kfn, g, dim3(FM_NW * 64), sh, st, a, n_pairs);          \
+    } while (0)
         switch (lpr_up) {
-            case 32: FM_UP(32); break;
-            default: return FM_ERR_UNSUPPORTED;
+            case 4: FM_UP(4); break;
+            case 8: FM_UP(8); break;
+            default: FM_UP(16); break;
         }
 #undef FM_UP
-    }
-    if (kev) (void)hipEventRecord(kev[1], st);
-    if (mfma_down) {
-        DecodeArgs am = a;
-        am.items_per_pair = n_pairs;
-        dim3 g = stream_grid((long)n_pairs * (a.g.hidden / (FM_WAVE / lpr_down)));
-#define FM_DOWNM(L) hipLaunchKernelGGL((fm_down_mfma<BITS, L, FP16>), g, b, 0, st, am)
-        switch (lpr_down) {
-            case 1: FM_DOWNM(1); break;
-            case 2: FM_DOWNM(2); break;
-            case 4: FM_DOWNM(4); break;
-            case 8: FM_DOWNM(8); break;
-            default: FM_DOWNM(16); break;
-        }
-#undef FM_DOWNM
+    } else if (lpr_up == 32) {
+        DecodeArgs a1 = a;
+        a1.rows_per_item = rpi_up;
+        a1.items_per_pair = a.g.inter / rpi_up;
+        hipLaunchKernelGGL((fm_gate_up_swiglu<BITS, 32, FP16>), dim3(n_pairs * a1.items_per_pair),
+                           b, 0, st, a1);
     } else {
         return FM_ERR_UNSUPPORTED;
     }
-    (void)a2;
+    (void)rpi_down;
+    if (kev) (void)hipEventRecord(kev[1], st);
+    {
+        const long units = (long)n_pairs * (a.g.hidden / (FM_WAVE / lpr_down));
+        const dim3 g = fm_stream_grid(units, n_cu, 2);
+#define FM_DOWN(L)                                                                 \
+    do {                                                                           \
+        auto kfn = fm_down_lds<BITS, L, FP16>;                                     \
+        const size_t sh = FmDma<BITS>::WG_BYTES + sizeof(FmActLds<L>);             \
+        if (!fm_dyn_lds_ok((const void *)kfn, sh)) return FM_ERR_HIP;              \
+        hipLaunchKernelGGL(kfn, g, dim3(FM_NW * 64), sh, st, a, n_pairs);          \
+    } while (0)
+        switch (lpr_down) {
+            case 1: FM_DOWN(1); break;
+            case 2: FM_DOWN(2); break;
+            case 4: FM_DOWN(4); break;
+            case 8: FM_DOWN(8); break;
+            default: FM_DOWN(16); break;
+        }
+#undef FM_DOWN
+    }
     const int n_groups = n_pairs / a.K;
     if (a.flags & FM_GUARD)
         hipLaunchKernelGGL(fm_combine<true>, dim3(n_groups), b, 0, st, a);
@@ -489,7 +801,7 @@ int pick_rows_per_item(int rows, int n_pairs, int min_rows, int cap, int want) {
 
 }  // namespace
 
-// Enqueue both kernels for n_layers x K pairs (n_layers groups of K slots: the
+// Enqueue the operator for n_layers x K pairs (n_layers groups of K slots: the
 // layers of a decode step, or with layer_stride 0 the positions of a chunk).  Shapes are validated by the
 // caller (fm_api.cpp): hidden, inter multiples of 128 with a supported
 // lanes-per-row, every layer resident.
@@ -498,7 +810,8 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
                                        int n_layers, const float *d_x, const int32_t *d_idx,
                                        const float *d_w, int K, float *d_act,
                                        float *d_expert_out, float *d_out,
-                                       unsigned int *d_counters, int flags, int n_cu,
+                                       unsigned int *d_sync, unsigned int *epoch,
+                                       unsigned int spin_limit, int flags, int n_cu,
                                        hipStream_t st, hipEvent_t *kev) {
     DecodeArgs a;
     a.layer_ptrs = d_layer_ptrs;
@@ -512,7 +825,6 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     a.act = d_act;
     a.expert_out = d_expert_out;
     a.out = d_out;
-    (void)d_counters;
     a.flags = flags;
     a.rows_per_item = a.items_per_pair = 0;
     const int n_pairs = n_layers * K;
@@ -524,13 +836,13 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     const int want = 4 * n_cu;
     const int rpi_up = pick_rows_per_item(g->inter, n_pairs, min_up, 64, want);
     const int rpi_down = pick_rows_per_item(g->hidden, n_pairs, min_down, 256, want);
-    if (g->bits == 3) {
-        return g->scale_fp16 ? launch_decode_t<3, true>(a, n_pairs, rpi_up, rpi_down, n_cu, st, kev)
-                             : launch_decode_t<3, false>(a, n_pairs, rpi_up, rpi_down, n_cu, st, kev);
-    }
-    if (g->bits == 4) {
-        return g->scale_fp16 ? launch_decode_t<4, true>(a, n_pairs, rpi_up, rpi_down, n_cu, st, kev)
-                             : launch_decode_t<4, false>(a, n_pairs, rpi_up, rpi_down, n_cu, st, kev);
-    }
+    // d_sync[0] = arrival counter, d_sync[1] = error flag; without them (or with
+    // epoch == NULL) the phases run as separate kernels
+    FmGridSync sy{d_sync, d_sync ? d_sync + 1 : nullptr, 0u, spin_limit};
+    const FmGridSync *syp = d_sync && epoch ? &sy : nullptr;
+#define FM_DEC(B, F) launch_decode_t<B, F>(a, n_pairs, rpi_up, rpi_down, n_cu, st, kev, syp, epoch)
+    if (g->bits == 3) return g->scale_fp16 ? FM_DEC(3, true) : FM_DEC(3, false);
+    if (g->bits == 4) return g->scale_fp16 ? FM_DEC(4, true) : FM_DEC(4, false);
+#undef FM_DEC
     return FM_ERR_UNSUPPORTED;
 }

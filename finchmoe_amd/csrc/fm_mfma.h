@@ -176,9 +176,17 @@ struct FmBuildSlot {
 
 // All 256 threads.  x = the 128*LPR activations in global memory.  The caller
 // puts a barrier before (previous readers done) and after (image complete).
-template <int BITS, int LPR>
+// SHARED: x was written earlier in this launch or by another CU's kernel and is
+// read with device-scope loads.
+template <int BITS, int LPR, bool SHARED = false>
 __device__ __forceinline__ void fm_build_act_lds(const float *x, const FmBuildSlot<BITS> &bs,
                                                  FmActLds<LPR> &L) {
+    auto ld = [](const float *p) {
+        if constexpr (SHARED)
+            return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else
+            return *p;
+    };
     constexpr int NE = 4 * LPR;
     constexpr int NIT = (LPR + 3) / 4;     // chunks per thread
     const int w = threadIdx.x & 63;
@@ -187,8 +195,8 @@ __device__ __forceinline__ void fm_build_act_lds(const float *x, const FmBuildSl
     for (int i = 0; i < NIT; i++) {
         const int ch = (threadIdx.x >> 6) + 4 * i;
         const bool on = ch < LPR;
-        xl[i] = on ? x[ch * FM_CPL + bs.lo] : 0.0f;
-        xh[i] = on ? x[ch * FM_CPL + bs.hi] : 0.0f;
+        xl[i] = on ? ld(x + ch * FM_CPL + bs.lo) : 0.0f;
+        xh[i] = on ? ld(x + ch * FM_CPL + bs.hi) : 0.0f;
     }
     uint32_t *flat = reinterpret_cast<uint32_t *>(L.a);
 #pragma unroll
