@@ -138,6 +138,7 @@ def run_decode_step(args):
         ctx.moe_decode_step_dev(0, n_layers, d_x.data_ptr(), d_idx.data_ptr() + t * isz,
                                 d_w.data_ptr() + t * isz, K, d_out.data_ptr())
 
+    _ramp_clocks(ctx, step, args.ramp_seconds)
     for t in range(args.warmup):
         step(t)
     ctx.sync()
@@ -230,8 +231,23 @@ def _finish(res, metric, workload, bytes_step, ms_per_step, args, extra_cfg=None
     return out
 
 
+def _ramp_clocks(ctx, step, seconds):
+    """Untimed: keep the GPU busy with the workload for `seconds` before the W warmup
+    steps.  The first launches after an idle period run 10-20 % slower (clock and
+    power state ramp), which a warmup counted in steps does not cover when a step
+    is ~100 us."""
+    t_end = time.perf_counter() + seconds
+    t = 0
+    while time.perf_counter() < t_end:
+        for _ in range(50):
+            step(t)
+            t += 1
+        ctx.sync()
+
+
 def _timed(ctx, step, args):
     import torch
+    _ramp_clocks(ctx, step, args.ramp_seconds)
     for t in range(args.warmup):
         step(t)
     ctx.sync()
@@ -457,11 +473,13 @@ def run_copy_probe(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="decode_step")
     ap.add_argument("--layers", type=int, default=L)
     ap.add_argument("--chunk", type=int, default=512, help="positions per chunk (prefill workload)")
+    ap.add_argument("--ramp-seconds", type=float, default=0.5,
+                    help="untimed busy period before the warmup steps (clock ramp)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()

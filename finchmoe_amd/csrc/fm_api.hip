@@ -22,9 +22,8 @@ extern "C" {
 int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs, const FmExpertGeom *g,
                             int layer0, int layer_stride, int n_layers, const float *d_x,
                             const int32_t *d_idx, const float *d_w, int K, float *d_act,
-                            float *d_expert_out, float *d_out, unsigned int *d_sync,
-                            unsigned int *epoch, unsigned int spin_limit, int flags, int n_cu,
-                            hipStream_t st, hipEvent_t *kev);
+                            float *d_expert_out, float *d_out, FmDecodeFlags *df, int flags,
+                            int n_cu, hipStream_t st, hipEvent_t *kev);
 int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
                     const float *d_x, int M, int n_cu, hipStream_t st);
 int fm_launch_dequant_affine(const void *W, const void *S, const void *B, int out_dim,
@@ -69,11 +68,11 @@ struct fm_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     hipEvent_t kev[3] = {nullptr, nullptr, nullptr};
     int ktiming = 0;   // 0 off, 1 whole operator, 2 phases as separate kernels
-    // grid barrier of the fused decode kernel: [0] arrival counter (only grows; the
-    // host tracks its value in sync_epoch), [1] error flag raised by a timed-out wait
-    unsigned int *d_sync = nullptr;
-    unsigned int sync_epoch = 0;
-    unsigned int spin_limit = 1u << 20;
+    // fused decode kernel: the word a timed-out wait raises (pinned host memory the
+    // device writes directly, so checking it after a sync costs nothing) and the
+    // dependency counters (allocated with the scratch)
+    unsigned int *h_err = nullptr, *d_err = nullptr;
+    FmDecodeFlags dflags{};
     bool split_phases = false;     // run the phases as separate kernels
     bool sync_unchecked = false;   // a fused launch has not had its error flag read yet
     double k1_ms = 0.0, k2_ms = 0.0;
@@ -171,13 +170,26 @@ int ensure_scratch(fm_ctx *c, int groups, int hidden, int inter) {
     if (c->d_act) (void)hipFree(c->d_act);
     if (c->d_eo) (void)hipFree(c->d_eo);
     if (c->d_counters) (void)hipFree(c->d_counters);
+    if (c->dflags.set[0]) (void)hipFree(c->dflags.set[0]);
     c->d_act = c->d_eo = nullptr;
     c->d_counters = nullptr;
+    c->dflags = FmDecodeFlags{};
     c->cap_groups = 0;
     HIPCHK(c, hipMalloc((void **)&c->d_act, (size_t)g * FM_MAX_K * in * sizeof(float)));
     HIPCHK(c, hipMalloc((void **)&c->d_eo, (size_t)g * FM_MAX_K * h * sizeof(float)));
     HIPCHK(c, hipMalloc((void **)&c->d_counters, (size_t)g * sizeof(unsigned int)));
     HIPCHK(c, hipMemsetAsync(c->d_counters, 0, (size_t)g * sizeof(unsigned int), c->stream));
+    {   // two sets of (pairs + groups) dependency counters, cleared once
+        const size_t cap = (size_t)g * (FM_MAX_K + 1);
+        unsigned int *p = nullptr;
+        HIPCHK(c, hipMalloc((void **)&p, 2 * cap * sizeof(unsigned int)));
+        HIPCHK(c, hipMemsetAsync(p, 0, 2 * cap * sizeof(unsigned int), c->stream));
+        c->dflags.set[0] = p;
+        c->dflags.set[1] = p + cap;
+        c->dflags.cap = (unsigned int)cap;
+        c->dflags.err = c->d_err;
+        c->dflags.spin_limit = 1u << 20;
+    }
     c->cap_groups = g;
     c->cap_hidden = h;
     c->cap_inter = in;
@@ -243,11 +255,13 @@ extern "C" int fm_ctx_create(int device, fm_ctx **out) {
             delete c;
             return FM_ERR_HIP;
         }
-    if (hipMalloc((void **)&c->d_sync, 2 * sizeof(unsigned int)) != hipSuccess ||
-        hipMemset(c->d_sync, 0, 2 * sizeof(unsigned int)) != hipSuccess) {
+    if (hipHostMalloc((void **)&c->h_err, sizeof(unsigned int), hipHostMallocMapped) !=
+            hipSuccess ||
+        hipHostGetDevicePointer((void **)&c->d_err, c->h_err, 0) != hipSuccess) {
         delete c;
         return FM_ERR_NOMEM;
     }
+    *c->h_err = 0u;
     if (const char *e = getenv("FINCH_DECODE_SPLIT")) c->split_phases = e[0] == '1';
     *out = c;
     return FM_OK;
@@ -267,7 +281,9 @@ extern "C" int fm_ctx_destroy(fm_ctx *c) {
             (void)hipFree(t.S);
             (void)hipFree(t.B);
         }
-    void *ptrs[] = {c->d_layer_ptrs, c->d_gg_ptrs, c->d_act, c->d_eo, c->d_counters, c->d_sync,
+    if (c->h_err) (void)hipHostFree(c->h_err);
+    void *ptrs[] = {c->d_layer_ptrs, c->d_gg_ptrs, c->d_act, c->d_eo, c->d_counters,
+                    c->dflags.set[0],
                     c->d_stage, c->d_ws};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
@@ -279,15 +295,14 @@ extern "C" int fm_ctx_destroy(fm_ctx *c) {
     return FM_OK;
 }
 
-// After the stream has drained: did a fused decode launch give up on its grid barrier?
+// After the stream has drained: did a fused decode launch give up on a wait?
 static int check_grid_error(fm_ctx *c) {
     if (!c->sync_unchecked) return FM_OK;
     c->sync_unchecked = false;
-    unsigned int flag = 0;
-    HIPCHK(c, hipMemcpy(&flag, c->d_sync + 1, sizeof flag, hipMemcpyDeviceToHost));
-    if (!flag) return FM_OK;
-    HIPCHK(c, hipMemset(c->d_sync + 1, 0, sizeof flag));
-    return fail(c, FM_ERR_HIP, "decode kernel: grid barrier timed out, results are invalid");
+    volatile unsigned int *flag = c->h_err;
+    if (!*flag) return FM_OK;
+    *flag = 0u;
+    return fail(c, FM_ERR_HIP, "decode kernel: a wait on another workgroup timed out, results are invalid");
 }
 
 extern "C" int fm_sync(fm_ctx *c) {
@@ -461,8 +476,8 @@ extern "C" int fm_moe_decode_step_dev(fm_ctx *c, int layer0, int n_layers, const
     const bool split = c->split_phases || c->ktiming == 2;
     rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer0, 1, n_layers, d_x, d_idx, d_w,
                                  K, c->d_act, d_expert_out ? d_expert_out : c->d_eo, d_out,
-                                 split ? nullptr : c->d_sync, &c->sync_epoch, c->spin_limit,
-                                 flags, c->n_cu, c->stream, c->ktiming ? c->kev : nullptr);
+                                 split ? nullptr : &c->dflags, flags, c->n_cu, c->stream,
+                                 c->ktiming ? c->kev : nullptr);
     if (rc) return fail(c, rc, "decode launch failed: %s", hipGetErrorString(hipGetLastError()));
     if (!split) c->sync_unchecked = true;
     if (c->ktiming) return ktiming_collect(c);
@@ -557,9 +572,8 @@ extern "C" int fm_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, const 
     rc = ensure_scratch(c, M, c->geom.hidden, c->geom.inter);
     if (rc) return rc;
     rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer, 0, M, d_X, d_idx, d_w, K,
-                                 c->d_act, c->d_eo, d_out, c->split_phases ? nullptr : c->d_sync,
-                                 &c->sync_epoch, c->spin_limit, flags, c->n_cu, c->stream,
-                                 nullptr);
+                                 c->d_act, c->d_eo, d_out, c->split_phases ? nullptr : &c->dflags,
+                                 flags, c->n_cu, c->stream, nullptr);
     if (rc) return fail(c, rc, "prefill launch failed: %s", hipGetErrorString(hipGetLastError()));
     if (!c->split_phases) c->sync_unchecked = true;
     return FM_OK;

@@ -18,6 +18,19 @@ struct FmExpertGeom {
     uint64_t expert_size;
 };
 
+// Host-side state of the dependency counters of the fused decode kernel: two
+// sets of `cap` counters that alternate between launches (a launch counts in
+// set[parity] and clears the used[parity ^ 1] entries the launch before it left
+// in the other set), and the device word a timed-out wait raises.
+struct FmDecodeFlags {
+    unsigned int *set[2];
+    unsigned int used[2];
+    unsigned int cap;
+    int parity;
+    unsigned int *err;
+    unsigned int spin_limit;
+};
+
 // Geometry of the GGUF slabs of one layer (finchmoe/infer.m:1017-1022).
 struct FmGgufGeom {
     int hidden, inter, n_experts;

@@ -345,13 +345,14 @@ __device__ __forceinline__ uint32_t fm_dma_read(uint32_t slot, uint32_t woff, ui
 // activation image, then (gate/up only) the layer's blob table and valid mask.
 extern __shared__ __attribute__((aligned(16))) uint8_t fm_dyn_lds[];
 
-template <int BITS, int LPR_UP>
-constexpr size_t fm_stream_lds_bytes() {
-    return FmDma<BITS>::WG_BYTES + sizeof(FmActLds<LPR_UP>) + FM_MAX_K * sizeof(void *) + 16;
-}
-
-struct FmNoSync {
-    __device__ __forceinline__ void operator()() const {}
+// Dependencies of a phase on other workgroups (used by the fused kernel; the
+// separate kernels have none):
+//   wait_in(s)            before segment s's input vector is read
+//   publish(s, first, n)  by wave 0, once units [first, first+n) of segment s are
+//                         complete and their stores have completed
+struct FmNoDeps {
+    __device__ __forceinline__ void wait_in(int) const {}
+    __device__ __forceinline__ void publish(int, uint32_t, uint32_t) const {}
 };
 
 // Units of a segment are handed out one at a time from a counter in LDS: the
@@ -378,302 +379,383 @@ __device__ __forceinline__ uint32_t fm_claim_unit(unsigned int *next, int lane) 
 __device__ __forceinline__ void fm_slot_tag(uint32_t slot_tag_addr, uint32_t tag) {
     asm volatile("ds_write_b32 %0, %1" ::"v"(slot_tag_addr), "v"(tag) : "memory");
 }
+__device__ __forceinline__ uint32_t fm_slot_peek(uint32_t slot_tag_addr) {
+    uint32_t tag;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&v"(tag)
+                 : "v"(slot_tag_addr)
+                 : "memory");
+    return __builtin_amdgcn_readfirstlane(tag);
+}
 
-// gate + up + SwiGLU over this workgroup's share of the n_pairs * inter/RPS units.
-// An invalid expert index streams expert 0 and contributes zero.  `before_build`
-// runs once, after the first segment's loads are in flight and before the first
-// read of a.x.
-template <int BITS, int LPR, bool FP16, class Sync>
-__device__ __forceinline__ void fm_gate_up_phase(const DecodeArgs &a, int n_pairs,
-                                                 unsigned int *next_unit, Sync before_build) {
+// What the loaders need to know about a segment (a layer's K experts for gate/up,
+// one pair for down) plus the segment's unit counter.  Three of them, used round
+// robin: while segment s is multiplied the loaders read those of s and s+1, and
+// the one of s+1 is written while slower waves may still be loading s-1.
+struct FmSegTable {
+    const uint8_t *blob[FM_MAX_K];
+    uint32_t valid;          // bit k: slot k has a valid expert index
+    uint32_t next_unit;
+    uint32_t pad[2];
+};
+
+template <int BITS, int LPR>
+constexpr size_t fm_phase_lds_bytes() {
+    return FmDma<BITS>::WG_BYTES + 2 * sizeof(FmActLds<LPR>) + 3 * sizeof(FmSegTable);
+}
+
+// One phase of the operator over this workgroup's share [U*g/G, U*(g+1)/G) of
+// the phase's units:
+//   GU = true : gate + up + SwiGLU.  unit = RPS rows of gate and of up (two
+//               slices), segment = layer, input a.x, output a.act
+//   GU = false: down projection.  unit = RPS rows (one slice), segment = pair,
+//               input a.act, output a.expert_out
+// An invalid expert index streams expert 0 and contributes zero.
+//
+// The share is one continuous stream.  Per segment only the activation image
+// changes, and everything a change needs is fetched a segment ahead (the next
+// segment's activations into registers, its expert indices two segments ahead),
+// while the loaders run on into the next segment's units as soon as the current
+// one is handed out — a slice's tag says which segment it belongs to, and a
+// wave that meets a slice of the next segment waits for the workgroup to switch
+// image.
+template <int BITS, int LPR, bool FP16, bool GU, class Deps>
+__device__ __forceinline__ void fm_stream_phase(const DecodeArgs &a, int n_pairs,
+                                                const Deps &deps) {
     using D = FmDma<BITS>;
     constexpr int RPS = FM_WAVE / LPR, RING = D::RING;
-    FmActLds<LPR> &lds = *reinterpret_cast<FmActLds<LPR> *>(fm_dyn_lds + D::WG_BYTES);
-    const uint8_t **lds_blob =
-        reinterpret_cast<const uint8_t **>(fm_dyn_lds + D::WG_BYTES + sizeof(FmActLds<LPR>));
-    uint32_t *lds_valid = reinterpret_cast<uint32_t *>(lds_blob + FM_MAX_K);
+    FmActLds<LPR> *img = reinterpret_cast<FmActLds<LPR> *>(fm_dyn_lds + D::WG_BYTES);
+    FmSegTable *tab =
+        reinterpret_cast<FmSegTable *>(fm_dyn_lds + D::WG_BYTES + 2 * sizeof(FmActLds<LPR>));
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t ring0 =
         (uint32_t)(uintptr_t)(fm_lptr)fm_dyn_lds + (uint32_t)wave * (RING * D::BYTES);
-    const int upp = a.g.inter / RPS;        // units per pair
-    const long upl = (long)upp * a.K;       // units per layer
+    const int in_dim = GU ? a.g.hidden : a.g.inter, out_dim = GU ? a.g.inter : a.g.hidden;
+    const uint32_t upp = (uint32_t)(out_dim / RPS);               // units per pair
+    const long segu = GU ? (long)upp * a.K : (long)upp;           // units per segment
+    const int NK = GU ? a.K : 1;                                  // experts per segment
     const long total = (long)n_pairs * upp;
     const long wg0 = total * blockIdx.x / gridDim.x, wg1 = total * (blockIdx.x + 1) / gridDim.x;
-    const int row_bytes = a.g.hidden * BITS / 8, sb_row_bytes = (a.g.hidden / 64) * 2;
+    if (wg0 >= wg1) return;
+    const int s_begin = (int)(wg0 / segu), s_end = (int)((wg1 - 1) / segu) + 1;
+    const int row_bytes = in_dim * BITS / 8, sb_row_bytes = (in_dim / 64) * 2;
     uint32_t woff, soff;
     int ris, ch;
     fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff, soff, ris, ch);
     const uint32_t wstep = (uint32_t)(RPS * row_bytes), sstep = (uint32_t)(RPS * sb_row_bytes);
     // region offsets as scalars (selected per half step with a scalar select)
-    const auto gw = a.g.gate_w, gs = a.g.gate_s, gb = a.g.gate_b;
-    const auto uw = a.g.up_w, us = a.g.up_s, ub = a.g.up_b;
+    const uint32_t w0 = GU ? a.g.gate_w : a.g.down_w, s0 = GU ? a.g.gate_s : a.g.down_s,
+                   b0 = GU ? a.g.gate_b : a.g.down_b;
+    const uint32_t w1 = a.g.up_w, s1 = a.g.up_s, b1 = a.g.up_b;
     FmBuildSlot<BITS> bslot;
     bslot.init();
-    bool first = true;
 
-    for (long seg0 = wg0; seg0 < wg1;) {
-        const int l = (int)(seg0 / upl);
-        long seg1 = (long)(l + 1) * upl;
-        if (seg1 > wg1) seg1 = wg1;
-        const uint32_t seg_n = (uint32_t)(seg1 - seg0);
-        const uint32_t u_first = (uint32_t)(seg0 - (long)l * upl);   // first unit, in the layer
-        __syncthreads();                          // previous segment's readers are done
-        if (threadIdx.x < 64) {
-            bool ok = false;
-            if (lane < a.K) {
-                const int e = a.idx[l * a.K + lane];
-                ok = (unsigned)e < (unsigned)a.g.n_experts;
-                lds_blob[lane] = a.layer_ptrs[a.layer0 + l * a.layer_stride] +
-                                 (size_t)(ok ? e : 0) * a.g.expert_size;
-            }
+    // this workgroup's part of segment s: first unit (inside the segment) and count
+    auto seg_part = [&](int s, uint32_t &first, uint32_t &n) {
+        const long lo = (long)s * segu > wg0 ? (long)s * segu : wg0;
+        const long hi = (long)(s + 1) * segu < wg1 ? (long)(s + 1) * segu : wg1;
+        first = (uint32_t)(lo - (long)s * segu);
+        n = (uint32_t)(hi - lo);
+    };
+    // expert index and layer blob of this lane's slot of segment s (wave 0, lanes < NK)
+    struct Raw {
+        int e;
+        const uint8_t *layer;
+    };
+    auto load_raw = [&](int s) {
+        Raw r{0, nullptr};
+        if (wave == 0 && lane < NK) {
+            const int l = GU ? s : s / a.K;
+            r.e = a.idx[GU ? s * a.K + lane : s];
+            r.layer = a.layer_ptrs[a.layer0 + l * a.layer_stride];
+        }
+        return r;
+    };
+    auto write_table = [&](int s, const Raw &r) {
+        if (wave == 0) {
+            FmSegTable &t = tab[s % 3];
+            const bool ok = lane < NK && (unsigned)r.e < (unsigned)a.g.n_experts;
+            if (lane < NK) t.blob[lane] = r.layer + (size_t)(ok ? r.e : 0) * a.g.expert_size;
             const uint64_t m = __ballot(ok);
             if (lane == 0) {
-                lds_valid[0] = (uint32_t)m;
-                *next_unit = 0u;
+                t.valid = (uint32_t)m;
+                t.next_unit = 0u;
             }
         }
-        __syncthreads();
-        const uint32_t valid = __builtin_amdgcn_readfirstlane(lds_valid[0]);
-        // loader: the next half step (gate rows, then up rows of the same unit)
-        int hn = 0;
-        uint32_t tag_n = 0, rsn = 0, issued = 0, consumed = 0;
-        const uint8_t *blob_n = nullptr;
-        bool drain = false;
-        auto issue = [&](int slot_idx) {
-            if (drain) return;
-            if (hn == 0) {
-                const uint32_t ul = fm_claim_unit(next_unit, lane);
-                if (ul >= seg_n) {
-                    drain = true;
-                    return;
+    };
+    auto in_vec = [&](int s) {
+        return GU ? a.x + (size_t)s * a.g.hidden : a.act + (size_t)s * a.g.inter;
+    };
+
+    // ---- loader: the next slice (gate rows, then up rows of the same unit)
+    int ls = s_begin, cs = s_begin;     // segment of the loader / of the multiply
+    uint32_t l_first, l_n;
+    seg_part(ls, l_first, l_n);
+    int hn = 0, wpos = 0;
+    uint32_t tag_n = 0, rsn = 0, issued = 0, consumed = 0;
+    const uint8_t *blob_n = nullptr;
+    bool dry = false;                   // nothing more to hand out for now
+    auto issue = [&]() {
+        if (dry) return;
+        if (!GU || hn == 0) {
+            uint32_t ul;
+            for (;;) {
+                ul = fm_claim_unit(&tab[ls % 3].next_unit, lane);
+                if (ul < l_n) break;
+                if (ls + 1 < s_end && ls == cs) {       // run on into the next segment
+                    ls++;
+                    seg_part(ls, l_first, l_n);
+                    continue;
                 }
-                const uint32_t uq = u_first + ul;            // unit inside the layer
-                const uint32_t pn = uq / (uint32_t)upp;
-                rsn = uq - pn * (uint32_t)upp;
-                tag_n = (pn << 28) | ul;
-                blob_n = fm_uniform(lds_blob[pn]);
+                dry = true;
+                return;
             }
-            const uint32_t slot = ring0 + (uint32_t)slot_idx * D::BYTES;
-            fm_slot_tag(slot + D::TAG, tag_n);
-            const uint8_t *b = blob_n + (size_t)rsn * wstep;
-            const uint8_t *sb = blob_n + (size_t)rsn * sstep;
-            fm_dma_issue<BITS>(slot, b + (hn ? uw : gw), sb + (hn ? us : gs),
-                               sb + (hn ? ub : gb), lane);
-            hn ^= 1;
-            issued++;
-        };
-#pragma unroll
-        for (int k = 0; k < RING; k++) issue(k);
-        if (first) {
-            before_build();
-            first = false;
+            const uint32_t uq = l_first + ul;                     // unit inside the segment
+            const uint32_t pn = GU ? uq / upp : 0u;
+            rsn = uq - pn * upp;
+            tag_n = ((uint32_t)(ls & 1) << 31) | (pn << 28) | ul;
+            blob_n = fm_uniform(tab[ls % 3].blob[pn]);
         }
-        if (threadIdx.x < 256)
-            fm_build_act_lds<BITS, LPR, false>(a.x + (size_t)l * a.g.hidden, bslot, lds);
+        const uint32_t slot = ring0 + (uint32_t)wpos * D::BYTES;
+        fm_slot_tag(slot + D::TAG, tag_n);
+        const uint8_t *b = blob_n + (size_t)rsn * wstep;
+        const uint8_t *sb = blob_n + (size_t)rsn * sstep;
+        const bool second = GU && hn;
+        fm_dma_issue<BITS>(slot, b + (second ? w1 : w0), sb + (second ? s1 : s0),
+                           sb + (second ? b1 : b0), lane);
+        if (GU) hn ^= 1;
+        wpos = wpos + 1 == RING ? 0 : wpos + 1;
+        issued++;
+    };
+
+    // ---- start: tables of the first two segments, first loads, first input vector
+    FmActX<LPR> xr;
+    if (GU && threadIdx.x < 256) fm_act_load<BITS, LPR, false>(in_vec(s_begin), bslot, xr);
+    __syncthreads();                              // the previous phase is done with this LDS
+    {
+        const Raw r0 = load_raw(s_begin);
+        const Raw r1 = load_raw(s_begin + 1 < s_end ? s_begin + 1 : s_begin);
+        write_table(s_begin, r0);
+        if (s_begin + 1 < s_end) write_table(s_begin + 1, r1);
+    }
+    Raw raw_next = load_raw(s_begin + 2 < s_end ? s_begin + 2 : s_begin);   // for segment cs + 2
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < RING; k++) issue();
+    if (!GU && threadIdx.x < 256) {
+        deps.wait_in(s_begin);
+        fm_act_load<BITS, LPR, true>(in_vec(s_begin), bslot, xr);
+    }
+
+    int c = 0;
+    for (; cs < s_end; cs++) {
+        // ---- switch to the image of segment cs
+        if (threadIdx.x < 256) fm_act_build<BITS, LPR>(xr, bslot, img[cs & 1]);
+        const bool new_table = cs > s_begin && cs + 1 < s_end;
+        // every loader has left segment cs-2: its table becomes that of cs+1
+        if (new_table) write_table(cs + 1, raw_next);
         __syncthreads();
+        if (cs > s_begin && wave == 0) {          // every wave is done with segment cs-1
+            uint32_t pf, pn_;
+            seg_part(cs - 1, pf, pn_);
+            deps.publish(cs - 1, pf, pn_);
+        }
         FmActRegs ar;
-        fm_read_act_lds<LPR>(lds, lane, ar);
-        int c = 0;
-        uint32_t tag = 0;
-        auto half = [&]() {
+        fm_read_act_lds<LPR>(img[cs & 1], lane, ar);
+        const uint32_t valid = __builtin_amdgcn_readfirstlane(tab[cs % 3].valid);
+        uint32_t c_first, c_n;
+        seg_part(cs, c_first, c_n);
+        const size_t out0 = (size_t)((long)cs * segu + c_first) * RPS + ris;
+        float *out_vec = GU ? a.act : a.expert_out;
+        // fetched now, used at the next switch
+        if (cs + 1 < s_end && threadIdx.x < 256) {
+            deps.wait_in(cs + 1);
+            fm_act_load<BITS, LPR, !GU>(in_vec(cs + 1), bslot, xr);
+        }
+        if (new_table) raw_next = load_raw(cs + 2 < s_end ? cs + 2 : cs);
+        dry = false;
+        while (issued - consumed < (uint32_t)RING && !dry) issue();
+
+        // ---- multiply the slices of this segment
+        auto take = [&]() {
             FmRowSlice<BITS> t;
-            fm_dma_wait<D::LOADS *(RING - 1)>(drain);
-            tag = fm_dma_read<BITS>(ring0 + (uint32_t)c * D::BYTES, woff, soff, t);
+            if (issued - consumed == (uint32_t)RING) fm_dma_wait<D::LOADS *(RING - 1)>(false);
+            else fm_dma_wait<0>(true);
+            fm_dma_read<BITS>(ring0 + (uint32_t)c * D::BYTES, woff, soff, t);
             consumed++;
-            issue(c);
             c = c + 1 == RING ? 0 : c + 1;
+            issue();
             return fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(t, ar));
         };
         while (consumed < issued) {
-            const float gv = half();
-            const float uv = half();
-            const uint32_t pc = tag >> 28, ul = tag & 0x0FFFFFFFu;
-            const float v = ((valid >> pc) & 1u) ? fm_silu_mul(gv, uv) : 0.0f;
-            // unit (pair, row step): act is [pair][inter], rows are contiguous
-            if (ch == 0) fm_st_shared(a.act + (size_t)(seg0 + ul) * RPS + ris, v);
-        }
-        seg0 = seg1;
-    }
-    if (first) before_build();
-}
-
-// down projection -> per-expert output vectors over this workgroup's share of
-// the n_pairs * hidden/RPS units.  `before_build` as above (first read of a.act).
-template <int BITS, int LPR, bool FP16, class Sync>
-__device__ __forceinline__ void fm_down_phase(const DecodeArgs &a, int n_pairs,
-                                              unsigned int *next_unit, Sync before_build) {
-    using D = FmDma<BITS>;
-    constexpr int RPS = FM_WAVE / LPR, RING = D::RING;
-    FmActLds<LPR> &lds = *reinterpret_cast<FmActLds<LPR> *>(fm_dyn_lds + D::WG_BYTES);
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t ring0 =
-        (uint32_t)(uintptr_t)(fm_lptr)fm_dyn_lds + (uint32_t)wave * (RING * D::BYTES);
-    const int upp = a.g.hidden / RPS;
-    const long total = (long)n_pairs * upp;
-    const long wg0 = total * blockIdx.x / gridDim.x, wg1 = total * (blockIdx.x + 1) / gridDim.x;
-    const int row_bytes = a.g.inter * BITS / 8, sb_row_bytes = (a.g.inter / 64) * 2;
-    uint32_t woff, soff;
-    int ris, ch;
-    fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff, soff, ris, ch);
-    const uint32_t wstep = (uint32_t)(RPS * row_bytes), sstep = (uint32_t)(RPS * sb_row_bytes);
-    FmBuildSlot<BITS> bslot;
-    bslot.init();
-    bool first = true;
-
-    for (long seg0 = wg0; seg0 < wg1;) {
-        const int p = (int)(seg0 / upp);
-        long seg1 = (long)(p + 1) * upp;
-        if (seg1 > wg1) seg1 = wg1;
-        const uint32_t seg_n = (uint32_t)(seg1 - seg0);
-        const uint32_t rs_first = (uint32_t)(seg0 - (long)p * upp);
-        const uint8_t *blob = fm_pair_blob(a, p);
-        uint32_t issued = 0, consumed = 0;
-        bool drain = false;
-        auto issue = [&](int slot_idx) {
-            if (drain) return;
-            const uint32_t ul = fm_claim_unit(next_unit, lane);
-            if (ul >= seg_n) {
-                drain = true;
-                return;
+            const uint32_t tag = fm_slot_peek(ring0 + (uint32_t)c * D::BYTES + D::TAG);
+            if ((tag >> 31) != (uint32_t)(cs & 1)) break;         // belongs to the next segment
+            const uint32_t pc = (tag >> 28) & 7u, ul = tag & 0x0FFFFFFFu;
+            float v;
+            if constexpr (GU) {
+                const float gv = take();
+                const float uv = take();
+                v = fm_silu_mul(gv, uv);
+            } else {
+                v = take();
             }
-            const uint32_t slot = ring0 + (uint32_t)slot_idx * D::BYTES;
-            fm_slot_tag(slot + D::TAG, ul);
-            const uint8_t *b = blob + (size_t)(rs_first + ul) * wstep;
-            const uint8_t *sb = blob + (size_t)(rs_first + ul) * sstep;
-            fm_dma_issue<BITS>(slot, b + a.g.down_w, sb + a.g.down_s, sb + a.g.down_b, lane);
-            issued++;
-        };
-        __syncthreads();                          // previous segment's readers are done
-        if (threadIdx.x == 0) *next_unit = 0u;
-        __syncthreads();
-        if (blob) {
-#pragma unroll
-            for (int k = 0; k < RING; k++) issue(k);
+            if (!((valid >> pc) & 1u)) v = 0.0f;
+            // unit (pair, row step): the output is [pair][rows], rows are contiguous
+            if (ch == 0) fm_st_shared(out_vec + out0 + (size_t)ul * RPS, v);
         }
-        if (first) {
-            before_build();
-            first = false;
-        }
-        if (blob) {
-            if (threadIdx.x < 256)
-                fm_build_act_lds<BITS, LPR, true>(a.act + (size_t)p * a.g.inter, bslot, lds);
-            __syncthreads();
-            FmActRegs ar;
-            fm_read_act_lds<LPR>(lds, lane, ar);
-            int c = 0;
-            while (consumed < issued) {
-                FmRowSlice<BITS> t;
-                fm_dma_wait<D::LOADS *(RING - 1)>(drain);
-                const uint32_t ul = fm_dma_read<BITS>(ring0 + (uint32_t)c * D::BYTES, woff, soff, t);
-                consumed++;
-                issue(c);
-                c = c + 1 == RING ? 0 : c + 1;
-                const float v = fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(t, ar));
-                if (ch == 0) fm_st_shared(a.expert_out + (size_t)(seg0 + ul) * RPS + ris, v);
-            }
-        } else {
-            for (long u = seg0 + (threadIdx.x >> 6); u < seg1; u += FM_NW)
-                if (ch == 0) fm_st_shared(a.expert_out + (size_t)u * RPS + ris, 0.0f);
-        }
-        seg0 = seg1;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's stores have completed
     }
-    if (first) before_build();
+    __syncthreads();
+    if (wave == 0) {
+        uint32_t pf, pn_;
+        seg_part(s_end - 1, pf, pn_);
+        deps.publish(s_end - 1, pf, pn_);
+    }
 }
 
 template <int BITS, int LPR, bool FP16>
 __global__ __launch_bounds__(FM_NW * 64) void fm_gate_up_swiglu_lds(DecodeArgs a, int n_pairs) {
-    __shared__ unsigned int next_unit;
-    fm_gate_up_phase<BITS, LPR, FP16>(a, n_pairs, &next_unit, FmNoSync());
+    fm_stream_phase<BITS, LPR, FP16, true>(a, n_pairs, FmNoDeps());
 }
 
 template <int BITS, int LPR, bool FP16>
 __global__ __launch_bounds__(FM_NW * 64) void fm_down_lds(DecodeArgs a, int n_pairs) {
-    __shared__ unsigned int next_unit;
-    fm_down_phase<BITS, LPR, FP16>(a, n_pairs, &next_unit, FmNoSync());
+    fm_stream_phase<BITS, LPR, FP16, false>(a, n_pairs, FmNoDeps());
 }
 
 // ======================================================================
 // One launch for the whole operator: gate/up, down and combine as three phases
-// of one persistent grid, separated by grid-wide barriers.
+// of one persistent grid.
 //
-// What the barrier buys: a phase's weights do not depend on the previous
-// phase, so every wave issues the first RING slices of its next share before
-// it waits — the memory pipeline stays full across the phase change, where
-// separate kernels drain it, relaunch and refill it.
+// A phase's weights do not depend on the previous phase, so every wave issues
+// the first slices of its next share before it looks at its input: the memory
+// pipeline stays full across the phase change, where separate kernels drain
+// it, relaunch and refill it.
 //
-// The barrier is an arrival counter in device memory that only ever grows: the
-// host hands each launch the value the counter had before it (`base`) and adds
-// two arrivals per workgroup afterwards, so nothing is reset between launches.
-// What crosses the barrier (act, expert_out) is stored and loaded at device
-// scope (fm_st_shared / fm_ld_shared), so a workgroup arrives once its waves'
-// stores have completed and no cache is written back or invalidated — device-
-// scope fences cost more here than the barrier saves.  Every workgroup of the grid must be resident at once — the
-// launcher sizes the grid from the occupancy query — and the wait is bounded:
-// past `spin_limit` polls a workgroup raises `*err` and goes on (results are
-// then wrong, the host reports the error, and the counter stays consistent
-// because every workgroup still arrives exactly twice).
+// Dependencies are per vector, not grid-wide: a counter per pair says how many
+// units of its activation vector exist, a counter per group how many units of
+// its K expert outputs.  Both phases split their units over the workgroups in
+// proportion, so a workgroup's down share needs activations that it or its
+// neighbours produced a moment ago, and nobody waits for the slowest workgroup
+// of the grid.  Producers add to a counter after their stores have completed;
+// the vectors themselves are stored and loaded at device scope (fm_st_shared /
+// fm_ld_shared), so no cache is written back or invalidated.
+//
+// Two sets of counters alternate between launches: a launch uses one and
+// clears the part of the other that the launch before it used, so nothing has
+// to be reset in between and a failed launch leaves no state behind.  Every
+// workgroup must be resident at once (the launcher sizes the grid from the
+// occupancy query), a workgroup finishes a phase before it starts the next, and
+// every wait is bounded: past `spin_limit` polls the thread raises `*err` and
+// goes on (the results are then wrong and the host reports the error).
 // ======================================================================
-struct FmGridSync {
-    unsigned int *counter;
-    unsigned int *err;
-    unsigned int base;
+struct FmFlags {
+    unsigned int *cur;        // [n_pairs] activation units, then [n_groups] expert-output units
+    unsigned int *other;      // the set of the previous and of the next launch
+    unsigned int clear_n;     // entries of `other` to clear
+    unsigned int *err;        // host memory
     unsigned int spin_limit;
 };
 
-__device__ __forceinline__ void fm_grid_arrive(const FmGridSync &s) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's stores have completed
-    __syncthreads();
-    if (threadIdx.x == 0)
-        __hip_atomic_fetch_add(s.counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ void fm_flag_wait(const FmFlags &f, const unsigned int *flag,
+                                             unsigned int target) {
+    unsigned int polls = 0;
+    while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+        if (++polls > f.spin_limit) {
+            __hip_atomic_store(f.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(8);
+    }
 }
 
-__device__ __forceinline__ void fm_grid_wait(const FmGridSync &s, unsigned int target) {
-    if (threadIdx.x == 0) {
-        unsigned int polls = 0;
-        while ((int)(__hip_atomic_load(s.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) -
-                     target) < 0) {
-            if (++polls > s.spin_limit) {
-                __hip_atomic_store(s.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                break;
-            }
-            __builtin_amdgcn_s_sleep(8);
+// gate/up: publishes per pair how many of its units this workgroup finished
+struct FmGateUpDeps {
+    const FmFlags &f;
+    int K;
+    uint32_t upp;
+    __device__ __forceinline__ void wait_in(int) const {}
+    __device__ __forceinline__ void publish(int s, uint32_t first, uint32_t n) const {
+        const int k = threadIdx.x & 63;
+        if (k < K) {
+            const uint32_t lo = max(first, (uint32_t)k * upp), hi = min(first + n, (uint32_t)(k + 1) * upp);
+            if (hi > lo)
+                __hip_atomic_fetch_add(f.cur + (size_t)s * K + k, hi - lo, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
         }
     }
-    __syncthreads();
-}
+};
+
+// down: waits for a pair's activation vector, publishes per group
+struct FmDownDeps {
+    const FmFlags &f;
+    int K, n_pairs;
+    uint32_t upp_up;          // units of a complete activation vector
+    __device__ __forceinline__ void wait_in(int p) const { fm_flag_wait(f, f.cur + p, upp_up); }
+    __device__ __forceinline__ void publish(int p, uint32_t, uint32_t n) const {
+        if ((threadIdx.x & 63) == 0)
+            __hip_atomic_fetch_add(f.cur + n_pairs + p / K, n, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+    }
+};
 
 template <int BITS, int LPR_UP, bool FP16>
 __global__ __launch_bounds__(FM_NW * 64)
-void fm_moe_fused(DecodeArgs a, int n_pairs, FmGridSync sy) {
+void fm_moe_fused(DecodeArgs a, int n_pairs, FmFlags f) {
     constexpr int LPR_DOWN = LPR_UP / 4;
     __shared__ float red[FM_NW];
-    __shared__ unsigned int next_unit;
-    const unsigned int G = gridDim.x;
-    fm_gate_up_phase<BITS, LPR_UP, FP16>(a, n_pairs, &next_unit, FmNoSync());
-    fm_grid_arrive(sy);
-    fm_down_phase<BITS, LPR_DOWN, FP16>(a, n_pairs, &next_unit,
-                                        [&]() { fm_grid_wait(sy, sy.base + G); });
-    fm_grid_arrive(sy);
-    fm_grid_wait(sy, sy.base + 2 * G);
-    const int n_groups = n_pairs / a.K, H = a.g.hidden;
+    const int G = gridDim.x, n_groups = n_pairs / a.K, H = a.g.hidden;
+    for (unsigned int i = blockIdx.x * blockDim.x + threadIdx.x; i < f.clear_n;
+         i += G * blockDim.x)
+        f.other[i] = 0u;
+    const uint32_t upp_up = (uint32_t)(a.g.inter / (FM_WAVE / LPR_UP));
+    const uint32_t upp_down = (uint32_t)(H / (FM_WAVE / LPR_DOWN));
+    fm_stream_phase<BITS, LPR_UP, FP16, true>(a, n_pairs, FmGateUpDeps{f, a.K, upp_up});
+    fm_stream_phase<BITS, LPR_DOWN, FP16, false>(a, n_pairs,
+                                                 FmDownDeps{f, a.K, n_pairs, upp_up});
+    // combine: a group's K expert outputs are complete at K * upp_down units
+    const unsigned int full = (unsigned int)a.K * upp_down;
     if (a.flags & FM_GUARD) {
-        for (int l = blockIdx.x; l < n_groups; l += G) fm_combine_rows<true>(a, l, 0, H, red);
+        for (int l = blockIdx.x; l < n_groups; l += G) {
+            fm_flag_wait(f, f.cur + n_pairs + l, full);
+            fm_combine_rows<true>(a, l, 0, H, red);
+        }
     } else {
-        const int cols = FM_NW * 64, per = (H + cols - 1) / cols;
-        for (int it = blockIdx.x; it < n_groups * per; it += G) {
+        // column blocks of a group go to neighbouring workgroups, groups in the
+        // order in which the down phase finishes them
+        const int cols = FM_NW * 64, per = (H + cols - 1) / cols, items = n_groups * per;
+        for (int it = (int)((long)blockIdx.x * items / G); it < (int)((long)(blockIdx.x + 1) * items / G); it++) {
             const int l = it / per, j0 = (it - l * per) * cols;
+            fm_flag_wait(f, f.cur + n_pairs + l, full);
             fm_combine_rows<false>(a, l, j0, min(H, j0 + cols), red);
         }
     }
 }
 
-// Raise a kernel's dynamic LDS limit (the default stops at 64 KB).  Called on
-// every launch: the attribute belongs to the current device's copy of the kernel.
-bool fm_dyn_lds_ok(const void *fn, size_t bytes) {
-    return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) ==
-           hipSuccess;
+// Raise a kernel's dynamic LDS limit (the default stops at 64 KB).  The
+// attribute belongs to a device's copy of the kernel: done once per kernel and
+// device (these runtime calls cost more host time than a launch).
+constexpr int FM_MAX_DEVICES = 64;
+struct FmKernelSetup {
+    bool lds_set[FM_MAX_DEVICES] = {};
+    int per_cu[FM_MAX_DEVICES] = {};   // resident workgroups per CU, 0 = not asked yet
+};
+
+int fm_current_device() {
+    int d = 0;
+    (void)hipGetDevice(&d);
+    return d >= 0 && d < FM_MAX_DEVICES ? d : -1;
+}
+
+bool fm_dyn_lds_ok(FmKernelSetup &ks, const void *fn, size_t bytes) {
+    const int d = fm_current_device();
+    if (d >= 0 && ks.lds_set[d]) return true;
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) !=
+        hipSuccess)
+        return false;
+    if (d >= 0) ks.lds_set[d] = true;
+    return true;
 }
 
 // workgroups of a streaming launch: one per CU (LDS budget), fewer when there
@@ -689,16 +771,21 @@ dim3 fm_stream_grid(long units, int n_cu, int per_wave) {
 // One fused launch.  Returns FM_ERR_UNSUPPORTED when the grid cannot be made
 // fully resident (the caller then uses separate kernels).
 template <int BITS, int LPR_UP, bool FP16>
-int launch_fused(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st, FmGridSync sy,
-                 unsigned int *epoch) {
+int launch_fused(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st, const FmFlags &f) {
     auto kfn = fm_moe_fused<BITS, LPR_UP, FP16>;
-    const size_t sh = fm_stream_lds_bytes<BITS, LPR_UP>();
-    if (!fm_dyn_lds_ok((const void *)kfn, sh)) return FM_ERR_HIP;
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kfn, FM_NW * 64, sh) !=
-            hipSuccess ||
-        per_cu < 1)
-        return FM_ERR_UNSUPPORTED;
+    const size_t sh = fm_phase_lds_bytes<BITS, LPR_UP>();
+    static FmKernelSetup ks;
+    if (!fm_dyn_lds_ok(ks, (const void *)kfn, sh)) return FM_ERR_HIP;
+    const int dev = fm_current_device();
+    int per_cu = dev >= 0 ? ks.per_cu[dev] : 0;
+    if (per_cu == 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kfn, FM_NW * 64, sh) !=
+            hipSuccess)
+            per_cu = 0;
+        if (per_cu < 1) per_cu = -1;
+        if (dev >= 0) ks.per_cu[dev] = per_cu;
+    }
+    if (per_cu < 1) return FM_ERR_UNSUPPORTED;   // the grid could not be resident at once
     per_cu = 1;
     const long up_units = (long)n_pairs * (a.g.inter / (FM_WAVE / LPR_UP));
     const long down_units = (long)n_pairs * (a.g.hidden / (FM_WAVE / (LPR_UP / 4)));
@@ -706,28 +793,27 @@ int launch_fused(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st, FmG
     const long small = up_units < down_units ? up_units : down_units;
     if (small < FM_NW * wgs) wgs = (small + FM_NW - 1) / FM_NW;
     if (wgs < 1) wgs = 1;
-    sy.base = *epoch;
-    *epoch += 2u * (unsigned)wgs;
-    hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(FM_NW * 64), sh, st, a, n_pairs, sy);
+    hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(FM_NW * 64), sh, st, a, n_pairs, f);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 
 template <int BITS, bool FP16>
 int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down, int n_cu,
-                    hipStream_t st, hipEvent_t *kev, const FmGridSync *sy, unsigned int *epoch) {
+                    hipStream_t st, hipEvent_t *kev, const FmFlags *fl, bool *fused) {
     dim3 b(256);
     const int lpr_up = a.g.hidden / FM_CPL, lpr_down = a.g.inter / FM_CPL;
     const bool lds_up = lpr_up >= 4 && lpr_up <= 16, lds_down = lpr_down <= 16;
     if (!lds_down) return FM_ERR_UNSUPPORTED;
     if (kev) (void)hipEventRecord(kev[0], st);
-    if (sy && epoch && lds_up && lpr_down * 4 == lpr_up) {
+    if (fl && lds_up && lpr_down * 4 == lpr_up) {
         int rc = FM_ERR_UNSUPPORTED;
         switch (lpr_up) {
-            case 4: rc = launch_fused<BITS, 4, FP16>(a, n_pairs, n_cu, st, *sy, epoch); break;
-            case 8: rc = launch_fused<BITS, 8, FP16>(a, n_pairs, n_cu, st, *sy, epoch); break;
-            case 16: rc = launch_fused<BITS, 16, FP16>(a, n_pairs, n_cu, st, *sy, epoch); break;
+            case 4: rc = launch_fused<BITS, 4, FP16>(a, n_pairs, n_cu, st, *fl); break;
+            case 8: rc = launch_fused<BITS, 8, FP16>(a, n_pairs, n_cu, st, *fl); break;
+            case 16: rc = launch_fused<BITS, 16, FP16>(a, n_pairs, n_cu, st, *fl); break;
         }
         if (rc != FM_ERR_UNSUPPORTED) {
+            *fused = rc == FM_OK;
             if (kev) {
                 (void)hipEventRecord(kev[1], st);
                 (void)hipEventRecord(kev[2], st);
@@ -741,8 +827,9 @@ int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down, 
 #define FM_UP(L)                                                                   \
     do {                                                                           \
         auto kfn = fm_gate_up_swiglu_lds<BITS, L, FP16>;                           \
-        const size_t sh = fm_stream_lds_bytes<BITS, L>();                          \
-        if (!fm_dyn_lds_ok((const void *)kfn, sh)) return FM_ERR_HIP;              \
+        const size_t sh = fm_phase_lds_bytes<BITS, L>();                           \
+        static FmKernelSetup ks;                                                   \
+        if (!fm_dyn_lds_ok(ks, (const void *)kfn, sh)) return FM_ERR_HIP;          \
         hipLaunchKernelGGL(kfn, g, dim3(FM_NW * 64), sh, st, a, n_pairs);          \
     } while (0)
         switch (lpr_up) {
@@ -768,8 +855,9 @@ int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down, 
 #define FM_DOWN(L)                                                                 \
     do {                                                                           \
         auto kfn = fm_down_lds<BITS, L, FP16>;                                     \
-        const size_t sh = FmDma<BITS>::WG_BYTES + sizeof(FmActLds<L>);             \
-        if (!fm_dyn_lds_ok((const void *)kfn, sh)) return FM_ERR_HIP;              \
+        const size_t sh = fm_phase_lds_bytes<BITS, L>();                           \
+        static FmKernelSetup ks;                                                   \
+        if (!fm_dyn_lds_ok(ks, (const void *)kfn, sh)) return FM_ERR_HIP;          \
         hipLaunchKernelGGL(kfn, g, dim3(FM_NW * 64), sh, st, a, n_pairs);          \
     } while (0)
         switch (lpr_down) {
@@ -810,8 +898,7 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
                                        int n_layers, const float *d_x, const int32_t *d_idx,
                                        const float *d_w, int K, float *d_act,
                                        float *d_expert_out, float *d_out,
-                                       unsigned int *d_sync, unsigned int *epoch,
-                                       unsigned int spin_limit, int flags, int n_cu,
+                                       FmDecodeFlags *df, int flags, int n_cu,
                                        hipStream_t st, hipEvent_t *kev) {
     DecodeArgs a;
     a.layer_ptrs = d_layer_ptrs;
@@ -836,13 +923,29 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     const int want = 4 * n_cu;
     const int rpi_up = pick_rows_per_item(g->inter, n_pairs, min_up, 64, want);
     const int rpi_down = pick_rows_per_item(g->hidden, n_pairs, min_down, 256, want);
-    // d_sync[0] = arrival counter, d_sync[1] = error flag; without them (or with
-    // epoch == NULL) the phases run as separate kernels
-    FmGridSync sy{d_sync, d_sync ? d_sync + 1 : nullptr, 0u, spin_limit};
-    const FmGridSync *syp = d_sync && epoch ? &sy : nullptr;
-#define FM_DEC(B, F) launch_decode_t<B, F>(a, n_pairs, rpi_up, rpi_down, n_cu, st, kev, syp, epoch)
-    if (g->bits == 3) return g->scale_fp16 ? FM_DEC(3, true) : FM_DEC(3, false);
-    if (g->bits == 4) return g->scale_fp16 ? FM_DEC(4, true) : FM_DEC(4, false);
+    // with dependency counters (and room in them) the operator is one launch,
+    // otherwise the phases run as separate kernels
+    const unsigned int need = (unsigned int)(n_pairs + n_layers);
+    FmFlags fl{};
+    const FmFlags *flp = nullptr;
+    if (df && df->set[0] && need <= df->cap) {
+        fl.cur = df->set[df->parity];
+        fl.other = df->set[df->parity ^ 1];
+        fl.clear_n = df->used[df->parity ^ 1];
+        fl.err = df->err;
+        fl.spin_limit = df->spin_limit;
+        flp = &fl;
+    }
+    bool fused = false;
+#define FM_DEC(B, F) launch_decode_t<B, F>(a, n_pairs, rpi_up, rpi_down, n_cu, st, kev, flp, &fused)
+    int rc = FM_ERR_UNSUPPORTED;
+    if (g->bits == 3) rc = g->scale_fp16 ? FM_DEC(3, true) : FM_DEC(3, false);
+    else if (g->bits == 4) rc = g->scale_fp16 ? FM_DEC(4, true) : FM_DEC(4, false);
 #undef FM_DEC
-    return FM_ERR_UNSUPPORTED;
+    if (fused) {   // the set just used is dirty, the other one is clean again
+        df->used[df->parity] = need;
+        df->used[df->parity ^ 1] = 0u;
+        df->parity ^= 1;
+    }
+    return rc;
 }

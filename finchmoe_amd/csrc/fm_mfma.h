@@ -174,30 +174,45 @@ struct FmBuildSlot {
     }
 };
 
-// All 256 threads.  x = the 128*LPR activations in global memory.  The caller
-// puts a barrier before (previous readers done) and after (image complete).
+// The image is built by the first 256 threads of the workgroup in two steps, so
+// that the loads can be issued long before the values are needed:
+//   fm_act_load : this thread's activations -> registers (x = the 128*LPR
+//                 activations in global memory)
+//   fm_act_build: registers -> image.  The caller puts a barrier before the
+//                 image's previous readers are done and after (image complete).
 // SHARED: x was written earlier in this launch or by another CU's kernel and is
 // read with device-scope loads.
-template <int BITS, int LPR, bool SHARED = false>
-__device__ __forceinline__ void fm_build_act_lds(const float *x, const FmBuildSlot<BITS> &bs,
-                                                 FmActLds<LPR> &L) {
+template <int LPR>
+struct FmActX {
+    static constexpr int NIT = (LPR + 3) / 4;     // chunks per thread
+    float xl[NIT], xh[NIT];
+};
+
+template <int BITS, int LPR, bool SHARED>
+__device__ __forceinline__ void fm_act_load(const float *x, const FmBuildSlot<BITS> &bs,
+                                            FmActX<LPR> &r) {
     auto ld = [](const float *p) {
         if constexpr (SHARED)
             return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else
             return *p;
     };
-    constexpr int NE = 4 * LPR;
-    constexpr int NIT = (LPR + 3) / 4;     // chunks per thread
-    const int w = threadIdx.x & 63;
-    float xl[NIT], xh[NIT];
 #pragma unroll
-    for (int i = 0; i < NIT; i++) {
+    for (int i = 0; i < FmActX<LPR>::NIT; i++) {
         const int ch = (threadIdx.x >> 6) + 4 * i;
         const bool on = ch < LPR;
-        xl[i] = on ? ld(x + ch * FM_CPL + bs.lo) : 0.0f;
-        xh[i] = on ? ld(x + ch * FM_CPL + bs.hi) : 0.0f;
+        r.xl[i] = on ? ld(x + ch * FM_CPL + bs.lo) : 0.0f;
+        r.xh[i] = on ? ld(x + ch * FM_CPL + bs.hi) : 0.0f;
     }
+}
+
+template <int BITS, int LPR>
+__device__ __forceinline__ void fm_act_build(const FmActX<LPR> &r, const FmBuildSlot<BITS> &bs,
+                                             FmActLds<LPR> &L) {
+    constexpr int NE = 4 * LPR;
+    constexpr int NIT = FmActX<LPR>::NIT;
+    const int w = threadIdx.x & 63;
+    const float *xl = r.xl, *xh = r.xh;
     uint32_t *flat = reinterpret_cast<uint32_t *>(L.a);
 #pragma unroll
     for (int i = 0; i < NIT; i++) {
