@@ -17,6 +17,8 @@
 // 16-bit, two groups per lane = one dword per lane.
 #include "fm_mfma.h"
 
+#include <type_traits>
+
 namespace {
 
 // waves per workgroup of the streaming kernels: one workgroup per CU, two waves per SIMD
@@ -404,224 +406,350 @@ constexpr size_t fm_phase_lds_bytes() {
     return FmDma<BITS>::WG_BYTES + 2 * sizeof(FmActLds<LPR>) + 3 * sizeof(FmSegTable);
 }
 
-// One phase of the operator over this workgroup's share [U*g/G, U*(g+1)/G) of
-// the phase's units:
-//   GU = true : gate + up + SwiGLU.  unit = RPS rows of gate and of up (two
-//               slices), segment = layer, input a.x, output a.act
-//   GU = false: down projection.  unit = RPS rows (one slice), segment = pair,
-//               input a.act, output a.expert_out
-// An invalid expert index streams expert 0 and contributes zero.
+// The operator's two streaming phases over this workgroup's shares
+// [U*g/G, U*(g+1)/G) of each phase's units:
+//   gate/up: unit = RPS rows of gate and of up (two slices), segment = layer,
+//            input a.x, output a.act (SwiGLU applied)
+//   down   : unit = RPS rows (one slice), segment = pair, input a.act, output
+//            a.expert_out
+// DO_UP / DO_DOWN select the phases (one of them: the separate kernels).  An
+// invalid expert index streams expert 0 and contributes zero.
 //
-// The share is one continuous stream.  Per segment only the activation image
-// changes, and everything a change needs is fetched a segment ahead (the next
-// segment's activations into registers, its expert indices two segments ahead),
-// while the loaders run on into the next segment's units as soon as the current
-// one is handed out — a slice's tag says which segment it belongs to, and a
-// wave that meets a slice of the next segment waits for the workgroup to switch
-// image.
-template <int BITS, int LPR, bool FP16, bool GU, class Deps>
-__device__ __forceinline__ void fm_stream_phase(const DecodeArgs &a, int n_pairs,
-                                                const Deps &deps) {
+// The shares form one continuous stream of segments, numbered in sequence
+// across both phases.  Per segment only the activation image changes, and what
+// a change needs is fetched ahead (the next segment's activations into
+// registers, its expert indices two segments ahead), while the loaders run on
+// into the next segment's units — also from the last gate/up segment into the
+// first down segment, whose weights depend on nothing — as soon as the current
+// one is handed out.  A slice's tag says which segment it belongs to, and a
+// wave that meets a slice of the next segment waits for the workgroup to
+// switch image.
+// (A struct with inlined member functions rather than nested lambdas: the
+// compiler keeps lambda closures that capture one another in private memory,
+// and every access to it counts against the vector-memory counter the ring's
+// waits rely on.)
+template <int BITS, int LPR_UP, int LPR_DOWN, bool FP16, bool DO_UP, bool DO_DOWN, class DepsUp,
+          class DepsDown>
+struct FmOperatorStream {
     using D = FmDma<BITS>;
-    constexpr int RPS = FM_WAVE / LPR, RING = D::RING;
-    FmActLds<LPR> *img = reinterpret_cast<FmActLds<LPR> *>(fm_dyn_lds + D::WG_BYTES);
-    FmSegTable *tab =
-        reinterpret_cast<FmSegTable *>(fm_dyn_lds + D::WG_BYTES + 2 * sizeof(FmActLds<LPR>));
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t ring0 =
-        (uint32_t)(uintptr_t)(fm_lptr)fm_dyn_lds + (uint32_t)wave * (RING * D::BYTES);
-    const int in_dim = GU ? a.g.hidden : a.g.inter, out_dim = GU ? a.g.inter : a.g.hidden;
-    const uint32_t upp = (uint32_t)(out_dim / RPS);               // units per pair
-    const long segu = GU ? (long)upp * a.K : (long)upp;           // units per segment
-    const int NK = GU ? a.K : 1;                                  // experts per segment
-    const long total = (long)n_pairs * upp;
-    const long wg0 = total * blockIdx.x / gridDim.x, wg1 = total * (blockIdx.x + 1) / gridDim.x;
-    if (wg0 >= wg1) return;
-    const int s_begin = (int)(wg0 / segu), s_end = (int)((wg1 - 1) / segu) + 1;
-    const int row_bytes = in_dim * BITS / 8, sb_row_bytes = (in_dim / 64) * 2;
-    uint32_t woff, soff;
-    int ris, ch;
-    fm_unit_lane_offsets<BITS, LPR>(lane, row_bytes, sb_row_bytes, woff, soff, ris, ch);
-    const uint32_t wstep = (uint32_t)(RPS * row_bytes), sstep = (uint32_t)(RPS * sb_row_bytes);
-    // region offsets as scalars (selected per half step with a scalar select)
-    const uint32_t w0 = GU ? a.g.gate_w : a.g.down_w, s0 = GU ? a.g.gate_s : a.g.down_s,
-                   b0 = GU ? a.g.gate_b : a.g.down_b;
-    const uint32_t w1 = a.g.up_w, s1 = a.g.up_s, b1 = a.g.up_b;
-    FmBuildSlot<BITS> bslot;
-    bslot.init();
-
-    // this workgroup's part of segment s: first unit (inside the segment) and count
-    auto seg_part = [&](int s, uint32_t &first, uint32_t &n) {
-        const long lo = (long)s * segu > wg0 ? (long)s * segu : wg0;
-        const long hi = (long)(s + 1) * segu < wg1 ? (long)(s + 1) * segu : wg1;
-        first = (uint32_t)(lo - (long)s * segu);
-        n = (uint32_t)(hi - lo);
-    };
-    // expert index and layer blob of this lane's slot of segment s (wave 0, lanes < NK)
-    struct Raw {
+    static constexpr int RING = D::RING;
+    static constexpr int LPR_MAX = LPR_UP > LPR_DOWN ? LPR_UP : LPR_DOWN;
+    static constexpr int RPS_UP = FM_WAVE / LPR_UP, RPS_DN = FM_WAVE / LPR_DOWN;
+    struct Raw {            // expert index and layer blob of one slot of a segment
         int e;
         const uint8_t *layer;
     };
-    auto load_raw = [&](int s) {
+
+    const DecodeArgs &a;
+    const DepsUp &deps_up;
+    const DepsDown &deps_down;
+    int lane, wave;
+    uint32_t ring0;
+    uint8_t *img_mem;       // two images
+    FmSegTable *tab;        // three tables
+    // geometry of the two phases: units per pair / per segment, this workgroup's
+    // units and segments, bytes per unit in the code and in the scale/bias regions
+    uint32_t gu_upp, dn_upp;
+    long gu_segu, dn_segu, gu_wg0, gu_wg1, dn_wg0, dn_wg1;
+    int gu_s0, dn_s0, n_up, n_seq;
+    uint32_t gu_wstep, gu_sstep, dn_wstep, dn_sstep;
+    // Loader's current phase: bytes per unit, region offsets of a unit's first
+    // slice, and how far the second slice (up after gate) lies behind it.  Kept
+    // as plain members that are assigned at the phase change: a `c ? m1 : m2` on
+    // two members turns into one load from a selected address, which pins the
+    // whole object in private memory.
+    bool l_gu;
+    uint32_t cur_wstep, cur_sstep, cur_w, cur_s, cur_b, d_w, d_s, d_b;
+    int dn_adj;             // dn_s0 - gu_s0 - n_up
+    // loader / multiply state
+    int lq, cq;             // segment of the loader / of the multiply
+    uint32_t l_first, l_n;
+    int hn, wpos, c;
+    uint32_t tag_n, rsn, issued, consumed;
+    const uint8_t *blob_n;
+    bool dry;               // nothing more to hand out for now
+    Raw raw_next;           // of segment cq + 2
+    FmBuildSlot<BITS> bslot;
+
+    __device__ __forceinline__ FmOperatorStream(const DecodeArgs &a_, int n_pairs,
+                                                const DepsUp &du, const DepsDown &dd)
+        : a(a_), deps_up(du), deps_down(dd) {
+        lane = threadIdx.x & 63;
+        wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        ring0 = (uint32_t)(uintptr_t)(fm_lptr)fm_dyn_lds + (uint32_t)wave * (RING * D::BYTES);
+        img_mem = fm_dyn_lds + D::WG_BYTES;
+        tab = reinterpret_cast<FmSegTable *>(fm_dyn_lds + D::WG_BYTES +
+                                             2 * sizeof(FmActLds<LPR_MAX>));
+        gu_upp = (uint32_t)(a.g.inter / RPS_UP);
+        dn_upp = (uint32_t)(a.g.hidden / RPS_DN);
+        gu_segu = (long)gu_upp * a.K;
+        dn_segu = (long)dn_upp;
+        const long gu_total = DO_UP ? (long)n_pairs * gu_upp : 0;
+        const long dn_total = DO_DOWN ? (long)n_pairs * dn_upp : 0;
+        gu_wg0 = gu_total * blockIdx.x / gridDim.x;
+        gu_wg1 = gu_total * (blockIdx.x + 1) / gridDim.x;
+        dn_wg0 = dn_total * blockIdx.x / gridDim.x;
+        dn_wg1 = dn_total * (blockIdx.x + 1) / gridDim.x;
+        gu_s0 = (int)(gu_wg0 / gu_segu);
+        dn_s0 = (int)(dn_wg0 / dn_segu);
+        n_up = gu_wg1 > gu_wg0 ? (int)((gu_wg1 - 1) / gu_segu) + 1 - gu_s0 : 0;
+        const int n_dn = dn_wg1 > dn_wg0 ? (int)((dn_wg1 - 1) / dn_segu) + 1 - dn_s0 : 0;
+        n_seq = n_up + n_dn;
+        gu_wstep = (uint32_t)(RPS_UP * (a.g.hidden * BITS / 8));
+        gu_sstep = (uint32_t)(RPS_UP * (a.g.hidden / 64) * 2);
+        dn_wstep = (uint32_t)(RPS_DN * (a.g.inter * BITS / 8));
+        dn_sstep = (uint32_t)(RPS_DN * (a.g.inter / 64) * 2);
+        dn_adj = dn_s0 - gu_s0 - n_up;
+        d_w = a.g.up_w - a.g.gate_w;
+        d_s = a.g.up_s - a.g.gate_s;
+        d_b = a.g.up_b - a.g.gate_b;
+        if (DO_UP && n_up > 0) {
+            l_gu = true;
+            cur_wstep = gu_wstep, cur_sstep = gu_sstep;
+            cur_w = a.g.gate_w, cur_s = a.g.gate_s, cur_b = a.g.gate_b;
+        } else {
+            loader_to_down();
+        }
+        lq = cq = 0;
+        l_first = l_n = 0;
+        hn = wpos = c = 0;
+        tag_n = rsn = issued = consumed = 0;
+        blob_n = nullptr;
+        dry = false;
+        raw_next = Raw{0, nullptr};
+        bslot.init();
+    }
+
+    __device__ __forceinline__ void loader_to_down() {
+        l_gu = false;
+        cur_wstep = dn_wstep, cur_sstep = dn_sstep;
+        cur_w = a.g.down_w, cur_s = a.g.down_s, cur_b = a.g.down_b;
+    }
+    // segment number q of the sequence -> phase and segment of that phase
+    __device__ __forceinline__ bool seq_gu(int q) const { return q < n_up; }
+    __device__ __forceinline__ int seq_seg(int q) const {
+        return gu_s0 + q + (q < n_up ? 0 : dn_adj);
+    }
+    // this workgroup's part of it: first unit (inside the segment) and count
+    template <bool GU>
+    __device__ __forceinline__ void seq_part(int q, uint32_t &first, uint32_t &n) const {
+        const long s = seq_seg(q);
+        long segu, w0, w1;
+        if constexpr (GU) segu = gu_segu, w0 = gu_wg0, w1 = gu_wg1;
+        else segu = dn_segu, w0 = dn_wg0, w1 = dn_wg1;
+        const long lo = s * segu > w0 ? s * segu : w0;
+        const long hi = (s + 1) * segu < w1 ? (s + 1) * segu : w1;
+        first = (uint32_t)(lo - s * segu);
+        n = (uint32_t)(hi - lo);
+    }
+    // the loader enters segment q
+    __device__ __forceinline__ void loader_enter(int q) {
+        if (l_gu && q >= n_up) loader_to_down();
+        if (l_gu) seq_part<true>(q, l_first, l_n);
+        else seq_part<false>(q, l_first, l_n);
+    }
+    // wave 0, lanes < K (gate/up) or lane 0 (down)
+    __device__ __forceinline__ Raw load_raw(int q) const {
         Raw r{0, nullptr};
-        if (wave == 0 && lane < NK) {
-            const int l = GU ? s : s / a.K;
-            r.e = a.idx[GU ? s * a.K + lane : s];
+        const bool gu = seq_gu(q);
+        const int s = seq_seg(q);
+        if (wave == 0 && lane < (gu ? a.K : 1)) {
+            const int l = gu ? s : s / a.K;
+            r.e = a.idx[gu ? s * a.K + lane : s];
             r.layer = a.layer_ptrs[a.layer0 + l * a.layer_stride];
         }
         return r;
-    };
-    auto write_table = [&](int s, const Raw &r) {
+    }
+    __device__ __forceinline__ void write_table(int q, const Raw &r) const {
         if (wave == 0) {
-            FmSegTable &t = tab[s % 3];
-            const bool ok = lane < NK && (unsigned)r.e < (unsigned)a.g.n_experts;
-            if (lane < NK) t.blob[lane] = r.layer + (size_t)(ok ? r.e : 0) * a.g.expert_size;
+            FmSegTable &t = tab[q % 3];
+            const int nk = seq_gu(q) ? a.K : 1;
+            const bool ok = lane < nk && (unsigned)r.e < (unsigned)a.g.n_experts;
+            if (lane < nk) t.blob[lane] = r.layer + (size_t)(ok ? r.e : 0) * a.g.expert_size;
             const uint64_t m = __ballot(ok);
             if (lane == 0) {
                 t.valid = (uint32_t)m;
                 t.next_unit = 0u;
             }
         }
-    };
-    auto in_vec = [&](int s) {
-        return GU ? a.x + (size_t)s * a.g.hidden : a.act + (size_t)s * a.g.inter;
-    };
+    }
+    template <bool GU>
+    __device__ __forceinline__ void publish(int q) const {   // by wave 0, after a barrier
+        if (wave == 0) {
+            uint32_t pf, pc;
+            seq_part<GU>(q, pf, pc);
+            if constexpr (GU) deps_up.publish(seq_seg(q), pf, pc);
+            else deps_down.publish(seq_seg(q), pf, pc);
+        }
+    }
 
-    // ---- loader: the next slice (gate rows, then up rows of the same unit)
-    int ls = s_begin, cs = s_begin;     // segment of the loader / of the multiply
-    uint32_t l_first, l_n;
-    seg_part(ls, l_first, l_n);
-    int hn = 0, wpos = 0;
-    uint32_t tag_n = 0, rsn = 0, issued = 0, consumed = 0;
-    const uint8_t *blob_n = nullptr;
-    bool dry = false;                   // nothing more to hand out for now
-    auto issue = [&]() {
+    // loader: the next slice of the stream (gate rows, then up rows of the same unit)
+    __device__ __forceinline__ void issue() {
         if (dry) return;
-        if (!GU || hn == 0) {
+        if (!l_gu || hn == 0) {
             uint32_t ul;
             for (;;) {
-                ul = fm_claim_unit(&tab[ls % 3].next_unit, lane);
+                ul = fm_claim_unit(&tab[lq % 3].next_unit, lane);
                 if (ul < l_n) break;
-                if (ls + 1 < s_end && ls == cs) {       // run on into the next segment
-                    ls++;
-                    seg_part(ls, l_first, l_n);
+                if (lq + 1 < n_seq && lq == cq) {       // run on into the next segment
+                    lq++;
+                    loader_enter(lq);
                     continue;
                 }
                 dry = true;
                 return;
             }
             const uint32_t uq = l_first + ul;                     // unit inside the segment
-            const uint32_t pn = GU ? uq / upp : 0u;
-            rsn = uq - pn * upp;
-            tag_n = ((uint32_t)(ls & 1) << 31) | (pn << 28) | ul;
-            blob_n = fm_uniform(tab[ls % 3].blob[pn]);
+            const uint32_t pn = l_gu ? uq / gu_upp : 0u;
+            rsn = uq - pn * gu_upp;
+            tag_n = ((uint32_t)(lq & 1) << 31) | (pn << 28) | ul;
+            blob_n = fm_uniform(tab[lq % 3].blob[pn]);
         }
         const uint32_t slot = ring0 + (uint32_t)wpos * D::BYTES;
         fm_slot_tag(slot + D::TAG, tag_n);
-        const uint8_t *b = blob_n + (size_t)rsn * wstep;
-        const uint8_t *sb = blob_n + (size_t)rsn * sstep;
-        const bool second = GU && hn;
-        fm_dma_issue<BITS>(slot, b + (second ? w1 : w0), sb + (second ? s1 : s0),
-                           sb + (second ? b1 : b0), lane);
-        if (GU) hn ^= 1;
+        const uint8_t *b = blob_n + (size_t)rsn * cur_wstep;
+        const uint8_t *sb = blob_n + (size_t)rsn * cur_sstep;
+        const uint32_t second = (uint32_t)hn;                     // 1: the up rows of a unit
+        fm_dma_issue<BITS>(slot, b + cur_w + second * d_w, sb + cur_s + second * d_s,
+                           sb + cur_b + second * d_b, lane);
+        if (l_gu) hn ^= 1;
         wpos = wpos + 1 == RING ? 0 : wpos + 1;
         issued++;
-    };
-
-    // ---- start: tables of the first two segments, first loads, first input vector
-    FmActX<LPR> xr;
-    if (GU && threadIdx.x < 256) fm_act_load<BITS, LPR, false>(in_vec(s_begin), bslot, xr);
-    __syncthreads();                              // the previous phase is done with this LDS
-    {
-        const Raw r0 = load_raw(s_begin);
-        const Raw r1 = load_raw(s_begin + 1 < s_end ? s_begin + 1 : s_begin);
-        write_table(s_begin, r0);
-        if (s_begin + 1 < s_end) write_table(s_begin + 1, r1);
-    }
-    Raw raw_next = load_raw(s_begin + 2 < s_end ? s_begin + 2 : s_begin);   // for segment cs + 2
-    __syncthreads();
-#pragma unroll
-    for (int k = 0; k < RING; k++) issue();
-    if (!GU && threadIdx.x < 256) {
-        deps.wait_in(s_begin);
-        fm_act_load<BITS, LPR, true>(in_vec(s_begin), bslot, xr);
     }
 
-    int c = 0;
-    for (; cs < s_end; cs++) {
-        // ---- switch to the image of segment cs
-        if (threadIdx.x < 256) fm_act_build<BITS, LPR>(xr, bslot, img[cs & 1]);
-        const bool new_table = cs > s_begin && cs + 1 < s_end;
-        // every loader has left segment cs-2: its table becomes that of cs+1
-        if (new_table) write_table(cs + 1, raw_next);
+    // the oldest slice of the ring times the activation registers
+    template <int LPR>
+    __device__ __forceinline__ float take(uint32_t woff, uint32_t soff, const FmActRegs &ar) {
+        FmRowSlice<BITS> t;
+        if (issued - consumed == (uint32_t)RING) fm_dma_wait<D::LOADS *(RING - 1)>(false);
+        else fm_dma_wait<0>(true);
+        fm_dma_read<BITS>(ring0 + (uint32_t)c * D::BYTES, woff, soff, t);
+        consumed++;
+        c = c + 1 == RING ? 0 : c + 1;
+        issue();
+        return fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(t, ar));
+    }
+
+    // tables of the first two segments, first loads
+    __device__ __forceinline__ void start() {
+        loader_enter(0);
+        __syncthreads();                              // LDS is free
+        const Raw r0 = load_raw(0);
+        const Raw r1 = load_raw(n_seq > 1 ? 1 : 0);
+        write_table(0, r0);
+        if (n_seq > 1) write_table(1, r1);
+        raw_next = load_raw(n_seq > 2 ? 2 : 0);
         __syncthreads();
-        if (cs > s_begin && wave == 0) {          // every wave is done with segment cs-1
-            uint32_t pf, pn_;
-            seg_part(cs - 1, pf, pn_);
-            deps.publish(cs - 1, pf, pn_);
-        }
-        FmActRegs ar;
-        fm_read_act_lds<LPR>(img[cs & 1], lane, ar);
-        const uint32_t valid = __builtin_amdgcn_readfirstlane(tab[cs % 3].valid);
-        uint32_t c_first, c_n;
-        seg_part(cs, c_first, c_n);
-        const size_t out0 = (size_t)((long)cs * segu + c_first) * RPS + ris;
-        float *out_vec = GU ? a.act : a.expert_out;
-        // fetched now, used at the next switch
-        if (cs + 1 < s_end && threadIdx.x < 256) {
-            deps.wait_in(cs + 1);
-            fm_act_load<BITS, LPR, !GU>(in_vec(cs + 1), bslot, xr);
-        }
-        if (new_table) raw_next = load_raw(cs + 2 < s_end ? cs + 2 : cs);
-        dry = false;
-        while (issued - consumed < (uint32_t)RING && !dry) issue();
+#pragma unroll
+        for (int k = 0; k < RING; k++) issue();
+    }
 
-        // ---- multiply the slices of this segment
-        auto take = [&]() {
-            FmRowSlice<BITS> t;
-            if (issued - consumed == (uint32_t)RING) fm_dma_wait<D::LOADS *(RING - 1)>(false);
-            else fm_dma_wait<0>(true);
-            fm_dma_read<BITS>(ring0 + (uint32_t)c * D::BYTES, woff, soff, t);
-            consumed++;
-            c = c + 1 == RING ? 0 : c + 1;
-            issue();
-            return fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(t, ar));
-        };
-        while (consumed < issued) {
-            const uint32_t tag = fm_slot_peek(ring0 + (uint32_t)c * D::BYTES + D::TAG);
-            if ((tag >> 31) != (uint32_t)(cs & 1)) break;         // belongs to the next segment
-            const uint32_t pc = (tag >> 28) & 7u, ul = tag & 0x0FFFFFFFu;
-            float v;
-            if constexpr (GU) {
-                const float gv = take();
-                const float uv = take();
-                v = fm_silu_mul(gv, uv);
-            } else {
-                v = take();
+    // the segments [cq, q1) of one phase.  xr: the first segment's input vector
+    // (gate/up), or nothing yet (down)
+    template <int LPR, bool GU, class Deps>
+    __device__ __forceinline__ void run_phase(FmActX<LPR> &xr, const Deps &deps, int q1) {
+        constexpr int RPS = FM_WAVE / LPR;
+        const int q0 = cq;
+        const long segu_c = GU ? gu_segu : dn_segu;
+        const int in_dim = GU ? a.g.hidden : a.g.inter;
+        uint32_t woff, soff;
+        int ris, ch;
+        fm_unit_lane_offsets<BITS, LPR>(lane, in_dim * BITS / 8, (in_dim / 64) * 2, woff, soff, ris,
+                                        ch);
+        const float *in_base = GU ? a.x : a.act;
+        float *out_vec = GU ? a.act : a.expert_out;
+        for (; cq < q1; cq++) {
+            const int s = seq_seg(cq);
+            FmActLds<LPR> &img = *reinterpret_cast<FmActLds<LPR> *>(
+                img_mem + (cq & 1) * sizeof(FmActLds<LPR_MAX>));
+            // ---- switch to the image of this segment
+            const bool first_down = !GU && cq == q0;
+            if (first_down) {
+                // the first down vector may be this workgroup's own: it is not fetched
+                // ahead, and what the workgroup has produced is published before the wait
+                __syncthreads();
+                if (cq > 0) publish<true>(cq - 1);
+                if (threadIdx.x < 256) {
+                    deps.wait_in(s);
+                    fm_act_load<BITS, LPR, true>(in_base + (size_t)s * in_dim, bslot, xr);
+                }
             }
-            if (!((valid >> pc) & 1u)) v = 0.0f;
-            // unit (pair, row step): the output is [pair][rows], rows are contiguous
-            if (ch == 0) fm_st_shared(out_vec + out0 + (size_t)ul * RPS, v);
+            if (threadIdx.x < 256) fm_act_build<BITS, LPR>(xr, bslot, img);
+            const bool new_table = cq > 0 && cq + 1 < n_seq;
+            // every loader has left segment cq-2: its table becomes that of cq+1
+            if (new_table) write_table(cq + 1, raw_next);
+            __syncthreads();
+            if (!first_down && cq > 0) publish<GU>(cq - 1);   // every wave is done with it
+            FmActRegs ar;
+            fm_read_act_lds<LPR>(img, lane, ar);
+            const uint32_t valid = __builtin_amdgcn_readfirstlane(tab[cq % 3].valid);
+            uint32_t c_first, c_n;
+            seq_part<GU>(cq, c_first, c_n);
+            const size_t out0 = (size_t)((long)s * segu_c + c_first) * RPS + ris;
+            // fetched now, used at the next switch
+            if (cq + 1 < q1 && threadIdx.x < 256) {
+                deps.wait_in(s + 1);
+                fm_act_load<BITS, LPR, !GU>(in_base + (size_t)(s + 1) * in_dim, bslot, xr);
+            }
+            if (new_table) raw_next = load_raw(cq + 2 < n_seq ? cq + 2 : cq);
+            dry = false;
+            while (issued - consumed < (uint32_t)RING && !dry) issue();
+
+            // ---- multiply the slices of this segment
+            while (consumed < issued) {
+                const uint32_t tag = fm_slot_peek(ring0 + (uint32_t)c * D::BYTES + D::TAG);
+                if ((tag >> 31) != (uint32_t)(cq & 1)) break;     // belongs to the next segment
+                const uint32_t pc = (tag >> 28) & 7u, ul = tag & 0x0FFFFFFFu;
+                float v;
+                if constexpr (GU) {
+                    const float gv = take<LPR>(woff, soff, ar);
+                    const float uv = take<LPR>(woff, soff, ar);
+                    v = fm_silu_mul(gv, uv);
+                } else {
+                    v = take<LPR>(woff, soff, ar);
+                }
+                if (!((valid >> pc) & 1u)) v = 0.0f;
+                // unit (pair, row step): the output is [pair][rows], rows are contiguous
+                if (ch == 0) fm_st_shared(out_vec + out0 + (size_t)ul * RPS, v);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's stores have completed
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's stores have completed
     }
-    __syncthreads();
-    if (wave == 0) {
-        uint32_t pf, pn_;
-        seg_part(s_end - 1, pf, pn_);
-        deps.publish(s_end - 1, pf, pn_);
+
+    __device__ __forceinline__ void run() {
+        if (n_seq == 0) return;
+        FmActX<LPR_UP> xr_up;
+        if (n_up > 0 && threadIdx.x < 256)
+            fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)seq_seg(0) * a.g.hidden, bslot, xr_up);
+        start();
+        if constexpr (DO_UP) run_phase<LPR_UP, true>(xr_up, deps_up, n_up);
+        if constexpr (DO_DOWN) {
+            FmActX<LPR_DOWN> xr_dn;
+            run_phase<LPR_DOWN, false>(xr_dn, deps_down, n_seq);
+        }
+        __syncthreads();
+        publish<!DO_DOWN>(n_seq - 1);
     }
+};
+
+template <int BITS, int LPR_UP, int LPR_DOWN, bool FP16, bool DO_UP, bool DO_DOWN, class DepsUp,
+          class DepsDown>
+__device__ __forceinline__ void fm_stream_operator(const DecodeArgs &a, int n_pairs,
+                                                   const DepsUp &deps_up,
+                                                   const DepsDown &deps_down) {
+    FmOperatorStream<BITS, LPR_UP, LPR_DOWN, FP16, DO_UP, DO_DOWN, DepsUp, DepsDown> st(
+        a, n_pairs, deps_up, deps_down);
+    st.run();
 }
 
 template <int BITS, int LPR, bool FP16>
 __global__ __launch_bounds__(FM_NW * 64) void fm_gate_up_swiglu_lds(DecodeArgs a, int n_pairs) {
-    fm_stream_phase<BITS, LPR, FP16, true>(a, n_pairs, FmNoDeps());
+    fm_stream_operator<BITS, LPR, LPR, FP16, true, false>(a, n_pairs, FmNoDeps(), FmNoDeps());
 }
 
 template <int BITS, int LPR, bool FP16>
 __global__ __launch_bounds__(FM_NW * 64) void fm_down_lds(DecodeArgs a, int n_pairs) {
-    fm_stream_phase<BITS, LPR, FP16, false>(a, n_pairs, FmNoDeps());
+    fm_stream_operator<BITS, LPR, LPR, FP16, false, true>(a, n_pairs, FmNoDeps(), FmNoDeps());
 }
 
 // ======================================================================
@@ -711,9 +839,8 @@ void fm_moe_fused(DecodeArgs a, int n_pairs, FmFlags f) {
         f.other[i] = 0u;
     const uint32_t upp_up = (uint32_t)(a.g.inter / (FM_WAVE / LPR_UP));
     const uint32_t upp_down = (uint32_t)(H / (FM_WAVE / LPR_DOWN));
-    fm_stream_phase<BITS, LPR_UP, FP16, true>(a, n_pairs, FmGateUpDeps{f, a.K, upp_up});
-    fm_stream_phase<BITS, LPR_DOWN, FP16, false>(a, n_pairs,
-                                                 FmDownDeps{f, a.K, n_pairs, upp_up});
+    fm_stream_operator<BITS, LPR_UP, LPR_DOWN, FP16, true, true>(
+        a, n_pairs, FmGateUpDeps{f, a.K, upp_up}, FmDownDeps{f, a.K, n_pairs, upp_up});
     // combine: a group's K expert outputs are complete at K * upp_down units
     const unsigned int full = (unsigned int)a.K * upp_down;
     if (a.flags & FM_GUARD) {
