@@ -28,10 +28,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 peak
-# HBM bytes per launch of the gate+up kernel on the default workload, from rocprofv3 --pmc
-# FETCH_SIZE (x2: calibrated against a 1 GiB copy) + WRITE_SIZE, see
+# HBM bytes per launch of the fused decode kernel on the default workload, from rocprofv3
+# --pmc FETCH_SIZE (x2: calibrated against a 1 GiB copy) + WRITE_SIZE, see
 # profiles/decode_step_3bit_hbm_traffic.md.  Offline measurement; null for other sizes.
-GATE_UP_TRAFFIC_BYTES_40L = 289838 * 1024 + 676 * 1024
+FUSED_TRAFFIC_BYTES_40L = int((218295.98 * 2 + 4186.4) * 1024)
 
 H, I, E, K, L = 2048, 512, 256, 8, 40
 
@@ -153,12 +153,15 @@ def run_decode_step(args):
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
 
-    # per-kernel durations (HIP events on the library's stream, call by call)
-    ctx.kernel_timing(True)
-    for t in range(args.steps):
+    # The operator is one kernel per step, so the HIP events around the timed region
+    # (on the library's stream) give its average launch duration: ev_ms / steps.
+    op_us = ev_ms / args.steps * 1e3
+    # the phases as separate kernels, each call bracketed by events and waited for
+    ctx.kernel_timing(2)
+    for t in range(min(args.steps, 300)):
         step(args.warmup + t)
     k1_ms, k2_ms, n = ctx.kernel_timing_read()
-    ctx.kernel_timing(False)
+    ctx.kernel_timing(0)
     k1_us, k2_us = k1_ms / n * 1e3, k2_ms / n * 1e3
 
     # per-token latency distribution over 256 consecutive tokens (wall clock incl. sync)
@@ -199,16 +202,17 @@ def run_decode_step(args):
         "token_latency_us": {"mean": round(float(lat.mean()), 1), "p50": round(float(np.median(lat)), 1),
                              "p99": round(float(np.percentile(lat, 99)), 1)},
         "unique_experts_touched_in_256_tokens": uniq,
-        "kernels_us": {"fm_gate_up_swiglu": round(k1_us, 2), "fm_down+fm_combine": round(k2_us, 2)},
-        "roofline": {"bound": "hbm", "kernel": "fm_gate_up_swiglu<3,16>",
-                     "achieved": round(k1_bytes / (k1_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(k1_bytes / (k1_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": GATE_UP_TRAFFIC_BYTES_40L if (n_layers, E, K) == (40, 256, 8) else None,
-                     "bytes_per_launch": k1_bytes},
-        "roofline_down": {"bound": "hbm", "kernel": "fm_down<3,4> + fm_combine",
-                          "achieved": round((bytes_step - k1_bytes) / (k2_us * 1e-6) / 1e9, 1),
-                          "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": round((bytes_step - k1_bytes) / (k2_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)},
+        "roofline": {"bound": "hbm", "kernel": "fm_moe_fused<3,16> (gate/up, down, combine in one launch)",
+                     "achieved": round(bytes_step / (op_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(bytes_step / (op_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": FUSED_TRAFFIC_BYTES_40L if (n_layers, E, K) == (40, 256, 8) else None,
+                     "bytes_per_launch": bytes_step, "us_per_launch": round(op_us, 2)},
+        # the same work as three separate kernels (isolated launches, so a little slower
+        # than back to back): where the time goes
+        "phases_as_kernels_us": {"fm_gate_up_swiglu_lds": round(k1_us, 2),
+                                 "fm_down_lds+fm_combine": round(k2_us, 2),
+                                 "gate_up_GBps": round(k1_bytes / (k1_us * 1e-6) / 1e9, 1),
+                                 "down_GBps": round((bytes_step - k1_bytes) / (k2_us * 1e-6) / 1e9, 1)},
     }
     if not args.no_cpu:
         res["cpu_baseline"] = cpu_baseline_decode(blob, lo, idx, w, x, args.cpu_seconds)
