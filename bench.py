@@ -298,13 +298,13 @@ def run_decode_layer(args):
                            d_out.data_ptr() + l * H * 4)
 
     ms, ev = _timed(ctx, step, args)
-    ctx.kernel_timing(True)
+    ctx.kernel_timing(2)   # the phases as separate kernels, isolated launches
     for t in range(args.steps):
         step(t)
     k1, k2, n = ctx.kernel_timing_read()
-    ctx.kernel_timing(False)
-    res = {"kernels_us": {"fm_gate_up_swiglu_mfma": round(k1 / n * 1e3, 2),
-                          "fm_down_mfma+fm_combine": round(k2 / n * 1e3, 2)},
+    ctx.kernel_timing(0)
+    res = {"phases_as_kernels_us": {"fm_gate_up_swiglu_lds": round(k1 / n * 1e3, 2),
+                                    "fm_down_lds+fm_combine": round(k2 / n * 1e3, 2)},
            "event_ms_per_step": round(ev, 5)}
     ctx.close()
     return _finish(res, "3-bit expert GEMV HBM GB/s, one MoE layer per call", "config 0: single MoE layer, decode "
@@ -397,7 +397,7 @@ def run_gguf(args):
     for t in range(args.steps):
         step(t)
     k1, k2, n = ctx.kernel_timing_read()
-    ctx.kernel_timing(False)
+    ctx.kernel_timing(0)
     assert torch.isfinite(d_out).all()
     res = {"kernels_us": {"fm_gguf_gate_up": round(k1 / n * 1e3, 2),
                           "fm_gguf_down+combine": round(k2 / n * 1e3, 2)},

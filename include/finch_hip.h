@@ -83,13 +83,17 @@ FM_API const char *fm_status_string(int status);
 FM_API int fm_timer_start(fm_ctx *ctx);
 FM_API int fm_timer_stop(fm_ctx *ctx, float *elapsed_ms);   /* waits for the stop event */
 
-/* Per-kernel timing of the routed-expert decode calls.  While enabled, every
- * fm_*moe_decode*_dev call brackets its two kernels (gate+up+SwiGLU, then
- * down+combine) with events on the context's stream and waits for them, so the
- * call becomes synchronous; the durations accumulate until read.  For
- * measurement runs only (the reference's --timing accumulators,
- * finchmoe/infer.m:281-298, play this role). */
-FM_API int fm_kernel_timing(fm_ctx *ctx, int enable);
+/* Timing of the routed-expert decode calls with events on the context's stream.
+ * mode 1: events around the operator as it is launched (one fused kernel where the
+ *         shape allows): fm_kernel_timing_read returns its duration in gate_up_ms
+ *         and ~0 in down_ms.
+ * mode 2: the phases run as separate kernels (gate+up+SwiGLU, then down+combine)
+ *         and each is timed.
+ * mode 0: off.  While on, every fm_*moe_decode*_dev call waits for its events, so the
+ * call becomes synchronous; the durations accumulate until read.  For measurement
+ * runs only (the reference's --timing accumulators, finchmoe/infer.m:281-298, play
+ * this role). */
+FM_API int fm_kernel_timing(fm_ctx *ctx, int mode);
 /* sums in milliseconds since the last read, and the number of calls; resets */
 FM_API int fm_kernel_timing_read(fm_ctx *ctx, double *gate_up_ms, double *down_ms, int *calls);
 
