@@ -61,6 +61,7 @@ def load():
         "fm_timer_start": (i, [vp]),
         "fm_timer_stop": (i, [vp, C.POINTER(C.c_float)]),
         "fm_kernel_timing": (i, [vp, i]),
+        "fm_set_wait_limit": (i, [vp, C.c_uint]),
         "fm_kernel_timing_read": (i, [vp, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i)]),
         "fm_experts_config": (i, [vp, i, i, i, i, i, i, i]),
         "fm_experts_expert_size": (sz, [vp]),
@@ -152,6 +153,9 @@ class FinchHip:
 
     def kernel_timing(self, enable):
         self._chk(self.L.fm_kernel_timing(self.h, int(enable)))
+
+    def set_wait_limit(self, polls):
+        self._chk(self.L.fm_set_wait_limit(self.h, C.c_uint(polls)))
 
     def kernel_timing_read(self):
         a, b, n = C.c_double(), C.c_double(), C.c_int()

@@ -73,6 +73,7 @@ struct fm_ctx {
     // dependency counters (allocated with the scratch)
     unsigned int *h_err = nullptr, *d_err = nullptr;
     FmDecodeFlags dflags{};
+    unsigned int wait_limit = 1u << 20;
     bool split_phases = false;     // run the phases as separate kernels
     bool sync_unchecked = false;   // a fused launch has not had its error flag read yet
     double k1_ms = 0.0, k2_ms = 0.0;
@@ -188,7 +189,7 @@ int ensure_scratch(fm_ctx *c, int groups, int hidden, int inter) {
         c->dflags.set[1] = p + cap;
         c->dflags.cap = (unsigned int)cap;
         c->dflags.err = c->d_err;
-        c->dflags.spin_limit = 1u << 20;
+        c->dflags.spin_limit = c->wait_limit;
     }
     c->cap_groups = g;
     c->cap_hidden = h;
@@ -349,6 +350,13 @@ extern "C" int fm_kernel_timing(fm_ctx *c, int enable) {
     c->ktiming = enable < 0 ? 0 : (enable > 2 ? 2 : enable);
     c->k1_ms = c->k2_ms = 0.0;
     c->kcalls = 0;
+    return FM_OK;
+}
+
+extern "C" int fm_set_wait_limit(fm_ctx *c, unsigned int polls) {
+    if (!c) return FM_ERR_ARG;
+    c->wait_limit = polls;
+    c->dflags.spin_limit = polls;
     return FM_OK;
 }
 

@@ -94,6 +94,12 @@ FM_API int fm_timer_stop(fm_ctx *ctx, float *elapsed_ms);   /* waits for the sto
  * runs only (the reference's --timing accumulators, finchmoe/infer.m:281-298, play
  * this role). */
 FM_API int fm_kernel_timing(fm_ctx *ctx, int mode);
+/* Bound of the waits inside the fused decode kernel (a workgroup waiting for a
+ * vector another workgroup produces), in polls of about a microsecond; default
+ * 1 << 20.  A wait that runs out does not hang: the kernel goes on, and the next
+ * fm_sync / host-pointer call returns FM_ERR_HIP ("results are invalid").  No
+ * counterpart in the reference (its kernels are separate Metal dispatches). */
+FM_API int fm_set_wait_limit(fm_ctx *ctx, unsigned int polls);
 /* sums in milliseconds since the last read, and the number of calls; resets */
 FM_API int fm_kernel_timing_read(fm_ctx *ctx, double *gate_up_ms, double *down_ms, int *calls);
 

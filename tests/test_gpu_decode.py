@@ -139,6 +139,72 @@ def test_decode_step_batched_layers(hip, orc, store3):
         assert_parity(deo[l].cpu().numpy(), ref_eo, "expert_out layer %d" % l)
 
 
+def _step_inputs(orc, seed, L, K):
+    import torch
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((L, H)).astype(np.float32)
+    idx = np.stack([_route(orc, rng, 12, K)[0] for _ in range(L)])
+    w = np.stack([orc.normalize_weights(rng.random(K).astype(np.float32)) for _ in range(L)])
+    return x, idx, w, tuple(torch.from_numpy(a).cuda() for a in (x, idx, w))
+
+
+def test_fused_launch_equals_separate_kernels(hip, orc, store3):
+    """One fused launch (default) == the phases as three kernels (timing mode 2), bitwise,
+    also with the guard flag and with repeated launches (the two counter sets alternate)."""
+    import torch
+    L, K = 4, 8
+    x, idx, w, (dx, di, dw) = _step_inputs(orc, 21, L, K)
+    outs = {}
+    for flags in (0, fb.GUARD):
+        for mode in (0, 2, 0, 0):
+            dout = torch.zeros(L, H, device="cuda")
+            deo = torch.zeros(L, K, H, device="cuda")
+            torch.cuda.synchronize()
+            hip.kernel_timing(mode)
+            hip.moe_decode_step_dev(0, L, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K,
+                                    dout.data_ptr(), deo.data_ptr(), flags)
+            hip.sync()
+            hip.kernel_timing(0)
+            got = (dout.cpu().numpy(), deo.cpu().numpy())
+            if flags in outs:
+                assert np.array_equal(got[0], outs[flags][0]), (flags, mode)
+                assert np.array_equal(got[1], outs[flags][1]), (flags, mode)
+            outs[flags] = got
+    ref, _ = orc.moe_experts_forward(store3[1], x[1], idx[1], w[1], H, I, 3)
+    assert_parity(outs[0][0][1], ref, "fused layer 1")
+
+
+def test_wait_limit_reports_instead_of_hanging(hip, orc, store3):
+    """With a wait limit of zero polls the fused kernel cannot wait for other workgroups:
+    it must still finish, the next sync must report the failure, and the context must work
+    again afterwards."""
+    import torch
+    L, K = 4, 8
+    x, idx, w, (dx, di, dw) = _step_inputs(orc, 22, L, K)
+    dout = torch.zeros(L, H, device="cuda")
+    torch.cuda.synchronize()
+    hip.set_wait_limit(0)
+    try:
+        failed = 0
+        for _ in range(20):    # a single launch can get through when every producer is early
+            hip.moe_decode_step_dev(0, L, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K,
+                                    dout.data_ptr())
+            try:
+                hip.sync()
+            except fb.FinchError as e:
+                assert e.status == fb.ERR_HIP and "invalid" in str(e)
+                failed += 1
+        assert failed > 0
+    finally:
+        hip.set_wait_limit(1 << 20)
+    hip.moe_decode_step_dev(0, L, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K, dout.data_ptr())
+    hip.sync()
+    out = dout.cpu().numpy()
+    for l in range(L):
+        ref, _ = orc.moe_experts_forward(store3[l], x[l], idx[l], w[l], H, I, 3)
+        assert_parity(out[l], ref, "after recovery, layer %d" % l)
+
+
 @pytest.mark.parametrize("bits,dtype", [(4, "bf16"), (3, "fp16"), (4, "fp16")])
 def test_other_formats(orc, bits, dtype):
     """4-bit experts and the fp16-scale variant of the benchmark text."""
