@@ -169,52 +169,6 @@ __global__ __launch_bounds__(256) void fm_combine(DecodeArgs a) {
     fm_combine_rows<GUARD>(a, blockIdx.x, j0, j1, red);
 }
 
-// ---------------------------------------------------------------- kernel 2
-template <int BITS, int LPR, bool FP16>
-__global__ __launch_bounds__(256) void fm_down(DecodeArgs a) {
-    constexpr int RPS = FM_WAVE / LPR;
-    constexpr int BPL = FmLaneBytes<BITS>::value;
-    const int item = blockIdx.x;
-    const int pair = item / a.items_per_pair;
-    const int chunk = item - pair * a.items_per_pair;
-    const int l = pair / a.K;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int c = lane % LPR, r = lane / LPR;
-    const int rows_per_wave = a.rows_per_item >> 2;
-    const int row0 = chunk * a.rows_per_item + wave * rows_per_wave;
-    float *eo = a.expert_out + (size_t)pair * a.g.hidden;
-
-    const int e = a.idx[pair];
-    if ((unsigned)e >= (unsigned)a.g.n_experts) {
-        for (int i = lane; i < rows_per_wave; i += FM_WAVE) eo[row0 + i] = 0.0f;
-    } else {
-        const uint8_t *blob = a.layer_ptrs[a.layer0 + l * a.layer_stride] + (size_t)e * a.g.expert_size;
-        const int row_bytes = a.g.inter * BITS / 8;
-        const int sb_row_bytes = (a.g.inter / 64) * 2;
-        size_t woff = (size_t)(row0 + r) * row_bytes + (size_t)c * BPL;
-        size_t soff = (size_t)(row0 + r) * sb_row_bytes + (size_t)c * 4;
-        const size_t wstep = (size_t)RPS * row_bytes, sstep = (size_t)RPS * sb_row_bytes;
-        FmRowSlice<BITS> cur, next;
-        fm_load_slice<BITS>(cur, blob + a.g.down_w + woff, blob + a.g.down_s + soff,
-                            blob + a.g.down_b + soff);
-        float xs[FM_CPL], xsum0, xsum1;
-        fm_load_x<BITS>(a.act + (size_t)pair * a.g.inter + c * FM_CPL, xs, xsum0, xsum1);
-        const int steps = rows_per_wave / RPS;
-        for (int it = 0; it < steps; it++) {
-            if (it + 1 < steps) {
-                woff += wstep;
-                soff += sstep;
-                fm_load_slice<BITS>(next, blob + a.g.down_w + woff, blob + a.g.down_s + soff,
-                                    blob + a.g.down_b + soff);
-            }
-            float v = fm_group_sum<LPR>(fm_lane_dot<BITS, FP16>(cur, xs, xsum0, xsum1));
-            if (c == 0) eo[row0 + it * RPS + r] = v;
-            cur = next;
-        }
-    }
-
-}
-
 // ======================================================================
 // Matrix-core path (fm_mfma.h): persistent workgroups over a static partition,
 // weight ring in LDS.
@@ -271,12 +225,6 @@ __device__ __forceinline__ void fm_unit_lane_offsets(int lane, int row_bytes, in
     row_in_step = 4 * rq + j;
     woff = (uint32_t)(row_in_step * row_bytes + ch * FmLaneBytes<BITS>::value);
     soff = (uint32_t)(row_in_step * sb_row_bytes + ch * 4);
-}
-
-__device__ __forceinline__ const uint8_t *fm_pair_blob(const DecodeArgs &a, int p) {
-    int e = a.idx[p];
-    if ((unsigned)e >= (unsigned)a.g.n_experts) return nullptr;   // treated as weight 0
-    return a.layer_ptrs[a.layer0 + (p / a.K) * a.layer_stride] + (size_t)e * a.g.expert_size;
 }
 
 // A pointer every lane of the wave agrees on, moved to scalar registers.
@@ -925,7 +873,7 @@ int launch_fused(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st, con
 }
 
 template <int BITS, bool FP16>
-int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down, int n_cu,
+int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int n_cu,
                     hipStream_t st, hipEvent_t *kev, const FmFlags *fl, bool *fused) {
     dim3 b(256);
     const int lpr_up = a.g.hidden / FM_CPL, lpr_down = a.g.inter / FM_CPL;
@@ -974,7 +922,6 @@ int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int rpi_down, 
     } else {
         return FM_ERR_UNSUPPORTED;
     }
-    (void)rpi_down;
     if (kev) (void)hipEventRecord(kev[1], st);
     {
         const long units = (long)n_pairs * (a.g.hidden / (FM_WAVE / lpr_down));
@@ -1049,7 +996,6 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     if (g->inter % min_up || g->hidden % min_down) return FM_ERR_UNSUPPORTED;
     const int want = 4 * n_cu;
     const int rpi_up = pick_rows_per_item(g->inter, n_pairs, min_up, 64, want);
-    const int rpi_down = pick_rows_per_item(g->hidden, n_pairs, min_down, 256, want);
     // with dependency counters (and room in them) the operator is one launch,
     // otherwise the phases run as separate kernels
     const unsigned int need = (unsigned int)(n_pairs + n_layers);
@@ -1064,7 +1010,7 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
         flp = &fl;
     }
     bool fused = false;
-#define FM_DEC(B, F) launch_decode_t<B, F>(a, n_pairs, rpi_up, rpi_down, n_cu, st, kev, flp, &fused)
+#define FM_DEC(B, F) launch_decode_t<B, F>(a, n_pairs, rpi_up, n_cu, st, kev, flp, &fused)
     int rc = FM_ERR_UNSUPPORTED;
     if (g->bits == 3) rc = g->scale_fp16 ? FM_DEC(3, true) : FM_DEC(3, false);
     else if (g->bits == 4) rc = g->scale_fp16 ? FM_DEC(4, true) : FM_DEC(4, false);

@@ -111,9 +111,11 @@ extern "C" int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, 
     const int min_rows = 4 * (FM_WAVE / lpr);
     long total_rows = 0;
     for (int i = 0; i < n; i++) total_rows += specs[i].out_dim;
-    // as many rows per workgroup as still leaves >= 4 workgroups per CU
+    // Rows per workgroup: the register budget keeps two workgroups per CU resident, and a
+    // launch that needs a second round of workgroups pays its start-up latencies twice —
+    // so grow the tile until the launch fits in one round (or the tile is 8 steps deep).
     int rpi = min_rows;
-    while (rpi * 2 <= 8 * min_rows && (total_rows * M) / (rpi * 2) >= 4L * n_cu) rpi *= 2;
+    while (rpi * 2 <= 8 * min_rows && (total_rows * M + rpi - 1) / rpi > 2L * n_cu) rpi *= 2;
     FmDenseArgs a;
     a.n = n;
     a.in_dim = in_dim;
