@@ -173,75 +173,152 @@ __device__ void pf_stage(PfLds<NG> &L, int count, RowFn xrow) {
     }
 }
 
-// One (row tile of 32 weight rows) x (all groups) pass.  Returns in acc the 16
-// results of the lane's weight row: register i = M row 8*(i/4) + 4*h + i%4.
-//   wrow  : the lane's weight row (packed codes), srow/brow: its scales/biases
+// A wave's share of an item is a sequence of passes; a pass = PF_R tiles of 32
+// weight rows x all groups, in NG/2 iterations of two groups.  The tiles of a
+// pass share every activation operand read from LDS (the gate tile and the up
+// tile of the same rows; two row tiles of down): the LDS pipe, not the matrix
+// core, was the busiest unit with one tile per read, and the independent MFMA
+// chains of the tiles fill each other's latency.  The passes run as ONE
+// software pipeline: the loads of iteration s + DEPTH are issued while
+// iteration s is multiplied, across pass boundaries — with the loads only one
+// iteration ahead every iteration exposed a full memory latency.
+//
+// Results of a pass, per tile: acc register i = M row 8*(i/4) + 4*h + i%4 of the
+// lane's weight row (rows 0..15 the hi pieces of the positions, 16..31 the lo pieces).
+//   ptrs(p, r, wrow, srow, brow): tile r of pass p: the lane's weight row, its scales, biases
+//   done(p, acc[PF_R])          : called after the last iteration of pass p
+#define PF_R 2
+
+typedef uint32_t pf_u3 __attribute__((ext_vector_type(3)));
+
+struct PfLoad {          // one iteration of one tile: the lane's halves of two groups + two scales
+    pf_u3 c0, c1;
+    uint32_t s;
+};
+
 template <int NG>
-__device__ __forceinline__ void pf_tile_pass(const PfLds<NG> &L, gptr wrow, gptr srow, gptr brow,
-                                             int lane, uint32_t ones, f16v &acc) {
-    const int h = lane >> 5;
+struct PfSide {          // scales and biases of the lane's k slots of the group-index products
+    static constexpr int NM2 = (NG + 15) / 16;
+    fm_u4 sv[NM2], bv[NM2];
+};
+
+template <int NG, int PF_DEPTH, class PtrFn, class DoneFn>
+__device__ __forceinline__ void pf_passes(const PfLds<NG> &L, int n_pass, int lane, uint32_t ones,
+                                          PtrFn ptrs, DoneFn done) {
+    constexpr int NI = NG / 2, NM2 = PfSide<NG>::NM2;
+    static_assert(NI >= PF_DEPTH, "one pending side load at most");
     typedef const __attribute__((address_space(1))) fm_u4 *gq_t;
-    typedef const __attribute__((address_space(1))) uint16_t *gh_t;
+    typedef const __attribute__((address_space(1))) pf_u3 *g3_t;
+    typedef const __attribute__((address_space(1))) uint32_t *gd_t;
+    const int h = lane >> 5;
+    const int S = n_pass * NI;
+    auto load = [&](int s, PfLoad *b) {
+        const int p = s / NI, g2 = s - p * NI;
 #pragma unroll
-    for (int i = 0; i < 16; i++) acc[i] = 0.0f;
-    // bias and offset products over the group index: k slot i of step m2 = group 16*m2 + 8*h + i
-    constexpr int NM2 = (NG + 15) / 16;
-#pragma unroll
-    for (int m2 = 0; m2 < NM2; m2++) {
-        fm_u4 sv = {0, 0, 0, 0}, bv = {0, 0, 0, 0};
-        if (16 * m2 + 8 * h < NG) {
-            sv = *(gq_t)(srow + 2 * (16 * m2 + 8 * h));
-            bv = *(gq_t)(brow + 2 * (16 * m2 + 8 * h));
+        for (int r = 0; r < PF_R; r++) {
+            gptr w, sr, br;
+            ptrs(p, r, w, sr, br);
+            b[r].c0 = *(g3_t)(w + 12 * h + 48 * g2);
+            b[r].c1 = *(g3_t)(w + 12 * h + 48 * g2 + 24);
+            b[r].s = *(gd_t)(sr + 4 * g2);
         }
-        bf8 sb = __builtin_bit_cast(bf8, sv), bb = __builtin_bit_cast(bf8, bv);
+    };
+    auto load_side = [&](int p, PfSide<NG> *sd) {
 #pragma unroll
-        for (int piece = 0; piece < 3; piece++) {
-            bf8 a0 = __builtin_bit_cast(bf8, L.side[(((0 * 3 + piece) * 2 + m2) * 2) * 32 + lane]);
-            bf8 a1 = __builtin_bit_cast(bf8, L.side[(((1 * 3 + piece) * 2 + m2) * 2) * 32 + lane]);
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, bb, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, sb, acc, 0, 0, 0);
-        }
-    }
-    // main product, two groups per iteration; the lane reads its own half (12 bytes) of each
-    typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
-    typedef const __attribute__((address_space(1))) u32x3 *g3_t;
-    gptr wmine = wrow + 12 * h;
-    u32x3 cur0, cur1, nxt0, nxt1;
-    uint32_t scur, snxt;
-    cur0 = *(g3_t)wmine;
-    cur1 = *(g3_t)(wmine + 24);
-    scur = *(const __attribute__((address_space(1))) uint32_t *)srow;
-    for (int g2 = 0; g2 < NG / 2; g2++) {
-        if (g2 + 1 < NG / 2) {
-            nxt0 = *(g3_t)(wmine + 48 * (g2 + 1));
-            nxt1 = *(g3_t)(wmine + 48 * (g2 + 1) + 24);
-            snxt = *(const __attribute__((address_space(1))) uint32_t *)(srow + 4 * (g2 + 1));
-        }
+        for (int r = 0; r < PF_R; r++) {
+            gptr w, sr, br;
+            ptrs(p, r, w, sr, br);
 #pragma unroll
-        for (int gg = 0; gg < 2; gg++) {
-            uint32_t my[3];
-            my[0] = gg ? cur1.x : cur0.x;
-            my[1] = gg ? cur1.y : cur0.y;
-            my[2] = gg ? cur1.z : cur0.z;
-            uint32_t v[16];
-            pf_unpack<0>(my, ones, v);
-            f16v dg;
-#pragma unroll
-            for (int i = 0; i < 16; i++) dg[i] = 0.0f;
-            const int g = 2 * g2 + gg;
-#pragma unroll
-            for (int s = 0; s < 4; s++) {
-                bf8 a = __builtin_bit_cast(bf8, L.act[(g * 4 + s) * 64 + lane]);
-                bf8 b = __builtin_bit_cast(bf8, make_uint4(v[4 * s], v[4 * s + 1], v[4 * s + 2], v[4 * s + 3]));
-                dg = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, dg, 0, 0, 0);
+            for (int m2 = 0; m2 < NM2; m2++) {
+                sd[r].sv[m2] = fm_u4{0, 0, 0, 0};
+                sd[r].bv[m2] = fm_u4{0, 0, 0, 0};
+                if (16 * m2 + 8 * h < NG) {
+                    sd[r].sv[m2] = *(gq_t)(sr + 2 * (16 * m2 + 8 * h));
+                    sd[r].bv[m2] = *(gq_t)(br + 2 * (16 * m2 + 8 * h));
+                }
             }
-            const float sc = gg ? fm_bf16_hi(scur) : fm_bf16_lo(scur);
-#pragma unroll
-            for (int i = 0; i < 16; i++) acc[i] = fmaf(sc, dg[i], acc[i]);
         }
-        cur0 = nxt0;
-        cur1 = nxt1;
-        scur = snxt;
+    };
+    PfLoad buf[PF_DEPTH][PF_R];
+    PfSide<NG> side[PF_R];
+    if (S > 0) load_side(0, side);
+#pragma unroll
+    for (int j = 0; j < PF_DEPTH; j++)
+        if (j < S) load(j, buf[j]);
+    f16v acc[PF_R];
+    for (int s0 = 0; s0 < S; s0 += PF_DEPTH) {
+#pragma unroll
+        for (int j = 0; j < PF_DEPTH; j++) {
+            const int s = s0 + j;
+            if (s < S) {
+                const int p = s / NI, g2 = s - p * NI;
+                if (g2 == 0) {
+                    // bias and offset products over the group index: k slot i of step m2 =
+                    // group 16*m2 + 8*h + i
+#pragma unroll
+                    for (int r = 0; r < PF_R; r++)
+#pragma unroll
+                        for (int i = 0; i < 16; i++) acc[r][i] = 0.0f;
+#pragma unroll
+                    for (int m2 = 0; m2 < NM2; m2++) {
+#pragma unroll
+                        for (int piece = 0; piece < 3; piece++) {
+                            bf8 a0 = __builtin_bit_cast(
+                                bf8, L.side[(((0 * 3 + piece) * 2 + m2) * 2) * 32 + lane]);
+                            bf8 a1 = __builtin_bit_cast(
+                                bf8, L.side[(((1 * 3 + piece) * 2 + m2) * 2) * 32 + lane]);
+#pragma unroll
+                            for (int r = 0; r < PF_R; r++) {
+                                bf8 sb = __builtin_bit_cast(bf8, side[r].sv[m2]);
+                                bf8 bb = __builtin_bit_cast(bf8, side[r].bv[m2]);
+                                acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, bb, acc[r], 0, 0, 0);
+                                acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, sb, acc[r], 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+                PfLoad cur[PF_R];
+#pragma unroll
+                for (int r = 0; r < PF_R; r++) cur[r] = buf[j][r];
+                if (s + PF_DEPTH < S) load(s + PF_DEPTH, buf[j]);
+                // the side operands of the next pass, once its first loads are on their way
+                if (g2 == NI - PF_DEPTH && p + 1 < n_pass) load_side(p + 1, side);
+#pragma unroll
+                for (int gg = 0; gg < 2; gg++) {
+                    const int g = 2 * g2 + gg;
+                    uint32_t v[PF_R][16];
+                    f16v dg[PF_R];
+#pragma unroll
+                    for (int r = 0; r < PF_R; r++) {
+                        uint32_t my[3];
+                        my[0] = gg ? cur[r].c1.x : cur[r].c0.x;
+                        my[1] = gg ? cur[r].c1.y : cur[r].c0.y;
+                        my[2] = gg ? cur[r].c1.z : cur[r].c0.z;
+                        pf_unpack<0>(my, ones, v[r]);
+#pragma unroll
+                        for (int i = 0; i < 16; i++) dg[r][i] = 0.0f;
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        bf8 a = __builtin_bit_cast(bf8, L.act[(g * 4 + k) * 64 + lane]);
+#pragma unroll
+                        for (int r = 0; r < PF_R; r++) {
+                            bf8 b = __builtin_bit_cast(
+                                bf8, make_uint4(v[r][4 * k], v[r][4 * k + 1], v[r][4 * k + 2],
+                                                v[r][4 * k + 3]));
+                            dg[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, dg[r], 0, 0, 0);
+                        }
+                    }
+#pragma unroll
+                    for (int r = 0; r < PF_R; r++) {
+                        const float sc = gg ? fm_bf16_hi(cur[r].s) : fm_bf16_lo(cur[r].s);
+#pragma unroll
+                        for (int i = 0; i < 16; i++) acc[r][i] = fmaf(sc, dg[r][i], acc[r][i]);
+                    }
+                }
+                if (g2 == NI - 1) done(p, acc);
+            }
+        }
     }
 }
 
@@ -307,24 +384,28 @@ __global__ __launch_bounds__(512) void fm_pf_gate_up(PfArgs a) {
         __syncthreads();
         const uint8_t *blob = a.layer + (size_t)item.expert * a.g.expert_size;
         const int n = lane & 31, h = lane >> 5;
-        for (int rt = wave; rt < a.g.inter / 32; rt += blockDim.x / 64) {
-            const int row = rt * 32 + n;
-            f16v accg, accu;
-            pf_tile_pass<NG>(L, (gptr)(uintptr_t)(blob + a.g.gate_w + (size_t)row * row_bytes),
-                             (gptr)(uintptr_t)(blob + a.g.gate_s + (size_t)row * sb_bytes),
-                             (gptr)(uintptr_t)(blob + a.g.gate_b + (size_t)row * sb_bytes), lane, ones, accg);
-            pf_tile_pass<NG>(L, (gptr)(uintptr_t)(blob + a.g.up_w + (size_t)row * row_bytes),
-                             (gptr)(uintptr_t)(blob + a.g.up_s + (size_t)row * sb_bytes),
-                             (gptr)(uintptr_t)(blob + a.g.up_b + (size_t)row * sb_bytes), lane, ones, accu);
+        const int NW = blockDim.x / 64;
+        // pass p: row tile wave + NW*p, gate and up rows together
+        const int n_tiles = (a.g.inter / 32 - wave + NW - 1) / NW;
+        pf_passes<NG, 4>(
+            L, n_tiles, lane, ones,
+            [&](int p, int r, gptr &w, gptr &sr, gptr &br) {
+                const int row = (wave + NW * p) * 32 + n;
+                w = (gptr)(uintptr_t)(blob + (r ? a.g.up_w : a.g.gate_w) + (size_t)row * row_bytes);
+                sr = (gptr)(uintptr_t)(blob + (r ? a.g.up_s : a.g.gate_s) + (size_t)row * sb_bytes);
+                br = (gptr)(uintptr_t)(blob + (r ? a.g.up_b : a.g.gate_b) + (size_t)row * sb_bytes);
+            },
+            [&](int p, const f16v *acc) {
+                const int row = (wave + NW * p) * 32 + n;
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int tok = 8 * (i / 4) + 4 * h + (i % 4);   // M row of register i (hi piece)
-                if (tok < item.count) {
-                    float gv = accg[i] + accg[i + 8], uv = accu[i] + accu[i + 8];
-                    a.act[(size_t)(item.start + tok) * a.g.inter + row] = fm_silu_mul(gv, uv);
+                for (int i = 0; i < 8; i++) {
+                    const int tok = 8 * (i / 4) + 4 * h + (i % 4);   // M row of register i (hi piece)
+                    if (tok < item.count) {
+                        float gv = acc[0][i] + acc[0][i + 8], uv = acc[1][i] + acc[1][i + 8];
+                        a.act[(size_t)(item.start + tok) * a.g.inter + row] = fm_silu_mul(gv, uv);
+                    }
                 }
-            }
-        }
+            });
     }
 }
 
@@ -344,21 +425,31 @@ __global__ __launch_bounds__(512) void fm_pf_down(PfArgs a) {
         __syncthreads();
         const uint8_t *blob = a.layer + (size_t)item.expert * a.g.expert_size;
         const int n = lane & 31, h = lane >> 5;
-        for (int rt = wave; rt < a.g.hidden / 32; rt += blockDim.x / 64) {
-            const int row = rt * 32 + n;
-            f16v acc;
-            pf_tile_pass<NG>(L, (gptr)(uintptr_t)(blob + a.g.down_w + (size_t)row * row_bytes),
-                             (gptr)(uintptr_t)(blob + a.g.down_s + (size_t)row * sb_bytes),
-                             (gptr)(uintptr_t)(blob + a.g.down_b + (size_t)row * sb_bytes), lane, ones, acc);
+        const int NW = blockDim.x / 64;
+        // pass p: row tiles wave + NW*(2p) and wave + NW*(2p+1) (hidden is a multiple of 64*NW)
+        const int n_tiles = (a.g.hidden / 32 - wave + NW - 1) / NW;
+        pf_passes<NG, 4>(
+            L, n_tiles / 2, lane, ones,
+            [&](int p, int r, gptr &w, gptr &sr, gptr &br) {
+                const int row = (wave + NW * (2 * p + r)) * 32 + n;
+                w = (gptr)(uintptr_t)(blob + a.g.down_w + (size_t)row * row_bytes);
+                sr = (gptr)(uintptr_t)(blob + a.g.down_s + (size_t)row * sb_bytes);
+                br = (gptr)(uintptr_t)(blob + a.g.down_b + (size_t)row * sb_bytes);
+            },
+            [&](int p, const f16v *acc) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int tok = 8 * (i / 4) + 4 * h + (i % 4);
-                if (tok < item.count) {
-                    const int pair = a.sorted[item.start + tok];
-                    a.eo[(size_t)pair * a.g.hidden + row] = acc[i] + acc[i + 8];
+                for (int r = 0; r < PF_R; r++) {
+                    const int row = (wave + NW * (2 * p + r)) * 32 + n;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const int tok = 8 * (i / 4) + 4 * h + (i % 4);
+                        if (tok < item.count) {
+                            const int pair = a.sorted[item.start + tok];
+                            a.eo[(size_t)pair * a.g.hidden + row] = acc[r][i] + acc[r][i + 8];
+                        }
+                    }
                 }
-            }
-        }
+            });
     }
 }
 
