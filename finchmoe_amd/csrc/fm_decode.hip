@@ -16,6 +16,7 @@
 // The scales (and biases) of those rows are contiguous too — [rows][groups]
 // 16-bit, two groups per lane = one dword per lane.
 #include "fm_mfma.h"
+#include "fm_ring.h"
 
 #include <type_traits>
 
@@ -212,9 +213,6 @@ struct FmDma {
     static constexpr int WG_BYTES = FM_NW * RING * BYTES;
 };
 
-typedef const __attribute__((address_space(1))) void *fm_gptr;
-typedef __attribute__((address_space(3))) void *fm_lptr;
-
 template <int BITS, int LPR>
 __device__ __forceinline__ void fm_unit_lane_offsets(int lane, int row_bytes, int sb_row_bytes,
                                                      uint32_t &woff, uint32_t &soff,
@@ -225,14 +223,6 @@ __device__ __forceinline__ void fm_unit_lane_offsets(int lane, int row_bytes, in
     row_in_step = 4 * rq + j;
     woff = (uint32_t)(row_in_step * row_bytes + ch * FmLaneBytes<BITS>::value);
     soff = (uint32_t)(row_in_step * sb_row_bytes + ch * 4);
-}
-
-// A pointer every lane of the wave agrees on, moved to scalar registers.
-__device__ __forceinline__ const uint8_t *fm_uniform(const uint8_t *p) {
-    uintptr_t v = (uintptr_t)p;
-    uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-    uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return (const uint8_t *)(((uintptr_t)hi << 32) | lo);
 }
 
 template <int BITS, int I>
@@ -253,12 +243,6 @@ __device__ __forceinline__ void fm_dma_issue(uint32_t slot, const uint8_t *w, co
                                      (fm_lptr)(uintptr_t)(slot + FmDma<BITS>::WBYTES), 4, 0, 0);
     __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(b + lane * 4),
                                      (fm_lptr)(uintptr_t)(slot + FmDma<BITS>::WBYTES + 256), 4, 0, 0);
-}
-
-template <int N>
-__device__ __forceinline__ void fm_dma_wait(bool drain) {
-    if (drain) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
 // this lane's codes and scale/bias words out of a landed slot

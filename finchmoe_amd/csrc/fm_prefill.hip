@@ -30,6 +30,7 @@
 // items round-robin; per item it builds the activation operand image in LDS
 // (128 KB for 2048 columns) and its eight waves sweep the row tiles.
 #include "fm_mfma.h"
+#include "fm_ring.h"
 
 namespace {
 
@@ -453,6 +454,382 @@ __global__ __launch_bounds__(512) void fm_pf_down(PfArgs a) {
     }
 }
 
+// ======================================================================
+// K-slab kernels.
+//
+// The kernels above keep the whole activation operand of an item in LDS
+// (128 KB) and let every wave sweep row tiles over the full K; their weight
+// loads are per-lane 12-byte pieces of 32 different rows, and the address
+// unit, not the matrix core, is the busiest part of the CU.  Here the K
+// dimension is split over the eight waves of the workgroup instead: wave w
+// owns groups [GPW*w, GPW*(w+1)) of every row.
+//   * Its share of the activation operand is 16 registers per group: it is
+//     built straight from global memory into registers, once per item; LDS
+//     holds no activations.
+//   * Every wave visits every row tile.  A tile-matrix (32 rows of one matrix)
+//     x slab is 32 runs of 24*GPW bytes: the wave copies them, with the rows'
+//     scales and biases, into a ring slot with LDS-direct loads (whole runs,
+//     several slots in flight), and every lane reads its 12-byte pieces back.
+//   * Bias and offset terms ride in one or two extra MFMAs per tile-matrix
+//     whose K slots are (piece, group) of the wave's own groups.
+//   * The eight partial tiles are summed through LDS in wave order (wave r sums
+//     result register r of every lane), SwiGLU / store happen there.  One
+//     barrier per step (two tile-matrices), two partial buffers.
+// ======================================================================
+template <int GPW>
+struct PfSlab {
+    static constexpr int NG = 8 * GPW;                  // groups of a whole row
+    static constexpr int CB = 24 * GPW;                 // code bytes of a row inside the slab
+    static constexpr int CODE_BYTES = 32 * CB;          // 3072 / 768
+    static constexpr int PS = GPW == 4 ? 16 : 4;        // bytes a lane copies per load (24 B runs: dwords)
+    static constexpr int RP = CB / PS;                  // pieces per row: 6
+    // GPW = 4: a row takes 7 piece slots in LDS (the 7th stays empty): with 96-byte rows the
+    // 128-bit reads of eight neighbouring rows hit the same banks twice over
+    static constexpr int RS = GPW == 4 ? RP + 1 : RP;   // piece slots per row in LDS
+    static constexpr int PIECES = 32 * RS;              // piece slots of a tile-matrix: 224 / 192
+    static constexpr int NQ = (PIECES + 63) / 64;       // LDS-direct loads for the codes
+    static constexpr int LDS_CODE = PIECES * PS;        // 3584 / 768
+    static constexpr int SLOT = LDS_CODE + 512;         // + scales 256 + biases 256
+    static constexpr int LOADS = NQ + 2;
+    static constexpr int RING = 3;
+    static constexpr int NSIDE = GPW == 4 ? 2 : 1;      // MFMAs for the bias/offset terms
+    static constexpr int RED_BYTES = 2 * 2 * 8 * 8 * 64 * 4;   // [buffer][matrix][wave][reg][lane]
+    static constexpr int LDS_BYTES = 8 * RING * SLOT + RED_BYTES;
+};
+
+// three bf16 pieces (bit patterns) of v, the last one truncated
+__device__ __forceinline__ void pf_pieces(float v, uint32_t *pc) {
+    uint32_t b = __float_as_uint(v) & 0xFFFF0000u;
+    pc[0] = b >> 16;
+    v -= __uint_as_float(b);
+    b = __float_as_uint(v) & 0xFFFF0000u;
+    pc[1] = b >> 16;
+    v -= __uint_as_float(b);
+    pc[2] = __float_as_uint(v) >> 16;
+}
+
+// the operand registers of k steps S.. of one group for this lane: the hi pieces
+// (take_hi) or the lo pieces of its 32 activations
+template <int S>
+__device__ __forceinline__ void pf_stage_group(const float *x, bool take_hi, uint4 *A, float &xs,
+                                               float &xo) {
+    if constexpr (S < 4) {
+        uint32_t hi[4], lo[4];
+        pf_stage_pair<S, 0>(x, hi, lo, xs, xo);
+        pf_stage_pair<S, 1>(x, hi, lo, xs, xo);
+        pf_stage_pair<S, 2>(x, hi, lo, xs, xo);
+        pf_stage_pair<S, 3>(x, hi, lo, xs, xo);
+        A[S] = take_hi ? make_uint4(hi[0], hi[1], hi[2], hi[3]) : make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        pf_stage_group<S + 1>(x, take_hi, A, xs, xo);
+    }
+}
+
+template <int GPW, bool GU>
+__global__ __launch_bounds__(512) void fm_pf_slab(PfArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)   // (the host pass cannot allocate the registers of the asm blocks)
+    using P = PfSlab<GPW>;
+    constexpr int RING = P::RING;
+    extern __shared__ __attribute__((aligned(16))) uint8_t pf2_smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = lane & 31, hh = lane >> 5;
+    const uint32_t lds0 = fm_lds_addr(pf2_smem);
+    const uint32_t ring0 = lds0 + (uint32_t)wave * (RING * P::SLOT);
+    const uint32_t red0 = lds0 + 8 * RING * P::SLOT;
+    const int n_items = *a.n_items;
+    const int in_dim = GU ? a.g.hidden : a.g.inter;
+    const int row_bytes = in_dim * 3 / 8, sb_bytes = (in_dim / 64) * 2;
+    const int n_steps = GU ? a.g.inter / 32 : a.g.hidden / 64;   // two tile-matrices per step
+    const uint32_t ones = fm_opaque(0x3F803F80u);
+    // region offsets of the two tile-matrices of a step and their row distance
+    const uint32_t w_off0 = GU ? a.g.gate_w : a.g.down_w, s_off0 = GU ? a.g.gate_s : a.g.down_s,
+                   b_off0 = GU ? a.g.gate_b : a.g.down_b;
+    const uint32_t w_d = GU ? a.g.up_w - a.g.gate_w : 32u * row_bytes;
+    const uint32_t s_d = GU ? a.g.up_s - a.g.gate_s : 32u * sb_bytes;
+    const uint32_t b_d = GU ? a.g.up_b - a.g.gate_b : 32u * sb_bytes;
+    const uint32_t step_rows = GU ? 32u : 64u;
+    // this lane's pieces of a slot copy
+    uint32_t coff[P::NQ];
+    bool cvalid[P::NQ];
+#pragma unroll
+    for (int j = 0; j < P::NQ; j++) {
+        const int q = 64 * j + lane;
+        const int row = q / P::RS, piece = q - row * P::RS;
+        cvalid[j] = q < P::PIECES && piece < P::RP;
+        coff[j] = (uint32_t)(row * row_bytes + P::CB * wave + P::PS * piece);
+    }
+    // scales / biases of the slab: 2*GPW bytes per row, fetched as whole dwords
+    const int sb_slab = (2 * GPW * wave) & ~3;
+    const bool svalid = GPW >= 2 ? true : lane < 32;
+    const uint32_t soff = GPW >= 2 ? (uint32_t)((lane >> 1) * sb_bytes + sb_slab + 4 * (lane & 1))
+                                   : (uint32_t)(lane * sb_bytes + sb_slab);
+
+    // ---- loader: tile-matrices of this workgroup's items, in order
+    int l_it = blockIdx.x, l_s = 0, l_mat = 0, wpos = 0;
+    uint32_t issued = 0, consumed = 0;
+    bool l_done = l_it >= n_items;
+    const uint8_t *l_blob = nullptr;
+    if (!l_done) l_blob = fm_uniform(a.layer + (size_t)a.items[l_it].expert * a.g.expert_size);
+    auto issue = [&]() __attribute__((always_inline)) {
+        if (l_done) return;
+        const uint32_t slot = ring0 + (uint32_t)wpos * P::SLOT;
+        const size_t row0 = (size_t)l_s * step_rows;
+        const uint8_t *wb = l_blob + w_off0 + (l_mat ? w_d : 0u) + row0 * row_bytes;
+        const uint8_t *sb = l_blob + s_off0 + (l_mat ? s_d : 0u) + row0 * sb_bytes;
+        const uint8_t *bb = l_blob + b_off0 + (l_mat ? b_d : 0u) + row0 * sb_bytes;
+#pragma unroll
+        for (int j = 0; j < P::NQ; j++)
+            if (cvalid[j])
+                __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(wb + coff[j]),
+                                                 (fm_lptr)(uintptr_t)(slot + 64 * P::PS * j),
+                                                 P::PS, 0, 0);
+        if (svalid) {
+            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(sb + soff),
+                                             (fm_lptr)(uintptr_t)(slot + P::LDS_CODE), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(bb + soff),
+                                             (fm_lptr)(uintptr_t)(slot + P::LDS_CODE + 256), 4, 0, 0);
+        }
+        wpos = wpos + 1 == RING ? 0 : wpos + 1;
+        issued++;
+        l_mat ^= 1;
+        if (l_mat == 0 && ++l_s == n_steps) {
+            l_s = 0;
+            l_it += gridDim.x;
+            if (l_it < n_items)
+                l_blob = fm_uniform(a.layer + (size_t)a.items[l_it].expert * a.g.expert_size);
+            else
+                l_done = true;
+        }
+    };
+#pragma unroll
+    for (int k = 0; k < RING; k++) issue();
+
+    int c = 0, buf = 0;
+    for (int it = blockIdx.x; it < n_items; it += gridDim.x) {
+        const PfItem item = a.items[it];
+        // ---- this wave's share of the activation operand, straight into registers:
+        // lane (m, hh): M row m = hi piece of position m (m < 16) or lo piece of position
+        // m - 16; k slots 8*hh .. 8*hh+7 of every k step = columns 32*hh .. 32*hh+31 of the group
+        uint4 A[GPW][4];
+        uint32_t sideA[P::NSIDE][4];
+        {
+            const int pos = n & 15;
+            const bool on = pos < item.count;
+            const float *xrow = nullptr;
+            if (on)
+                xrow = GU ? a.X + (size_t)(a.sorted[item.start + pos] / a.K) * a.g.hidden
+                          : a.act + (size_t)(item.start + pos) * a.g.inter;
+            float xs[GPW], xo[GPW];
+#pragma unroll
+            for (int gi = 0; gi < GPW; gi++) {
+                float x[32];
+                if (on) {
+                    const float4 *xp =
+                        reinterpret_cast<const float4 *>(xrow + 64 * (GPW * wave + gi) + 32 * hh);
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        float4 v = xp[i];
+                        x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 32; i++) x[i] = 0.0f;
+                }
+                float s0 = 0.0f, o0 = 0.0f;
+                pf_stage_group<0>(x, n < 16, A[gi], s0, o0);
+                // the two halves of a group sit in lanes 32 apart
+                xs[gi] = s0 + __shfl_xor(s0, 32);
+                xo[gi] = o0 + __shfl_xor(o0, 32);
+            }
+            // K slots of the bias/offset MFMAs.  GPW = 4: slot = 4*piece + group, one MFMA
+            // per term (xsum for the biases, -xoff for the scales).  GPW = 1: slot = 3*term +
+            // piece, one MFMA.  Rows 16..31 (lo pieces) take no part.
+            if constexpr (GPW == 4) {
+#pragma unroll
+                for (int term = 0; term < 2; term++) {
+                    uint32_t pc[4][3];
+#pragma unroll
+                    for (int gi = 0; gi < 4; gi++) pf_pieces(term ? -xo[gi] : xs[gi], pc[gi]);
+                    const int p0 = hh ? 2 : 0;
+                    sideA[term][0] = pc[0][p0] | (pc[1][p0] << 16);
+                    sideA[term][1] = pc[2][p0] | (pc[3][p0] << 16);
+                    sideA[term][2] = hh ? 0u : pc[0][1] | (pc[1][1] << 16);
+                    sideA[term][3] = hh ? 0u : pc[2][1] | (pc[3][1] << 16);
+                    if (n >= 16) sideA[term][0] = sideA[term][1] = sideA[term][2] = sideA[term][3] = 0u;
+                }
+            } else {
+                uint32_t ps[3], po[3];
+                pf_pieces(xs[0], ps);
+                pf_pieces(-xo[0], po);
+                const bool z = hh || n >= 16;
+                sideA[0][0] = z ? 0u : ps[0] | (ps[1] << 16);
+                sideA[0][1] = z ? 0u : ps[2] | (po[0] << 16);
+                sideA[0][2] = z ? 0u : po[1] | (po[2] << 16);
+                sideA[0][3] = 0u;
+            }
+        }
+        // output position of result register r = wave of this lane, and (down) its pair
+        const int my_pos = 8 * (wave >> 2) + 4 * hh + (wave & 3);
+        const bool my_on = my_pos < item.count;
+        int my_pair = 0;
+        if (!GU && my_on) my_pair = a.sorted[item.start + my_pos];
+
+        for (int s = 0; s < n_steps; s++) {
+#pragma unroll
+            for (int mat = 0; mat < 2; mat++) {
+                // The hardware issues the older of two waves on a SIMD first, which lets waves
+                // 0-3 run ahead and wait at every barrier for waves 4-7: take turns instead.
+                if (((wave >> 2) ^ mat) & 1) __builtin_amdgcn_s_setprio(1);
+                else __builtin_amdgcn_s_setprio(0);
+                // ---- the oldest slot of the ring
+                if (issued - consumed == (uint32_t)RING) fm_dma_wait<P::LOADS *(RING - 1)>(false);
+                else fm_dma_wait<0>(true);
+                const uint32_t slot = ring0 + (uint32_t)c * P::SLOT;
+                uint32_t cw[GPW][3], sw[2], bw[2];
+                if constexpr (GPW == 4) {
+                    // the whole 96-byte run of the row (both half lanes read the same
+                    // pieces), then this lane's half of every group
+                    const uint32_t ac = slot + (uint32_t)(n * (P::RS * 16));
+                    const uint32_t as = slot + P::LDS_CODE + 8 * n;
+                    fm_u4 r0, r1, r2, r3, r4, r5;
+                    asm volatile(
+                        "ds_read_b128 %0, %10\n\tds_read_b128 %1, %10 offset:16\n\t"
+                        "ds_read_b128 %2, %10 offset:32\n\tds_read_b128 %3, %10 offset:48\n\t"
+                        "ds_read_b128 %4, %10 offset:64\n\tds_read_b128 %5, %10 offset:80\n\t"
+                        "ds_read_b32 %6, %11\n\tds_read_b32 %7, %11 offset:4\n\t"
+                        "ds_read_b32 %8, %11 offset:256\n\tds_read_b32 %9, %11 offset:260\n\t"
+                        "s_waitcnt lgkmcnt(0)"
+                        : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(r4), "=&v"(r5),
+                          "=&v"(sw[0]), "=&v"(sw[1]), "=&v"(bw[0]), "=&v"(bw[1])
+                        : "v"(ac), "v"(as)
+                        : "memory");
+                    const uint32_t rd[24] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w,
+                                             r2.x, r2.y, r2.z, r2.w, r3.x, r3.y, r3.z, r3.w,
+                                             r4.x, r4.y, r4.z, r4.w, r5.x, r5.y, r5.z, r5.w};
+#pragma unroll
+                    for (int gi = 0; gi < 4; gi++)
+#pragma unroll
+                        for (int d = 0; d < 3; d++) cw[gi][d] = hh ? rd[6 * gi + 3 + d] : rd[6 * gi + d];
+                } else {
+                    const uint32_t ac = slot + (uint32_t)(n * P::CB + 12 * hh);
+                    const uint32_t as = slot + P::LDS_CODE + 4 * n;
+                    asm volatile("ds_read_b32 %0, %5\n\tds_read_b32 %1, %5 offset:4\n\t"
+                                 "ds_read_b32 %2, %5 offset:8\n\tds_read_b32 %3, %6\n\t"
+                                 "ds_read_b32 %4, %6 offset:256\n\ts_waitcnt lgkmcnt(0)"
+                                 : "=&v"(cw[0][0]), "=&v"(cw[0][1]), "=&v"(cw[0][2]), "=&v"(sw[0]),
+                                   "=&v"(bw[0])
+                                 : "v"(ac), "v"(as)
+                                 : "memory");
+                    // the slab's 16-bit scale / bias inside the dword that was fetched
+                    const int sh = 16 * (wave & 1);
+                    sw[0] = (sw[0] >> sh) & 0xFFFFu;
+                    bw[0] = (bw[0] >> sh) & 0xFFFFu;
+                    sw[1] = bw[1] = 0u;
+                }
+                consumed++;
+                c = c + 1 == RING ? 0 : c + 1;
+                issue();
+
+                // ---- bias and offset terms, then the groups of the slab
+                f16v acc;
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[i] = 0.0f;
+                if constexpr (GPW == 4) {
+                    const uint4 Bb = hh ? make_uint4(bw[0], bw[1], 0u, 0u) : make_uint4(bw[0], bw[1], bw[0], bw[1]);
+                    const uint4 Bs = hh ? make_uint4(sw[0], sw[1], 0u, 0u) : make_uint4(sw[0], sw[1], sw[0], sw[1]);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf8, make_uint4(sideA[0][0], sideA[0][1], sideA[0][2], sideA[0][3])),
+                        __builtin_bit_cast(bf8, Bb), acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf8, make_uint4(sideA[1][0], sideA[1][1], sideA[1][2], sideA[1][3])),
+                        __builtin_bit_cast(bf8, Bs), acc, 0, 0, 0);
+                } else {
+                    const uint32_t b = bw[0], sc16 = sw[0];
+                    const uint4 B1 = hh ? make_uint4(0u, 0u, 0u, 0u)
+                                        : make_uint4(b | (b << 16), b | (sc16 << 16), sc16 | (sc16 << 16), 0u);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf8, make_uint4(sideA[0][0], sideA[0][1], sideA[0][2], sideA[0][3])),
+                        __builtin_bit_cast(bf8, B1), acc, 0, 0, 0);
+                }
+#pragma unroll
+                for (int gi = 0; gi < GPW; gi++) {
+                    uint32_t v[16];
+                    pf_unpack<0>(cw[gi], ones, v);
+                    f16v dg;
+#pragma unroll
+                    for (int i = 0; i < 16; i++) dg[i] = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        bf8 bop = __builtin_bit_cast(
+                            bf8, make_uint4(v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3]));
+                        dg = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8, A[gi][k]),
+                                                                     bop, dg, 0, 0, 0);
+                    }
+                    float sc;
+                    if constexpr (GPW == 4) sc = (gi & 1) ? fm_bf16_hi(sw[gi >> 1]) : fm_bf16_lo(sw[gi >> 1]);
+                    else sc = fm_bf16_lo(sw[0]);
+#pragma unroll
+                    for (int i = 0; i < 16; i++) acc[i] = fmaf(sc, dg[i], acc[i]);
+                }
+                // ---- this wave's partial tile: hi + lo rows, register i of every lane
+                {
+                    const uint32_t aw = red0 + (uint32_t)(((buf * 2 + mat) * 8 + wave) * 2048 + 4 * lane);
+                    float o[8];
+#pragma unroll
+                    for (int i = 0; i < 8; i++) o[i] = acc[i] + acc[i + 8];
+                    asm volatile("ds_write_b32 %0, %1\n\tds_write_b32 %0, %2 offset:256\n\t"
+                                 "ds_write_b32 %0, %3 offset:512\n\tds_write_b32 %0, %4 offset:768\n\t"
+                                 "ds_write_b32 %0, %5 offset:1024\n\tds_write_b32 %0, %6 offset:1280\n\t"
+                                 "ds_write_b32 %0, %7 offset:1536\n\tds_write_b32 %0, %8 offset:1792"
+                                 :
+                                 : "v"(aw), "v"(o[0]), "v"(o[1]), "v"(o[2]), "v"(o[3]), "v"(o[4]),
+                                   "v"(o[5]), "v"(o[6]), "v"(o[7])
+                                 : "memory");
+                }
+            }
+            // ---- every wave has written both partial tiles of this step
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            {
+                // wave r sums result register r (position my_pos) over the waves, in wave order
+                const uint32_t ar = red0 + (uint32_t)((buf * 2 * 8) * 2048 + wave * 256 + 4 * lane);
+                float p[16];
+                asm volatile(
+                    "ds_read_b32 %0, %16\n\tds_read_b32 %1, %16 offset:2048\n\tds_read_b32 %2, %16 offset:4096\n\t"
+                    "ds_read_b32 %3, %16 offset:6144\n\tds_read_b32 %4, %16 offset:8192\n\tds_read_b32 %5, %16 offset:10240\n\t"
+                    "ds_read_b32 %6, %16 offset:12288\n\tds_read_b32 %7, %16 offset:14336\n\t"
+                    "ds_read_b32 %8, %16 offset:16384\n\tds_read_b32 %9, %16 offset:18432\n\tds_read_b32 %10, %16 offset:20480\n\t"
+                    "ds_read_b32 %11, %16 offset:22528\n\tds_read_b32 %12, %16 offset:24576\n\tds_read_b32 %13, %16 offset:26624\n\t"
+                    "ds_read_b32 %14, %16 offset:28672\n\tds_read_b32 %15, %16 offset:30720\n\t"
+                    "s_waitcnt lgkmcnt(0)"
+                    : "=&v"(p[0]), "=&v"(p[1]), "=&v"(p[2]), "=&v"(p[3]), "=&v"(p[4]), "=&v"(p[5]),
+                      "=&v"(p[6]), "=&v"(p[7]), "=&v"(p[8]), "=&v"(p[9]), "=&v"(p[10]), "=&v"(p[11]),
+                      "=&v"(p[12]), "=&v"(p[13]), "=&v"(p[14]), "=&v"(p[15])
+                    : "v"(ar)
+                    : "memory");
+                float t0 = p[0], t1 = p[8];
+#pragma unroll
+                for (int w2 = 1; w2 < 8; w2++) {
+                    t0 += p[w2];
+                    t1 += p[8 + w2];
+                }
+                if (my_on) {
+                    if constexpr (GU) {
+                        a.act[(size_t)(item.start + my_pos) * a.g.inter + 32 * s + n] = fm_silu_mul(t0, t1);
+                    } else {
+                        float *o = a.eo + (size_t)my_pair * a.g.hidden + 64 * s + n;
+                        o[0] = t0;
+                        o[32] = t1;
+                    }
+                }
+            }
+            buf ^= 1;
+        }
+    }
+#else
+    (void)a;
+#endif
+}
+
 // out[m][j] = sum_k w[m][k] * eo[m*K + k][j] in slot order (finchmoe/shaders.metal:2764-2802)
 __global__ __launch_bounds__(256) void fm_pf_combine(PfArgs a, float *out, int flags) {
     const int m = blockIdx.x, H = a.g.hidden, K = a.K;
@@ -533,9 +910,32 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
     // tiles, a group tile, 16 operand registers, loads in flight), which caps a SIMD at two
     // waves; capping the registers instead made them spill and run 2-5x slower
     const int grid = max_items < n_cu ? max_items : n_cu;
-    if (g->hidden == 2048) PF_LAUNCH(fm_pf_gate_up, 32, grid, 512);
-    else PF_LAUNCH(fm_pf_gate_up, 16, grid, 512);
-    PF_LAUNCH(fm_pf_down, 8, grid, 512);
+    static const bool old_path = getenv("FINCH_PREFILL_OLD") != nullptr;
+    if (!old_path && g->hidden == 2048) {
+#define PF_SLAB(GPW, GU)                                                                           \
+    do {                                                                                           \
+        static bool attr_set = false;                                                              \
+        auto kfn = fm_pf_slab<GPW, GU>;                                                            \
+        if (!attr_set) {                                                                           \
+            if (hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                    PfSlab<GPW>::LDS_BYTES) != hipSuccess)                         \
+                return FM_ERR_HIP;                                                                 \
+            attr_set = true;                                                                       \
+        }                                                                                          \
+        hipLaunchKernelGGL(kfn, dim3(grid), dim3(512), PfSlab<GPW>::LDS_BYTES, st, a);             \
+    } while (0)
+        // gate/up: K split over the waves.  down keeps the kernel above: with one group
+        // (four MFMAs) per wave and tile the per-tile overhead of the split outweighs it.
+        PF_SLAB(4, true);
+        static const bool slab_down = getenv("FINCH_PREFILL_SLAB_DOWN") != nullptr;
+        if (slab_down) PF_SLAB(1, false);
+        else PF_LAUNCH(fm_pf_down, 8, grid, 512);
+#undef PF_SLAB
+    } else {
+        if (g->hidden == 2048) PF_LAUNCH(fm_pf_gate_up, 32, grid, 512);
+        else PF_LAUNCH(fm_pf_gate_up, 16, grid, 512);
+        PF_LAUNCH(fm_pf_down, 8, grid, 512);
+    }
 #undef PF_LAUNCH
     hipLaunchKernelGGL(fm_pf_combine, dim3(M, (g->hidden + 1023) / 1024), dim3(256), 0, st, a, d_out, flags);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
