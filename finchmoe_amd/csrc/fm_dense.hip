@@ -8,7 +8,8 @@
 // Same lane mapping as the expert kernels: a lane owns 128 columns, LPR =
 // in_dim/128 lanes share a row, a wave step covers 64/LPR rows that are
 // contiguous in memory.
-#include "fm_unpack.h"
+#include "fm_mfma.h"
+#include "fm_ring.h"
 
 #define FM_MAX_BATCH 8
 
@@ -26,6 +27,7 @@ struct FmDenseArgs {
     int rows_per_item;
     const float *x;      // [M][in_dim]
     size_t out_stride;   // elements between positions in every out (= out_dim of that tensor if 0)
+    int unit_first[FM_MAX_BATCH + 1];   // streaming kernel: first wave step of every tensor
 };
 
 namespace {
@@ -82,6 +84,209 @@ __global__ __launch_bounds__(256) void fm_dense_gemv(FmDenseArgs a) {
     }
 }
 
+// ----------------------------------------------------------------------
+// Streaming form (3- and 4-bit, in_dim up to 2048, or 4096 at 4 bits): the
+// structure of the expert kernels (fm_decode.hip) without segments.  All wave
+// steps ("units", 64/LPR rows) of all tensors of the launch form one sequence;
+// workgroup g (8 waves, one per CU) takes [U*g/G, U*(g+1)/G), its waves claim
+// units from an LDS counter, copy their bytes into a per-wave ring in LDS with
+// LDS-direct loads (three or four units in flight, no destination registers)
+// and multiply on the matrix cores against the activation registers, which the
+// workgroup builds once.  in_dim = 4096 is two slabs of 2048 columns: a unit is
+// two slices, each against its own activation registers, summed in slab order.
+// ----------------------------------------------------------------------
+template <int BITS>
+struct FmDenseRing {
+    static constexpr int RING = BITS == 3 ? 4 : 3;
+    static constexpr int BYTES = 8 * RING * FmSlot<BITS>::BYTES;
+};
+
+template <int BITS, int LPR, int NS>
+constexpr size_t fm_dense_stream_lds() {
+    return FmDenseRing<BITS>::BYTES + NS * sizeof(FmActLds<LPR>);
+}
+
+extern __shared__ __attribute__((aligned(16))) uint8_t fm_dense_lds[];
+
+template <int BITS, int LPR, int NS, bool FP16>
+__global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_units) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    using SL = FmSlot<BITS>;
+    constexpr int RPS = FM_WAVE / LPR, RING = FmDenseRing<BITS>::RING;
+    constexpr int SLAB_COLS = FM_CPL * LPR;
+    constexpr int SLAB_ROW_BYTES = LPR * FmLaneBytes<BITS>::value, SLAB_SB = 4 * LPR;
+    static_assert(NS == 1 || (SLAB_ROW_BYTES == 1024 && RPS == SL::NQ), "one load per row and slab");
+    __shared__ unsigned int next_unit;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int m = blockIdx.y;
+    const uint32_t ring0 = fm_lds_addr(fm_dense_lds) + (uint32_t)wave * (RING * SL::BYTES);
+    FmActLds<LPR> *img = reinterpret_cast<FmActLds<LPR> *>(fm_dense_lds + FmDenseRing<BITS>::BYTES);
+    const int row_bytes = NS * SLAB_ROW_BYTES, sb_row_bytes = NS * SLAB_SB;
+    const long wg0 = (long)total_units * blockIdx.x / gridDim.x,
+               wg1 = (long)total_units * (blockIdx.x + 1) / gridDim.x;
+    const uint32_t n_units = (uint32_t)(wg1 - wg0);
+    if (threadIdx.x == 0) next_unit = 0u;
+    __syncthreads();                 // the counter is set
+    uint32_t woff, soff;
+    int ris, ch;
+    fm_unit_lane_offsets<BITS, LPR>(lane, SLAB_ROW_BYTES, SLAB_SB, woff, soff, ris, ch);
+
+    // unit u of the launch -> tensor and first row (no indexing of the argument arrays
+    // with a run-time value: that would move them to private memory)
+    struct Where {
+        const uint8_t *W, *S, *B;
+        float *out;
+        int row0, out_dim;
+    };
+    auto locate = [&](long u) __attribute__((always_inline)) {
+        Where w{a.spec[0].W, a.spec[0].S, a.spec[0].B, a.spec[0].out, 0, a.spec[0].out_dim};
+        int first = 0;
+#pragma unroll
+        for (int i = 1; i < FM_MAX_BATCH; i++)
+            if (i < a.n && u >= a.unit_first[i]) {
+                w.W = a.spec[i].W, w.S = a.spec[i].S, w.B = a.spec[i].B, w.out = a.spec[i].out;
+                w.out_dim = a.spec[i].out_dim;
+                first = a.unit_first[i];
+            }
+        w.row0 = (int)(u - first) * RPS;
+        return w;
+    };
+
+    // ---- loader
+    int kn = 0, wpos = 0;
+    uint32_t issued = 0, consumed = 0, tag_n = 0;
+    const uint8_t *wp = nullptr, *sp = nullptr, *bp = nullptr;
+    bool dry = false;
+    auto issue = [&]() __attribute__((always_inline)) {
+        if (dry) return;
+        if (kn == 0) {
+            const uint32_t ul = fm_claim_unit(&next_unit, lane);
+            if (ul >= n_units) {
+                dry = true;
+                return;
+            }
+            const Where w = locate(wg0 + ul);
+            wp = fm_uniform(w.W + (size_t)w.row0 * row_bytes);
+            sp = fm_uniform(w.S + (size_t)w.row0 * sb_row_bytes);
+            bp = fm_uniform(w.B + (size_t)w.row0 * sb_row_bytes);
+            tag_n = ul;
+        }
+        const uint32_t slot = ring0 + (uint32_t)wpos * SL::BYTES;
+        fm_slot_tag(slot + SL::TAG, tag_n);
+        if constexpr (NS == 1) {
+            fm_dma_issue<BITS>(slot, wp, sp, bp, lane);
+        } else {
+            // slab kn of the unit's rows: one 1 KB run per row, 64 B of scales / biases per row
+#pragma unroll
+            for (int i = 0; i < RPS; i++)
+                __builtin_amdgcn_global_load_lds(
+                    (fm_gptr)(uintptr_t)(wp + (size_t)i * row_bytes + kn * SLAB_ROW_BYTES + lane * 16),
+                    (fm_lptr)(uintptr_t)(slot + 1024 * i), 16, 0, 0);
+            const uint32_t so = (uint32_t)((lane >> 4) * sb_row_bytes + kn * SLAB_SB + (lane & 15) * 4);
+            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(sp + so),
+                                             (fm_lptr)(uintptr_t)(slot + SL::WBYTES), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(bp + so),
+                                             (fm_lptr)(uintptr_t)(slot + SL::WBYTES + 256), 4, 0, 0);
+        }
+        kn = kn + 1 == NS ? 0 : kn + 1;
+        wpos = wpos + 1 == RING ? 0 : wpos + 1;
+        issued++;
+    };
+#pragma unroll
+    for (int k = 0; k < RING; k++) issue();      // the weights do not wait for the activations
+
+    // the activation registers of every slab, built once
+    FmBuildSlot<BITS> bslot;
+    bslot.init();
+#pragma unroll
+    for (int k = 0; k < NS; k++) {
+        if (threadIdx.x < 256) {
+            FmActX<LPR> xr;
+            fm_act_load<BITS, LPR, false>(a.x + (size_t)m * a.in_dim + k * SLAB_COLS, bslot, xr);
+            fm_act_build<BITS, LPR>(xr, bslot, img[k]);
+        }
+    }
+    __syncthreads();
+    FmActRegs ar[NS];
+#pragma unroll
+    for (int k = 0; k < NS; k++) fm_read_act_lds<LPR>(img[k], lane, ar[k]);
+
+    int c = 0;
+    while (consumed < issued) {
+        float v = 0.0f;
+        uint32_t tag = 0;
+#pragma unroll
+        for (int k = 0; k < NS; k++) {
+            FmRowSlice<BITS> t;
+            if (issued - consumed == (uint32_t)RING) fm_dma_wait<SL::LOADS *(RING - 1)>(false);
+            else fm_dma_wait<0>(true);
+            tag = fm_dma_read<BITS>(ring0 + (uint32_t)c * SL::BYTES, woff, soff, t);
+            consumed++;
+            c = c + 1 == RING ? 0 : c + 1;
+            issue();
+            v += fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(t, ar[k]));
+        }
+        const Where w = locate(wg0 + tag);
+        if (ch == 0) w.out[(size_t)m * w.out_dim + w.row0 + ris] = v;
+    }
+#else
+    (void)a;
+    (void)total_units;
+#endif
+}
+
+// launches the streaming kernel when the shapes allow it; FM_ERR_UNSUPPORTED otherwise
+template <int BITS, bool FP16>
+int launch_dense_stream_t(FmDenseArgs &a, int M, int n_cu, hipStream_t st) {
+    const int lpr_full = a.in_dim / FM_CPL;
+    const int ns = lpr_full == 32 ? 2 : 1, lpr = lpr_full / ns;
+    if (!(lpr == 4 || lpr == 8 || lpr == 16) || (ns == 2 && BITS != 4)) return FM_ERR_UNSUPPORTED;
+    const int rps = FM_WAVE / lpr;
+    int units = 0;
+    for (int i = 0; i < a.n; i++) {
+        if (a.spec[i].out_dim % rps) return FM_ERR_UNSUPPORTED;
+        a.unit_first[i] = units;
+        units += a.spec[i].out_dim / rps;
+    }
+    for (int i = a.n; i <= FM_MAX_BATCH; i++) a.unit_first[i] = units;
+    // Worth it only when every wave of the chip gets a unit: below that the launch is a
+    // chain of latencies either way, and the plain kernel's chain is shorter (measured:
+    // 2048 rows of 4096 columns take 6.0 us there and 12.4 us here).
+    // (decided by the tensor shapes alone, so that M positions and one position take the same
+    // kernel and stay bitwise equal)
+    if (units < 8L * n_cu) return FM_ERR_UNSUPPORTED;
+    long wgs = n_cu;
+    if (units < 8 * wgs) wgs = (units + 7) / 8;
+    dim3 grid((unsigned)wgs, M);
+#define FM_DS(L, NS_)                                                                          \
+    do {                                                                                       \
+        auto kfn = fm_dense_stream<BITS, L, NS_, FP16>;                                        \
+        const size_t sh = fm_dense_stream_lds<BITS, L, NS_>();                                 \
+        static bool attr_set[64] = {};                                                         \
+        int dev = 0;                                                                           \
+        (void)hipGetDevice(&dev);                                                              \
+        if (dev < 0 || dev >= 64 || !attr_set[dev]) {                                          \
+            if (hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                    (int)sh) != hipSuccess)                                    \
+                return FM_ERR_HIP;                                                             \
+            if (dev >= 0 && dev < 64) attr_set[dev] = true;                                    \
+        }                                                                                      \
+        hipLaunchKernelGGL(kfn, grid, dim3(512), sh, st, a, units);                            \
+    } while (0)
+    if (ns == 2) {
+        if constexpr (BITS == 4) FM_DS(16, 2);
+    } else {
+        switch (lpr) {
+            case 4: FM_DS(4, 1); break;
+            case 8: FM_DS(8, 1); break;
+            default: FM_DS(16, 1); break;
+        }
+    }
+#undef FM_DS
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
+
 template <int BITS, bool FP16>
 int launch_dense_t(const FmDenseArgs &a, int total_items, int M, hipStream_t st) {
     dim3 grid(total_items, M), b(256);
@@ -129,6 +334,15 @@ extern "C" int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, 
         a.spec[i] = specs[i];
     }
     for (int i = n; i < FM_MAX_BATCH; i++) a.spec[i] = a.spec[0];
+    static const bool no_stream = getenv("FINCH_DENSE_VALU") != nullptr;
+    if (!no_stream && (bits == 3 || bits == 4)) {
+        int rc = FM_ERR_UNSUPPORTED;
+        if (bits == 3) rc = scale_fp16 ? launch_dense_stream_t<3, true>(a, M, n_cu, st)
+                                       : launch_dense_stream_t<3, false>(a, M, n_cu, st);
+        else rc = scale_fp16 ? launch_dense_stream_t<4, true>(a, M, n_cu, st)
+                             : launch_dense_stream_t<4, false>(a, M, n_cu, st);
+        if (rc != FM_ERR_UNSUPPORTED) return rc;
+    }
     switch (bits) {
         case 3: return scale_fp16 ? launch_dense_t<3, true>(a, items, M, st)
                                   : launch_dense_t<3, false>(a, items, M, st);

@@ -11,7 +11,7 @@
 // the consumers wait and read with explicit instructions.
 #pragma once
 
-#include "fm_common.h"
+#include "fm_unpack.h"
 
 #if defined(__HIPCC__)
 
@@ -37,5 +37,117 @@ __device__ __forceinline__ void fm_dma_wait(bool drain) {
 __device__ __forceinline__ uint32_t fm_lds_addr(const void *p) {
     return (uint32_t)(uintptr_t)(fm_lptr)p;
 }
+
+
+// One ring slot = one slice (a wave step's rows of one matrix): 64 lanes' worth of
+// codes laid out as the rows lie in memory, 256 B of scales, 256 B of biases, and a
+// 16-byte trailer for the tag (which unit the slice belongs to).
+template <int BITS>
+struct FmSlot {
+    static constexpr int NQ = FmLaneBytes<BITS>::value / 16;
+    static constexpr int WBYTES = FM_WAVE * FmLaneBytes<BITS>::value;
+    static constexpr int TAG = WBYTES + 512;
+    static constexpr int BYTES = WBYTES + 512 + 16;
+    static constexpr int LOADS = NQ + 2;            // LDS-direct loads per slice
+};
+
+// Lane map of a wave step: LPR lanes share a row (lane = 4*chunk + row-in-quad), the
+// step covers 64/LPR consecutive rows.  woff / soff: this lane's 48/64 code bytes and
+// its scale/bias word inside a slot whose rows are row_bytes / sb_row_bytes apart.
+template <int BITS, int LPR>
+__device__ __forceinline__ void fm_unit_lane_offsets(int lane, int row_bytes, int sb_row_bytes,
+                                                     uint32_t &woff, uint32_t &soff,
+                                                     int &row_in_step, int &ch) {
+    const int j = lane & 3;
+    ch = (lane >> 2) % LPR;
+    const int rq = lane / (4 * LPR);
+    row_in_step = 4 * rq + j;
+    woff = (uint32_t)(row_in_step * row_bytes + ch * FmLaneBytes<BITS>::value);
+    soff = (uint32_t)(row_in_step * sb_row_bytes + ch * 4);
+}
+
+template <int BITS, int I>
+__device__ __forceinline__ void fm_dma_codes(uint32_t slot, fm_gptr w) {
+    if constexpr (I < FmSlot<BITS>::NQ) {
+        // the instruction offset moves the global and the LDS address alike
+        __builtin_amdgcn_global_load_lds(w, (fm_lptr)(uintptr_t)slot, 16, 1024 * I, 0);
+        fm_dma_codes<BITS, I + 1>(slot, w);
+    }
+}
+
+// w, s, b: first byte of the unit's rows in the weight, scale and bias regions
+template <int BITS>
+__device__ __forceinline__ void fm_dma_issue(uint32_t slot, const uint8_t *w, const uint8_t *s,
+                                             const uint8_t *b, int lane) {
+    fm_dma_codes<BITS, 0>(slot, (fm_gptr)(uintptr_t)(w + lane * 16));
+    __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(s + lane * 4),
+                                     (fm_lptr)(uintptr_t)(slot + FmSlot<BITS>::WBYTES), 4, 0, 0);
+    __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(b + lane * 4),
+                                     (fm_lptr)(uintptr_t)(slot + FmSlot<BITS>::WBYTES + 256), 4, 0, 0);
+}
+
+// this lane's codes and scale/bias words out of a landed slot
+// (returns the slot's tag)
+template <int BITS>
+__device__ __forceinline__ uint32_t fm_dma_read(uint32_t slot, uint32_t woff, uint32_t soff,
+                                                FmRowSlice<BITS> &t) {
+    const uint32_t aw = slot + woff, as = slot + FmSlot<BITS>::WBYTES + soff;
+    const uint32_t at = slot + FmSlot<BITS>::TAG;
+    uint32_t tag;
+    if constexpr (BITS == 3) {
+        asm volatile("ds_read_b128 %0, %6\n\tds_read_b128 %1, %6 offset:16\n\t"
+                     "ds_read_b128 %2, %6 offset:32\n\tds_read_b32 %3, %7\n\t"
+                     "ds_read_b32 %4, %7 offset:256\n\tds_read_b32 %5, %8\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&v"(t.q[0]), "=&v"(t.q[1]), "=&v"(t.q[2]), "=&v"(t.s), "=&v"(t.b),
+                       "=&v"(tag)
+                     : "v"(aw), "v"(as), "v"(at)
+                     : "memory");
+    } else {
+        asm volatile("ds_read_b128 %0, %7\n\tds_read_b128 %1, %7 offset:16\n\t"
+                     "ds_read_b128 %2, %7 offset:32\n\tds_read_b128 %3, %7 offset:48\n\t"
+                     "ds_read_b32 %4, %8\n\tds_read_b32 %5, %8 offset:256\n\t"
+                     "ds_read_b32 %6, %9\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(t.q[0]), "=&v"(t.q[1]), "=&v"(t.q[2]), "=&v"(t.q[3]), "=&v"(t.s),
+                       "=&v"(t.b), "=&v"(tag)
+                     : "v"(aw), "v"(as), "v"(at)
+                     : "memory");
+    }
+    return __builtin_amdgcn_readfirstlane(tag);
+}
+
+// Units of a segment are handed out one at a time from a counter in LDS: the
+// hardware favours the older of two waves that share a SIMD, so with a fixed
+// share per wave the favoured half finishes early and the CU runs the rest of
+// the kernel half empty.  With a shared counter every wave of the workgroup
+// ends within one unit of the others.
+// (Written as an instruction: the compiler would make an LDS atomic wait for
+// every outstanding LDS-direct load, which empties the ring.)
+__device__ __forceinline__ uint32_t fm_claim_unit(unsigned int *next, int lane) {
+    uint32_t v = 0;
+    if (lane == 0) {
+        const uint32_t addr = (uint32_t)(uintptr_t)(fm_lptr)next, one = 1u;
+        asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(v)
+                     : "v"(addr), "v"(one)
+                     : "memory");
+    }
+    return __builtin_amdgcn_readfirstlane(v);
+}
+
+// tag of the slice in a slot (which unit it belongs to), kept in the slot's
+// trailer so that the consumer needs no queue in registers
+__device__ __forceinline__ void fm_slot_tag(uint32_t slot_tag_addr, uint32_t tag) {
+    asm volatile("ds_write_b32 %0, %1" ::"v"(slot_tag_addr), "v"(tag) : "memory");
+}
+__device__ __forceinline__ uint32_t fm_slot_peek(uint32_t slot_tag_addr) {
+    uint32_t tag;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&v"(tag)
+                 : "v"(slot_tag_addr)
+                 : "memory");
+    return __builtin_amdgcn_readfirstlane(tag);
+}
+
 
 #endif

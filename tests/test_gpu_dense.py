@@ -59,6 +59,27 @@ def test_matvec_shapes_and_widths(hip, orc, bits, dtype, out_dim, in_dim):
     hip.tensor_release(t)
 
 
+@pytest.mark.parametrize("bits,dtype,out_dim,in_dim", [
+    (4, "bf16", 8192, 4096), (3, "bf16", 8192, 2048), (4, "fp16", 16384, 1024),
+    (3, "fp16", 32768, 512)])
+def test_streaming_kernel_shapes(hip, orc, bits, dtype, out_dim, in_dim):
+    """Launches large enough for the streaming kernel (a wave step for every wave of the
+    chip): two column slabs at in_dim 4096, every lanes-per-row specialisation, both widths
+    and scale types; M positions equal the single call bitwise."""
+    rng = np.random.default_rng(out_dim + in_dim + bits)
+    t, (codes, W, S, B, sd) = _tensor(hip, rng, out_dim, in_dim, bits, dtype)
+    X = rng.standard_normal((2, in_dim)).astype(np.float32)
+    (got,) = hip.matvec_batch([t], X[0], [out_dim])
+    ref = orc.dequant_matvec(W, S, B, X[0], out_dim, in_dim, bits, scale_dtype=sd, nthreads=8)
+    r, _ = assert_parity(got, ref, "matvec")
+    assert r < 2e-5, r
+    out = hip.matvec_prefill(t, X, out_dim)
+    assert np.array_equal(out[0], got)
+    assert_parity(out[1], orc.dequant_matvec(W, S, B, X[1], out_dim, in_dim, bits,
+                                             scale_dtype=sd, nthreads=8), "position 1")
+    hip.tensor_release(t)
+
+
 def test_matvec_prefill_positions(hip, orc):
     """M-position clone (dequant_matvec_4bit_prefill): every position equals the single call."""
     rng = np.random.default_rng(3)
