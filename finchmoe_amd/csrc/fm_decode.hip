@@ -692,12 +692,10 @@ void fm_moe_fused(DecodeArgs a, int n_pairs, FmFlags f) {
     }
 }
 
-// Raise a kernel's dynamic LDS limit (the default stops at 64 KB).  The
-// attribute belongs to a device's copy of the kernel: done once per kernel and
-// device (these runtime calls cost more host time than a launch).
+// per kernel and device: dynamic LDS limit raised, resident workgroups per CU asked
 constexpr int FM_MAX_DEVICES = 64;
 struct FmKernelSetup {
-    bool lds_set[FM_MAX_DEVICES] = {};
+    FmLdsAttr lds;
     int per_cu[FM_MAX_DEVICES] = {};   // resident workgroups per CU, 0 = not asked yet
 };
 
@@ -708,13 +706,7 @@ int fm_current_device() {
 }
 
 bool fm_dyn_lds_ok(FmKernelSetup &ks, const void *fn, size_t bytes) {
-    const int d = fm_current_device();
-    if (d >= 0 && ks.lds_set[d]) return true;
-    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) !=
-        hipSuccess)
-        return false;
-    if (d >= 0) ks.lds_set[d] = true;
-    return true;
+    return fm_dyn_lds_ready(ks.lds, fn, bytes);
 }
 
 // workgroups of a streaming launch: one per CU (LDS budget), fewer when there

@@ -263,15 +263,8 @@ int launch_dense_stream_t(FmDenseArgs &a, int M, int n_cu, hipStream_t st) {
     do {                                                                                       \
         auto kfn = fm_dense_stream<BITS, L, NS_, FP16>;                                        \
         const size_t sh = fm_dense_stream_lds<BITS, L, NS_>();                                 \
-        static bool attr_set[64] = {};                                                         \
-        int dev = 0;                                                                           \
-        (void)hipGetDevice(&dev);                                                              \
-        if (dev < 0 || dev >= 64 || !attr_set[dev]) {                                          \
-            if (hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                    (int)sh) != hipSuccess)                                    \
-                return FM_ERR_HIP;                                                             \
-            if (dev >= 0 && dev < 64) attr_set[dev] = true;                                    \
-        }                                                                                      \
+        static FmLdsAttr attr;                                                                 \
+        if (!fm_dyn_lds_ready(attr, (const void *)kfn, sh)) return FM_ERR_HIP;                 \
         hipLaunchKernelGGL(kfn, grid, dim3(512), sh, st, a, units);                            \
     } while (0)
     if (ns == 2) {

@@ -897,13 +897,8 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
     const int max_items = g->n_experts + (int)(n / PF_TM);
 #define PF_LAUNCH(KERN, NG, GRID, NT)                                                              \
     do {                                                                                           \
-        static bool attr_set = false;                                                              \
-        if (!attr_set) {                                                                           \
-            if (hipFuncSetAttribute((const void *)KERN<NG>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                    (int)sizeof(PfLds<NG>)) != hipSuccess)                         \
-                return FM_ERR_HIP;                                                                 \
-            attr_set = true;                                                                       \
-        }                                                                                          \
+        static FmLdsAttr attr;                                                                     \
+        if (!fm_dyn_lds_ready(attr, (const void *)KERN<NG>, sizeof(PfLds<NG>))) return FM_ERR_HIP; \
         hipLaunchKernelGGL(KERN<NG>, dim3(GRID), dim3(NT), sizeof(PfLds<NG>), st, a);              \
     } while (0)
     // one 8-wave workgroup per CU: the kernels need ~200 registers per lane (two accumulator
@@ -914,14 +909,9 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
     if (!old_path && g->hidden == 2048) {
 #define PF_SLAB(GPW, GU)                                                                           \
     do {                                                                                           \
-        static bool attr_set = false;                                                              \
+        static FmLdsAttr attr;                                                                     \
         auto kfn = fm_pf_slab<GPW, GU>;                                                            \
-        if (!attr_set) {                                                                           \
-            if (hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                    PfSlab<GPW>::LDS_BYTES) != hipSuccess)                         \
-                return FM_ERR_HIP;                                                                 \
-            attr_set = true;                                                                       \
-        }                                                                                          \
+        if (!fm_dyn_lds_ready(attr, (const void *)kfn, PfSlab<GPW>::LDS_BYTES)) return FM_ERR_HIP; \
         hipLaunchKernelGGL(kfn, dim3(grid), dim3(512), PfSlab<GPW>::LDS_BYTES, st, a);             \
     } while (0)
         // gate/up: K split over the waves.  down keeps the kernel above: with one group

@@ -150,4 +150,21 @@ __device__ __forceinline__ uint32_t fm_slot_peek(uint32_t slot_tag_addr) {
 }
 
 
+// Host side: raise a kernel's dynamic LDS limit above the 64 KB default, once per
+// kernel and device (the attribute belongs to a device's copy of the kernel, and the
+// runtime call costs more host time than a launch).
+struct FmLdsAttr {
+    bool set[64] = {};
+};
+inline bool fm_dyn_lds_ready(FmLdsAttr &a, const void *fn, size_t bytes) {
+    int d = 0;
+    (void)hipGetDevice(&d);
+    const bool known = d >= 0 && d < 64;
+    if (known && a.set[d]) return true;
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
+        return false;
+    if (known) a.set[d] = true;
+    return true;
+}
+
 #endif
