@@ -367,49 +367,6 @@ __global__ __launch_bounds__(1024) void fm_pf_sort(PfArgs a) {
     }
 }
 
-// gate + up + SwiGLU for every item -> act[sorted position][inter]
-template <int NG>
-__global__ __launch_bounds__(512) void fm_pf_gate_up(PfArgs a) {
-    extern __shared__ uint4 pf_smem[];
-    PfLds<NG> &L = *reinterpret_cast<PfLds<NG> *>(pf_smem);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n_items = *a.n_items;
-    const int row_bytes = a.g.hidden * 3 / 8, sb_bytes = (a.g.hidden / 64) * 2;
-    const uint32_t ones = fm_opaque(0x3F803F80u);
-    for (int it = blockIdx.x; it < n_items; it += gridDim.x) {
-        const PfItem item = a.items[it];
-        __syncthreads();    // readers of the previous image are done
-        pf_stage<NG>(L, item.count, [&](int j) {
-            return a.X + (size_t)(a.sorted[item.start + j] / a.K) * a.g.hidden;
-        });
-        __syncthreads();
-        const uint8_t *blob = a.layer + (size_t)item.expert * a.g.expert_size;
-        const int n = lane & 31, h = lane >> 5;
-        const int NW = blockDim.x / 64;
-        // pass p: row tile wave + NW*p, gate and up rows together
-        const int n_tiles = (a.g.inter / 32 - wave + NW - 1) / NW;
-        pf_passes<NG, 4>(
-            L, n_tiles, lane, ones,
-            [&](int p, int r, gptr &w, gptr &sr, gptr &br) {
-                const int row = (wave + NW * p) * 32 + n;
-                w = (gptr)(uintptr_t)(blob + (r ? a.g.up_w : a.g.gate_w) + (size_t)row * row_bytes);
-                sr = (gptr)(uintptr_t)(blob + (r ? a.g.up_s : a.g.gate_s) + (size_t)row * sb_bytes);
-                br = (gptr)(uintptr_t)(blob + (r ? a.g.up_b : a.g.gate_b) + (size_t)row * sb_bytes);
-            },
-            [&](int p, const f16v *acc) {
-                const int row = (wave + NW * p) * 32 + n;
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    const int tok = 8 * (i / 4) + 4 * h + (i % 4);   // M row of register i (hi piece)
-                    if (tok < item.count) {
-                        float gv = acc[0][i] + acc[0][i + 8], uv = acc[1][i] + acc[1][i + 8];
-                        a.act[(size_t)(item.start + tok) * a.g.inter + row] = fm_silu_mul(gv, uv);
-                    }
-                }
-            });
-    }
-}
-
 // down for every item -> eo[pair][hidden]
 template <int NG>
 __global__ __launch_bounds__(512) void fm_pf_down(PfArgs a) {
@@ -859,8 +816,8 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 bool pf_supported(const FmExpertGeom *g) {
     // 3-bit codes, BF16 scales (their bits are MFMA operands), whole 32-row tiles and
     // an even number of groups; LDS image must fit
-    return g->bits == 3 && !g->scale_fp16 && g->n_experts <= PF_MAX_EXPERTS &&
-           (g->hidden == 2048 || g->hidden == 1024) && g->inter == 512;
+    return g->bits == 3 && !g->scale_fp16 && g->n_experts <= PF_MAX_EXPERTS && g->hidden == 2048 &&
+           g->inter == 512;
 }
 
 }  // namespace
@@ -905,27 +862,16 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
     // tiles, a group tile, 16 operand registers, loads in flight), which caps a SIMD at two
     // waves; capping the registers instead made them spill and run 2-5x slower
     const int grid = max_items < n_cu ? max_items : n_cu;
-    static const bool old_path = getenv("FINCH_PREFILL_OLD") != nullptr;
-    if (!old_path && g->hidden == 2048) {
-#define PF_SLAB(GPW, GU)                                                                           \
-    do {                                                                                           \
-        static FmLdsAttr attr;                                                                     \
-        auto kfn = fm_pf_slab<GPW, GU>;                                                            \
-        if (!fm_dyn_lds_ready(attr, (const void *)kfn, PfSlab<GPW>::LDS_BYTES)) return FM_ERR_HIP; \
-        hipLaunchKernelGGL(kfn, dim3(grid), dim3(512), PfSlab<GPW>::LDS_BYTES, st, a);             \
-    } while (0)
-        // gate/up: K split over the waves.  down keeps the kernel above: with one group
-        // (four MFMAs) per wave and tile the per-tile overhead of the split outweighs it.
-        PF_SLAB(4, true);
-        static const bool slab_down = getenv("FINCH_PREFILL_SLAB_DOWN") != nullptr;
-        if (slab_down) PF_SLAB(1, false);
-        else PF_LAUNCH(fm_pf_down, 8, grid, 512);
-#undef PF_SLAB
-    } else {
-        if (g->hidden == 2048) PF_LAUNCH(fm_pf_gate_up, 32, grid, 512);
-        else PF_LAUNCH(fm_pf_gate_up, 16, grid, 512);
-        PF_LAUNCH(fm_pf_down, 8, grid, 512);
+    // gate/up: K split over the waves (fm_pf_slab).  down: whole K per wave (fm_pf_down) —
+    // with one group (four MFMAs) per wave and tile the split's per-tile overhead outweighs
+    // what it saves.
+    {
+        static FmLdsAttr attr;
+        auto kfn = fm_pf_slab<4, true>;
+        if (!fm_dyn_lds_ready(attr, (const void *)kfn, PfSlab<4>::LDS_BYTES)) return FM_ERR_HIP;
+        hipLaunchKernelGGL(kfn, dim3(grid), dim3(512), PfSlab<4>::LDS_BYTES, st, a);
     }
+    PF_LAUNCH(fm_pf_down, 8, grid, 512);
 #undef PF_LAUNCH
     hipLaunchKernelGGL(fm_pf_combine, dim3(M, (g->hidden + 1023) / 1024), dim3(256), 0, st, a, d_out, flags);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
