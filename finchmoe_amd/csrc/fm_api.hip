@@ -100,6 +100,7 @@ struct fm_ctx {
     unsigned int *d_counters = nullptr;
     // staging for the host-pointer entry points
     void *d_stage = nullptr;
+    void *h_stage = nullptr;   // pinned mirror of d_stage: one copy in, one copy out per call
     size_t stage_bytes = 0;
     void *d_ws = nullptr;
     size_t ws_bytes = 0;
@@ -142,10 +143,13 @@ struct DeviceGuard {
 
 int ensure_stage(fm_ctx *c, size_t bytes) {
     if (c->stage_bytes >= bytes) return FM_OK;
+    HIPCHK(c, hipStreamSynchronize(c->stream));
     if (c->d_stage) HIPCHK(c, hipFree(c->d_stage));
-    c->d_stage = nullptr;
+    if (c->h_stage) HIPCHK(c, hipHostFree(c->h_stage));
+    c->d_stage = c->h_stage = nullptr;
     c->stage_bytes = 0;
     HIPCHK(c, hipMalloc(&c->d_stage, bytes));
+    HIPCHK(c, hipHostMalloc(&c->h_stage, bytes, hipHostMallocDefault));
     c->stage_bytes = bytes;
     return FM_OK;
 }
@@ -286,6 +290,7 @@ extern "C" int fm_ctx_destroy(fm_ctx *c) {
     void *ptrs[] = {c->d_layer_ptrs, c->d_gg_ptrs, c->d_act, c->d_eo, c->d_counters,
                     c->dflags.set[0],
                     c->d_stage, c->d_ws};
+    if (c->h_stage) (void)hipHostFree(c->h_stage);
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     (void)hipEventDestroy(c->ev0);
@@ -515,20 +520,27 @@ static int moe_host_call(fm_ctx *c, moe_dev_fn fn, int hidden, int layer, const 
     size_t off_o = off_w + ((ni + 255) & ~(size_t)255), off_e = off_o + nx;
     int rc = ensure_stage(c, off_e + (expert_out ? ne : 0));
     if (rc) return rc;
-    char *st = (char *)c->d_stage;
-    HIPCHK(c, hipMemcpyAsync(st + off_x, x, nx, hipMemcpyHostToDevice, c->stream));
-    HIPCHK(c, hipMemcpyAsync(st + off_i, idx, ni, hipMemcpyHostToDevice, c->stream));
-    HIPCHK(c, hipMemcpyAsync(st + off_w, w, ni, hipMemcpyHostToDevice, c->stream));
-    if (flags & FM_ACCUMULATE)
-        HIPCHK(c, hipMemcpyAsync(st + off_o, out, nx, hipMemcpyHostToDevice, c->stream));
+    // inputs through the pinned mirror: one copy in (x | idx | w | out if accumulating), one
+    // copy out (out | expert_out) — pageable copies cost ~10 us each
+    char *st = (char *)c->d_stage, *hs = (char *)c->h_stage;
+    memcpy(hs + off_x, x, nx);
+    memcpy(hs + off_i, idx, ni);
+    memcpy(hs + off_w, w, ni);
+    size_t in_bytes = off_w + ni;
+    if (flags & FM_ACCUMULATE) {
+        memcpy(hs + off_o, out, nx);
+        in_bytes = off_o + nx;
+    }
+    HIPCHK(c, hipMemcpyAsync(st, hs, in_bytes, hipMemcpyHostToDevice, c->stream));
     rc = fn(c, layer, (const float *)(st + off_x), (const int32_t *)(st + off_i),
             (const float *)(st + off_w), M, K, (float *)(st + off_o),
             expert_out ? (float *)(st + off_e) : nullptr, flags);
     if (rc) return rc;
-    HIPCHK(c, hipMemcpyAsync(out, st + off_o, nx, hipMemcpyDeviceToHost, c->stream));
-    if (expert_out)
-        HIPCHK(c, hipMemcpyAsync(expert_out, st + off_e, ne, hipMemcpyDeviceToHost, c->stream));
+    const size_t out_bytes = nx + (expert_out ? ne : 0);
+    HIPCHK(c, hipMemcpyAsync(hs + off_o, st + off_o, out_bytes, hipMemcpyDeviceToHost, c->stream));
     HIPCHK(c, hipStreamSynchronize(c->stream));
+    memcpy(out, hs + off_o, nx);
+    if (expert_out) memcpy(expert_out, hs + off_e, ne);
     return check_grid_error(c);
 }
 
