@@ -72,7 +72,7 @@ def zipf_routing(rng, tokens, layers, n_experts, k):
     return idx, w
 
 
-def cpu_baseline_decode(blob_t, lo, idx, w, x, budget_s=12.0):
+def cpu_baseline_decode(blob_t, lo, idx, w, x, budget_s=12.0, bits=3):
     """Oracle expert loop, 1 thread, on (token, layer) samples until ~budget_s of CPU time.
     Only the 8 routed experts of each sample are copied back from HBM."""
     from oracle import oracle
@@ -86,7 +86,7 @@ def cpu_baseline_decode(blob_t, lo, idx, w, x, budget_s=12.0):
         mini = np.concatenate([blob_t[l, int(e)].cpu().numpy() for e in sel])
         t0 = time.perf_counter()
         oracle.moe_experts_forward(mini, x[l % x.shape[0]], np.arange(len(sel), dtype=np.int32),
-                                   w[t, l], H, I, 3, nthreads=1)
+                                   w[t, l], H, I, bits, nthreads=1)
         t_cpu += time.perf_counter() - t0
         done += 1
         if t_cpu >= budget_s:
@@ -109,16 +109,17 @@ def run_decode_step(args):
     from finchmoe_amd import FinchHip, formats
     dev = torch.device("cuda:0")
     n_layers = args.layers
-    lo = formats.expert_layout(H, I, 3)
+    bits = args.bits
+    lo = formats.expert_layout(H, I, bits)
     es = lo["expert_size"]
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
     blob = torch.empty(n_layers, E, es, dtype=torch.uint8, device=dev)
     for l in range(n_layers):
-        fill_affine_layer(blob[l], lo, 3, gen)
+        fill_affine_layer(blob[l], lo, bits, gen)
     torch.cuda.synchronize()
     ctx = FinchHip(0)
-    ctx.experts_config(n_layers, E, H, I, 64, 3, 0)
+    ctx.experts_config(n_layers, E, H, I, 64, bits, 0)
     for l in range(n_layers):
         ctx.experts_adopt_layer(l, blob[l].data_ptr(), E * es)
 
@@ -182,16 +183,16 @@ def run_decode_step(args):
     k1_bytes = n_layers * K * gu_bytes
     uniq = len({(l, int(e)) for t in range(tokens) for l in range(n_layers) for e in idx[t, l]})
     res = {
-        "metric": "3-bit expert GEMV HBM GB/s over the %d-layer MoE decode step" % n_layers,
+        "metric": "%d-bit expert GEMV HBM GB/s over the %d-layer MoE decode step" % (bits, n_layers),
         "value": round(bytes_step / (ms_per_step * 1e-3) / 1e9, 2),
         "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "config 2: %d-layer routed-expert decode step, batch 1, %dx%d 3-bit "
+        "config": {"workload": "config 2: %d-layer routed-expert decode step, batch 1, %dx%d %d-bit "
                                "g64 experts resident in HBM (%.2f GB), top-%d Zipf(1.1) routing, "
-                               "x~N(0,1) fp32" % (n_layers, n_layers, E, n_layers * E * es / 1e9, K),
+                               "x~N(0,1) fp32" % (n_layers, n_layers, E, bits, n_layers * E * es / 1e9, K),
                    "hidden": H, "moe_intermediate": I, "experts": E, "top_k": K, "layers": n_layers,
                    "bytes_per_step": bytes_step, "scale_dtype": "bf16"},
         "us_per_step": round(ms_per_step * 1e3, 2),
@@ -202,10 +203,10 @@ def run_decode_step(args):
         "token_latency_us": {"mean": round(float(lat.mean()), 1), "p50": round(float(np.median(lat)), 1),
                              "p99": round(float(np.percentile(lat, 99)), 1)},
         "unique_experts_touched_in_256_tokens": uniq,
-        "roofline": {"bound": "hbm", "kernel": "fm_moe_fused<3,16> (gate/up, down, combine in one launch)",
+        "roofline": {"bound": "hbm", "kernel": "fm_moe_fused<%d,16> (gate/up, down, combine in one launch)" % bits,
                      "achieved": round(bytes_step / (op_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(bytes_step / (op_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": FUSED_TRAFFIC_BYTES_40L if (n_layers, E, K) == (40, 256, 8) else None,
+                     "traffic": FUSED_TRAFFIC_BYTES_40L if (n_layers, E, K, bits) == (40, 256, 8, 3) else None,
                      "bytes_per_launch": bytes_step, "us_per_launch": round(op_us, 2)},
         # the same work as three separate kernels (isolated launches, so a little slower
         # than back to back): where the time goes
@@ -215,7 +216,7 @@ def run_decode_step(args):
                                  "down_GBps": round((bytes_step - k1_bytes) / (k2_us * 1e-6) / 1e9, 1)},
     }
     if not args.no_cpu:
-        res["cpu_baseline"] = cpu_baseline_decode(blob, lo, idx, w, x, args.cpu_seconds)
+        res["cpu_baseline"] = cpu_baseline_decode(blob, lo, idx, w, x, args.cpu_seconds, bits)
     ctx.close()
     return res
 
@@ -481,6 +482,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="decode_step")
     ap.add_argument("--layers", type=int, default=L)
+    ap.add_argument("--bits", type=int, default=3, choices=(3, 4),
+                    help="affine code width of the decode_step workload")
     ap.add_argument("--chunk", type=int, default=512, help="positions per chunk (prefill workload)")
     ap.add_argument("--ramp-seconds", type=float, default=0.5,
                     help="untimed busy period before the warmup steps (clock ramp)")
