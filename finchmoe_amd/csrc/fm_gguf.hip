@@ -13,6 +13,10 @@
 //         per 128-value half: q = (ql nibble | qh 2 bits << 4) - 32,
 //         y = d*sc[v/16]*q
 //
+// Two sets of kernels.  Shapes with 4, 8 or 16 lanes per row take the streaming
+// kernels further down (LDS ring + matrix cores); every other shape, and the
+// single matvec, take the plain kernels described next.
+//
 // Lane map.  A lane owns one 128-value HALF block of one row (its 128
 // activations live in registers), LPR = in_dim/128 adjacent lanes share a row,
 // a wave step covers 64/LPR consecutive rows.  Per row the lane contributes
@@ -26,7 +30,10 @@
 // Q6_K blocks are only 2-byte aligned (210 = 2 mod 4).  The loads below are
 // plain multi-dword loads at that alignment, which gfx950 serves in its
 // unaligned-access mode.
-#include "fm_unpack.h"
+#include "fm_mfma.h"
+#include "fm_ring.h"
+
+#include <stdlib.h>
 
 namespace {
 
@@ -397,6 +404,437 @@ __global__ __launch_bounds__(256) void fm_gguf_matvec_k(const uint8_t *W, const 
     if (lane == 0) out[row] = acc;
 }
 
+// ---------------------------------------------------------------- streaming kernels
+// The large launches take the form of the affine decode kernels: one workgroup of
+// eight waves per CU, each wave keeps a ring of slices in LDS filled by LDS-direct
+// loads (a slice = the rows of one wave step exactly as they lie in memory, block
+// headers included), units are claimed from a counter in LDS, and the multiply
+// runs on the matrix cores with the codes placed in bf16 mantissas (fm_mfma.h).
+//
+// Lane map of a wave step: lane = 4*chunk + row-in-quad as in fm_mfma.h, with
+//   Q4_K  chunk = one 128-value half block          (LPR = in_dim / 128)
+//   Q6_K  chunk = 64 values: side sd of half hf of a block, i.e. ql bytes
+//         [64 hf + 32 sd, +32) — their low nibbles are values 32 sd + v and their
+//         high nibbles values 64 + 32 sd + v of the half, v < 32 — with bits
+//         2 sd.. and 2 sd + 4.. of qh bytes [32 hf, +32)      (LPR = in_dim / 64)
+// so a slice is 4608 B (Q4_K) or 3360 B (Q6_K) whatever the row length.
+//
+// Codes in mantissas.  Q4_K: (w >> 4k) & 0x000F000F, k = 0..3, is the pair of
+// nibbles (k, k + 4) of a word; nibbles of equal parity belong to one sub-block,
+// so pairs k = 0, 2 feed the accumulator of the even sub-block and k = 1, 3 the
+// odd one.  Q6_K: the four 6-bit codes of a ql word are assembled one per byte as
+// in the scalar kernel, then (q & 0x003F003F) and ((q >> 8) & 0x003F003F) are the
+// pairs of bytes (0, 2) and (1, 3).  OR-ed with 0x3F803F80 each half reads as
+// 1 + q / 128; the activation registers hold 128 x split into three bf16 pieces
+// and the accumulator starts at -128 sum(x) (-160 sum(x) for Q6_K, whose codes
+// are offset by 32), so that it ends as sum(q x) resp. sum((q - 32) x) exactly
+// as in the affine kernels.
+//
+// Register r of a chunk (both formats) pairs local values
+//   lo(r) = 32 (r / 16) + 4 ((r % 16) / 2) + r % 2   and   hi(r) = lo(r) + 2,
+// accumulator group = r / 16 (Q4_K sub-block of 32) or r / 8 (Q6_K scale group of 16).
+enum { GG_Q4 = 0, GG_Q6 = 1 };
+
+template <int KIND, int LPR>
+struct GgLane;
+template <int LPR>
+struct GgLane<GG_Q4, LPR> {
+    static constexpr int NREG = 64, GROUP_REGS = 16;
+    static constexpr int ROW_BYTES = (LPR / 2) * 144;
+    static constexpr int SLOT_DATA = (FM_WAVE / LPR) * ROW_BYTES;      // 4608
+    __device__ static int col(int c, int v) { return 128 * c + v; }
+};
+template <int LPR>
+struct GgLane<GG_Q6, LPR> {
+    static constexpr int NREG = 32, GROUP_REGS = 8;
+    static constexpr int ROW_BYTES = (LPR / 4) * 210;
+    static constexpr int SLOT_DATA = (FM_WAVE / LPR) * ROW_BYTES;      // 3360
+    __device__ static int col(int c, int v) { return 128 * (c >> 1) + 32 * (c & 1) + (v < 32 ? v : v + 32); }
+};
+
+template <int KIND, bool GU>
+struct GgRing {
+    static constexpr int value = KIND == GG_Q6 ? 5 : 3;
+};
+
+// activation image of one input vector: register quad q of entry e = 4*chunk + piece,
+// and the plain sums of x over the four accumulator groups of each chunk
+template <int NREG, int LPR>
+struct GgImage {
+    uint4 a[NREG / 4][4 * LPR];
+    float4 sum[LPR];
+};
+template <int NREG>
+struct GgAct {
+    uint32_t a[NREG];
+    float xsum[4];
+};
+
+template <int KIND, int LPR>
+__device__ __forceinline__ void gg_build_image(const float *x, GgImage<GgLane<KIND, LPR>::NREG, LPR> &L) {
+    using G = GgLane<KIND, LPR>;
+    constexpr int NE = 4 * LPR;
+    uint32_t *flat = reinterpret_cast<uint32_t *>(L.a);
+    for (int it = threadIdx.x; it < LPR * G::NREG; it += blockDim.x) {
+        const int ch = it / G::NREG, r = it % G::NREG;
+        const int lo = 32 * (r >> 4) + 4 * ((r & 15) >> 1) + (r & 1);
+        const float xl = x[G::col(ch, lo)], xh = x[G::col(ch, lo + 2)];
+        const float vl = xl * 128.0f, vh = xh * 128.0f;
+        uint32_t l0 = __float_as_uint(vl) & 0xFFFF0000u, h0 = __float_as_uint(vh) & 0xFFFF0000u;
+        float rl = vl - __uint_as_float(l0), rh = vh - __uint_as_float(h0);
+        uint32_t l1 = __float_as_uint(rl) & 0xFFFF0000u, h1 = __float_as_uint(rh) & 0xFFFF0000u;
+        rl -= __uint_as_float(l1);
+        rh -= __uint_as_float(h1);
+        uint32_t l2 = __float_as_uint(rl), h2 = __float_as_uint(rh) & 0xFFFF0000u;
+        uint32_t *dst = flat + ((r >> 2) * NE + 4 * ch) * 4 + (r & 3);
+        dst[0] = (l0 >> 16) | h0;
+        dst[4] = (l1 >> 16) | h1;
+        dst[8] = (l2 >> 16) | h2;
+        dst[12] = 0u;
+        const float gs = fm_group_sum<G::GROUP_REGS>(xl + xh);
+        if (r % G::GROUP_REGS == 0) reinterpret_cast<float *>(&L.sum[ch])[r / G::GROUP_REGS] = gs;
+    }
+}
+
+// a lane's activation registers out of an image, while LDS-direct loads are in flight
+// (explicit reads: see fm_ring.h)
+template <int NREG>
+__device__ __forceinline__ void gg_read_image(uint32_t img_addr, int n_entries, int lane, GgAct<NREG> &ar) {
+    const int e = lane % n_entries;
+    uint32_t addr = img_addr + (uint32_t)e * 16u;
+    const uint32_t stride = (uint32_t)n_entries * 16u;
+#pragma unroll
+    for (int q = 0; q < NREG / 4; q++) {
+        fm_u4 v;
+        asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
+        ar.a[4 * q + 0] = v[0];
+        ar.a[4 * q + 1] = v[1];
+        ar.a[4 * q + 2] = v[2];
+        ar.a[4 * q + 3] = v[3];
+        addr += stride;
+    }
+    fm_u4 sm;
+    const uint32_t sa = img_addr + (uint32_t)(NREG / 4) * stride + (uint32_t)(e >> 2) * 16u;
+    asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(sm) : "v"(sa) : "memory");
+#pragma unroll
+    for (int g = 0; g < 4; g++) ar.xsum[g] = __uint_as_float(sm[g]);
+}
+
+__device__ __forceinline__ fm_f4 gg_mfma(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, fm_f4 acc) {
+    fm_s4 av = __builtin_bit_cast(fm_s4, make_uint2(a0, a1));
+    fm_s4 bv = __builtin_bit_cast(fm_s4, make_uint2(b0, b1));
+    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(av, bv, acc, 0, 0, 0);
+}
+
+// ---- Q4_K lane: header + 64 bytes of nibbles out of a landed slice
+struct GgQ4Lane {
+    uint32_t hdr_off, q_off;
+    int half;
+    template <int LPR>
+    __device__ __forceinline__ void init(int row_in_step, int ch) {
+        hdr_off = (uint32_t)(row_in_step * GgLane<GG_Q4, LPR>::ROW_BYTES + (ch >> 1) * 144);
+        half = ch & 1;
+        q_off = hdr_off + 16u + 64u * (uint32_t)half;
+    }
+    __device__ __forceinline__ uint32_t read(uint32_t slot, uint32_t tag_addr, Q4Half &t) const {
+        const uint32_t ah = slot + hdr_off, aq = slot + q_off;
+        uint32_t tag;
+        asm volatile("ds_read_b128 %0, %6\n\tds_read_b128 %1, %7\n\tds_read_b128 %2, %7 offset:16\n\t"
+                     "ds_read_b128 %3, %7 offset:32\n\tds_read_b128 %4, %7 offset:48\n\t"
+                     "ds_read_b32 %5, %8\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(t.hdr), "=&v"(t.q[0]), "=&v"(t.q[1]), "=&v"(t.q[2]), "=&v"(t.q[3]),
+                       "=&v"(tag)
+                     : "v"(ah), "v"(aq), "v"(tag_addr)
+                     : "memory");
+        return __builtin_amdgcn_readfirstlane(tag);
+    }
+    __device__ __forceinline__ float dot(const Q4Half &t, const GgAct<64> &ar, uint32_t ones) const {
+        const float d = f16bits(t.hdr[0]), dmin = f16bits(t.hdr[0] >> 16);
+        const uint32_t *qd = reinterpret_cast<const uint32_t *>(t.q);
+        float r = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            fm_f4 ae = {-128.0f * ar.xsum[2 * c], 0.0f, 0.0f, 0.0f};
+            fm_f4 ao = {-128.0f * ar.xsum[2 * c + 1], 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const uint32_t w = qd[8 * c + k];
+                const uint32_t p0 = (w & 0x000F000Fu) | ones, p1 = ((w >> 4) & 0x000F000Fu) | ones;
+                const uint32_t p2 = ((w >> 8) & 0x000F000Fu) | ones, p3 = ((w >> 12) & 0x000F000Fu) | ones;
+                const uint32_t *ap = ar.a + 32 * c + 2 * k;
+                ae = gg_mfma(ap[0], ap[1], p0, p2, ae);
+                ao = gg_mfma(ap[16], ap[17], p1, p3, ao);
+            }
+            float sc, mn;
+            q4_scale_min(t.hdr, half, 2 * c, sc, mn);
+            r = fmaf(d * sc, (ae[0] + ae[1]) + ae[2], r);
+            r = fmaf(-(dmin * mn), ar.xsum[2 * c], r);
+            q4_scale_min(t.hdr, half, 2 * c + 1, sc, mn);
+            r = fmaf(d * sc, (ao[0] + ao[1]) + ao[2], r);
+            r = fmaf(-(dmin * mn), ar.xsum[2 * c + 1], r);
+        }
+        return r;
+    }
+};
+
+// ---- Q6_K lane: 32 ql bytes, 32 qh bytes, four scales and d.  Blocks are only 2-byte
+// aligned, so the words are read at the 4-byte boundary below and funnel-shifted; the
+// same shift drops the lane's side bits of qh.
+struct GgQ6Data {
+    uint32_t ql[9], qh[9], sc_a, sc_b, d;
+};
+struct GgQ6Lane {
+    uint32_t ql_off, qh_off, sc_off, d_off, sh_l, sh_h;
+    template <int LPR>
+    __device__ __forceinline__ void init(int row_in_step, int ch) {
+        const int hf = (ch >> 1) & 1, sd = ch & 1;
+        const uint32_t blk = (uint32_t)(row_in_step * GgLane<GG_Q6, LPR>::ROW_BYTES + (ch >> 2) * 210);
+        const uint32_t ql = blk + 64u * hf + 32u * sd, qh = blk + 128u + 32u * hf;
+        ql_off = ql & ~3u;
+        qh_off = qh & ~3u;
+        sh_l = (ql & 3u) * 8u;
+        sh_h = (qh & 3u) * 8u + 2u * sd;
+        sc_off = blk + 192u + 8u * hf + 2u * sd;
+        d_off = blk + 208u;
+    }
+    __device__ __forceinline__ uint32_t read(uint32_t slot, uint32_t tag_addr, GgQ6Data &t) const {
+        const uint32_t al = slot + ql_off, ah = slot + qh_off, as = slot + sc_off, ad = slot + d_off;
+        u32x2 l0, l1, l2, l3, h0, h1, h2, h3;
+        uint32_t tag;
+        asm volatile("ds_read2_b32 %0, %14 offset1:1\n\tds_read2_b32 %1, %14 offset0:2 offset1:3\n\t"
+                     "ds_read2_b32 %2, %14 offset0:4 offset1:5\n\tds_read2_b32 %3, %14 offset0:6 offset1:7\n\t"
+                     "ds_read_b32 %4, %14 offset:32\n\t"
+                     "ds_read2_b32 %5, %15 offset1:1\n\tds_read2_b32 %6, %15 offset0:2 offset1:3\n\t"
+                     "ds_read2_b32 %7, %15 offset0:4 offset1:5\n\tds_read2_b32 %8, %15 offset0:6 offset1:7\n\t"
+                     "ds_read_b32 %9, %15 offset:32\n\t"
+                     "ds_read_u16 %10, %16\n\tds_read_u16 %11, %16 offset:4\n\tds_read_u16 %12, %17\n\t"
+                     "ds_read_b32 %13, %18\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(l0), "=&v"(l1), "=&v"(l2), "=&v"(l3), "=&v"(t.ql[8]), "=&v"(h0), "=&v"(h1),
+                       "=&v"(h2), "=&v"(h3), "=&v"(t.qh[8]), "=&v"(t.sc_a), "=&v"(t.sc_b), "=&v"(t.d),
+                       "=&v"(tag)
+                     : "v"(al), "v"(ah), "v"(as), "v"(ad), "v"(tag_addr)
+                     : "memory");
+        t.ql[0] = l0[0], t.ql[1] = l0[1], t.ql[2] = l1[0], t.ql[3] = l1[1];
+        t.ql[4] = l2[0], t.ql[5] = l2[1], t.ql[6] = l3[0], t.ql[7] = l3[1];
+        t.qh[0] = h0[0], t.qh[1] = h0[1], t.qh[2] = h1[0], t.qh[3] = h1[1];
+        t.qh[4] = h2[0], t.qh[5] = h2[1], t.qh[6] = h3[0], t.qh[7] = h3[1];
+        return __builtin_amdgcn_readfirstlane(tag);
+    }
+    __device__ __forceinline__ float dot(const GgQ6Data &t, const GgAct<32> &ar, uint32_t ones) const {
+        fm_f4 acc[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) acc[g] = {-160.0f * ar.xsum[g], 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint32_t a = __builtin_amdgcn_alignbit(t.ql[i + 1], t.ql[i], sh_l);
+            // bits 30, 31 may hold the next byte's: no mask below looks at them
+            const uint32_t h = __builtin_amdgcn_alignbit(t.qh[i + 1], t.qh[i], sh_h);
+            const uint32_t qa = ((h << 4) & 0x30303030u) | (a & 0x0F0F0F0Fu);
+            const uint32_t qb = (h & 0x30303030u) | ((a >> 4) & 0x0F0F0F0Fu);
+            const uint32_t pa0 = (qa & 0x003F003Fu) | ones, pa1 = ((qa >> 8) & 0x003F003Fu) | ones;
+            const uint32_t pb0 = (qb & 0x003F003Fu) | ones, pb1 = ((qb >> 8) & 0x003F003Fu) | ones;
+            acc[i >> 2] = gg_mfma(ar.a[2 * i], ar.a[2 * i + 1], pa0, pa1, acc[i >> 2]);
+            acc[2 + (i >> 2)] = gg_mfma(ar.a[16 + 2 * i], ar.a[17 + 2 * i], pb0, pb1, acc[2 + (i >> 2)]);
+        }
+        const float s0 = (float)(int)(int8_t)(t.sc_a & 0xFFu), s1 = (float)(int)(int8_t)(t.sc_a >> 8);
+        const float s2 = (float)(int)(int8_t)(t.sc_b & 0xFFu), s3 = (float)(int)(int8_t)(t.sc_b >> 8);
+        float r = s0 * ((acc[0][0] + acc[0][1]) + acc[0][2]);
+        r = fmaf(s1, (acc[1][0] + acc[1][1]) + acc[1][2], r);
+        r = fmaf(s2, (acc[2][0] + acc[2][1]) + acc[2][2], r);
+        r = fmaf(s3, (acc[3][0] + acc[3][1]) + acc[3][2], r);
+        return f16bits(t.d) * r;
+    }
+};
+
+// BYTES of a slice, 16 per lane and load; the last load is partial.  The
+// instruction offset moves the global and the LDS address alike.
+template <int BYTES, int I>
+__device__ __forceinline__ void gg_dma(uint32_t slot, const uint8_t *src, int lane) {
+    if constexpr (I * 1024 < BYTES) {
+        // (the offset field holds -4096..4095: from the fifth load on it starts again from
+        // addresses moved by 4096)
+        constexpr int BASE = (I / 4) * 4096, IMM = (I % 4) * 1024;
+        if (I * 1024 + lane * 16 < BYTES)
+            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(src + BASE),
+                                             (fm_lptr)(uintptr_t)(slot + BASE), 16, IMM, 0);
+        gg_dma<BYTES, I + 1>(slot, src, lane);
+    }
+}
+
+template <int KIND> struct GgLaneOps;
+template <> struct GgLaneOps<GG_Q4> { using Lane = GgQ4Lane; using Data = Q4Half; };
+template <> struct GgLaneOps<GG_Q6> { using Lane = GgQ6Lane; using Data = GgQ6Data; };
+
+template <int KIND, int LPR, bool GU>
+constexpr size_t gg_stream_lds() {
+    using G = GgLane<KIND, LPR>;
+    return (size_t)8 * GgRing<KIND, GU>::value * (G::SLOT_DATA + 16) +
+           (GU ? 2 : 3) * sizeof(GgImage<G::NREG, LPR>);
+}
+
+extern __shared__ __attribute__((aligned(16))) uint8_t fm_gguf_lds[];
+
+// GU: gate and up rows (both Q4_K) of a unit, SwiGLU -> act.  Otherwise: down rows -> expert_out.
+// upp = units (wave steps) per pair; units of the launch are numbered pair-major.
+template <int KIND, int LPR, bool GU>
+__global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_units, int upp) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    using G = GgLane<KIND, LPR>;
+    using Lane = typename GgLaneOps<KIND>::Lane;
+    using Data = typename GgLaneOps<KIND>::Data;
+    using Image = GgImage<G::NREG, LPR>;
+    constexpr int RPS = FM_WAVE / LPR, NS = GU ? 2 : 1, NIMG = GU ? 2 : 3;
+    constexpr int RING = GgRing<KIND, GU>::value;
+    constexpr int SLOT = G::SLOT_DATA + 16, TAG = G::SLOT_DATA, LOADS = (G::SLOT_DATA + 1023) / 1024;
+    __shared__ unsigned int next_unit;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t ring0 = fm_lds_addr(fm_gguf_lds) + (uint32_t)wave * (RING * SLOT);
+    Image *img = reinterpret_cast<Image *>(fm_gguf_lds + 8 * RING * SLOT);
+    const uint32_t img0 = fm_lds_addr(img);
+    const long wg0 = (long)total_units * blockIdx.x / gridDim.x,
+               wg1 = (long)total_units * (blockIdx.x + 1) / gridDim.x;
+    const uint32_t n_units = (uint32_t)(wg1 - wg0);
+    if (n_units == 0) return;
+    if (threadIdx.x == 0) next_unit = 0u;
+    __syncthreads();
+    const int in_dim = GU ? a.g.hidden : a.g.inter;
+    const int upv = GU ? upp * a.K : upp;              // units per input vector
+    const int vid0 = (int)(wg0 / upv), n_img = (int)((wg1 - 1) / upv) - vid0 + 1;
+    const float *xbase = GU ? a.x : a.act;
+
+    const int j = lane & 3, ch = (lane >> 2) % LPR, ris = 4 * (lane / (4 * LPR)) + j;
+    Lane ln;
+    ln.template init<LPR>(ris, ch);
+
+    // ---- loader
+    int kn = 0, wpos = 0;
+    uint32_t issued = 0, consumed = 0, tag_n = 0;
+    const uint8_t *p0 = nullptr;
+    ptrdiff_t p_second = 0;
+    bool dry = false;
+    auto issue = [&]() __attribute__((always_inline)) {
+        if (dry) return;
+        if (kn == 0) {
+            const uint32_t ul = fm_claim_unit(&next_unit, lane);
+            if (ul >= n_units) {
+                dry = true;
+                return;
+            }
+            const uint32_t u = (uint32_t)wg0 + ul;
+            const uint32_t pair = u / (uint32_t)upp, step = u - pair * (uint32_t)upp;
+            int e = a.idx[pair];
+            const bool ok = (unsigned)e < (unsigned)a.g.n_experts;
+            if (!ok) e = 0;                              // stream something valid, store zeros
+            const int li = a.layer0 + (int)(pair / (uint32_t)a.K) * a.layer_stride;
+            const size_t so = (size_t)step * G::SLOT_DATA;
+            if constexpr (GU) {
+                const uint8_t *g = a.gate[li] + (size_t)e * a.g.gate_slab + so;
+                const uint8_t *up = a.up[li] + (size_t)e * a.g.up_slab + so;
+                p0 = fm_uniform(g);
+                p_second = fm_uniform(up) - p0;
+            } else {
+                p0 = fm_uniform(a.down[li] + (size_t)e * a.g.down_slab + so);
+            }
+            tag_n = ul | (ok ? 0u : 0x80000000u);
+        }
+        const uint32_t slot = ring0 + (uint32_t)wpos * SLOT;
+        fm_slot_tag(slot + TAG, tag_n);
+        const uint8_t *src = p0 + (ptrdiff_t)kn * p_second + lane * 16;
+        gg_dma<G::SLOT_DATA, 0>(slot, src, lane);
+        kn = kn + 1 == NS ? 0 : kn + 1;
+        wpos = wpos + 1 == RING ? 0 : wpos + 1;
+        issued++;
+    };
+#pragma unroll
+    for (int k = 0; k < RING; k++) issue();
+
+    // the images of every input vector this workgroup's units touch
+    for (int v = 0; v < n_img && v < NIMG; v++)
+        gg_build_image<KIND, LPR>(xbase + (size_t)(vid0 + v) * in_dim, img[v]);
+    __syncthreads();
+
+    GgAct<G::NREG> ar;
+    int cur_v = -1;
+    const uint32_t ones = fm_opaque(0x3F803F80u);
+    int c = 0;
+    while (consumed < issued) {
+        float v[NS];
+        uint32_t tag = 0;
+#pragma unroll
+        for (int k = 0; k < NS; k++) {
+            Data t;
+            if (issued - consumed == (uint32_t)RING) fm_dma_wait<LOADS *(RING - 1)>(false);
+            else fm_dma_wait<0>(true);
+            const uint32_t slot = ring0 + (uint32_t)c * SLOT;
+            tag = ln.read(slot, slot + TAG, t);
+            consumed++;
+            c = c + 1 == RING ? 0 : c + 1;
+            issue();
+            if (k == 0) {
+                const int vid = (int)(((uint32_t)wg0 + (tag & 0x7FFFFFFFu)) / (uint32_t)upv);
+                if (vid != cur_v) {
+                    gg_read_image<G::NREG>(img0 + (uint32_t)(vid - vid0) * (uint32_t)sizeof(Image), 4 * LPR,
+                                           lane, ar);
+                    cur_v = vid;
+                }
+            }
+            v[k] = fm_chunk_sum<LPR>(ln.dot(t, ar, ones));
+        }
+        const uint32_t u = (uint32_t)wg0 + (tag & 0x7FFFFFFFu);
+        const uint32_t pair = u / (uint32_t)upp, step = u - pair * (uint32_t)upp;
+        const bool ok = !(tag >> 31);
+        if (ch == 0) {
+            if constexpr (GU)
+                a.act[(size_t)pair * a.g.inter + step * RPS + ris] = ok ? fm_silu_mul(v[0], v[NS - 1]) : 0.0f;
+            else
+                a.expert_out[(size_t)pair * a.g.hidden + step * RPS + ris] = ok ? v[0] : 0.0f;
+        }
+    }
+#else
+    (void)a;
+    (void)total_units;
+    (void)upp;
+#endif
+}
+
+// launch of one streaming phase; FM_ERR_UNSUPPORTED when the shape has no instance
+template <int KIND, bool GU>
+int gg_launch_stream(const GgufArgs &a, int n_pairs, int n_cu, hipStream_t st) {
+    const int in_dim = GU ? a.g.hidden : a.g.inter, rows = GU ? a.g.inter : a.g.hidden;
+    const int per_lane = KIND == GG_Q6 ? 64 : 128;
+    const int lpr = in_dim / per_lane;
+    if (in_dim % per_lane || !(lpr == 4 || lpr == 8 || lpr == 16)) return FM_ERR_UNSUPPORTED;
+    const int rps = FM_WAVE / lpr;
+    if (rows % rps) return FM_ERR_UNSUPPORTED;
+    const int upp = rows / rps;
+    const long total = (long)n_pairs * upp;
+    if (total >= (1L << 31)) return FM_ERR_UNSUPPORTED;
+    // a workgroup holds the images of 2 layers (gate/up) or 3 pairs (down): keep its share
+    // of the units within that span
+    const long upv = GU ? (long)upp * a.K : upp, max_share = upv * ((GU ? 2 : 3) - 1);
+    long wgs = n_cu;
+    if (total < 8 * wgs) wgs = (total + 7) / 8;
+    if ((total + wgs - 1) / wgs > max_share) wgs = (total + max_share - 1) / max_share;
+    // every share must be <= max_share: shares differ by at most one unit
+    while (wgs < total && (total + wgs - 1) / wgs > max_share) wgs++;
+#define GG_ST(L)                                                                               \
+    do {                                                                                       \
+        auto kfn = fm_gguf_stream<KIND, L, GU>;                                                \
+        const size_t sh = gg_stream_lds<KIND, L, GU>();                                        \
+        static FmLdsAttr attr;                                                                 \
+        if (!fm_dyn_lds_ready(attr, (const void *)kfn, sh)) return FM_ERR_HIP;                 \
+        hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(512), sh, st, a, (int)total, upp);   \
+    } while (0)
+    switch (lpr) {
+        case 4: GG_ST(4); break;
+        case 8: GG_ST(8); break;
+        default: GG_ST(16); break;
+    }
+#undef GG_ST
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
+
 int pick_rpi(int rows, int n_pairs, int min_rows, int cap, int want) {
     int rpi = min_rows;
     while (rpi * 2 <= cap && rows % (rpi * 2) == 0 && (rows / (rpi * 2)) * n_pairs >= want) rpi *= 2;
@@ -440,8 +878,12 @@ extern "C" int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t
     a2.rows_per_item = pick_rpi(g->hidden, n_pairs, min_down, 256, 4 * n_cu);
     a2.items_per_pair = g->hidden / a2.rows_per_item;
     if (kev) (void)hipEventRecord(kev[0], st);
+    static const bool no_stream = getenv("FINCH_GGUF_VALU") != nullptr;
+    int rc_up = FM_ERR_UNSUPPORTED;
+    if (!no_stream) rc_up = gg_launch_stream<GG_Q4, true>(a, n_pairs, n_cu, st);
+    if (rc_up != FM_OK && rc_up != FM_ERR_UNSUPPORTED) return rc_up;
 #define GG_UP(L) hipLaunchKernelGGL(fm_gguf_gate_up<L>, dim3(n_pairs * a1.items_per_pair), b, 0, st, a1)
-    switch (lpr_up) {
+    if (rc_up == FM_ERR_UNSUPPORTED) switch (lpr_up) {
         case 2: GG_UP(2); break;
         case 4: GG_UP(4); break;
         case 8: GG_UP(8); break;
@@ -457,7 +899,11 @@ extern "C" int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t
         if (q6) hipLaunchKernelGGL((fm_gguf_down<L, true>), dim3(n_pairs * a2.items_per_pair), b, 0, st, a2); \
         else hipLaunchKernelGGL((fm_gguf_down<L, false>), dim3(n_pairs * a2.items_per_pair), b, 0, st, a2);   \
     } while (0)
-    switch (lpr_down) {
+    int rc_dn = FM_ERR_UNSUPPORTED;
+    if (!no_stream) rc_dn = q6 ? gg_launch_stream<GG_Q6, false>(a, n_pairs, n_cu, st)
+                               : gg_launch_stream<GG_Q4, false>(a, n_pairs, n_cu, st);
+    if (rc_dn != FM_OK && rc_dn != FM_ERR_UNSUPPORTED) return rc_dn;
+    if (rc_dn == FM_ERR_UNSUPPORTED) switch (lpr_down) {
         case 2: GG_DOWN(2); break;
         case 4: GG_DOWN(4); break;
         case 8: GG_DOWN(8); break;
