@@ -536,22 +536,29 @@ struct GgQ4Lane {
         half = ch & 1;
         q_off = hdr_off + 16u + 64u * (uint32_t)half;
     }
-    __device__ __forceinline__ uint32_t read(uint32_t slot, uint32_t tag_addr, Q4Half &t) const {
+    __device__ __forceinline__ fm_u4 read(uint32_t slot, uint32_t tag_addr, Q4Half &t) const {
         const uint32_t ah = slot + hdr_off, aq = slot + q_off;
-        uint32_t tag;
+        fm_u4 tag;
         asm volatile("ds_read_b128 %0, %6\n\tds_read_b128 %1, %7\n\tds_read_b128 %2, %7 offset:16\n\t"
                      "ds_read_b128 %3, %7 offset:32\n\tds_read_b128 %4, %7 offset:48\n\t"
-                     "ds_read_b32 %5, %8\n\ts_waitcnt lgkmcnt(0)"
+                     "ds_read_b128 %5, %8\n\ts_waitcnt lgkmcnt(0)"
                      : "=&v"(t.hdr), "=&v"(t.q[0]), "=&v"(t.q[1]), "=&v"(t.q[2]), "=&v"(t.q[3]),
                        "=&v"(tag)
                      : "v"(ah), "v"(aq), "v"(tag_addr)
                      : "memory");
-        return __builtin_amdgcn_readfirstlane(tag);
+        return tag;
     }
     __device__ __forceinline__ float dot(const Q4Half &t, const GgAct<64> &ar, uint32_t ones) const {
         const float d = f16bits(t.hdr[0]), dmin = f16bits(t.hdr[0] >> 16);
         const uint32_t *qd = reinterpret_cast<const uint32_t *>(t.q);
-        float r = 0.0f;
+        // the four (scale, min) pairs of this half, one per byte (finchmoe/infer.m:1595-1603)
+        const uint32_t s0 = t.hdr[1], s1 = t.hdr[2], s2 = t.hdr[3];
+        const uint32_t sc4 = half ? (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u) : s0 & 0x3F3F3F3Fu;
+        const uint32_t mn4 = half ? ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u)
+                                  : s1 & 0x3F3F3F3Fu;
+        const float sc[4] = {fm_ubyte<0>(sc4), fm_ubyte<1>(sc4), fm_ubyte<2>(sc4), fm_ubyte<3>(sc4)};
+        const float mn[4] = {fm_ubyte<0>(mn4), fm_ubyte<1>(mn4), fm_ubyte<2>(mn4), fm_ubyte<3>(mn4)};
+        float r = 0.0f, rm = 0.0f;
 #pragma unroll
         for (int c = 0; c < 2; c++) {
             fm_f4 ae = {-128.0f * ar.xsum[2 * c], 0.0f, 0.0f, 0.0f};
@@ -565,15 +572,12 @@ struct GgQ4Lane {
                 ae = gg_mfma(ap[0], ap[1], p0, p2, ae);
                 ao = gg_mfma(ap[16], ap[17], p1, p3, ao);
             }
-            float sc, mn;
-            q4_scale_min(t.hdr, half, 2 * c, sc, mn);
-            r = fmaf(d * sc, (ae[0] + ae[1]) + ae[2], r);
-            r = fmaf(-(dmin * mn), ar.xsum[2 * c], r);
-            q4_scale_min(t.hdr, half, 2 * c + 1, sc, mn);
-            r = fmaf(d * sc, (ao[0] + ao[1]) + ao[2], r);
-            r = fmaf(-(dmin * mn), ar.xsum[2 * c + 1], r);
+            r = fmaf(sc[2 * c], (ae[0] + ae[1]) + ae[2], r);
+            rm = fmaf(mn[2 * c], ar.xsum[2 * c], rm);
+            r = fmaf(sc[2 * c + 1], (ao[0] + ao[1]) + ao[2], r);
+            rm = fmaf(mn[2 * c + 1], ar.xsum[2 * c + 1], rm);
         }
-        return r;
+        return d * r - dmin * rm;
     }
 };
 
@@ -597,10 +601,10 @@ struct GgQ6Lane {
         sc_off = blk + 192u + 8u * hf + 2u * sd;
         d_off = blk + 208u;
     }
-    __device__ __forceinline__ uint32_t read(uint32_t slot, uint32_t tag_addr, GgQ6Data &t) const {
+    __device__ __forceinline__ fm_u4 read(uint32_t slot, uint32_t tag_addr, GgQ6Data &t) const {
         const uint32_t al = slot + ql_off, ah = slot + qh_off, as = slot + sc_off, ad = slot + d_off;
         u32x2 l0, l1, l2, l3, h0, h1, h2, h3;
-        uint32_t tag;
+        fm_u4 tag;
         asm volatile("ds_read2_b32 %0, %14 offset1:1\n\tds_read2_b32 %1, %14 offset0:2 offset1:3\n\t"
                      "ds_read2_b32 %2, %14 offset0:4 offset1:5\n\tds_read2_b32 %3, %14 offset0:6 offset1:7\n\t"
                      "ds_read_b32 %4, %14 offset:32\n\t"
@@ -608,7 +612,7 @@ struct GgQ6Lane {
                      "ds_read2_b32 %7, %15 offset0:4 offset1:5\n\tds_read2_b32 %8, %15 offset0:6 offset1:7\n\t"
                      "ds_read_b32 %9, %15 offset:32\n\t"
                      "ds_read_u16 %10, %16\n\tds_read_u16 %11, %16 offset:4\n\tds_read_u16 %12, %17\n\t"
-                     "ds_read_b32 %13, %18\n\ts_waitcnt lgkmcnt(0)"
+                     "ds_read_b128 %13, %18\n\ts_waitcnt lgkmcnt(0)"
                      : "=&v"(l0), "=&v"(l1), "=&v"(l2), "=&v"(l3), "=&v"(t.ql[8]), "=&v"(h0), "=&v"(h1),
                        "=&v"(h2), "=&v"(h3), "=&v"(t.qh[8]), "=&v"(t.sc_a), "=&v"(t.sc_b), "=&v"(t.d),
                        "=&v"(tag)
@@ -618,7 +622,7 @@ struct GgQ6Lane {
         t.ql[4] = l2[0], t.ql[5] = l2[1], t.ql[6] = l3[0], t.ql[7] = l3[1];
         t.qh[0] = h0[0], t.qh[1] = h0[1], t.qh[2] = h1[0], t.qh[3] = h1[1];
         t.qh[4] = h2[0], t.qh[5] = h2[1], t.qh[6] = h3[0], t.qh[7] = h3[1];
-        return __builtin_amdgcn_readfirstlane(tag);
+        return tag;
     }
     __device__ __forceinline__ float dot(const GgQ6Data &t, const GgAct<32> &ar, uint32_t ones) const {
         fm_f4 acc[4];
@@ -674,10 +678,45 @@ constexpr size_t gg_stream_lds() {
 
 extern __shared__ __attribute__((aligned(16))) uint8_t fm_gguf_lds[];
 
+// u / d for u < 2^31 without the division sequence: with l = ceil(log2 d),
+// mul = ceil(2^(31 + l) / d) fits 32 bits and floor(u * mul / 2^(31 + l)) is exact.
+struct GgDiv {
+    uint32_t mul, shift, d;
+    __device__ __forceinline__ uint32_t operator()(uint32_t u) const {
+        return d == 1u ? u : __umulhi(u, mul) >> shift;
+    }
+};
+inline GgDiv gg_div_make(uint32_t d) {
+    GgDiv r{0u, 0u, d};
+    if (d > 1u) {
+        uint32_t l = 0;
+        while ((1ull << l) < d) l++;
+        r.mul = (uint32_t)(((1ull << (31 + l)) + d - 1) / d);
+        r.shift = l - 1;
+    }
+    return r;
+}
+
+// Where the rows of a pair's expert start, looked up once per workgroup: a global
+// (scalar) load per claimed unit would stall its wave for a memory round trip
+// behind the weight stream.
+struct __attribute__((aligned(16))) GgPairEntry {
+    uint64_t first;        // gate (or down) rows of the expert
+    int64_t second;        // up rows - gate rows
+    uint32_t invalid, pad[3];
+};
+
+// what a slice's trailer says about its unit
+struct GgUnit {
+    uint32_t flags, pair, step, image;     // flags bit 0: the pair's expert index is invalid
+};
+
 // GU: gate and up rows (both Q4_K) of a unit, SwiGLU -> act.  Otherwise: down rows -> expert_out.
-// upp = units (wave steps) per pair; units of the launch are numbered pair-major.
+// Units (wave steps) of the launch are numbered pair-major, by_upp divides by the units per pair,
+// by_k by K.
 template <int KIND, int LPR, bool GU>
-__global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_units, int upp) {
+__global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_units, GgDiv by_upp,
+                                                      GgDiv by_k) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using G = GgLane<KIND, LPR>;
     using Lane = typename GgLaneOps<KIND>::Lane;
@@ -686,7 +725,10 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
     constexpr int RPS = FM_WAVE / LPR, NS = GU ? 2 : 1, NIMG = GU ? 2 : 3;
     constexpr int RING = GgRing<KIND, GU>::value;
     constexpr int SLOT = G::SLOT_DATA + 16, TAG = G::SLOT_DATA, LOADS = (G::SLOT_DATA + 1023) / 1024;
+    // pairs a workgroup's share can touch: it spans at most NIMG - 1 input vectors' worth
+    constexpr int NPAIR = GU ? FM_MAX_K + 1 : NIMG;
     __shared__ unsigned int next_unit;
+    __shared__ GgPairEntry ptab[NPAIR];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t ring0 = fm_lds_addr(fm_gguf_lds) + (uint32_t)wave * (RING * SLOT);
@@ -696,12 +738,37 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
                wg1 = (long)total_units * (blockIdx.x + 1) / gridDim.x;
     const uint32_t n_units = (uint32_t)(wg1 - wg0);
     if (n_units == 0) return;
-    if (threadIdx.x == 0) next_unit = 0u;
-    __syncthreads();
     const int in_dim = GU ? a.g.hidden : a.g.inter;
-    const int upv = GU ? upp * a.K : upp;              // units per input vector
-    const int vid0 = (int)(wg0 / upv), n_img = (int)((wg1 - 1) / upv) - vid0 + 1;
+    // input vector of a pair: its layer's x (gate/up) or its own act (down)
+    auto vector_of = [&](uint32_t pair) __attribute__((always_inline)) {
+        return GU ? by_k(pair) : pair;
+    };
+    const uint32_t pair0 = by_upp((uint32_t)wg0), pair_last = by_upp((uint32_t)wg1 - 1u);
+    const uint32_t vid0 = vector_of(pair0);
+    const int n_img = (int)(vector_of(pair_last) - vid0) + 1;
     const float *xbase = GU ? a.x : a.act;
+    if (threadIdx.x == 0) next_unit = 0u;
+    if (threadIdx.x <= pair_last - pair0 && threadIdx.x < NPAIR) {
+        const uint32_t pair = pair0 + threadIdx.x;
+        int e = a.idx[pair];
+        const bool ok = (unsigned)e < (unsigned)a.g.n_experts;
+        if (!ok) e = 0;                                  // stream something valid, store zeros
+        const int li = a.layer0 + (int)by_k(pair) * a.layer_stride;
+        GgPairEntry pe;
+        if constexpr (GU) {
+            const uint8_t *g = a.gate[li] + (size_t)e * a.g.gate_slab;
+            pe.first = (uint64_t)(uintptr_t)g;
+            pe.second = (int64_t)((a.up[li] + (size_t)e * a.g.up_slab) - g);
+        } else {
+            pe.first = (uint64_t)(uintptr_t)(a.down[li] + (size_t)e * a.g.down_slab);
+            pe.second = 0;
+        }
+        pe.invalid = ok ? 0u : 1u;
+        pe.pad[0] = pe.pad[1] = pe.pad[2] = 0u;
+        ptab[threadIdx.x] = pe;
+    }
+    __syncthreads();
+    const uint32_t ptab0 = fm_lds_addr(ptab);
 
     const int j = lane & 3, ch = (lane >> 2) % LPR, ris = 4 * (lane / (4 * LPR)) + j;
     Lane ln;
@@ -709,7 +776,8 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
 
     // ---- loader
     int kn = 0, wpos = 0;
-    uint32_t issued = 0, consumed = 0, tag_n = 0;
+    uint32_t issued = 0, consumed = 0;
+    GgUnit un{0u, 0u, 0u, 0u};
     const uint8_t *p0 = nullptr;
     ptrdiff_t p_second = 0;
     bool dry = false;
@@ -722,24 +790,29 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
                 return;
             }
             const uint32_t u = (uint32_t)wg0 + ul;
-            const uint32_t pair = u / (uint32_t)upp, step = u - pair * (uint32_t)upp;
-            int e = a.idx[pair];
-            const bool ok = (unsigned)e < (unsigned)a.g.n_experts;
-            if (!ok) e = 0;                              // stream something valid, store zeros
-            const int li = a.layer0 + (int)(pair / (uint32_t)a.K) * a.layer_stride;
-            const size_t so = (size_t)step * G::SLOT_DATA;
-            if constexpr (GU) {
-                const uint8_t *g = a.gate[li] + (size_t)e * a.g.gate_slab + so;
-                const uint8_t *up = a.up[li] + (size_t)e * a.g.up_slab + so;
-                p0 = fm_uniform(g);
-                p_second = fm_uniform(up) - p0;
-            } else {
-                p0 = fm_uniform(a.down[li] + (size_t)e * a.g.down_slab + so);
-            }
-            tag_n = ul | (ok ? 0u : 0x80000000u);
+            un.pair = by_upp(u);
+            un.step = u - un.pair * by_upp.d;
+            un.image = vector_of(un.pair) - vid0;
+            fm_u4 pe;
+            uint32_t inv;
+            const uint32_t pa = ptab0 + (un.pair - pair0) * (uint32_t)sizeof(GgPairEntry);
+            asm volatile("ds_read_b128 %0, %2\n\tds_read_b32 %1, %2 offset:16\n\ts_waitcnt lgkmcnt(0)"
+                         : "=&v"(pe), "=&v"(inv)
+                         : "v"(pa)
+                         : "memory");
+            un.flags = __builtin_amdgcn_readfirstlane(inv);
+            // (readfirstlane returns int: widen as unsigned)
+            const uint32_t f_lo = __builtin_amdgcn_readfirstlane(pe[0]), f_hi = __builtin_amdgcn_readfirstlane(pe[1]);
+            const uint32_t s_lo = __builtin_amdgcn_readfirstlane(pe[2]), s_hi = __builtin_amdgcn_readfirstlane(pe[3]);
+            p0 = (const uint8_t *)(uintptr_t)(((uint64_t)f_hi << 32) | f_lo) + (size_t)un.step * G::SLOT_DATA;
+            if constexpr (GU) p_second = (ptrdiff_t)(((uint64_t)s_hi << 32) | s_lo);
         }
         const uint32_t slot = ring0 + (uint32_t)wpos * SLOT;
-        fm_slot_tag(slot + TAG, tag_n);
+        {
+            const uint32_t ta = slot + TAG;
+            const fm_u4 tv = {un.flags, un.pair, un.step, un.image};
+            asm volatile("ds_write_b128 %0, %1" ::"v"(ta), "v"(tv) : "memory");
+        }
         const uint8_t *src = p0 + (ptrdiff_t)kn * p_second + lane * 16;
         gg_dma<G::SLOT_DATA, 0>(slot, src, lane);
         kn = kn + 1 == NS ? 0 : kn + 1;
@@ -755,12 +828,12 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
     __syncthreads();
 
     GgAct<G::NREG> ar;
-    int cur_v = -1;
+    uint32_t cur_image = ~0u;
     const uint32_t ones = fm_opaque(0x3F803F80u);
     int c = 0;
     while (consumed < issued) {
         float v[NS];
-        uint32_t tag = 0;
+        fm_u4 tag;
 #pragma unroll
         for (int k = 0; k < NS; k++) {
             Data t;
@@ -772,18 +845,17 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
             c = c + 1 == RING ? 0 : c + 1;
             issue();
             if (k == 0) {
-                const int vid = (int)(((uint32_t)wg0 + (tag & 0x7FFFFFFFu)) / (uint32_t)upv);
-                if (vid != cur_v) {
-                    gg_read_image<G::NREG>(img0 + (uint32_t)(vid - vid0) * (uint32_t)sizeof(Image), 4 * LPR,
-                                           lane, ar);
-                    cur_v = vid;
+                const uint32_t image = __builtin_amdgcn_readfirstlane(tag[3]);
+                if (image != cur_image) {
+                    gg_read_image<G::NREG>(img0 + image * (uint32_t)sizeof(Image), 4 * LPR, lane, ar);
+                    cur_image = image;
                 }
             }
             v[k] = fm_chunk_sum<LPR>(ln.dot(t, ar, ones));
         }
-        const uint32_t u = (uint32_t)wg0 + (tag & 0x7FFFFFFFu);
-        const uint32_t pair = u / (uint32_t)upp, step = u - pair * (uint32_t)upp;
-        const bool ok = !(tag >> 31);
+        const uint32_t pair = __builtin_amdgcn_readfirstlane(tag[1]);
+        const uint32_t step = __builtin_amdgcn_readfirstlane(tag[2]);
+        const bool ok = __builtin_amdgcn_readfirstlane(tag[0]) == 0u;
         if (ch == 0) {
             if constexpr (GU)
                 a.act[(size_t)pair * a.g.inter + step * RPS + ris] = ok ? fm_silu_mul(v[0], v[NS - 1]) : 0.0f;
@@ -794,7 +866,8 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
 #else
     (void)a;
     (void)total_units;
-    (void)upp;
+    (void)by_upp;
+    (void)by_k;
 #endif
 }
 
@@ -824,7 +897,8 @@ int gg_launch_stream(const GgufArgs &a, int n_pairs, int n_cu, hipStream_t st) {
         const size_t sh = gg_stream_lds<KIND, L, GU>();                                        \
         static FmLdsAttr attr;                                                                 \
         if (!fm_dyn_lds_ready(attr, (const void *)kfn, sh)) return FM_ERR_HIP;                 \
-        hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(512), sh, st, a, (int)total, upp);   \
+        hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(512), sh, st, a, (int)total,            \
+                           gg_div_make((uint32_t)upp), gg_div_make((uint32_t)a.K));   \
     } while (0)
     switch (lpr) {
         case 4: GG_ST(4); break;
