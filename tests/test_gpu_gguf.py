@@ -124,3 +124,44 @@ def test_gguf_q4k_down_and_errors(orc):
         assert_parity(out, ref, "Q4_K down")
     finally:
         ctx.close()
+
+
+@pytest.mark.parametrize("h,i,down_t,layers,K", [(1024, 256, 14, 2, 8), (512, 1024, 14, 1, 4),
+                                                 (2048, 2048, 12, 1, 2), (1024, 512, 12, 3, 8)])
+def test_gguf_streaming_shapes(orc, h, i, down_t, layers, K):
+    """Every lane count of the streaming kernels (4, 8, 16 lanes per row, both down formats), shares
+    of the launch that cross pair and layer boundaries, and an expert index outside the store
+    (contributes nothing: its slot of expert_out is zero)."""
+    import torch
+    from finchmoe_amd import FinchHip
+    rng = np.random.default_rng(h + i + down_t)
+    e = 10
+    store = [F.synth_gguf_layer(rng, e, h, i, (12, 12, down_t)) for _ in range(layers)]
+    ctx = FinchHip(0)
+    try:
+        ctx.gguf_config(layers, e, h, i, (fb.Q4_K, fb.Q4_K, down_t))
+        for l, (g, u, d) in enumerate(store):
+            ctx.gguf_upload_layer(l, g, u, d)
+        x = rng.standard_normal((layers, h)).astype(np.float32)
+        idx = np.stack([rng.permutation(e)[:K] for _ in range(layers)]).astype(np.int32)
+        w = np.stack([orc.normalize_weights(rng.random(K).astype(np.float32)) for _ in range(layers)])
+        idx[0, K - 1] = -1
+        dx, di, dw = (torch.from_numpy(a).cuda() for a in (x, idx, w))
+        dout = torch.empty(layers, h, device="cuda")
+        deo = torch.empty(layers, K, h, device="cuda")
+        torch.cuda.synchronize()
+        ctx.gguf_moe_decode_step_dev(0, layers, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K,
+                                     dout.data_ptr(), deo.data_ptr())
+        ctx.sync()
+        out, eo = dout.cpu().numpy(), deo.cpu().numpy()
+        for l in range(layers):
+            ok = idx[l] >= 0
+            ref, ref_eo = orc.moe_gguf_forward(*store[l], x[l], np.where(ok, idx[l], 0).astype(np.int32),
+                                               np.where(ok, w[l], 0).astype(np.float32), h, i,
+                                               types=(12, 12, down_t))
+            ref_eo[~ok] = 0
+            assert_parity(eo[l], ref_eo, "expert_out layer %d" % l)
+            assert_parity(out[l], ref, "layer %d" % l)
+        assert not eo[0, K - 1].any()
+    finally:
+        ctx.close()
