@@ -376,20 +376,28 @@ __global__ __launch_bounds__(512) void fm_pf_down(PfArgs a) {
     const int n_items = *a.n_items;
     const int row_bytes = a.g.inter * 3 / 8, sb_bytes = (a.g.inter / 64) * 2;
     const uint32_t ones = fm_opaque(0x3F803F80u);
-    for (int it = blockIdx.x; it < n_items; it += gridDim.x) {
+    // The launch is the sequence (item, pass) — a pass = two row tiles per wave, 64 * NW
+    // rows of the item — and this workgroup takes passes [t0, t1) of it: every workgroup
+    // the same number (within one) whatever the number of items.
+    const int NW = blockDim.x / 64;
+    const int NP = a.g.hidden / (64 * NW);            // hidden is a multiple of 64 * NW
+    const long T = (long)n_items * NP;
+    const int t0 = (int)(T * blockIdx.x / gridDim.x), t1 = (int)(T * (blockIdx.x + 1) / gridDim.x);
+    for (int t = t0; t < t1;) {
+        const int it = t / NP, pb = t - it * NP;
+        const int pe = t1 - t < NP - pb ? pb + (t1 - t) : NP;
+        t += pe - pb;
         const PfItem item = a.items[it];
         __syncthreads();
         pf_stage<NG>(L, item.count, [&](int j) { return a.act + (size_t)(item.start + j) * a.g.inter; });
         __syncthreads();
         const uint8_t *blob = a.layer + (size_t)item.expert * a.g.expert_size;
         const int n = lane & 31, h = lane >> 5;
-        const int NW = blockDim.x / 64;
-        // pass p: row tiles wave + NW*(2p) and wave + NW*(2p+1) (hidden is a multiple of 64*NW)
-        const int n_tiles = (a.g.hidden / 32 - wave + NW - 1) / NW;
+        // pass p of the item: row tiles wave + NW*(2p) and wave + NW*(2p+1)
         pf_passes<NG, 4>(
-            L, n_tiles / 2, lane, ones,
+            L, pe - pb, lane, ones,
             [&](int p, int r, gptr &w, gptr &sr, gptr &br) {
-                const int row = (wave + NW * (2 * p + r)) * 32 + n;
+                const int row = (wave + NW * (2 * (pb + p) + r)) * 32 + n;
                 w = (gptr)(uintptr_t)(blob + a.g.down_w + (size_t)row * row_bytes);
                 sr = (gptr)(uintptr_t)(blob + a.g.down_s + (size_t)row * sb_bytes);
                 br = (gptr)(uintptr_t)(blob + a.g.down_b + (size_t)row * sb_bytes);
@@ -397,7 +405,7 @@ __global__ __launch_bounds__(512) void fm_pf_down(PfArgs a) {
             [&](int p, const f16v *acc) {
 #pragma unroll
                 for (int r = 0; r < PF_R; r++) {
-                    const int row = (wave + NW * (2 * p + r)) * 32 + n;
+                    const int row = (wave + NW * (2 * (pb + p) + r)) * 32 + n;
 #pragma unroll
                     for (int i = 0; i < 8; i++) {
                         const int tok = 8 * (i / 4) + 4 * h + (i % 4);
@@ -521,10 +529,18 @@ __global__ __launch_bounds__(512) void fm_pf_slab(PfArgs a) {
     const uint32_t soff = GPW >= 2 ? (uint32_t)((lane >> 1) * sb_bytes + sb_slab + 4 * (lane & 1))
                                    : (uint32_t)(lane * sb_bytes + sb_slab);
 
-    // ---- loader: tile-matrices of this workgroup's items, in order
-    int l_it = blockIdx.x, l_s = 0, l_mat = 0, wpos = 0;
+    // ---- this workgroup's share of the launch: steps [t0, t1) of the sequence
+    // (item, step), items in order — every workgroup gets the same number of steps
+    // (within one) whatever the number of items, at the price of building the
+    // activation operand of an item in two workgroups when a share ends inside it
+    const long T = (long)n_items * n_steps;
+    const int t0 = (int)(T * blockIdx.x / gridDim.x), t1 = (int)(T * (blockIdx.x + 1) / gridDim.x);
+
+    // ---- loader: tile-matrices of the share, in order
+    int l_t = t0, l_it = t0 / n_steps, l_mat = 0, wpos = 0;
+    int l_s = t0 - l_it * n_steps;
     uint32_t issued = 0, consumed = 0;
-    bool l_done = l_it >= n_items;
+    bool l_done = t0 >= t1;
     const uint8_t *l_blob = nullptr;
     if (!l_done) l_blob = fm_uniform(a.layer + (size_t)a.items[l_it].expert * a.g.expert_size);
     auto issue = [&]() __attribute__((always_inline)) {
@@ -549,20 +565,24 @@ __global__ __launch_bounds__(512) void fm_pf_slab(PfArgs a) {
         wpos = wpos + 1 == RING ? 0 : wpos + 1;
         issued++;
         l_mat ^= 1;
-        if (l_mat == 0 && ++l_s == n_steps) {
-            l_s = 0;
-            l_it += gridDim.x;
-            if (l_it < n_items)
-                l_blob = fm_uniform(a.layer + (size_t)a.items[l_it].expert * a.g.expert_size);
-            else
+        if (l_mat == 0) {
+            if (++l_t >= t1) {
                 l_done = true;
+            } else if (++l_s == n_steps) {
+                l_s = 0;
+                l_it++;
+                l_blob = fm_uniform(a.layer + (size_t)a.items[l_it].expert * a.g.expert_size);
+            }
         }
     };
 #pragma unroll
     for (int k = 0; k < RING; k++) issue();
 
     int c = 0, buf = 0;
-    for (int it = blockIdx.x; it < n_items; it += gridDim.x) {
+    for (int t = t0; t < t1;) {
+        const int it = t / n_steps, s_begin = t - it * n_steps;
+        const int s_end = t1 - t < n_steps - s_begin ? s_begin + (t1 - t) : n_steps;
+        t += s_end - s_begin;
         const PfItem item = a.items[it];
         // ---- this wave's share of the activation operand, straight into registers:
         // lane (m, hh): M row m = hi piece of position m (m < 16) or lo piece of position
@@ -631,7 +651,7 @@ __global__ __launch_bounds__(512) void fm_pf_slab(PfArgs a) {
         int my_pair = 0;
         if (!GU && my_on) my_pair = a.sorted[item.start + my_pos];
 
-        for (int s = 0; s < n_steps; s++) {
+        for (int s = s_begin; s < s_end; s++) {
 #pragma unroll
             for (int mat = 0; mat < 2; mat++) {
                 // The hardware issues the older of two waves on a SIMD first, which lets waves
