@@ -571,6 +571,8 @@ extern "C" int fm_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, const 
     if (!d_X || !d_idx || !d_w || !d_out) return fail(c, FM_ERR_ARG, "null pointer");
     if (M < 1) return fail(c, FM_ERR_ARG, "M %d", M);
     if (K < 1 || K > FM_MAX_K) return fail(c, FM_ERR_ARG, "K %d outside 1..%d", K, FM_MAX_K);
+    if (((uintptr_t)d_X | (uintptr_t)d_out) & 15)
+        return fail(c, FM_ERR_ARG, "X / out not 16-byte aligned");
     int rc = check_layers(c, c->layers, layer, 1);
     if (rc) return rc;
     DeviceGuard dg(c->device);

@@ -820,14 +820,29 @@ __global__ __launch_bounds__(256) void fm_pf_combine(PfArgs a, float *out, int f
         }
         wk[k] = w;
     }
-    const float *eo = a.eo + (size_t)m * K * H;
-    for (int j = blockIdx.y * blockDim.x + threadIdx.x; j < H; j += gridDim.y * blockDim.x) {
-        float acc = 0.0f;
+    // four columns per thread (hidden is a multiple of 4)
+    const float4 *eo = reinterpret_cast<const float4 *>(a.eo + (size_t)m * K * H);
+    float4 *o4 = reinterpret_cast<float4 *>(out + (size_t)m * H);
+    const int H4 = H / 4;
+    for (int j = blockIdx.y * blockDim.x + threadIdx.x; j < H4; j += gridDim.y * blockDim.x) {
+        float4 v[FM_MAX_K];
 #pragma unroll
         for (int k = 0; k < FM_MAX_K; k++)
-            if (k < K && wk[k] != 0.0f) acc += wk[k] * eo[(size_t)k * H + j];
-        float *o = out + (size_t)m * H + j;
-        *o = (flags & FM_ACCUMULATE) ? *o + acc : acc;
+            if (k < K && wk[k] != 0.0f) v[k] = eo[(size_t)k * H4 + j];
+        float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+        for (int k = 0; k < FM_MAX_K; k++)
+            if (k < K && wk[k] != 0.0f) {
+                acc.x += wk[k] * v[k].x;
+                acc.y += wk[k] * v[k].y;
+                acc.z += wk[k] * v[k].z;
+                acc.w += wk[k] * v[k].w;
+            }
+        if (flags & FM_ACCUMULATE) {
+            const float4 p = o4[j];
+            acc.x += p.x, acc.y += p.y, acc.z += p.z, acc.w += p.w;
+        }
+        o4[j] = acc;
     }
 }
 
