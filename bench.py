@@ -7,7 +7,7 @@ HBM, per-layer top-8 indices from a Zipf(1.1) distribution with a per-layer rank
 router weights = renormalised softmax of N(0,1) logits at those indices.  A "step" is one
 token: one pass of the hot path over all 40 layers.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_layer|gdn|gguf|prefill]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_layer|gdn|gguf|prefill|lm_head]
 
 Prints ONE JSON line.  `value` is algorithmic weight bytes per step / wall time per step with
 all inputs resident in HBM.  `roofline` prices the dominant kernel against the 8 TB/s HBM
@@ -354,6 +354,40 @@ def run_gdn(args):
                    bytes_set, ms, args)
 
 
+def run_lm_head(args):
+    """Next row after the expert path: the 8-bit [vocab 248320, 2048] output projection
+    (finchmoe/infer.m:5728-5760), batch 1, three weight sets cycled (1.6 GB)."""
+    import torch
+    from finchmoe_amd import FinchHip
+    dev = torch.device("cuda:0")
+    ctx = FinchHip(0)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(11)
+    V, D = 248320, 2048
+    keep, sets = [], []
+    for _ in range(3):
+        W = torch.empty(V * D, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
+        s = torch.randn(V * (D // 64), device=dev, generator=gen).abs_() * (0.02 / 127.5)
+        b = s * -127.5
+        S, B = _bf16_trunc_bits(s), _bf16_trunc_bits(b)
+        keep.extend([W, S, B])
+        sets.append(ctx.tensor_adopt(W.data_ptr(), S.data_ptr(), B.data_ptr(), V, D, 8))
+    d_x = torch.randn(D, device=dev)
+    d_o = torch.empty(V, device=dev)
+    torch.cuda.synchronize()
+
+    def step(t):
+        ctx.matvec_batch_dev([sets[t % 3]], d_x.data_ptr(), [d_o.data_ptr()])
+
+    ms, ev = _timed(ctx, step, args)
+    assert torch.isfinite(d_o).all()
+    bytes_set = V * D + 2 * V * (D // 64) * 2
+    res = {"event_ms_per_step": round(ev, 5)}
+    ctx.close()
+    return _finish(res, "8-bit output projection GEMV HBM GB/s", "lm_head 2048->248320, 8-bit g64, "
+                   "batch 1, 3 weight sets cycled", bytes_set, ms, args)
+
+
 def run_gguf(args):
     """config 4: GGUF experts (Q4_K gate/up, Q6_K down), 40-layer decode step, batch 1."""
     import torch
@@ -499,7 +533,8 @@ def main():
         print("bench.py: no GPU visible; there is no CPU fallback", file=sys.stderr)
         sys.exit(3)
     runners = {"decode_step": run_decode_step, "decode_layer": run_decode_layer, "gdn": run_gdn,
-               "gguf": run_gguf, "prefill": run_prefill, "copy_probe": run_copy_probe}
+               "gguf": run_gguf, "prefill": run_prefill, "lm_head": run_lm_head,
+               "copy_probe": run_copy_probe}
     if args.workload not in runners:
         print("bench.py: unknown workload %r (have: %s)" % (args.workload, ", ".join(runners)),
               file=sys.stderr)

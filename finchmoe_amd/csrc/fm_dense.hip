@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void fm_dense_gemv(FmDenseArgs a) {
 }
 
 // ----------------------------------------------------------------------
-// Streaming form (3- and 4-bit, in_dim up to 2048, or 4096 at 4 bits): the
+// Streaming form (3-, 4- and 8-bit, in_dim up to 2048, or 4096 at 4 bits): the
 // structure of the expert kernels (fm_decode.hip) without segments.  All wave
 // steps ("units", 64/LPR rows) of all tensors of the launch form one sequence;
 // workgroup g (8 waves, one per CU) takes [U*g/G, U*(g+1)/G), its waves claim
@@ -94,16 +94,18 @@ __global__ __launch_bounds__(256) void fm_dense_gemv(FmDenseArgs a) {
 // and multiply on the matrix cores against the activation registers, which the
 // workgroup builds once.  in_dim = 4096 is two slabs of 2048 columns: a unit is
 // two slices, each against its own activation registers, summed in slab order.
+// 8-bit (the vocabulary projection, finchmoe/infer.m:5728-5760): same ring, two
+// 8 KB units in flight per wave, multiply on the vector ALU.
 // ----------------------------------------------------------------------
 template <int BITS>
 struct FmDenseRing {
-    static constexpr int RING = BITS == 3 ? 4 : 3;
+    static constexpr int RING = BITS == 3 ? 4 : (BITS == 8 ? 2 : 3);
     static constexpr int BYTES = 8 * RING * FmSlot<BITS>::BYTES;
 };
 
 template <int BITS, int LPR, int NS>
 constexpr size_t fm_dense_stream_lds() {
-    return FmDenseRing<BITS>::BYTES + NS * sizeof(FmActLds<LPR>);
+    return FmDenseRing<BITS>::BYTES + (BITS == 8 ? 0 : NS * sizeof(FmActLds<LPR>));
 }
 
 extern __shared__ __attribute__((aligned(16))) uint8_t fm_dense_lds[];
@@ -196,6 +198,27 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
 #pragma unroll
     for (int k = 0; k < RING; k++) issue();      // the weights do not wait for the activations
 
+    if constexpr (BITS == 8) {
+        // A byte does not fit a bf16 mantissa, and at one byte per code the vector ALU has
+        // time for convert + multiply-add: the plain dot product against the lane's 128
+        // activations, fed from the ring.
+        static_assert(BITS != 8 || NS == 1, "one slab");
+        float xs[FM_CPL], xsum0, xsum1;
+        fm_load_x<8>(a.x + (size_t)m * a.in_dim + ch * FM_CPL, xs, xsum0, xsum1);
+        int c8 = 0;
+        while (consumed < issued) {
+            FmRowSlice<BITS> t;
+            if (issued - consumed == (uint32_t)RING) fm_dma_wait<SL::LOADS *(RING - 1)>(false);
+            else fm_dma_wait<0>(true);
+            const uint32_t tag = fm_dma_read<BITS>(ring0 + (uint32_t)c8 * SL::BYTES, woff, soff, t);
+            consumed++;
+            c8 = c8 + 1 == RING ? 0 : c8 + 1;
+            issue();
+            const float v = fm_chunk_sum<LPR>(fm_lane_dot<BITS, FP16>(t, xs, xsum0, xsum1));
+            const Where w = locate(wg0 + tag);
+            if (ch == 0) w.out[(size_t)m * w.out_dim + w.row0 + ris] = v;
+        }
+    } else {
     // the activation registers of every slab, built once
     FmBuildSlot<BITS> bslot;
     bslot.init();
@@ -230,6 +253,7 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
         const Where w = locate(wg0 + tag);
         if (ch == 0) w.out[(size_t)m * w.out_dim + w.row0 + ris] = v;
     }
+    }
 #else
     (void)a;
     (void)total_units;
@@ -242,6 +266,7 @@ int launch_dense_stream_t(FmDenseArgs &a, int M, int n_cu, hipStream_t st) {
     const int lpr_full = a.in_dim / FM_CPL;
     const int ns = lpr_full == 32 ? 2 : 1, lpr = lpr_full / ns;
     if (!(lpr == 4 || lpr == 8 || lpr == 16) || (ns == 2 && BITS != 4)) return FM_ERR_UNSUPPORTED;
+    if (BITS == 8 && ((uintptr_t)a.x & 15)) return FM_ERR_UNSUPPORTED;
     const int rps = FM_WAVE / lpr;
     int units = 0;
     for (int i = 0; i < a.n; i++) {
@@ -328,10 +353,12 @@ extern "C" int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, 
     }
     for (int i = n; i < FM_MAX_BATCH; i++) a.spec[i] = a.spec[0];
     static const bool no_stream = getenv("FINCH_DENSE_VALU") != nullptr;
-    if (!no_stream && (bits == 3 || bits == 4)) {
+    if (!no_stream && (bits == 3 || bits == 4 || bits == 8)) {
         int rc = FM_ERR_UNSUPPORTED;
         if (bits == 3) rc = scale_fp16 ? launch_dense_stream_t<3, true>(a, M, n_cu, st)
                                        : launch_dense_stream_t<3, false>(a, M, n_cu, st);
+        else if (bits == 8) rc = scale_fp16 ? launch_dense_stream_t<8, true>(a, M, n_cu, st)
+                                            : launch_dense_stream_t<8, false>(a, M, n_cu, st);
         else rc = scale_fp16 ? launch_dense_stream_t<4, true>(a, M, n_cu, st)
                              : launch_dense_stream_t<4, false>(a, M, n_cu, st);
         if (rc != FM_ERR_UNSUPPORTED) return rc;

@@ -69,8 +69,11 @@ __device__ __forceinline__ void fm_unit_lane_offsets(int lane, int row_bytes, in
 template <int BITS, int I>
 __device__ __forceinline__ void fm_dma_codes(uint32_t slot, fm_gptr w) {
     if constexpr (I < FmSlot<BITS>::NQ) {
-        // the instruction offset moves the global and the LDS address alike
-        __builtin_amdgcn_global_load_lds(w, (fm_lptr)(uintptr_t)slot, 16, 1024 * I, 0);
+        // the instruction offset moves the global and the LDS address alike; it holds
+        // -4096..4095, so from the fifth load on both addresses move by 4096 instead
+        constexpr int BASE = (I / 4) * 4096, IMM = (I % 4) * 1024;
+        __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)((const uint8_t *)w + BASE),
+                                         (fm_lptr)(uintptr_t)(slot + BASE), 16, IMM, 0);
         fm_dma_codes<BITS, I + 1>(slot, w);
     }
 }
@@ -101,6 +104,17 @@ __device__ __forceinline__ uint32_t fm_dma_read(uint32_t slot, uint32_t woff, ui
                      "s_waitcnt lgkmcnt(0)"
                      : "=&v"(t.q[0]), "=&v"(t.q[1]), "=&v"(t.q[2]), "=&v"(t.s), "=&v"(t.b),
                        "=&v"(tag)
+                     : "v"(aw), "v"(as), "v"(at)
+                     : "memory");
+    } else if constexpr (BITS == 8) {
+        asm volatile("ds_read_b128 %0, %11\n\tds_read_b128 %1, %11 offset:16\n\t"
+                     "ds_read_b128 %2, %11 offset:32\n\tds_read_b128 %3, %11 offset:48\n\t"
+                     "ds_read_b128 %4, %11 offset:64\n\tds_read_b128 %5, %11 offset:80\n\t"
+                     "ds_read_b128 %6, %11 offset:96\n\tds_read_b128 %7, %11 offset:112\n\t"
+                     "ds_read_b32 %8, %12\n\tds_read_b32 %9, %12 offset:256\n\t"
+                     "ds_read_b32 %10, %13\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(t.q[0]), "=&v"(t.q[1]), "=&v"(t.q[2]), "=&v"(t.q[3]), "=&v"(t.q[4]),
+                       "=&v"(t.q[5]), "=&v"(t.q[6]), "=&v"(t.q[7]), "=&v"(t.s), "=&v"(t.b), "=&v"(tag)
                      : "v"(aw), "v"(as), "v"(at)
                      : "memory");
     } else {

@@ -61,7 +61,7 @@ def test_matvec_shapes_and_widths(hip, orc, bits, dtype, out_dim, in_dim):
 
 @pytest.mark.parametrize("bits,dtype,out_dim,in_dim", [
     (4, "bf16", 8192, 4096), (3, "bf16", 8192, 2048), (4, "fp16", 16384, 1024),
-    (3, "fp16", 32768, 512)])
+    (3, "fp16", 32768, 512), (8, "bf16", 16384, 2048), (8, "fp16", 32768, 1024), (8, "bf16", 65536, 512)])
 def test_streaming_kernel_shapes(hip, orc, bits, dtype, out_dim, in_dim):
     """Launches large enough for the streaming kernel (a wave step for every wave of the
     chip): two column slabs at in_dim 4096, every lanes-per-row specialisation, both widths
