@@ -7,7 +7,7 @@ HBM, per-layer top-8 indices from a Zipf(1.1) distribution with a per-layer rank
 router weights = renormalised softmax of N(0,1) logits at those indices.  A "step" is one
 token: one pass of the hot path over all 40 layers.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_layer|gdn|gguf|prefill|lm_head]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_layer|gdn|gguf|prefill|lm_head|layer_tail]
 
 Prints ONE JSON line.  `value` is algorithmic weight bytes per step / wall time per step with
 all inputs resident in HBM.  `roofline` prices the dominant kernel against the 8 TB/s HBM
@@ -388,6 +388,46 @@ def run_lm_head(args):
                    "batch 1, 3 weight sets cycled", bytes_set, ms, args)
 
 
+def run_layer_tail(args):
+    """Next row after the expert path: shared-expert down projection + combine with residual +
+    next layer's RMS norm in one launch (finchmoe/infer.m:9608-9760), 40 layers' tensors cycled."""
+    import torch
+    from finchmoe_amd import FinchHip
+    dev = torch.device("cuda:0")
+    ctx = FinchHip(0)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(13)
+    SI = 512
+    keep, ts = [], []
+    for _ in range(40):
+        W = torch.empty(H * SI // 2, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
+        s = torch.randn(H * (SI // 64), device=dev, generator=gen).abs_() * (0.02 / 7.5)
+        S, B = _bf16_trunc_bits(s), _bf16_trunc_bits(s * -7.5)
+        keep.extend([W, S, B])
+        ts.append(ctx.tensor_adopt(W.data_ptr(), S.data_ptr(), B.data_ptr(), H, SI, 4))
+    h_mid, eo = torch.randn(H, device=dev), torch.randn(K, H, device=dev)
+    params = torch.zeros(10, device=dev)
+    params[:K] = 1.0 / K
+    sg, su = torch.randn(SI, device=dev), torch.randn(SI, device=dev)
+    nw = torch.ones(H, device=dev).to(torch.bfloat16)
+    hid, nxt = torch.empty(H, device=dev), torch.empty(H, device=dev)
+    torch.cuda.synchronize()
+
+    def step(t):
+        ctx.layer_tail_dev(ts[t % 40], h_mid.data_ptr(), eo.data_ptr(), params.data_ptr(), K,
+                           sg.data_ptr(), su.data_ptr(), nw.data_ptr(), 1e-6, hid.data_ptr(),
+                           nxt.data_ptr())
+
+    ms, ev = _timed(ctx, step, args)
+    assert torch.isfinite(nxt).all()
+    bytes_call = H * SI // 2 + 2 * H * (SI // 64) * 2 + (K + 4) * H * 4
+    res = {"event_ms_per_step": round(ev, 5)}
+    ctx.close()
+    return _finish(res, "layer tail (shared down + combine + residual + RMS norm) GB/s",
+                   "one launch per layer: 4-bit [2048,512] shared down projection, K=8 combine, "
+                   "next-layer norm; 40 tensors cycled", bytes_call, ms, args)
+
+
 def run_gguf(args):
     """config 4: GGUF experts (Q4_K gate/up, Q6_K down), 40-layer decode step, batch 1."""
     import torch
@@ -533,7 +573,7 @@ def main():
         print("bench.py: no GPU visible; there is no CPU fallback", file=sys.stderr)
         sys.exit(3)
     runners = {"decode_step": run_decode_step, "decode_layer": run_decode_layer, "gdn": run_gdn,
-               "gguf": run_gguf, "prefill": run_prefill, "lm_head": run_lm_head,
+               "gguf": run_gguf, "prefill": run_prefill, "lm_head": run_lm_head, "layer_tail": run_layer_tail,
                "copy_probe": run_copy_probe}
     if args.workload not in runners:
         print("bench.py: unknown workload %r (have: %s)" % (args.workload, ", ".join(runners)),

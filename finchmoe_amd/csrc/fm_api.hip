@@ -44,6 +44,7 @@ int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGeom *g, cons
                              float *d_out, void *d_ws, size_t ws_bytes, int flags, int n_cu,
                              hipStream_t st);
 size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K);
+int fm_launch_layer_tail(const FmTailArgs *a, int bits, int scale_fp16, hipStream_t st);
 }
 
 namespace {
@@ -104,6 +105,8 @@ struct fm_ctx {
     size_t stage_bytes = 0;
     void *d_ws = nullptr;
     size_t ws_bytes = 0;
+    // layer tail: one partial sum per workgroup, then the ticket counter
+    float *d_tail = nullptr;
 
     std::vector<Tensor> tensors;
 };
@@ -289,7 +292,7 @@ extern "C" int fm_ctx_destroy(fm_ctx *c) {
     if (c->h_err) (void)hipHostFree(c->h_err);
     void *ptrs[] = {c->d_layer_ptrs, c->d_gg_ptrs, c->d_act, c->d_eo, c->d_counters,
                     c->dflags.set[0],
-                    c->d_stage, c->d_ws};
+                    c->d_stage, c->d_ws, c->d_tail};
     if (c->h_stage) (void)hipHostFree(c->h_stage);
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
@@ -789,6 +792,58 @@ extern "C" int fm_matvec_prefill(fm_ctx *c, fm_tensor t, const float *X, float *
     if (M < 1 || M > 65535) return fail(c, FM_ERR_ARG, "M %d outside 1..65535", M);
     float *outs[1] = {out};
     return matvec_host(c, &t, 1, X, outs, M);
+}
+
+// ============================================================================
+// layer tail
+// ============================================================================
+#define FM_TAIL_PARTIALS 4096
+
+extern "C" int fm_layer_tail_dev(fm_ctx *c, fm_tensor shared_down, const float *d_h_mid,
+                                 const float *d_expert_out, const float *d_params, int K,
+                                 const float *d_shared_gate, const float *d_shared_up,
+                                 const uint16_t *d_next_norm_w, float eps, float *d_hidden_out,
+                                 float *d_next_input) {
+    if (!c) return FM_ERR_ARG;
+    Tensor *t = get_tensor(c, shared_down);
+    if (!t) return fail(c, FM_ERR_ARG, "bad tensor handle %d", shared_down);
+    if (!d_h_mid || !d_params || !d_shared_gate || !d_shared_up || !d_hidden_out ||
+        (K > 0 && !d_expert_out))
+        return fail(c, FM_ERR_ARG, "null pointer");
+    if (K < 0 || K > FM_MAX_K) return fail(c, FM_ERR_ARG, "K %d outside 0..%d", K, FM_MAX_K);
+    if ((d_next_input != nullptr) != (d_next_norm_w != nullptr))
+        return fail(c, FM_ERR_ARG, "next input and its norm weights go together");
+    if (((uintptr_t)d_shared_gate | (uintptr_t)d_shared_up) & 3)
+        return fail(c, FM_ERR_ARG, "vector not 4-byte aligned");
+    if (t->group_size != 64) return fail(c, FM_ERR_UNSUPPORTED, "group size %d", t->group_size);
+    if (t->out_dim / 4 > FM_TAIL_PARTIALS) return fail(c, FM_ERR_UNSUPPORTED, "hidden %d", t->out_dim);
+    DeviceGuard dg(c->device);
+    if (!c->d_tail) {
+        HIPCHK(c, hipMalloc((void **)&c->d_tail, (FM_TAIL_PARTIALS + 64) * sizeof(float)));
+        HIPCHK(c, hipMemsetAsync(c->d_tail, 0, (FM_TAIL_PARTIALS + 64) * sizeof(float), c->stream));
+    }
+    FmTailArgs a;
+    a.W = (const uint8_t *)t->W;
+    a.S = (const uint8_t *)t->S;
+    a.B = (const uint8_t *)t->B;
+    a.hidden = t->out_dim;
+    a.inter = t->in_dim;
+    a.K = K;
+    a.h_mid = d_h_mid;
+    a.expert_out = d_expert_out;
+    a.params = d_params;
+    a.shared_gate = d_shared_gate;
+    a.shared_up = d_shared_up;
+    a.norm_w = d_next_norm_w;
+    a.eps = eps;
+    a.hidden_out = d_hidden_out;
+    a.next_in = d_next_input;
+    a.partial = c->d_tail;
+    a.counter = (unsigned int *)(c->d_tail + FM_TAIL_PARTIALS);
+    int rc = fm_launch_layer_tail(&a, t->bits, t->scale_fp16, c->stream);
+    if (rc) return fail(c, rc, "layer tail: shape [%d, %d] at %d bits has no kernel", t->out_dim,
+                        t->in_dim, t->bits);
+    return FM_OK;
 }
 
 // ============================================================================

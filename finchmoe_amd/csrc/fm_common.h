@@ -39,6 +39,19 @@ struct FmGgufGeom {
     uint32_t gu_row_bytes, down_row_bytes;
 };
 
+// Operands of the layer tail (fm_tail.hip): shared expert's down projection W/S/B
+// [hidden][inter], the vectors it combines, and the scratch of the norm's reduction.
+struct FmTailArgs {
+    const uint8_t *W, *S, *B;
+    int hidden, inter, K;
+    const float *h_mid, *expert_out, *params, *shared_gate, *shared_up;
+    const uint16_t *norm_w;
+    float eps;
+    float *hidden_out, *next_in;
+    float *partial;
+    unsigned int *counter;
+};
+
 // ---------------------------------------------------------------- device helpers
 #if defined(__HIPCC__)
 

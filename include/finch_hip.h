@@ -172,6 +172,26 @@ FM_API int fm_matvec_batch(fm_ctx *ctx, const fm_tensor *tensors, int n, const f
 FM_API int fm_matvec_prefill_dev(fm_ctx *ctx, fm_tensor t, const float *d_X, float *d_out, int M);
 FM_API int fm_matvec_prefill(fm_ctx *ctx, fm_tensor t, const float *X, float *out, int M);
 
+/* ---------------------------------------------------------------- layer tail
+ * Replaces the five dispatches the reference appends to a layer's expert command
+ * buffer (finchmoe/infer.m:9608-9760): swiglu_fused on the shared expert's gate/up
+ * outputs, its down projection (dequant_matvec), moe_combine_residual
+ * (shaders.metal:2196-2231), rms_norm_sum_sq + rms_norm_apply_bf16
+ * (shaders.metal:1134-1205).
+ *   shared_down : registered tensor [hidden][shared_inter], 3/4/8-bit g64
+ *   h_mid[hidden], expert_out[K][hidden] (as fm_moe_decode leaves them),
+ *   params[10] = expert weights 0..7 (0 for an invalid slot), shared gate score
+ *   at [8] (buf_combine_params), shared_gate / shared_up [shared_inter],
+ *   next_norm_w[hidden] bf16 + next_input[hidden], both NULL for the last layer.
+ * hidden_out = h_mid + sum_k params[k]*expert_out[k] + sigmoid(params[8])*shared_out;
+ * next_input = hidden_out / sqrt(mean(hidden_out^2) + eps) * next_norm_w.
+ * All pointers device memory; asynchronous on the context's stream. */
+FM_API int fm_layer_tail_dev(fm_ctx *ctx, fm_tensor shared_down, const float *d_h_mid,
+                      const float *d_expert_out, const float *d_params, int K,
+                      const float *d_shared_gate, const float *d_shared_up,
+                      const uint16_t *d_next_norm_w, float eps, float *d_hidden_out,
+                      float *d_next_input);
+
 /* ---------------------------------------------------------------- GGUF expert store
  * Replaces GgufExpertInfo + the slab copies of gpu_gguf_experts_forward
  * (finchmoe/infer.m:1017-1022, 3239-3290).  gate/up/down are the stacked

@@ -501,6 +501,46 @@ void orc_vec_madd(float *dst, const float *src, float scale, int dim) {
 }
 
 /* ------------------------------------------------------------------ */
+/* layer tail: shared expert, combine with residual, next layer's norm */
+/* ------------------------------------------------------------------ */
+
+/* infer.m:1766-1777 */
+void orc_rms_norm(const float *x, const uint16_t *w_bf16, float *out, int dim, float eps) {
+    float sum_sq = 0.0f;
+    for (int i = 0; i < dim; i++) sum_sq += x[i] * x[i];
+    float rms = sqrtf(sum_sq / dim + eps);
+    float inv_rms = 1.0f / rms;
+    for (int i = 0; i < dim; i++) out[i] = x[i] * inv_rms * orc_bf16_to_f32(w_bf16[i]);
+}
+
+/* What CMD3 appends after the routed experts (infer.m:9608-9760): SwiGLU of the
+ * shared expert's gate/up outputs (1780-1786), its down projection (1676-1763),
+ * hidden = h_mid + sum_k params[k] * expert_out[k] + sigmoid(params[8]) * shared_out
+ * in slot order (shaders.metal:2196-2231; CPU twin infer.m:7390-7412), then the
+ * next layer's input norm (1766-1777; shaders.metal:1134-1205).  next_in may be NULL. */
+void orc_layer_tail(const void *sdW, const uint16_t *sdS, const uint16_t *sdB,
+                    int hidden, int shared_inter, int group_size, int bits, int scale_dtype,
+                    const float *h_mid, const float *expert_out, const float *params, int K,
+                    const float *shared_gate, const float *shared_up,
+                    const uint16_t *next_norm_w, float eps,
+                    float *hidden_out, float *next_in) {
+    float *act = (float *)malloc((size_t)shared_inter * sizeof(float));
+    float *shared_out = (float *)malloc((size_t)hidden * sizeof(float));
+    orc_swiglu(shared_gate, shared_up, act, shared_inter);
+    orc_dequant_matvec(sdW, sdS, sdB, act, shared_out, hidden, shared_inter, group_size, bits,
+                       scale_dtype);
+    float shared_w = 1.0f / (1.0f + expf(-params[8]));
+    for (int i = 0; i < hidden; i++) {
+        float moe = 0.0f;
+        for (int k = 0; k < K; k++) moe += params[k] * expert_out[(size_t)k * hidden + i];
+        hidden_out[i] = h_mid[i] + moe + shared_w * shared_out[i];
+    }
+    if (next_in && next_norm_w) orc_rms_norm(hidden_out, next_norm_w, next_in, hidden, eps);
+    free(act);
+    free(shared_out);
+}
+
+/* ------------------------------------------------------------------ */
 /* routed-expert block                                                 */
 /* ------------------------------------------------------------------ */
 

@@ -118,6 +118,20 @@ void orc_moe_experts_forward(const uint8_t *layer_blob, int hidden, int inter,
                              float *gate_out, float *up_out, float *act_out,
                              int nthreads);
 
+/* infer.m:1766-1777 */
+void orc_rms_norm(const float *x, const uint16_t *w_bf16, float *out, int dim, float eps);
+
+/* The tail of a layer's expert command buffer (infer.m:9608-9760): shared-expert SwiGLU
+ * and down projection, hidden = h_mid + sum_k params[k]*expert_out[k] +
+ * sigmoid(params[8])*shared_out (shaders.metal:2196-2231), next layer's input RMS norm
+ * with bf16 weights (shaders.metal:1134-1205).  params[10] as buf_combine_params. */
+void orc_layer_tail(const void *sdW, const uint16_t *sdS, const uint16_t *sdB,
+                    int hidden, int shared_inter, int group_size, int bits, int scale_dtype,
+                    const float *h_mid, const float *expert_out, const float *params, int K,
+                    const float *shared_gate, const float *shared_up,
+                    const uint16_t *next_norm_w, float eps,
+                    float *hidden_out, float *next_in);
+
 /* GGUF routed-expert block (infer.m:3153-3347, CPU twin infer.m:10011-10099):
  * gate/up/down slabs are the stacked per-layer tensors, expert e at e*slab. */
 void orc_moe_gguf_forward(const uint8_t *gate, const uint8_t *up, const uint8_t *down,

@@ -70,6 +70,9 @@ def lib():
                                               f32p, f32p, f32p, f32p, f32p, i]
         L.orc_moe_gguf_forward.argtypes = [u8p, u8p, u8p, i, i, i, i, i, f32p, i32p, f32p,
                                            i, i, f32p, f32p, i]
+        L.orc_rms_norm.argtypes = [f32p, u16p, f32p, i, C.c_float]
+        L.orc_layer_tail.argtypes = [vp, u16p, u16p, i, i, i, i, i, f32p, f32p, f32p, i, f32p, f32p,
+                                     u16p, C.c_float, f32p, f32p]
         _LIB = L
     return _LIB
 
@@ -209,6 +212,33 @@ def swiglu(g, u):
     out = np.empty_like(g)
     lib().orc_swiglu(_p(g), _p(u), _p(out), g.size)
     return out
+
+
+def rms_norm(x, w_bf16, eps=1e-6):
+    x = _c(x, np.float32)
+    w = _c(w_bf16, np.uint16)
+    out = np.empty_like(x)
+    lib().orc_rms_norm(_p(x), _p(w), _p(out), x.size, eps)
+    return out
+
+
+def layer_tail(sdW, sdS, sdB, h_mid, expert_out, params, K, shared_gate, shared_up, next_norm_w,
+               bits=4, group_size=64, scale_dtype=SCALE_BF16, eps=1e-6):
+    """-> (hidden_out, next_in or None)"""
+    sdW = np.ascontiguousarray(sdW)
+    sdS, sdB = _c(sdS, np.uint16), _c(sdB, np.uint16)
+    h_mid = _c(h_mid, np.float32)
+    eo = _c(expert_out, np.float32)
+    params = _c(params, np.float32)
+    sg, su = _c(shared_gate, np.float32), _c(shared_up, np.float32)
+    nw = None if next_norm_w is None else _c(next_norm_w, np.uint16)
+    hidden, si = h_mid.size, sg.size
+    hid = np.empty(hidden, np.float32)
+    nxt = None if nw is None else np.empty(hidden, np.float32)
+    lib().orc_layer_tail(_p(sdW), _p(sdS), _p(sdB), hidden, si, group_size, bits, scale_dtype,
+                         _p(h_mid), _p(eo), _p(params), K, _p(sg), _p(su), _p(nw), eps,
+                         _p(hid), _p(nxt))
+    return hid, nxt
 
 
 def softmax(x):

@@ -221,3 +221,42 @@ def test_bf16_operand_model_bound(orc):
     b = orc.dequant_matvec_bf16model(W, S, B, x, out_dim, in_dim, 3)
     print("bf16 model vs fp32 path: rel_err %.3e cosine %.8f" % (rel_err(b, a), cosine(b, a)))
     assert cosine(b, a) > 0.9999
+
+
+def test_layer_tail_against_float64_and_special_cases(orc):
+    """orc_layer_tail (infer.m:9608-9760, shaders.metal:2196-2231, 1134-1205) against a float64
+    evaluation built from the dequantized weights, and the cases that pin each term: zero
+    expert weights drop the expert sum, a very negative gate score drops the shared expert,
+    the norm of c*x equals the norm of x for eps -> 0."""
+    from finchmoe_amd import formats as F
+    rng = np.random.default_rng(21)
+    hidden, si, K = 256, 128, 4
+    codes, W, S, B = F.synth_affine_tensor(rng, hidden, si, 4, "bf16")
+    wd = orc.dequant_affine(W, S, B, hidden, si, 4)[1].astype(np.float64)
+    h_mid = rng.standard_normal(hidden).astype(np.float32)
+    eo = rng.standard_normal((K, hidden)).astype(np.float32)
+    params = np.zeros(10, np.float32)
+    params[:K] = [0.4, 0.3, 0.2, 0.1]
+    params[8] = 0.7
+    sg = rng.standard_normal(si).astype(np.float32)
+    su = rng.standard_normal(si).astype(np.float32)
+    nw = ((1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    hid, nxt = orc.layer_tail(W, S, B, h_mid, eo, params, K, sg, su, nw)
+    g = sg.astype(np.float64)
+    act = g / (1 + np.exp(-g)) * su
+    want = h_mid + (params[:K, None].astype(np.float64) * eo).sum(0) + wd @ act / (1 + np.exp(-0.7))
+    assert np.abs(hid - want).max() < 1e-5 * np.abs(want).max()
+    wn = (nw.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    want_n = want / np.sqrt(np.mean(want ** 2) + 1e-6) * wn
+    assert np.abs(nxt - want_n).max() < 1e-5 * np.abs(want_n).max()
+    # special cases
+    p0 = params.copy()
+    p0[:K] = 0
+    p0[8] = -200.0
+    hid0, _ = orc.layer_tail(W, S, B, h_mid, eo, p0, K, sg, su, None)
+    assert np.array_equal(hid0, h_mid)
+    a = orc.rms_norm(h_mid, nw, 0.0)
+    b = orc.rms_norm(3.0 * h_mid, nw, 0.0)
+    assert np.abs(a - b).max() < 1e-6
+    ones = np.full(hidden, 0x3F80, np.uint16)
+    assert abs(float(np.mean(orc.rms_norm(h_mid, ones, 0.0).astype(np.float64) ** 2)) - 1.0) < 1e-6
