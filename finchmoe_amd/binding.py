@@ -79,6 +79,7 @@ def load():
         "fm_matvec_batch": (i, [vp, C.POINTER(i), i, vp, C.POINTER(vp)]),
         "fm_matvec_prefill_dev": (i, [vp, i, vp, vp, i]),
         "fm_matvec_prefill": (i, [vp, i, vp, vp, i]),
+        "fm_route_topk_dev": (i, [vp, vp, i, i, vp, vp, vp, vp]),
         "fm_layer_tail_dev": (i, [vp, i, vp, vp, vp, i, vp, vp, vp, C.c_float, vp, vp]),
         "fm_gguf_config": (i, [vp, i, i, i, i, i, i, i]),
         "fm_gguf_upload_layer": (i, [vp, i, vp, vp, vp]),
@@ -257,6 +258,10 @@ class FinchHip:
         self._chk(self.L.fm_matvec_prefill_dev(self.h, t, d_X, d_out, M))
 
     # ---- GGUF
+    def route_topk_dev(self, d_logits, n_experts, K, d_seg_score, d_idx, d_w, d_params=None):
+        self._chk(self.L.fm_route_topk_dev(self.h, d_logits, n_experts, K, d_seg_score, d_idx, d_w,
+                                           d_params))
+
     def layer_tail_dev(self, shared_down, d_h_mid, d_eo, d_params, K, d_shared_gate, d_shared_up,
                        d_next_norm_w, eps, d_hidden_out, d_next_input):
         self._chk(self.L.fm_layer_tail_dev(self.h, shared_down, d_h_mid, d_eo, d_params, K,

@@ -45,6 +45,8 @@ int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGeom *g, cons
                              hipStream_t st);
 size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K);
 int fm_launch_layer_tail(const FmTailArgs *a, int bits, int scale_fp16, hipStream_t st);
+int fm_launch_route(const float *d_logits, int n, int K, const float *d_seg_score, int32_t *d_idx,
+                    float *d_w, float *d_params, hipStream_t st);
 }
 
 namespace {
@@ -792,6 +794,22 @@ extern "C" int fm_matvec_prefill(fm_ctx *c, fm_tensor t, const float *X, float *
     if (M < 1 || M > 65535) return fail(c, FM_ERR_ARG, "M %d outside 1..65535", M);
     float *outs[1] = {out};
     return matvec_host(c, &t, 1, X, outs, M);
+}
+
+// ============================================================================
+// routing
+// ============================================================================
+extern "C" int fm_route_topk_dev(fm_ctx *c, const float *d_logits, int n_experts, int K,
+                                 const float *d_seg_score, int32_t *d_idx, float *d_w,
+                                 float *d_params) {
+    if (!c) return FM_ERR_ARG;
+    if (!d_logits || !d_idx || !d_w) return fail(c, FM_ERR_ARG, "null pointer");
+    if (K < 1 || K > FM_MAX_K || K > n_experts)
+        return fail(c, FM_ERR_ARG, "K %d outside 1..min(%d, n_experts)", K, FM_MAX_K);
+    DeviceGuard dg(c->device);
+    int rc = fm_launch_route(d_logits, n_experts, K, d_seg_score, d_idx, d_w, d_params, c->stream);
+    if (rc) return fail(c, rc, "routing over %d experts has no kernel (1..4096)", n_experts);
+    return FM_OK;
 }
 
 // ============================================================================

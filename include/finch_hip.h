@@ -172,6 +172,18 @@ FM_API int fm_matvec_batch(fm_ctx *ctx, const fm_tensor *tensors, int n, const f
 FM_API int fm_matvec_prefill_dev(fm_ctx *ctx, fm_tensor t, const float *d_X, float *d_out, int M);
 FM_API int fm_matvec_prefill(fm_ctx *ctx, fm_tensor t, const float *X, float *out, int M);
 
+/* ---------------------------------------------------------------- routing
+ * Replaces cpu_softmax + cpu_topk + cpu_normalize_weights between the routing GEMVs and
+ * the expert launch (finchmoe/infer.m:1794-1840, 9285-9289), on the device: softmax over
+ * logits[n_experts] (the 8-bit mlp.gate GEMV's output, fm_matvec_batch_dev), the K largest
+ * in the reference's slot order (a score replaces the smallest kept one when strictly
+ * larger; among equal minima the lowest slot), weights renormalised to sum 1.
+ * idx[K], w[K] feed fm_moe_decode_dev as they are.  params (optional, [10]) is filled as
+ * the reference's buf_combine_params: w[0..K-1], zeros, *seg_score (the shared expert's
+ * gate score, optional) at [8] — the operand of fm_layer_tail_dev. */
+FM_API int fm_route_topk_dev(fm_ctx *ctx, const float *d_logits, int n_experts, int K,
+                      const float *d_seg_score, int32_t *d_idx, float *d_w, float *d_params);
+
 /* ---------------------------------------------------------------- layer tail
  * Replaces the five dispatches the reference appends to a layer's expert command
  * buffer (finchmoe/infer.m:9608-9760): swiglu_fused on the shared expert's gate/up

@@ -86,3 +86,121 @@ def test_layer_tail_argument_errors(hip):
     with pytest.raises(FinchError) as e:
         hip.layer_tail_dev(12345, 16, 16, 16, 8, 16, 16, None, 1e-6, 16, None)
     assert e.value.status == fb.ERR_ARG
+
+
+def _route(hip, logits, K, seg=None):
+    import torch
+    d_l = torch.from_numpy(np.ascontiguousarray(logits, np.float32)).cuda()
+    d_idx = torch.full((K,), -7, dtype=torch.int32, device="cuda")
+    d_w = torch.zeros(K, device="cuda")
+    d_p = torch.full((10,), 9.0, device="cuda")
+    d_seg = None if seg is None else torch.tensor([seg], dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    hip.route_topk_dev(d_l.data_ptr(), logits.size, K, None if seg is None else d_seg.data_ptr(),
+                       d_idx.data_ptr(), d_w.data_ptr(), d_p.data_ptr())
+    hip.sync()
+    return d_idx.cpu().numpy(), d_w.cpu().numpy(), d_p.cpu().numpy()
+
+
+@pytest.mark.parametrize("n,K", [(256, 8), (256, 1), (64, 8), (100, 5), (1000, 8), (8, 8)])
+def test_route_matches_reference_scan(hip, orc, n, K):
+    """Indices in the reference's slot order (exact), weights within rounding of the
+    sequential softmax sum."""
+    rng = np.random.default_rng(n * 10 + K)
+    for trial in range(6):
+        logits = (rng.standard_normal(n) * (1 + trial)).astype(np.float32)
+        idx, w, p = _route(hip, logits, K, seg=0.25 * trial)
+        ref_idx, ref_val = orc.topk(orc.softmax(logits), K)
+        ref_w = orc.normalize_weights(ref_val)
+        assert np.array_equal(idx, ref_idx), (trial, idx, ref_idx)
+        assert np.abs(w - ref_w).max() <= 2e-6 * ref_w.max()
+        assert np.array_equal(p[:K], w) and not p[K:8].any() and p[9] == 0
+        assert p[8] == np.float32(0.25 * trial)
+        assert abs(float(w.sum()) - 1) < 1e-6
+
+
+def test_route_ties_and_order(hip, orc):
+    """Equal scores: the earlier index is kept, and a later equal score does not replace it.
+    Ascending scores: every element replaces the then-smallest slot."""
+    logits = np.zeros(256, np.float32)
+    idx, w, _ = _route(hip, logits, 8)
+    assert np.array_equal(idx, np.arange(8))
+    assert np.allclose(w, 1 / 8)
+    logits = np.arange(256, dtype=np.float32) * 0.01
+    idx, _, _ = _route(hip, logits, 8)
+    assert np.array_equal(idx, orc.topk(orc.softmax(logits), 8)[0])
+    assert sorted(idx.tolist()) == list(range(248, 256))
+    logits = np.zeros(256, np.float32)
+    logits[[5, 77, 200]] = 3.0
+    logits[[6, 78]] = 3.0
+    idx, _, _ = _route(hip, logits, 4)
+    assert np.array_equal(idx, orc.topk(orc.softmax(logits), 4)[0])
+
+
+def test_moe_half_of_a_layer_on_device(orc):
+    """routing GEMV -> route -> routed experts -> layer tail without a host round trip
+    (infer.m:9285-9760), against the same chain on the CPU oracle."""
+    from finchmoe_amd import FinchHip
+    hip = FinchHip(0)       # its own expert store
+    try:
+        _moe_half(hip, orc)
+    finally:
+        hip.close()
+
+
+def _moe_half(hip, orc):
+    import torch
+    rng = np.random.default_rng(31)
+    Hh, Ii, Ee, Kk = 2048, 512, 16, 8
+    lo = F.expert_layout(Hh, Ii, 3)
+    blob = F.synth_expert_layer(rng, Ee, Hh, Ii, 3)
+    hip.experts_config(1, Ee, Hh, Ii, 64, 3, 0)
+    hip.experts_upload_layer(0, blob)
+    gate = F.synth_affine_tensor(rng, Ee, Hh, 8, "bf16")
+    seg = F.synth_affine_tensor(rng, 1, Hh, 8, "bf16")
+    sgt = F.synth_affine_tensor(rng, Ii, Hh, 4, "bf16")
+    sut = F.synth_affine_tensor(rng, Ii, Hh, 4, "bf16")
+    sdt = F.synth_affine_tensor(rng, Hh, Ii, 4, "bf16")
+    t_gate = hip.tensor_register(*gate[1:], Ee, Hh, 8)
+    t_seg = hip.tensor_register(*seg[1:], 1, Hh, 8)
+    t_sg = hip.tensor_register(*sgt[1:], Ii, Hh, 4)
+    t_su = hip.tensor_register(*sut[1:], Ii, Hh, 4)
+    t_sd = hip.tensor_register(*sdt[1:], Hh, Ii, 4)
+    x = rng.standard_normal(Hh).astype(np.float32)
+    h_mid = rng.standard_normal(Hh).astype(np.float32)
+    nw = _bf16(1.0 + 0.1 * rng.standard_normal(Hh))
+    d_x, d_hmid = torch.from_numpy(x).cuda(), torch.from_numpy(h_mid).cuda()
+    d_nw = torch.from_numpy(nw.view(np.int16)).cuda()
+    d_log, d_seg = torch.empty(Ee, device="cuda"), torch.empty(1, device="cuda")
+    d_sg, d_su = torch.empty(Ii, device="cuda"), torch.empty(Ii, device="cuda")
+    d_idx = torch.empty(Kk, dtype=torch.int32, device="cuda")
+    d_w, d_p = torch.empty(Kk, device="cuda"), torch.empty(10, device="cuda")
+    d_moe, d_eo = torch.empty(Hh, device="cuda"), torch.empty(Kk, Hh, device="cuda")
+    d_hid, d_next = torch.empty(Hh, device="cuda"), torch.empty(Hh, device="cuda")
+    torch.cuda.synchronize()
+    hip.matvec_batch_dev([t_gate, t_seg, t_sg, t_su], d_x.data_ptr(),
+                         [d_log.data_ptr(), d_seg.data_ptr(), d_sg.data_ptr(), d_su.data_ptr()])
+    hip.route_topk_dev(d_log.data_ptr(), Ee, Kk, d_seg.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(),
+                       d_p.data_ptr())
+    hip.moe_decode_dev(0, d_x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), Kk, d_moe.data_ptr(),
+                       d_eo.data_ptr())
+    hip.layer_tail_dev(t_sd, d_hmid.data_ptr(), d_eo.data_ptr(), d_p.data_ptr(), Kk, d_sg.data_ptr(),
+                       d_su.data_ptr(), d_nw.data_ptr(), 1e-6, d_hid.data_ptr(), d_next.data_ptr())
+    hip.sync()
+    # the same chain on the CPU
+    logits = orc.dequant_matvec(*gate[1:], x, Ee, Hh, 8)
+    segv = orc.dequant_matvec(*seg[1:], x, 1, Hh, 8)
+    sg = orc.dequant_matvec(*sgt[1:], x, Ii, Hh, 4)
+    su = orc.dequant_matvec(*sut[1:], x, Ii, Hh, 4)
+    ridx, rval = orc.topk(orc.softmax(logits), Kk)
+    rw = orc.normalize_weights(rval)
+    assert np.array_equal(d_idx.cpu().numpy(), ridx)
+    _, ref_eo = orc.moe_experts_forward(blob, x, ridx, rw, Hh, Ii, 3)
+    params = np.zeros(10, np.float32)
+    params[:Kk] = rw
+    params[8] = segv[0]
+    ref_h, ref_n = orc.layer_tail(*sdt[1:], h_mid, ref_eo, params, Kk, sg, su, nw)
+    assert_parity(d_hid.cpu().numpy(), ref_h, "hidden")
+    assert_parity(d_next.cpu().numpy(), ref_n, "next input")
+    for t in (t_gate, t_seg, t_sg, t_su, t_sd):
+        hip.tensor_release(t)
