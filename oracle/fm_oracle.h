@@ -26,9 +26,11 @@
  *   matvec                    float64 accumulation, scale=0 and one-hot cases
  *   softmax/top-k/normalise   brute force on small inputs, tie rule
  *   expert loop / combine     float64 recomputation, Inf-scale and w=0 injection
- *   quantizer (orc_quantize_affine)  parity unpinned: bit-exact agreement with
- *                             numpy's float32 division + round-half-even is
- *                             checked against a numpy restatement only.
+ *   quantizer (orc_quantize_affine)  golden vectors written by the reference's own
+ *                             quantizers (tests/golden/quantizer_vectors.npz, made by
+ *                             tests/golden/make_quantizer_vectors.py): codes, packed bytes,
+ *                             scales and biases bit for bit, exact .5 ties and clamped
+ *                             scales included.
  */
 #ifndef FM_ORACLE_H
 #define FM_ORACLE_H

@@ -4,6 +4,8 @@ Each check is chosen so that a plausible mistake (wrong shift, swapped nibble,
 dropped bias, wrong group index) fails it; none of them re-types the oracle's
 own formula against itself.
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -234,8 +236,7 @@ def test_scale_min_k4_all_fields(orc):
 
 @pytest.mark.parametrize("bits", [3, 4])
 def test_quantizer_roundtrip(orc, bits):
-    """Quantizer (parity unpinned against the reference's numpy build, see oracle header):
-    checked against a numpy restatement of the same float32 steps and by the bound
+    """Quantizer against a numpy restatement of the same float32 steps and by the bound
     |w - dequant(q)| <= scale/2 (+ bf16 truncation of scale and bias)."""
     rng = np.random.default_rng(bits)
     w = (rng.standard_normal((16, 256)) * 0.02).astype(np.float32)
@@ -252,3 +253,43 @@ def test_quantizer_roundtrip(orc, bits):
     err = np.abs(deq.reshape(16, 4, 64) - wg)
     bound = scale[:, :, None] * 0.5 + np.abs(scale[:, :, None]) * maxv / 128 + np.abs(lo[:, :, None]) / 128
     assert np.all(err <= bound + 1e-9)
+
+
+def _golden_quantizer():
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "quantizer_vectors.npz")
+    return np.load(path, allow_pickle=False)
+
+
+@pytest.mark.parametrize("key,bits", [("pack3", 3), ("pack4", 4), ("q3", 3), ("qm4", 4), ("qm8", 8),
+                                      ("qne4", 4), ("qne8", 8)])
+def test_quantizer_against_reference_vectors(orc, key, bits):
+    """Codes, packed bytes, scales and biases bit for bit against what the reference's own
+    quantizers produced for the committed inputs (tests/golden/make_quantizer_vectors.py:
+    repack_experts.quantize_affine_pack / quantize_affine_3bit, quantize_model.quantize_affine,
+    quantize_non_experts.quantize_affine) — exact .5 ties, clamped scales, negative ranges."""
+    g = _golden_quantizer()
+    w = g["w"]
+    codes, S, B = orc.quantize_affine(w, bits)
+    packed = np.ascontiguousarray(F.pack_codes(codes, bits)).view(np.uint8).reshape(w.shape[0], -1)
+    assert np.array_equal(packed, g[key + "_w"]), key
+    assert np.array_equal(S, g[key + "_s"]) and np.array_equal(B, g[key + "_b"]), key
+    # and the oracle's own packers on the same codes
+    if bits == 3:
+        assert np.array_equal(orc.pack_3bit(codes).reshape(w.shape[0], -1), g[key + "_w"])
+    else:
+        assert np.array_equal(orc.pack_u32(codes, bits).view(np.uint8).reshape(w.shape[0], -1),
+                              g[key + "_w"])
+
+
+def test_quantizer_vectors_hold_the_hard_cases():
+    """The fixture is worth something only if it contains ties and clamped groups."""
+    g = _golden_quantizer()
+    w = g["w"].reshape(-1, 4, 64)
+    lo, hi = w.min(2), w.max(2)
+    for bits in (3, 4, 8):
+        maxv = np.float32((1 << bits) - 1)
+        scale = np.maximum((hi - lo) / maxv, np.float32(1e-8)).astype(np.float32)
+        q = (w - lo[:, :, None]) / scale[:, :, None]
+        frac = q - np.floor(q)
+        assert np.count_nonzero((frac == 0.5) & (q < maxv)) >= 20, bits
+    assert np.count_nonzero((hi - lo) / np.float32(7) < np.float32(1e-8)) >= 2
