@@ -55,6 +55,8 @@ struct PfArgs {
     int *n_items;
     float *act;        // [M*K][inter], by sorted position
     float *eo;         // [M*K][hidden], by pair id
+    uint4 *xop;        // [M][hidden/64][k step 4][half 2][piece 2]: X as MFMA operand registers
+    float2 *xsums;     // [M][hidden/64]: (xsum, xoff) of every group of every position
 };
 
 // ---- pairing of the 32 codes a lane holds for one group -------------------
@@ -326,9 +328,67 @@ __device__ __forceinline__ void pf_passes(const PfLds<NG> &L, int n_pass, int la
 // ---------------------------------------------------------------- kernels
 // pairs -> grouped by expert, cut into items of <= PF_TM positions.  One workgroup of
 // 1024 threads, one expert per thread for the two prefix sums.
+// X in the form the gate/up kernel multiplies with: per position, group, k step and column
+// half the four operand registers of the hi pieces and of the lo pieces (pf_stage_pair), and
+// per position and group the two sums the bias and offset terms need.  Done once per chunk:
+// a position is multiplied by K experts, and splitting it inside the multiply kernel cost a
+// fifth of that kernel's time.  Task = (position, group, half).
+template <int S>
+__device__ __forceinline__ void pf_prepare_steps(const float *x, uint4 *dst, float &xs, float &xo) {
+    if constexpr (S < 4) {
+        uint32_t hi[4], lo[4];
+        pf_stage_pair<S, 0>(x, hi, lo, xs, xo);
+        pf_stage_pair<S, 1>(x, hi, lo, xs, xo);
+        pf_stage_pair<S, 2>(x, hi, lo, xs, xo);
+        pf_stage_pair<S, 3>(x, hi, lo, xs, xo);
+        dst[4 * S] = make_uint4(hi[0], hi[1], hi[2], hi[3]);          // [k step][half][piece]
+        dst[4 * S + 1] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        pf_prepare_steps<S + 1>(x, dst, xs, xo);
+    }
+}
+
+__device__ __forceinline__ void pf_prepare(const PfArgs &a, int task) {
+    const int NG = a.g.hidden / 64;
+    const int h = task & 1, g = (task >> 1) % NG, m = task / (2 * NG);
+    const bool on = m < a.M;
+    float x[32];
+    if (on) {
+        const float4 *xp = reinterpret_cast<const float4 *>(a.X + (size_t)m * a.g.hidden + 64 * g + 32 * h);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float4 v = xp[i];
+            x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 32; i++) x[i] = 0.0f;
+    }
+    float xs = 0.0f, xo = 0.0f;
+    // this half's registers: index ((m*NG + g)*4 + k)*4 + 2*half + piece
+    uint4 regs[16];
+    pf_prepare_steps<0>(x, regs, xs, xo);
+    // the two halves of a group sit in adjacent lanes
+    xs += fm_dpp<0xB1>(xs);
+    xo += fm_dpp<0xB1>(xo);
+    if (on) {
+        uint4 *dst = a.xop + ((size_t)m * NG + g) * 16;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            dst[4 * k + 2 * h] = regs[4 * k];
+            dst[4 * k + 2 * h + 1] = regs[4 * k + 1];
+        }
+        if (h == 0) a.xsums[(size_t)m * NG + g] = make_float2(xs, xo);
+    }
+}
+
+// workgroup 0 sorts, the others prepare X
 __global__ __launch_bounds__(1024) void fm_pf_sort(PfArgs a) {
     __shared__ int hist[PF_MAX_EXPERTS], cursor[PF_MAX_EXPERTS], scan_a[PF_MAX_EXPERTS],
         scan_b[PF_MAX_EXPERTS];
+    if (blockIdx.x > 0) {
+        pf_prepare(a, (int)((blockIdx.x - 1) * blockDim.x + threadIdx.x));
+        return;
+    }
     const int E = a.g.n_experts, n = a.M * a.K, e = threadIdx.x;
     hist[e] = 0;
     __syncthreads();
@@ -490,7 +550,7 @@ __device__ __forceinline__ void pf_stage_group(const float *x, bool take_hi, uin
 }
 
 template <int GPW, bool GU>
-__global__ __launch_bounds__(512) void fm_pf_slab(PfArgs a) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fm_pf_slab(PfArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // (the host pass cannot allocate the registers of the asm blocks)
     using P = PfSlab<GPW>;
     constexpr int RING = P::RING;
@@ -592,11 +652,37 @@ __global__ __launch_bounds__(512) void fm_pf_slab(PfArgs a) {
         {
             const int pos = n & 15;
             const bool on = pos < item.count;
-            const float *xrow = nullptr;
-            if (on)
-                xrow = GU ? a.X + (size_t)(a.sorted[item.start + pos] / a.K) * a.g.hidden
-                          : a.act + (size_t)(item.start + pos) * a.g.inter;
             float xs[GPW], xo[GPW];
+            if constexpr (GU) {
+                // X was turned into operand registers once per chunk (pf_prepare): lane (m, hh)
+                // takes the hi (m < 16) or lo registers of its position, its groups, its half
+                const int piece = n < 16 ? 0 : 1;
+                const size_t m = on ? (size_t)(a.sorted[item.start + pos] / a.K) : 0;
+                const uint4 *src = a.xop + (m * (a.g.hidden / 64) + GPW * wave) * 16 + 2 * hh + piece;
+                const float2 *sm = a.xsums + m * (a.g.hidden / 64) + GPW * wave;
+#pragma unroll
+                for (int gi = 0; gi < GPW; gi++) {
+#pragma unroll
+                    for (int k = 0; k < 4; k++) A[gi][k] = src[16 * gi + 4 * k];
+                    const float2 v = sm[gi];
+                    xs[gi] = on ? v.x : 0.0f;
+                    xo[gi] = on ? v.y : 0.0f;
+                }
+                // The registers are first used inside the multiply loop, which issues LDS-direct
+                // loads of its own: left alone, the compiler's wait for THESE loads lands in the
+                // loop and drains the ring on every pass.  Touch them here so that it waits now.
+#pragma unroll
+                for (int gi = 0; gi < GPW; gi++)
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        fm_u4 t = __builtin_bit_cast(fm_u4, A[gi][k]);
+                        asm volatile("" : "+v"(t));
+                        if (!on) t = fm_u4{0u, 0u, 0u, 0u};     // rows past the item's positions
+                        A[gi][k] = __builtin_bit_cast(uint4, t);
+                    }
+            } else {
+            const float *xrow = nullptr;
+            if (on) xrow = a.act + (size_t)(item.start + pos) * a.g.inter;
 #pragma unroll
             for (int gi = 0; gi < GPW; gi++) {
                 float x[32];
@@ -617,6 +703,7 @@ __global__ __launch_bounds__(512) void fm_pf_slab(PfArgs a) {
                 // the two halves of a group sit in lanes 32 apart
                 xs[gi] = s0 + __shfl_xor(s0, 32);
                 xo[gi] = o0 + __shfl_xor(o0, 32);
+            }
             }
             // K slots of the bias/offset MFMAs.  GPW = 4: slot = 4*piece + group, one MFMA
             // per term (xsum for the biases, -xoff for the scales).  GPW = 1: slot = 3*term +
@@ -686,7 +773,11 @@ __global__ __launch_bounds__(512) void fm_pf_slab(PfArgs a) {
 #pragma unroll
                     for (int gi = 0; gi < 4; gi++)
 #pragma unroll
-                        for (int d = 0; d < 3; d++) cw[gi][d] = hh ? rd[6 * gi + 3 + d] : rd[6 * gi + d];
+                        // (one side made opaque: the compiler otherwise turns the select into
+                        // rd[6*gi + 3*hh + d], a run-time index into registers, which it expands
+                        // into a compare-and-select over all 24 of them)
+                        for (int d = 0; d < 3; d++)
+                            cw[gi][d] = hh ? fm_opaque(rd[6 * gi + 3 + d]) : rd[6 * gi + d];
                 } else {
                     const uint32_t ac = slot + (uint32_t)(n * P::CB + 12 * hh);
                     const uint32_t as = slot + P::LDS_CODE + 4 * n;
@@ -728,25 +819,36 @@ __global__ __launch_bounds__(512) void fm_pf_slab(PfArgs a) {
                         __builtin_bit_cast(bf8, make_uint4(sideA[0][0], sideA[0][1], sideA[0][2], sideA[0][3])),
                         __builtin_bit_cast(bf8, B1), acc, 0, 0, 0);
                 }
+                // the groups' MFMA chains interleaved (a chain's next MFMA needs the previous
+                // one's result: back to back it would idle the matrix core for most of its
+                // 8 passes), the scales applied once all four are done
+                {
+                    uint32_t v[GPW][16];
+                    f16v dg[GPW];
 #pragma unroll
-                for (int gi = 0; gi < GPW; gi++) {
-                    uint32_t v[16];
-                    pf_unpack<0>(cw[gi], ones, v);
-                    f16v dg;
+                    for (int gi = 0; gi < GPW; gi++) {
+                        pf_unpack<0>(cw[gi], ones, v[gi]);
 #pragma unroll
-                    for (int i = 0; i < 16; i++) dg[i] = 0.0f;
-#pragma unroll
-                    for (int k = 0; k < 4; k++) {
-                        bf8 bop = __builtin_bit_cast(
-                            bf8, make_uint4(v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3]));
-                        dg = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8, A[gi][k]),
-                                                                     bop, dg, 0, 0, 0);
+                        for (int i = 0; i < 16; i++) dg[gi][i] = 0.0f;
                     }
-                    float sc;
-                    if constexpr (GPW == 4) sc = (gi & 1) ? fm_bf16_hi(sw[gi >> 1]) : fm_bf16_lo(sw[gi >> 1]);
-                    else sc = fm_bf16_lo(sw[0]);
 #pragma unroll
-                    for (int i = 0; i < 16; i++) acc[i] = fmaf(sc, dg[i], acc[i]);
+                    for (int k = 0; k < 4; k++)
+#pragma unroll
+                        for (int gi = 0; gi < GPW; gi++) {
+                            bf8 bop = __builtin_bit_cast(
+                                bf8, make_uint4(v[gi][4 * k], v[gi][4 * k + 1], v[gi][4 * k + 2],
+                                                v[gi][4 * k + 3]));
+                            dg[gi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                __builtin_bit_cast(bf8, A[gi][k]), bop, dg[gi], 0, 0, 0);
+                        }
+#pragma unroll
+                    for (int gi = 0; gi < GPW; gi++) {
+                        float sc;
+                        if constexpr (GPW == 4) sc = (gi & 1) ? fm_bf16_hi(sw[gi >> 1]) : fm_bf16_lo(sw[gi >> 1]);
+                        else sc = fm_bf16_lo(sw[0]);
+#pragma unroll
+                        for (int i = 0; i < 16; i++) acc[i] = fmaf(sc, dg[gi][i], acc[i]);
+                    }
                 }
                 // ---- this wave's partial tile: hi + lo rows, register i of every lane
                 {
@@ -861,7 +963,9 @@ extern "C" size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K
     if (!pf_supported(g)) return 0;
     size_t n = (size_t)M * K;
     return align256(n * 4) + align256((g->n_experts + n / PF_TM + 1) * sizeof(PfItem)) + 256 +
-           align256(n * g->inter * 4) + align256(n * g->hidden * 4);
+           align256(n * g->inter * 4) + align256(n * g->hidden * 4) +
+           align256((size_t)M * (g->hidden / 64) * 16 * sizeof(uint4)) +
+           align256((size_t)M * (g->hidden / 64) * sizeof(float2));
 }
 
 extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGeom *g,
@@ -884,8 +988,13 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
     a.items = (PfItem *)ws;               ws += align256((g->n_experts + n / PF_TM + 1) * sizeof(PfItem));
     a.n_items = (int *)ws;                ws += 256;
     a.act = (float *)ws;                  ws += align256(n * g->inter * 4);
-    a.eo = (float *)ws;
-    hipLaunchKernelGGL(fm_pf_sort, dim3(1), dim3(1024), 0, st, a);
+    a.eo = (float *)ws;                   ws += align256(n * g->hidden * 4);
+    a.xop = (uint4 *)ws;                  ws += align256((size_t)M * (g->hidden / 64) * 16 * sizeof(uint4));
+    a.xsums = (float2 *)ws;
+    // workgroup 0 sorts, the rest turn X into operand registers (one thread per position,
+    // group and half)
+    const int prep_tasks = M * (g->hidden / 64) * 2;
+    hipLaunchKernelGGL(fm_pf_sort, dim3(1 + (prep_tasks + 1023) / 1024), dim3(1024), 0, st, a);
     const int max_items = g->n_experts + (int)(n / PF_TM);
 #define PF_LAUNCH(KERN, NG, GRID, NT)                                                              \
     do {                                                                                           \
