@@ -602,7 +602,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     uint32_t issued = 0, consumed = 0;
     bool l_done = t0 >= t1;
     const uint8_t *l_blob = nullptr;
-    if (!l_done) l_blob = fm_uniform(a.layer + (size_t)a.items[l_it].expert * a.g.expert_size);
+    // expert of the item after the one being multiplied: the loader enters that item a few
+    // slices before the multiply does, and a load here would wait for the whole ring
+    int e_ahead = 0;
+    if (!l_done) {
+        l_blob = fm_uniform(a.layer + (size_t)a.items[l_it].expert * a.g.expert_size);
+        if (l_it + 1 < n_items) e_ahead = a.items[l_it + 1].expert;
+    }
     auto issue = [&]() __attribute__((always_inline)) {
         if (l_done) return;
         const uint32_t slot = ring0 + (uint32_t)wpos * P::SLOT;
@@ -631,7 +637,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             } else if (++l_s == n_steps) {
                 l_s = 0;
                 l_it++;
-                l_blob = fm_uniform(a.layer + (size_t)a.items[l_it].expert * a.g.expert_size);
+                l_blob = fm_uniform(a.layer + (size_t)e_ahead * a.g.expert_size);
             }
         }
     };
@@ -639,11 +645,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int k = 0; k < RING; k++) issue();
 
     int c = 0, buf = 0;
+    // What an item's start needs is fetched one item ahead — the item itself, the position
+    // (row of X) this lane multiplies, the next expert for the loader — so that the start
+    // costs one memory round trip (the operand registers) instead of a chain of three, each
+    // of which would also drain the ring.
+    PfItem item_next = PfItem{0, 0, 0, 0};
+    int pair_next = 0;              // pair id of this lane's position (divided by K when used)
+    if (t0 < t1) {
+        item_next = a.items[t0 / n_steps];
+        if (GU && (n & 15) < item_next.count) pair_next = a.sorted[item_next.start + (n & 15)];
+    }
     for (int t = t0; t < t1;) {
         const int it = t / n_steps, s_begin = t - it * n_steps;
         const int s_end = t1 - t < n_steps - s_begin ? s_begin + (t1 - t) : n_steps;
         t += s_end - s_begin;
-        const PfItem item = a.items[it];
+        const PfItem item = item_next;
+        const int m_cur = pair_next / a.K;
+        const bool more = t < t1;                  // this workgroup goes on to item it + 1
+        if (more) item_next = a.items[it + 1];
         // ---- this wave's share of the activation operand, straight into registers:
         // lane (m, hh): M row m = hi piece of position m (m < 16) or lo piece of position
         // m - 16; k slots 8*hh .. 8*hh+7 of every k step = columns 32*hh .. 32*hh+31 of the group
@@ -657,7 +676,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 // X was turned into operand registers once per chunk (pf_prepare): lane (m, hh)
                 // takes the hi (m < 16) or lo registers of its position, its groups, its half
                 const int piece = n < 16 ? 0 : 1;
-                const size_t m = on ? (size_t)(a.sorted[item.start + pos] / a.K) : 0;
+                const size_t m = on ? (size_t)m_cur : 0;
                 const uint4 *src = a.xop + (m * (a.g.hidden / 64) + GPW * wave) * 16 + 2 * hh + piece;
                 const float2 *sm = a.xsums + m * (a.g.hidden / 64) + GPW * wave;
 #pragma unroll
@@ -680,6 +699,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                         if (!on) t = fm_u4{0u, 0u, 0u, 0u};     // rows past the item's positions
                         A[gi][k] = __builtin_bit_cast(uint4, t);
                     }
+                // the next item has arrived with them: its position row, used at its start
+                // (no arithmetic on it here: that would wait for the load now)
+                pair_next = 0;
+                if (more && pos < item_next.count) pair_next = a.sorted[item_next.start + pos];
+                if (more) e_ahead = item_next.expert;     // the loader enters it during this item
             } else {
             const float *xrow = nullptr;
             if (on) xrow = a.act + (size_t)(item.start + pos) * a.g.inter;
