@@ -480,44 +480,40 @@ __global__ __launch_bounds__(512) void fm_pf_down(PfArgs a) {
 }
 
 // ======================================================================
-// K-slab kernels.
+// K-slab kernel (gate/up).
 //
 // The kernels above keep the whole activation operand of an item in LDS
 // (128 KB) and let every wave sweep row tiles over the full K; their weight
 // loads are per-lane 12-byte pieces of 32 different rows, and the address
 // unit, not the matrix core, is the busiest part of the CU.  Here the K
 // dimension is split over the eight waves of the workgroup instead: wave w
-// owns groups [GPW*w, GPW*(w+1)) of every row.
-//   * Its share of the activation operand is 16 registers per group: it is
-//     built straight from global memory into registers, once per item; LDS
-//     holds no activations.
+// owns groups [4w, 4w+4) of every row.
+//   * Its share of the activation operand is 16 registers per group, loaded
+//     ready-made (pf_prepare) once per item; LDS holds no activations.
 //   * Every wave visits every row tile.  A tile-matrix (32 rows of one matrix)
-//     x slab is 32 runs of 24*GPW bytes: the wave copies them, with the rows'
+//     x slab is 32 runs of 96 bytes: the wave copies them, with the rows'
 //     scales and biases, into a ring slot with LDS-direct loads (whole runs,
 //     several slots in flight), and every lane reads its 12-byte pieces back.
-//   * Bias and offset terms ride in one or two extra MFMAs per tile-matrix
-//     whose K slots are (piece, group) of the wave's own groups.
+//   * Bias and offset terms ride in two extra MFMAs per tile-matrix whose K
+//     slots are (piece, group) of the wave's own groups.
 //   * The eight partial tiles are summed through LDS in wave order (wave r sums
 //     result register r of every lane), SwiGLU / store happen there.  One
 //     barrier per step (two tile-matrices), two partial buffers.
 // ======================================================================
-template <int GPW>
 struct PfSlab {
-    static constexpr int NG = 8 * GPW;                  // groups of a whole row
+    static constexpr int GPW = 4;                       // groups per wave
     static constexpr int CB = 24 * GPW;                 // code bytes of a row inside the slab
-    static constexpr int CODE_BYTES = 32 * CB;          // 3072 / 768
-    static constexpr int PS = GPW == 4 ? 16 : 4;        // bytes a lane copies per load (24 B runs: dwords)
+    static constexpr int PS = 16;                       // bytes a lane copies per load
     static constexpr int RP = CB / PS;                  // pieces per row: 6
-    // GPW = 4: a row takes 7 piece slots in LDS (the 7th stays empty): with 96-byte rows the
+    // a row takes 7 piece slots in LDS (the 7th stays empty): with 96-byte rows the
     // 128-bit reads of eight neighbouring rows hit the same banks twice over
-    static constexpr int RS = GPW == 4 ? RP + 1 : RP;   // piece slots per row in LDS
-    static constexpr int PIECES = 32 * RS;              // piece slots of a tile-matrix: 224 / 192
+    static constexpr int RS = RP + 1;                   // piece slots per row in LDS
+    static constexpr int PIECES = 32 * RS;              // piece slots of a tile-matrix: 224
     static constexpr int NQ = (PIECES + 63) / 64;       // LDS-direct loads for the codes
-    static constexpr int LDS_CODE = PIECES * PS;        // 3584 / 768
+    static constexpr int LDS_CODE = PIECES * PS;        // 3584
     static constexpr int SLOT = LDS_CODE + 512;         // + scales 256 + biases 256
     static constexpr int LOADS = NQ + 2;
     static constexpr int RING = 3;
-    static constexpr int NSIDE = GPW == 4 ? 2 : 1;      // MFMAs for the bias/offset terms
     static constexpr int RED_BYTES = 2 * 2 * 8 * 8 * 64 * 4;   // [buffer][matrix][wave][reg][lane]
     static constexpr int LDS_BYTES = 8 * RING * SLOT + RED_BYTES;
 };
@@ -533,26 +529,10 @@ __device__ __forceinline__ void pf_pieces(float v, uint32_t *pc) {
     pc[2] = __float_as_uint(v) >> 16;
 }
 
-// the operand registers of k steps S.. of one group for this lane: the hi pieces
-// (take_hi) or the lo pieces of its 32 activations
-template <int S>
-__device__ __forceinline__ void pf_stage_group(const float *x, bool take_hi, uint4 *A, float &xs,
-                                               float &xo) {
-    if constexpr (S < 4) {
-        uint32_t hi[4], lo[4];
-        pf_stage_pair<S, 0>(x, hi, lo, xs, xo);
-        pf_stage_pair<S, 1>(x, hi, lo, xs, xo);
-        pf_stage_pair<S, 2>(x, hi, lo, xs, xo);
-        pf_stage_pair<S, 3>(x, hi, lo, xs, xo);
-        A[S] = take_hi ? make_uint4(hi[0], hi[1], hi[2], hi[3]) : make_uint4(lo[0], lo[1], lo[2], lo[3]);
-        pf_stage_group<S + 1>(x, take_hi, A, xs, xo);
-    }
-}
-
-template <int GPW, bool GU>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fm_pf_slab(PfArgs a) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fm_pf_gate_up(PfArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // (the host pass cannot allocate the registers of the asm blocks)
-    using P = PfSlab<GPW>;
+    using P = PfSlab;
+    constexpr int GPW = P::GPW;
     constexpr int RING = P::RING;
     extern __shared__ __attribute__((aligned(16))) uint8_t pf2_smem[];
     const int lane = threadIdx.x & 63;
@@ -562,17 +542,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint32_t ring0 = lds0 + (uint32_t)wave * (RING * P::SLOT);
     const uint32_t red0 = lds0 + 8 * RING * P::SLOT;
     const int n_items = *a.n_items;
-    const int in_dim = GU ? a.g.hidden : a.g.inter;
+    const int in_dim = a.g.hidden;
     const int row_bytes = in_dim * 3 / 8, sb_bytes = (in_dim / 64) * 2;
-    const int n_steps = GU ? a.g.inter / 32 : a.g.hidden / 64;   // two tile-matrices per step
+    const int n_steps = a.g.inter / 32;          // a step = the gate and the up tile of 32 rows
     const uint32_t ones = fm_opaque(0x3F803F80u);
     // region offsets of the two tile-matrices of a step and their row distance
-    const uint32_t w_off0 = GU ? a.g.gate_w : a.g.down_w, s_off0 = GU ? a.g.gate_s : a.g.down_s,
-                   b_off0 = GU ? a.g.gate_b : a.g.down_b;
-    const uint32_t w_d = GU ? a.g.up_w - a.g.gate_w : 32u * row_bytes;
-    const uint32_t s_d = GU ? a.g.up_s - a.g.gate_s : 32u * sb_bytes;
-    const uint32_t b_d = GU ? a.g.up_b - a.g.gate_b : 32u * sb_bytes;
-    const uint32_t step_rows = GU ? 32u : 64u;
+    const uint32_t w_off0 = a.g.gate_w, s_off0 = a.g.gate_s, b_off0 = a.g.gate_b;
+    const uint32_t w_d = a.g.up_w - a.g.gate_w, s_d = a.g.up_s - a.g.gate_s, b_d = a.g.up_b - a.g.gate_b;
+    const uint32_t step_rows = 32u;
     // this lane's pieces of a slot copy
     uint32_t coff[P::NQ];
     bool cvalid[P::NQ];
@@ -585,9 +562,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     // scales / biases of the slab: 2*GPW bytes per row, fetched as whole dwords
     const int sb_slab = (2 * GPW * wave) & ~3;
-    const bool svalid = GPW >= 2 ? true : lane < 32;
-    const uint32_t soff = GPW >= 2 ? (uint32_t)((lane >> 1) * sb_bytes + sb_slab + 4 * (lane & 1))
-                                   : (uint32_t)(lane * sb_bytes + sb_slab);
+    const uint32_t soff = (uint32_t)((lane >> 1) * sb_bytes + sb_slab + 4 * (lane & 1));
 
     // ---- this workgroup's share of the launch: steps [t0, t1) of the sequence
     // (item, step), items in order — every workgroup gets the same number of steps
@@ -622,12 +597,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(wb + coff[j]),
                                                  (fm_lptr)(uintptr_t)(slot + 64 * P::PS * j),
                                                  P::PS, 0, 0);
-        if (svalid) {
-            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(sb + soff),
-                                             (fm_lptr)(uintptr_t)(slot + P::LDS_CODE), 4, 0, 0);
-            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(bb + soff),
-                                             (fm_lptr)(uintptr_t)(slot + P::LDS_CODE + 256), 4, 0, 0);
-        }
+        __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(sb + soff),
+                                         (fm_lptr)(uintptr_t)(slot + P::LDS_CODE), 4, 0, 0);
+        __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(bb + soff),
+                                         (fm_lptr)(uintptr_t)(slot + P::LDS_CODE + 256), 4, 0, 0);
         wpos = wpos + 1 == RING ? 0 : wpos + 1;
         issued++;
         l_mat ^= 1;
@@ -653,7 +626,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     int pair_next = 0;              // pair id of this lane's position (divided by K when used)
     if (t0 < t1) {
         item_next = a.items[t0 / n_steps];
-        if (GU && (n & 15) < item_next.count) pair_next = a.sorted[item_next.start + (n & 15)];
+        if ((n & 15) < item_next.count) pair_next = a.sorted[item_next.start + (n & 15)];
     }
     for (int t = t0; t < t1;) {
         const int it = t / n_steps, s_begin = t - it * n_steps;
@@ -667,12 +640,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         // lane (m, hh): M row m = hi piece of position m (m < 16) or lo piece of position
         // m - 16; k slots 8*hh .. 8*hh+7 of every k step = columns 32*hh .. 32*hh+31 of the group
         uint4 A[GPW][4];
-        uint32_t sideA[P::NSIDE][4];
+        uint32_t sideA[2][4];
         {
             const int pos = n & 15;
             const bool on = pos < item.count;
             float xs[GPW], xo[GPW];
-            if constexpr (GU) {
+            {
                 // X was turned into operand registers once per chunk (pf_prepare): lane (m, hh)
                 // takes the hi (m < 16) or lo registers of its position, its groups, its half
                 const int piece = n < 16 ? 0 : 1;
@@ -704,63 +677,25 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 pair_next = 0;
                 if (more && pos < item_next.count) pair_next = a.sorted[item_next.start + pos];
                 if (more) e_ahead = item_next.expert;     // the loader enters it during this item
-            } else {
-            const float *xrow = nullptr;
-            if (on) xrow = a.act + (size_t)(item.start + pos) * a.g.inter;
-#pragma unroll
-            for (int gi = 0; gi < GPW; gi++) {
-                float x[32];
-                if (on) {
-                    const float4 *xp =
-                        reinterpret_cast<const float4 *>(xrow + 64 * (GPW * wave + gi) + 32 * hh);
-#pragma unroll
-                    for (int i = 0; i < 8; i++) {
-                        float4 v = xp[i];
-                        x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
-                    }
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 32; i++) x[i] = 0.0f;
-                }
-                float s0 = 0.0f, o0 = 0.0f;
-                pf_stage_group<0>(x, n < 16, A[gi], s0, o0);
-                // the two halves of a group sit in lanes 32 apart
-                xs[gi] = s0 + __shfl_xor(s0, 32);
-                xo[gi] = o0 + __shfl_xor(o0, 32);
             }
-            }
-            // K slots of the bias/offset MFMAs.  GPW = 4: slot = 4*piece + group, one MFMA
-            // per term (xsum for the biases, -xoff for the scales).  GPW = 1: slot = 3*term +
-            // piece, one MFMA.  Rows 16..31 (lo pieces) take no part.
-            if constexpr (GPW == 4) {
+            // K slots of the bias/offset MFMAs: slot = 4*piece + group, one MFMA per term (xsum
+            // for the biases, -xoff for the scales).  Rows 16..31 (lo pieces) take no part.
 #pragma unroll
-                for (int term = 0; term < 2; term++) {
-                    uint32_t pc[4][3];
+            for (int term = 0; term < 2; term++) {
+                uint32_t pc[4][3];
 #pragma unroll
-                    for (int gi = 0; gi < 4; gi++) pf_pieces(term ? -xo[gi] : xs[gi], pc[gi]);
-                    const int p0 = hh ? 2 : 0;
-                    sideA[term][0] = pc[0][p0] | (pc[1][p0] << 16);
-                    sideA[term][1] = pc[2][p0] | (pc[3][p0] << 16);
-                    sideA[term][2] = hh ? 0u : pc[0][1] | (pc[1][1] << 16);
-                    sideA[term][3] = hh ? 0u : pc[2][1] | (pc[3][1] << 16);
-                    if (n >= 16) sideA[term][0] = sideA[term][1] = sideA[term][2] = sideA[term][3] = 0u;
-                }
-            } else {
-                uint32_t ps[3], po[3];
-                pf_pieces(xs[0], ps);
-                pf_pieces(-xo[0], po);
-                const bool z = hh || n >= 16;
-                sideA[0][0] = z ? 0u : ps[0] | (ps[1] << 16);
-                sideA[0][1] = z ? 0u : ps[2] | (po[0] << 16);
-                sideA[0][2] = z ? 0u : po[1] | (po[2] << 16);
-                sideA[0][3] = 0u;
+                for (int gi = 0; gi < 4; gi++) pf_pieces(term ? -xo[gi] : xs[gi], pc[gi]);
+                const int p0 = hh ? 2 : 0;
+                sideA[term][0] = pc[0][p0] | (pc[1][p0] << 16);
+                sideA[term][1] = pc[2][p0] | (pc[3][p0] << 16);
+                sideA[term][2] = hh ? 0u : pc[0][1] | (pc[1][1] << 16);
+                sideA[term][3] = hh ? 0u : pc[2][1] | (pc[3][1] << 16);
+                if (n >= 16) sideA[term][0] = sideA[term][1] = sideA[term][2] = sideA[term][3] = 0u;
             }
         }
-        // output position of result register r = wave of this lane, and (down) its pair
+        // output position of result register r = wave of this lane
         const int my_pos = 8 * (wave >> 2) + 4 * hh + (wave & 3);
         const bool my_on = my_pos < item.count;
-        int my_pair = 0;
-        if (!GU && my_on) my_pair = a.sorted[item.start + my_pos];
 
         for (int s = s_begin; s < s_end; s++) {
 #pragma unroll
@@ -774,7 +709,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 else fm_dma_wait<0>(true);
                 const uint32_t slot = ring0 + (uint32_t)c * P::SLOT;
                 uint32_t cw[GPW][3], sw[2], bw[2];
-                if constexpr (GPW == 4) {
+                {
                     // the whole 96-byte run of the row (both half lanes read the same
                     // pieces), then this lane's half of every group
                     const uint32_t ac = slot + (uint32_t)(n * (P::RS * 16));
@@ -794,29 +729,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     const uint32_t rd[24] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w,
                                              r2.x, r2.y, r2.z, r2.w, r3.x, r3.y, r3.z, r3.w,
                                              r4.x, r4.y, r4.z, r4.w, r5.x, r5.y, r5.z, r5.w};
+                    // (one side made opaque: the compiler otherwise turns the select into
+                    // rd[6*gi + 3*hh + d], a run-time index into registers, which it expands
+                    // into a compare-and-select over all 24 of them)
 #pragma unroll
                     for (int gi = 0; gi < 4; gi++)
 #pragma unroll
-                        // (one side made opaque: the compiler otherwise turns the select into
-                        // rd[6*gi + 3*hh + d], a run-time index into registers, which it expands
-                        // into a compare-and-select over all 24 of them)
                         for (int d = 0; d < 3; d++)
                             cw[gi][d] = hh ? fm_opaque(rd[6 * gi + 3 + d]) : rd[6 * gi + d];
-                } else {
-                    const uint32_t ac = slot + (uint32_t)(n * P::CB + 12 * hh);
-                    const uint32_t as = slot + P::LDS_CODE + 4 * n;
-                    asm volatile("ds_read_b32 %0, %5\n\tds_read_b32 %1, %5 offset:4\n\t"
-                                 "ds_read_b32 %2, %5 offset:8\n\tds_read_b32 %3, %6\n\t"
-                                 "ds_read_b32 %4, %6 offset:256\n\ts_waitcnt lgkmcnt(0)"
-                                 : "=&v"(cw[0][0]), "=&v"(cw[0][1]), "=&v"(cw[0][2]), "=&v"(sw[0]),
-                                   "=&v"(bw[0])
-                                 : "v"(ac), "v"(as)
-                                 : "memory");
-                    // the slab's 16-bit scale / bias inside the dword that was fetched
-                    const int sh = 16 * (wave & 1);
-                    sw[0] = (sw[0] >> sh) & 0xFFFFu;
-                    bw[0] = (bw[0] >> sh) & 0xFFFFu;
-                    sw[1] = bw[1] = 0u;
                 }
                 consumed++;
                 c = c + 1 == RING ? 0 : c + 1;
@@ -826,23 +746,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 f16v acc;
 #pragma unroll
                 for (int i = 0; i < 16; i++) acc[i] = 0.0f;
-                if constexpr (GPW == 4) {
-                    const uint4 Bb = hh ? make_uint4(bw[0], bw[1], 0u, 0u) : make_uint4(bw[0], bw[1], bw[0], bw[1]);
-                    const uint4 Bs = hh ? make_uint4(sw[0], sw[1], 0u, 0u) : make_uint4(sw[0], sw[1], sw[0], sw[1]);
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf8, make_uint4(sideA[0][0], sideA[0][1], sideA[0][2], sideA[0][3])),
-                        __builtin_bit_cast(bf8, Bb), acc, 0, 0, 0);
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf8, make_uint4(sideA[1][0], sideA[1][1], sideA[1][2], sideA[1][3])),
-                        __builtin_bit_cast(bf8, Bs), acc, 0, 0, 0);
-                } else {
-                    const uint32_t b = bw[0], sc16 = sw[0];
-                    const uint4 B1 = hh ? make_uint4(0u, 0u, 0u, 0u)
-                                        : make_uint4(b | (b << 16), b | (sc16 << 16), sc16 | (sc16 << 16), 0u);
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf8, make_uint4(sideA[0][0], sideA[0][1], sideA[0][2], sideA[0][3])),
-                        __builtin_bit_cast(bf8, B1), acc, 0, 0, 0);
-                }
+                const uint4 Bb = hh ? make_uint4(bw[0], bw[1], 0u, 0u) : make_uint4(bw[0], bw[1], bw[0], bw[1]);
+                const uint4 Bs = hh ? make_uint4(sw[0], sw[1], 0u, 0u) : make_uint4(sw[0], sw[1], sw[0], sw[1]);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                    __builtin_bit_cast(bf8, make_uint4(sideA[0][0], sideA[0][1], sideA[0][2], sideA[0][3])),
+                    __builtin_bit_cast(bf8, Bb), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                    __builtin_bit_cast(bf8, make_uint4(sideA[1][0], sideA[1][1], sideA[1][2], sideA[1][3])),
+                    __builtin_bit_cast(bf8, Bs), acc, 0, 0, 0);
                 // the groups' MFMA chains interleaved (a chain's next MFMA needs the previous
                 // one's result: back to back it would idle the matrix core for most of its
                 // 8 passes), the scales applied once all four are done
@@ -867,9 +778,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                         }
 #pragma unroll
                     for (int gi = 0; gi < GPW; gi++) {
-                        float sc;
-                        if constexpr (GPW == 4) sc = (gi & 1) ? fm_bf16_hi(sw[gi >> 1]) : fm_bf16_lo(sw[gi >> 1]);
-                        else sc = fm_bf16_lo(sw[0]);
+                        const float sc = (gi & 1) ? fm_bf16_hi(sw[gi >> 1]) : fm_bf16_lo(sw[gi >> 1]);
 #pragma unroll
                         for (int i = 0; i < 16; i++) acc[i] = fmaf(sc, dg[gi][i], acc[i]);
                     }
@@ -916,13 +825,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     t1 += p[8 + w2];
                 }
                 if (my_on) {
-                    if constexpr (GU) {
-                        a.act[(size_t)(item.start + my_pos) * a.g.inter + 32 * s + n] = fm_silu_mul(t0, t1);
-                    } else {
-                        float *o = a.eo + (size_t)my_pair * a.g.hidden + 64 * s + n;
-                        o[0] = t0;
-                        o[32] = t1;
-                    }
+                    a.act[(size_t)(item.start + my_pos) * a.g.inter + 32 * s + n] = fm_silu_mul(t0, t1);
                 }
             }
             buf ^= 1;
@@ -1030,14 +933,13 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
     // tiles, a group tile, 16 operand registers, loads in flight), which caps a SIMD at two
     // waves; capping the registers instead made them spill and run 2-5x slower
     const int grid = max_items < n_cu ? max_items : n_cu;
-    // gate/up: K split over the waves (fm_pf_slab).  down: whole K per wave (fm_pf_down) —
+    // gate/up: K split over the waves (fm_pf_gate_up).  down: whole K per wave (fm_pf_down) —
     // with one group (four MFMAs) per wave and tile the split's per-tile overhead outweighs
     // what it saves.
     {
         static FmLdsAttr attr;
-        auto kfn = fm_pf_slab<4, true>;
-        if (!fm_dyn_lds_ready(attr, (const void *)kfn, PfSlab<4>::LDS_BYTES)) return FM_ERR_HIP;
-        hipLaunchKernelGGL(kfn, dim3(grid), dim3(512), PfSlab<4>::LDS_BYTES, st, a);
+        if (!fm_dyn_lds_ready(attr, (const void *)fm_pf_gate_up, PfSlab::LDS_BYTES)) return FM_ERR_HIP;
+        hipLaunchKernelGGL(fm_pf_gate_up, dim3(grid), dim3(512), PfSlab::LDS_BYTES, st, a);
     }
     PF_LAUNCH(fm_pf_down, 8, grid, 512);
 #undef PF_LAUNCH
