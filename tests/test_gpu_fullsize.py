@@ -1,0 +1,105 @@
+"""The benchmark's full sizes (40 layers x 256 experts of 3-bit g64 weights resident, 14.09 GB;
+512-position chunk on 256 experts), checked through properties that do not need the oracle to
+process 14 GB: the 40-layer step equals the 40 single-layer calls bit for bit; the weighted sum
+equals the per-expert outputs combined in slot order; sampled (layer, slot) expert outputs equal
+the CPU oracle on the routed experts' bytes copied back; a prefill chunk equals the per-position
+path.  Weights are generated on the device exactly as bench.py does."""
+import numpy as np
+import pytest
+
+from finchmoe_amd import formats as F
+from .conftest import assert_parity, cosine, rel_err
+
+pytestmark = pytest.mark.gpu
+
+H, I, E, K, L = 2048, 512, 256, 8, 40
+
+
+@pytest.fixture(scope="module")
+def full_store():
+    import torch
+    from bench import fill_affine_layer, zipf_routing
+    from finchmoe_amd import FinchHip
+    dev = torch.device("cuda:0")
+    lo = F.expert_layout(H, I, 3)
+    es = lo["expert_size"]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2024)
+    blob = torch.empty(L, E, es, dtype=torch.uint8, device=dev)
+    for l in range(L):
+        fill_affine_layer(blob[l], lo, 3, gen)
+    ctx = FinchHip(0)
+    ctx.experts_config(L, E, H, I, 64, 3, 0)
+    for l in range(L):
+        ctx.experts_adopt_layer(l, blob[l].data_ptr(), E * es)
+    idx, w = zipf_routing(np.random.default_rng(5), 2, L, E, K)
+    yield ctx, blob, lo, idx, w
+    ctx.close()
+    del blob
+    torch.cuda.empty_cache()
+
+
+def test_full_step_equals_layer_calls_and_oracle(full_store, orc):
+    import torch
+    ctx, blob, lo, idx, w = full_store
+    es = lo["expert_size"]
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((L, H)).astype(np.float32)
+    d_x = torch.from_numpy(x).cuda()
+    for tok in range(2):
+        d_idx, d_w = torch.from_numpy(idx[tok]).cuda(), torch.from_numpy(w[tok]).cuda()
+        d_out = torch.zeros(L, H, device="cuda")
+        d_eo = torch.zeros(L, K, H, device="cuda")
+        torch.cuda.synchronize()
+        ctx.moe_decode_step_dev(0, L, d_x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K,
+                                d_out.data_ptr(), d_eo.data_ptr())
+        ctx.sync()
+        out, eo = d_out.cpu().numpy(), d_eo.cpu().numpy()
+        assert np.isfinite(out).all()
+        # (1) one launch over 40 layers == 40 launches
+        s_out = torch.zeros(H, device="cuda")
+        s_eo = torch.zeros(K, H, device="cuda")
+        for l in range(L):
+            ctx.moe_decode_dev(l, d_x.data_ptr() + l * H * 4, d_idx.data_ptr() + l * K * 4,
+                               d_w.data_ptr() + l * K * 4, K, s_out.data_ptr(), s_eo.data_ptr())
+            ctx.sync()
+            assert np.array_equal(s_out.cpu().numpy(), out[l]), l
+            assert np.array_equal(s_eo.cpu().numpy(), eo[l]), l
+        # (2) the weighted sum in slot order, fp32 (shaders.metal:2213-2228)
+        for l in range(L):
+            acc = np.zeros(H, np.float32)
+            for k in range(K):
+                acc = acc + w[tok, l, k] * eo[l, k]
+            assert rel_err(out[l], acc) < 1e-6, l
+        # (3) the routed experts of three layers against the oracle on their own bytes
+        for l in (0, 17, 39):
+            mini = np.concatenate([blob[l, int(e)].cpu().numpy() for e in idx[tok, l]])
+            ref, ref_eo = orc.moe_experts_forward(mini, x[l], np.arange(K, dtype=np.int32), w[tok, l],
+                                                  H, I, 3, nthreads=8)
+            assert_parity(eo[l], ref_eo, "expert_out layer %d" % l)
+            assert_parity(out[l], ref, "layer %d" % l)
+
+
+def test_full_chunk_equals_positions(full_store, orc):
+    """512 positions x top-8 over all 256 experts of a layer (4096 pairs): every sampled position
+    equals its per-position call within the bar, a repeat is bit-identical, and one position is
+    checked against the oracle."""
+    import torch
+    from bench import zipf_routing
+    ctx, blob, lo, _, _ = full_store
+    M, layer = 512, 3
+    rng = np.random.default_rng(8)
+    idx, w = zipf_routing(rng, M, 1, E, K)
+    idx, w = np.ascontiguousarray(idx[:, 0]), np.ascontiguousarray(w[:, 0])
+    X = torch.randn(M, H).to(torch.bfloat16).to(torch.float32).numpy()
+    out = ctx.moe_prefill(layer, X, idx, w)
+    assert np.isfinite(out).all()
+    assert np.array_equal(ctx.moe_prefill(layer, X, idx, w), out)
+    # cover the hot experts' many items as well as the tail
+    for m in list(range(0, M, 37)) + [M - 1]:
+        single, _ = ctx.moe_decode(layer, X[m], idx[m], w[m])
+        assert rel_err(out[m], single) < 1e-3 and cosine(out[m], single) > 0.99999, m
+    m = 123
+    mini = np.concatenate([blob[layer, int(e)].cpu().numpy() for e in idx[m]])
+    ref, _ = orc.moe_experts_forward(mini, X[m], np.arange(K, dtype=np.int32), w[m], H, I, 3, nthreads=8)
+    assert_parity(out[m], ref, "position %d" % m)
