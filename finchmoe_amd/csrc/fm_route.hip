@@ -23,16 +23,27 @@ struct RouteArgs {
     float *params;               // [10] or null: weights, zeros, score at [8]
 };
 
+// max / min over the wave's 64 lanes, the result in a scalar register: DPP inside each row
+// of 16 lanes, then the four row results read lane by lane (no LDS round trips)
+template <bool MAX>
+__device__ __forceinline__ float pick(float a, float b) { return MAX ? fmaxf(a, b) : fminf(a, b); }
+template <bool MAX>
+__device__ __forceinline__ float row_reduce(float v) {
+    v = pick<MAX>(v, fm_dpp<0xB1>(v));     // quad_perm [1,0,3,2]
+    v = pick<MAX>(v, fm_dpp<0x4E>(v));     // quad_perm [2,3,0,1]
+    v = pick<MAX>(v, fm_dpp<0x141>(v));    // row_half_mirror: 8 lanes
+    return v;
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) v = fmaxf(v, __shfl_xor(v, d));
-    return v;
+    v = row_reduce<true>(v);
+    v = fmaxf(v, fm_dpp<0x140>(v));        // row_mirror: 16 lanes
+    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
 }
-__device__ __forceinline__ float wave_min(float v) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) v = fminf(v, __shfl_xor(v, d));
-    return v;
-}
+// min over lanes 0..7 (the K slots; lanes K.. hold +inf)
+__device__ __forceinline__ float slots_min(float v) { return lane_value(row_reduce<false>(v), 0); }
 
 #define FM_ROUTE_MAX 4096
 
@@ -69,12 +80,12 @@ __global__ __launch_bounds__(64) void fm_route(RouteArgs a) {
         uint64_t pending = __ballot(s > min_val);
         while (pending) {
             const int src = __ffsll((unsigned long long)pending) - 1;
-            const float sv = __shfl(s, src);
+            const float sv = lane_value(s, src);
             if (lane == min_k) {
                 val = sv;
                 ind = base + src;
             }
-            min_val = wave_min(val);
+            min_val = slots_min(val);
             min_k = __ffsll((unsigned long long)__ballot(val == min_val)) - 1;
             // scores after src that still beat the new minimum
             const uint64_t later = src == 63 ? 0ull : ~0ull << (src + 1);
@@ -83,7 +94,9 @@ __global__ __launch_bounds__(64) void fm_route(RouteArgs a) {
     }
     // renormalise in slot order (infer.m:1833-1840)
     float total = 0.0f;
-    for (int k = 0; k < a.K; k++) total += __shfl(val, k);
+#pragma unroll
+    for (int k = 0; k < FM_MAX_K; k++)
+        if (k < a.K) total += lane_value(val, k);
     float wk = val;
     if (total > 0.0f) wk = val * (1.0f / total);
     if (lane < a.K) {
