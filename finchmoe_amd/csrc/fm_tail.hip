@@ -36,11 +36,19 @@ __global__ __launch_bounds__(256) void fm_layer_tail(FmTailArgs a) {
     const int row = (blockIdx.x * 4 + wave) * RPS + r;
     const int row_bytes = a.inter * BITS / 8, sb_row_bytes = (a.inter / 64) * 2;
 
-    // the row's codes first: they do not depend on the activations
+    // everything that depends on nothing is fetched first, so that the loads overlap: the
+    // row's codes, and what the combine adds to the row (all lanes of a row load the same)
     FmRowSlice<BITS> ws;
     fm_load_slice<BITS>(ws, a.W + (size_t)row * row_bytes + (size_t)c * BPL,
                         a.S + (size_t)row * sb_row_bytes + (size_t)c * 4,
                         a.B + (size_t)row * sb_row_bytes + (size_t)c * 4);
+    float eo[FM_MAX_K], pw[FM_MAX_K];
+#pragma unroll
+    for (int k = 0; k < FM_MAX_K; k++) {
+        eo[k] = k < a.K ? a.expert_out[(size_t)k * a.hidden + row] : 0.0f;
+        pw[k] = k < a.K ? a.params[k] : 0.0f;
+    }
+    const float hm = a.h_mid[row], score = a.params[8];
     for (int j = threadIdx.x; j < a.inter; j += blockDim.x)
         tail_act[j] = fm_silu_mul(a.shared_gate[j], a.shared_up[j]);
     __syncthreads();
@@ -53,9 +61,9 @@ __global__ __launch_bounds__(256) void fm_layer_tail(FmTailArgs a) {
         float moe = 0.0f;
 #pragma unroll
         for (int k = 0; k < FM_MAX_K; k++)
-            if (k < a.K) moe += a.params[k] * a.expert_out[(size_t)k * a.hidden + row];
-        const float shared_gate = 1.0f / (1.0f + expf(-a.params[8]));
-        const float hv = a.h_mid[row] + moe + shared_gate * shared_out;
+            if (k < a.K) moe += pw[k] * eo[k];
+        const float shared_gate = 1.0f / (1.0f + expf(-score));
+        const float hv = hm + moe + shared_gate * shared_out;
         tail_st(a.hidden_out + row, hv);
         sq = hv * hv;
     }
@@ -73,9 +81,13 @@ __global__ __launch_bounds__(256) void fm_layer_tail(FmTailArgs a) {
     __syncthreads();
     if (ticket != gridDim.x - 1) return;
 
-    // last workgroup: every other one has stored its rows and its partial sum
+    // last workgroup: every other one has stored its rows and its partial sum.  The partials
+    // are fetched side by side and added in workgroup order.
+    __shared__ float parts[1024];
+    for (unsigned int i = threadIdx.x; i < gridDim.x; i += blockDim.x) parts[i] = tail_ld(a.partial + i);
+    __syncthreads();
     float sum_sq = 0.0f;
-    for (unsigned int i = 0; i < gridDim.x; i++) sum_sq += tail_ld(a.partial + i);
+    for (unsigned int i = 0; i < gridDim.x; i++) sum_sq += parts[i];
     const float inv_rms = 1.0f / sqrtf(sum_sq / (float)a.hidden + a.eps);   // infer.m:1771-1772
     for (int j = threadIdx.x; j < a.hidden; j += blockDim.x)
         a.next_in[j] = tail_ld(a.hidden_out + j) * inv_rms * __uint_as_float((uint32_t)a.norm_w[j] << 16);
@@ -90,7 +102,7 @@ int launch_tail_t(const FmTailArgs &a, hipStream_t st) {
 #define FM_T(L)                                                                                  \
     do {                                                                                         \
         const int rows = 4 * (FM_WAVE / L);                                                      \
-        if (a.hidden % rows) return FM_ERR_UNSUPPORTED;                                          \
+        if (a.hidden % rows || a.hidden / rows > 1024) return FM_ERR_UNSUPPORTED;                \
         hipLaunchKernelGGL((fm_layer_tail<BITS, L, FP16>), dim3(a.hidden / rows), dim3(256), sh, \
                            st, a);                                                               \
     } while (0)
