@@ -11,6 +11,8 @@
 #include "fm_mfma.h"
 #include "fm_ring.h"
 
+#include <type_traits>
+
 #define FM_MAX_BATCH 8
 
 struct FmDenseSpec {
@@ -128,6 +130,18 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
     const long wg0 = (long)total_units * blockIdx.x / gridDim.x,
                wg1 = (long)total_units * (blockIdx.x + 1) / gridDim.x;
     const uint32_t n_units = (uint32_t)(wg1 - wg0);
+    // The launch is a chain of memory round trips; the activations' is started first so
+    // that it runs beside the counter set-up and the first weight loads instead of after them.
+    typedef typename std::conditional<BITS == 8, FmBuildSlot<4>, FmBuildSlot<BITS>>::type BuildSlot;
+    BuildSlot bslot;
+    FmActX<LPR> xr[NS];
+    if constexpr (BITS != 8) {
+        bslot.init();
+#pragma unroll
+        for (int k = 0; k < NS; k++)
+            if (threadIdx.x < 256)
+                fm_act_load<BITS, LPR, false>(a.x + (size_t)m * a.in_dim + k * SLAB_COLS, bslot, xr[k]);
+    }
     if (threadIdx.x == 0) next_unit = 0u;
     __syncthreads();                 // the counter is set
     uint32_t woff, soff;
@@ -219,17 +233,11 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
             if (ch == 0) w.out[(size_t)m * w.out_dim + w.row0 + ris] = v;
         }
     } else {
-    // the activation registers of every slab, built once
-    FmBuildSlot<BITS> bslot;
-    bslot.init();
+    // the activation registers of every slab, built once (the activations were requested
+    // at the kernel's start)
 #pragma unroll
-    for (int k = 0; k < NS; k++) {
-        if (threadIdx.x < 256) {
-            FmActX<LPR> xr;
-            fm_act_load<BITS, LPR, false>(a.x + (size_t)m * a.in_dim + k * SLAB_COLS, bslot, xr);
-            fm_act_build<BITS, LPR>(xr, bslot, img[k]);
-        }
-    }
+    for (int k = 0; k < NS; k++)
+        if (threadIdx.x < 256) fm_act_build<BITS, LPR>(xr[k], bslot, img[k]);
     __syncthreads();
     FmActRegs ar[NS];
 #pragma unroll
