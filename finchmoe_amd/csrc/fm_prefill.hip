@@ -398,18 +398,29 @@ __global__ __launch_bounds__(1024) void fm_pf_sort(PfArgs a) {
     }
     __syncthreads();
     const int cnt = e < E ? hist[e] : 0, nit = (cnt + PF_TM - 1) / PF_TM;
-    // inclusive scans of the pair counts and the item counts (Hillis-Steele)
-    scan_a[e] = cnt;
-    scan_b[e] = nit;
-    __syncthreads();
-    for (int d = 1; d < 1024; d <<= 1) {
-        int va = e >= d ? scan_a[e - d] : 0, vb = e >= d ? scan_b[e - d] : 0;
-        __syncthreads();
-        scan_a[e] += va;
-        scan_b[e] += vb;
-        __syncthreads();
+    // inclusive scans of the pair counts and the item counts: inside each wave by lane
+    // shifts, the 16 wave totals by wave 0, two barriers in all
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    int sa = cnt, sb = nit;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int va = __shfl_up(sa, d), vb = __shfl_up(sb, d);
+        if (lane >= d) sa += va, sb += vb;
     }
-    const int off = scan_a[e] - cnt, ioff = scan_b[e] - nit;
+    if (lane == 63) scan_a[wv] = sa, scan_b[wv] = sb;
+    __syncthreads();
+    if (wv == 0) {
+        int ta = lane < 16 ? scan_a[lane] : 0, tb = lane < 16 ? scan_b[lane] : 0;
+#pragma unroll
+        for (int d = 1; d < 16; d <<= 1) {
+            const int va = __shfl_up(ta, d), vb = __shfl_up(tb, d);
+            if (lane >= d) ta += va, tb += vb;
+        }
+        if (lane < 16) scan_a[lane] = ta, scan_b[lane] = tb;     // inclusive totals of waves 0..lane
+    }
+    __syncthreads();
+    if (wv > 0) sa += scan_a[wv - 1], sb += scan_b[wv - 1];
+    const int off = sa - cnt, ioff = sb - nit;
     cursor[e] = off;
     for (int s = 0; s < nit; s++) {
         PfItem it;
@@ -419,7 +430,7 @@ __global__ __launch_bounds__(1024) void fm_pf_sort(PfArgs a) {
         it.pad = 0;
         a.items[ioff + s] = it;
     }
-    if (e == 1023) *a.n_items = scan_b[1023];
+    if (e == 1023) *a.n_items = sb;
     __syncthreads();
     for (int p = threadIdx.x; p < n; p += blockDim.x) {
         int x = a.idx[p];
