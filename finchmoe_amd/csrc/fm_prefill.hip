@@ -26,9 +26,13 @@
 // 16 results, all of weight row n — so a lane needs ONE scale per group.
 // A lane's codes for one group are half a group: 32 codes = 12 bytes.
 //
-// Work item = (expert, up to 16 of its positions).  A 512-thread workgroup takes
-// items round-robin; per item it builds the activation operand image in LDS
-// (128 KB for 2048 columns) and its eight waves sweep the row tiles.
+// Work item = (expert, up to 16 of its positions).  Four kinds of kernel per chunk:
+//   fm_pf_sort         workgroup 0 groups the pairs by expert and cuts them into items; the
+//                      others turn X into MFMA operand registers (pf_prepare)
+//   fm_pf_gemm<false>  gate/up + SwiGLU for every item -> act (by sorted position)
+//   fm_pf_prepare_act  act -> operand registers
+//   fm_pf_gemm<true>   down for every item -> expert_out (by pair)
+//   fm_pf_combine      weighted sum in slot order
 #include "fm_mfma.h"
 #include "fm_ring.h"
 
@@ -57,6 +61,8 @@ struct PfArgs {
     float *eo;         // [M*K][hidden], by pair id
     uint4 *xop;        // [M][hidden/64][k step 4][half 2][piece 2]: X as MFMA operand registers
     float2 *xsums;     // [M][hidden/64]: (xsum, xoff) of every group of every position
+    uint4 *aop;        // [M*K][inter/64][4][2][2]: act (by sorted position) in the same form
+    float2 *asums;     // [M*K][inter/64]
 };
 
 // ---- pairing of the 32 codes a lane holds for one group -------------------
@@ -84,17 +90,6 @@ __device__ __forceinline__ void pf_unpack(const uint32_t *d, uint32_t ones, uint
     }
 }
 
-// ---- LDS images -------------------------------------------------------------
-// act  [group][kstep 4][h 2][mrow 32] x 16 bytes : 8 bf16, k slots of that step
-// side [term 2][piece 3][m2 2][h 2][mrow 32] x 16 bytes : xsum / -xoff pieces over groups
-template <int NG>
-struct PfLds {
-    uint4 act[NG * 4 * 2 * 32];
-    uint4 side[2 * 3 * 2 * 2 * 32];
-};
-
-__device__ __forceinline__ uint32_t bf16_trunc(float v) { return __float_as_uint(v) >> 16; }
-
 template <int S, int Q>
 __device__ __forceinline__ void pf_stage_pair(const float *x, uint32_t *hi, uint32_t *lo, float &xs,
                                               float &xo) {
@@ -110,219 +105,6 @@ __device__ __forceinline__ void pf_stage_pair(const float *x, uint32_t *hi, uint
     float tl = __uint_as_float(l0) + __uint_as_float(l1), th = __uint_as_float(h0) + __uint_as_float(h1);
     xo += tl + th;
     xs += tl * (1.0f / cl) + th * (1.0f / ch);
-}
-
-template <int NG, int S>
-__device__ __forceinline__ void pf_stage_steps(PfLds<NG> &L, const float *x, int g, int h, int j,
-                                               float &xs, float &xo) {
-    if constexpr (S < 4) {
-        uint32_t hi[4], lo[4];
-        pf_stage_pair<S, 0>(x, hi, lo, xs, xo);
-        pf_stage_pair<S, 1>(x, hi, lo, xs, xo);
-        pf_stage_pair<S, 2>(x, hi, lo, xs, xo);
-        pf_stage_pair<S, 3>(x, hi, lo, xs, xo);
-        const int base = ((g * 4 + S) * 2 + h) * 32;
-        L.act[base + j] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-        L.act[base + 16 + j] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-        pf_stage_steps<NG, S + 1>(L, x, g, h, j, xs, xo);
-    }
-}
-
-// Build the operand images for `count` positions whose activation rows are
-// xrow(j) (fp32, NG*64 columns).  A task = (position, group, half): 32 activations
-// read with eight 128-bit loads, all k steps of that half built from registers.
-// The caller has a barrier before (previous readers done) and after.
-template <int NG, class RowFn>
-__device__ void pf_stage(PfLds<NG> &L, int count, RowFn xrow) {
-    for (int t = threadIdx.x; t < 2 * 3 * 2 * 2 * 32 * 4; t += blockDim.x)
-        reinterpret_cast<uint32_t *>(L.side)[t] = 0u;
-    __syncthreads();
-    for (int t = threadIdx.x; t < PF_TM * NG * 2; t += blockDim.x) {
-        const int h = t & 1, g = (t >> 1) % NG, j = t / (2 * NG);
-        float x[32];
-        if (j < count) {
-            const float4 *xp = reinterpret_cast<const float4 *>(xrow(j) + 64 * g + 32 * h);
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                float4 v = xp[i];
-                x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 32; i++) x[i] = 0.0f;
-        }
-        float xs = 0.0f, xo = 0.0f;
-        pf_stage_steps<NG, 0>(L, x, g, h, j, xs, xo);
-        // the two halves of a group sit in adjacent lanes
-        xs += fm_dpp<0xB1>(xs);
-        xo += fm_dpp<0xB1>(xo);
-        if (h == 0 && j < count) {
-            // three bf16 pieces of xsum and of -xoff, on the hi row (M row j) of the position
-            float vals[2] = {xs, -xo};
-            const int m2 = g >> 4, hh = (g >> 3) & 1, i = g & 7;
-#pragma unroll
-            for (int term = 0; term < 2; term++) {
-                float r = vals[term];
-#pragma unroll
-                for (int piece = 0; piece < 3; piece++) {
-                    uint32_t b = __float_as_uint(r) & 0xFFFF0000u;
-                    r -= __uint_as_float(b);
-                    uint16_t *e = reinterpret_cast<uint16_t *>(
-                        &L.side[(((term * 3 + piece) * 2 + m2) * 2 + hh) * 32 + j]);
-                    e[i] = (uint16_t)(b >> 16);
-                }
-            }
-        }
-    }
-}
-
-// A wave's share of an item is a sequence of passes; a pass = PF_R tiles of 32
-// weight rows x all groups, in NG/2 iterations of two groups.  The tiles of a
-// pass share every activation operand read from LDS (the gate tile and the up
-// tile of the same rows; two row tiles of down): the LDS pipe, not the matrix
-// core, was the busiest unit with one tile per read, and the independent MFMA
-// chains of the tiles fill each other's latency.  The passes run as ONE
-// software pipeline: the loads of iteration s + DEPTH are issued while
-// iteration s is multiplied, across pass boundaries — with the loads only one
-// iteration ahead every iteration exposed a full memory latency.
-//
-// Results of a pass, per tile: acc register i = M row 8*(i/4) + 4*h + i%4 of the
-// lane's weight row (rows 0..15 the hi pieces of the positions, 16..31 the lo pieces).
-//   ptrs(p, r, wrow, srow, brow): tile r of pass p: the lane's weight row, its scales, biases
-//   done(p, acc[PF_R])          : called after the last iteration of pass p
-#define PF_R 2
-
-typedef uint32_t pf_u3 __attribute__((ext_vector_type(3)));
-
-struct PfLoad {          // one iteration of one tile: the lane's halves of two groups + two scales
-    pf_u3 c0, c1;
-    uint32_t s;
-};
-
-template <int NG>
-struct PfSide {          // scales and biases of the lane's k slots of the group-index products
-    static constexpr int NM2 = (NG + 15) / 16;
-    fm_u4 sv[NM2], bv[NM2];
-};
-
-template <int NG, int PF_DEPTH, class PtrFn, class DoneFn>
-__device__ __forceinline__ void pf_passes(const PfLds<NG> &L, int n_pass, int lane, uint32_t ones,
-                                          PtrFn ptrs, DoneFn done) {
-    constexpr int NI = NG / 2, NM2 = PfSide<NG>::NM2;
-    static_assert(NI >= PF_DEPTH, "one pending side load at most");
-    typedef const __attribute__((address_space(1))) fm_u4 *gq_t;
-    typedef const __attribute__((address_space(1))) pf_u3 *g3_t;
-    typedef const __attribute__((address_space(1))) uint32_t *gd_t;
-    const int h = lane >> 5;
-    const int S = n_pass * NI;
-    auto load = [&](int s, PfLoad *b) {
-        const int p = s / NI, g2 = s - p * NI;
-#pragma unroll
-        for (int r = 0; r < PF_R; r++) {
-            gptr w, sr, br;
-            ptrs(p, r, w, sr, br);
-            b[r].c0 = *(g3_t)(w + 12 * h + 48 * g2);
-            b[r].c1 = *(g3_t)(w + 12 * h + 48 * g2 + 24);
-            b[r].s = *(gd_t)(sr + 4 * g2);
-        }
-    };
-    auto load_side = [&](int p, PfSide<NG> *sd) {
-#pragma unroll
-        for (int r = 0; r < PF_R; r++) {
-            gptr w, sr, br;
-            ptrs(p, r, w, sr, br);
-#pragma unroll
-            for (int m2 = 0; m2 < NM2; m2++) {
-                sd[r].sv[m2] = fm_u4{0, 0, 0, 0};
-                sd[r].bv[m2] = fm_u4{0, 0, 0, 0};
-                if (16 * m2 + 8 * h < NG) {
-                    sd[r].sv[m2] = *(gq_t)(sr + 2 * (16 * m2 + 8 * h));
-                    sd[r].bv[m2] = *(gq_t)(br + 2 * (16 * m2 + 8 * h));
-                }
-            }
-        }
-    };
-    PfLoad buf[PF_DEPTH][PF_R];
-    PfSide<NG> side[PF_R];
-    if (S > 0) load_side(0, side);
-#pragma unroll
-    for (int j = 0; j < PF_DEPTH; j++)
-        if (j < S) load(j, buf[j]);
-    f16v acc[PF_R];
-    for (int s0 = 0; s0 < S; s0 += PF_DEPTH) {
-#pragma unroll
-        for (int j = 0; j < PF_DEPTH; j++) {
-            const int s = s0 + j;
-            if (s < S) {
-                const int p = s / NI, g2 = s - p * NI;
-                if (g2 == 0) {
-                    // bias and offset products over the group index: k slot i of step m2 =
-                    // group 16*m2 + 8*h + i
-#pragma unroll
-                    for (int r = 0; r < PF_R; r++)
-#pragma unroll
-                        for (int i = 0; i < 16; i++) acc[r][i] = 0.0f;
-#pragma unroll
-                    for (int m2 = 0; m2 < NM2; m2++) {
-#pragma unroll
-                        for (int piece = 0; piece < 3; piece++) {
-                            bf8 a0 = __builtin_bit_cast(
-                                bf8, L.side[(((0 * 3 + piece) * 2 + m2) * 2) * 32 + lane]);
-                            bf8 a1 = __builtin_bit_cast(
-                                bf8, L.side[(((1 * 3 + piece) * 2 + m2) * 2) * 32 + lane]);
-#pragma unroll
-                            for (int r = 0; r < PF_R; r++) {
-                                bf8 sb = __builtin_bit_cast(bf8, side[r].sv[m2]);
-                                bf8 bb = __builtin_bit_cast(bf8, side[r].bv[m2]);
-                                acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, bb, acc[r], 0, 0, 0);
-                                acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, sb, acc[r], 0, 0, 0);
-                            }
-                        }
-                    }
-                }
-                PfLoad cur[PF_R];
-#pragma unroll
-                for (int r = 0; r < PF_R; r++) cur[r] = buf[j][r];
-                if (s + PF_DEPTH < S) load(s + PF_DEPTH, buf[j]);
-                // the side operands of the next pass, once its first loads are on their way
-                if (g2 == NI - PF_DEPTH && p + 1 < n_pass) load_side(p + 1, side);
-#pragma unroll
-                for (int gg = 0; gg < 2; gg++) {
-                    const int g = 2 * g2 + gg;
-                    uint32_t v[PF_R][16];
-                    f16v dg[PF_R];
-#pragma unroll
-                    for (int r = 0; r < PF_R; r++) {
-                        uint32_t my[3];
-                        my[0] = gg ? cur[r].c1.x : cur[r].c0.x;
-                        my[1] = gg ? cur[r].c1.y : cur[r].c0.y;
-                        my[2] = gg ? cur[r].c1.z : cur[r].c0.z;
-                        pf_unpack<0>(my, ones, v[r]);
-#pragma unroll
-                        for (int i = 0; i < 16; i++) dg[r][i] = 0.0f;
-                    }
-#pragma unroll
-                    for (int k = 0; k < 4; k++) {
-                        bf8 a = __builtin_bit_cast(bf8, L.act[(g * 4 + k) * 64 + lane]);
-#pragma unroll
-                        for (int r = 0; r < PF_R; r++) {
-                            bf8 b = __builtin_bit_cast(
-                                bf8, make_uint4(v[r][4 * k], v[r][4 * k + 1], v[r][4 * k + 2],
-                                                v[r][4 * k + 3]));
-                            dg[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, dg[r], 0, 0, 0);
-                        }
-                    }
-#pragma unroll
-                    for (int r = 0; r < PF_R; r++) {
-                        const float sc = gg ? fm_bf16_hi(cur[r].s) : fm_bf16_lo(cur[r].s);
-#pragma unroll
-                        for (int i = 0; i < 16; i++) acc[r][i] = fmaf(sc, dg[r][i], acc[r][i]);
-                    }
-                }
-                if (g2 == NI - 1) done(p, acc);
-            }
-        }
-    }
 }
 
 // ---------------------------------------------------------------- kernels
@@ -347,13 +129,14 @@ __device__ __forceinline__ void pf_prepare_steps(const float *x, uint4 *dst, flo
     }
 }
 
-__device__ __forceinline__ void pf_prepare(const PfArgs &a, int task) {
-    const int NG = a.g.hidden / 64;
+__device__ __forceinline__ void pf_prepare(const float *src, int rows, int cols, uint4 *dst_op,
+                                           float2 *dst_sums, int task) {
+    const int NG = cols / 64;
     const int h = task & 1, g = (task >> 1) % NG, m = task / (2 * NG);
-    const bool on = m < a.M;
+    const bool on = m < rows;
     float x[32];
     if (on) {
-        const float4 *xp = reinterpret_cast<const float4 *>(a.X + (size_t)m * a.g.hidden + 64 * g + 32 * h);
+        const float4 *xp = reinterpret_cast<const float4 *>(src + (size_t)m * cols + 64 * g + 32 * h);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             float4 v = xp[i];
@@ -371,14 +154,19 @@ __device__ __forceinline__ void pf_prepare(const PfArgs &a, int task) {
     xs += fm_dpp<0xB1>(xs);
     xo += fm_dpp<0xB1>(xo);
     if (on) {
-        uint4 *dst = a.xop + ((size_t)m * NG + g) * 16;
+        uint4 *dst = dst_op + ((size_t)m * NG + g) * 16;
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             dst[4 * k + 2 * h] = regs[4 * k];
             dst[4 * k + 2 * h + 1] = regs[4 * k + 1];
         }
-        if (h == 0) a.xsums[(size_t)m * NG + g] = make_float2(xs, xo);
+        if (h == 0) dst_sums[(size_t)m * NG + g] = make_float2(xs, xo);
     }
+}
+
+// the SwiGLU outputs (by sorted position) as operand registers for the down product
+__global__ __launch_bounds__(256) void fm_pf_prepare_act(PfArgs a) {
+    pf_prepare(a.act, a.M * a.K, a.g.inter, a.aop, a.asums, (int)(blockIdx.x * blockDim.x + threadIdx.x));
 }
 
 // workgroup 0 sorts, the others prepare X
@@ -386,7 +174,7 @@ __global__ __launch_bounds__(1024) void fm_pf_sort(PfArgs a) {
     __shared__ int hist[PF_MAX_EXPERTS], cursor[PF_MAX_EXPERTS], scan_a[PF_MAX_EXPERTS],
         scan_b[PF_MAX_EXPERTS];
     if (blockIdx.x > 0) {
-        pf_prepare(a, (int)((blockIdx.x - 1) * blockDim.x + threadIdx.x));
+        pf_prepare(a.X, a.M, a.g.hidden, a.xop, a.xsums, (int)((blockIdx.x - 1) * blockDim.x + threadIdx.x));
         return;
     }
     const int E = a.g.n_experts, n = a.M * a.K, e = threadIdx.x;
@@ -438,78 +226,26 @@ __global__ __launch_bounds__(1024) void fm_pf_sort(PfArgs a) {
     }
 }
 
-// down for every item -> eo[pair][hidden]
-template <int NG>
-__global__ __launch_bounds__(512) void fm_pf_down(PfArgs a) {
-    extern __shared__ uint4 pf_smem[];
-    PfLds<NG> &L = *reinterpret_cast<PfLds<NG> *>(pf_smem);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n_items = *a.n_items;
-    const int row_bytes = a.g.inter * 3 / 8, sb_bytes = (a.g.inter / 64) * 2;
-    const uint32_t ones = fm_opaque(0x3F803F80u);
-    // The launch is the sequence (item, pass) — a pass = two row tiles per wave, 64 * NW
-    // rows of the item — and this workgroup takes passes [t0, t1) of it: every workgroup
-    // the same number (within one) whatever the number of items.
-    const int NW = blockDim.x / 64;
-    const int NP = a.g.hidden / (64 * NW);            // hidden is a multiple of 64 * NW
-    const long T = (long)n_items * NP;
-    const int t0 = (int)(T * blockIdx.x / gridDim.x), t1 = (int)(T * (blockIdx.x + 1) / gridDim.x);
-    for (int t = t0; t < t1;) {
-        const int it = t / NP, pb = t - it * NP;
-        const int pe = t1 - t < NP - pb ? pb + (t1 - t) : NP;
-        t += pe - pb;
-        const PfItem item = a.items[it];
-        __syncthreads();
-        pf_stage<NG>(L, item.count, [&](int j) { return a.act + (size_t)(item.start + j) * a.g.inter; });
-        __syncthreads();
-        const uint8_t *blob = a.layer + (size_t)item.expert * a.g.expert_size;
-        const int n = lane & 31, h = lane >> 5;
-        // pass p of the item: row tiles wave + NW*(2p) and wave + NW*(2p+1)
-        pf_passes<NG, 4>(
-            L, pe - pb, lane, ones,
-            [&](int p, int r, gptr &w, gptr &sr, gptr &br) {
-                const int row = (wave + NW * (2 * (pb + p) + r)) * 32 + n;
-                w = (gptr)(uintptr_t)(blob + a.g.down_w + (size_t)row * row_bytes);
-                sr = (gptr)(uintptr_t)(blob + a.g.down_s + (size_t)row * sb_bytes);
-                br = (gptr)(uintptr_t)(blob + a.g.down_b + (size_t)row * sb_bytes);
-            },
-            [&](int p, const f16v *acc) {
-#pragma unroll
-                for (int r = 0; r < PF_R; r++) {
-                    const int row = (wave + NW * (2 * (pb + p) + r)) * 32 + n;
-#pragma unroll
-                    for (int i = 0; i < 8; i++) {
-                        const int tok = 8 * (i / 4) + 4 * h + (i % 4);
-                        if (tok < item.count) {
-                            const int pair = a.sorted[item.start + tok];
-                            a.eo[(size_t)pair * a.g.hidden + row] = acc[r][i] + acc[r][i + 8];
-                        }
-                    }
-                }
-            });
-    }
-}
-
 // ======================================================================
-// K-slab kernel (gate/up).
+// The GEMM kernel (fm_pf_gemm): 512 threads, one workgroup per CU.
 //
-// The kernels above keep the whole activation operand of an item in LDS
-// (128 KB) and let every wave sweep row tiles over the full K; their weight
-// loads are per-lane 12-byte pieces of 32 different rows, and the address
-// unit, not the matrix core, is the busiest part of the CU.  Here the K
-// dimension is split over the eight waves of the workgroup instead: wave w
-// owns groups [4w, 4w+4) of every row.
-//   * Its share of the activation operand is 16 registers per group, loaded
-//     ready-made (pf_prepare) once per item; LDS holds no activations.
-//   * Every wave visits every row tile.  A tile-matrix (32 rows of one matrix)
-//     x slab is 32 runs of 96 bytes: the wave copies them, with the rows'
-//     scales and biases, into a ring slot with LDS-direct loads (whole runs,
-//     several slots in flight), and every lane reads its 12-byte pieces back.
+// The K dimension is cut into slabs of four groups (256 columns) and a wave
+// owns one slab of every row it visits: gate/up has eight slabs, one per wave;
+// down has two, and the eight waves form four teams on different rows.
+//   * A wave's share of the activation operand is 16 registers per group,
+//     loaded ready-made (pf_prepare) once per item; LDS holds no activations.
+//     (An earlier form kept the whole operand of an item in LDS and let every
+//     wave sweep row tiles over the full K with per-lane 12-byte weight loads:
+//     the address unit, not the matrix core, was its busiest part.)
+//   * A tile-matrix (32 rows of one matrix) x slab is 32 runs of 96 bytes: the
+//     wave copies them, with the rows' scales and biases, into a ring slot with
+//     LDS-direct loads (whole runs, several slots in flight), and every lane
+//     reads its 12-byte pieces back.
 //   * Bias and offset terms ride in two extra MFMAs per tile-matrix whose K
 //     slots are (piece, group) of the wave's own groups.
-//   * The eight partial tiles are summed through LDS in wave order (wave r sums
-//     result register r of every lane), SwiGLU / store happen there.  One
-//     barrier per step (two tile-matrices), two partial buffers.
+//   * The partial tiles of a row tile's slabs are summed through LDS in slab
+//     order; SwiGLU / store happen there.  One barrier per step (two
+//     tile-matrices per wave), two partial buffers.
 // ======================================================================
 struct PfSlab {
     static constexpr int GPW = 4;                       // groups per wave
@@ -540,7 +276,15 @@ __device__ __forceinline__ void pf_pieces(float v, uint32_t *pc) {
     pc[2] = __float_as_uint(v) >> 16;
 }
 
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fm_pf_gate_up(PfArgs a) {
+// DOWN = false: gate/up.  K = hidden is eight slabs, wave w owns slab w, all waves work on the
+//   same 32 rows; a step = the gate tile and the up tile of those rows; sum over eight waves,
+//   SwiGLU, act.
+// DOWN = true: K = inter is two slabs: the workgroup is four teams of two waves (slab = wave & 1),
+//   every team on its own 64 rows of a step's 256; a step = two row tiles per team; sum over
+//   the team's two waves, expert_out.  The activation operand comes from aop / asums
+//   (fm_pf_prepare_act), indexed by sorted position.
+template <bool DOWN>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fm_pf_gemm(PfArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // (the host pass cannot allocate the registers of the asm blocks)
     using P = PfSlab;
     constexpr int GPW = P::GPW;
@@ -553,14 +297,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint32_t ring0 = lds0 + (uint32_t)wave * (RING * P::SLOT);
     const uint32_t red0 = lds0 + 8 * RING * P::SLOT;
     const int n_items = *a.n_items;
-    const int in_dim = a.g.hidden;
+    const int in_dim = DOWN ? a.g.inter : a.g.hidden;
     const int row_bytes = in_dim * 3 / 8, sb_bytes = (in_dim / 64) * 2;
-    const int n_steps = a.g.inter / 32;          // a step = the gate and the up tile of 32 rows
+    const int slab = DOWN ? (wave & 1) : wave, team = DOWN ? (wave >> 1) : 0;
+    const int n_steps = DOWN ? a.g.hidden / 256 : a.g.inter / 32;
     const uint32_t ones = fm_opaque(0x3F803F80u);
-    // region offsets of the two tile-matrices of a step and their row distance
-    const uint32_t w_off0 = a.g.gate_w, s_off0 = a.g.gate_s, b_off0 = a.g.gate_b;
-    const uint32_t w_d = a.g.up_w - a.g.gate_w, s_d = a.g.up_s - a.g.gate_s, b_d = a.g.up_b - a.g.gate_b;
-    const uint32_t step_rows = 32u;
+    // region offsets of the first tile-matrix of a step (this team's), the distance to the
+    // second one, rows per step
+    const uint32_t w_off0 = DOWN ? a.g.down_w + 64u * team * row_bytes : a.g.gate_w;
+    const uint32_t s_off0 = DOWN ? a.g.down_s + 64u * team * sb_bytes : a.g.gate_s;
+    const uint32_t b_off0 = DOWN ? a.g.down_b + 64u * team * sb_bytes : a.g.gate_b;
+    const uint32_t w_d = DOWN ? 32u * row_bytes : a.g.up_w - a.g.gate_w;
+    const uint32_t s_d = DOWN ? 32u * sb_bytes : a.g.up_s - a.g.gate_s;
+    const uint32_t b_d = DOWN ? 32u * sb_bytes : a.g.up_b - a.g.gate_b;
+    const uint32_t step_rows = DOWN ? 256u : 32u;
     // this lane's pieces of a slot copy
     uint32_t coff[P::NQ];
     bool cvalid[P::NQ];
@@ -569,10 +319,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int q = 64 * j + lane;
         const int row = q / P::RS, piece = q - row * P::RS;
         cvalid[j] = q < P::PIECES && piece < P::RP;
-        coff[j] = (uint32_t)(row * row_bytes + P::CB * wave + P::PS * piece);
+        coff[j] = (uint32_t)(row * row_bytes + P::CB * slab + P::PS * piece);
     }
     // scales / biases of the slab: 2*GPW bytes per row, fetched as whole dwords
-    const int sb_slab = (2 * GPW * wave) & ~3;
+    const int sb_slab = (2 * GPW * slab) & ~3;
     const uint32_t soff = (uint32_t)((lane >> 1) * sb_bytes + sb_slab + 4 * (lane & 1));
 
     // ---- this workgroup's share of the launch: steps [t0, t1) of the sequence
@@ -635,16 +385,29 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // of which would also drain the ring.
     PfItem item_next = PfItem{0, 0, 0, 0};
     int pair_next = 0;              // pair id of this lane's position (divided by K when used)
+    int out_pairs_next[8];          // DOWN: pair ids of the eight positions this lane stores
+#pragma unroll
+    for (int i = 0; i < 8; i++) out_pairs_next[i] = 0;
     if (t0 < t1) {
         item_next = a.items[t0 / n_steps];
-        if ((n & 15) < item_next.count) pair_next = a.sorted[item_next.start + (n & 15)];
+        if constexpr (DOWN) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int tok = 8 * (i / 4) + 4 * hh + (i % 4);
+                if (tok < item_next.count) out_pairs_next[i] = a.sorted[item_next.start + tok];
+            }
+        } else {
+            if ((n & 15) < item_next.count) pair_next = a.sorted[item_next.start + (n & 15)];
+        }
     }
     for (int t = t0; t < t1;) {
         const int it = t / n_steps, s_begin = t - it * n_steps;
         const int s_end = t1 - t < n_steps - s_begin ? s_begin + (t1 - t) : n_steps;
         t += s_end - s_begin;
         const PfItem item = item_next;
-        const int m_cur = pair_next / a.K;
+        int out_pairs[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) out_pairs[i] = out_pairs_next[i];
         const bool more = t < t1;                  // this workgroup goes on to item it + 1
         if (more) item_next = a.items[it + 1];
         // ---- this wave's share of the activation operand, straight into registers:
@@ -660,9 +423,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 // X was turned into operand registers once per chunk (pf_prepare): lane (m, hh)
                 // takes the hi (m < 16) or lo registers of its position, its groups, its half
                 const int piece = n < 16 ? 0 : 1;
-                const size_t m = on ? (size_t)m_cur : 0;
-                const uint4 *src = a.xop + (m * (a.g.hidden / 64) + GPW * wave) * 16 + 2 * hh + piece;
-                const float2 *sm = a.xsums + m * (a.g.hidden / 64) + GPW * wave;
+                const size_t m = !on ? 0 : DOWN ? (size_t)(item.start + pos) : (size_t)(pair_next / a.K);
+                const int ng = in_dim / 64;
+                const uint4 *src = (DOWN ? a.aop : a.xop) + (m * ng + GPW * slab) * 16 + 2 * hh + piece;
+                const float2 *sm = (DOWN ? a.asums : a.xsums) + m * ng + GPW * slab;
 #pragma unroll
                 for (int gi = 0; gi < GPW; gi++) {
 #pragma unroll
@@ -685,8 +449,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     }
                 // the next item has arrived with them: its position row, used at its start
                 // (no arithmetic on it here: that would wait for the load now)
-                pair_next = 0;
-                if (more && pos < item_next.count) pair_next = a.sorted[item_next.start + pos];
+                if constexpr (DOWN) {
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const int tok = 8 * (i / 4) + 4 * hh + (i % 4);
+                        out_pairs_next[i] = 0;
+                        if (more && tok < item_next.count) out_pairs_next[i] = a.sorted[item_next.start + tok];
+                    }
+                } else {
+                    pair_next = 0;
+                    if (more && pos < item_next.count) pair_next = a.sorted[item_next.start + pos];
+                }
                 if (more) e_ahead = item_next.expert;     // the loader enters it during this item
             }
             // K slots of the bias/offset MFMAs: slot = 4*piece + group, one MFMA per term (xsum
@@ -812,7 +585,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
             // ---- every wave has written both partial tiles of this step
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            {
+            if constexpr (!DOWN) {
                 // wave r sums result register r (position my_pos) over the waves, in wave order
                 const uint32_t ar = red0 + (uint32_t)((buf * 2 * 8) * 2048 + wave * 256 + 4 * lane);
                 float p[16];
@@ -837,6 +610,32 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 }
                 if (my_on) {
                     a.act[(size_t)(item.start + my_pos) * a.g.inter + 32 * s + n] = fm_silu_mul(t0, t1);
+                }
+            } else {
+                // wave (team, j) sums tile j of its team over the team's two waves (slab 0, then
+                // slab 1): all eight registers = the eight positions this lane stores
+                const int j = wave & 1;
+                const uint32_t ar = red0 + (uint32_t)(((buf * 2 + j) * 8 + 2 * team) * 2048 + 4 * lane);
+                float p[16];
+                asm volatile(
+                    "ds_read_b32 %0, %16\n\tds_read_b32 %1, %16 offset:256\n\tds_read_b32 %2, %16 offset:512\n\t"
+                    "ds_read_b32 %3, %16 offset:768\n\tds_read_b32 %4, %16 offset:1024\n\tds_read_b32 %5, %16 offset:1280\n\t"
+                    "ds_read_b32 %6, %16 offset:1536\n\tds_read_b32 %7, %16 offset:1792\n\t"
+                    "ds_read_b32 %8, %16 offset:2048\n\tds_read_b32 %9, %16 offset:2304\n\tds_read_b32 %10, %16 offset:2560\n\t"
+                    "ds_read_b32 %11, %16 offset:2816\n\tds_read_b32 %12, %16 offset:3072\n\tds_read_b32 %13, %16 offset:3328\n\t"
+                    "ds_read_b32 %14, %16 offset:3584\n\tds_read_b32 %15, %16 offset:3840\n\t"
+                    "s_waitcnt lgkmcnt(0)"
+                    : "=&v"(p[0]), "=&v"(p[1]), "=&v"(p[2]), "=&v"(p[3]), "=&v"(p[4]), "=&v"(p[5]),
+                      "=&v"(p[6]), "=&v"(p[7]), "=&v"(p[8]), "=&v"(p[9]), "=&v"(p[10]), "=&v"(p[11]),
+                      "=&v"(p[12]), "=&v"(p[13]), "=&v"(p[14]), "=&v"(p[15])
+                    : "v"(ar)
+                    : "memory");
+                const int row = 256 * s + 64 * team + 32 * j + n;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const int tok = 8 * (i / 4) + 4 * hh + (i % 4);
+                    if (tok < item.count)
+                        a.eo[(size_t)out_pairs[i] * a.g.hidden + row] = p[i] + p[8 + i];
                 }
             }
             buf ^= 1;
@@ -903,7 +702,9 @@ extern "C" size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K
     return align256(n * 4) + align256((g->n_experts + n / PF_TM + 1) * sizeof(PfItem)) + 256 +
            align256(n * g->inter * 4) + align256(n * g->hidden * 4) +
            align256((size_t)M * (g->hidden / 64) * 16 * sizeof(uint4)) +
-           align256((size_t)M * (g->hidden / 64) * sizeof(float2));
+           align256((size_t)M * (g->hidden / 64) * sizeof(float2)) +
+           align256(n * (g->inter / 64) * 16 * sizeof(uint4)) +
+           align256(n * (g->inter / 64) * sizeof(float2));
 }
 
 extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGeom *g,
@@ -928,32 +729,24 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
     a.act = (float *)ws;                  ws += align256(n * g->inter * 4);
     a.eo = (float *)ws;                   ws += align256(n * g->hidden * 4);
     a.xop = (uint4 *)ws;                  ws += align256((size_t)M * (g->hidden / 64) * 16 * sizeof(uint4));
-    a.xsums = (float2 *)ws;
+    a.xsums = (float2 *)ws;               ws += align256((size_t)M * (g->hidden / 64) * sizeof(float2));
+    a.aop = (uint4 *)ws;                  ws += align256(n * (g->inter / 64) * 16 * sizeof(uint4));
+    a.asums = (float2 *)ws;
     // workgroup 0 sorts, the rest turn X into operand registers (one thread per position,
     // group and half)
     const int prep_tasks = M * (g->hidden / 64) * 2;
     hipLaunchKernelGGL(fm_pf_sort, dim3(1 + (prep_tasks + 1023) / 1024), dim3(1024), 0, st, a);
     const int max_items = g->n_experts + (int)(n / PF_TM);
-#define PF_LAUNCH(KERN, NG, GRID, NT)                                                              \
-    do {                                                                                           \
-        static FmLdsAttr attr;                                                                     \
-        if (!fm_dyn_lds_ready(attr, (const void *)KERN<NG>, sizeof(PfLds<NG>))) return FM_ERR_HIP; \
-        hipLaunchKernelGGL(KERN<NG>, dim3(GRID), dim3(NT), sizeof(PfLds<NG>), st, a);              \
-    } while (0)
-    // one 8-wave workgroup per CU: the kernels need ~200 registers per lane (two accumulator
-    // tiles, a group tile, 16 operand registers, loads in flight), which caps a SIMD at two
-    // waves; capping the registers instead made them spill and run 2-5x slower
+    // one 8-wave workgroup per CU (LDS: the ring and the partial tiles take all 160 KB; ~220-245
+    // registers per lane cap a SIMD at two waves)
     const int grid = max_items < n_cu ? max_items : n_cu;
-    // gate/up: K split over the waves (fm_pf_gate_up).  down: whole K per wave (fm_pf_down) —
-    // with one group (four MFMAs) per wave and tile the split's per-tile overhead outweighs
-    // what it saves.
-    {
-        static FmLdsAttr attr;
-        if (!fm_dyn_lds_ready(attr, (const void *)fm_pf_gate_up, PfSlab::LDS_BYTES)) return FM_ERR_HIP;
-        hipLaunchKernelGGL(fm_pf_gate_up, dim3(grid), dim3(512), PfSlab::LDS_BYTES, st, a);
-    }
-    PF_LAUNCH(fm_pf_down, 8, grid, 512);
-#undef PF_LAUNCH
+    static FmLdsAttr attr_up, attr_down;
+    if (!fm_dyn_lds_ready(attr_up, (const void *)fm_pf_gemm<false>, PfSlab::LDS_BYTES)) return FM_ERR_HIP;
+    if (!fm_dyn_lds_ready(attr_down, (const void *)fm_pf_gemm<true>, PfSlab::LDS_BYTES)) return FM_ERR_HIP;
+    hipLaunchKernelGGL(fm_pf_gemm<false>, dim3(grid), dim3(512), PfSlab::LDS_BYTES, st, a);
+    const int act_tasks = (int)n * (g->inter / 64) * 2;
+    hipLaunchKernelGGL(fm_pf_prepare_act, dim3((act_tasks + 255) / 256), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(fm_pf_gemm<true>, dim3(grid), dim3(512), PfSlab::LDS_BYTES, st, a);
     hipLaunchKernelGGL(fm_pf_combine, dim3(M, (g->hidden + 1023) / 1024), dim3(256), 0, st, a, d_out, flags);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
