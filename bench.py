@@ -7,7 +7,7 @@ HBM, per-layer top-8 indices from a Zipf(1.1) distribution with a per-layer rank
 router weights = renormalised softmax of N(0,1) logits at those indices.  A "step" is one
 token: one pass of the hot path over all 40 layers.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_layer|gdn|gguf|prefill|lm_head|layer_tail]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_layer|gdn|gguf|gguf_chunk|prefill|lm_head|layer_tail]
 
 Prints ONE JSON line.  `value` is algorithmic weight bytes per step / wall time per step with
 all inputs resident in HBM.  `roofline` prices the dominant kernel against the 8 TB/s HBM
@@ -456,6 +456,30 @@ def run_gguf(args):
     rng = np.random.default_rng(7)
     tokens = 64
     idx, w = zipf_routing(rng, tokens, n_layers, E, K)
+    if args.workload == "gguf_chunk":
+        # the chunked-prefill variant of config 4: M positions of one layer per call (per-position
+        # products, as the reference runs them), the layer changes from call to call
+        M = args.chunk if args.chunk <= tokens else 8
+        c_idx = torch.from_numpy(np.ascontiguousarray(idx.transpose(1, 0, 2))).to(dev)   # [layer][token][k]
+        c_w = torch.from_numpy(np.ascontiguousarray(w.transpose(1, 0, 2))).to(dev)
+        c_x = torch.randn(M, H, device=dev)
+        c_out = torch.empty(M, H, device=dev)
+        torch.cuda.synchronize()
+        lsz = tokens * K * 4
+
+        def cstep(t):
+            l = t % n_layers
+            ctx.gguf_moe_prefill_dev(l, c_x.data_ptr(), c_idx.data_ptr() + l * lsz, c_w.data_ptr() + l * lsz,
+                                     M, K, c_out.data_ptr())
+
+        ms, ev = _timed(ctx, cstep, args)
+        assert torch.isfinite(c_out).all()
+        ctx.close()
+        return _finish({"event_ms_per_step": round(ev, 5)},
+                       "GGUF Q4_K/Q6_K expert GEMV HBM GB/s, %d-position chunk of one layer" % M,
+                       "config 4, chunk variant: %d positions x top-8 Zipf(1.1) on one of %d GGUF layers "
+                       "(Q4_K gate/up, Q6_K down), per-position products" % (M, n_layers),
+                       M * K * (2 * gsl + dsl), ms, args)
     d_idx, d_w = torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)
     d_x = torch.randn(n_layers, H, device=dev)
     d_out = torch.empty(n_layers, H, device=dev)
@@ -573,7 +597,7 @@ def main():
         print("bench.py: no GPU visible; there is no CPU fallback", file=sys.stderr)
         sys.exit(3)
     runners = {"decode_step": run_decode_step, "decode_layer": run_decode_layer, "gdn": run_gdn,
-               "gguf": run_gguf, "prefill": run_prefill, "lm_head": run_lm_head, "layer_tail": run_layer_tail,
+               "gguf": run_gguf, "gguf_chunk": run_gguf, "prefill": run_prefill, "lm_head": run_lm_head, "layer_tail": run_layer_tail,
                "copy_probe": run_copy_probe}
     if args.workload not in runners:
         print("bench.py: unknown workload %r (have: %s)" % (args.workload, ", ".join(runners)),
