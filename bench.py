@@ -513,16 +513,17 @@ def run_prefill(args):
     from finchmoe_amd import FinchHip, formats
     dev = torch.device("cuda:0")
     M = args.chunk
-    lo = formats.expert_layout(H, I, 3)
+    bits = args.bits
+    lo = formats.expert_layout(H, I, bits)
     es = lo["expert_size"]
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
     nl = 8
     blob = torch.empty(nl, E, es, dtype=torch.uint8, device=dev)
     for l in range(nl):
-        fill_affine_layer(blob[l], lo, 3, gen)
+        fill_affine_layer(blob[l], lo, bits, gen)
     ctx = FinchHip(0)
-    ctx.experts_config(nl, E, H, I, 64, 3, 0)
+    ctx.experts_config(nl, E, H, I, 64, bits, 0)
     for l in range(nl):
         ctx.experts_adopt_layer(l, blob[l].data_ptr(), E * es)
     rng = np.random.default_rng(7)
@@ -547,8 +548,8 @@ def run_prefill(args):
            "unique_experts_per_chunk": uniq, "event_ms_per_step": round(ev, 5)}
     ctx.close()
     out = _finish(res, "chunked-prefill expert product, %d-position chunk" % M,
-                  "config 3: %d-token chunk, top-8 Zipf(1.1), 3-bit g64 experts, x~N(0,1) bf16 values in fp32"
-                  % M, int(uniq * es), ms, args, {"flops_per_step": flops})
+                  "config 3: %d-token chunk, top-8 Zipf(1.1), %d-bit g64 experts, x~N(0,1) bf16 values in fp32"
+                  % (M, bits), int(uniq * es), ms, args, {"flops_per_step": flops})
     return out
 
 
@@ -581,7 +582,7 @@ def main():
     ap.add_argument("--workload", default="decode_step")
     ap.add_argument("--layers", type=int, default=L)
     ap.add_argument("--bits", type=int, default=3, choices=(3, 4),
-                    help="affine code width of the decode_step workload")
+                    help="affine code width of the decode_step and prefill workloads")
     ap.add_argument("--chunk", type=int, default=512, help="positions per chunk (prefill workload)")
     ap.add_argument("--ramp-seconds", type=float, default=0.5,
                     help="untimed busy period before the warmup steps (clock ramp)")

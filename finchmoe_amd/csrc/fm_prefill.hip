@@ -11,7 +11,7 @@
 // the bar (max relative error 1.8e-3 on the benchmark's weight distribution).
 // Instead
 //   * the CODES are the MFMA operand, as exact bf16 numbers 1 + q*2^t/128 (the
-//     mantissa trick of fm_mfma.h: one V_AND_OR_B32 per two codes);
+//     mantissa trick of fm_mfma.h: one V_AND_OR_B32 per two codes; 4-bit codes: t = 0);
 //   * each quantization group (64 columns) is accumulated by its own MFMA chain
 //     and its scale is applied to the result in fp32: acc += s[row][g] * D_g;
 //   * activations are split hi + lo (two bf16 pieces, 16 significant bits); the
@@ -24,7 +24,8 @@
 // V_MFMA_F32_32X32X16_BF16 with positions on M and weight rows on N: lane
 // (n = lane%32, h = lane/32) supplies 8 consecutive k of weight row n and holds
 // 16 results, all of weight row n — so a lane needs ONE scale per group.
-// A lane's codes for one group are half a group: 32 codes = 12 bytes.
+// A lane's codes for one group are half a group: 32 codes = 12 bytes (3-bit) or 16 bytes
+// (4-bit).  The kernels are instantiated for both widths.
 //
 // Work item = (expert, up to 16 of its positions).  Four kinds of kernel per chunk:
 //   fm_pf_sort         workgroup 0 groups the pairs by expert and cuts them into items; the
@@ -66,36 +67,57 @@ struct PfArgs {
 };
 
 // ---- pairing of the 32 codes a lane holds for one group -------------------
-// 16 pairs: two blocks of 10 codes 5 apart (tl=4, th=3), one block of 12 codes 6
-// apart (tl=2, th=4).  Pair p fills k slots 2p (low half) and 2p+1 (high half).
-__host__ __device__ constexpr int pf_lo(int p) { return p < 10 ? 10 * (p / 5) + p % 5 : 20 + (p - 10); }
-__host__ __device__ constexpr int pf_hi(int p) { return pf_lo(p) + (p < 10 ? 5 : 6); }
-__host__ __device__ constexpr int pf_tl(int p) { return p < 10 ? 4 : 2; }
-__host__ __device__ constexpr int pf_th(int p) { return p < 10 ? 3 : 4; }
-__host__ __device__ constexpr int pf_start(int p) { return 3 * pf_lo(p) - pf_tl(p); }
-__host__ __device__ constexpr uint32_t pf_mask(int p) { return (7u << pf_tl(p)) | (7u << (16 + pf_th(p))); }
+// Pair p fills k slots 2p (low half of the register, code lo(p) at mantissa bit tl(p)) and
+// 2p+1 (high half, code hi(p) at bit th(p)); the pair is cut out of the lane's DW dwords at
+// stream bit start(p) with one mask.
+template <int BITS>
+struct PfCode;
+// 3 bits: two blocks of 10 codes 5 apart (tl=4, th=3), one block of 12 codes 6 apart (tl=2, th=4)
+template <>
+struct PfCode<3> {
+    static constexpr int DW = 3;
+    static constexpr int lo(int p) { return p < 10 ? 10 * (p / 5) + p % 5 : 20 + (p - 10); }
+    static constexpr int hi(int p) { return lo(p) + (p < 10 ? 5 : 6); }
+    static constexpr int tl(int p) { return p < 10 ? 4 : 2; }
+    static constexpr int th(int p) { return p < 10 ? 3 : 4; }
+    static constexpr int start(int p) { return 3 * lo(p) - tl(p); }
+    static constexpr uint32_t mask(int p) { return (7u << tl(p)) | (7u << (16 + th(p))); }
+};
+// 4 bits: nibbles a and a + 4 of a dword are 16 bits apart already
+template <>
+struct PfCode<4> {
+    static constexpr int DW = 4;
+    static constexpr int lo(int p) { return 8 * (p / 4) + p % 4; }
+    static constexpr int hi(int p) { return lo(p) + 4; }
+    static constexpr int tl(int) { return 0; }
+    static constexpr int th(int) { return 0; }
+    static constexpr int start(int p) { return 4 * lo(p); }
+    static constexpr uint32_t mask(int) { return 0x000F000Fu; }
+};
 
-template <int P>
+template <int BITS, int P>
 __device__ __forceinline__ uint32_t pf_pair(const uint32_t *d, uint32_t ones) {
-    uint32_t w = fm_window<pf_start(P), 3>(d);
-    return (w & pf_mask(P)) | ones;
+    using C = PfCode<BITS>;
+    uint32_t w = fm_window<C::start(P), C::DW>(d);
+    return (w & C::mask(P)) | ones;
 }
 
 // the 16 operand registers of a lane's 32 codes
-template <int P>
+template <int BITS, int P>
 __device__ __forceinline__ void pf_unpack(const uint32_t *d, uint32_t ones, uint32_t *v) {
     if constexpr (P < 16) {
-        v[P] = pf_pair<P>(d, ones);
-        pf_unpack<P + 1>(d, ones, v);
+        v[P] = pf_pair<BITS, P>(d, ones);
+        pf_unpack<BITS, P + 1>(d, ones, v);
     }
 }
 
-template <int S, int Q>
+template <int BITS, int S, int Q>
 __device__ __forceinline__ void pf_stage_pair(const float *x, uint32_t *hi, uint32_t *lo, float &xs,
                                               float &xo) {
+    using C = PfCode<BITS>;
     constexpr int p = 4 * S + Q;
-    constexpr float cl = (float)(128 >> pf_tl(p)), ch = (float)(128 >> pf_th(p));
-    float vl = x[pf_lo(p)] * cl, vh = x[pf_hi(p)] * ch;
+    constexpr float cl = (float)(128 >> C::tl(p)), ch = (float)(128 >> C::th(p));
+    float vl = x[C::lo(p)] * cl, vh = x[C::hi(p)] * ch;
     // exact split into bf16 pieces; hi + lo = the value truncated to 16 significant bits
     uint32_t l0 = __float_as_uint(vl) & 0xFFFF0000u, h0 = __float_as_uint(vh) & 0xFFFF0000u;
     float rl = vl - __uint_as_float(l0), rh = vh - __uint_as_float(h0);
@@ -115,20 +137,21 @@ __device__ __forceinline__ void pf_stage_pair(const float *x, uint32_t *hi, uint
 // per position and group the two sums the bias and offset terms need.  Done once per chunk:
 // a position is multiplied by K experts, and splitting it inside the multiply kernel cost a
 // fifth of that kernel's time.  Task = (position, group, half).
-template <int S>
+template <int BITS, int S>
 __device__ __forceinline__ void pf_prepare_steps(const float *x, uint4 *dst, float &xs, float &xo) {
     if constexpr (S < 4) {
         uint32_t hi[4], lo[4];
-        pf_stage_pair<S, 0>(x, hi, lo, xs, xo);
-        pf_stage_pair<S, 1>(x, hi, lo, xs, xo);
-        pf_stage_pair<S, 2>(x, hi, lo, xs, xo);
-        pf_stage_pair<S, 3>(x, hi, lo, xs, xo);
+        pf_stage_pair<BITS, S, 0>(x, hi, lo, xs, xo);
+        pf_stage_pair<BITS, S, 1>(x, hi, lo, xs, xo);
+        pf_stage_pair<BITS, S, 2>(x, hi, lo, xs, xo);
+        pf_stage_pair<BITS, S, 3>(x, hi, lo, xs, xo);
         dst[4 * S] = make_uint4(hi[0], hi[1], hi[2], hi[3]);          // [k step][half][piece]
         dst[4 * S + 1] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-        pf_prepare_steps<S + 1>(x, dst, xs, xo);
+        pf_prepare_steps<BITS, S + 1>(x, dst, xs, xo);
     }
 }
 
+template <int BITS>
 __device__ __forceinline__ void pf_prepare(const float *src, int rows, int cols, uint4 *dst_op,
                                            float2 *dst_sums, int task) {
     const int NG = cols / 64;
@@ -149,7 +172,7 @@ __device__ __forceinline__ void pf_prepare(const float *src, int rows, int cols,
     float xs = 0.0f, xo = 0.0f;
     // this half's registers: index ((m*NG + g)*4 + k)*4 + 2*half + piece
     uint4 regs[16];
-    pf_prepare_steps<0>(x, regs, xs, xo);
+    pf_prepare_steps<BITS, 0>(x, regs, xs, xo);
     // the two halves of a group sit in adjacent lanes
     xs += fm_dpp<0xB1>(xs);
     xo += fm_dpp<0xB1>(xo);
@@ -165,16 +188,18 @@ __device__ __forceinline__ void pf_prepare(const float *src, int rows, int cols,
 }
 
 // the SwiGLU outputs (by sorted position) as operand registers for the down product
+template <int BITS>
 __global__ __launch_bounds__(256) void fm_pf_prepare_act(PfArgs a) {
-    pf_prepare(a.act, a.M * a.K, a.g.inter, a.aop, a.asums, (int)(blockIdx.x * blockDim.x + threadIdx.x));
+    pf_prepare<BITS>(a.act, a.M * a.K, a.g.inter, a.aop, a.asums, (int)(blockIdx.x * blockDim.x + threadIdx.x));
 }
 
 // workgroup 0 sorts, the others prepare X
+template <int BITS>
 __global__ __launch_bounds__(1024) void fm_pf_sort(PfArgs a) {
     __shared__ int hist[PF_MAX_EXPERTS], cursor[PF_MAX_EXPERTS], scan_a[PF_MAX_EXPERTS],
         scan_b[PF_MAX_EXPERTS];
     if (blockIdx.x > 0) {
-        pf_prepare(a.X, a.M, a.g.hidden, a.xop, a.xsums, (int)((blockIdx.x - 1) * blockDim.x + threadIdx.x));
+        pf_prepare<BITS>(a.X, a.M, a.g.hidden, a.xop, a.xsums, (int)((blockIdx.x - 1) * blockDim.x + threadIdx.x));
         return;
     }
     const int E = a.g.n_experts, n = a.M * a.K, e = threadIdx.x;
@@ -247,22 +272,25 @@ __global__ __launch_bounds__(1024) void fm_pf_sort(PfArgs a) {
 //     order; SwiGLU / store happen there.  One barrier per step (two
 //     tile-matrices per wave), two partial buffers.
 // ======================================================================
+template <int BITS>
 struct PfSlab {
     static constexpr int GPW = 4;                       // groups per wave
-    static constexpr int CB = 24 * GPW;                 // code bytes of a row inside the slab
+    static constexpr int CB = 8 * BITS * GPW;           // code bytes of a row inside the slab: 96 / 128
     static constexpr int PS = 16;                       // bytes a lane copies per load
-    static constexpr int RP = CB / PS;                  // pieces per row: 6
-    // a row takes 7 piece slots in LDS (the 7th stays empty): with 96-byte rows the
-    // 128-bit reads of eight neighbouring rows hit the same banks twice over
-    static constexpr int RS = RP + 1;                   // piece slots per row in LDS
-    static constexpr int PIECES = 32 * RS;              // piece slots of a tile-matrix: 224
+    static constexpr int RP = CB / PS;                  // pieces per row: 6 / 8
+    // a row takes one piece slot more in LDS (it stays empty): with 96- or 128-byte rows the
+    // 128-bit reads of neighbouring rows would hit the same banks
+    static constexpr int RS = RP + 1;                   // piece slots per row in LDS: 7 / 9
+    static constexpr int PIECES = 32 * RS;              // piece slots of a tile-matrix: 224 / 288
     static constexpr int NQ = (PIECES + 63) / 64;       // LDS-direct loads for the codes
-    static constexpr int LDS_CODE = PIECES * PS;        // 3584
+    static constexpr int LDS_CODE = PIECES * PS;        // 3584 / 4608
     static constexpr int SLOT = LDS_CODE + 512;         // + scales 256 + biases 256
     static constexpr int LOADS = NQ + 2;
-    static constexpr int RING = 3;
     static constexpr int RED_BYTES = 2 * 2 * 8 * 8 * 64 * 4;   // [buffer][matrix][wave][reg][lane]
+    // what is left of the 160 KB for the eight waves' rings: 3 slots of 4096 B / 2 of 5120 B
+    static constexpr int RING = (160 * 1024 - RED_BYTES) / (8 * SLOT);
     static constexpr int LDS_BYTES = 8 * RING * SLOT + RED_BYTES;
+    static_assert(RING >= 2, "a ring needs a slot in flight beside the one being multiplied");
 };
 
 // three bf16 pieces (bit patterns) of v, the last one truncated
@@ -283,10 +311,11 @@ __device__ __forceinline__ void pf_pieces(float v, uint32_t *pc) {
 //   every team on its own 64 rows of a step's 256; a step = two row tiles per team; sum over
 //   the team's two waves, expert_out.  The activation operand comes from aop / asums
 //   (fm_pf_prepare_act), indexed by sorted position.
-template <bool DOWN>
+template <bool DOWN, int BITS>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fm_pf_gemm(PfArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // (the host pass cannot allocate the registers of the asm blocks)
-    using P = PfSlab;
+    using P = PfSlab<BITS>;
+    constexpr int DW = PfCode<BITS>::DW;
     constexpr int GPW = P::GPW;
     constexpr int RING = P::RING;
     extern __shared__ __attribute__((aligned(16))) uint8_t pf2_smem[];
@@ -298,7 +327,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint32_t red0 = lds0 + 8 * RING * P::SLOT;
     const int n_items = *a.n_items;
     const int in_dim = DOWN ? a.g.inter : a.g.hidden;
-    const int row_bytes = in_dim * 3 / 8, sb_bytes = (in_dim / 64) * 2;
+    const int row_bytes = in_dim * BITS / 8, sb_bytes = (in_dim / 64) * 2;
     const int slab = DOWN ? (wave & 1) : wave, team = DOWN ? (wave >> 1) : 0;
     const int n_steps = DOWN ? a.g.hidden / 256 : a.g.inter / 32;
     const uint32_t ones = fm_opaque(0x3F803F80u);
@@ -492,35 +521,48 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 if (issued - consumed == (uint32_t)RING) fm_dma_wait<P::LOADS *(RING - 1)>(false);
                 else fm_dma_wait<0>(true);
                 const uint32_t slot = ring0 + (uint32_t)c * P::SLOT;
-                uint32_t cw[GPW][3], sw[2], bw[2];
-                {
-                    // the whole 96-byte run of the row (both half lanes read the same
-                    // pieces), then this lane's half of every group
-                    const uint32_t ac = slot + (uint32_t)(n * (P::RS * 16));
+                uint32_t cw[GPW][DW], sw[2], bw[2];
+                if constexpr (BITS == 4) {
+                    // a lane's half of a group is one 16-byte piece
+                    const uint32_t ac = slot + (uint32_t)(n * (P::RS * 16) + 16 * hh);
                     const uint32_t as = slot + P::LDS_CODE + 8 * n;
-                    fm_u4 r0, r1, r2, r3, r4, r5;
+                    fm_u4 r0, r1, r2, r3;
                     asm volatile(
-                        "ds_read_b128 %0, %10\n\tds_read_b128 %1, %10 offset:16\n\t"
-                        "ds_read_b128 %2, %10 offset:32\n\tds_read_b128 %3, %10 offset:48\n\t"
-                        "ds_read_b128 %4, %10 offset:64\n\tds_read_b128 %5, %10 offset:80\n\t"
-                        "ds_read_b32 %6, %11\n\tds_read_b32 %7, %11 offset:4\n\t"
-                        "ds_read_b32 %8, %11 offset:256\n\tds_read_b32 %9, %11 offset:260\n\t"
+                        "ds_read_b128 %0, %8\n\tds_read_b128 %1, %8 offset:32\n\t"
+                        "ds_read_b128 %2, %8 offset:64\n\tds_read_b128 %3, %8 offset:96\n\t"
+                        "ds_read_b32 %4, %9\n\tds_read_b32 %5, %9 offset:4\n\t"
+                        "ds_read_b32 %6, %9 offset:256\n\tds_read_b32 %7, %9 offset:260\n\t"
                         "s_waitcnt lgkmcnt(0)"
-                        : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(r4), "=&v"(r5),
-                          "=&v"(sw[0]), "=&v"(sw[1]), "=&v"(bw[0]), "=&v"(bw[1])
+                        : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(sw[0]), "=&v"(sw[1]),
+                          "=&v"(bw[0]), "=&v"(bw[1])
                         : "v"(ac), "v"(as)
                         : "memory");
-                    const uint32_t rd[24] = {r0.x, r0.y, r0.z, r0.w, r1.x, r1.y, r1.z, r1.w,
-                                             r2.x, r2.y, r2.z, r2.w, r3.x, r3.y, r3.z, r3.w,
-                                             r4.x, r4.y, r4.z, r4.w, r5.x, r5.y, r5.z, r5.w};
-                    // (one side made opaque: the compiler otherwise turns the select into
-                    // rd[6*gi + 3*hh + d], a run-time index into registers, which it expands
-                    // into a compare-and-select over all 24 of them)
+                    const fm_u4 rr[4] = {r0, r1, r2, r3};
 #pragma unroll
-                    for (int gi = 0; gi < 4; gi++)
-#pragma unroll
-                        for (int d = 0; d < 3; d++)
-                            cw[gi][d] = hh ? fm_opaque(rd[6 * gi + 3 + d]) : rd[6 * gi + d];
+                    for (int gi = 0; gi < 4; gi++) {
+                        cw[gi][0] = rr[gi].x, cw[gi][1] = rr[gi].y;
+                        cw[gi][DW - 2] = rr[gi].z, cw[gi][DW - 1] = rr[gi].w;
+                    }
+                } else {
+                    // a lane's half of a group is 12 bytes, 4-byte aligned: three dword reads per
+                    // group.  (Reading the row's whole 96-byte run with 128-bit reads and picking
+                    // the half out of the registers costs twice the LDS bytes and a select per
+                    // register: 4 us per 512-position chunk.)
+                    const uint32_t ac = slot + (uint32_t)(n * (P::RS * 16) + 12 * hh);
+                    const uint32_t as = slot + P::LDS_CODE + 8 * n;
+                    asm volatile(
+                        "ds_read_b32 %0, %16\n\tds_read_b32 %1, %16 offset:4\n\tds_read_b32 %2, %16 offset:8\n\t"
+                        "ds_read_b32 %3, %16 offset:24\n\tds_read_b32 %4, %16 offset:28\n\tds_read_b32 %5, %16 offset:32\n\t"
+                        "ds_read_b32 %6, %16 offset:48\n\tds_read_b32 %7, %16 offset:52\n\tds_read_b32 %8, %16 offset:56\n\t"
+                        "ds_read_b32 %9, %16 offset:72\n\tds_read_b32 %10, %16 offset:76\n\tds_read_b32 %11, %16 offset:80\n\t"
+                        "ds_read_b32 %12, %17\n\tds_read_b32 %13, %17 offset:4\n\t"
+                        "ds_read_b32 %14, %17 offset:256\n\tds_read_b32 %15, %17 offset:260\n\t"
+                        "s_waitcnt lgkmcnt(0)"
+                        : "=&v"(cw[0][0]), "=&v"(cw[0][1]), "=&v"(cw[0][2]), "=&v"(cw[1][0]), "=&v"(cw[1][1]),
+                          "=&v"(cw[1][2]), "=&v"(cw[2][0]), "=&v"(cw[2][1]), "=&v"(cw[2][2]), "=&v"(cw[3][0]),
+                          "=&v"(cw[3][1]), "=&v"(cw[3][2]), "=&v"(sw[0]), "=&v"(sw[1]), "=&v"(bw[0]), "=&v"(bw[1])
+                        : "v"(ac), "v"(as)
+                        : "memory");
                 }
                 consumed++;
                 c = c + 1 == RING ? 0 : c + 1;
@@ -546,7 +588,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     f16v dg[GPW];
 #pragma unroll
                     for (int gi = 0; gi < GPW; gi++) {
-                        pf_unpack<0>(cw[gi], ones, v[gi]);
+                        pf_unpack<BITS, 0>(cw[gi], ones, v[gi]);
 #pragma unroll
                         for (int i = 0; i < 16; i++) dg[gi][i] = 0.0f;
                     }
@@ -688,10 +730,34 @@ __global__ __launch_bounds__(256) void fm_pf_combine(PfArgs a, float *out, int f
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 bool pf_supported(const FmExpertGeom *g) {
-    // 3-bit codes, BF16 scales (their bits are MFMA operands), whole 32-row tiles and
-    // an even number of groups; LDS image must fit
-    return g->bits == 3 && !g->scale_fp16 && g->n_experts <= PF_MAX_EXPERTS && g->hidden == 2048 &&
+    // 3- or 4-bit codes, BF16 scales (their bits are MFMA operands), the benchmark's widths
+    // (eight and two slabs of four groups)
+    return (g->bits == 3 || g->bits == 4) && !g->scale_fp16 && g->n_experts <= PF_MAX_EXPERTS && g->hidden == 2048 &&
            g->inter == 512;
+}
+
+template <int BITS>
+int pf_launch(const PfArgs &a, const FmExpertGeom *g, int M, float *d_out, int flags, int n_cu,
+              hipStream_t st) {
+    const size_t n = (size_t)M * a.K;
+    // workgroup 0 sorts, the rest turn X into operand registers (one thread per position,
+    // group and half)
+    const int prep_tasks = M * (g->hidden / 64) * 2;
+    hipLaunchKernelGGL(fm_pf_sort<BITS>, dim3(1 + (prep_tasks + 1023) / 1024), dim3(1024), 0, st, a);
+    const int max_items = g->n_experts + (int)(n / PF_TM);
+    // one 8-wave workgroup per CU (LDS: the ring and the partial tiles take all 160 KB; ~220-245
+    // registers per lane cap a SIMD at two waves)
+    const int grid = max_items < n_cu ? max_items : n_cu;
+    constexpr int LDS = PfSlab<BITS>::LDS_BYTES;
+    static FmLdsAttr attr_up, attr_down;
+    if (!fm_dyn_lds_ready(attr_up, (const void *)fm_pf_gemm<false, BITS>, LDS)) return FM_ERR_HIP;
+    if (!fm_dyn_lds_ready(attr_down, (const void *)fm_pf_gemm<true, BITS>, LDS)) return FM_ERR_HIP;
+    hipLaunchKernelGGL((fm_pf_gemm<false, BITS>), dim3(grid), dim3(512), LDS, st, a);
+    const int act_tasks = (int)n * (g->inter / 64) * 2;
+    hipLaunchKernelGGL(fm_pf_prepare_act<BITS>, dim3((act_tasks + 255) / 256), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((fm_pf_gemm<true, BITS>), dim3(grid), dim3(512), LDS, st, a);
+    hipLaunchKernelGGL(fm_pf_combine, dim3(M, (g->hidden + 1023) / 1024), dim3(256), 0, st, a, d_out, flags);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 
 }  // namespace
@@ -732,21 +798,7 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
     a.xsums = (float2 *)ws;               ws += align256((size_t)M * (g->hidden / 64) * sizeof(float2));
     a.aop = (uint4 *)ws;                  ws += align256(n * (g->inter / 64) * 16 * sizeof(uint4));
     a.asums = (float2 *)ws;
-    // workgroup 0 sorts, the rest turn X into operand registers (one thread per position,
-    // group and half)
-    const int prep_tasks = M * (g->hidden / 64) * 2;
-    hipLaunchKernelGGL(fm_pf_sort, dim3(1 + (prep_tasks + 1023) / 1024), dim3(1024), 0, st, a);
-    const int max_items = g->n_experts + (int)(n / PF_TM);
-    // one 8-wave workgroup per CU (LDS: the ring and the partial tiles take all 160 KB; ~220-245
-    // registers per lane cap a SIMD at two waves)
-    const int grid = max_items < n_cu ? max_items : n_cu;
-    static FmLdsAttr attr_up, attr_down;
-    if (!fm_dyn_lds_ready(attr_up, (const void *)fm_pf_gemm<false>, PfSlab::LDS_BYTES)) return FM_ERR_HIP;
-    if (!fm_dyn_lds_ready(attr_down, (const void *)fm_pf_gemm<true>, PfSlab::LDS_BYTES)) return FM_ERR_HIP;
-    hipLaunchKernelGGL(fm_pf_gemm<false>, dim3(grid), dim3(512), PfSlab::LDS_BYTES, st, a);
-    const int act_tasks = (int)n * (g->inter / 64) * 2;
-    hipLaunchKernelGGL(fm_pf_prepare_act, dim3((act_tasks + 255) / 256), dim3(256), 0, st, a);
-    hipLaunchKernelGGL(fm_pf_gemm<true>, dim3(grid), dim3(512), PfSlab::LDS_BYTES, st, a);
-    hipLaunchKernelGGL(fm_pf_combine, dim3(M, (g->hidden + 1023) / 1024), dim3(256), 0, st, a, d_out, flags);
-    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+    return g->bits == 3 ? pf_launch<3>(a, g, M, d_out, flags, n_cu, st)
+                        : pf_launch<4>(a, g, M, d_out, flags, n_cu, st);
 }
+
