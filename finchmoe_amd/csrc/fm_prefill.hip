@@ -19,7 +19,8 @@
 //     which land in registers i and i+8 of the same lane;
 //   * the bias term sum_g b[row][g] * xsum[pos][g] and the offset the "1 +" adds,
 //     sum_g s[row][g] * xoff[pos][g], are two small products over the group index,
-//     also on MFMA: the bf16 bits of b and s are operands as they are.
+//     also on MFMA: the bf16 bits of b and s are operands as they are (FP16 ones are
+//     split into a bf16 head and tail first, pf_side_b).
 //
 // V_MFMA_F32_32X32X16_BF16 with positions on M and weight rows on N: lane
 // (n = lane%32, h = lane/32) supplies 8 consecutive k of weight row n and holds
@@ -304,6 +305,33 @@ __device__ __forceinline__ void pf_pieces(float v, uint32_t *pc) {
     pc[2] = __float_as_uint(v) >> 16;
 }
 
+// B operands of the bias / offset MFMAs: the slab's four 16-bit values of a row (w0 = groups
+// 0, 1; w1 = groups 2, 3) against the K slots of this half lane — hh = 0: piece 0 and piece 1
+// of the activation sums, hh = 1: piece 2 and piece 0 again.  BF16 values are operands as they
+// are (the fourth slot group stays empty).  An FP16 value (11 significant bits) is split exactly
+// into a bf16 head (8 bits) and tail (3 bits): heads everywhere, the tails in the fourth slot
+// group; tail x piece 1, as large as head x piece 2, goes into one more MFMA for both terms
+// (`tails`); tail x piece 2 is below fp32 precision.
+template <bool FP16>
+__device__ __forceinline__ uint4 pf_side_b(uint32_t w0, uint32_t w1, int hh, uint2 &tails) {
+    if constexpr (!FP16) {
+        tails = make_uint2(0u, 0u);
+        return hh ? make_uint4(w0, w1, 0u, 0u) : make_uint4(w0, w1, w0, w1);
+    } else {
+        uint32_t head[4], tail[4];
+        const float f[4] = {fm_fp16_bits(w0 & 0xFFFFu), fm_fp16_bits(w0 >> 16), fm_fp16_bits(w1 & 0xFFFFu),
+                            fm_fp16_bits(w1 >> 16)};
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            head[g] = __float_as_uint(f[g]) & 0xFFFF0000u;
+            tail[g] = __float_as_uint(f[g] - __uint_as_float(head[g]));
+        }
+        const uint32_t h0 = (head[0] >> 16) | head[1], h1 = (head[2] >> 16) | head[3];
+        tails = make_uint2((tail[0] >> 16) | (tail[1] & 0xFFFF0000u), (tail[2] >> 16) | (tail[3] & 0xFFFF0000u));
+        return hh ? make_uint4(h0, h1, tails.x, tails.y) : make_uint4(h0, h1, h0, h1);
+    }
+}
+
 // DOWN = false: gate/up.  K = hidden is eight slabs, wave w owns slab w, all waves work on the
 //   same 32 rows; a step = the gate tile and the up tile of those rows; sum over eight waves,
 //   SwiGLU, act.
@@ -311,7 +339,7 @@ __device__ __forceinline__ void pf_pieces(float v, uint32_t *pc) {
 //   every team on its own 64 rows of a step's 256; a step = two row tiles per team; sum over
 //   the team's two waves, expert_out.  The activation operand comes from aop / asums
 //   (fm_pf_prepare_act), indexed by sorted position.
-template <bool DOWN, int BITS>
+template <bool DOWN, int BITS, bool FP16>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fm_pf_gemm(PfArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // (the host pass cannot allocate the registers of the asm blocks)
     using P = PfSlab<BITS>;
@@ -501,8 +529,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 const int p0 = hh ? 2 : 0;
                 sideA[term][0] = pc[0][p0] | (pc[1][p0] << 16);
                 sideA[term][1] = pc[2][p0] | (pc[3][p0] << 16);
-                sideA[term][2] = hh ? 0u : pc[0][1] | (pc[1][1] << 16);
-                sideA[term][3] = hh ? 0u : pc[2][1] | (pc[3][1] << 16);
+                // (hh = 1: piece 0 once more, for the tails of FP16 scales and biases; BF16 ones
+                // put zeros against it)
+                sideA[term][2] = hh ? pc[0][0] | (pc[1][0] << 16) : pc[0][1] | (pc[1][1] << 16);
+                sideA[term][3] = hh ? pc[2][0] | (pc[3][0] << 16) : pc[2][1] | (pc[3][1] << 16);
                 if (n >= 16) sideA[term][0] = sideA[term][1] = sideA[term][2] = sideA[term][3] = 0u;
             }
         }
@@ -572,14 +602,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 f16v acc;
 #pragma unroll
                 for (int i = 0; i < 16; i++) acc[i] = 0.0f;
-                const uint4 Bb = hh ? make_uint4(bw[0], bw[1], 0u, 0u) : make_uint4(bw[0], bw[1], bw[0], bw[1]);
-                const uint4 Bs = hh ? make_uint4(sw[0], sw[1], 0u, 0u) : make_uint4(sw[0], sw[1], sw[0], sw[1]);
+                uint2 tb, ts;
+                const uint4 Bb = pf_side_b<FP16>(bw[0], bw[1], hh, tb);
+                const uint4 Bs = pf_side_b<FP16>(sw[0], sw[1], hh, ts);
                 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
                     __builtin_bit_cast(bf8, make_uint4(sideA[0][0], sideA[0][1], sideA[0][2], sideA[0][3])),
                     __builtin_bit_cast(bf8, Bb), acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
                     __builtin_bit_cast(bf8, make_uint4(sideA[1][0], sideA[1][1], sideA[1][2], sideA[1][3])),
                     __builtin_bit_cast(bf8, Bs), acc, 0, 0, 0);
+                if constexpr (FP16) {
+                    // tails x piece 1 of both terms: K slots 0..3 biases, 4..7 scales (hh = 0 lanes)
+                    const uint4 At = hh ? make_uint4(0u, 0u, 0u, 0u)
+                                        : make_uint4(sideA[0][2], sideA[0][3], sideA[1][2], sideA[1][3]);
+                    const uint4 Bt = hh ? make_uint4(0u, 0u, 0u, 0u) : make_uint4(tb.x, tb.y, ts.x, ts.y);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8, At),
+                                                                  __builtin_bit_cast(bf8, Bt), acc, 0, 0, 0);
+                }
                 // the groups' MFMA chains interleaved (a chain's next MFMA needs the previous
                 // one's result: back to back it would idle the matrix core for most of its
                 // 8 passes), the scales applied once all four are done
@@ -604,7 +643,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                         }
 #pragma unroll
                     for (int gi = 0; gi < GPW; gi++) {
-                        const float sc = (gi & 1) ? fm_bf16_hi(sw[gi >> 1]) : fm_bf16_lo(sw[gi >> 1]);
+                        const float sc = (gi & 1) ? fm_widen_hi<FP16>(sw[gi >> 1]) : fm_widen_lo<FP16>(sw[gi >> 1]);
 #pragma unroll
                         for (int i = 0; i < 16; i++) acc[i] = fmaf(sc, dg[gi][i], acc[i]);
                     }
@@ -730,13 +769,12 @@ __global__ __launch_bounds__(256) void fm_pf_combine(PfArgs a, float *out, int f
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 bool pf_supported(const FmExpertGeom *g) {
-    // 3- or 4-bit codes, BF16 scales (their bits are MFMA operands), the benchmark's widths
-    // (eight and two slabs of four groups)
-    return (g->bits == 3 || g->bits == 4) && !g->scale_fp16 && g->n_experts <= PF_MAX_EXPERTS && g->hidden == 2048 &&
+    // 3- or 4-bit codes at the benchmark's widths (eight and two slabs of four groups)
+    return (g->bits == 3 || g->bits == 4) && g->n_experts <= PF_MAX_EXPERTS && g->hidden == 2048 &&
            g->inter == 512;
 }
 
-template <int BITS>
+template <int BITS, bool FP16>
 int pf_launch(const PfArgs &a, const FmExpertGeom *g, int M, float *d_out, int flags, int n_cu,
               hipStream_t st) {
     const size_t n = (size_t)M * a.K;
@@ -750,12 +788,12 @@ int pf_launch(const PfArgs &a, const FmExpertGeom *g, int M, float *d_out, int f
     const int grid = max_items < n_cu ? max_items : n_cu;
     constexpr int LDS = PfSlab<BITS>::LDS_BYTES;
     static FmLdsAttr attr_up, attr_down;
-    if (!fm_dyn_lds_ready(attr_up, (const void *)fm_pf_gemm<false, BITS>, LDS)) return FM_ERR_HIP;
-    if (!fm_dyn_lds_ready(attr_down, (const void *)fm_pf_gemm<true, BITS>, LDS)) return FM_ERR_HIP;
-    hipLaunchKernelGGL((fm_pf_gemm<false, BITS>), dim3(grid), dim3(512), LDS, st, a);
+    if (!fm_dyn_lds_ready(attr_up, (const void *)fm_pf_gemm<false, BITS, FP16>, LDS)) return FM_ERR_HIP;
+    if (!fm_dyn_lds_ready(attr_down, (const void *)fm_pf_gemm<true, BITS, FP16>, LDS)) return FM_ERR_HIP;
+    hipLaunchKernelGGL((fm_pf_gemm<false, BITS, FP16>), dim3(grid), dim3(512), LDS, st, a);
     const int act_tasks = (int)n * (g->inter / 64) * 2;
     hipLaunchKernelGGL(fm_pf_prepare_act<BITS>, dim3((act_tasks + 255) / 256), dim3(256), 0, st, a);
-    hipLaunchKernelGGL((fm_pf_gemm<true, BITS>), dim3(grid), dim3(512), LDS, st, a);
+    hipLaunchKernelGGL((fm_pf_gemm<true, BITS, FP16>), dim3(grid), dim3(512), LDS, st, a);
     hipLaunchKernelGGL(fm_pf_combine, dim3(M, (g->hidden + 1023) / 1024), dim3(256), 0, st, a, d_out, flags);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
@@ -798,7 +836,10 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
     a.xsums = (float2 *)ws;               ws += align256((size_t)M * (g->hidden / 64) * sizeof(float2));
     a.aop = (uint4 *)ws;                  ws += align256(n * (g->inter / 64) * 16 * sizeof(uint4));
     a.asums = (float2 *)ws;
-    return g->bits == 3 ? pf_launch<3>(a, g, M, d_out, flags, n_cu, st)
-                        : pf_launch<4>(a, g, M, d_out, flags, n_cu, st);
+    if (g->scale_fp16)
+        return g->bits == 3 ? pf_launch<3, true>(a, g, M, d_out, flags, n_cu, st)
+                            : pf_launch<4, true>(a, g, M, d_out, flags, n_cu, st);
+    return g->bits == 3 ? pf_launch<3, false>(a, g, M, d_out, flags, n_cu, st)
+                        : pf_launch<4, false>(a, g, M, d_out, flags, n_cu, st);
 }
 

@@ -12,16 +12,18 @@ pytestmark = pytest.mark.gpu
 H, I, E = 2048, 512, 12
 
 
-@pytest.fixture(scope="module", params=[3, 4], ids=["3bit", "4bit"])
+@pytest.fixture(scope="module", params=[(3, "bf16"), (4, "bf16"), (3, "fp16"), (4, "fp16")],
+                ids=["3bit", "4bit", "3bit-fp16scales", "4bit-fp16scales"])
 def pstore(request):
     from finchmoe_amd import FinchHip
-    bits = request.param
+    bits, dtype = request.param
+    sd = fb.SCALE_BF16 if dtype == "bf16" else fb.SCALE_FP16
     rng = np.random.default_rng(404)
-    blob = F.synth_expert_layer(rng, E, H, I, bits)
+    blob = F.synth_expert_layer(rng, E, H, I, bits, dtype)
     ctx = FinchHip(0)
-    ctx.experts_config(1, E, H, I, 64, bits, fb.SCALE_BF16)
+    ctx.experts_config(1, E, H, I, 64, bits, sd)
     ctx.experts_upload_layer(0, blob)
-    yield ctx, blob, bits
+    yield ctx, blob, (bits, sd)
     ctx.close()
 
 
@@ -33,14 +35,14 @@ def _routing(orc, rng, M, K, n_experts=E):
 
 @pytest.mark.parametrize("M,K", [(64, 8), (33, 8), (40, 3), (128, 8)])
 def test_grouped_gemm_matches_per_position(pstore, orc, M, K):
-    ctx, blob, bits = pstore
+    ctx, blob, (bits, sd) = pstore
     rng = np.random.default_rng(M * 10 + K)
     X = rng.standard_normal((M, H)).astype(np.float32)
     idx, w = _routing(orc, rng, M, K)
     out = ctx.moe_prefill(0, X, idx, w)
     worst = 0.0
     for m in range(0, M, max(1, M // 16)):       # the oracle is slow: check a spread of positions
-        ref, _ = orc.moe_experts_forward(blob, X[m], idx[m], w[m], H, I, bits, nthreads=8)
+        ref, _ = orc.moe_experts_forward(blob, X[m], idx[m], w[m], H, I, bits, scale_dtype=sd, nthreads=8)
         r, c = assert_parity(out[m], ref, "position %d" % m)
         worst = max(worst, r)
     # every position against the per-position GPU path (itself checked against the oracle)
@@ -56,7 +58,7 @@ def test_grouped_gemm_edge_inputs(pstore, orc):
     """bf16-valued activations (the benchmark's x), zero weights, out-of-range indices, all
     positions on one expert, accumulate flag."""
     import torch
-    ctx, blob, bits = pstore
+    ctx, blob, (bits, sd) = pstore
     rng = np.random.default_rng(9)
     M, K = 48, 8
     X = torch.randn(M, H).to(torch.bfloat16).to(torch.float32).numpy()
@@ -69,13 +71,13 @@ def test_grouped_gemm_edge_inputs(pstore, orc):
     out = ctx.moe_prefill(0, X, idx, w, flags=fb.ACCUMULATE, out=base.copy())
     for m in (0, 5, 7, 9, 10, 47):
         keep = [k for k in range(K) if w[m, k] != 0 and 0 <= idx[m, k] < E]
-        ref, _ = orc.moe_experts_forward(blob, X[m], idx[m, keep], w[m, keep], H, I, bits, nthreads=8)
+        ref, _ = orc.moe_experts_forward(blob, X[m], idx[m, keep], w[m, keep], H, I, bits, scale_dtype=sd, nthreads=8)
         assert rel_err(out[m] - base[m], ref) < 1e-3 and cosine(out[m] - base[m], ref) > 0.99999, m
 
 
 def test_small_chunks_and_guard_use_position_path(pstore, orc):
     """Below the GEMM threshold, and with FM_GUARD, the chunk equals per-position calls bitwise."""
-    ctx, blob, bits = pstore
+    ctx, blob, (bits, sd) = pstore
     rng = np.random.default_rng(10)
     for M, flags in ((8, 0), (40, fb.GUARD)):
         X = rng.standard_normal((M, H)).astype(np.float32)
