@@ -103,3 +103,40 @@ def test_full_chunk_equals_positions(full_store, orc):
     mini = np.concatenate([blob[layer, int(e)].cpu().numpy() for e in idx[m]])
     ref, _ = orc.moe_experts_forward(mini, X[m], np.arange(K, dtype=np.int32), w[m], H, I, 3, nthreads=8)
     assert_parity(out[m], ref, "position %d" % m)
+
+
+def test_full_chunk_4bit_equals_positions(orc):
+    """The same 512-position chunk on one layer of 256 4-bit experts (453 MB): the grouped
+    product against per-position calls, and one position against the oracle."""
+    import torch
+    from bench import fill_affine_layer, zipf_routing
+    from finchmoe_amd import FinchHip
+    dev = torch.device("cuda:0")
+    lo = F.expert_layout(H, I, 4)
+    es = lo["expert_size"]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(77)
+    blob = torch.empty(1, E, es, dtype=torch.uint8, device=dev)
+    fill_affine_layer(blob[0], lo, 4, gen)
+    ctx = FinchHip(0)
+    try:
+        ctx.experts_config(1, E, H, I, 64, 4, 0)
+        ctx.experts_adopt_layer(0, blob[0].data_ptr(), E * es)
+        M = 512
+        idx, w = zipf_routing(np.random.default_rng(9), M, 1, E, K)
+        idx, w = np.ascontiguousarray(idx[:, 0]), np.ascontiguousarray(w[:, 0])
+        X = torch.randn(M, H).to(torch.bfloat16).to(torch.float32).numpy()
+        out = ctx.moe_prefill(0, X, idx, w)
+        assert np.isfinite(out).all()
+        assert np.array_equal(ctx.moe_prefill(0, X, idx, w), out)
+        for m in list(range(0, M, 41)) + [M - 1]:
+            single, _ = ctx.moe_decode(0, X[m], idx[m], w[m])
+            assert rel_err(out[m], single) < 1e-3 and cosine(out[m], single) > 0.99999, m
+        m = 77
+        mini = np.concatenate([blob[0, int(e)].cpu().numpy() for e in idx[m]])
+        ref, _ = orc.moe_experts_forward(mini, X[m], np.arange(K, dtype=np.int32), w[m], H, I, 4, nthreads=8)
+        assert_parity(out[m], ref, "position %d" % m)
+    finally:
+        ctx.close()
+        del blob
+        torch.cuda.empty_cache()
