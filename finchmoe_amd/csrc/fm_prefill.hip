@@ -386,8 +386,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // (item, step), items in order — every workgroup gets the same number of steps
     // (within one) whatever the number of items, at the price of building the
     // activation operand of an item in two workgroups when a share ends inside it
+    // Workgroups are dealt out to the eight XCDs in turn and every XCD has an L2 of its own:
+    // workgroup b takes share (b % 8) * (grid / 8) + b / 8, so that neighbouring shares — the
+    // items of one expert — run behind the same L2 and its weights come from HBM once.
     const long T = (long)n_items * n_steps;
-    const int t0 = (int)(T * blockIdx.x / gridDim.x), t1 = (int)(T * (blockIdx.x + 1) / gridDim.x);
+    const unsigned int share = gridDim.x % 8u == 0u ? (blockIdx.x % 8u) * (gridDim.x / 8u) + blockIdx.x / 8u
+                                                    : blockIdx.x;
+    const int t0 = (int)(T * share / gridDim.x), t1 = (int)(T * (share + 1) / gridDim.x);
 
     // ---- loader: tile-matrices of the share, in order
     int l_t = t0, l_it = t0 / n_steps, l_mat = 0, wpos = 0;
