@@ -189,13 +189,14 @@ int ensure_scratch(fm_ctx *c, int groups, int hidden, int inter) {
     HIPCHK(c, hipMalloc((void **)&c->d_eo, (size_t)g * FM_MAX_K * h * sizeof(float)));
     HIPCHK(c, hipMalloc((void **)&c->d_counters, (size_t)g * sizeof(unsigned int)));
     HIPCHK(c, hipMemsetAsync(c->d_counters, 0, (size_t)g * sizeof(unsigned int), c->stream));
-    {   // two sets of (pairs + groups) dependency counters, cleared once
+    {   // three sets of (pairs + groups) dependency counters, cleared once
         const size_t cap = (size_t)g * (FM_MAX_K + 1);
         unsigned int *p = nullptr;
-        HIPCHK(c, hipMalloc((void **)&p, 2 * cap * sizeof(unsigned int)));
-        HIPCHK(c, hipMemsetAsync(p, 0, 2 * cap * sizeof(unsigned int), c->stream));
+        HIPCHK(c, hipMalloc((void **)&p, 3 * cap * sizeof(unsigned int)));
+        HIPCHK(c, hipMemsetAsync(p, 0, 3 * cap * sizeof(unsigned int), c->stream));
         c->dflags.set[0] = p;
         c->dflags.set[1] = p + cap;
+        c->dflags.graph_set = p + 2 * cap;
         c->dflags.cap = (unsigned int)cap;
         c->dflags.err = c->d_err;
         c->dflags.spin_limit = c->wait_limit;

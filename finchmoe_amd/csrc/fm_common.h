@@ -21,9 +21,12 @@ struct FmExpertGeom {
 // Host-side state of the dependency counters of the fused decode kernel: two
 // sets of `cap` counters that alternate between launches (a launch counts in
 // set[parity] and clears the used[parity ^ 1] entries the launch before it left
-// in the other set), and the device word a timed-out wait raises.
+// in the other set), and the device word a timed-out wait raises.  A launch that is being
+// captured into a graph is replayed without the host code that alternates the sets: it counts
+// in `graph_set`, which a fill kernel recorded in front of it clears on every replay.
 struct FmDecodeFlags {
     unsigned int *set[2];
+    unsigned int *graph_set;
     unsigned int used[2];
     unsigned int cap;
     int parity;

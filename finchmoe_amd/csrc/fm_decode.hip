@@ -692,6 +692,11 @@ void fm_moe_fused(DecodeArgs a, int n_pairs, FmFlags f) {
     }
 }
 
+__global__ __launch_bounds__(256) void fm_clear_counters(unsigned int *p, unsigned int n) {
+    const unsigned int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
 // per kernel and device: dynamic LDS limit raised, resident workgroups per CU asked
 constexpr int FM_MAX_DEVICES = 64;
 struct FmKernelSetup {
@@ -877,10 +882,23 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     const unsigned int need = (unsigned int)(n_pairs + n_layers);
     FmFlags fl{};
     const FmFlags *flp = nullptr;
+    // A launch that is being captured into a graph will be replayed without this function: it
+    // gets the counter set kept for graphs and, recorded in front of it, a kernel that clears it.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (df && df->set[0]) (void)hipStreamIsCapturing(st, &capture);
+    const bool captured = capture == hipStreamCaptureStatusActive;
     if (df && df->set[0] && need <= df->cap) {
-        fl.cur = df->set[df->parity];
-        fl.other = df->set[df->parity ^ 1];
-        fl.clear_n = df->used[df->parity ^ 1];
+        if (captured) {
+            hipLaunchKernelGGL(fm_clear_counters, dim3((need + 255) / 256), dim3(256), 0, st,
+                               df->graph_set, need);
+            fl.cur = df->graph_set;
+            fl.other = df->graph_set;
+            fl.clear_n = 0u;
+        } else {
+            fl.cur = df->set[df->parity];
+            fl.other = df->set[df->parity ^ 1];
+            fl.clear_n = df->used[df->parity ^ 1];
+        }
         fl.err = df->err;
         fl.spin_limit = df->spin_limit;
         flp = &fl;
@@ -891,7 +909,7 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     if (g->bits == 3) rc = g->scale_fp16 ? FM_DEC(3, true) : FM_DEC(3, false);
     else if (g->bits == 4) rc = g->scale_fp16 ? FM_DEC(4, true) : FM_DEC(4, false);
 #undef FM_DEC
-    if (fused) {   // the set just used is dirty, the other one is clean again
+    if (fused && !captured) {   // the set just used is dirty, the other one is clean again
         df->used[df->parity] = need;
         df->used[df->parity ^ 1] = 0u;
         df->parity ^= 1;
