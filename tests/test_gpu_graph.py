@@ -83,3 +83,68 @@ def test_decode_step_replayed_from_graph():
         hip.hipGraphDestroy(graph)
     finally:
         ctx.close()
+
+
+def test_moe_half_of_a_layer_replayed_from_graph():
+    """routing GEMVs -> route -> routed experts -> layer tail (four kinds of launch, two of them
+    with counters or tickets in device memory) captured once and replayed with new inputs."""
+    import torch
+    from finchmoe_amd import FinchHip
+    hip = _hip()
+    rng = np.random.default_rng(32)
+    Ee = 16
+    ctx = FinchHip(0)
+    try:
+        ctx.experts_config(1, Ee, H, I, 64, 3, fb.SCALE_BF16)
+        ctx.experts_upload_layer(0, F.synth_expert_layer(rng, Ee, H, I, 3))
+        tens = [F.synth_affine_tensor(rng, r, c, b, "bf16")
+                for (r, c, b) in ((Ee, H, 8), (1, H, 8), (I, H, 4), (I, H, 4), (H, I, 4))]
+        t_gate, t_seg, t_sg, t_su, t_sd = [ctx.tensor_register(*t[1:], r, c, b) for t, (r, c, b) in
+                                           zip(tens, ((Ee, H, 8), (1, H, 8), (I, H, 4), (I, H, 4), (H, I, 4)))]
+        nw = (1.0 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+        d_nw = torch.from_numpy((nw.view(np.uint32) >> 16).astype(np.uint16).view(np.int16)).cuda()
+        d_x, d_hmid = torch.zeros(H, device="cuda"), torch.zeros(H, device="cuda")
+        d_log, d_seg = torch.empty(Ee, device="cuda"), torch.empty(1, device="cuda")
+        d_sg, d_su = torch.empty(I, device="cuda"), torch.empty(I, device="cuda")
+        d_idx = torch.empty(K, dtype=torch.int32, device="cuda")
+        d_w, d_p = torch.empty(K, device="cuda"), torch.empty(10, device="cuda")
+        d_moe, d_eo = torch.empty(H, device="cuda"), torch.empty(K, H, device="cuda")
+        outs = [torch.zeros(H, device="cuda") for _ in range(4)]     # hidden, next: graph / eager
+
+        def chain(d_hid, d_next):
+            ctx.matvec_batch_dev([t_gate, t_seg, t_sg, t_su], d_x.data_ptr(),
+                                 [d_log.data_ptr(), d_seg.data_ptr(), d_sg.data_ptr(), d_su.data_ptr()])
+            ctx.route_topk_dev(d_log.data_ptr(), Ee, K, d_seg.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(),
+                               d_p.data_ptr())
+            ctx.moe_decode_dev(0, d_x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, d_moe.data_ptr(),
+                               d_eo.data_ptr())
+            ctx.layer_tail_dev(t_sd, d_hmid.data_ptr(), d_eo.data_ptr(), d_p.data_ptr(), K, d_sg.data_ptr(),
+                               d_su.data_ptr(), d_nw.data_ptr(), 1e-6, d_hid.data_ptr(), d_next.data_ptr())
+
+        def new_inputs():
+            d_x.copy_(torch.from_numpy(rng.standard_normal(H).astype(np.float32)))
+            d_hmid.copy_(torch.from_numpy(rng.standard_normal(H).astype(np.float32)))
+            torch.cuda.synchronize()
+
+        new_inputs()
+        chain(outs[2], outs[3])
+        ctx.sync()
+        stream = C.c_void_p(ctx.stream())
+        graph, gexec = C.c_void_p(), C.c_void_p()
+        assert hip.hipStreamBeginCapture(stream, 2) == 0
+        chain(outs[0], outs[1])
+        assert hip.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        for rep in range(4):
+            new_inputs()
+            chain(outs[2], outs[3])
+            ctx.sync()
+            assert hip.hipGraphLaunch(gexec, stream) == 0
+            ctx.sync()
+            assert np.array_equal(outs[0].cpu().numpy(), outs[2].cpu().numpy()), rep
+            assert np.array_equal(outs[1].cpu().numpy(), outs[3].cpu().numpy()), rep
+            assert np.isfinite(outs[1].cpu().numpy()).all() and np.abs(outs[1].cpu().numpy()).max() > 0
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)
+    finally:
+        ctx.close()
