@@ -7,7 +7,7 @@ HBM, per-layer top-8 indices from a Zipf(1.1) distribution with a per-layer rank
 router weights = renormalised softmax of N(0,1) logits at those indices.  A "step" is one
 token: one pass of the hot path over all 40 layers.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_layer|gdn|gguf|gguf_chunk|prefill|lm_head|layer_tail]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_layer|gdn|gguf|gguf_chunk|prefill|lm_head|layer_tail|moe_layer]
 
 Prints ONE JSON line.  `value` is algorithmic weight bytes per step / wall time per step with
 all inputs resident in HBM.  `roofline` prices the dominant kernel against the 8 TB/s HBM
@@ -428,6 +428,95 @@ def run_layer_tail(args):
                    "next-layer norm; 40 tensors cycled", bytes_call, ms, args)
 
 
+def run_moe_layer(args):
+    """The MoE half of every layer without a host round trip, one token per step: routing and
+    shared-expert GEMVs (8-bit gate [256,2048] and shared-gate score, 4-bit shared gate/up
+    [512,2048]) -> softmax/top-8 -> routed experts -> shared down + combine + residual + next
+    layer's norm (finchmoe/infer.m:9285-9760), layer l+1 reading what layer l wrote.  Four
+    launches per layer; with --graph the whole token is one captured HIP graph."""
+    import ctypes as C
+    import torch
+    from finchmoe_amd import FinchHip, formats
+    dev = torch.device("cuda:0")
+    n_layers = args.layers
+    lo = formats.expert_layout(H, I, 3)
+    es = lo["expert_size"]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(99)
+    blob = torch.empty(n_layers, E, es, dtype=torch.uint8, device=dev)
+    for l in range(n_layers):
+        fill_affine_layer(blob[l], lo, 3, gen)
+    ctx = FinchHip(0)
+    ctx.experts_config(n_layers, E, H, I, 64, 3, 0)
+    for l in range(n_layers):
+        ctx.experts_adopt_layer(l, blob[l].data_ptr(), E * es)
+    keep, dense_bytes = [], 0
+
+    def tensor(rows, cols, bits, gain):
+        nonlocal dense_bytes
+        W = torch.empty(rows * cols * bits // 8, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
+        half = ((1 << bits) - 1) / 2.0
+        sc = torch.randn(rows * (cols // 64), device=dev, generator=gen).abs_() * (gain / half)
+        S, B = _bf16_trunc_bits(sc), _bf16_trunc_bits(sc * -half)
+        keep.extend([W, S, B])
+        dense_bytes += W.numel() + 4 * S.numel()
+        return ctx.tensor_adopt(W.data_ptr(), S.data_ptr(), B.data_ptr(), rows, cols, bits)
+
+    layers = []
+    for l in range(n_layers):
+        layers.append((tensor(E, H, 8, 0.05), tensor(1, H, 8, 0.02), tensor(I, H, 4, 0.02),
+                       tensor(I, H, 4, 0.02), tensor(H, I, 4, 0.02)))
+    x0 = torch.randn(H, device=dev)
+    hid = [torch.empty(H, device=dev) for _ in range(2)]
+    xin = [torch.empty(H, device=dev) for _ in range(2)]
+    d_log, d_seg = torch.empty(E, device=dev), torch.empty(1, device=dev)
+    d_sg, d_su = torch.empty(I, device=dev), torch.empty(I, device=dev)
+    d_idx = torch.empty(K, dtype=torch.int32, device=dev)
+    d_w, d_p = torch.empty(K, device=dev), torch.empty(10, device=dev)
+    d_moe, d_eo = torch.empty(H, device=dev), torch.empty(K, H, device=dev)
+    nw = torch.ones(H, device=dev).to(torch.bfloat16)
+    torch.cuda.synchronize()
+
+    def token():
+        for l in range(n_layers):
+            t_gate, t_seg, t_sg, t_su, t_sd = layers[l]
+            x = x0 if l == 0 else xin[(l - 1) & 1]
+            h_mid = x0 if l == 0 else hid[(l - 1) & 1]
+            ctx.matvec_batch_dev([t_gate, t_seg, t_sg, t_su], x.data_ptr(),
+                                 [d_log.data_ptr(), d_seg.data_ptr(), d_sg.data_ptr(), d_su.data_ptr()])
+            ctx.route_topk_dev(d_log.data_ptr(), E, K, d_seg.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(),
+                               d_p.data_ptr())
+            ctx.moe_decode_dev(l, x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, d_moe.data_ptr(),
+                               d_eo.data_ptr())
+            ctx.layer_tail_dev(t_sd, h_mid.data_ptr(), d_eo.data_ptr(), d_p.data_ptr(), K, d_sg.data_ptr(),
+                               d_su.data_ptr(), nw.data_ptr(), 1e-6, hid[l & 1].data_ptr(), xin[l & 1].data_ptr())
+
+    token()
+    ctx.sync()
+    ref = xin[(n_layers - 1) & 1].clone()
+    assert torch.isfinite(ref).all() and ref.abs().max() > 0
+    step = lambda t: token()
+    if args.graph:
+        hip = C.CDLL("libamdhip64.so")
+        stream, graph, gexec = C.c_void_p(ctx.stream()), C.c_void_p(), C.c_void_p()
+        assert hip.hipStreamBeginCapture(stream, C.c_int(2)) == 0
+        token()
+        assert hip.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+        step = lambda t: hip.hipGraphLaunch(gexec, stream)
+    ms, ev = _timed(ctx, step, args)
+    ctx.sync()
+    assert torch.equal(xin[(n_layers - 1) & 1], ref)      # same inputs, same result on every step
+    res = {"us_per_layer": round(ms * 1e3 / n_layers, 2), "launches_per_layer": 4,
+           "graph": bool(args.graph), "event_ms_per_step": round(ev, 5)}
+    ctx.close()
+    return _finish(res, "MoE half of a layer on the device, GB/s over a %d-layer token" % n_layers,
+                   "routing + shared-expert GEMVs, top-8, routed 3-bit experts (router-chosen), shared "
+                   "down + combine + norm; %d layers chained, %s" % (n_layers, "one HIP graph per token"
+                                                                     if args.graph else "eager launches"),
+                   n_layers * K * es + dense_bytes, ms, args)
+
+
 def run_gguf(args):
     """config 4: GGUF experts (Q4_K gate/up, Q6_K down), 40-layer decode step, batch 1."""
     import torch
@@ -586,6 +675,8 @@ def main():
     ap.add_argument("--chunk", type=int, default=512, help="positions per chunk (prefill workload)")
     ap.add_argument("--ramp-seconds", type=float, default=0.5,
                     help="untimed busy period before the warmup steps (clock ramp)")
+    ap.add_argument("--graph", action="store_true",
+                    help="moe_layer workload: replay the token from a captured HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
@@ -599,6 +690,7 @@ def main():
         sys.exit(3)
     runners = {"decode_step": run_decode_step, "decode_layer": run_decode_layer, "gdn": run_gdn,
                "gguf": run_gguf, "gguf_chunk": run_gguf, "prefill": run_prefill, "lm_head": run_lm_head, "layer_tail": run_layer_tail,
+               "moe_layer": run_moe_layer,
                "copy_probe": run_copy_probe}
     if args.workload not in runners:
         print("bench.py: unknown workload %r (have: %s)" % (args.workload, ", ".join(runners)),
