@@ -1,0 +1,55 @@
+"""bench.py's contract where no GPU is needed: one GPU only, no CPU fallback, the routing
+generator of the benchmark (distinct experts per layer, weights summing to one, Zipf skew)."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _run(*args):
+    return subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), *args], capture_output=True,
+                          text=True, timeout=300)
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = _run("--gpus", "2", "--steps", "1", "--warmup", "0")
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_no_gpu_means_no_result():
+    import torch
+    if torch.cuda.is_available():
+        return
+    r = _run("--steps", "1", "--warmup", "0", "--no-cpu")
+    assert r.returncode != 0 and "no CPU fallback" in r.stderr and r.stdout.strip() == ""
+
+
+def test_unknown_workload_is_refused():
+    import torch
+    if not torch.cuda.is_available():
+        return      # the GPU check comes first
+    r = _run("--workload", "nonsense")
+    assert r.returncode != 0 and "unknown workload" in r.stderr
+
+
+def test_zipf_routing_of_the_benchmark():
+    sys.path.insert(0, ROOT)
+    from bench import zipf_routing
+    idx, w = zipf_routing(np.random.default_rng(7), 64, 3, 256, 8)
+    assert idx.shape == (64, 3, 8) and w.shape == (64, 3, 8)
+    assert idx.min() >= 0 and idx.max() < 256
+    for t in range(64):
+        for l in range(3):
+            assert len(set(idx[t, l].tolist())) == 8          # distinct per (token, layer)
+    assert np.allclose(w.sum(-1), 1.0, atol=1e-6) and (w > 0).all()
+    # skewed: the most frequent expert of a layer is hit far more often than the uniform 8/256
+    for l in range(3):
+        counts = np.bincount(idx[:, l].reshape(-1), minlength=256)
+        assert counts.max() > 0.5 * 64
+    # a fresh permutation per layer: the hot experts differ between layers
+    hot = [int(np.bincount(idx[:, l].reshape(-1), minlength=256).argmax()) for l in range(3)]
+    assert len(set(hot)) > 1
