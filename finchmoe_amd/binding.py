@@ -93,6 +93,8 @@ def load():
         "fm_dequant_expert": (i, [vp, i, i, i, vp, vp, vp]),
         "fm_dequant_tensor": (i, [vp, i, vp, vp, vp]),
         "fm_gguf_dequant_expert": (i, [vp, i, i, i, vp]),
+        "fm_embed_lookup_dev": (i, [vp, i, vp, i, vp]),
+        "fm_embed_lookup": (i, [vp, i, i, vp]),
     }
     for name, (res, args) in sig.items():
         f = getattr(L, name)
@@ -335,6 +337,14 @@ class FinchHip:
         w16 = np.empty((out_dim, in_dim), np.uint16)
         self._chk(self.L.fm_dequant_tensor(self.h, t, _ptr(codes), _ptr(w32), _ptr(w16)))
         return codes, w32, w16
+
+    def embed_lookup_dev(self, t, d_token_ids, n_tokens, d_out):
+        self._chk(self.L.fm_embed_lookup_dev(self.h, t, d_token_ids, n_tokens, d_out))
+
+    def embed_lookup(self, t, token_id, in_dim):
+        out = np.empty(in_dim, np.float32)
+        self._chk(self.L.fm_embed_lookup(self.h, t, int(token_id), _ptr(out)))
+        return out
 
     def gguf_dequant_expert(self, layer, expert, which):
         rows, cols = (self.g_hidden, self.g_inter) if which == DOWN else (self.g_inter, self.g_hidden)

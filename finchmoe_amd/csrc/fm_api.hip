@@ -1087,6 +1087,43 @@ extern "C" int fm_dequant_tensor(fm_ctx *c, fm_tensor t, uint8_t *codes, float *
                           codes, w_f32, w_f16);
 }
 
+extern "C" int fm_launch_embed_rows(const void *W, const void *S, const void *B, int rows, int in_dim,
+                                    int group_size, int bits, int scale_fp16, const int32_t *d_ids,
+                                    int n, float *d_out, hipStream_t st);
+
+extern "C" int fm_embed_lookup_dev(fm_ctx *c, fm_tensor t, const int32_t *d_token_ids, int n_tokens,
+                                   float *d_out) {
+    if (!c) return FM_ERR_ARG;
+    Tensor *p = get_tensor(c, t);
+    if (!p) return fail(c, FM_ERR_ARG, "bad tensor handle %d", t);
+    if (!d_token_ids || !d_out) return fail(c, FM_ERR_ARG, "null pointer");
+    if (n_tokens < 1) return fail(c, FM_ERR_ARG, "n_tokens %d", n_tokens);
+    DeviceGuard dg(c->device);
+    int rc = fm_launch_embed_rows(p->W, p->S, p->B, p->out_dim, p->in_dim, p->group_size, p->bits,
+                                  p->scale_fp16, d_token_ids, n_tokens, d_out, c->stream);
+    if (rc) return fail(c, rc, "embedding lookup launch failed: %s", hipGetErrorString(hipGetLastError()));
+    return FM_OK;
+}
+
+extern "C" int fm_embed_lookup(fm_ctx *c, fm_tensor t, int token_id, float *out) {
+    if (!c) return FM_ERR_ARG;
+    Tensor *p = get_tensor(c, t);
+    if (!p) return fail(c, FM_ERR_ARG, "bad tensor handle %d", t);
+    if (!out) return fail(c, FM_ERR_ARG, "null pointer");
+    DeviceGuard dg(c->device);
+    const size_t need = 256 + (size_t)p->in_dim * sizeof(float);
+    int rc = ensure_stage(c, need);
+    if (rc) return rc;
+    *(int32_t *)c->h_stage = token_id;          // pinned mirror of the staging buffer
+    HIPCHK(c, hipMemcpyAsync(c->d_stage, c->h_stage, sizeof(int32_t), hipMemcpyHostToDevice, c->stream));
+    float *d_out = (float *)((char *)c->d_stage + 256);
+    rc = fm_embed_lookup_dev(c, t, (const int32_t *)c->d_stage, 1, d_out);
+    if (rc) return rc;
+    HIPCHK(c, hipMemcpyAsync(out, d_out, (size_t)p->in_dim * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(c, hipStreamSynchronize(c->stream));
+    return FM_OK;
+}
+
 extern "C" int fm_gguf_dequant_expert(fm_ctx *c, int layer, int expert, int which, float *w_f32) {
     if (!c) return FM_ERR_ARG;
     if (!c->gguf_cfg) return fail(c, FM_ERR_STATE, "GGUF store not configured");

@@ -6,6 +6,31 @@
 
 namespace {
 
+// code and fp32 weight of element (r, col) of an affine tensor
+__device__ __forceinline__ float fm_affine_elem(const uint8_t *W, const uint16_t *S, const uint16_t *B,
+                                                int r, int col, int in_dim, int group_size, int bits,
+                                                int scale_fp16, uint32_t &q) {
+    if (bits == 3) {
+        // 8 codes per 24-bit little-endian field (repack_experts.py:250-257)
+        const uint8_t *p = W + (size_t)r * (in_dim * 3 / 8) + 3 * (col >> 3);
+        uint32_t v = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
+        q = (v >> (3 * (col & 7))) & 7u;
+    } else {
+        // LSB-first fields of a little-endian u32 (quantize_model.py:35-43)
+        int vpu = 32 / bits;
+        const uint32_t *p = reinterpret_cast<const uint32_t *>(W) + (size_t)r * (in_dim / vpu);
+        q = (p[col / vpu] >> ((col % vpu) * bits)) & ((1u << bits) - 1u);
+    }
+    int ng = in_dim / group_size;
+    uint32_t sbits = S[(size_t)r * ng + col / group_size];
+    uint32_t bbits = B[(size_t)r * ng + col / group_size];
+    float s = scale_fp16 ? fm_fp16_bits(sbits) : fm_bf16_lo(sbits);
+    float b = scale_fp16 ? fm_fp16_bits(bbits) : fm_bf16_lo(bbits);
+    // code * scale is exact in fp32 (<= 8 + 11 significant bits), so the sum
+    // is rounded once whether or not the compiler contracts it into an FMA
+    return (float)q * s + b;
+}
+
 __global__ void fm_dequant_affine_k(const uint8_t *W, const uint16_t *S, const uint16_t *B,
                                     int out_dim, int in_dim, int group_size, int bits,
                                     int scale_fp16, uint8_t *codes, float *w32,
@@ -15,31 +40,30 @@ __global__ void fm_dequant_affine_k(const uint8_t *W, const uint16_t *S, const u
          i += (size_t)gridDim.x * blockDim.x) {
         int r = (int)(i / in_dim), col = (int)(i % in_dim);
         uint32_t q;
-        if (bits == 3) {
-            // 8 codes per 24-bit little-endian field (repack_experts.py:250-257)
-            const uint8_t *p = W + (size_t)r * (in_dim * 3 / 8) + 3 * (col >> 3);
-            uint32_t v = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
-            q = (v >> (3 * (col & 7))) & 7u;
-        } else {
-            // LSB-first fields of a little-endian u32 (quantize_model.py:35-43)
-            int vpu = 32 / bits;
-            const uint32_t *p = reinterpret_cast<const uint32_t *>(W) + (size_t)r * (in_dim / vpu);
-            q = (p[col / vpu] >> ((col % vpu) * bits)) & ((1u << bits) - 1u);
-        }
-        int ng = in_dim / group_size;
-        uint32_t sbits = S[(size_t)r * ng + col / group_size];
-        uint32_t bbits = B[(size_t)r * ng + col / group_size];
-        float s = scale_fp16 ? fm_fp16_bits(sbits) : fm_bf16_lo(sbits);
-        float b = scale_fp16 ? fm_fp16_bits(bbits) : fm_bf16_lo(bbits);
-        // code * scale is exact in fp32 (<= 8 + 11 significant bits), so the sum
-        // is rounded once whether or not the compiler contracts it into an FMA
-        float w = (float)q * s + b;
+        float w = fm_affine_elem(W, S, B, r, col, in_dim, group_size, bits, scale_fp16, q);
         if (codes) codes[i] = (uint8_t)q;
         if (w32) w32[i] = w;
         if (w16) {
             _Float16 h = (_Float16)w;   // round-to-nearest-even
             w16[i] = __builtin_bit_cast(unsigned short, h);
         }
+    }
+}
+
+// Embedding lookup: out[i] = dequantized row ids[i] of an affine tensor [rows][in_dim], one
+// workgroup per id (embed_lookup, finchmoe/infer.m:5664-5722: the 4-/8-bit branch; a missing
+// tensor gives zeros there, an id outside the tensor gives zeros here).
+__global__ __launch_bounds__(256) void fm_embed_rows_k(const uint8_t *W, const uint16_t *S,
+                                                       const uint16_t *B, int rows, int in_dim,
+                                                       int group_size, int bits, int scale_fp16,
+                                                       const int32_t *ids, float *out) {
+    const int r = ids[blockIdx.x];
+    float *o = out + (size_t)blockIdx.x * in_dim;
+    for (int col = threadIdx.x; col < in_dim; col += blockDim.x) {
+        uint32_t q;
+        o[col] = (unsigned)r < (unsigned)rows
+                     ? fm_affine_elem(W, S, B, r, col, in_dim, group_size, bits, scale_fp16, q)
+                     : 0.0f;
     }
 }
 
@@ -98,6 +122,15 @@ extern "C" int fm_launch_dequant_affine(const void *W, const void *S, const void
     hipLaunchKernelGGL(fm_dequant_affine_k, dim3(blocks), dim3(256), 0, st,
                        (const uint8_t *)W, (const uint16_t *)S, (const uint16_t *)B, out_dim,
                        in_dim, group_size, bits, scale_fp16, codes, w32, w16);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
+
+extern "C" int fm_launch_embed_rows(const void *W, const void *S, const void *B, int rows, int in_dim,
+                                    int group_size, int bits, int scale_fp16, const int32_t *d_ids,
+                                    int n, float *d_out, hipStream_t st) {
+    hipLaunchKernelGGL(fm_embed_rows_k, dim3(n), dim3(256), 0, st, (const uint8_t *)W,
+                       (const uint16_t *)S, (const uint16_t *)B, rows, in_dim, group_size, bits,
+                       scale_fp16, d_ids, d_out);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 

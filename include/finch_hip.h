@@ -234,6 +234,16 @@ FM_API int fm_gguf_moe_prefill(fm_ctx *ctx, int layer, const float *X, const int
 FM_API int fm_gguf_matvec(fm_ctx *ctx, const void *W, int ggml_type, const float *x, float *out,
                    int out_dim, int in_dim);
 
+/* ---------------------------------------------------------------- embedding lookup
+ * embed_lookup(wf, token_id, out) (finchmoe/infer.m:5664-5722, the 4-/8-bit branch): row
+ * token_id of a registered affine tensor [vocab][hidden], dequantized to fp32 —
+ * out[j] = (float)code * scale + bias, the same value fm_dequant_tensor gives for that row.
+ * The _dev form takes n ids from device memory (one row each, out [n][in_dim], asynchronous
+ * on the context's stream); an id outside the tensor gives a row of zeros. */
+FM_API int fm_embed_lookup_dev(fm_ctx *ctx, fm_tensor t, const int32_t *d_token_ids, int n_tokens,
+                        float *d_out);
+FM_API int fm_embed_lookup(fm_ctx *ctx, fm_tensor t, int token_id, float *out);
+
 /* ---------------------------------------------------------------- dequant (bit-exact checks)
  * The reference has no such call; these expose what its kernels compute on the
  * fly — code = field of the packed word, w = (float)code * scale + bias in fp32

@@ -112,3 +112,31 @@ def test_mixed_batch_and_errors(hip, orc):
     assert e.value.status == fb.ERR_UNSUPPORTED
     for t in (t4, t8, t5):
         hip.tensor_release(t)
+
+
+@pytest.mark.parametrize("bits,dtype", [(8, "bf16"), (4, "bf16"), (4, "fp16")])
+def test_embedding_lookup_is_the_dequantized_row(hip, orc, bits, dtype):
+    """embed_lookup (infer.m:5664-5722): the row of a token, bit for bit the oracle's dequant of
+    that row; ids from device memory, an id outside the table gives zeros."""
+    import torch
+    rng = np.random.default_rng(50 + bits)
+    vocab, hidden = 1000, 2048
+    _, W, S, B = F.synth_affine_tensor(rng, vocab, hidden, bits, dtype)
+    sd = fb.SCALE_BF16 if dtype == "bf16" else fb.SCALE_FP16
+    t = hip.tensor_register(W, S, B, vocab, hidden, bits, scale_dtype=sd)
+    try:
+        _, ref32 = orc.dequant_affine(W, S, B, vocab, hidden, bits, scale_dtype=sd)
+        for tok in (0, 1, 517, vocab - 1):
+            got = hip.embed_lookup(t, tok, hidden)
+            assert np.array_equal(got.view(np.uint32), ref32[tok].view(np.uint32)), tok
+        ids = np.array([3, 999, 3, -1, vocab, 42], np.int32)
+        d_ids = torch.from_numpy(ids).cuda()
+        d_out = torch.full((len(ids), hidden), 7.0, device="cuda")
+        hip.embed_lookup_dev(t, d_ids.data_ptr(), len(ids), d_out.data_ptr())
+        hip.sync()
+        out = d_out.cpu().numpy()
+        for i, tok in enumerate(ids):
+            want = ref32[tok] if 0 <= tok < vocab else np.zeros(hidden, np.float32)
+            assert np.array_equal(out[i].view(np.uint32), want.view(np.uint32)), (i, tok)
+    finally:
+        hip.tensor_release(t)
