@@ -41,9 +41,10 @@ def _bf16_trunc_bits(t):
     return (t.contiguous().view(torch.int32) >> 16).to(torch.int16)
 
 
-def fill_affine_layer(view, lo, bits, gen):
+def fill_affine_layer(view, lo, bits, gen, fp16=False):
     """view: uint8 [E, expert_size] on the GPU.  Random codes (all bit patterns are uniform
-    codes), scale = bf16(|N(0,0.02)|/3.5), bias = bf16(-3.5*scale)."""
+    codes), scale = bf16(|N(0,0.02)|/3.5), bias = bf16(-3.5*scale) — or both as IEEE halves
+    (fp16: the benchmark text's wording; the reference's files hold bf16)."""
     import torch
     view.random_(0, 256, generator=gen)
     for name, rows, cols in (("gate", I, H), ("up", I, H), ("down", H, I)):
@@ -52,7 +53,8 @@ def fill_affine_layer(view, lo, bits, gen):
         b = s * -3.5
         for part, val in (("s", s), ("b", b)):
             o = lo[name + "_" + part]
-            view[:, o:o + 2 * n] = _bf16_trunc_bits(val).view(torch.uint8).view(view.shape[0], 2 * n)
+            bits16 = val.to(torch.float16).view(torch.int16) if fp16 else _bf16_trunc_bits(val)
+            view[:, o:o + 2 * n] = bits16.contiguous().view(torch.uint8).view(view.shape[0], 2 * n)
 
 
 def zipf_routing(rng, tokens, layers, n_experts, k):
@@ -72,7 +74,7 @@ def zipf_routing(rng, tokens, layers, n_experts, k):
     return idx, w
 
 
-def cpu_baseline_decode(blob_t, lo, idx, w, x, budget_s=12.0, bits=3):
+def cpu_baseline_decode(blob_t, lo, idx, w, x, budget_s=12.0, bits=3, scale_dtype=0):
     """Oracle expert loop, 1 thread (the reference's path is single-threaded), on (token, layer)
     samples until ~budget_s of CPU time; then a shorter leg with the rows split over 16 threads
     (per-row arithmetic unchanged).  Only the 8 routed experts of each sample are copied back
@@ -90,7 +92,7 @@ def cpu_baseline_decode(blob_t, lo, idx, w, x, budget_s=12.0, bits=3):
             mini = np.concatenate([blob_t[l, int(e)].cpu().numpy() for e in sel])
             t0 = time.perf_counter()
             oracle.moe_experts_forward(mini, x[l % x.shape[0]], np.arange(len(sel), dtype=np.int32),
-                                       w[t, l], H, I, bits, nthreads=nthreads)
+                                       w[t, l], H, I, bits, scale_dtype=scale_dtype, nthreads=nthreads)
             t_cpu += time.perf_counter() - t0
             done += 1
             if t_cpu >= budget:
@@ -127,11 +129,12 @@ def run_decode_step(args):
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
     blob = torch.empty(n_layers, E, es, dtype=torch.uint8, device=dev)
+    fp16 = args.scale_dtype == "fp16"
     for l in range(n_layers):
-        fill_affine_layer(blob[l], lo, bits, gen)
+        fill_affine_layer(blob[l], lo, bits, gen, fp16)
     torch.cuda.synchronize()
     ctx = FinchHip(0)
-    ctx.experts_config(n_layers, E, H, I, 64, bits, 0)
+    ctx.experts_config(n_layers, E, H, I, 64, bits, 1 if fp16 else 0)
     for l in range(n_layers):
         ctx.experts_adopt_layer(l, blob[l].data_ptr(), E * es)
 
@@ -206,7 +209,7 @@ def run_decode_step(args):
                                "g64 experts resident in HBM (%.2f GB), top-%d Zipf(1.1) routing, "
                                "x~N(0,1) fp32" % (n_layers, n_layers, E, bits, n_layers * E * es / 1e9, K),
                    "hidden": H, "moe_intermediate": I, "experts": E, "top_k": K, "layers": n_layers,
-                   "bytes_per_step": bytes_step, "scale_dtype": "bf16"},
+                   "bytes_per_step": bytes_step, "scale_dtype": args.scale_dtype},
         "us_per_step": round(ms_per_step * 1e3, 2),
         "us_per_layer": round(ms_per_step * 1e3 / n_layers, 3),
         "tokens_per_s": round(1e3 / ms_per_step, 1),
@@ -228,7 +231,7 @@ def run_decode_step(args):
                                  "down_GBps": round((bytes_step - k1_bytes) / (k2_us * 1e-6) / 1e9, 1)},
     }
     if not args.no_cpu:
-        res["cpu_baseline"] = cpu_baseline_decode(blob, lo, idx, w, x, args.cpu_seconds, bits)
+        res["cpu_baseline"] = cpu_baseline_decode(blob, lo, idx, w, x, args.cpu_seconds, bits, 1 if fp16 else 0)
     ctx.close()
     return res
 
@@ -621,10 +624,11 @@ def run_prefill(args):
     gen.manual_seed(1234)
     nl = 8
     blob = torch.empty(nl, E, es, dtype=torch.uint8, device=dev)
+    fp16 = args.scale_dtype == "fp16"
     for l in range(nl):
-        fill_affine_layer(blob[l], lo, bits, gen)
+        fill_affine_layer(blob[l], lo, bits, gen, fp16)
     ctx = FinchHip(0)
-    ctx.experts_config(nl, E, H, I, 64, bits, 0)
+    ctx.experts_config(nl, E, H, I, 64, bits, 1 if fp16 else 0)
     for l in range(nl):
         ctx.experts_adopt_layer(l, blob[l].data_ptr(), E * es)
     rng = np.random.default_rng(7)
@@ -649,8 +653,8 @@ def run_prefill(args):
            "unique_experts_per_chunk": uniq, "event_ms_per_step": round(ev, 5)}
     ctx.close()
     out = _finish(res, "chunked-prefill expert product, %d-position chunk" % M,
-                  "config 3: %d-token chunk, top-8 Zipf(1.1), %d-bit g64 experts, x~N(0,1) bf16 values in fp32"
-                  % (M, bits), int(uniq * es), ms, args, {"flops_per_step": flops})
+                  "config 3: %d-token chunk, top-8 Zipf(1.1), %d-bit g64 experts (%s scales), x~N(0,1) bf16 values in fp32"
+                  % (M, bits, args.scale_dtype), int(uniq * es), ms, args, {"flops_per_step": flops})
     return out
 
 
@@ -684,6 +688,8 @@ def main():
     ap.add_argument("--layers", type=int, default=L)
     ap.add_argument("--bits", type=int, default=3, choices=(3, 4),
                     help="affine code width of the decode_step and prefill workloads")
+    ap.add_argument("--scale-dtype", default="bf16", choices=("bf16", "fp16"),
+                    help="type of the group scales and biases (decode_step and prefill workloads)")
     ap.add_argument("--chunk", type=int, default=512, help="positions per chunk (prefill workload)")
     ap.add_argument("--ramp-seconds", type=float, default=0.5,
                     help="untimed busy period before the warmup steps (clock ramp)")
