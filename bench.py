@@ -7,7 +7,7 @@ HBM, per-layer top-8 indices from a Zipf(1.1) distribution with a per-layer rank
 router weights = renormalised softmax of N(0,1) logits at those indices.  A "step" is one
 token: one pass of the hot path over all 40 layers.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_layer|gdn|gguf|gguf_chunk|prefill|lm_head|layer_tail|moe_layer]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_step|decode_layer|gdn|gguf|gguf_chunk|prefill|lm_head|layer_tail|moe_layer|gdn_prefill]
 
 Prints ONE JSON line.  `value` is algorithmic weight bytes per step / wall time per step with
 all inputs resident in HBM.  `roofline` prices the dominant kernel against the 8 TB/s HBM
@@ -532,6 +532,53 @@ def run_moe_layer(args):
                    n_layers * K * es + dense_bytes, ms, args)
 
 
+def run_gdn_prefill(args):
+    """config 1's tensors against M positions (M = --chunk, the reference's
+    gpu_encode_prefill_matvec): in_proj_qkv [8192,2048] and in_proj_z [4096,2048] from X[M,2048],
+    out_proj [2048,4096] from Y[M,4096]; 4-bit g64.  From 16 positions on the products run on the
+    matrix cores."""
+    import torch
+    from finchmoe_amd import FinchHip
+    dev = torch.device("cuda:0")
+    M = args.chunk
+    ctx = FinchHip(0)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(21)
+    keep, sets, nsets = [], [], 8
+
+    def tensor(rows, cols):
+        W = torch.empty(rows * cols // 2, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
+        sc = torch.randn(rows * (cols // 64), device=dev, generator=gen).abs_() * (0.02 / 7.5)
+        S, B = _bf16_trunc_bits(sc), _bf16_trunc_bits(sc * -7.5)
+        keep.extend([W, S, B])
+        return ctx.tensor_adopt(W.data_ptr(), S.data_ptr(), B.data_ptr(), rows, cols, 4)
+
+    for _ in range(nsets):
+        sets.append((tensor(8192, 2048), tensor(4096, 2048), tensor(2048, 4096)))
+    X, Y = torch.randn(M, 2048, device=dev), torch.randn(M, 4096, device=dev)
+    oq, oz, oo = (torch.empty(M, 8192, device=dev), torch.empty(M, 4096, device=dev),
+                  torch.empty(M, 2048, device=dev))
+    torch.cuda.synchronize()
+
+    def step(t):
+        tq, tz, to = sets[t % nsets]
+        ctx.matvec_prefill_dev(tq, X.data_ptr(), oq.data_ptr(), M)
+        ctx.matvec_prefill_dev(tz, X.data_ptr(), oz.data_ptr(), M)
+        ctx.matvec_prefill_dev(to, Y.data_ptr(), oo.data_ptr(), M)
+
+    ms, ev = _timed(ctx, step, args)
+    assert torch.isfinite(oo).all() and torch.isfinite(oq).all()
+    flops = 2.0 * M * (12288 * 2048 + 2048 * 4096)
+    res = {"tflops": round(flops / (ms * 1e-3) / 1e12, 2),
+           "frac_of_bf16_mfma_peak": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+           "event_ms_per_step": round(ev, 5)}
+    ctx.close()
+    return _finish(res, "dense 4-bit GatedDeltaNet projections against %d positions" % M,
+                   "config 1's weight set (qkv 8192x2048, z 4096x2048, out_proj 2048x4096, 4-bit g64) "
+                   "x %d positions, three calls per set, %d sets cycled" % (M, nsets),
+                   18874368, ms, args, {"flops_per_step": flops})
+
+
 def run_gguf(args):
     """config 4: GGUF experts (Q4_K gate/up, Q6_K down), 40-layer decode step, batch 1."""
     import torch
@@ -708,7 +755,7 @@ def main():
         sys.exit(3)
     runners = {"decode_step": run_decode_step, "decode_layer": run_decode_layer, "gdn": run_gdn,
                "gguf": run_gguf, "gguf_chunk": run_gguf, "prefill": run_prefill, "lm_head": run_lm_head, "layer_tail": run_layer_tail,
-               "moe_layer": run_moe_layer,
+               "moe_layer": run_moe_layer, "gdn_prefill": run_gdn_prefill,
                "copy_probe": run_copy_probe}
     if args.workload not in runners:
         print("bench.py: unknown workload %r (have: %s)" % (args.workload, ", ".join(runners)),

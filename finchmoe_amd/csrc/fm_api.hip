@@ -745,10 +745,38 @@ extern "C" int fm_matvec_batch_dev(fm_ctx *c, const fm_tensor *ts, int n, const 
     return matvec_dev(c, ts, n, d_x, d_outs, 1);
 }
 
+extern "C" size_t fm_prefill_dense_ws_bytes(int out_dim, int in_dim, int group_size, int bits, int M);
+extern "C" int fm_launch_prefill_dense(const void *d_W, const void *d_S, const void *d_B, int out_dim,
+                                       int in_dim, int group_size, int bits, int scale_fp16,
+                                       const float *d_X, int M, float *d_out, void *d_ws,
+                                       size_t ws_bytes, int flags, int n_cu, hipStream_t st);
+
+// positions from which the dense product runs on the matrix cores (below: one GEMV per position)
+#define FM_DENSE_GEMM_MIN_M 16
+
 extern "C" int fm_matvec_prefill_dev(fm_ctx *c, fm_tensor t, const float *d_X, float *d_out,
                                      int M) {
     if (!c) return FM_ERR_ARG;
     if (M < 1 || M > 65535) return fail(c, FM_ERR_ARG, "M %d outside 1..65535", M);
+    Tensor *p = get_tensor(c, t);
+    if (p && d_X && d_out && M >= FM_DENSE_GEMM_MIN_M && ((uintptr_t)d_X & 15) == 0 &&
+        ((uintptr_t)d_out & 3) == 0) {
+        static const bool no_gemm = getenv("FINCH_DENSE_NO_GEMM") != nullptr;
+        const size_t ws = no_gemm ? 0 : fm_prefill_dense_ws_bytes(p->out_dim, p->in_dim, p->group_size,
+                                                                  p->bits, M);
+        if (ws) {
+            DeviceGuard dg(c->device);
+            int rc = ensure_ws(c, ws);
+            if (rc) return rc;
+            rc = fm_launch_prefill_dense(p->W, p->S, p->B, p->out_dim, p->in_dim, p->group_size,
+                                         p->bits, p->scale_fp16, d_X, M, d_out, c->d_ws, c->ws_bytes,
+                                         0, c->n_cu, c->stream);
+            if (rc != FM_ERR_UNSUPPORTED) {
+                if (rc) return fail(c, rc, "dense prefill launch failed: %s", hipGetErrorString(hipGetLastError()));
+                return FM_OK;
+            }
+        }
+    }
     float *outs[1] = {d_out};
     return matvec_dev(c, &t, 1, d_X, outs, M);
 }

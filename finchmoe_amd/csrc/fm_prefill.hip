@@ -65,7 +65,15 @@ struct PfArgs {
     float2 *xsums;     // [M][hidden/64]: (xsum, xoff) of every group of every position
     uint4 *aop;        // [M*K][inter/64][4][2][2]: act (by sorted position) in the same form
     float2 *asums;     // [M*K][inter/64]
+    // dense tensor (PF_DENSE): out[M][d_rows] = X[M][d_cols] * W^T, scales / biases d_sb bytes
+    // behind / before W; one launch covers the 2048 columns of pass d_pass
+    const uint8_t *d_w;
+    ptrdiff_t d_s, d_b;
+    int d_rows, d_cols, d_pass, d_flags;
+    float *d_out;
 };
+
+enum { PF_GATE_UP = 0, PF_DOWN = 1, PF_DENSE = 2 };
 
 // ---- pairing of the 32 codes a lane holds for one group -------------------
 // Pair p fills k slots 2p (low half of the register, code lo(p) at mantissa bit tl(p)) and
@@ -332,18 +340,22 @@ __device__ __forceinline__ uint4 pf_side_b(uint32_t w0, uint32_t w1, int hh, uin
     }
 }
 
-// DOWN = false: gate/up.  K = hidden is eight slabs, wave w owns slab w, all waves work on the
+// MODE PF_GATE_UP (DOWN = false): K = hidden is eight slabs, wave w owns slab w, all waves work on the
 //   same 32 rows; a step = the gate tile and the up tile of those rows; sum over eight waves,
 //   SwiGLU, act.
-// DOWN = true: K = inter is two slabs: the workgroup is four teams of two waves (slab = wave & 1),
+// MODE PF_DOWN: K = inter is two slabs: the workgroup is four teams of two waves (slab = wave & 1),
 //   every team on its own 64 rows of a step's 256; a step = two row tiles per team; sum over
 //   the team's two waves, expert_out.  The activation operand comes from aop / asums
 //   (fm_pf_prepare_act), indexed by sorted position.
-template <bool DOWN, int BITS, bool FP16>
+// MODE PF_DENSE: one dense tensor against M positions, 2048 of its columns per launch (eight slabs
+//   as in gate/up; column pass d_pass adds to what the passes before it stored); an item is a
+//   block of 16 positions, a step = two row tiles (64 rows), the operand comes from xop.
+template <int MODE, int BITS, bool FP16>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fm_pf_gemm(PfArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // (the host pass cannot allocate the registers of the asm blocks)
     using P = PfSlab<BITS>;
     constexpr int DW = PfCode<BITS>::DW;
+    constexpr bool DOWN = MODE == PF_DOWN, DENSE = MODE == PF_DENSE;
     constexpr int GPW = P::GPW;
     constexpr int RING = P::RING;
     extern __shared__ __attribute__((aligned(16))) uint8_t pf2_smem[];
@@ -354,20 +366,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint32_t ring0 = lds0 + (uint32_t)wave * (RING * P::SLOT);
     const uint32_t red0 = lds0 + 8 * RING * P::SLOT;
     const int n_items = *a.n_items;
-    const int in_dim = DOWN ? a.g.inter : a.g.hidden;
+    const int in_dim = DENSE ? a.d_cols : DOWN ? a.g.inter : a.g.hidden;
     const int row_bytes = in_dim * BITS / 8, sb_bytes = (in_dim / 64) * 2;
-    const int slab = DOWN ? (wave & 1) : wave, team = DOWN ? (wave >> 1) : 0;
-    const int n_steps = DOWN ? a.g.hidden / 256 : a.g.inter / 32;
+    const int slab = DENSE ? wave + 8 * a.d_pass : DOWN ? (wave & 1) : wave, team = DOWN ? (wave >> 1) : 0;
+    const int n_steps = DENSE ? a.d_rows / 64 : DOWN ? a.g.hidden / 256 : a.g.inter / 32;
     const uint32_t ones = fm_opaque(0x3F803F80u);
     // region offsets of the first tile-matrix of a step (this team's), the distance to the
     // second one, rows per step
-    const uint32_t w_off0 = DOWN ? a.g.down_w + 64u * team * row_bytes : a.g.gate_w;
-    const uint32_t s_off0 = DOWN ? a.g.down_s + 64u * team * sb_bytes : a.g.gate_s;
-    const uint32_t b_off0 = DOWN ? a.g.down_b + 64u * team * sb_bytes : a.g.gate_b;
-    const uint32_t w_d = DOWN ? 32u * row_bytes : a.g.up_w - a.g.gate_w;
-    const uint32_t s_d = DOWN ? 32u * sb_bytes : a.g.up_s - a.g.gate_s;
-    const uint32_t b_d = DOWN ? 32u * sb_bytes : a.g.up_b - a.g.gate_b;
-    const uint32_t step_rows = DOWN ? 256u : 32u;
+    // (byte offsets from the blob's — the dense tensor's W — first byte, modulo 2^64)
+    const size_t w_off0 = DENSE ? 0 : DOWN ? a.g.down_w + 64u * team * row_bytes : a.g.gate_w;
+    const size_t s_off0 = DENSE ? (size_t)a.d_s : DOWN ? a.g.down_s + 64u * team * sb_bytes : a.g.gate_s;
+    const size_t b_off0 = DENSE ? (size_t)a.d_b : DOWN ? a.g.down_b + 64u * team * sb_bytes : a.g.gate_b;
+    const uint32_t w_d = DOWN || DENSE ? 32u * row_bytes : a.g.up_w - a.g.gate_w;
+    const uint32_t s_d = DOWN || DENSE ? 32u * sb_bytes : a.g.up_s - a.g.gate_s;
+    const uint32_t b_d = DOWN || DENSE ? 32u * sb_bytes : a.g.up_b - a.g.gate_b;
+    const uint32_t step_rows = DENSE ? 64u : DOWN ? 256u : 32u;
+    const uint8_t *store = DENSE ? a.d_w : a.layer;          // what an item's "expert" indexes into
+    const size_t expert_size = DENSE ? 0 : a.g.expert_size;
     // this lane's pieces of a slot copy
     uint32_t coff[P::NQ];
     bool cvalid[P::NQ];
@@ -404,16 +419,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // slices before the multiply does, and a load here would wait for the whole ring
     int e_ahead = 0;
     if (!l_done) {
-        l_blob = fm_uniform(a.layer + (size_t)a.items[l_it].expert * a.g.expert_size);
+        l_blob = fm_uniform(store + (size_t)a.items[l_it].expert * expert_size);
         if (l_it + 1 < n_items) e_ahead = a.items[l_it + 1].expert;
     }
     auto issue = [&]() __attribute__((always_inline)) {
         if (l_done) return;
         const uint32_t slot = ring0 + (uint32_t)wpos * P::SLOT;
         const size_t row0 = (size_t)l_s * step_rows;
-        const uint8_t *wb = l_blob + w_off0 + (l_mat ? w_d : 0u) + row0 * row_bytes;
-        const uint8_t *sb = l_blob + s_off0 + (l_mat ? s_d : 0u) + row0 * sb_bytes;
-        const uint8_t *bb = l_blob + b_off0 + (l_mat ? b_d : 0u) + row0 * sb_bytes;
+        const uint8_t *wb = l_blob + (w_off0 + (l_mat ? w_d : 0u) + row0 * row_bytes);
+        const uint8_t *sb = l_blob + (s_off0 + (l_mat ? s_d : 0u) + row0 * sb_bytes);
+        const uint8_t *bb = l_blob + (b_off0 + (l_mat ? b_d : 0u) + row0 * sb_bytes);
 #pragma unroll
         for (int j = 0; j < P::NQ; j++)
             if (cvalid[j])
@@ -433,7 +448,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             } else if (++l_s == n_steps) {
                 l_s = 0;
                 l_it++;
-                l_blob = fm_uniform(a.layer + (size_t)e_ahead * a.g.expert_size);
+                l_blob = fm_uniform(store + (size_t)e_ahead * expert_size);
             }
         }
     };
@@ -458,7 +473,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 const int tok = 8 * (i / 4) + 4 * hh + (i % 4);
                 if (tok < item_next.count) out_pairs_next[i] = a.sorted[item_next.start + tok];
             }
-        } else {
+        } else if constexpr (!DENSE) {
             if ((n & 15) < item_next.count) pair_next = a.sorted[item_next.start + (n & 15)];
         }
     }
@@ -485,7 +500,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 // X was turned into operand registers once per chunk (pf_prepare): lane (m, hh)
                 // takes the hi (m < 16) or lo registers of its position, its groups, its half
                 const int piece = n < 16 ? 0 : 1;
-                const size_t m = !on ? 0 : DOWN ? (size_t)(item.start + pos) : (size_t)(pair_next / a.K);
+                const size_t m = !on ? 0 : DOWN || DENSE ? (size_t)(item.start + pos) : (size_t)(pair_next / a.K);
                 const int ng = in_dim / 64;
                 const uint4 *src = (DOWN ? a.aop : a.xop) + (m * ng + GPW * slab) * 16 + 2 * hh + piece;
                 const float2 *sm = (DOWN ? a.asums : a.xsums) + m * ng + GPW * slab;
@@ -518,7 +533,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                         out_pairs_next[i] = 0;
                         if (more && tok < item_next.count) out_pairs_next[i] = a.sorted[item_next.start + tok];
                     }
-                } else {
+                } else if constexpr (!DENSE) {
                     pair_next = 0;
                     if (more && pos < item_next.count) pair_next = a.sorted[item_next.start + pos];
                 }
@@ -694,7 +709,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     t0 += p[w2];
                     t1 += p[8 + w2];
                 }
-                if (my_on) {
+                if constexpr (DENSE) {
+                    // the two row tiles of the step; later column passes add to the earlier ones
+                    if (my_on) {
+                        float *o = a.d_out + (size_t)(item.start + my_pos) * a.d_rows + 64 * s + n;
+                        const bool add = a.d_pass > 0 || (a.d_flags & FM_ACCUMULATE);
+                        o[0] = add ? o[0] + t0 : t0;
+                        o[32] = add ? o[32] + t1 : t1;
+                    }
+                } else if (my_on) {
                     a.act[(size_t)(item.start + my_pos) * a.g.inter + 32 * s + n] = fm_silu_mul(t0, t1);
                 }
             } else {
@@ -771,6 +794,25 @@ __global__ __launch_bounds__(256) void fm_pf_combine(PfArgs a, float *out, int f
     }
 }
 
+// dense product: workgroup 0 cuts the M positions into items of PF_TM, the others prepare X
+template <int BITS>
+__global__ __launch_bounds__(1024) void fm_pf_dense_prep(PfArgs a) {
+    if (blockIdx.x > 0) {
+        pf_prepare<BITS>(a.X, a.M, a.d_cols, a.xop, a.xsums, (int)((blockIdx.x - 1) * blockDim.x + threadIdx.x));
+        return;
+    }
+    const int n = (a.M + PF_TM - 1) / PF_TM;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        PfItem it;
+        it.expert = 0;
+        it.start = i * PF_TM;
+        it.count = a.M - i * PF_TM < PF_TM ? a.M - i * PF_TM : PF_TM;
+        it.pad = 0;
+        a.items[i] = it;
+    }
+    if (threadIdx.x == 0) *a.n_items = n;
+}
+
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 bool pf_supported(const FmExpertGeom *g) {
@@ -793,17 +835,77 @@ int pf_launch(const PfArgs &a, const FmExpertGeom *g, int M, float *d_out, int f
     const int grid = max_items < n_cu ? max_items : n_cu;
     constexpr int LDS = PfSlab<BITS>::LDS_BYTES;
     static FmLdsAttr attr_up, attr_down;
-    if (!fm_dyn_lds_ready(attr_up, (const void *)fm_pf_gemm<false, BITS, FP16>, LDS)) return FM_ERR_HIP;
-    if (!fm_dyn_lds_ready(attr_down, (const void *)fm_pf_gemm<true, BITS, FP16>, LDS)) return FM_ERR_HIP;
-    hipLaunchKernelGGL((fm_pf_gemm<false, BITS, FP16>), dim3(grid), dim3(512), LDS, st, a);
+    if (!fm_dyn_lds_ready(attr_up, (const void *)fm_pf_gemm<PF_GATE_UP, BITS, FP16>, LDS)) return FM_ERR_HIP;
+    if (!fm_dyn_lds_ready(attr_down, (const void *)fm_pf_gemm<PF_DOWN, BITS, FP16>, LDS)) return FM_ERR_HIP;
+    hipLaunchKernelGGL((fm_pf_gemm<PF_GATE_UP, BITS, FP16>), dim3(grid), dim3(512), LDS, st, a);
     const int act_tasks = (int)n * (g->inter / 64) * 2;
     hipLaunchKernelGGL(fm_pf_prepare_act<BITS>, dim3((act_tasks + 255) / 256), dim3(256), 0, st, a);
-    hipLaunchKernelGGL((fm_pf_gemm<true, BITS, FP16>), dim3(grid), dim3(512), LDS, st, a);
+    hipLaunchKernelGGL((fm_pf_gemm<PF_DOWN, BITS, FP16>), dim3(grid), dim3(512), LDS, st, a);
     hipLaunchKernelGGL(fm_pf_combine, dim3(M, (g->hidden + 1023) / 1024), dim3(256), 0, st, a, d_out, flags);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 
+template <int BITS, bool FP16>
+int pf_launch_dense(PfArgs a, int n_cu, hipStream_t st) {
+    const int prep_tasks = a.M * (a.d_cols / 64) * 2;
+    hipLaunchKernelGGL(fm_pf_dense_prep<BITS>, dim3(1 + (prep_tasks + 1023) / 1024), dim3(1024), 0, st, a);
+    const long steps = (long)((a.M + PF_TM - 1) / PF_TM) * (a.d_rows / 64);
+    const int grid = steps < n_cu ? (int)steps : n_cu;
+    constexpr int LDS = PfSlab<BITS>::LDS_BYTES;
+    static FmLdsAttr attr;
+    if (!fm_dyn_lds_ready(attr, (const void *)fm_pf_gemm<PF_DENSE, BITS, FP16>, LDS)) return FM_ERR_HIP;
+    for (int pass = 0; pass < a.d_cols / 2048; pass++) {
+        a.d_pass = pass;
+        hipLaunchKernelGGL((fm_pf_gemm<PF_DENSE, BITS, FP16>), dim3(grid), dim3(512), LDS, st, a);
+    }
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
+
+bool pf_dense_supported(int out_dim, int in_dim, int group_size, int bits) {
+    // eight slabs of four groups per column pass, two 32-row tiles per step
+    return (bits == 3 || bits == 4) && group_size == 64 && in_dim >= 2048 && in_dim % 2048 == 0 &&
+           in_dim <= 16384 && out_dim >= 64 && out_dim % 64 == 0;
+}
+
 }  // namespace
+
+// Dense tensor against M positions on the same matrix-core kernel as the expert products
+// (gpu_encode_prefill_matvec, finchmoe/infer.m:3672: the reference runs M matvecs).
+extern "C" size_t fm_prefill_dense_ws_bytes(int out_dim, int in_dim, int group_size, int bits, int M) {
+    if (!pf_dense_supported(out_dim, in_dim, group_size, bits) || M < 1) return 0;
+    return align256(((size_t)M / PF_TM + 1) * sizeof(PfItem)) + 256 +
+           align256((size_t)M * (in_dim / 64) * 16 * sizeof(uint4)) +
+           align256((size_t)M * (in_dim / 64) * sizeof(float2));
+}
+
+extern "C" int fm_launch_prefill_dense(const void *d_W, const void *d_S, const void *d_B, int out_dim,
+                                       int in_dim, int group_size, int bits, int scale_fp16,
+                                       const float *d_X, int M, float *d_out, void *d_ws,
+                                       size_t ws_bytes, int flags, int n_cu, hipStream_t st) {
+    const size_t need = fm_prefill_dense_ws_bytes(out_dim, in_dim, group_size, bits, M);
+    if (need == 0) return FM_ERR_UNSUPPORTED;
+    if (ws_bytes < need) return FM_ERR_ARG;
+    char *ws = (char *)d_ws;
+    PfArgs a{};
+    a.X = d_X;
+    a.M = M;
+    a.K = 1;
+    a.items = (PfItem *)ws;               ws += align256(((size_t)M / PF_TM + 1) * sizeof(PfItem));
+    a.n_items = (int *)ws;                ws += 256;
+    a.xop = (uint4 *)ws;                  ws += align256((size_t)M * (in_dim / 64) * 16 * sizeof(uint4));
+    a.xsums = (float2 *)ws;
+    a.d_w = (const uint8_t *)d_W;
+    a.d_s = (const uint8_t *)d_S - (const uint8_t *)d_W;
+    a.d_b = (const uint8_t *)d_B - (const uint8_t *)d_W;
+    a.d_rows = out_dim;
+    a.d_cols = in_dim;
+    a.d_pass = 0;
+    a.d_flags = flags;
+    a.d_out = d_out;
+    if (scale_fp16)
+        return bits == 3 ? pf_launch_dense<3, true>(a, n_cu, st) : pf_launch_dense<4, true>(a, n_cu, st);
+    return bits == 3 ? pf_launch_dense<3, false>(a, n_cu, st) : pf_launch_dense<4, false>(a, n_cu, st);
+}
 
 extern "C" size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K) {
     if (!pf_supported(g)) return 0;

@@ -168,7 +168,12 @@ FM_API int fm_matvec_batch_dev(fm_ctx *ctx, const fm_tensor *tensors, int n, con
                         float *const *d_outs);
 FM_API int fm_matvec_batch(fm_ctx *ctx, const fm_tensor *tensors, int n, const float *x,
                     float *const *outs);
-/* M positions: X[M][in_dim] -> out[M][out_dim] */
+/* M positions: X[M][in_dim] -> out[M][out_dim] (gpu_encode_prefill_matvec,
+ * finchmoe/infer.m:3672).  Fewer than 16 positions (and shapes the matrix-core kernel does
+ * not cover) run one GEMV per position, bitwise equal to the one-position call; from 16
+ * positions on a 3-/4-bit tensor with in_dim a multiple of 2048 and out_dim a multiple of 64
+ * is multiplied on the matrix cores (equal to the one-position call within the parity bar;
+ * d_X must be 16-byte aligned for it). */
 FM_API int fm_matvec_prefill_dev(fm_ctx *ctx, fm_tensor t, const float *d_X, float *d_out, int M);
 FM_API int fm_matvec_prefill(fm_ctx *ctx, fm_tensor t, const float *X, float *out, int M);
 

@@ -140,3 +140,29 @@ def test_embedding_lookup_is_the_dequantized_row(hip, orc, bits, dtype):
             assert np.array_equal(out[i].view(np.uint32), want.view(np.uint32)), (i, tok)
     finally:
         hip.tensor_release(t)
+
+
+@pytest.mark.parametrize("bits,dtype,out_dim,in_dim,M", [
+    (4, "bf16", 512, 2048, 64), (4, "bf16", 256, 4096, 40), (4, "fp16", 128, 2048, 33),
+    (3, "bf16", 192, 2048, 100), (4, "bf16", 64, 8192, 32), (4, "bf16", 128, 2048, 16)])
+def test_dense_prefill_gemm_matches_positions(hip, orc, bits, dtype, out_dim, in_dim, M):
+    """From 16 positions on, a dense 3-/4-bit tensor with in_dim a multiple of 2048 runs on the
+    matrix cores (one column pass per 2048 columns): every position against the oracle's GEMV and
+    against the one-position call."""
+    rng = np.random.default_rng(out_dim + in_dim + M)
+    t, (codes, W, S, B, sd) = _tensor(hip, rng, out_dim, in_dim, bits, dtype)
+    try:
+        X = rng.standard_normal((M, in_dim)).astype(np.float32)
+        X[3] *= 1e-3
+        X[5] *= 300.0
+        out = hip.matvec_prefill(t, X, out_dim)
+        assert out.shape == (M, out_dim) and np.isfinite(out).all()
+        for m in range(M):
+            (single,) = hip.matvec_batch([t], X[m], [out_dim])
+            assert_parity(out[m], single, "position %d vs one-position call" % m)
+        for m in (0, 3, 5, M - 1):
+            ref = orc.dequant_matvec(W, S, B, X[m], out_dim, in_dim, bits, scale_dtype=sd, nthreads=8)
+            assert_parity(out[m], ref, "position %d vs oracle" % m)
+        assert np.array_equal(hip.matvec_prefill(t, X, out_dim), out)
+    finally:
+        hip.tensor_release(t)
