@@ -94,6 +94,7 @@ def load():
         "fm_dequant_tensor": (i, [vp, i, vp, vp, vp]),
         "fm_gguf_dequant_expert": (i, [vp, i, i, i, vp]),
         "fm_embed_lookup_dev": (i, [vp, i, vp, i, vp]),
+        "fm_matvec_prefill_batch_dev": (i, [vp, vp, i, vp, vp, i]),
         "fm_embed_lookup": (i, [vp, i, i, vp]),
     }
     for name, (res, args) in sig.items():
@@ -258,6 +259,12 @@ class FinchHip:
 
     def matvec_prefill_dev(self, t, d_X, d_out, M):
         self._chk(self.L.fm_matvec_prefill_dev(self.h, t, d_X, d_out, M))
+
+    def matvec_prefill_batch_dev(self, tensors, d_X, d_outs, M):
+        n = len(tensors)
+        ts = (C.c_int * n)(*tensors)
+        outs = (C.c_void_p * n)(*d_outs)
+        self._chk(self.L.fm_matvec_prefill_batch_dev(self.h, ts, n, d_X, outs, M))
 
     # ---- GGUF
     def route_topk_dev(self, d_logits, n_experts, K, d_seg_score, d_idx, d_w, d_params=None):

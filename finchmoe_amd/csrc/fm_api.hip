@@ -749,36 +749,58 @@ extern "C" size_t fm_prefill_dense_ws_bytes(int out_dim, int in_dim, int group_s
 extern "C" int fm_launch_prefill_dense(const void *d_W, const void *d_S, const void *d_B, int out_dim,
                                        int in_dim, int group_size, int bits, int scale_fp16,
                                        const float *d_X, int M, float *d_out, void *d_ws,
-                                       size_t ws_bytes, int flags, int n_cu, hipStream_t st);
+                                       size_t ws_bytes, int flags, int prepare, int n_cu,
+                                       hipStream_t st);
 
 // positions from which the dense product runs on the matrix cores (below: one GEMV per position)
 #define FM_DENSE_GEMM_MIN_M 16
 
-extern "C" int fm_matvec_prefill_dev(fm_ctx *c, fm_tensor t, const float *d_X, float *d_out,
-                                     int M) {
+// n tensors against the same M positions.  Tensors the matrix-core kernel covers share one
+// pass that turns X into operand registers (per code width); the others run one GEMV per position.
+extern "C" int fm_matvec_prefill_batch_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_X,
+                                           float *const *d_outs, int M) {
     if (!c) return FM_ERR_ARG;
+    if (!ts || !d_X || !d_outs) return fail(c, FM_ERR_ARG, "null pointer");
+    if (n < 1 || n > 64) return fail(c, FM_ERR_ARG, "n %d outside 1..64", n);
     if (M < 1 || M > 65535) return fail(c, FM_ERR_ARG, "M %d outside 1..65535", M);
-    Tensor *p = get_tensor(c, t);
-    if (p && d_X && d_out && M >= FM_DENSE_GEMM_MIN_M && ((uintptr_t)d_X & 15) == 0 &&
-        ((uintptr_t)d_out & 3) == 0) {
-        static const bool no_gemm = getenv("FINCH_DENSE_NO_GEMM") != nullptr;
-        const size_t ws = no_gemm ? 0 : fm_prefill_dense_ws_bytes(p->out_dim, p->in_dim, p->group_size,
-                                                                  p->bits, M);
+    static const bool no_gemm = getenv("FINCH_DENSE_NO_GEMM") != nullptr;
+    int prepared_bits = 0, prepared_in = 0;
+    for (int i = 0; i < n; i++) {
+        Tensor *p = get_tensor(c, ts[i]);
+        if (!p) return fail(c, FM_ERR_ARG, "bad tensor handle %d", ts[i]);
+        if (!d_outs[i]) return fail(c, FM_ERR_ARG, "null output %d", i);
+        size_t ws = 0;
+        if (!no_gemm && M >= FM_DENSE_GEMM_MIN_M && ((uintptr_t)d_X & 15) == 0 && ((uintptr_t)d_outs[i] & 3) == 0)
+            ws = fm_prefill_dense_ws_bytes(p->out_dim, p->in_dim, p->group_size, p->bits, M);
         if (ws) {
             DeviceGuard dg(c->device);
+            // (growing the workspace drops what was prepared in it)
+            if (c->ws_bytes < ws) prepared_bits = 0;
             int rc = ensure_ws(c, ws);
             if (rc) return rc;
+            const int prepare = !(prepared_bits == p->bits && prepared_in == p->in_dim);
             rc = fm_launch_prefill_dense(p->W, p->S, p->B, p->out_dim, p->in_dim, p->group_size,
-                                         p->bits, p->scale_fp16, d_X, M, d_out, c->d_ws, c->ws_bytes,
-                                         0, c->n_cu, c->stream);
-            if (rc != FM_ERR_UNSUPPORTED) {
-                if (rc) return fail(c, rc, "dense prefill launch failed: %s", hipGetErrorString(hipGetLastError()));
-                return FM_OK;
+                                         p->bits, p->scale_fp16, d_X, M, d_outs[i], c->d_ws, c->ws_bytes,
+                                         0, prepare, c->n_cu, c->stream);
+            if (rc == FM_OK) {
+                prepared_bits = p->bits;
+                prepared_in = p->in_dim;
+                continue;
             }
+            if (rc != FM_ERR_UNSUPPORTED)
+                return fail(c, rc, "dense prefill launch failed: %s", hipGetErrorString(hipGetLastError()));
         }
+        float *outs[1] = {d_outs[i]};
+        int rc = matvec_dev(c, &ts[i], 1, d_X, outs, M);
+        if (rc) return rc;
     }
+    return FM_OK;
+}
+
+extern "C" int fm_matvec_prefill_dev(fm_ctx *c, fm_tensor t, const float *d_X, float *d_out,
+                                     int M) {
     float *outs[1] = {d_out};
-    return matvec_dev(c, &t, 1, d_X, outs, M);
+    return fm_matvec_prefill_batch_dev(c, &t, 1, d_X, outs, M);
 }
 
 static int matvec_host(fm_ctx *c, const fm_tensor *ts, int n, const float *x, float *const *outs,
@@ -803,7 +825,9 @@ static int matvec_host(fm_ctx *c, const fm_tensor *ts, int n, const float *x, fl
     HIPCHK(c, hipMemcpyAsync(st, x, nx, hipMemcpyHostToDevice, c->stream));
     std::vector<float *> d_outs(n);
     for (int i = 0; i < n; i++) d_outs[i] = (float *)(st + offs[i]);
-    rc = matvec_dev(c, ts, n, (const float *)st, d_outs.data(), M);
+    // (M positions: the same path as the device-pointer entry, matrix cores from 16 positions on)
+    rc = M > 1 ? fm_matvec_prefill_batch_dev(c, ts, n, (const float *)st, d_outs.data(), M)
+               : matvec_dev(c, ts, n, (const float *)st, d_outs.data(), M);
     if (rc) return rc;
     for (int i = 0; i < n; i++)
         HIPCHK(c, hipMemcpyAsync(outs[i], d_outs[i], (size_t)M * get_tensor(c, ts[i])->out_dim * 4,

@@ -846,9 +846,10 @@ int pf_launch(const PfArgs &a, const FmExpertGeom *g, int M, float *d_out, int f
 }
 
 template <int BITS, bool FP16>
-int pf_launch_dense(PfArgs a, int n_cu, hipStream_t st) {
+int pf_launch_dense(PfArgs a, int n_cu, bool prepare, hipStream_t st) {
     const int prep_tasks = a.M * (a.d_cols / 64) * 2;
-    hipLaunchKernelGGL(fm_pf_dense_prep<BITS>, dim3(1 + (prep_tasks + 1023) / 1024), dim3(1024), 0, st, a);
+    if (prepare)
+        hipLaunchKernelGGL(fm_pf_dense_prep<BITS>, dim3(1 + (prep_tasks + 1023) / 1024), dim3(1024), 0, st, a);
     const long steps = (long)((a.M + PF_TM - 1) / PF_TM) * (a.d_rows / 64);
     const int grid = steps < n_cu ? (int)steps : n_cu;
     constexpr int LDS = PfSlab<BITS>::LDS_BYTES;
@@ -881,7 +882,8 @@ extern "C" size_t fm_prefill_dense_ws_bytes(int out_dim, int in_dim, int group_s
 extern "C" int fm_launch_prefill_dense(const void *d_W, const void *d_S, const void *d_B, int out_dim,
                                        int in_dim, int group_size, int bits, int scale_fp16,
                                        const float *d_X, int M, float *d_out, void *d_ws,
-                                       size_t ws_bytes, int flags, int n_cu, hipStream_t st) {
+                                       size_t ws_bytes, int flags, int prepare, int n_cu,
+                                       hipStream_t st) {
     const size_t need = fm_prefill_dense_ws_bytes(out_dim, in_dim, group_size, bits, M);
     if (need == 0) return FM_ERR_UNSUPPORTED;
     if (ws_bytes < need) return FM_ERR_ARG;
@@ -902,9 +904,12 @@ extern "C" int fm_launch_prefill_dense(const void *d_W, const void *d_S, const v
     a.d_pass = 0;
     a.d_flags = flags;
     a.d_out = d_out;
+    // prepare = 0: the workspace holds X's operand form from the call before (same X, M, in_dim
+    // and code width: the pairing of the codes depends on the width)
+    const bool prep = prepare != 0;
     if (scale_fp16)
-        return bits == 3 ? pf_launch_dense<3, true>(a, n_cu, st) : pf_launch_dense<4, true>(a, n_cu, st);
-    return bits == 3 ? pf_launch_dense<3, false>(a, n_cu, st) : pf_launch_dense<4, false>(a, n_cu, st);
+        return bits == 3 ? pf_launch_dense<3, true>(a, n_cu, prep, st) : pf_launch_dense<4, true>(a, n_cu, prep, st);
+    return bits == 3 ? pf_launch_dense<3, false>(a, n_cu, prep, st) : pf_launch_dense<4, false>(a, n_cu, prep, st);
 }
 
 extern "C" size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K) {

@@ -175,6 +175,10 @@ FM_API int fm_matvec_batch(fm_ctx *ctx, const fm_tensor *tensors, int n, const f
  * is multiplied on the matrix cores (equal to the one-position call within the parity bar;
  * d_X must be 16-byte aligned for it). */
 FM_API int fm_matvec_prefill_dev(fm_ctx *ctx, fm_tensor t, const float *d_X, float *d_out, int M);
+/* n tensors against the same X[M][in_dim] (each tensor as fm_matvec_prefill_dev; tensors the
+ * matrix-core kernel covers share one preparation of X) */
+FM_API int fm_matvec_prefill_batch_dev(fm_ctx *ctx, const fm_tensor *tensors, int n, const float *d_X,
+                                float *const *d_outs, int M);
 FM_API int fm_matvec_prefill(fm_ctx *ctx, fm_tensor t, const float *X, float *out, int M);
 
 /* ---------------------------------------------------------------- routing

@@ -166,3 +166,27 @@ def test_dense_prefill_gemm_matches_positions(hip, orc, bits, dtype, out_dim, in
         assert np.array_equal(hip.matvec_prefill(t, X, out_dim), out)
     finally:
         hip.tensor_release(t)
+
+
+def test_dense_prefill_batch_shares_the_prepared_input(hip, orc):
+    """Two tensors of the same width (and a third of another) against the same positions in one
+    call equal the single-tensor calls bit for bit."""
+    import torch
+    rng = np.random.default_rng(77)
+    M = 48
+    ta, _ = _tensor(hip, rng, 256, 2048, 4)
+    tb, _ = _tensor(hip, rng, 128, 2048, 4)
+    tc, _ = _tensor(hip, rng, 64, 2048, 3)
+    td, _ = _tensor(hip, rng, 96, 2048, 8)          # no matrix-core form: one GEMV per position
+    try:
+        X = rng.standard_normal((M, 2048)).astype(np.float32)
+        d_X = torch.from_numpy(X).cuda()
+        dims = (256, 128, 64, 96)
+        outs = [torch.zeros(M, d, device="cuda") for d in dims]
+        hip.matvec_prefill_batch_dev([ta, tb, tc, td], d_X.data_ptr(), [o.data_ptr() for o in outs], M)
+        hip.sync()
+        for t, d, o in zip((ta, tb, tc, td), dims, outs):
+            assert np.array_equal(o.cpu().numpy(), hip.matvec_prefill(t, X, d)), d
+    finally:
+        for t in (ta, tb, tc, td):
+            hip.tensor_release(t)
