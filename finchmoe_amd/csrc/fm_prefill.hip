@@ -73,7 +73,7 @@ struct PfArgs {
     float *d_out;
 };
 
-enum { PF_GATE_UP = 0, PF_DOWN = 1, PF_DENSE = 2 };
+enum { PF_GATE_UP = 0, PF_DOWN = 1, PF_DENSE = 2, PF_DENSE_TEAMS = 3 };
 
 // ---- pairing of the 32 codes a lane holds for one group -------------------
 // Pair p fills k slots 2p (low half of the register, code lo(p) at mantissa bit tl(p)) and
@@ -350,11 +350,17 @@ __device__ __forceinline__ uint4 pf_side_b(uint32_t w0, uint32_t w1, int hh, uin
 // MODE PF_DENSE: one dense tensor against M positions, 2048 of its columns per launch (eight slabs
 //   as in gate/up; column pass d_pass adds to what the passes before it stored); an item is a
 //   block of 16 positions, a step = two row tiles (64 rows), the operand comes from xop.
+// MODE PF_DENSE_TEAMS: a dense tensor of 512 columns: the slabs and teams of PF_DOWN (a step =
+//   256 rows), operand and output as in PF_DENSE.
 template <int MODE, int BITS, bool FP16>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fm_pf_gemm(PfArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // (the host pass cannot allocate the registers of the asm blocks)
     using P = PfSlab<BITS>;
     constexpr int DW = PfCode<BITS>::DW;
+    // TEAMS: geometry of the down product; DTENSOR: operands of a dense tensor; DENSE / DOWN: the
+    // two pure forms
+    constexpr bool TEAMS = MODE == PF_DOWN || MODE == PF_DENSE_TEAMS;
+    constexpr bool DTENSOR = MODE == PF_DENSE || MODE == PF_DENSE_TEAMS;
     constexpr bool DOWN = MODE == PF_DOWN, DENSE = MODE == PF_DENSE;
     constexpr int GPW = P::GPW;
     constexpr int RING = P::RING;
@@ -366,23 +372,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint32_t ring0 = lds0 + (uint32_t)wave * (RING * P::SLOT);
     const uint32_t red0 = lds0 + 8 * RING * P::SLOT;
     const int n_items = *a.n_items;
-    const int in_dim = DENSE ? a.d_cols : DOWN ? a.g.inter : a.g.hidden;
+    const int in_dim = DTENSOR ? a.d_cols : DOWN ? a.g.inter : a.g.hidden;
     const int row_bytes = in_dim * BITS / 8, sb_bytes = (in_dim / 64) * 2;
-    const int slab = DENSE ? wave + 8 * a.d_pass : DOWN ? (wave & 1) : wave, team = DOWN ? (wave >> 1) : 0;
-    const int n_steps = DENSE ? a.d_rows / 64 : DOWN ? a.g.hidden / 256 : a.g.inter / 32;
+    const int slab = DENSE ? wave + 8 * a.d_pass : TEAMS ? (wave & 1) : wave, team = TEAMS ? (wave >> 1) : 0;
+    const int n_steps = DENSE ? a.d_rows / 64 : DTENSOR ? a.d_rows / 256 : DOWN ? a.g.hidden / 256 : a.g.inter / 32;
     const uint32_t ones = fm_opaque(0x3F803F80u);
     // region offsets of the first tile-matrix of a step (this team's), the distance to the
     // second one, rows per step
     // (byte offsets from the blob's — the dense tensor's W — first byte, modulo 2^64)
-    const size_t w_off0 = DENSE ? 0 : DOWN ? a.g.down_w + 64u * team * row_bytes : a.g.gate_w;
-    const size_t s_off0 = DENSE ? (size_t)a.d_s : DOWN ? a.g.down_s + 64u * team * sb_bytes : a.g.gate_s;
-    const size_t b_off0 = DENSE ? (size_t)a.d_b : DOWN ? a.g.down_b + 64u * team * sb_bytes : a.g.gate_b;
-    const uint32_t w_d = DOWN || DENSE ? 32u * row_bytes : a.g.up_w - a.g.gate_w;
-    const uint32_t s_d = DOWN || DENSE ? 32u * sb_bytes : a.g.up_s - a.g.gate_s;
-    const uint32_t b_d = DOWN || DENSE ? 32u * sb_bytes : a.g.up_b - a.g.gate_b;
-    const uint32_t step_rows = DENSE ? 64u : DOWN ? 256u : 32u;
-    const uint8_t *store = DENSE ? a.d_w : a.layer;          // what an item's "expert" indexes into
-    const size_t expert_size = DENSE ? 0 : a.g.expert_size;
+    const size_t team_w = 64u * team * row_bytes, team_sb = 64u * team * sb_bytes;
+    const size_t w_off0 = DTENSOR ? team_w : DOWN ? a.g.down_w + team_w : a.g.gate_w;
+    const size_t s_off0 = DTENSOR ? (size_t)a.d_s + team_sb : DOWN ? a.g.down_s + team_sb : a.g.gate_s;
+    const size_t b_off0 = DTENSOR ? (size_t)a.d_b + team_sb : DOWN ? a.g.down_b + team_sb : a.g.gate_b;
+    const uint32_t w_d = TEAMS || DENSE ? 32u * row_bytes : a.g.up_w - a.g.gate_w;
+    const uint32_t s_d = TEAMS || DENSE ? 32u * sb_bytes : a.g.up_s - a.g.gate_s;
+    const uint32_t b_d = TEAMS || DENSE ? 32u * sb_bytes : a.g.up_b - a.g.gate_b;
+    const uint32_t step_rows = DENSE ? 64u : TEAMS ? 256u : 32u;
+    const uint8_t *store = DTENSOR ? a.d_w : a.layer;        // what an item's "expert" indexes into
+    const size_t expert_size = DTENSOR ? 0 : a.g.expert_size;
     // this lane's pieces of a slot copy
     uint32_t coff[P::NQ];
     bool cvalid[P::NQ];
@@ -473,7 +480,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 const int tok = 8 * (i / 4) + 4 * hh + (i % 4);
                 if (tok < item_next.count) out_pairs_next[i] = a.sorted[item_next.start + tok];
             }
-        } else if constexpr (!DENSE) {
+        } else if constexpr (!DTENSOR) {
             if ((n & 15) < item_next.count) pair_next = a.sorted[item_next.start + (n & 15)];
         }
     }
@@ -500,7 +507,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 // X was turned into operand registers once per chunk (pf_prepare): lane (m, hh)
                 // takes the hi (m < 16) or lo registers of its position, its groups, its half
                 const int piece = n < 16 ? 0 : 1;
-                const size_t m = !on ? 0 : DOWN || DENSE ? (size_t)(item.start + pos) : (size_t)(pair_next / a.K);
+                const size_t m = !on ? 0 : DOWN || DTENSOR ? (size_t)(item.start + pos) : (size_t)(pair_next / a.K);
                 const int ng = in_dim / 64;
                 const uint4 *src = (DOWN ? a.aop : a.xop) + (m * ng + GPW * slab) * 16 + 2 * hh + piece;
                 const float2 *sm = (DOWN ? a.asums : a.xsums) + m * ng + GPW * slab;
@@ -533,7 +540,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                         out_pairs_next[i] = 0;
                         if (more && tok < item_next.count) out_pairs_next[i] = a.sorted[item_next.start + tok];
                     }
-                } else if constexpr (!DENSE) {
+                } else if constexpr (!DTENSOR) {
                     pair_next = 0;
                     if (more && pos < item_next.count) pair_next = a.sorted[item_next.start + pos];
                 }
@@ -686,7 +693,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
             // ---- every wave has written both partial tiles of this step
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            if constexpr (!DOWN) {
+            if constexpr (!TEAMS) {
                 // wave r sums result register r (position my_pos) over the waves, in wave order
                 const uint32_t ar = red0 + (uint32_t)((buf * 2 * 8) * 2048 + wave * 256 + 4 * lane);
                 float p[16];
@@ -743,8 +750,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
                 for (int i = 0; i < 8; i++) {
                     const int tok = 8 * (i / 4) + 4 * hh + (i % 4);
-                    if (tok < item.count)
-                        a.eo[(size_t)out_pairs[i] * a.g.hidden + row] = p[i] + p[8 + i];
+                    if (tok < item.count) {
+                        const float v = p[i] + p[8 + i];
+                        if constexpr (DTENSOR) {
+                            float *o = a.d_out + (size_t)(item.start + tok) * a.d_rows + row;
+                            *o = (a.d_flags & FM_ACCUMULATE) ? *o + v : v;
+                        } else {
+                            a.eo[(size_t)out_pairs[i] * a.g.hidden + row] = v;
+                        }
+                    }
                 }
             }
             buf ^= 1;
@@ -855,6 +869,14 @@ int pf_launch_dense(PfArgs a, int n_cu, bool prepare, hipStream_t st) {
     constexpr int LDS = PfSlab<BITS>::LDS_BYTES;
     static FmLdsAttr attr;
     if (!fm_dyn_lds_ready(attr, (const void *)fm_pf_gemm<PF_DENSE, BITS, FP16>, LDS)) return FM_ERR_HIP;
+    if (a.d_cols == 512) {       // two slabs: the teams of the down product, 256 rows per step
+        const long tsteps = (long)((a.M + PF_TM - 1) / PF_TM) * (a.d_rows / 256);
+        const int tgrid = tsteps < n_cu ? (int)tsteps : n_cu;
+        static FmLdsAttr attr_t;
+        if (!fm_dyn_lds_ready(attr_t, (const void *)fm_pf_gemm<PF_DENSE_TEAMS, BITS, FP16>, LDS)) return FM_ERR_HIP;
+        hipLaunchKernelGGL((fm_pf_gemm<PF_DENSE_TEAMS, BITS, FP16>), dim3(tgrid), dim3(512), LDS, st, a);
+        return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+    }
     for (int pass = 0; pass < a.d_cols / 2048; pass++) {
         a.d_pass = pass;
         hipLaunchKernelGGL((fm_pf_gemm<PF_DENSE, BITS, FP16>), dim3(grid), dim3(512), LDS, st, a);
@@ -863,9 +885,11 @@ int pf_launch_dense(PfArgs a, int n_cu, bool prepare, hipStream_t st) {
 }
 
 bool pf_dense_supported(int out_dim, int in_dim, int group_size, int bits) {
+    if (!(bits == 3 || bits == 4) || group_size != 64) return false;
+    // 512 columns: two slabs, four teams on 64 rows each
+    if (in_dim == 512) return out_dim >= 256 && out_dim % 256 == 0;
     // eight slabs of four groups per column pass, two 32-row tiles per step
-    return (bits == 3 || bits == 4) && group_size == 64 && in_dim >= 2048 && in_dim % 2048 == 0 &&
-           in_dim <= 16384 && out_dim >= 64 && out_dim % 64 == 0;
+    return in_dim >= 2048 && in_dim % 2048 == 0 && in_dim <= 16384 && out_dim >= 64 && out_dim % 64 == 0;
 }
 
 }  // namespace

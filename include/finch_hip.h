@@ -171,8 +171,8 @@ FM_API int fm_matvec_batch(fm_ctx *ctx, const fm_tensor *tensors, int n, const f
 /* M positions: X[M][in_dim] -> out[M][out_dim] (gpu_encode_prefill_matvec,
  * finchmoe/infer.m:3672).  Fewer than 16 positions (and shapes the matrix-core kernel does
  * not cover) run one GEMV per position, bitwise equal to the one-position call; from 16
- * positions on a 3-/4-bit tensor with in_dim a multiple of 2048 and out_dim a multiple of 64
- * is multiplied on the matrix cores (equal to the one-position call within the parity bar;
+ * positions on a 3-/4-bit tensor with in_dim a multiple of 2048 and out_dim a multiple of 64,
+ * or in_dim 512 and out_dim a multiple of 256, is multiplied on the matrix cores (equal to the one-position call within the parity bar;
  * d_X must be 16-byte aligned for it). */
 FM_API int fm_matvec_prefill_dev(fm_ctx *ctx, fm_tensor t, const float *d_X, float *d_out, int M);
 /* n tensors against the same X[M][in_dim] (each tensor as fm_matvec_prefill_dev; tensors the

@@ -144,10 +144,11 @@ def test_embedding_lookup_is_the_dequantized_row(hip, orc, bits, dtype):
 
 @pytest.mark.parametrize("bits,dtype,out_dim,in_dim,M", [
     (4, "bf16", 512, 2048, 64), (4, "bf16", 256, 4096, 40), (4, "fp16", 128, 2048, 33),
-    (3, "bf16", 192, 2048, 100), (4, "bf16", 64, 8192, 32), (4, "bf16", 128, 2048, 16)])
+    (3, "bf16", 192, 2048, 100), (4, "bf16", 64, 8192, 32), (4, "bf16", 128, 2048, 16),
+    (4, "bf16", 2048, 512, 40), (3, "fp16", 512, 512, 33)])
 def test_dense_prefill_gemm_matches_positions(hip, orc, bits, dtype, out_dim, in_dim, M):
-    """From 16 positions on, a dense 3-/4-bit tensor with in_dim a multiple of 2048 runs on the
-    matrix cores (one column pass per 2048 columns): every position against the oracle's GEMV and
+    """From 16 positions on, a dense 3-/4-bit tensor with in_dim 512 or a multiple of 2048 runs on
+    the matrix cores (one column pass per 2048 columns): every position against the oracle's GEMV and
     against the one-position call."""
     rng = np.random.default_rng(out_dim + in_dim + M)
     t, (codes, W, S, B, sd) = _tensor(hip, rng, out_dim, in_dim, bits, dtype)
