@@ -341,6 +341,18 @@ static void matvec_rows(const void *W, const uint16_t *S, const uint16_t *B,
                          bits == 10 ? ORC_GGML_Q4_K : ORC_GGML_Q6_K);
         return;
     }
+    /* infer.m:1689-1701 — scales == NULL (or biases == NULL) means an unquantized BF16
+     * weight [out_dim][in_dim]; checked after the GGUF types, as upstream */
+    if (!S || !B) {
+        const uint16_t *wb = (const uint16_t *)W;
+        for (int r = r0; r < r1; r++) {
+            const uint16_t *wr = wb + (size_t)r * in_dim;
+            float acc = 0.0f;
+            for (int i = 0; i < in_dim; i++) acc += orc_bf16_to_f32(wr[i]) * x[i];
+            out[r] = acc;
+        }
+        return;
+    }
     int ng = in_dim / group_size;
     if (bits == 3) {
         int trip = in_dim / 8, tpg = group_size / 8;

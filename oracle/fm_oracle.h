@@ -12,6 +12,11 @@
  * for timing purposes as well.
  *
  * Parity pins (what each function is checked against, see tests/test_oracle_*):
+ *   every function below that has a twin in infer.m:686-702, 1575-1881 (widening,
+ *   get_scale_min_k4, gguf_dequant_row, cpu_dequant_matvec at bits 3/4/8/10/11 and raw
+ *   BF16, RMS norm, SwiGLU, softmax, top-K, normalise, vec_madd) is compared BIT FOR BIT
+ *   with the reference's own C text compiled by build_ref.sh (oracle/_ref/libfm_ref.so,
+ *   tests/test_oracle_ref.py).  Independently of that build:
  *   bf16/fp16 widening        exhaustive 65,536 values vs numpy
  *   3-bit / u32 packing       exhaustive 2^24 triplets pack<->unpack; closed form
  *   affine dequant            exactly-rounded closed form vs float64
@@ -87,7 +92,8 @@ void orc_gguf_dequant_row(const void *row, float *y, int n, int ggml_type);
 float orc_gguf_block_value_wordform(const uint8_t *block, int e, int ggml_type);
 size_t orc_gguf_row_bytes(int in_dim, int ggml_type);
 
-/* matvec (infer.m:1660-1763).  bits in {1,2,3,4,8}: affine; 10/11: Q4_K/Q6_K */
+/* matvec (infer.m:1660-1763).  bits in {1,2,3,4,8}: affine; 10/11: Q4_K/Q6_K;
+ * S == NULL or B == NULL (and bits not 10/11): W is raw BF16 [out_dim][in_dim] */
 void orc_dequant_matvec(const void *W, const uint16_t *S, const uint16_t *B,
                         const float *x, float *out, int out_dim, int in_dim,
                         int group_size, int bits, int scale_dtype);

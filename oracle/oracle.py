@@ -77,6 +77,41 @@ def lib():
     return _LIB
 
 
+_REF = None
+
+
+def ref_lib():
+    """oracle/_ref/libfm_ref.so: the reference's own CPU functions (finchmoe/infer.m:686-702,
+    1575-1881) compiled by build_ref.sh.  None when it has not been built (the reference tree
+    is not mounted and no prebuilt copy travelled with the tree)."""
+    global _REF
+    if _REF is None:
+        path = os.path.join(_HERE, "_ref", "libfm_ref.so")
+        if not os.path.exists(path):
+            return None
+        R = C.CDLL(path)
+        vp, i, f = C.c_void_p, C.c_int, C.c_float
+        R.ref_bf16_to_f32.restype = f
+        R.ref_bf16_to_f32.argtypes = [C.c_uint16]
+        R.ref_f32_to_bf16.restype = C.c_uint16
+        R.ref_f32_to_bf16.argtypes = [f]
+        R.ref_fp16_to_f32.restype = f
+        R.ref_fp16_to_f32.argtypes = [C.c_uint16]
+        R.ref_get_scale_min_k4.argtypes = [i, vp, vp, vp]
+        R.ref_gguf_dequant_row.argtypes = [vp, vp, i, i]
+        R.ref_cpu_dequant_matvec.argtypes = [vp, vp, vp, vp, vp, i, i, i, i]
+        R.ref_cpu_rms_norm.argtypes = [vp, vp, vp, i, f]
+        R.ref_cpu_swiglu.argtypes = [vp, vp, vp, i]
+        R.ref_cpu_sigmoid.restype = f
+        R.ref_cpu_sigmoid.argtypes = [f]
+        R.ref_cpu_softmax.argtypes = [vp, i]
+        R.ref_cpu_topk.argtypes = [vp, i, i, vp, vp]
+        R.ref_cpu_normalize_weights.argtypes = [vp, i]
+        R.ref_cpu_vec_madd.argtypes = [vp, vp, f, i]
+        _REF = R
+    return _REF
+
+
 def _p(a):
     return None if a is None else a.ctypes.data
 
