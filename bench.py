@@ -29,9 +29,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 peak
 # HBM bytes per launch of the fused decode kernel on the default workload, from rocprofv3
-# --pmc FETCH_SIZE (x2: calibrated against a 1 GiB copy) + WRITE_SIZE, see
-# profiles/decode_step_3bit_hbm_traffic.md.  Offline measurement; null for other sizes.
+# --pmc FETCH_SIZE (x2: calibrated against a 1 GiB copy) + WRITE_SIZE.  An OFFLINE constant
+# (hardware counters cannot be read from inside this process): the JSON line names the file
+# it comes from in roofline.traffic_source, and it is null for any other size.
 FUSED_TRAFFIC_BYTES_40L = int((218295.98 * 2 + 4186.4) * 1024)
+FUSED_TRAFFIC_SOURCE = "offline constant from profiles/decode_step_3bit_hbm_traffic.md (rocprofv3 --pmc), not measured in this run"
 
 H, I, E, K, L = 2048, 512, 256, 8, 40
 
@@ -222,6 +224,7 @@ def run_decode_step(args):
                      "achieved": round(bytes_step / (op_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(bytes_step / (op_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                      "traffic": FUSED_TRAFFIC_BYTES_40L if (n_layers, E, K, bits) == (40, 256, 8, 3) else None,
+                     "traffic_source": FUSED_TRAFFIC_SOURCE if (n_layers, E, K, bits) == (40, 256, 8, 3) else None,
                      "bytes_per_launch": bytes_step, "us_per_launch": round(op_us, 2)},
         # the same work as three separate kernels (isolated launches, so a little slower
         # than back to back): where the time goes
@@ -602,7 +605,7 @@ def run_gguf(args):
         u = slab(E * I * (H // 256), 144, 0, 2)
         d = slab(E * H * (I // 256), 210, 208, 1)
         keep.extend([g, u, d])
-        ctx.gguf_adopt_layer(l, g.data_ptr(), u.data_ptr(), d.data_ptr())
+        ctx.gguf_adopt_layer(l, g.data_ptr(), g.numel(), u.data_ptr(), u.numel(), d.data_ptr(), d.numel())
     rng = np.random.default_rng(7)
     tokens = 64
     idx, w = zipf_routing(rng, tokens, n_layers, E, K)
@@ -725,6 +728,31 @@ def run_copy_probe(args):
                    2 * n, ms, args)
 
 
+def run_stream_probe(args):
+    """The streaming ceiling: 2 GiB read once per step by the library's probe kernel (one
+    workgroup of eight waves per CU, LDS-direct 16-byte loads into a ring, contiguous shares,
+    no arithmetic) — what the memory system delivers to a kernel built like the expert kernels."""
+    import torch
+    from finchmoe_amd import FinchHip
+    dev = torch.device("cuda:0")
+    n = 2 << 30
+    bufs = [torch.empty(n, dtype=torch.uint8, device=dev).random_(0, 256) for _ in range(2)]
+    ctx = FinchHip(0)
+    torch.cuda.synchronize()
+
+    def step(t):
+        ctx.stream_probe_dev(bufs[t & 1].data_ptr(), n)
+
+    ms, ev = _timed(ctx, step, args)
+    ctx.close()
+    res = {"event_ms_per_step": round(ev, 5),
+           "roofline": {"bound": "hbm", "kernel": "fm_stream_probe_k", "achieved": round(n / (ev * 1e-3) / 1e9, 1),
+                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(n / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                        "traffic": None, "bytes_per_launch": n, "us_per_launch": round(ev * 1e3, 2)}}
+    return _finish(res, "streaming read GB/s of the probe kernel", "stream probe: 2 GiB read once per step, "
+                   "two buffers alternating (4 GiB > every cache)", n, ms, args)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -755,7 +783,7 @@ def main():
     runners = {"decode_step": run_decode_step, "decode_layer": run_decode_layer, "gdn": run_gdn,
                "gguf": run_gguf, "gguf_chunk": run_gguf, "prefill": run_prefill, "lm_head": run_lm_head, "layer_tail": run_layer_tail,
                "moe_layer": run_moe_layer, "gdn_prefill": run_gdn_prefill,
-               "copy_probe": run_copy_probe}
+               "copy_probe": run_copy_probe, "stream_probe": run_stream_probe}
     if args.workload not in runners:
         print("bench.py: unknown workload %r (have: %s)" % (args.workload, ", ".join(runners)),
               file=sys.stderr)

@@ -63,6 +63,7 @@ def load():
         "fm_kernel_timing": (i, [vp, i]),
         "fm_set_wait_limit": (i, [vp, C.c_uint]),
         "fm_kernel_timing_read": (i, [vp, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i)]),
+        "fm_stream_probe_dev": (i, [vp, vp, sz]),
         "fm_experts_config": (i, [vp, i, i, i, i, i, i, i]),
         "fm_experts_expert_size": (sz, [vp]),
         "fm_experts_upload_layer": (i, [vp, i, vp, sz]),
@@ -82,8 +83,8 @@ def load():
         "fm_route_topk_dev": (i, [vp, vp, i, i, vp, vp, vp, vp]),
         "fm_layer_tail_dev": (i, [vp, i, vp, vp, vp, i, vp, vp, vp, C.c_float, vp, vp]),
         "fm_gguf_config": (i, [vp, i, i, i, i, i, i, i]),
-        "fm_gguf_upload_layer": (i, [vp, i, vp, vp, vp]),
-        "fm_gguf_adopt_layer": (i, [vp, i, vp, vp, vp]),
+        "fm_gguf_upload_layer": (i, [vp, i, vp, sz, vp, sz, vp, sz]),
+        "fm_gguf_adopt_layer": (i, [vp, i, vp, sz, vp, sz, vp, sz]),
         "fm_gguf_moe_decode_dev": (i, [vp, i, vp, vp, vp, i, vp, vp, i]),
         "fm_gguf_moe_decode": (i, [vp, i, vp, vp, vp, i, vp, vp, i]),
         "fm_gguf_moe_decode_step_dev": (i, [vp, i, i, vp, vp, vp, i, vp, vp, i]),
@@ -168,6 +169,9 @@ class FinchHip:
         return a.value, b.value, n.value
 
     # ---- affine expert store
+    def stream_probe_dev(self, d_buf, nbytes):
+        self._chk(self.L.fm_stream_probe_dev(self.h, d_buf, nbytes))
+
     def experts_config(self, n_layers, n_experts, hidden=2048, inter=512, group_size=64, bits=3,
                        scale_dtype=SCALE_BF16):
         self._chk(self.L.fm_experts_config(self.h, n_layers, n_experts, hidden, inter, group_size,
@@ -219,7 +223,9 @@ class FinchHip:
     def tensor_register(self, W, S, B, out_dim, in_dim, bits=4, group_size=64,
                         scale_dtype=SCALE_BF16):
         W = np.ascontiguousarray(W)
-        S, B = _np(S, np.uint16), _np(B, np.uint16)
+        # S = B = None: an unquantized BF16 tensor [out_dim][in_dim] (bits is ignored)
+        S = None if S is None else _np(S, np.uint16)
+        B = None if B is None else _np(B, np.uint16)
         t = C.c_int(-1)
         self._chk(self.L.fm_tensor_register(self.h, _ptr(W), _ptr(S), _ptr(B), out_dim, in_dim,
                                             group_size, bits, scale_dtype, C.byref(t)))
@@ -284,10 +290,12 @@ class FinchHip:
 
     def gguf_upload_layer(self, layer, gate, up, down):
         gate, up, down = (_np(a, np.uint8).reshape(-1) for a in (gate, up, down))
-        self._chk(self.L.fm_gguf_upload_layer(self.h, layer, _ptr(gate), _ptr(up), _ptr(down)))
+        self._chk(self.L.fm_gguf_upload_layer(self.h, layer, _ptr(gate), gate.size, _ptr(up), up.size,
+                                              _ptr(down), down.size))
 
-    def gguf_adopt_layer(self, layer, d_gate, d_up, d_down):
-        self._chk(self.L.fm_gguf_adopt_layer(self.h, layer, d_gate, d_up, d_down))
+    def gguf_adopt_layer(self, layer, d_gate, gate_bytes, d_up, up_bytes, d_down, down_bytes):
+        self._chk(self.L.fm_gguf_adopt_layer(self.h, layer, d_gate, gate_bytes, d_up, up_bytes,
+                                             d_down, down_bytes))
 
     def gguf_moe_decode(self, layer, x, idx, w, flags=0, out=None, want_expert_out=True):
         x, idx, w = _np(x, np.float32), _np(idx, np.int32), _np(w, np.float32)

@@ -12,7 +12,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libfinchhip.so")
 HOSTLIB = os.path.join(HERE, "libfinchops.so")
 SOURCES = ["fm_api.hip", "fm_decode.hip", "fm_dense.hip", "fm_dequant.hip", "fm_gguf.hip",
-           "fm_prefill.hip", "fm_tail.hip", "fm_route.hip"]
+           "fm_prefill.hip", "fm_tail.hip", "fm_route.hip", "fm_probe.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops off: v_pk_*_f32 forms are not trusted on the target pool
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

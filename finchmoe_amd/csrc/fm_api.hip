@@ -27,6 +27,10 @@ int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs, const FmExpertGe
 int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
                     const float *d_x, int M, int n_cu, hipStream_t st);
 int fm_launch_dequant_affine(const void *W, const void *S, const void *B, int out_dim,
+int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim, const float *d_x, int M,
+                         hipStream_t st);
+int fm_launch_stream_probe(const void *d_buf, size_t nbytes, unsigned int *d_sink, int n_cu,
+                           hipStream_t st);
                              int in_dim, int group_size, int bits, int scale_fp16,
                              uint8_t *codes, float *w32, uint16_t *w16, hipStream_t st);
 int fm_launch_dequant_gguf(const void *W, int out_dim, int in_dim, int ggml_type, float *w32,
@@ -47,6 +51,10 @@ size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K);
 int fm_launch_layer_tail(const FmTailArgs *a, int bits, int scale_fp16, hipStream_t st);
 int fm_launch_route(const float *d_logits, int n, int K, const float *d_seg_score, int32_t *d_idx,
                     float *d_w, float *d_params, hipStream_t st);
+// `bits` of a tensor registered without scales and biases: unquantized BF16 [out_dim][in_dim]
+// (cpu_dequant_matvec's scales == NULL branch, finchmoe/infer.m:1689-1701)
+constexpr int FM_BITS_RAW_BF16 = 16;
+
 }
 
 namespace {
@@ -82,6 +90,7 @@ struct fm_ctx {
     double k1_ms = 0.0, k2_ms = 0.0;
     int kcalls = 0;
     std::string err;
+    bool raw_bf16() const { return bits == FM_BITS_RAW_BF16; }
 
     // affine expert store
     bool aff_cfg = false;
@@ -289,8 +298,8 @@ extern "C" int fm_ctx_destroy(fm_ctx *c) {
     for (auto &t : c->tensors)
         if (t.used && t.owned) {
             (void)hipFree(t.W);
-            (void)hipFree(t.S);
-            (void)hipFree(t.B);
+            if (t.S) (void)hipFree(t.S);
+            if (t.B) (void)hipFree(t.B);
         }
     if (c->h_err) (void)hipHostFree(c->h_err);
     void *ptrs[] = {c->d_layer_ptrs, c->d_gg_ptrs, c->d_act, c->d_eo, c->d_counters,
@@ -427,6 +436,16 @@ extern "C" int fm_experts_config(fm_ctx *c, int n_layers, int n_experts, int hid
     g.n_experts = n_experts;
     // finchmoe/repack_experts.py:76-87, 141-151: W, scales, biases of gate, up, down
     uint64_t gu_w = (uint64_t)inter * hidden * bits / 8, gu_s = (uint64_t)inter * (hidden / 64) * 2;
+extern "C" int fm_stream_probe_dev(fm_ctx *c, const void *d_buf, size_t nbytes) {
+    if (!c) return FM_ERR_ARG;
+    if (!d_buf || nbytes < 4096 || ((uintptr_t)d_buf & 15))
+        return fail(c, FM_ERR_ARG, "stream probe: a 16-byte aligned buffer of 4 KB or more");
+    DeviceGuard dg(c->device);
+    int rc = fm_launch_stream_probe(d_buf, nbytes, nullptr, c->n_cu, c->stream);
+    if (rc) return fail(c, rc, "stream probe launch failed: %s", hipGetErrorString(hipGetLastError()));
+    return FM_OK;
+}
+
     uint64_t d_w = (uint64_t)hidden * inter * bits / 8, d_s = (uint64_t)hidden * (inter / 64) * 2;
     uint64_t o = 0;
     g.gate_w = (uint32_t)o; o += gu_w; g.gate_s = (uint32_t)o; o += gu_s; g.gate_b = (uint32_t)o; o += gu_s;
@@ -529,25 +548,36 @@ static int moe_host_call(fm_ctx *c, moe_dev_fn fn, int hidden, int layer, const 
     // inputs through the pinned mirror: one copy in (x | idx | w | out if accumulating), one
     // copy out (out | expert_out) — pageable copies cost ~10 us each
     char *st = (char *)c->d_stage, *hs = (char *)c->h_stage;
-    memcpy(hs + off_x, x, nx);
-    memcpy(hs + off_i, idx, ni);
-    memcpy(hs + off_w, w, ni);
-    size_t in_bytes = off_w + ni;
-    if (flags & FM_ACCUMULATE) {
-        memcpy(hs + off_o, out, nx);
-        in_bytes = off_o + nx;
+    // A synchronous caller can be given a second try: if the one-launch kernel reports that a
+    // wait on another workgroup ran out (its grid was not resident at once, say under another
+    // tenant of the GPU), the call is repeated once as separate kernels, which wait for nothing.
+    const bool split_before = c->split_phases;
+    for (int attempt = 0; attempt < 2; attempt++) {
+        memcpy(hs + off_x, x, nx);
+        memcpy(hs + off_i, idx, ni);
+        memcpy(hs + off_w, w, ni);
+        size_t in_bytes = off_w + ni;
+        if (flags & FM_ACCUMULATE) {
+            memcpy(hs + off_o, out, nx);
+            in_bytes = off_o + nx;
+        }
+        HIPCHK(c, hipMemcpyAsync(st, hs, in_bytes, hipMemcpyHostToDevice, c->stream));
+        rc = fn(c, layer, (const float *)(st + off_x), (const int32_t *)(st + off_i),
+                (const float *)(st + off_w), M, K, (float *)(st + off_o),
+                expert_out ? (float *)(st + off_e) : nullptr, flags);
+        c->split_phases = split_before;
+        if (rc) return rc;
+        const size_t out_bytes = nx + (expert_out ? ne : 0);
+        HIPCHK(c, hipMemcpyAsync(hs + off_o, st + off_o, out_bytes, hipMemcpyDeviceToHost, c->stream));
+        HIPCHK(c, hipStreamSynchronize(c->stream));
+        rc = check_grid_error(c);
+        if (rc == FM_OK) break;
+        if (attempt == 1 || split_before) return rc;
+        c->split_phases = true;
     }
-    HIPCHK(c, hipMemcpyAsync(st, hs, in_bytes, hipMemcpyHostToDevice, c->stream));
-    rc = fn(c, layer, (const float *)(st + off_x), (const int32_t *)(st + off_i),
-            (const float *)(st + off_w), M, K, (float *)(st + off_o),
-            expert_out ? (float *)(st + off_e) : nullptr, flags);
-    if (rc) return rc;
-    const size_t out_bytes = nx + (expert_out ? ne : 0);
-    HIPCHK(c, hipMemcpyAsync(hs + off_o, st + off_o, out_bytes, hipMemcpyDeviceToHost, c->stream));
-    HIPCHK(c, hipStreamSynchronize(c->stream));
     memcpy(out, hs + off_o, nx);
     if (expert_out) memcpy(expert_out, hs + off_e, ne);
-    return check_grid_error(c);
+    return FM_OK;
 }
 
 static int aff_decode_fn(fm_ctx *c, int layer, const float *x, const int32_t *idx, const float *w,
@@ -627,39 +657,49 @@ static int tensor_add(fm_ctx *c, const void *W, const void *S, const void *B, in
                       int in_dim, int group_size, int bits, int scale_dtype, bool adopt,
                       fm_tensor *out) {
     if (!c) return FM_ERR_ARG;
-    if (!W || !S || !B || !out) return fail(c, FM_ERR_ARG, "null pointer");
+    if (!W || !out) return fail(c, FM_ERR_ARG, "null pointer");
     if (out_dim < 1 || in_dim < 1) return fail(c, FM_ERR_ARG, "non-positive dimension");
-    if (group_size != 64) return fail(c, FM_ERR_UNSUPPORTED, "group_size %d (only 64)", group_size);
-    if (bits != 3 && bits != 4 && bits != 8)
-        return fail(c, FM_ERR_UNSUPPORTED, "tensor bits %d (3, 4 or 8)", bits);
-    if (scale_dtype != FM_SCALE_BF16 && scale_dtype != FM_SCALE_FP16)
-        return fail(c, FM_ERR_ARG, "scale_dtype %d", scale_dtype);
-    int lpr = in_dim / 128;
-    if (in_dim % 128 || !pow2(lpr) || lpr > 64)
-        return fail(c, FM_ERR_UNSUPPORTED, "in_dim %d: need 128*2^j, j<=6", in_dim);
+    // scales == NULL or biases == NULL: an unquantized BF16 weight, as in cpu_dequant_matvec
+    // (finchmoe/infer.m:1689); `bits` and `group_size` say nothing about it then
+    const bool raw = !S || !B;
+    if (raw && (bits == 10 || bits == 11))
+        return fail(c, FM_ERR_ARG, "GGUF tensors (bits 10/11) go through fm_gguf_matvec");
+    if (!raw) {
+        if (bits == 0) bits = 4;   // BatchMatvecSpec default, finchmoe/infer.m:4491
+        if (group_size != 64) return fail(c, FM_ERR_UNSUPPORTED, "group_size %d (only 64)", group_size);
+        if (bits != 3 && bits != 4 && bits != 8)
+            return fail(c, FM_ERR_UNSUPPORTED, "tensor bits %d (3, 4 or 8)", bits);
+        if (scale_dtype != FM_SCALE_BF16 && scale_dtype != FM_SCALE_FP16)
+            return fail(c, FM_ERR_ARG, "scale_dtype %d", scale_dtype);
+        int lpr = in_dim / 128;
+        if (in_dim % 128 || !pow2(lpr) || lpr > 64)
+            return fail(c, FM_ERR_UNSUPPORTED, "in_dim %d: need 128*2^j, j<=6", in_dim);
+    }
     DeviceGuard dg(c->device);
     Tensor t;
     t.used = true;
     t.out_dim = out_dim;
     t.in_dim = in_dim;
     t.group_size = group_size;
-    t.bits = bits;
-    t.scale_fp16 = scale_dtype == FM_SCALE_FP16;
-    size_t wb = (size_t)out_dim * in_dim * bits / 8, sb = (size_t)out_dim * (in_dim / 64) * 2;
+    t.bits = raw ? FM_BITS_RAW_BF16 : bits;
+    t.scale_fp16 = !raw && scale_dtype == FM_SCALE_FP16;
+    size_t wb = (size_t)out_dim * in_dim * t.bits / 8, sb = (size_t)out_dim * (in_dim / 64) * 2;
     if (adopt) {
-        if (((uintptr_t)W & 15) || ((uintptr_t)S & 3) || ((uintptr_t)B & 3))
-            return fail(c, FM_ERR_ARG, "device tensor not aligned (W 16, S/B 4 bytes)");
+        if (((uintptr_t)W & (raw ? 1 : 15)) || (!raw && (((uintptr_t)S & 3) || ((uintptr_t)B & 3))))
+            return fail(c, FM_ERR_ARG, "device tensor not aligned (W 16, S/B 4 bytes; raw BF16 2)");
         t.W = const_cast<void *>(W);
-        t.S = const_cast<void *>(S);
-        t.B = const_cast<void *>(B);
+        t.S = raw ? nullptr : const_cast<void *>(S);
+        t.B = raw ? nullptr : const_cast<void *>(B);
     } else {
         t.owned = true;
         HIPCHK(c, hipMalloc(&t.W, wb));
-        HIPCHK(c, hipMalloc(&t.S, sb));
-        HIPCHK(c, hipMalloc(&t.B, sb));
         HIPCHK(c, hipMemcpy(t.W, W, wb, hipMemcpyHostToDevice));
-        HIPCHK(c, hipMemcpy(t.S, S, sb, hipMemcpyHostToDevice));
-        HIPCHK(c, hipMemcpy(t.B, B, sb, hipMemcpyHostToDevice));
+        if (!raw) {
+            HIPCHK(c, hipMalloc(&t.S, sb));
+            HIPCHK(c, hipMalloc(&t.B, sb));
+            HIPCHK(c, hipMemcpy(t.S, S, sb, hipMemcpyHostToDevice));
+            HIPCHK(c, hipMemcpy(t.B, B, sb, hipMemcpyHostToDevice));
+        }
     }
     for (size_t i = 0; i < c->tensors.size(); i++)
         if (!c->tensors[i].used) {
@@ -696,8 +736,8 @@ extern "C" int fm_tensor_release(fm_ctx *c, fm_tensor t) {
     HIPCHK(c, hipStreamSynchronize(c->stream));
     if (p->owned) {
         (void)hipFree(p->W);
-        (void)hipFree(p->S);
-        (void)hipFree(p->B);
+        if (p->S) (void)hipFree(p->S);
+        if (p->B) (void)hipFree(p->B);
     }
     *p = Tensor();
     return FM_OK;
@@ -732,8 +772,10 @@ static int matvec_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
             m++;
             i++;
         }
-        int rc = fm_launch_dense(specs, m, t0->in_dim, t0->bits, t0->scale_fp16, d_x, M, c->n_cu,
-                                 c->stream);
+        int rc = t0->raw_bf16()
+                     ? fm_launch_dense_bf16(specs, m, t0->in_dim, d_x, M, c->stream)
+                     : fm_launch_dense(specs, m, t0->in_dim, t0->bits, t0->scale_fp16, d_x, M,
+                                       c->n_cu, c->stream);
         if (rc) return fail(c, rc, "matvec launch failed: %s", hipGetErrorString(hipGetLastError()));
     }
     return FM_OK;
@@ -767,10 +809,9 @@ extern "C" int fm_matvec_prefill_batch_dev(fm_ctx *c, const fm_tensor *ts, int n
     int prepared_bits = 0, prepared_in = 0;
     for (int i = 0; i < n; i++) {
         Tensor *p = get_tensor(c, ts[i]);
-        if (!p) return fail(c, FM_ERR_ARG, "bad tensor handle %d", ts[i]);
         if (!d_outs[i]) return fail(c, FM_ERR_ARG, "null output %d", i);
         size_t ws = 0;
-        if (!no_gemm && M >= FM_DENSE_GEMM_MIN_M && ((uintptr_t)d_X & 15) == 0 && ((uintptr_t)d_outs[i] & 3) == 0)
+        if (!no_gemm && !p->raw_bf16() && M >= FM_DENSE_GEMM_MIN_M && ((uintptr_t)d_X & 15) == 0 && ((uintptr_t)d_outs[i] & 3) == 0)
             ws = fm_prefill_dense_ws_bytes(p->out_dim, p->in_dim, p->group_size, p->bits, M);
         if (ws) {
             DeviceGuard dg(c->device);
@@ -842,6 +883,13 @@ extern "C" int fm_matvec_batch(fm_ctx *c, const fm_tensor *ts, int n, const floa
     return matvec_host(c, ts, n, x, outs, 1);
 }
 
+    for (int i = 0; i < n; i++) {   // one X for all: the tensors must agree on its width
+        Tensor *p = get_tensor(c, ts[i]), *p0 = get_tensor(c, ts[0]);
+        if (!p) return fail(c, FM_ERR_ARG, "bad tensor handle %d", ts[i]);
+        if (p->in_dim != p0->in_dim)
+            return fail(c, FM_ERR_ARG, "tensors of one batch must share in_dim (%d vs %d)", p->in_dim,
+                        p0->in_dim);
+    }
 extern "C" int fm_matvec_prefill(fm_ctx *c, fm_tensor t, const float *X, float *out, int M) {
     if (!c) return FM_ERR_ARG;
     if (M < 1 || M > 65535) return fail(c, FM_ERR_ARG, "M %d outside 1..65535", M);
@@ -886,13 +934,17 @@ extern "C" int fm_layer_tail_dev(fm_ctx *c, fm_tensor shared_down, const float *
         return fail(c, FM_ERR_ARG, "next input and its norm weights go together");
     if (((uintptr_t)d_shared_gate | (uintptr_t)d_shared_up) & 3)
         return fail(c, FM_ERR_ARG, "vector not 4-byte aligned");
-    if (t->group_size != 64) return fail(c, FM_ERR_UNSUPPORTED, "group size %d", t->group_size);
+    if (t->raw_bf16() || t->group_size != 64)
+        return fail(c, FM_ERR_UNSUPPORTED, "shared down projection must be 3/4/8-bit, group size 64");
     if (t->out_dim / 4 > FM_TAIL_PARTIALS) return fail(c, FM_ERR_UNSUPPORTED, "hidden %d", t->out_dim);
     DeviceGuard dg(c->device);
     if (!c->d_tail) {
         HIPCHK(c, hipMalloc((void **)&c->d_tail, (FM_TAIL_PARTIALS + 64) * sizeof(float)));
         HIPCHK(c, hipMemsetAsync(c->d_tail, 0, (FM_TAIL_PARTIALS + 64) * sizeof(float), c->stream));
     }
+        if (t->in_dim != t0->in_dim)   // the staging area holds one X of t0's width
+            return fail(c, FM_ERR_ARG, "tensors of one batch must share in_dim (%d vs %d)", t->in_dim,
+                        t0->in_dim);
     FmTailArgs a;
     a.W = (const uint8_t *)t->W;
     a.S = (const uint8_t *)t->S;
@@ -962,8 +1014,9 @@ extern "C" int fm_gguf_config(fm_ctx *c, int n_layers, int n_experts, int hidden
     return FM_OK;
 }
 
-static int gguf_set_layer(fm_ctx *c, int layer, const void *gate, const void *up,
-                          const void *down, bool adopt) {
+static int gguf_set_layer(fm_ctx *c, int layer, const void *gate, size_t gate_bytes,
+                          const void *up, size_t up_bytes, const void *down, size_t down_bytes,
+                          bool adopt) {
     if (!c) return FM_ERR_ARG;
     if (!c->gguf_cfg) return fail(c, FM_ERR_STATE, "GGUF store not configured");
     if (!gate || !up || !down || layer < 0 || layer >= c->g_layers)
@@ -972,11 +1025,33 @@ static int gguf_set_layer(fm_ctx *c, int layer, const void *gate, const void *up
         return fail(c, FM_ERR_ARG, "device slab not 16-byte aligned");
     DeviceGuard dg(c->device);
     HIPCHK(c, hipStreamSynchronize(c->stream));
-    const FmGgufGeom &g = c->ggeom;
-    int rc = set_layer(c, c->g_gate, layer, gate, (size_t)g.n_experts * g.gate_slab, adopt);
-    if (!rc) rc = set_layer(c, c->g_up, layer, up, (size_t)g.n_experts * g.up_slab, adopt);
-    if (!rc) rc = set_layer(c, c->g_down, layer, down, (size_t)g.n_experts * g.down_slab, adopt);
-    if (rc) return rc;
+    if (!adopt) {
+        // all three copies land in fresh buffers before the layer's pointers change
+        const void *src[3] = {gate, up, down};
+        void *fresh[3] = {nullptr, nullptr, nullptr};
+        hipError_t e = hipSuccess;
+        for (int i = 0; i < 3 && e == hipSuccess; i++) {
+            e = hipMalloc(&fresh[i], want[i]);
+            if (e == hipSuccess) e = hipMemcpy(fresh[i], src[i], want[i], hipMemcpyHostToDevice);
+        }
+        if (e != hipSuccess) {
+            for (void *f : fresh)
+                if (f) (void)hipFree(f);
+            return fail(c, FM_ERR_HIP, "GGUF layer upload: %s", hipGetErrorString(e));
+        }
+        std::vector<LayerBuf> *dst[3] = {&c->g_gate, &c->g_up, &c->g_down};
+        for (int i = 0; i < 3; i++) {
+            LayerBuf &lb = (*dst[i])[layer];
+            if (lb.owned && lb.ptr) (void)hipFree(lb.ptr);
+            lb.ptr = fresh[i];
+            lb.owned = true;
+        }
+    } else {
+        int rc = set_layer(c, c->g_gate, layer, gate, want[0], true);
+        if (!rc) rc = set_layer(c, c->g_up, layer, up, want[1], true);
+        if (!rc) rc = set_layer(c, c->g_down, layer, down, want[2], true);
+        if (rc) return rc;
+    }
     void *p[3] = {c->g_gate[layer].ptr, c->g_up[layer].ptr, c->g_down[layer].ptr};
     for (int i = 0; i < 3; i++)
         HIPCHK(c, hipMemcpy(c->d_gg_ptrs + (size_t)i * c->g_layers + layer, &p[i], sizeof(void *),
@@ -984,13 +1059,15 @@ static int gguf_set_layer(fm_ctx *c, int layer, const void *gate, const void *up
     return FM_OK;
 }
 
-extern "C" int fm_gguf_upload_layer(fm_ctx *c, int layer, const void *gate, const void *up,
-                                    const void *down) {
-    return gguf_set_layer(c, layer, gate, up, down, false);
+extern "C" int fm_gguf_upload_layer(fm_ctx *c, int layer, const void *gate, size_t gate_bytes,
+                                    const void *up, size_t up_bytes, const void *down,
+                                    size_t down_bytes) {
+    return gguf_set_layer(c, layer, gate, gate_bytes, up, up_bytes, down, down_bytes, false);
 }
-extern "C" int fm_gguf_adopt_layer(fm_ctx *c, int layer, const void *gate, const void *up,
-                                   const void *down) {
-    return gguf_set_layer(c, layer, gate, up, down, true);
+extern "C" int fm_gguf_adopt_layer(fm_ctx *c, int layer, const void *gate, size_t gate_bytes,
+                                   const void *up, size_t up_bytes, const void *down,
+                                   size_t down_bytes) {
+    return gguf_set_layer(c, layer, gate, gate_bytes, up, up_bytes, down, down_bytes, true);
 }
 
 static int gguf_decode_groups(fm_ctx *c, int layer0, int layer_stride, int groups,
@@ -1047,6 +1124,14 @@ static int gguf_prefill_fn(fm_ctx *c, int layer, const float *x, const int32_t *
 
 extern "C" int fm_gguf_moe_decode(fm_ctx *c, int layer, const float *x, const int32_t *idx,
                                   const float *w, int K, float *out, float *expert_out, int flags) {
+    const FmGgufGeom &g = c->ggeom;
+    const size_t want[3] = {(size_t)g.n_experts * g.gate_slab, (size_t)g.n_experts * g.up_slab,
+                            (size_t)g.n_experts * g.down_slab};
+    const size_t have[3] = {gate_bytes, up_bytes, down_bytes};
+    for (int i = 0; i < 3; i++)
+        if (have[i] != want[i])
+            return fail(c, FM_ERR_ARG, "GGUF %s tensor is %zu bytes, expected %zu",
+                        i == 0 ? "gate" : i == 1 ? "up" : "down", have[i], want[i]);
     if (!c) return FM_ERR_ARG;
     if (!c->gguf_cfg) return fail(c, FM_ERR_STATE, "GGUF store not configured");
     return moe_host_call(c, gguf_decode_fn, c->ggeom.hidden, layer, x, idx, w, 1, K, out,
@@ -1200,3 +1285,5 @@ extern "C" int fm_gguf_dequant_expert(fm_ctx *c, int layer, int expert, int whic
     }
     return dequant_common(c, base, nullptr, nullptr, rows, cols, 0, 0, type, nullptr, w_f32, nullptr);
 }
+    if (p->raw_bf16()) return fail(c, FM_ERR_UNSUPPORTED, "tensor %d is raw BF16: nothing to dequantize", t);
+    if (p->raw_bf16()) return fail(c, FM_ERR_UNSUPPORTED, "embedding lookup needs a quantized tensor");

@@ -628,6 +628,14 @@ __device__ __forceinline__ void fm_flag_wait(const FmFlags &f, const unsigned in
         }
         __builtin_amdgcn_s_sleep(8);
     }
+    // The vector this wait guards is read with relaxed device-scope loads, which carry no
+    // ordering of their own: without this the compiler may legally hoist them above the poll
+    // loop.  The hardware half: the producer's device-scope (sc1) stores write through to the
+    // memory side of the fabric, `s_waitcnt vmcnt(0)` returns only once they have been
+    // acknowledged from there, and only then is the counter incremented (an atomic performed
+    // at the same place) — so a device-scope load issued after the counter was seen reads the
+    // stored value whichever XCD's L2 sits in front of the reader, with no cache maintenance.
+    __atomic_signal_fence(__ATOMIC_ACQUIRE);
 }
 
 // gate/up: publishes per pair how many of its units this workgroup finished

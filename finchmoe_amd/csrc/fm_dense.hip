@@ -331,7 +331,78 @@ int launch_dense_t(const FmDenseArgs &a, int total_items, int M, hipStream_t st)
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 
+// ----------------------------------------------------------------------
+// Raw BF16 weights [out_dim][in_dim] (cpu_dequant_matvec with scales == NULL,
+// finchmoe/infer.m:1689-1701): the tensors the reference's quantizer leaves
+// unquantized (mlp.gate, shared_expert_gate, in_proj_a, in_proj_b:
+// finchmoe/quantize_non_experts.py:103-107).  One wave per row: a lane takes
+// eight weights per 128-bit load (bf16 -> fp32 is a shift), fp32 accumulate, sum
+// over the wave.  VEC: rows are 16-byte aligned and in_dim is a multiple of 8.
+// ----------------------------------------------------------------------
+template <bool VEC>
+__global__ __launch_bounds__(256) void fm_dense_bf16(FmDenseArgs a, int total_rows) {
+    const int lane = threadIdx.x & 63;
+    const int gr = blockIdx.x * 4 + (threadIdx.x >> 6);   // row of the launch (wave-uniform)
+    if (gr >= total_rows) return;
+    int t = 0;
+#pragma unroll
+    for (int i = 1; i < FM_MAX_BATCH; i++)
+        if (i < a.n && gr >= a.unit_first[i]) t = i;
+    const FmDenseSpec sp = a.spec[t];
+    const int row = gr - a.unit_first[t];
+    const int m = blockIdx.y;
+    const uint16_t *w = reinterpret_cast<const uint16_t *>(sp.W) + (size_t)row * a.in_dim;
+    const float *x = a.x + (size_t)m * a.in_dim;
+    float acc = 0.0f;
+    if constexpr (VEC) {
+        for (int c = lane * 8; c < a.in_dim; c += 64 * 8) {
+            const uint4 q = *reinterpret_cast<const uint4 *>(w + c);
+            const float4 x0 = *reinterpret_cast<const float4 *>(x + c);
+            const float4 x1 = *reinterpret_cast<const float4 *>(x + c + 4);
+            acc = fmaf(fm_bf16_lo(q.x), x0.x, acc);
+            acc = fmaf(fm_bf16_hi(q.x), x0.y, acc);
+            acc = fmaf(fm_bf16_lo(q.y), x0.z, acc);
+            acc = fmaf(fm_bf16_hi(q.y), x0.w, acc);
+            acc = fmaf(fm_bf16_lo(q.z), x1.x, acc);
+            acc = fmaf(fm_bf16_hi(q.z), x1.y, acc);
+            acc = fmaf(fm_bf16_lo(q.w), x1.z, acc);
+            acc = fmaf(fm_bf16_hi(q.w), x1.w, acc);
+        }
+    } else {
+        for (int c = lane; c < a.in_dim; c += 64)
+            acc = fmaf(__uint_as_float((uint32_t)w[c] << 16), x[c], acc);
+    }
+    acc = fm_group_sum<64>(acc);
+    if (lane == 0) sp.out[(size_t)m * sp.out_dim + row] = acc;
+}
+
 }  // namespace
+
+// n raw-BF16 tensors [out_dim][in_dim] sharing x[M][in_dim]; specs[i].S / .B are unused.
+extern "C" int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim, const float *d_x,
+                                    int M, hipStream_t st) {
+    if (n < 1 || n > FM_MAX_BATCH || M < 1 || in_dim < 1) return FM_ERR_ARG;
+    FmDenseArgs a;
+    a.n = n;
+    a.in_dim = in_dim;
+    a.rows_per_item = 0;
+    a.x = d_x;
+    a.out_stride = 0;
+    int rows = 0;
+    bool vec = in_dim % 8 == 0 && ((uintptr_t)d_x & 15) == 0;
+    for (int i = 0; i < n; i++) {
+        a.spec[i] = specs[i];
+        a.unit_first[i] = rows;
+        rows += specs[i].out_dim;
+        vec = vec && ((uintptr_t)specs[i].W & 15) == 0;
+    }
+    for (int i = n; i < FM_MAX_BATCH; i++) a.spec[i] = a.spec[0];
+    for (int i = n; i <= FM_MAX_BATCH; i++) a.unit_first[i] = rows;
+    const dim3 grid((rows + 3) / 4, M);
+    if (vec) hipLaunchKernelGGL(fm_dense_bf16<true>, grid, dim3(256), 0, st, a, rows);
+    else hipLaunchKernelGGL(fm_dense_bf16<false>, grid, dim3(256), 0, st, a, rows);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
 
 // specs[i].first_item is filled here.  in_dim must be 128 * 2^j, j <= 6.
 extern "C" int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,

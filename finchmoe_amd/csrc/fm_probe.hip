@@ -1,0 +1,71 @@
+// fm_probe.hip — the streaming ceiling of the memory system, measured the way the expert
+// kernels read: one workgroup of eight waves per CU, every wave a ring of 4 KB slots in LDS
+// filled with LDS-direct 16-byte loads over one contiguous share of a buffer, no arithmetic.
+// What this kernel reaches is what a bandwidth-bound kernel of that structure can reach at
+// best; the decode kernels are priced against the published peak and compared with this.
+// No counterpart in the reference (a measurement aid, like its --timing accumulators,
+// finchmoe/infer.m:281-298).
+#include "fm_ring.h"
+
+namespace {
+
+constexpr int PROBE_WAVES = 8;
+constexpr int PROBE_RING = 4;
+constexpr int PROBE_SLOT = 4096;       // 4 loads of 64 lanes x 16 bytes
+
+extern __shared__ __attribute__((aligned(16))) uint8_t fm_probe_lds[];
+
+__global__ __launch_bounds__(PROBE_WAVES * 64) void fm_stream_probe_k(const uint8_t *buf, size_t n_slots,
+                                                                      unsigned int *sink) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t ring0 = fm_lds_addr(fm_probe_lds) + (uint32_t)wave * (PROBE_RING * PROBE_SLOT);
+    // this workgroup's contiguous share of the slots, its waves interleaved over it
+    const size_t s0 = n_slots * blockIdx.x / gridDim.x, s1 = n_slots * (blockIdx.x + 1) / gridDim.x;
+    size_t next = s0 + wave;
+    uint32_t issued = 0, consumed = 0;
+    int wpos = 0, c = 0;
+    auto issue = [&]() __attribute__((always_inline)) {
+        if (next >= s1) return;
+        const uint8_t *src = fm_uniform(buf + next * PROBE_SLOT) + lane * 16;
+        const uint32_t slot = ring0 + (uint32_t)wpos * PROBE_SLOT;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(src + 1024 * j),
+                                             (fm_lptr)(uintptr_t)(slot + 1024 * j), 16, 0, 0);
+        next += PROBE_WAVES;
+        wpos = wpos + 1 == PROBE_RING ? 0 : wpos + 1;
+        issued++;
+    };
+#pragma unroll
+    for (int k = 0; k < PROBE_RING; k++) issue();
+    uint32_t acc = 0;
+    while (consumed < issued) {
+        if (issued - consumed == (uint32_t)PROBE_RING) fm_dma_wait<4 * (PROBE_RING - 1)>(false);
+        else fm_dma_wait<0>(true);
+        // one dword of the landed slot per lane, so that the data is really consumed
+        uint32_t v;
+        const uint32_t addr = ring0 + (uint32_t)c * PROBE_SLOT + 4 * lane;
+        asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
+        acc ^= v;
+        consumed++;
+        c = c + 1 == PROBE_RING ? 0 : c + 1;
+        issue();
+    }
+    if (acc == 0x9E3779B9u && sink) *sink = acc;     // practically never: keeps `acc` alive
+}
+
+}  // namespace
+
+// reads nbytes (rounded down to whole 4 KB slots) of d_buf once
+extern "C" int fm_launch_stream_probe(const void *d_buf, size_t nbytes, unsigned int *d_sink, int n_cu,
+                                      hipStream_t st) {
+    const size_t n_slots = nbytes / PROBE_SLOT;
+    if (!d_buf || n_slots == 0 || ((uintptr_t)d_buf & 15)) return FM_ERR_ARG;
+    const size_t sh = (size_t)PROBE_WAVES * PROBE_RING * PROBE_SLOT;
+    static FmLdsAttr attr;
+    if (!fm_dyn_lds_ready(attr, (const void *)fm_stream_probe_k, sh)) return FM_ERR_HIP;
+    hipLaunchKernelGGL(fm_stream_probe_k, dim3(n_cu), dim3(PROBE_WAVES * 64), sh, st,
+                       (const uint8_t *)d_buf, n_slots, d_sink);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}

@@ -80,6 +80,11 @@ __global__ __launch_bounds__(256) void fm_layer_tail(FmTailArgs a) {
     }
     __syncthreads();
     if (ticket != gridDim.x - 1) return;
+    // The loads below read what other workgroups stored before they drew their tickets.  They
+    // are relaxed device-scope accesses, which the compiler may move: keep them behind the
+    // ticket (the hardware side: a device-scope store that has left the wave under vmcnt(0)
+    // has been performed at the memory side of the L2s, where device-scope loads look).
+    __atomic_signal_fence(__ATOMIC_ACQUIRE);
 
     // last workgroup: every other one has stored its rows and its partial sum.  The partials
     // are fetched side by side and added in workgroup order.

@@ -71,6 +71,10 @@ static slot *tab_find(const void *key, int insert) {
 
 static int resident(const void *W, const void *S, const void *B, int out_dim, int in_dim,
                     int group_size, int bits, fm_tensor *t) {
+    /* scales == NULL: an unquantized BF16 tensor (infer.m:1689); otherwise bits 0 means 4
+     * (infer.m:4491).  Normalised here so that the table compares like with like. */
+    if (!S || !B) { S = B = NULL; bits = 16; }
+    else if (bits == 0) bits = 4;
     slot *s = tab_find(W, 1);
     if (s->t >= 0 && (s->out_dim != out_dim || s->in_dim != in_dim || s->bits != bits)) {
         fm_tensor_release(g_ctx, s->t);   /* host memory was reused for another tensor */
@@ -127,12 +131,11 @@ void fast_dequant_matvec(const uint32_t *W, const uint16_t *scales, const uint16
                          int bits) {
     if (!g_ctx) { fail(FM_ERR_STATE, "fast_dequant_matvec"); return; }
     int rc;
-    if (!scales || !biases) {
-        /* GGUF tensors carry no scales (infer.m:3378-3388); raw BF16 is not a quantized
-         * product and has no kernel here */
-        if (bits != 10 && bits != 11) { fail(FM_ERR_UNSUPPORTED, "fast_dequant_matvec (raw BF16)"); return; }
+    if ((!scales || !biases) && (bits == 10 || bits == 11)) {
+        /* GGUF tensors carry no scales (infer.m:3378-3388) */
         rc = fm_gguf_matvec(g_ctx, W, bits == 10 ? FM_GGML_Q4_K : FM_GGML_Q6_K, x, out, out_dim, in_dim);
     } else {
+        /* quantized, or scales == NULL: raw BF16 [out_dim][in_dim] (infer.m:1689-1701) */
         fm_tensor t;
         rc = resident(W, scales, biases, out_dim, in_dim, group_size, bits, &t);
         if (!rc) {
@@ -140,8 +143,18 @@ void fast_dequant_matvec(const uint32_t *W, const uint16_t *scales, const uint16
             rc = fm_matvec_batch(g_ctx, &t, 1, x, outs);
         }
     }
-    if (rc) fail(rc, "fast_dequant_matvec");
-    else g_status = FM_OK;
+    if (rc) {
+        /* the reference's call sites take a void result: never leave `out` uninitialised */
+        memset(out, 0, (size_t)out_dim * sizeof(float));
+        fail(rc, "fast_dequant_matvec");
+    } else {
+        g_status = FM_OK;
+    }
+}
+
+static void zero_batch_outputs(BatchMatvecSpec *specs, int num_specs) {
+    for (int i = 0; i < num_specs; i++)
+        if (specs[i].out_cpu) memset(specs[i].out_cpu, 0, (size_t)specs[i].out_dim * sizeof(float));
 }
 
 void fast_batch_matvec(const float *x, uint32_t x_dim, BatchMatvecSpec *specs, int num_specs) {
@@ -149,16 +162,30 @@ void fast_batch_matvec(const float *x, uint32_t x_dim, BatchMatvecSpec *specs, i
     if (num_specs < 1 || num_specs > 64) { fail(FM_ERR_ARG, "fast_batch_matvec"); return; }
     fm_tensor ts[64];
     float *outs[64];
-    for (int i = 0; i < num_specs; i++) {
-        if (specs[i].in_dim != x_dim) { fail(FM_ERR_ARG, "fast_batch_matvec (in_dim != x_dim)"); return; }
-        int rc = resident(specs[i].W, specs[i].scales, specs[i].biases, (int)specs[i].out_dim,
+    int rc = FM_OK;
+    const char *what = "fast_batch_matvec";
+    for (int i = 0; i < num_specs && !rc; i++) {
+        if (specs[i].in_dim != x_dim) {
+            rc = FM_ERR_ARG;
+            what = "fast_batch_matvec (in_dim != x_dim)";
+        } else if ((!specs[i].scales || !specs[i].biases) && (specs[i].bits == 10 || specs[i].bits == 11)) {
+            /* a GGUF spec has no batched kernel: the reference keeps such batches on its CPU
+             * path too (infer.m:4481-4483); issue it as a single fast_dequant_matvec */
+            rc = FM_ERR_UNSUPPORTED;
+            what = "fast_batch_matvec (GGUF spec: use fast_dequant_matvec)";
+        } else {
+            rc = resident(specs[i].W, specs[i].scales, specs[i].biases, (int)specs[i].out_dim,
                           (int)specs[i].in_dim, (int)specs[i].group_size, specs[i].bits, &ts[i]);
-        if (rc) { fail(rc, "fast_batch_matvec"); return; }
+        }
         outs[i] = specs[i].out_cpu;
     }
-    int rc = fm_matvec_batch(g_ctx, ts, num_specs, x, outs);
-    if (rc) fail(rc, "fast_batch_matvec");
-    else g_status = FM_OK;
+    if (!rc) rc = fm_matvec_batch(g_ctx, ts, num_specs, x, outs);
+    if (rc) {
+        zero_batch_outputs(specs, num_specs);   /* void result: never leave outputs uninitialised */
+        fail(rc, what);
+    } else {
+        g_status = FM_OK;
+    }
 }
 
 void fast_prefill_matvec(const uint32_t *W, const uint16_t *scales, const uint16_t *biases,
@@ -195,9 +222,10 @@ int finch_ops_config_gguf_experts(int n_layers, int n_experts, int hidden, int i
     return FM_OK;
 }
 
-int finch_ops_load_gguf_layer(int layer, const void *gate, const void *up, const void *down) {
+int finch_ops_load_gguf_layer(int layer, const void *gate, size_t gate_bytes, const void *up,
+                              size_t up_bytes, const void *down, size_t down_bytes) {
     if (!g_ctx) return fail(FM_ERR_STATE, "finch_ops_load_gguf_layer");
-    int rc = fm_gguf_upload_layer(g_ctx, layer, gate, up, down);
+    int rc = fm_gguf_upload_layer(g_ctx, layer, gate, gate_bytes, up, up_bytes, down, down_bytes);
     return rc ? fail(rc, "finch_ops_load_gguf_layer") : FM_OK;
 }
 

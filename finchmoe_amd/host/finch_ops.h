@@ -65,7 +65,8 @@ int finch_ops_load_expert_layer(int layer, const void *blob, size_t nbytes);
 /* GGUF stacked expert tensors of one layer (finchmoe/infer.m:1017-1022) */
 int finch_ops_config_gguf_experts(int n_layers, int n_experts, int hidden, int inter,
                                   int gate_type, int up_type, int down_type);
-int finch_ops_load_gguf_layer(int layer, const void *gate, const void *up, const void *down);
+int finch_ops_load_gguf_layer(int layer, const void *gate, size_t gate_bytes, const void *up,
+                              size_t up_bytes, const void *down, size_t down_bytes);
 
 /* routed experts of one layer: moe_out += sum_k w_k * expert_k(h_post), slot order, with
  * the CPU path's finite guard + renormalisation (finchmoe/infer.m:10109-10204).

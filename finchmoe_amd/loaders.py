@@ -82,7 +82,9 @@ class DenseFile:
             raise ValueError("%s is %s, not a packed tensor" % (weight_name, t["dtype"]))
         bits, gs = int(t["bits"]), int(t["group_size"])
         out_dim, packed_cols = t["shape"]
-        in_dim = packed_cols * (32 // bits)
+        in_dim = packed_cols * 32 // bits
+        if in_dim % gs:
+            raise ValueError("%s: in_dim %d is not a multiple of the group size %d" % (weight_name, in_dim, gs))
         base = weight_name[:-len(".weight")] if weight_name.endswith(".weight") else weight_name
         W = self.raw(weight_name, np.uint32).reshape(out_dim, packed_cols)
         S = self.raw(base + ".scales", np.uint16).reshape(out_dim, in_dim // gs)

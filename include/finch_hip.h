@@ -103,6 +103,13 @@ FM_API int fm_set_wait_limit(fm_ctx *ctx, unsigned int polls);
 /* sums in milliseconds since the last read, and the number of calls; resets */
 FM_API int fm_kernel_timing_read(fm_ctx *ctx, double *gate_up_ms, double *down_ms, int *calls);
 
+/* Streaming probe: reads nbytes (whole 4 KB slots) of the device buffer d_buf once, with the
+ * access structure of the expert kernels (one workgroup of eight waves per CU, LDS-direct
+ * 16-byte loads into a ring, contiguous shares) and no arithmetic; asynchronous on the
+ * context's stream.  Timed with fm_timer_start/stop it gives the rate the memory system
+ * delivers to a kernel of that structure.  No counterpart in the reference. */
+FM_API int fm_stream_probe_dev(fm_ctx *ctx, const void *d_buf, size_t nbytes);
+
 /* ---------------------------------------------------------------- expert store, affine
  * Replaces the packed-expert files + pread/LRU machinery
  * (finchmoe/infer.m:5816-6575, 15421-15425) by HBM residency.
@@ -220,10 +227,13 @@ FM_API int fm_layer_tail_dev(fm_ctx *ctx, fm_tensor shared_down, const float *d_
  * Q6_K (infer.m:3166). */
 FM_API int fm_gguf_config(fm_ctx *ctx, int n_layers, int n_experts, int hidden, int inter,
                    int gate_type, int up_type, int down_type);
-FM_API int fm_gguf_upload_layer(fm_ctx *ctx, int layer, const void *gate, const void *up,
-                         const void *down);
-FM_API int fm_gguf_adopt_layer(fm_ctx *ctx, int layer, const void *d_gate, const void *d_up,
-                        const void *d_down);
+/* the byte counts must equal n_experts * slab of the configured geometry (a file whose
+ * dimensions or types differ from the configuration is refused instead of over-read);
+ * on any failure the layer keeps what it held before */
+FM_API int fm_gguf_upload_layer(fm_ctx *ctx, int layer, const void *gate, size_t gate_bytes,
+                         const void *up, size_t up_bytes, const void *down, size_t down_bytes);
+FM_API int fm_gguf_adopt_layer(fm_ctx *ctx, int layer, const void *d_gate, size_t gate_bytes,
+                        const void *d_up, size_t up_bytes, const void *d_down, size_t down_bytes);
 /* gpu_gguf_experts_forward (finchmoe/infer.m:3153-3366) */
 FM_API int fm_gguf_moe_decode_dev(fm_ctx *ctx, int layer, const float *d_x, const int32_t *d_idx,
                            const float *d_w, int K, float *d_out, float *d_expert_out,

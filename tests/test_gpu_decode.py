@@ -321,3 +321,21 @@ def test_errors_are_codes_not_aborts(hip, store3):
         assert e.value.status == fb.ERR_STATE
     finally:
         c2.close()
+
+
+def test_host_call_falls_back_to_separate_kernels(hip, orc, store3):
+    """With a wait limit of zero polls the one-launch kernel gives up on its waits; the
+    synchronous entry point then repeats the call as separate kernels and still returns the
+    right result."""
+    rng = np.random.default_rng(23)
+    x = rng.standard_normal(H).astype(np.float32)
+    idx, w = _route(orc, rng, 12, 8)
+    ref, ref_eo = orc.moe_experts_forward(store3[1], x, idx, w, H, I, 3)
+    hip.set_wait_limit(0)
+    try:
+        for _ in range(8):
+            out, eo = hip.moe_decode(1, x, idx, w)
+            assert_parity(out, ref, "fallback result")
+            assert_parity(eo, ref_eo, "fallback expert outputs")
+    finally:
+        hip.set_wait_limit(1 << 20)

@@ -191,3 +191,45 @@ def test_dense_prefill_batch_shares_the_prepared_input(hip, orc):
     finally:
         for t in (ta, tb, tc, td):
             hip.tensor_release(t)
+
+
+@pytest.mark.parametrize("out_dim,in_dim", [(32, 2048), (256, 2048), (1, 2048), (7, 100), (33, 4096)])
+def test_raw_bf16_matvec(hip, orc, out_dim, in_dim):
+    """Tensors registered without scales and biases are unquantized BF16 [out][in]
+    (cpu_dequant_matvec's scales == NULL branch, infer.m:1689-1701)."""
+    rng = np.random.default_rng(out_dim * 7 + in_dim)
+    W = F.bf16_trunc(rng.standard_normal((out_dim, in_dim)).astype(np.float32) * np.float32(0.1))
+    t = hip.tensor_register(W, None, None, out_dim, in_dim, bits=0)
+    x = rng.standard_normal(in_dim).astype(np.float32)
+    (out,) = hip.matvec_batch([t], x, [out_dim])
+    ref = orc.dequant_matvec(W, None, None, x, out_dim, in_dim, 0)
+    want = F.bf16_to_f32(W).astype(np.float64) @ x.astype(np.float64)
+    scale = max(float(np.max(np.abs(want))), 1e-30)
+    assert np.max(np.abs(out - ref)) <= 1e-3 * scale and np.max(np.abs(out - want)) <= 1e-5 * scale
+    # M positions equal the single calls bit for bit
+    X = rng.standard_normal((5, in_dim)).astype(np.float32)
+    om = hip.matvec_prefill(t, X, out_dim)
+    for m in range(5):
+        (single,) = hip.matvec_batch([t], X[m], [out_dim])
+        assert np.array_equal(om[m], single)
+    from finchmoe_amd import FinchError
+    with pytest.raises(FinchError) as e:
+        hip.dequant_tensor(t, out_dim, in_dim)
+    assert e.value.status == fb.ERR_UNSUPPORTED
+    hip.tensor_release(t)
+
+
+def test_raw_bf16_in_a_mixed_batch(hip, orc):
+    """One fm_matvec_batch call over 4-bit and BF16 tensors that share x."""
+    rng = np.random.default_rng(77)
+    t4, a = _tensor(hip, rng, 128, 2048, 4)
+    Wb = F.bf16_trunc(rng.standard_normal((32, 2048)).astype(np.float32) * np.float32(0.1))
+    tb = hip.tensor_register(Wb, None, None, 32, 2048)
+    t4b, c = _tensor(hip, rng, 64, 2048, 4)
+    x = rng.standard_normal(2048).astype(np.float32)
+    o1, o2, o3 = hip.matvec_batch([t4, tb, t4b], x, [128, 32, 64])
+    assert_parity(o1, orc.dequant_matvec(a[1], a[2], a[3], x, 128, 2048, 4), "4-bit first")
+    assert_parity(o2, orc.dequant_matvec(Wb, None, None, x, 32, 2048, 0), "BF16")
+    assert_parity(o3, orc.dequant_matvec(c[1], c[2], c[3], x, 64, 2048, 4), "4-bit last")
+    for t in (t4, tb, t4b):
+        hip.tensor_release(t)

@@ -30,7 +30,7 @@ def ops():
     L.fast_batch_matvec.argtypes = [vp, C.c_uint32, C.POINTER(BatchMatvecSpec), i]
     L.fast_prefill_matvec.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, i]
     L.finch_ops_load_expert_layer.argtypes = [i, vp, C.c_size_t]
-    L.finch_ops_load_gguf_layer.argtypes = [i, vp, vp, vp]
+    L.finch_ops_load_gguf_layer.argtypes = [i, vp, C.c_size_t, vp, C.c_size_t, vp, C.c_size_t]
     L.moe_experts_forward.argtypes = [i, vp, vp, vp, i, vp]
     L.gpu_gguf_experts_forward.argtypes = [i, vp, vp, vp, i, vp]
     L.moe_experts_forward_chunk.argtypes = [i, vp, vp, vp, i, i, vp]
@@ -134,10 +134,61 @@ def test_host_ops_on_gpu(ops, orc):
         # GGUF experts
         g, u, d = F.synth_gguf_layer(rng, E, H, I)
         assert ops.finch_ops_config_gguf_experts(1, E, H, I, 12, 12, 14) == 0
-        assert ops.finch_ops_load_gguf_layer(0, g.ctypes.data, u.ctypes.data, d.ctypes.data) == 0
+        assert ops.finch_ops_load_gguf_layer(0, g.ctypes.data, g.size, u.ctypes.data, u.size, d.ctypes.data, d.size) == 0
         moe = np.zeros(H, np.float32)
         assert ops.gpu_gguf_experts_forward(0, x.ctypes.data, idx.ctypes.data, w.ctypes.data, 4, moe.ctypes.data) == 1
         refg, _ = orc.moe_gguf_forward(g, u, d, x, idx, w, H, I, guard=1)
         assert_parity(moe, refg, "gguf experts")
+    finally:
+        ops.finch_ops_shutdown()
+
+
+@pytest.mark.gpu
+def test_reference_gdn_batch_with_raw_bf16_specs(ops, orc):
+    """The reference's own decode batch {qkv 8192, z 4096, b 32, a 32} (infer.m:8118-8122):
+    qkv and z are 4-bit, in_proj_b / in_proj_a stay BF16 in the reference's checkpoints
+    (quantize_non_experts.py:103-107) and arrive with scales == biases == NULL.  Also the
+    routing gate [256, 2048] and the shared expert's gate [1, 2048] as single BF16 matvecs
+    (cpu_dequant_matvec's raw branch, infer.m:1689-1701)."""
+    H = 2048
+    rng = np.random.default_rng(21)
+    assert ops.finch_ops_init(0) == 0, ops.finch_ops_last_error()
+    try:
+        _, Wq, Sq, Bq = F.synth_affine_tensor(rng, 8192, H, 4)
+        _, Wz, Sz, Bz = F.synth_affine_tensor(rng, 4096, H, 4)
+        Wb = F.bf16_trunc(rng.standard_normal((32, H)).astype(np.float32) * np.float32(0.05))
+        Wa = F.bf16_trunc(rng.standard_normal((32, H)).astype(np.float32) * np.float32(0.05))
+        x = rng.standard_normal(H).astype(np.float32)
+        oq, oz = np.full(8192, np.nan, np.float32), np.full(4096, np.nan, np.float32)
+        ob, oa = np.full(32, np.nan, np.float32), np.full(32, np.nan, np.float32)
+        specs = (BatchMatvecSpec * 4)(
+            BatchMatvecSpec(Wq.ctypes.data, Sq.ctypes.data, Bq.ctypes.data, oq.ctypes.data, 8192, H, 64, 0, 4),
+            BatchMatvecSpec(Wz.ctypes.data, Sz.ctypes.data, Bz.ctypes.data, oz.ctypes.data, 4096, H, 64, 1, 0),
+            BatchMatvecSpec(Wb.ctypes.data, None, None, ob.ctypes.data, 32, H, 64, 2, 0),
+            BatchMatvecSpec(Wa.ctypes.data, None, None, oa.ctypes.data, 32, H, 64, 3, 4))
+        ops.fast_batch_matvec(x.ctypes.data, H, specs, 4)
+        assert ops.finch_ops_last_status() == 0, ops.finch_ops_last_error()
+        assert_parity(oq, orc.dequant_matvec(Wq, Sq, Bq, x, 8192, H, 4), "qkv")
+        assert_parity(oz, orc.dequant_matvec(Wz, Sz, Bz, x, 4096, H, 4), "z (bits 0 = 4)")
+        assert_parity(ob, orc.dequant_matvec(Wb, None, None, x, 32, H, 0), "in_proj_b (BF16)")
+        assert_parity(oa, orc.dequant_matvec(Wa, None, None, x, 32, H, 0), "in_proj_a (BF16)")
+        # single BF16 matvecs: routing gate and shared-expert gate score
+        Wg = F.bf16_trunc(rng.standard_normal((256, H)).astype(np.float32) * np.float32(0.05))
+        og = np.empty(256, np.float32)
+        for _ in range(2):    # second call hits the resident copy
+            ops.fast_dequant_matvec(Wg.ctypes.data, None, None, x.ctypes.data, og.ctypes.data, 256, H, 64, 0)
+            assert ops.finch_ops_last_status() == 0, ops.finch_ops_last_error()
+        assert_parity(og, orc.dequant_matvec(Wg, None, None, x, 256, H, 0), "mlp.gate (BF16)")
+        Ws = F.bf16_trunc(rng.standard_normal((1, H)).astype(np.float32))
+        os_ = np.empty(1, np.float32)
+        ops.fast_dequant_matvec(Ws.ctypes.data, None, None, x.ctypes.data, os_.ctypes.data, 1, H, 64, 0)
+        ref = orc.dequant_matvec(Ws, None, None, x, 1, H, 0)
+        assert abs(float(os_[0]) - float(ref[0])) <= 1e-3 * max(1.0, abs(float(ref[0])))
+        # a failing batch never leaves its outputs uninitialised (the call returns void)
+        bad = (BatchMatvecSpec * 1)(
+            BatchMatvecSpec(Wq.ctypes.data, Sq.ctypes.data, Bq.ctypes.data, oq.ctypes.data, 8192, H, 64, 0, 5))
+        oq[:] = np.nan
+        ops.fast_batch_matvec(x.ctypes.data, H, bad, 1)
+        assert ops.finch_ops_last_status() != 0 and np.all(oq == 0.0)
     finally:
         ops.finch_ops_shutdown()
