@@ -71,6 +71,7 @@ def load():
         "fm_moe_decode_dev": (i, [vp, i, vp, vp, vp, i, vp, vp, i]),
         "fm_moe_decode": (i, [vp, i, vp, vp, vp, i, vp, vp, i]),
         "fm_moe_decode_step_dev": (i, [vp, i, i, vp, vp, vp, i, vp, vp, i]),
+        "fm_moe_decode_step_noalloc_dev": (i, [vp, i, i, vp, vp, vp, i, vp, i]),
         "fm_moe_prefill_dev": (i, [vp, i, vp, vp, vp, i, i, vp, i]),
         "fm_moe_prefill": (i, [vp, i, vp, vp, vp, i, i, vp, i]),
         "fm_tensor_register": (i, [vp, vp, vp, vp, i, i, i, i, i, C.POINTER(i)]),
@@ -168,10 +169,10 @@ class FinchHip:
         self._chk(self.L.fm_kernel_timing_read(self.h, C.byref(a), C.byref(b), C.byref(n)))
         return a.value, b.value, n.value
 
-    # ---- affine expert store
     def stream_probe_dev(self, d_buf, nbytes):
         self._chk(self.L.fm_stream_probe_dev(self.h, d_buf, nbytes))
 
+    # ---- affine expert store
     def experts_config(self, n_layers, n_experts, hidden=2048, inter=512, group_size=64, bits=3,
                        scale_dtype=SCALE_BF16):
         self._chk(self.L.fm_experts_config(self.h, n_layers, n_experts, hidden, inter, group_size,
@@ -205,6 +206,10 @@ class FinchHip:
     def moe_decode_step_dev(self, layer0, n_layers, d_x, d_idx, d_w, K, d_out, d_eo=None, flags=0):
         self._chk(self.L.fm_moe_decode_step_dev(self.h, layer0, n_layers, d_x, d_idx, d_w, K,
                                                 d_out, d_eo, flags))
+
+    def moe_decode_step_noalloc_dev(self, layer0, n_layers, d_x, d_idx, d_w, K, d_out, flags=0):
+        self._chk(self.L.fm_moe_decode_step_noalloc_dev(self.h, layer0, n_layers, d_x, d_idx, d_w, K,
+                                                        d_out, flags))
 
     # ---- prefill
     def moe_prefill(self, layer, X, idx, w, flags=0, out=None):

@@ -6,6 +6,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -26,11 +27,11 @@ int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs, const FmExpertGe
                             int n_cu, hipStream_t st, hipEvent_t *kev);
 int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
                     const float *d_x, int M, int n_cu, hipStream_t st);
-int fm_launch_dequant_affine(const void *W, const void *S, const void *B, int out_dim,
 int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim, const float *d_x, int M,
                          hipStream_t st);
 int fm_launch_stream_probe(const void *d_buf, size_t nbytes, unsigned int *d_sink, int n_cu,
                            hipStream_t st);
+int fm_launch_dequant_affine(const void *W, const void *S, const void *B, int out_dim,
                              int in_dim, int group_size, int bits, int scale_fp16,
                              uint8_t *codes, float *w32, uint16_t *w16, hipStream_t st);
 int fm_launch_dequant_gguf(const void *W, int out_dim, int in_dim, int ggml_type, float *w32,
@@ -51,18 +52,45 @@ size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K);
 int fm_launch_layer_tail(const FmTailArgs *a, int bits, int scale_fp16, hipStream_t st);
 int fm_launch_route(const float *d_logits, int n, int K, const float *d_seg_score, int32_t *d_idx,
                     float *d_w, float *d_params, hipStream_t st);
+}
+
+// ---- scratch of the entry point that allocates nothing (fm_moe_decode_step_noalloc_dev) ----
+// One array per GPU, part of the library's device image, held until the process ends.  In
+// host code the array's name is only a handle for hipGetSymbolAddress: the address kernels
+// can use is looked up once per device (fm_ctx_create) and kept in g_noalloc_ptr.
+#define FM_NOALLOC_BYTES (4u << 20)
+static __device__ __align__(256) unsigned char fm_noalloc_scratch[FM_NOALLOC_BYTES];
+
+namespace {
+
+constexpr int FM_API_MAX_DEVICES = 64;
+unsigned char *g_noalloc_ptr[FM_API_MAX_DEVICES] = {};
+std::mutex g_noalloc_mutex;
+
+// with `device` current
+int noalloc_lookup(int device, unsigned char **out) {
+    *out = nullptr;
+    if (device < 0 || device >= FM_API_MAX_DEVICES) return FM_ERR_ARG;
+    std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+    if (!g_noalloc_ptr[device]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(fm_noalloc_scratch)) != hipSuccess || !p)
+            return FM_ERR_HIP;
+        g_noalloc_ptr[device] = (unsigned char *)p;
+    }
+    *out = g_noalloc_ptr[device];
+    return FM_OK;
+}
+
 // `bits` of a tensor registered without scales and biases: unquantized BF16 [out_dim][in_dim]
 // (cpu_dequant_matvec's scales == NULL branch, finchmoe/infer.m:1689-1701)
 constexpr int FM_BITS_RAW_BF16 = 16;
-
-}
-
-namespace {
 
 struct Tensor {
     bool used = false, owned = false;
     void *W = nullptr, *S = nullptr, *B = nullptr;
     int out_dim = 0, in_dim = 0, group_size = 0, bits = 0, scale_fp16 = 0;
+    bool raw_bf16() const { return bits == FM_BITS_RAW_BF16; }
 };
 
 struct LayerBuf {
@@ -90,7 +118,6 @@ struct fm_ctx {
     double k1_ms = 0.0, k2_ms = 0.0;
     int kcalls = 0;
     std::string err;
-    bool raw_bf16() const { return bits == FM_BITS_RAW_BF16; }
 
     // affine expert store
     bool aff_cfg = false;
@@ -118,6 +145,8 @@ struct fm_ctx {
     size_t ws_bytes = 0;
     // layer tail: one partial sum per workgroup, then the ticket counter
     float *d_tail = nullptr;
+    // this device's copy of fm_noalloc_scratch
+    unsigned char *noalloc = nullptr;
 
     std::vector<Tensor> tensors;
 };
@@ -282,6 +311,11 @@ extern "C" int fm_ctx_create(int device, fm_ctx **out) {
         return FM_ERR_NOMEM;
     }
     *c->h_err = 0u;
+    if (noalloc_lookup(device, &c->noalloc) != FM_OK) {
+        (void)hipHostFree(c->h_err);
+        delete c;
+        return FM_ERR_HIP;
+    }
     if (const char *e = getenv("FINCH_DECODE_SPLIT")) c->split_phases = e[0] == '1';
     *out = c;
     return FM_OK;
@@ -402,6 +436,16 @@ static int ktiming_collect(fm_ctx *c) {
     return check_grid_error(c);
 }
 
+extern "C" int fm_stream_probe_dev(fm_ctx *c, const void *d_buf, size_t nbytes) {
+    if (!c) return FM_ERR_ARG;
+    if (!d_buf || nbytes < 4096 || ((uintptr_t)d_buf & 15))
+        return fail(c, FM_ERR_ARG, "stream probe: a 16-byte aligned buffer of 4 KB or more");
+    DeviceGuard dg(c->device);
+    int rc = fm_launch_stream_probe(d_buf, nbytes, nullptr, c->n_cu, c->stream);
+    if (rc) return fail(c, rc, "stream probe launch failed: %s", hipGetErrorString(hipGetLastError()));
+    return FM_OK;
+}
+
 // ============================================================================
 // affine expert store
 // ============================================================================
@@ -436,16 +480,6 @@ extern "C" int fm_experts_config(fm_ctx *c, int n_layers, int n_experts, int hid
     g.n_experts = n_experts;
     // finchmoe/repack_experts.py:76-87, 141-151: W, scales, biases of gate, up, down
     uint64_t gu_w = (uint64_t)inter * hidden * bits / 8, gu_s = (uint64_t)inter * (hidden / 64) * 2;
-extern "C" int fm_stream_probe_dev(fm_ctx *c, const void *d_buf, size_t nbytes) {
-    if (!c) return FM_ERR_ARG;
-    if (!d_buf || nbytes < 4096 || ((uintptr_t)d_buf & 15))
-        return fail(c, FM_ERR_ARG, "stream probe: a 16-byte aligned buffer of 4 KB or more");
-    DeviceGuard dg(c->device);
-    int rc = fm_launch_stream_probe(d_buf, nbytes, nullptr, c->n_cu, c->stream);
-    if (rc) return fail(c, rc, "stream probe launch failed: %s", hipGetErrorString(hipGetLastError()));
-    return FM_OK;
-}
-
     uint64_t d_w = (uint64_t)hidden * inter * bits / 8, d_s = (uint64_t)hidden * (inter / 64) * 2;
     uint64_t o = 0;
     g.gate_w = (uint32_t)o; o += gu_w; g.gate_s = (uint32_t)o; o += gu_s; g.gate_b = (uint32_t)o; o += gu_s;
@@ -526,6 +560,49 @@ extern "C" int fm_moe_decode_dev(fm_ctx *c, int layer, const float *d_x, const i
                                  const float *d_w, int K, float *d_out, float *d_expert_out,
                                  int flags) {
     return fm_moe_decode_step_dev(c, layer, 1, d_x, d_idx, d_w, K, d_out, d_expert_out, flags);
+}
+
+// fm_moe_decode_step_dev for callers that must not allocate: the SwiGLU activations, the
+// per-expert vectors and one set of dependency counters live in this device's copy of
+// fm_noalloc_scratch instead of the context's growable buffers.  The array keeps the last
+// call's contents: the counters are cleared by a kernel in front of the operator (a fill
+// kernel, not a memset, so that the pair can be captured into a graph); the vectors are
+// fully rewritten before they are read.
+extern "C" int fm_moe_decode_step_noalloc_dev(fm_ctx *c, int layer0, int n_layers, const float *d_x,
+                                              const int32_t *d_idx, const float *d_w, int K,
+                                              float *d_out, int flags) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
+    if (!d_x || !d_idx || !d_w || !d_out) return fail(c, FM_ERR_ARG, "null pointer");
+    if (K < 1 || K > FM_MAX_K) return fail(c, FM_ERR_ARG, "K %d outside 1..%d", K, FM_MAX_K);
+    int rc = check_layers(c, c->layers, layer0, n_layers);
+    if (rc) return rc;
+    if (!c->noalloc) return fail(c, FM_ERR_STATE, "no scratch array on device %d", c->device);
+    // layout: act [n_layers][8][inter] | expert_out [n_layers][8][hidden] | counters
+    const size_t act_b = (size_t)n_layers * FM_MAX_K * c->geom.inter * sizeof(float);
+    const size_t eo_b = (size_t)n_layers * FM_MAX_K * c->geom.hidden * sizeof(float);
+    const size_t cnt_n = (size_t)n_layers * (FM_MAX_K + 1);
+    const size_t need = act_b + eo_b + cnt_n * sizeof(unsigned int);
+    if (need > FM_NOALLOC_BYTES)
+        return fail(c, FM_ERR_ARG,
+                    "%d layers of hidden %d / inter %d need %zu bytes of scratch, the fixed array "
+                    "holds %u (use fm_moe_decode_step_dev)", n_layers, c->geom.hidden, c->geom.inter,
+                    need, (unsigned)FM_NOALLOC_BYTES);
+    DeviceGuard dg(c->device);
+    unsigned char *s = c->noalloc;
+    FmDecodeFlags df{};
+    df.graph_set = (unsigned int *)(s + act_b + eo_b);
+    df.cap = (unsigned int)cnt_n;
+    df.err = c->d_err;
+    df.spin_limit = c->wait_limit;
+    df.always_graph_set = 1;
+    rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer0, 1, n_layers, d_x, d_idx, d_w,
+                                 K, (float *)s, (float *)(s + act_b), d_out,
+                                 c->split_phases ? nullptr : &df, flags, c->n_cu, c->stream,
+                                 nullptr);
+    if (rc) return fail(c, rc, "decode launch failed: %s", hipGetErrorString(hipGetLastError()));
+    if (!c->split_phases) c->sync_unchecked = true;
+    return FM_OK;
 }
 
 // host-pointer wrapper shared by the affine and GGUF stores and by decode
@@ -807,6 +884,13 @@ extern "C" int fm_matvec_prefill_batch_dev(fm_ctx *c, const fm_tensor *ts, int n
     if (M < 1 || M > 65535) return fail(c, FM_ERR_ARG, "M %d outside 1..65535", M);
     static const bool no_gemm = getenv("FINCH_DENSE_NO_GEMM") != nullptr;
     int prepared_bits = 0, prepared_in = 0;
+    for (int i = 0; i < n; i++) {   // one X for all: the tensors must agree on its width
+        Tensor *p = get_tensor(c, ts[i]), *p0 = get_tensor(c, ts[0]);
+        if (!p) return fail(c, FM_ERR_ARG, "bad tensor handle %d", ts[i]);
+        if (p->in_dim != p0->in_dim)
+            return fail(c, FM_ERR_ARG, "tensors of one batch must share in_dim (%d vs %d)", p->in_dim,
+                        p0->in_dim);
+    }
     for (int i = 0; i < n; i++) {
         Tensor *p = get_tensor(c, ts[i]);
         if (!d_outs[i]) return fail(c, FM_ERR_ARG, "null output %d", i);
@@ -857,6 +941,9 @@ static int matvec_host(fm_ctx *c, const fm_tensor *ts, int n, const float *x, fl
         Tensor *t = get_tensor(c, ts[i]);
         if (!t) return fail(c, FM_ERR_ARG, "bad tensor handle %d", ts[i]);
         if (!outs[i]) return fail(c, FM_ERR_ARG, "null output %d", i);
+        if (t->in_dim != t0->in_dim)   // the staging area holds one X of t0's width
+            return fail(c, FM_ERR_ARG, "tensors of one batch must share in_dim (%d vs %d)", t->in_dim,
+                        t0->in_dim);
         offs[i] = total;
         total += ((size_t)M * t->out_dim * 4 + 255) & ~(size_t)255;
     }
@@ -883,13 +970,6 @@ extern "C" int fm_matvec_batch(fm_ctx *c, const fm_tensor *ts, int n, const floa
     return matvec_host(c, ts, n, x, outs, 1);
 }
 
-    for (int i = 0; i < n; i++) {   // one X for all: the tensors must agree on its width
-        Tensor *p = get_tensor(c, ts[i]), *p0 = get_tensor(c, ts[0]);
-        if (!p) return fail(c, FM_ERR_ARG, "bad tensor handle %d", ts[i]);
-        if (p->in_dim != p0->in_dim)
-            return fail(c, FM_ERR_ARG, "tensors of one batch must share in_dim (%d vs %d)", p->in_dim,
-                        p0->in_dim);
-    }
 extern "C" int fm_matvec_prefill(fm_ctx *c, fm_tensor t, const float *X, float *out, int M) {
     if (!c) return FM_ERR_ARG;
     if (M < 1 || M > 65535) return fail(c, FM_ERR_ARG, "M %d outside 1..65535", M);
@@ -942,9 +1022,6 @@ extern "C" int fm_layer_tail_dev(fm_ctx *c, fm_tensor shared_down, const float *
         HIPCHK(c, hipMalloc((void **)&c->d_tail, (FM_TAIL_PARTIALS + 64) * sizeof(float)));
         HIPCHK(c, hipMemsetAsync(c->d_tail, 0, (FM_TAIL_PARTIALS + 64) * sizeof(float), c->stream));
     }
-        if (t->in_dim != t0->in_dim)   // the staging area holds one X of t0's width
-            return fail(c, FM_ERR_ARG, "tensors of one batch must share in_dim (%d vs %d)", t->in_dim,
-                        t0->in_dim);
     FmTailArgs a;
     a.W = (const uint8_t *)t->W;
     a.S = (const uint8_t *)t->S;
@@ -1023,6 +1100,14 @@ static int gguf_set_layer(fm_ctx *c, int layer, const void *gate, size_t gate_by
         return fail(c, FM_ERR_ARG, "layer %d", layer);
     if (adopt && (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)down) & 15))
         return fail(c, FM_ERR_ARG, "device slab not 16-byte aligned");
+    const FmGgufGeom &g = c->ggeom;
+    const size_t want[3] = {(size_t)g.n_experts * g.gate_slab, (size_t)g.n_experts * g.up_slab,
+                            (size_t)g.n_experts * g.down_slab};
+    const size_t have[3] = {gate_bytes, up_bytes, down_bytes};
+    for (int i = 0; i < 3; i++)
+        if (have[i] != want[i])
+            return fail(c, FM_ERR_ARG, "GGUF %s tensor is %zu bytes, expected %zu",
+                        i == 0 ? "gate" : i == 1 ? "up" : "down", have[i], want[i]);
     DeviceGuard dg(c->device);
     HIPCHK(c, hipStreamSynchronize(c->stream));
     if (!adopt) {
@@ -1124,14 +1209,6 @@ static int gguf_prefill_fn(fm_ctx *c, int layer, const float *x, const int32_t *
 
 extern "C" int fm_gguf_moe_decode(fm_ctx *c, int layer, const float *x, const int32_t *idx,
                                   const float *w, int K, float *out, float *expert_out, int flags) {
-    const FmGgufGeom &g = c->ggeom;
-    const size_t want[3] = {(size_t)g.n_experts * g.gate_slab, (size_t)g.n_experts * g.up_slab,
-                            (size_t)g.n_experts * g.down_slab};
-    const size_t have[3] = {gate_bytes, up_bytes, down_bytes};
-    for (int i = 0; i < 3; i++)
-        if (have[i] != want[i])
-            return fail(c, FM_ERR_ARG, "GGUF %s tensor is %zu bytes, expected %zu",
-                        i == 0 ? "gate" : i == 1 ? "up" : "down", have[i], want[i]);
     if (!c) return FM_ERR_ARG;
     if (!c->gguf_cfg) return fail(c, FM_ERR_STATE, "GGUF store not configured");
     return moe_host_call(c, gguf_decode_fn, c->ggeom.hidden, layer, x, idx, w, 1, K, out,
@@ -1219,6 +1296,7 @@ extern "C" int fm_dequant_tensor(fm_ctx *c, fm_tensor t, uint8_t *codes, float *
     if (!c) return FM_ERR_ARG;
     Tensor *p = get_tensor(c, t);
     if (!p) return fail(c, FM_ERR_ARG, "bad tensor handle %d", t);
+    if (p->raw_bf16()) return fail(c, FM_ERR_UNSUPPORTED, "tensor %d is raw BF16: nothing to dequantize", t);
     DeviceGuard dg(c->device);
     return dequant_common(c, p->W, p->S, p->B, p->out_dim, p->in_dim, p->bits, p->scale_fp16, 0,
                           codes, w_f32, w_f16);
@@ -1235,6 +1313,7 @@ extern "C" int fm_embed_lookup_dev(fm_ctx *c, fm_tensor t, const int32_t *d_toke
     if (!p) return fail(c, FM_ERR_ARG, "bad tensor handle %d", t);
     if (!d_token_ids || !d_out) return fail(c, FM_ERR_ARG, "null pointer");
     if (n_tokens < 1) return fail(c, FM_ERR_ARG, "n_tokens %d", n_tokens);
+    if (p->raw_bf16()) return fail(c, FM_ERR_UNSUPPORTED, "embedding lookup needs a quantized tensor");
     DeviceGuard dg(c->device);
     int rc = fm_launch_embed_rows(p->W, p->S, p->B, p->out_dim, p->in_dim, p->group_size, p->bits,
                                   p->scale_fp16, d_token_ids, n_tokens, d_out, c->stream);
@@ -1285,5 +1364,3 @@ extern "C" int fm_gguf_dequant_expert(fm_ctx *c, int layer, int expert, int whic
     }
     return dequant_common(c, base, nullptr, nullptr, rows, cols, 0, 0, type, nullptr, w_f32, nullptr);
 }
-    if (p->raw_bf16()) return fail(c, FM_ERR_UNSUPPORTED, "tensor %d is raw BF16: nothing to dequantize", t);
-    if (p->raw_bf16()) return fail(c, FM_ERR_UNSUPPORTED, "embedding lookup needs a quantized tensor");

@@ -32,6 +32,7 @@ struct FmDecodeFlags {
     int parity;
     unsigned int *err;
     unsigned int spin_limit;
+    int always_graph_set;   // count in graph_set behind a clearing kernel even when not capturing
 };
 
 // Geometry of the GGUF slabs of one layer (finchmoe/infer.m:1017-1022).

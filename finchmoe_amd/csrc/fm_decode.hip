@@ -895,8 +895,11 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     if (df && df->set[0]) (void)hipStreamIsCapturing(st, &capture);
     const bool captured = capture == hipStreamCaptureStatusActive;
-    if (df && df->set[0] && need <= df->cap) {
-        if (captured) {
+    // (the entry point that allocates nothing has one counter set only: it takes the graph's
+    // route whether or not the stream is capturing)
+    const bool own_clear = captured || (df && df->always_graph_set);
+    if (df && (df->set[0] || df->always_graph_set) && need <= df->cap) {
+        if (own_clear) {
             hipLaunchKernelGGL(fm_clear_counters, dim3((need + 255) / 256), dim3(256), 0, st,
                                df->graph_set, need);
             fl.cur = df->graph_set;
@@ -917,7 +920,7 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     if (g->bits == 3) rc = g->scale_fp16 ? FM_DEC(3, true) : FM_DEC(3, false);
     else if (g->bits == 4) rc = g->scale_fp16 ? FM_DEC(4, true) : FM_DEC(4, false);
 #undef FM_DEC
-    if (fused && !captured) {   // the set just used is dirty, the other one is clean again
+    if (fused && !own_clear) {   // the set just used is dirty, the other one is clean again
         df->used[df->parity] = need;
         df->used[df->parity ^ 1] = 0u;
         df->parity ^= 1;

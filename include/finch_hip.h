@@ -144,6 +144,19 @@ FM_API int fm_moe_decode_step_dev(fm_ctx *ctx, int layer0, int n_layers, const f
                            const int32_t *d_idx, const float *d_w, int K, float *d_out,
                            float *d_expert_out, int flags);
 
+/* fm_moe_decode_step_dev without a per-expert output, for callers that cannot allocate (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  It calls no hipMalloc / hipFree / allocating routine: the
+ * intermediate vectors and dependency counters live in a fixed 4 MiB array that is part of the
+ * library's device image (one copy per GPU, held until the process ends).  Limit:
+ *   n_layers * 8 * (hidden + inter) * 4 + n_layers * 9 * 4 bytes <= 4 MiB
+ * (40 layers at hidden 2048 / inter 512 need 3.13 MiB); larger calls return FM_ERR_ARG.
+ * Results are bit for bit those of fm_moe_decode_step_dev.  All contexts on one GPU share
+ * that GPU's array: calls that overlap on one GPU (two contexts, two streams) race. */
+FM_API int fm_moe_decode_step_noalloc_dev(fm_ctx *ctx, int layer0, int n_layers, const float *d_x,
+                                   const int32_t *d_idx, const float *d_w, int K, float *d_out,
+                                   int flags);
+
 /* ---------------------------------------------------------------- routed experts, chunked prefill
  * Replaces prefill_chunk_cmd3_encode / prefill_chunk_cmd3_batch_general
  * (finchmoe/infer.m:10704-11059): M positions, each with its own top-K.
