@@ -685,14 +685,20 @@ def run_prefill(args):
     idx = np.ascontiguousarray(idx.transpose(1, 0, 2))
     w = np.ascontiguousarray(w.transpose(1, 0, 2))
     d_idx, d_w = torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)
-    d_X = torch.randn(M, H, device=dev).to(torch.bfloat16).to(torch.float32)   # x ~ N(0,1) bf16
+    d_Xb = torch.randn(M, H, device=dev).to(torch.bfloat16)     # x ~ N(0,1) bf16
+    d_X = d_Xb.to(torch.float32)                                # the same values as fp32
     d_out = torch.empty(M, H, device=dev)
     torch.cuda.synchronize()
+    as_bf16 = args.x_dtype == "bf16"
 
     def step(t):
         l = t % nl
-        ctx.moe_prefill_dev(l, d_X.data_ptr(), d_idx.data_ptr() + l * M * K * 4,
-                            d_w.data_ptr() + l * M * K * 4, M, K, d_out.data_ptr())
+        if as_bf16:
+            ctx.moe_prefill_bf16_dev(l, d_Xb.data_ptr(), d_idx.data_ptr() + l * M * K * 4,
+                                     d_w.data_ptr() + l * M * K * 4, M, K, d_out.data_ptr())
+        else:
+            ctx.moe_prefill_dev(l, d_X.data_ptr(), d_idx.data_ptr() + l * M * K * 4,
+                                d_w.data_ptr() + l * M * K * 4, M, K, d_out.data_ptr())
 
     ms, ev = _timed(ctx, step, args)
     flops = M * K * 3 * 2 * H * I
@@ -702,8 +708,15 @@ def run_prefill(args):
            "unique_experts_per_chunk": uniq, "event_ms_per_step": round(ev, 5)}
     ctx.close()
     out = _finish(res, "chunked-prefill expert product, %d-position chunk" % M,
-                  "config 3: %d-token chunk, top-8 Zipf(1.1), %d-bit g64 experts (%s scales), x~N(0,1) bf16 values in fp32"
-                  % (M, bits, args.scale_dtype), int(uniq * es), ms, args, {"flops_per_step": flops})
+                  "config 3: %d-token chunk, top-8 Zipf(1.1), %d-bit g64 experts (%s scales), x~N(0,1) bf16%s"
+                  % (M, bits, args.scale_dtype, "" if as_bf16 else " values handed over as fp32"),
+                  int(uniq * es), ms, args, {"flops_per_step": flops, "x_dtype": args.x_dtype})
+    out["dtype"] = "bf16" if as_bf16 else "f32"
+    out["roofline"] = {"bound": "hbm", "kernel": "fm_pf_rows (gate/up + down launches of one chunk)",
+                       "achieved": round(uniq * es / (ev * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                       "frac": round(uniq * es / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                       "bytes_per_launch": int(uniq * es), "us_per_launch": round(ev * 1e3, 2),
+                       "mfma_frac_of_bf16_peak": round(flops / (ev * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
     return out
 
 
@@ -765,6 +778,8 @@ def main():
     ap.add_argument("--scale-dtype", default="bf16", choices=("bf16", "fp16"),
                     help="type of the group scales and biases (decode_step and prefill workloads)")
     ap.add_argument("--chunk", type=int, default=512, help="positions per chunk (prefill workload)")
+    ap.add_argument("--x-dtype", default="bf16", choices=("bf16", "f32"),
+                    help="prefill workload: hand the activations over as bf16 bits (config 3) or as fp32")
     ap.add_argument("--ramp-seconds", type=float, default=0.5,
                     help="untimed busy period before the warmup steps (clock ramp)")
     ap.add_argument("--graph", action="store_true",

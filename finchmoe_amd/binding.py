@@ -74,6 +74,8 @@ def load():
         "fm_moe_decode_step_noalloc_dev": (i, [vp, i, i, vp, vp, vp, i, vp, i]),
         "fm_moe_prefill_dev": (i, [vp, i, vp, vp, vp, i, i, vp, i]),
         "fm_moe_prefill": (i, [vp, i, vp, vp, vp, i, i, vp, i]),
+        "fm_moe_prefill_bf16_dev": (i, [vp, i, vp, vp, vp, i, i, vp, i]),
+        "fm_moe_prefill_bf16": (i, [vp, i, vp, vp, vp, i, i, vp, i]),
         "fm_tensor_register": (i, [vp, vp, vp, vp, i, i, i, i, i, C.POINTER(i)]),
         "fm_tensor_adopt": (i, [vp, vp, vp, vp, i, i, i, i, i, C.POINTER(i)]),
         "fm_tensor_release": (i, [vp, i]),
@@ -223,6 +225,19 @@ class FinchHip:
 
     def moe_prefill_dev(self, layer, d_X, d_idx, d_w, M, K, d_out, flags=0):
         self._chk(self.L.fm_moe_prefill_dev(self.h, layer, d_X, d_idx, d_w, M, K, d_out, flags))
+
+    def moe_prefill_bf16(self, layer, X_bits, idx, w, flags=0, out=None):
+        """X_bits: uint16 [M, hidden], the bfloat16 bit patterns of the activations."""
+        X, idx, w = _np(X_bits, np.uint16), _np(idx, np.int32), _np(w, np.float32)
+        M, K = idx.shape
+        if out is None:
+            out = np.zeros((M, self.hidden), np.float32)
+        self._chk(self.L.fm_moe_prefill_bf16(self.h, layer, _ptr(X), _ptr(idx), _ptr(w), M, K,
+                                             _ptr(out), flags))
+        return out
+
+    def moe_prefill_bf16_dev(self, layer, d_X, d_idx, d_w, M, K, d_out, flags=0):
+        self._chk(self.L.fm_moe_prefill_bf16_dev(self.h, layer, d_X, d_idx, d_w, M, K, d_out, flags))
 
     # ---- dense tensors
     def tensor_register(self, W, S, B, out_dim, in_dim, bits=4, group_size=64,

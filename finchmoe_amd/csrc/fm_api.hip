@@ -44,11 +44,12 @@ int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t *const *d_
                           int flags, int n_cu, hipStream_t st, hipEvent_t *kev);
 int fm_launch_gguf_matvec(const uint8_t *d_W, int ggml_type, const float *d_x, float *d_out,
                           int out_dim, int in_dim, int n_cu, hipStream_t st);
-int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGeom *g, const float *d_X,
-                             const int32_t *d_idx, const float *d_w, int M, int K,
+int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGeom *g, const void *d_X,
+                             int x_bf16, const int32_t *d_idx, const float *d_w, int M, int K,
                              float *d_out, void *d_ws, size_t ws_bytes, int flags, int n_cu,
                              hipStream_t st);
-size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K);
+size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K, int x_bf16);
+int fm_launch_widen_bf16(const uint16_t *d_src, float *d_dst, size_t n, hipStream_t st);
 int fm_launch_layer_tail(const FmTailArgs *a, int bits, int scale_fp16, hipStream_t st);
 int fm_launch_route(const float *d_logits, int n, int K, const float *d_seg_score, int32_t *d_idx,
                     float *d_w, float *d_params, hipStream_t st);
@@ -610,15 +611,18 @@ extern "C" int fm_moe_decode_step_noalloc_dev(fm_ctx *c, int layer0, int n_layer
 typedef int (*moe_dev_fn)(fm_ctx *, int, const float *, const int32_t *, const float *, int, int,
                           float *, float *, int);
 
-static int moe_host_call(fm_ctx *c, moe_dev_fn fn, int hidden, int layer, const float *x,
+// (x_elem: bytes per activation of x — 4 for fp32, 2 for bf16 bits; fn gets the staged x as
+// a float pointer either way and knows what it holds)
+static int moe_host_call(fm_ctx *c, moe_dev_fn fn, int hidden, int layer, const void *x,
                          const int32_t *idx, const float *w, int M, int K, float *out,
-                         float *expert_out, int flags) {
+                         float *expert_out, int flags, size_t x_elem = 4) {
     if (!x || !idx || !w || !out) return fail(c, FM_ERR_ARG, "null pointer");
     if (M < 1) return fail(c, FM_ERR_ARG, "M %d", M);
     if (K < 1 || K > FM_MAX_K) return fail(c, FM_ERR_ARG, "K %d outside 1..%d", K, FM_MAX_K);
     DeviceGuard dg(c->device);
     size_t nx = (size_t)M * hidden * 4, ni = (size_t)M * K * 4, ne = (size_t)M * K * hidden * 4;
-    size_t off_x = 0, off_i = off_x + nx, off_w = off_i + ((ni + 255) & ~(size_t)255);
+    const size_t nxi = (size_t)M * hidden * x_elem;
+    size_t off_x = 0, off_i = off_x + ((nxi + 255) & ~(size_t)255), off_w = off_i + ((ni + 255) & ~(size_t)255);
     size_t off_o = off_w + ((ni + 255) & ~(size_t)255), off_e = off_o + nx;
     int rc = ensure_stage(c, off_e + (expert_out ? ne : 0));
     if (rc) return rc;
@@ -630,7 +634,7 @@ static int moe_host_call(fm_ctx *c, moe_dev_fn fn, int hidden, int layer, const 
     // tenant of the GPU), the call is repeated once as separate kernels, which wait for nothing.
     const bool split_before = c->split_phases;
     for (int attempt = 0; attempt < 2; attempt++) {
-        memcpy(hs + off_x, x, nx);
+        memcpy(hs + off_x, x, nxi);
         memcpy(hs + off_i, idx, ni);
         memcpy(hs + off_w, w, ni);
         size_t in_bytes = off_w + ni;
@@ -677,8 +681,8 @@ extern "C" int fm_moe_decode(fm_ctx *c, int layer, const float *x, const int32_t
 // (grid-batched); larger chunks are grouped by expert for the MFMA GEMM.
 #define FM_PREFILL_GEMM_MIN_M 32
 
-extern "C" int fm_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, const int32_t *d_idx,
-                                  const float *d_w, int M, int K, float *d_out, int flags) {
+static int moe_prefill_any(fm_ctx *c, int layer, const void *d_X, bool x_bf16, const int32_t *d_idx,
+                           const float *d_w, int M, int K, float *d_out, int flags) {
     if (!c) return FM_ERR_ARG;
     if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
     if (!d_X || !d_idx || !d_w || !d_out) return fail(c, FM_ERR_ARG, "null pointer");
@@ -690,11 +694,11 @@ extern "C" int fm_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, const 
     if (rc) return rc;
     DeviceGuard dg(c->device);
     if (M >= FM_PREFILL_GEMM_MIN_M && !(flags & FM_GUARD)) {
-        size_t ws = fm_prefill_affine_ws_bytes(&c->geom, M, K);
+        size_t ws = fm_prefill_affine_ws_bytes(&c->geom, M, K, x_bf16);
         if (ws) {
             rc = ensure_ws(c, ws);
             if (rc) return rc;
-            rc = fm_launch_prefill_affine((const uint8_t *)c->layers[layer].ptr, &c->geom, d_X,
+            rc = fm_launch_prefill_affine((const uint8_t *)c->layers[layer].ptr, &c->geom, d_X, x_bf16,
                                           d_idx, d_w, M, K, d_out, c->d_ws, c->ws_bytes, flags,
                                           c->n_cu, c->stream);
             if (rc != FM_ERR_UNSUPPORTED) {
@@ -704,14 +708,35 @@ extern "C" int fm_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, const 
             }
         }
     }
+    // one decode group per position (small chunks, guarded calls, widths without a GEMM); the
+    // decode kernels read fp32: bf16 activations are widened into the workspace first
+    const float *xf = (const float *)d_X;
+    if (x_bf16) {
+        const size_t nx = (size_t)M * c->geom.hidden;
+        rc = ensure_ws(c, nx * sizeof(float));
+        if (rc) return rc;
+        rc = fm_launch_widen_bf16((const uint16_t *)d_X, (float *)c->d_ws, nx, c->stream);
+        if (rc) return fail(c, rc, "widening launch failed: %s", hipGetErrorString(hipGetLastError()));
+        xf = (const float *)c->d_ws;
+    }
     rc = ensure_scratch(c, M, c->geom.hidden, c->geom.inter);
     if (rc) return rc;
-    rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer, 0, M, d_X, d_idx, d_w, K,
+    rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer, 0, M, xf, d_idx, d_w, K,
                                  c->d_act, c->d_eo, d_out, c->split_phases ? nullptr : &c->dflags,
                                  flags, c->n_cu, c->stream, nullptr);
     if (rc) return fail(c, rc, "prefill launch failed: %s", hipGetErrorString(hipGetLastError()));
     if (!c->split_phases) c->sync_unchecked = true;
     return FM_OK;
+}
+
+extern "C" int fm_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, const int32_t *d_idx,
+                                  const float *d_w, int M, int K, float *d_out, int flags) {
+    return moe_prefill_any(c, layer, d_X, false, d_idx, d_w, M, K, d_out, flags);
+}
+
+extern "C" int fm_moe_prefill_bf16_dev(fm_ctx *c, int layer, const uint16_t *d_X, const int32_t *d_idx,
+                                       const float *d_w, int M, int K, float *d_out, int flags) {
+    return moe_prefill_any(c, layer, d_X, true, d_idx, d_w, M, K, d_out, flags);
 }
 
 static int aff_prefill_fn(fm_ctx *c, int layer, const float *x, const int32_t *idx,
@@ -725,6 +750,19 @@ extern "C" int fm_moe_prefill(fm_ctx *c, int layer, const float *X, const int32_
     if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
     return moe_host_call(c, aff_prefill_fn, c->geom.hidden, layer, X, idx, w, M, K, out, nullptr,
                          flags);
+}
+
+static int aff_prefill_bf16_fn(fm_ctx *c, int layer, const float *x, const int32_t *idx,
+                               const float *w, int M, int K, float *out, float *, int flags) {
+    return fm_moe_prefill_bf16_dev(c, layer, (const uint16_t *)x, idx, w, M, K, out, flags);
+}
+
+extern "C" int fm_moe_prefill_bf16(fm_ctx *c, int layer, const uint16_t *X, const int32_t *idx,
+                                   const float *w, int M, int K, float *out, int flags) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
+    return moe_host_call(c, aff_prefill_bf16_fn, c->geom.hidden, layer, X, idx, w, M, K, out, nullptr,
+                         flags, 2);
 }
 
 // ============================================================================

@@ -38,6 +38,8 @@
 #include "fm_mfma.h"
 #include "fm_ring.h"
 
+#include <type_traits>
+
 namespace {
 
 typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
@@ -71,6 +73,12 @@ struct PfArgs {
     ptrdiff_t d_s, d_b;
     int d_rows, d_cols, d_pass, d_flags;
     float *d_out;
+    // row-tile kernels (fm_pf_rows): X as bf16 bits when the caller has them, the two item
+    // lists (gate/up and down may cut an expert's positions into items of different size)
+    const uint16_t *Xbf;
+    PfItem *items_up, *items_dn;
+    int *n_items_up, *n_items_dn;
+    int tm_up, tm_dn;
 };
 
 enum { PF_GATE_UP = 0, PF_DOWN = 1, PF_DENSE = 2, PF_DENSE_TEAMS = 3 };
@@ -827,6 +835,683 @@ __global__ __launch_bounds__(1024) void fm_pf_dense_prep(PfArgs a) {
     if (threadIdx.x == 0) *a.n_items = n;
 }
 
+// ======================================================================
+// Row-tile kernels (fm_pf_rows): the expert products of a chunk.
+//
+// A wave owns 32 weight rows over the WHOLE K dimension, so a row tile is summed
+// inside one accumulator and nothing is exchanged between waves: no partial tiles
+// in LDS, no barrier per step.  What the waves of a workgroup share instead is the
+// activation operand of the current item, kept in LDS in MFMA register form (the
+// "image"), staged once per item.
+//
+//   item       (expert, up to 16 of its positions; 8 when the gate/up activations
+//              arrive as fp32: two bf16 pieces per value, in two M rows)
+//   task       32 weight rows of an item against all its positions: gate/up = 16
+//              gate rows + the same 16 up rows (SwiGLU needs both, and they meet in
+//              one lane), down = 32 rows
+//   slab       256 columns (four quantization groups) of a task's rows = one ring
+//              slot of 32 x 96 (128) code bytes, copied with LDS-direct loads; a task
+//              is 8 (gate/up) or 2 (down) slabs
+//   round      8 consecutive tasks of an item, one per wave; a workgroup takes a
+//              contiguous run of rounds of the chunk (every workgroup the same number
+//              within one), so every wave streams the same number of bytes and the
+//              waves meet again exactly where the item — the image — changes
+//
+// MFMA geometry.  V_MFMA_F32_16X16X32_BF16: positions on M (16), weight rows on N
+// (16: the task's rows are two N tiles), one product covers half a quantization
+// group (32 columns).  Lane (n, kb) holds, of weight row n, the 16 codes 16 kb ..
+// 16 kb + 15 of each group — 6 bytes (8 for 4-bit codes) — and supplies k slots
+// 8 kb .. 8 kb + 7 of both products of the group; codes c and c + 4 share a register
+// as bf16 values 1 + q * 2^t / 128 (fm_mfma.h; 3-bit: t = 4 and 0, one mask for all
+// pairs).  Each (tile, group) has its own accumulator of four registers and gets its
+// scale in fp32.  fp32 activations are two bf16 pieces: along K (two products on one
+// accumulator: the down product), or in M rows p and p + 8 (gate/up on fp32 X; the two
+// halves of the result are added at the end).  Bias and offset terms of a slab's four
+// groups are one more product per tile whose 32 k slots are (term, piece, group).
+//
+// What bounds these kernels is the number of cache-line requests of the LDS-direct
+// loads, not their bytes: a slab is 32 runs of 96 bytes, 768 bytes apart.  Measured on
+// the 512-position benchmark chunk (gate/up kernel): 101 us with the slab's scales and
+// biases fetched per slot (8 bytes per row, 64 bytes apart: as many line requests as
+// the codes), 82 us without them, 73 us with no loads at all — while taking out the
+// unpack arithmetic, the products or the image reads changes nothing.  Hence gate/up
+// keeps a task's scales and biases in registers, fetched as four contiguous KB.
+// ======================================================================
+enum { PFR_GATE_UP = 0, PFR_DOWN = 1 };
+
+template <int MODE, int BITS, int QK>
+struct PfRows {
+    static constexpr int S = MODE == PFR_GATE_UP ? 8 : 2;          // slabs of a task (K / 256)
+    static constexpr int CB = 8 * BITS * 4;                        // code bytes of a row inside a slab
+    static constexpr int RP = CB / 16;                             // 16-byte pieces per row
+    static constexpr int NQ = 32 * RP / 64;                        // LDS-direct loads for the codes
+    static constexpr int CODE = 32 * CB;
+    // gate/up keeps the scales and biases of a task in registers (SREG): its rows have 32
+    // groups, so a slab's 8 bytes per row are 64 bytes apart; a task's 16 rows x 64 bytes are
+    // one contiguous KB instead.  down (8 groups per row) fetches them with every slot.
+    static constexpr bool SREG = MODE == PFR_GATE_UP;
+    static constexpr int SLOT = CODE + (SREG ? 0 : 512);           // + scales 256 + biases 256
+    static constexpr int LOADS = NQ + (SREG ? 0 : 2);
+    static constexpr int OPB = 1024;                               // one operand of the image: 64 lanes x 16 B
+    static constexpr int SLAB_IMG = 4 * 2 * QK * OPB;              // [group][k step][piece]
+    static constexpr int IMG = S * SLAB_IMG;
+    static constexpr int SIDE = S * OPB;
+    static constexpr int RING_ROOM = (160 * 1024 - 2048 - IMG - SIDE) / (8 * SLOT);
+    static constexpr int RING = RING_ROOM > 4 ? 4 : RING_ROOM;
+    static constexpr int LDS_BYTES = 8 * RING * SLOT + IMG + SIDE;
+    static_assert(RING >= 2, "a ring needs a slot in flight beside the one being multiplied");
+    static_assert(IMG <= 65536, "image offsets are 16-bit immediates");
+};
+
+// mantissa positions of the two codes of a pair (low / high half of the register) and the
+// power of two each position costs the activation
+template <int BITS> struct PfrPair;
+template <> struct PfrPair<3> {
+    static constexpr uint32_t MASK = (7u << 4) | (7u << 16);
+    static constexpr float FL = 8.0f, FH = 128.0f;
+};
+template <> struct PfrPair<4> {
+    static constexpr uint32_t MASK = 0x000F000Fu;
+    static constexpr float FL = 128.0f, FH = 128.0f;
+};
+
+// One k step of a group of 64 activations as operand registers: register i holds columns
+// c0 + i (low half) and c0 + i + 4 (high half), scaled; hi (and, TWO, lo) bf16 piece.
+// xs / xo collect what the bias and offset terms multiply.
+template <int BITS, bool TWO>
+__device__ __forceinline__ void pfr_stage_op(const float *x, int c0, uint4 &hi, uint4 &lo, float &xs, float &xo) {
+    uint32_t h[4], l[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        constexpr float cl = PfrPair<BITS>::FL, ch = PfrPair<BITS>::FH;
+        const float vl = x[c0 + i] * cl, vh = x[c0 + i + 4] * ch;
+        const uint32_t l0 = __float_as_uint(vl) & 0xFFFF0000u, h0 = __float_as_uint(vh) & 0xFFFF0000u;
+        h[i] = (l0 >> 16) | h0;
+        float tl = __uint_as_float(l0), th = __uint_as_float(h0);
+        l[i] = 0u;
+        if constexpr (TWO) {
+            const float rl = vl - tl, rh = vh - th;
+            const uint32_t l1 = __float_as_uint(rl) & 0xFFFF0000u, h1 = __float_as_uint(rh) & 0xFFFF0000u;
+            l[i] = (l1 >> 16) | h1;
+            tl += __uint_as_float(l1);
+            th += __uint_as_float(h1);
+        }
+        xo += tl + th;
+        xs += tl * (1.0f / cl) + th * (1.0f / ch);
+    }
+    hi = make_uint4(h[0], h[1], h[2], h[3]);
+    lo = make_uint4(l[0], l[1], l[2], l[3]);
+}
+
+// 64 consecutive activations of one position as floats: bf16 bits or fp32
+template <bool XBF16>
+__device__ __forceinline__ void pfr_load64(const void *row, int col0, bool on, float *x) {
+    if constexpr (XBF16) {
+        const uint4 *p = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(row) + col0);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint4 v = on ? p[i] : make_uint4(0u, 0u, 0u, 0u);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                x[8 * i + 2 * k] = __uint_as_float(w[k] << 16);
+                x[8 * i + 2 * k + 1] = __uint_as_float(w[k] & 0xFFFF0000u);
+            }
+        }
+    } else {
+        const float4 *p = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(row) + col0);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float4 v = on ? p[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
+        }
+    }
+}
+
+// a dword of two 16-bit scales (biases) as MFMA operand halves: BF16 bits are operands as
+// they are; an FP16 value (11 significant bits) is split exactly into a bf16 head and tail
+template <bool FP16>
+__device__ __forceinline__ void pfr_head_tail(uint32_t w, uint32_t &head, uint32_t &tail) {
+    if constexpr (!FP16) {
+        head = w;
+        tail = 0u;
+    } else {
+        const float f0 = fm_fp16_bits(w & 0xFFFFu), f1 = fm_fp16_bits(w >> 16);
+        const uint32_t h0 = __float_as_uint(f0) & 0xFFFF0000u, h1 = __float_as_uint(f1) & 0xFFFF0000u;
+        const uint32_t t0 = __float_as_uint(f0 - __uint_as_float(h0)), t1 = __float_as_uint(f1 - __uint_as_float(h1));
+        head = (h0 >> 16) | h1;
+        tail = (t0 >> 16) | (t1 & 0xFFFF0000u);
+    }
+}
+
+typedef uint32_t pfr_u4 __attribute__((ext_vector_type(4)));
+typedef float pfr_f4 __attribute__((ext_vector_type(4)));
+
+// XBF16: gate/up reads X as bf16 bits; otherwise fp32 activations: gate/up puts their two
+// pieces in M rows p / p + 8 (8 positions per item), down along K (QK = 2)
+template <int MODE, int BITS, bool FP16, bool XBF16>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fm_pf_rows(PfArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr bool GU = MODE == PFR_GATE_UP;
+    constexpr int QK = GU ? 1 : 2;
+    constexpr bool ROWP = GU && !XBF16;                 // the two pieces in M rows
+    constexpr int TM = ROWP ? 8 : 16;
+    using P = PfRows<MODE, BITS, QK>;
+    constexpr int S = P::S, RING = P::RING;
+    extern __shared__ __attribute__((aligned(16))) uint8_t pfr_smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = lane & 15, kb = lane >> 4;
+    const uint32_t lds0 = fm_lds_addr(pfr_smem);
+    const uint32_t ring0 = lds0 + (uint32_t)wave * (RING * P::SLOT);
+    uint8_t *img_mem = pfr_smem + 8 * RING * P::SLOT;
+    uint8_t *side_mem = img_mem + P::IMG;
+    const uint32_t img0 = lds0 + 8 * RING * P::SLOT, side0 = img0 + P::IMG;
+    const int in_dim = GU ? a.g.hidden : a.g.inter, out_rows = GU ? a.g.inter : a.g.hidden;
+    const int row_bytes = in_dim * BITS / 8, sb_bytes = (in_dim / 64) * 2;
+    const PfItem *items = GU ? a.items_up : a.items_dn;
+    const int n_items = *(GU ? a.n_items_up : a.n_items_dn);
+    const int RPI = out_rows / (GU ? 16 : 32) / 8;      // rounds per item
+    const uint32_t ones = fm_opaque(0x3F803F80u);
+
+    // ---- this workgroup's rounds [R0, R1).  Workgroups are dealt out to the eight XCDs in
+    // turn and every XCD has an L2 of its own: workgroup b takes share (b % 8) * (grid / 8) +
+    // b / 8, so that neighbouring shares — the rounds of one expert — run behind one L2.
+    const long RT = (long)n_items * RPI;
+    const unsigned int share = gridDim.x % 8u == 0u ? (blockIdx.x % 8u) * (gridDim.x / 8u) + blockIdx.x / 8u
+                                                    : blockIdx.x;
+    const int R0 = (int)(RT * share / gridDim.x), R1 = (int)(RT * (share + 1) / gridDim.x);
+    if (R0 >= R1) return;
+    const int it0 = R0 / RPI;
+    // the items the share touches, one per lane (the launcher sizes the grid so that a share
+    // spans at most 64 items): expert, first sorted position, number of positions
+    const int it_last = (R1 - 1) / RPI;
+    int ev = 0, ev_start = 0, ev_count = 0;
+    if (it0 + lane <= it_last) {
+        const PfItem d = items[it0 + lane];
+        ev = d.expert, ev_start = d.start, ev_count = d.count;
+    }
+    // What staging an item needs from memory besides the activations themselves is fetched one
+    // item ahead: this thread's staging task is (group st_g, position st_pos), and st_pair is
+    // the pair id of that position (gate/up: its row of X is st_pair / K; down: threads 0-15
+    // publish the ids for the output addresses).
+    constexpr int NG = S * 4;
+    const int st_pos = threadIdx.x % TM, st_g = threadIdx.x / TM;
+    const bool st_has = threadIdx.x < TM * NG;
+    __shared__ int pairs_tab[16];
+    int st_pair = 0;
+    if (st_has && st_pos < __builtin_amdgcn_readlane(ev_count, 0))
+        st_pair = a.sorted[__builtin_amdgcn_readlane(ev_start, 0) + st_pos];
+
+    // ---- this lane's pieces of a slot copy
+    // codes: piece q = 64 j + lane of the slot = 16 bytes of row q / RP (the slot keeps the
+    // rows back to back).  gate/up: slot rows 0-15 = gate rows, 16-31 = the same rows of up
+    uint32_t coff[P::NQ];
+#pragma unroll
+    for (int j = 0; j < P::NQ; j++) {
+        const int q = 64 * j + lane, rr = q / P::RP, pc = q - rr * P::RP;
+        const uint32_t mat = GU ? (rr < 16 ? a.g.gate_w : a.g.up_w) : a.g.down_w;
+        coff[j] = mat + (uint32_t)((GU ? (rr & 15) : rr) * row_bytes + 16 * pc);
+    }
+    // scales / biases fetched with the slot (down): 8 bytes per row and slab, one dword per lane
+    uint32_t soff, boff;
+    {
+        const int rr = lane >> 1;
+        const uint32_t r = (uint32_t)((GU ? (rr & 15) : rr) * sb_bytes + 4 * (lane & 1));
+        soff = (GU ? (rr < 16 ? a.g.gate_s : a.g.up_s) : a.g.down_s) + r;
+        boff = (GU ? (rr < 16 ? a.g.gate_b : a.g.up_b) : a.g.down_b) + r;
+    }
+
+    // ---- loader: the slabs of this wave's tasks, in order
+    int l_r = R0, l_s = 0, wpos = 0;
+    uint32_t issued = 0, consumed = 0;
+    const uint8_t *l_w = nullptr, *l_sb = nullptr;
+    // SREG: scales and biases of the task the loader has entered, requested with four loads of
+    // one contiguous KB each — lane (n, kb) gets the 16 bytes (eight groups) 16 kb of its rows —
+    // in front of the task's first slot: once that slot has landed, so have they.  nsc: the
+    // task being loaded, csc: the task being multiplied; [tile 0 s, tile 0 b, tile 1 s, tile 1 b].
+    pfr_u4 nsc[4], csc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) nsc[i] = csc[i] = pfr_u4{0u, 0u, 0u, 0u};
+    const uint32_t sc_lane = (uint32_t)(n * sb_bytes + 16 * kb);
+    int sc_round = R0;            // the round nsc was requested for
+    auto loader_enter = [&]() __attribute__((always_inline)) {
+        const int it = l_r / RPI, t = (l_r - it * RPI) * 8 + wave;
+        const int e = __builtin_amdgcn_readlane(ev, it - it0);
+        const uint8_t *blob = a.layer + (size_t)e * a.g.expert_size;
+        const size_t r0 = (size_t)t * (GU ? 16 : 32);
+        l_w = fm_uniform(blob + r0 * row_bytes);
+        l_sb = fm_uniform(blob + r0 * sb_bytes);
+        if constexpr (P::SREG) {
+            const uint8_t *p0 = l_sb + a.g.gate_s, *p1 = l_sb + a.g.gate_b, *p2 = l_sb + a.g.up_s, *p3 = l_sb + a.g.up_b;
+            asm volatile("global_load_dwordx4 %0, %4, %5\n\tglobal_load_dwordx4 %1, %4, %6\n\t"
+                         "global_load_dwordx4 %2, %4, %7\n\tglobal_load_dwordx4 %3, %4, %8"
+                         : "=&v"(nsc[0]), "=&v"(nsc[1]), "=&v"(nsc[2]), "=&v"(nsc[3])
+                         : "v"(sc_lane), "s"(p0), "s"(p1), "s"(p2), "s"(p3)
+                         : "memory");
+            sc_round = l_r;
+        }
+    };
+    loader_enter();
+    auto issue = [&]() __attribute__((always_inline)) {
+        if (l_r >= R1) return;
+        const uint32_t slot = ring0 + (uint32_t)wpos * P::SLOT;
+        const uint8_t *wb = l_w + (size_t)l_s * P::CB, *sb = l_sb + (size_t)l_s * 8;
+#pragma unroll
+        for (int j = 0; j < P::NQ; j++)
+            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(wb + coff[j]),
+                                             (fm_lptr)(uintptr_t)(slot + 1024 * j), 16, 0, 0);
+        if constexpr (!P::SREG) {
+            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(sb + soff),
+                                             (fm_lptr)(uintptr_t)(slot + P::CODE), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(sb + boff),
+                                             (fm_lptr)(uintptr_t)(slot + P::CODE + 256), 4, 0, 0);
+        }
+        wpos = wpos + 1 == RING ? 0 : wpos + 1;
+        issued++;
+        if (++l_s == S) {
+            l_s = 0;
+            if (++l_r < R1) loader_enter();
+        }
+    };
+#pragma unroll
+    for (int k = 0; k < RING; k++) issue();
+
+    // ---- addresses of this lane inside a slot, the image and the side operands
+    // 3-bit: its 6 bytes of a (row, group) are read as the two aligned dwords around them
+    // and shifted down by 16 bits in the odd lanes
+    const uint32_t code_lane = BITS == 3 ? (uint32_t)(n * P::CB + 12 * (kb >> 1) + 4 * (kb & 1))
+                                         : (uint32_t)(n * P::CB + 8 * kb);
+    const uint32_t sh3 = 16u * (uint32_t)(kb & 1);
+    const uint32_t img_lane = img0 + 16u * (uint32_t)lane, side_lane = side0 + 16u * (uint32_t)lane;
+    // rows 8-15 of the side operands stay zero when the pieces sit in M rows
+    if constexpr (ROWP)
+        for (int i = threadIdx.x; i < P::SIDE / 16; i += blockDim.x)
+            reinterpret_cast<uint4 *>(side_mem)[i] = make_uint4(0u, 0u, 0u, 0u);
+
+    // block BLK of a slab's image operands (eight of them, in [group][k step][piece] order)
+    auto img_read = [&](uint32_t addr, pfr_u4 *buf, auto blk) __attribute__((always_inline)) {
+        constexpr int O = decltype(blk)::value * 8 * P::OPB;
+        asm volatile(
+            "ds_read_b128 %0, %8 offset:%9\n\tds_read_b128 %1, %8 offset:%10\n\t"
+            "ds_read_b128 %2, %8 offset:%11\n\tds_read_b128 %3, %8 offset:%12\n\t"
+            "ds_read_b128 %4, %8 offset:%13\n\tds_read_b128 %5, %8 offset:%14\n\t"
+            "ds_read_b128 %6, %8 offset:%15\n\tds_read_b128 %7, %8 offset:%16"
+            : "=&v"(buf[0]), "=&v"(buf[1]), "=&v"(buf[2]), "=&v"(buf[3]), "=&v"(buf[4]), "=&v"(buf[5]),
+              "=&v"(buf[6]), "=&v"(buf[7])
+            : "v"(addr), "n"(O), "n"(O + P::OPB), "n"(O + 2 * P::OPB), "n"(O + 3 * P::OPB),
+              "n"(O + 4 * P::OPB), "n"(O + 5 * P::OPB), "n"(O + 6 * P::OPB), "n"(O + 7 * P::OPB)
+            : "memory");
+    };
+    auto lgkm_wait = [&](pfr_u4 *buf) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(buf[0]), "+v"(buf[1]), "+v"(buf[2]), "+v"(buf[3]), "+v"(buf[4]), "+v"(buf[5]),
+                       "+v"(buf[6]), "+v"(buf[7])
+                     :
+                     : "memory");
+    };
+
+    int c = 0, cur_item = -1;
+    PfItem item = PfItem{0, 0, 0, 0};
+    uint32_t oidx[4];                  // output element offset of result register i, ~0u = no store
+#pragma unroll
+    for (int i = 0; i < 4; i++) oidx[i] = ~0u;
+
+    for (int r = R0; r < R1; r++) {
+        const int it = r / RPI;
+        if (it != cur_item) {
+            // ---- the workgroup moves to another item: stage its activations
+            cur_item = it;
+            item.expert = __builtin_amdgcn_readlane(ev, it - it0);
+            item.start = __builtin_amdgcn_readlane(ev_start, it - it0);
+            item.count = __builtin_amdgcn_readlane(ev_count, it - it0);
+            // the activations are requested before the barrier: their addresses are known
+            const bool on = st_has && st_pos < item.count;
+            const size_t m = !on ? 0 : GU ? (size_t)(st_pair / a.K) : (size_t)(item.start + st_pos);
+            float x[64];
+            if constexpr (GU && XBF16) pfr_load64<true>(a.Xbf + m * in_dim, 64 * st_g, on, x);
+            else pfr_load64<false>((GU ? a.X : a.act) + m * in_dim, 64 * st_g, on, x);
+            const int my_pair = st_pair;
+            // (and the next item's pair ids behind them)
+            st_pair = 0;
+            if (it < it_last && st_has && st_pos < __builtin_amdgcn_readlane(ev_count, it + 1 - it0))
+                st_pair = a.sorted[__builtin_amdgcn_readlane(ev_start, it + 1 - it0) + st_pos];
+            __syncthreads();                                   // every wave is done with the old image
+            if (st_has) {
+                // task = (group, position), positions fastest: a wave covers whole slabs
+                const int sl = st_g >> 2, gi = st_g & 3;
+                uint8_t *dst = img_mem + (size_t)sl * P::SLAB_IMG + (size_t)gi * 2 * QK * P::OPB + 16 * st_pos;
+                float xs = 0.0f, xo = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        uint4 hi, lo;
+                        pfr_stage_op<BITS, !XBF16 || !GU>(x, 16 * k + 8 * j, hi, lo, xs, xo);
+                        uint8_t *d = dst + (size_t)j * QK * P::OPB + 256 * k;       // lane 16 k + position
+                        *reinterpret_cast<uint4 *>(d) = hi;
+                        if constexpr (QK == 2) *reinterpret_cast<uint4 *>(d + P::OPB) = lo;
+                        if constexpr (ROWP) *reinterpret_cast<uint4 *>(d + 16 * 8) = lo;       // M row 8 + position
+                    }
+                // bias / offset operands of (slab, position): the four groups' sums sit in the
+                // lanes TM apart; the lane of group gi builds the operand of k block gi: piece gi
+                // (k block 3: piece 0 once more, against the tails of FP16 scales) of
+                // (xsum g0 g1, xsum g2 g3, -xoff g0 g1, -xoff g2 g3)
+                uint32_t pc[8][3];
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const int from = lane + (k - gi) * TM;
+                    pf_pieces(__shfl(xs, from), pc[k]);
+                    pf_pieces(-__shfl(xo, from), pc[4 + k]);
+                }
+                const int pi = gi < 3 ? gi : 0;
+                uint32_t sel[8];
+#pragma unroll
+                for (int k = 0; k < 8; k++) sel[k] = pi == 0 ? pc[k][0] : pi == 1 ? pc[k][1] : pc[k][2];
+                const uint4 sv = make_uint4(sel[0] | (sel[1] << 16), sel[2] | (sel[3] << 16),
+                                            sel[4] | (sel[5] << 16), sel[6] | (sel[7] << 16));
+                *reinterpret_cast<uint4 *>(side_mem + (size_t)sl * P::OPB + 16 * (16 * gi + st_pos)) = sv;
+                if (!GU && st_g == 0) pairs_tab[st_pos] = my_pair;
+            }
+            __syncthreads();                                   // the image is complete
+            // where this lane's results go: register i = position 4 * (lane / 16) + i
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int tok = (ROWP ? 4 * (kb & 1) : 4 * kb) + i;
+                oidx[i] = ~0u;
+                if (tok < item.count)
+                    oidx[i] = GU ? (uint32_t)(item.start + tok) * (uint32_t)a.g.inter
+                                 : (uint32_t)pairs_tab[tok] * (uint32_t)a.g.hidden;
+            }
+        }
+        const int t = (r - it * RPI) * 8 + wave;               // this wave's task of the round
+
+        pfr_f4 acc[2], side[2];
+#pragma unroll
+        for (int T = 0; T < 2; T++) acc[T] = pfr_f4{0.0f, 0.0f, 0.0f, 0.0f}, side[T] = pfr_f4{0.0f, 0.0f, 0.0f, 0.0f};
+
+        for (int s = 0; s < S; s++) {
+            const uint32_t ia = img_lane + (uint32_t)s * P::SLAB_IMG;
+            // image operands and the bias/offset operand: they depend on nothing
+            pfr_u4 abuf[QK][8], sA;
+            img_read(ia, abuf[0], std::integral_constant<int, 0>());
+            {
+                const uint32_t sa = side_lane + (uint32_t)s * P::OPB;
+                asm volatile("ds_read_b128 %0, %1" : "=&v"(sA) : "v"(sa) : "memory");
+            }
+            if constexpr (QK == 2) img_read(ia, abuf[1], std::integral_constant<int, 1>());
+            // ---- the oldest slot of the ring.  SREG: once the loader has entered the next task,
+            // that task's four scale loads are in flight too, behind every slot of this one
+            if (issued - consumed != (uint32_t)RING) fm_dma_wait<0>(true);
+            else if (P::SREG && sc_round > r) fm_dma_wait<P::LOADS *(RING - 1) + 4>(false);
+            else fm_dma_wait<P::LOADS *(RING - 1)>(false);
+            const uint32_t slot = ring0 + (uint32_t)c * P::SLOT;
+            uint32_t d0[2][4], d1[2][4], sw[2][2], bw[2][2];     // [tile][group] codes, [tile][dword] scales
+            const uint32_t a0 = slot + code_lane, a1 = a0 + 16 * P::CB;
+            uint2 q[2][4];
+            if constexpr (P::SREG) {
+                if (s == 0) {          // the task's first slot is there, and so are its scales
+#pragma unroll
+                    for (int i = 0; i < 4; i++) csc[i] = nsc[i];
+                }
+                // the slab's four groups are one dword pair of the lanes kb = s / 2
+                const uint32_t src = 4u * (uint32_t)(n + 16 * (s >> 1));
+                const bool hi = s & 1;
+                uint32_t v[8], o[8];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    v[2 * i] = hi ? csc[i][2] : csc[i][0];
+                    v[2 * i + 1] = hi ? csc[i][3] : csc[i][1];
+                }
+                asm volatile("ds_bpermute_b32 %0, %8, %9\n\tds_bpermute_b32 %1, %8, %10\n\t"
+                             "ds_bpermute_b32 %2, %8, %11\n\tds_bpermute_b32 %3, %8, %12\n\t"
+                             "ds_bpermute_b32 %4, %8, %13\n\tds_bpermute_b32 %5, %8, %14\n\t"
+                             "ds_bpermute_b32 %6, %8, %15\n\tds_bpermute_b32 %7, %8, %16"
+                             : "=&v"(o[0]), "=&v"(o[1]), "=&v"(o[2]), "=&v"(o[3]), "=&v"(o[4]), "=&v"(o[5]),
+                               "=&v"(o[6]), "=&v"(o[7])
+                             : "v"(src), "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]),
+                               "v"(v[7])
+                             : "memory");
+                if constexpr (BITS == 3) {
+                    asm volatile(
+                        "ds_read2_b32 %0, %8 offset0:0 offset1:1\n\tds_read2_b32 %1, %8 offset0:6 offset1:7\n\t"
+                        "ds_read2_b32 %2, %8 offset0:12 offset1:13\n\tds_read2_b32 %3, %8 offset0:18 offset1:19\n\t"
+                        "ds_read2_b32 %4, %9 offset0:0 offset1:1\n\tds_read2_b32 %5, %9 offset0:6 offset1:7\n\t"
+                        "ds_read2_b32 %6, %9 offset0:12 offset1:13\n\tds_read2_b32 %7, %9 offset0:18 offset1:19\n\t"
+                        "s_waitcnt lgkmcnt(0)"
+                        : "=&v"(q[0][0]), "=&v"(q[0][1]), "=&v"(q[0][2]), "=&v"(q[0][3]), "=&v"(q[1][0]), "=&v"(q[1][1]),
+                          "=&v"(q[1][2]), "=&v"(q[1][3])
+                        : "v"(a0), "v"(a1)
+                        : "memory");
+                } else {
+                    asm volatile(
+                        "ds_read_b64 %0, %8\n\tds_read_b64 %1, %8 offset:32\n\t"
+                        "ds_read_b64 %2, %8 offset:64\n\tds_read_b64 %3, %8 offset:96\n\t"
+                        "ds_read_b64 %4, %9\n\tds_read_b64 %5, %9 offset:32\n\t"
+                        "ds_read_b64 %6, %9 offset:64\n\tds_read_b64 %7, %9 offset:96\n\t"
+                        "s_waitcnt lgkmcnt(0)"
+                        : "=&v"(q[0][0]), "=&v"(q[0][1]), "=&v"(q[0][2]), "=&v"(q[0][3]), "=&v"(q[1][0]), "=&v"(q[1][1]),
+                          "=&v"(q[1][2]), "=&v"(q[1][3])
+                        : "v"(a0), "v"(a1)
+                        : "memory");
+                }
+                asm volatile("" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]), "+v"(o[4]), "+v"(o[5]), "+v"(o[6]),
+                             "+v"(o[7]));
+#pragma unroll
+                for (int T = 0; T < 2; T++)
+                    sw[T][0] = o[4 * T], sw[T][1] = o[4 * T + 1], bw[T][0] = o[4 * T + 2], bw[T][1] = o[4 * T + 3];
+            } else {
+                const uint32_t as = slot + P::CODE + 8 * n;
+                uint2 sq[2], bq[2];
+                if constexpr (BITS == 3) {
+                    asm volatile(
+                        "ds_read2_b32 %0, %12 offset0:0 offset1:1\n\tds_read2_b32 %1, %12 offset0:6 offset1:7\n\t"
+                        "ds_read2_b32 %2, %12 offset0:12 offset1:13\n\tds_read2_b32 %3, %12 offset0:18 offset1:19\n\t"
+                        "ds_read2_b32 %4, %13 offset0:0 offset1:1\n\tds_read2_b32 %5, %13 offset0:6 offset1:7\n\t"
+                        "ds_read2_b32 %6, %13 offset0:12 offset1:13\n\tds_read2_b32 %7, %13 offset0:18 offset1:19\n\t"
+                        "ds_read_b64 %8, %14\n\tds_read_b64 %9, %14 offset:128\n\t"
+                        "ds_read_b64 %10, %14 offset:256\n\tds_read_b64 %11, %14 offset:384\n\t"
+                        "s_waitcnt lgkmcnt(0)"
+                        : "=&v"(q[0][0]), "=&v"(q[0][1]), "=&v"(q[0][2]), "=&v"(q[0][3]), "=&v"(q[1][0]), "=&v"(q[1][1]),
+                          "=&v"(q[1][2]), "=&v"(q[1][3]), "=&v"(sq[0]), "=&v"(sq[1]), "=&v"(bq[0]), "=&v"(bq[1])
+                        : "v"(a0), "v"(a1), "v"(as)
+                        : "memory");
+                } else {
+                    asm volatile(
+                        "ds_read_b64 %0, %12\n\tds_read_b64 %1, %12 offset:32\n\t"
+                        "ds_read_b64 %2, %12 offset:64\n\tds_read_b64 %3, %12 offset:96\n\t"
+                        "ds_read_b64 %4, %13\n\tds_read_b64 %5, %13 offset:32\n\t"
+                        "ds_read_b64 %6, %13 offset:64\n\tds_read_b64 %7, %13 offset:96\n\t"
+                        "ds_read_b64 %8, %14\n\tds_read_b64 %9, %14 offset:128\n\t"
+                        "ds_read_b64 %10, %14 offset:256\n\tds_read_b64 %11, %14 offset:384\n\t"
+                        "s_waitcnt lgkmcnt(0)"
+                        : "=&v"(q[0][0]), "=&v"(q[0][1]), "=&v"(q[0][2]), "=&v"(q[0][3]), "=&v"(q[1][0]), "=&v"(q[1][1]),
+                          "=&v"(q[1][2]), "=&v"(q[1][3]), "=&v"(sq[0]), "=&v"(sq[1]), "=&v"(bq[0]), "=&v"(bq[1])
+                        : "v"(a0), "v"(a1), "v"(as)
+                        : "memory");
+                }
+#pragma unroll
+                for (int T = 0; T < 2; T++)
+                    sw[T][0] = sq[T].x, sw[T][1] = sq[T].y, bw[T][0] = bq[T].x, bw[T][1] = bq[T].y;
+            }
+#pragma unroll
+            for (int T = 0; T < 2; T++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) d0[T][g] = q[T][g].x, d1[T][g] = q[T][g].y;
+            consumed++;
+            c = c + 1 == RING ? 0 : c + 1;
+            issue();
+            // (that wait covered the image reads above as well)
+            lgkm_wait(abuf[0]);
+            if constexpr (QK == 2) lgkm_wait(abuf[1]);
+            asm volatile("" : "+v"(sA));
+
+            // ---- bias and offset terms of the slab's four groups, one product per tile
+#pragma unroll
+            for (int T = 0; T < 2; T++) {
+                uint32_t hb0, hb1, hs0, hs1, tb0, tb1, ts0, ts1;
+                pfr_head_tail<FP16>(bw[T][0], hb0, tb0);
+                pfr_head_tail<FP16>(bw[T][1], hb1, tb1);
+                pfr_head_tail<FP16>(sw[T][0], hs0, ts0);
+                pfr_head_tail<FP16>(sw[T][1], hs1, ts1);
+                const bool last = kb == 3;
+                const uint4 Bs = last ? make_uint4(tb0, tb1, ts0, ts1) : make_uint4(hb0, hb1, hs0, hs1);
+                side[T] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, sA), __builtin_bit_cast(bf8, Bs),
+                                                                  side[T], 0, 0, 0);
+                if constexpr (FP16) {
+                    // tails x piece 1 of both terms (k block 1 holds piece 1)
+                    const bool one = kb == 1;
+                    const uint4 A2 = one ? __builtin_bit_cast(uint4, sA) : make_uint4(0u, 0u, 0u, 0u);
+                    const uint4 B2 = one ? make_uint4(tb0, tb1, ts0, ts1) : make_uint4(0u, 0u, 0u, 0u);
+                    side[T] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, A2),
+                                                                      __builtin_bit_cast(bf8, B2), side[T], 0, 0, 0);
+                }
+            }
+
+            // ---- (tile, group): unpack this lane's 16 codes, two products per piece, scale
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                pfr_f4 D[2];
+#pragma unroll
+                for (int T = 0; T < 2; T++) {
+                    uint32_t op[8];
+                    if constexpr (BITS == 3) {
+                        const uint32_t q0 = __builtin_amdgcn_alignbit(d1[T][g], d0[T][g], sh3), q1 = d1[T][g] >> sh3;
+                        op[0] = ((q0 << 4) & PfrPair<3>::MASK) | ones;
+                        op[1] = ((q0 << 1) & PfrPair<3>::MASK) | ones;
+                        op[2] = ((q0 >> 2) & PfrPair<3>::MASK) | ones;
+                        op[3] = ((q0 >> 5) & PfrPair<3>::MASK) | ones;
+                        op[4] = (__builtin_amdgcn_alignbit(q1, q0, 20) & PfrPair<3>::MASK) | ones;
+                        op[5] = (__builtin_amdgcn_alignbit(q1, q0, 23) & PfrPair<3>::MASK) | ones;
+                        op[6] = (__builtin_amdgcn_alignbit(q1, q0, 26) & PfrPair<3>::MASK) | ones;
+                        op[7] = (__builtin_amdgcn_alignbit(q1, q0, 29) & PfrPair<3>::MASK) | ones;
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            op[i] = ((d0[T][g] >> (4 * i)) & PfrPair<4>::MASK) | ones;
+                            op[4 + i] = ((d1[T][g] >> (4 * i)) & PfrPair<4>::MASK) | ones;
+                        }
+                    }
+                    D[T] = pfr_f4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        const bf8 b = __builtin_bit_cast(bf8, make_uint4(op[4 * j], op[4 * j + 1], op[4 * j + 2], op[4 * j + 3]));
+#pragma unroll
+                        for (int qq = 0; qq < QK; qq++) {
+                            const int k = (g * 2 + j) * QK + qq;         // operand of the slab
+                            D[T] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, abuf[k / 8][k % 8]), b,
+                                                                           D[T], 0, 0, 0);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int T = 0; T < 2; T++) {
+                    const uint32_t w = sw[T][g >> 1];
+                    const float sc = (g & 1) ? fm_widen_hi<FP16>(w) : fm_widen_lo<FP16>(w);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc[T][i] = fmaf(sc, D[T][i], acc[T][i]);
+                }
+            }
+        }
+
+        // ---- the task's 32 rows x positions
+        const int r0 = t * (GU ? 16 : 32);
+        float val[2][4];
+#pragma unroll
+        for (int T = 0; T < 2; T++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                val[T][i] = acc[T][i] + side[T][i];
+                if constexpr (ROWP) {
+                    // M rows p (lanes 0-31) and p + 8 (lanes 32-63) hold the two pieces' results
+                    const uint32_t v = __float_as_uint(val[T][i]);
+                    const auto hl = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+                    val[T][i] = __uint_as_float(hl[0]) + __uint_as_float(hl[1]);
+                }
+            }
+        if constexpr (GU) {
+            // tile 0 = gate rows, tile 1 = the same rows of up, both in this lane
+            float *act = a.act + r0 + n;
+            const bool mine = !ROWP || kb < 2;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (mine && oidx[i] != ~0u) act[oidx[i]] = fm_silu_mul(val[0][i], val[1][i]);
+        } else {
+            float *eo = a.eo + r0 + n;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (oidx[i] != ~0u) {
+                    eo[oidx[i]] = val[0][i];
+                    eo[oidx[i] + 16] = val[1][i];
+                }
+        }
+    }
+#else
+    (void)a;
+#endif
+}
+
+// Pairs grouped by expert and cut into items, twice: items of tm_up positions for the gate/up
+// product and of tm_dn positions for the down product (the same grouping, `sorted`).  One
+// workgroup of 1024 threads, one expert per thread for the prefix sums.
+__global__ __launch_bounds__(1024) void fm_pf_group(PfArgs a) {
+    __shared__ int hist[PF_MAX_EXPERTS], cursor[PF_MAX_EXPERTS], scan_a[16], scan_b[16], scan_c[16];
+    const int E = a.g.n_experts, n = a.M * a.K, e = threadIdx.x;
+    hist[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < n; p += blockDim.x) {
+        int x = a.idx[p];
+        if ((unsigned)x < (unsigned)E) atomicAdd(&hist[x], 1);
+    }
+    __syncthreads();
+    const int cnt = e < E ? hist[e] : 0;
+    const int nu = (cnt + a.tm_up - 1) / a.tm_up, nd = (cnt + a.tm_dn - 1) / a.tm_dn;
+    // inclusive scans of the pair counts and of both item counts: inside each wave by lane
+    // shifts, the 16 wave totals by wave 0
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    int sa = cnt, sb = nu, sc = nd;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int va = __shfl_up(sa, d), vb = __shfl_up(sb, d), vc = __shfl_up(sc, d);
+        if (lane >= d) sa += va, sb += vb, sc += vc;
+    }
+    if (lane == 63) scan_a[wv] = sa, scan_b[wv] = sb, scan_c[wv] = sc;
+    __syncthreads();
+    if (wv == 0) {
+        int ta = lane < 16 ? scan_a[lane] : 0, tb = lane < 16 ? scan_b[lane] : 0, tc = lane < 16 ? scan_c[lane] : 0;
+#pragma unroll
+        for (int d = 1; d < 16; d <<= 1) {
+            const int va = __shfl_up(ta, d), vb = __shfl_up(tb, d), vc = __shfl_up(tc, d);
+            if (lane >= d) ta += va, tb += vb, tc += vc;
+        }
+        if (lane < 16) scan_a[lane] = ta, scan_b[lane] = tb, scan_c[lane] = tc;
+    }
+    __syncthreads();
+    if (wv > 0) sa += scan_a[wv - 1], sb += scan_b[wv - 1], sc += scan_c[wv - 1];
+    const int off = sa - cnt;
+    cursor[e] = off;
+    for (int s = 0; s < nu; s++) {
+        const int left = cnt - s * a.tm_up;
+        a.items_up[sb - nu + s] = PfItem{e, off + s * a.tm_up, left < a.tm_up ? left : a.tm_up, 0};
+    }
+    for (int s = 0; s < nd; s++) {
+        const int left = cnt - s * a.tm_dn;
+        a.items_dn[sc - nd + s] = PfItem{e, off + s * a.tm_dn, left < a.tm_dn ? left : a.tm_dn, 0};
+    }
+    if (e == 1023) *a.n_items_up = sb, *a.n_items_dn = sc;
+    __syncthreads();
+    for (int p = threadIdx.x; p < n; p += blockDim.x) {
+        int x = a.idx[p];
+        if ((unsigned)x < (unsigned)E) a.sorted[atomicAdd(&cursor[x], 1)] = p;
+    }
+}
+
+// bf16 bits -> fp32 (chunks that take the per-position path)
+__global__ __launch_bounds__(256) void fm_pf_widen(const uint16_t *src, float *dst, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = __uint_as_float((uint32_t)src[i] << 16);
+}
+
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 bool pf_supported(const FmExpertGeom *g) {
@@ -835,26 +1520,32 @@ bool pf_supported(const FmExpertGeom *g) {
            g->inter == 512;
 }
 
+// grid of a row-tile launch: one workgroup per CU, more when a share could span more than the
+// 64 items whose experts a workgroup keeps one per lane
+int pfr_grid(int max_items, int n_cu) {
+    const int need = (max_items + 31) / 32;
+    return need > n_cu ? need : n_cu;
+}
+
 template <int BITS, bool FP16>
 int pf_launch(const PfArgs &a, const FmExpertGeom *g, int M, float *d_out, int flags, int n_cu,
               hipStream_t st) {
     const size_t n = (size_t)M * a.K;
-    // workgroup 0 sorts, the rest turn X into operand registers (one thread per position,
-    // group and half)
-    const int prep_tasks = M * (g->hidden / 64) * 2;
-    hipLaunchKernelGGL(fm_pf_sort<BITS>, dim3(1 + (prep_tasks + 1023) / 1024), dim3(1024), 0, st, a);
-    const int max_items = g->n_experts + (int)(n / PF_TM);
-    // one 8-wave workgroup per CU (LDS: the ring and the partial tiles take all 160 KB; ~220-245
-    // registers per lane cap a SIMD at two waves)
-    const int grid = max_items < n_cu ? max_items : n_cu;
-    constexpr int LDS = PfSlab<BITS>::LDS_BYTES;
-    static FmLdsAttr attr_up, attr_down;
-    if (!fm_dyn_lds_ready(attr_up, (const void *)fm_pf_gemm<PF_GATE_UP, BITS, FP16>, LDS)) return FM_ERR_HIP;
-    if (!fm_dyn_lds_ready(attr_down, (const void *)fm_pf_gemm<PF_DOWN, BITS, FP16>, LDS)) return FM_ERR_HIP;
-    hipLaunchKernelGGL((fm_pf_gemm<PF_GATE_UP, BITS, FP16>), dim3(grid), dim3(512), LDS, st, a);
-    const int act_tasks = (int)n * (g->inter / 64) * 2;
-    hipLaunchKernelGGL(fm_pf_prepare_act<BITS>, dim3((act_tasks + 255) / 256), dim3(256), 0, st, a);
-    hipLaunchKernelGGL((fm_pf_gemm<PF_DOWN, BITS, FP16>), dim3(grid), dim3(512), LDS, st, a);
+    hipLaunchKernelGGL(fm_pf_group, dim3(1), dim3(1024), 0, st, a);
+    const int grid_up = pfr_grid(g->n_experts + (int)(n / a.tm_up), n_cu);
+    const int grid_dn = pfr_grid(g->n_experts + (int)(n / a.tm_dn), n_cu);
+#define PFR_LAUNCH(MODE, XB, GRID)                                                               \
+    do {                                                                                         \
+        auto kfn = fm_pf_rows<MODE, BITS, FP16, XB>;                                             \
+        constexpr int LDS = PfRows<MODE, BITS, MODE == PFR_GATE_UP ? 1 : 2>::LDS_BYTES;          \
+        static FmLdsAttr attr;                                                                   \
+        if (!fm_dyn_lds_ready(attr, (const void *)kfn, LDS)) return FM_ERR_HIP;                  \
+        hipLaunchKernelGGL(kfn, dim3(GRID), dim3(512), LDS, st, a);                              \
+    } while (0)
+    if (a.Xbf) PFR_LAUNCH(PFR_GATE_UP, true, grid_up);
+    else PFR_LAUNCH(PFR_GATE_UP, false, grid_up);
+    PFR_LAUNCH(PFR_DOWN, false, grid_dn);
+#undef PFR_LAUNCH
     hipLaunchKernelGGL(fm_pf_combine, dim3(M, (g->hidden + 1023) / 1024), dim3(256), 0, st, a, d_out, flags);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
@@ -936,42 +1627,44 @@ extern "C" int fm_launch_prefill_dense(const void *d_W, const void *d_S, const v
     return bits == 3 ? pf_launch_dense<3, false>(a, n_cu, prep, st) : pf_launch_dense<4, false>(a, n_cu, prep, st);
 }
 
-extern "C" size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K) {
+// positions per item of the two products: 16, or 8 for gate/up on fp32 activations
+static inline int pf_tm_up(int x_bf16) { return x_bf16 ? 16 : 8; }
+
+extern "C" size_t fm_prefill_affine_ws_bytes(const FmExpertGeom *g, int M, int K, int x_bf16) {
     if (!pf_supported(g)) return 0;
-    size_t n = (size_t)M * K;
-    return align256(n * 4) + align256((g->n_experts + n / PF_TM + 1) * sizeof(PfItem)) + 256 +
-           align256(n * g->inter * 4) + align256(n * g->hidden * 4) +
-           align256((size_t)M * (g->hidden / 64) * 16 * sizeof(uint4)) +
-           align256((size_t)M * (g->hidden / 64) * sizeof(float2)) +
-           align256(n * (g->inter / 64) * 16 * sizeof(uint4)) +
-           align256(n * (g->inter / 64) * sizeof(float2));
+    const size_t n = (size_t)M * K;
+    return align256(n * 4) + align256((g->n_experts + n / pf_tm_up(x_bf16) + 1) * sizeof(PfItem)) +
+           align256((g->n_experts + n / 16 + 1) * sizeof(PfItem)) + 256 + align256(n * g->inter * 4) +
+           align256(n * g->hidden * 4);
 }
 
+// d_X: fp32 [M][hidden], or bf16 bits [M][hidden] when x_bf16 is set
 extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGeom *g,
-                                        const float *d_X, const int32_t *d_idx, const float *d_w,
-                                        int M, int K, float *d_out, void *d_ws, size_t ws_bytes,
-                                        int flags, int n_cu, hipStream_t st) {
+                                        const void *d_X, int x_bf16, const int32_t *d_idx,
+                                        const float *d_w, int M, int K, float *d_out, void *d_ws,
+                                        size_t ws_bytes, int flags, int n_cu, hipStream_t st) {
     if (!pf_supported(g)) return FM_ERR_UNSUPPORTED;
-    if (ws_bytes < fm_prefill_affine_ws_bytes(g, M, K)) return FM_ERR_ARG;
+    if (ws_bytes < fm_prefill_affine_ws_bytes(g, M, K, x_bf16)) return FM_ERR_ARG;
     const size_t n = (size_t)M * K;
     char *ws = (char *)d_ws;
-    PfArgs a;
+    PfArgs a{};
     a.layer = d_layer;
     a.g = *g;
-    a.X = d_X;
+    a.X = x_bf16 ? nullptr : (const float *)d_X;
+    a.Xbf = x_bf16 ? (const uint16_t *)d_X : nullptr;
     a.idx = d_idx;
     a.w = d_w;
     a.M = M;
     a.K = K;
+    a.tm_up = pf_tm_up(x_bf16);
+    a.tm_dn = 16;
     a.sorted = (int *)ws;                 ws += align256(n * 4);
-    a.items = (PfItem *)ws;               ws += align256((g->n_experts + n / PF_TM + 1) * sizeof(PfItem));
-    a.n_items = (int *)ws;                ws += 256;
+    a.items_up = (PfItem *)ws;            ws += align256((g->n_experts + n / a.tm_up + 1) * sizeof(PfItem));
+    a.items_dn = (PfItem *)ws;            ws += align256((g->n_experts + n / a.tm_dn + 1) * sizeof(PfItem));
+    a.n_items_up = (int *)ws;
+    a.n_items_dn = (int *)ws + 1;         ws += 256;
     a.act = (float *)ws;                  ws += align256(n * g->inter * 4);
-    a.eo = (float *)ws;                   ws += align256(n * g->hidden * 4);
-    a.xop = (uint4 *)ws;                  ws += align256((size_t)M * (g->hidden / 64) * 16 * sizeof(uint4));
-    a.xsums = (float2 *)ws;               ws += align256((size_t)M * (g->hidden / 64) * sizeof(float2));
-    a.aop = (uint4 *)ws;                  ws += align256(n * (g->inter / 64) * 16 * sizeof(uint4));
-    a.asums = (float2 *)ws;
+    a.eo = (float *)ws;
     if (g->scale_fp16)
         return g->bits == 3 ? pf_launch<3, true>(a, g, M, d_out, flags, n_cu, st)
                             : pf_launch<4, true>(a, g, M, d_out, flags, n_cu, st);
@@ -979,3 +1672,7 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
                         : pf_launch<4, false>(a, g, M, d_out, flags, n_cu, st);
 }
 
+extern "C" int fm_launch_widen_bf16(const uint16_t *d_src, float *d_dst, size_t n, hipStream_t st) {
+    hipLaunchKernelGGL(fm_pf_widen, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, d_src, d_dst, n);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}

@@ -167,6 +167,15 @@ FM_API int fm_moe_prefill_dev(fm_ctx *ctx, int layer, const float *d_X, const in
                        const float *d_w, int M, int K, float *d_out, int flags);
 FM_API int fm_moe_prefill(fm_ctx *ctx, int layer, const float *X, const int32_t *idx,
                    const float *w, int M, int K, float *out, int flags);
+/* the same chunk with the activations as bfloat16 bits, X[M][hidden] uint16 (a prefill chunk
+ * of bf16 hidden states; the widening to fp32 the reference's callers do before
+ * prefill_chunk_cmd3_encode, finchmoe/infer.m:10704, is skipped).  Result contract: what
+ * fm_moe_prefill gives on the widened X.  From 32 positions on this is the fast form of the
+ * grouped product: a bf16 value is one matrix-core operand, an fp32 value two. */
+FM_API int fm_moe_prefill_bf16_dev(fm_ctx *ctx, int layer, const uint16_t *d_X, const int32_t *d_idx,
+                            const float *d_w, int M, int K, float *d_out, int flags);
+FM_API int fm_moe_prefill_bf16(fm_ctx *ctx, int layer, const uint16_t *X, const int32_t *idx,
+                        const float *w, int M, int K, float *out, int flags);
 
 /* ---------------------------------------------------------------- dense affine tensors
  * Replaces fast_dequant_matvec / BatchMatvecSpec + fast_batch_matvec /

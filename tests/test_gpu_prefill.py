@@ -86,3 +86,45 @@ def test_small_chunks_and_guard_use_position_path(pstore, orc):
         for m in range(0, M, 7):
             single, _ = ctx.moe_decode(0, X[m], idx[m], w[m], flags=flags)
             assert np.array_equal(out[m], single)
+
+
+@pytest.mark.parametrize("M,K", [(64, 8), (37, 5), (200, 8)])
+def test_bf16_activation_entry(pstore, orc, M, K):
+    """fm_moe_prefill_bf16: X as bfloat16 bits.  Contract: the fp32 entry on the widened X —
+    checked against the oracle on the widened X (the parity bar) and against the fp32 entry
+    (both are the same mathematics; they differ by fp32 summation order only)."""
+    ctx, blob, (bits, sd) = pstore
+    rng = np.random.default_rng(M + K)
+    Xb = F.bf16_trunc(rng.standard_normal((M, H)).astype(np.float32))
+    Xf = F.bf16_to_f32(Xb)
+    idx, w = _routing(orc, rng, M, K)
+    out = ctx.moe_prefill_bf16(0, Xb, idx, w)
+    for m in range(0, M, max(1, M // 12)):
+        ref, _ = orc.moe_experts_forward(blob, Xf[m], idx[m], w[m], H, I, bits, scale_dtype=sd, nthreads=8)
+        assert_parity(out[m], ref, "bf16 entry, position %d" % m)
+    wide = ctx.moe_prefill(0, Xf, idx, w)
+    assert rel_err(out, wide) < 1e-4 and cosine(out, wide) > 0.9999999
+    assert np.array_equal(ctx.moe_prefill_bf16(0, Xb, idx, w), out)
+    # accumulate flag and an out-of-range index
+    idx2 = idx.copy()
+    idx2[3, 0] = -5
+    base = rng.standard_normal((M, H)).astype(np.float32)
+    acc = ctx.moe_prefill_bf16(0, Xb, idx2, w, flags=fb.ACCUMULATE, out=base.copy())
+    plain = ctx.moe_prefill_bf16(0, Xb, idx2, w)
+    assert rel_err(acc - base, plain) < 1e-5
+    keep = [k for k in range(K) if 0 <= idx2[3, k] < E]
+    ref, _ = orc.moe_experts_forward(blob, Xf[3], idx2[3, keep], w[3, keep], H, I, bits, scale_dtype=sd, nthreads=8)
+    assert_parity(plain[3], ref, "invalid slot dropped")
+
+
+def test_bf16_entry_small_chunk_is_the_position_path(pstore, orc):
+    """Below the GEMM threshold the bf16 entry widens X and runs per-position decode: bitwise
+    the fp32 entry on the widened X."""
+    ctx, blob, (bits, sd) = pstore
+    rng = np.random.default_rng(77)
+    M, K = 8, 8
+    Xb = F.bf16_trunc(rng.standard_normal((M, H)).astype(np.float32))
+    idx, w = _routing(orc, rng, M, K)
+    a = ctx.moe_prefill_bf16(0, Xb, idx, w)
+    b = ctx.moe_prefill(0, F.bf16_to_f32(Xb), idx, w)
+    assert np.array_equal(a, b)
