@@ -63,7 +63,7 @@ def load():
         "fm_kernel_timing": (i, [vp, i]),
         "fm_set_wait_limit": (i, [vp, C.c_uint]),
         "fm_kernel_timing_read": (i, [vp, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i)]),
-        "fm_stream_probe_dev": (i, [vp, vp, sz]),
+        "fm_stream_probe_dev": (i, [vp, vp, sz, i]),
         "fm_experts_config": (i, [vp, i, i, i, i, i, i, i]),
         "fm_experts_expert_size": (sz, [vp]),
         "fm_experts_upload_layer": (i, [vp, i, vp, sz]),
@@ -171,8 +171,8 @@ class FinchHip:
         self._chk(self.L.fm_kernel_timing_read(self.h, C.byref(a), C.byref(b), C.byref(n)))
         return a.value, b.value, n.value
 
-    def stream_probe_dev(self, d_buf, nbytes):
-        self._chk(self.L.fm_stream_probe_dev(self.h, d_buf, nbytes))
+    def stream_probe_dev(self, d_buf, nbytes, pattern=0):
+        self._chk(self.L.fm_stream_probe_dev(self.h, d_buf, nbytes, pattern))
 
     # ---- affine expert store
     def experts_config(self, n_layers, n_experts, hidden=2048, inter=512, group_size=64, bits=3,

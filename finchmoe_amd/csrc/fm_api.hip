@@ -29,8 +29,8 @@ int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_f
                     const float *d_x, int M, int n_cu, hipStream_t st);
 int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim, const float *d_x, int M,
                          hipStream_t st);
-int fm_launch_stream_probe(const void *d_buf, size_t nbytes, unsigned int *d_sink, int n_cu,
-                           hipStream_t st);
+int fm_launch_stream_probe(const void *d_buf, size_t nbytes, int pattern, unsigned int *d_sink,
+                           int n_cu, hipStream_t st);
 int fm_launch_dequant_affine(const void *W, const void *S, const void *B, int out_dim,
                              int in_dim, int group_size, int bits, int scale_fp16,
                              uint8_t *codes, float *w32, uint16_t *w16, hipStream_t st);
@@ -437,12 +437,12 @@ static int ktiming_collect(fm_ctx *c) {
     return check_grid_error(c);
 }
 
-extern "C" int fm_stream_probe_dev(fm_ctx *c, const void *d_buf, size_t nbytes) {
+extern "C" int fm_stream_probe_dev(fm_ctx *c, const void *d_buf, size_t nbytes, int pattern) {
     if (!c) return FM_ERR_ARG;
-    if (!d_buf || nbytes < 4096 || ((uintptr_t)d_buf & 15))
-        return fail(c, FM_ERR_ARG, "stream probe: a 16-byte aligned buffer of 4 KB or more");
+    if (!d_buf || nbytes < 4096 || ((uintptr_t)d_buf & 15) || pattern < 0 || pattern > 2)
+        return fail(c, FM_ERR_ARG, "stream probe: a 16-byte aligned buffer of 4 KB or more, pattern 0..2");
     DeviceGuard dg(c->device);
-    int rc = fm_launch_stream_probe(d_buf, nbytes, nullptr, c->n_cu, c->stream);
+    int rc = fm_launch_stream_probe(d_buf, nbytes, pattern, nullptr, c->n_cu, c->stream);
     if (rc) return fail(c, rc, "stream probe launch failed: %s", hipGetErrorString(hipGetLastError()));
     return FM_OK;
 }

@@ -1,6 +1,7 @@
 // fm_probe.hip — the streaming ceiling of the memory system, measured the way the expert
 // kernels read: one workgroup of eight waves per CU, every wave a ring of 4 KB slots in LDS
-// filled with LDS-direct 16-byte loads over one contiguous share of a buffer, no arithmetic.
+// filled with LDS-direct 16-byte loads, no arithmetic; three orders in which the waves walk
+// the buffer (the rate depends on it).
 // What this kernel reaches is what a bandwidth-bound kernel of that structure can reach at
 // best; the decode kernels are priced against the published peak and compared with this.
 // No counterpart in the reference (a measurement aid, like its --timing accumulators,
@@ -15,25 +16,38 @@ constexpr int PROBE_SLOT = 4096;       // 4 loads of 64 lanes x 16 bytes
 
 extern __shared__ __attribute__((aligned(16))) uint8_t fm_probe_lds[];
 
+// PATTERN: which 4 KB slots a wave reads, in order
+//   0  dense: slot i of the buffer goes to wave i % (all waves of the grid) — at any moment the
+//      chip reads one contiguous window
+//   1  every workgroup a contiguous share, its eight waves interleaved over it (the order of
+//      the expert decode kernels)
+//   2  every wave a contiguous share
+template <int PATTERN>
 __global__ __launch_bounds__(PROBE_WAVES * 64) void fm_stream_probe_k(const uint8_t *buf, size_t n_slots,
                                                                       unsigned int *sink) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t ring0 = fm_lds_addr(fm_probe_lds) + (uint32_t)wave * (PROBE_RING * PROBE_SLOT);
-    // this workgroup's contiguous share of the slots, its waves interleaved over it
-    const size_t s0 = n_slots * blockIdx.x / gridDim.x, s1 = n_slots * (blockIdx.x + 1) / gridDim.x;
-    size_t next = s0 + wave;
+    const size_t gw = (size_t)blockIdx.x * PROBE_WAVES + wave, nw = (size_t)gridDim.x * PROBE_WAVES;
+    size_t next, end, step;
+    if constexpr (PATTERN == 0) {
+        next = gw, end = n_slots, step = nw;
+    } else if constexpr (PATTERN == 1) {
+        next = n_slots * blockIdx.x / gridDim.x + wave, end = n_slots * (blockIdx.x + 1) / gridDim.x, step = PROBE_WAVES;
+    } else {
+        next = n_slots * gw / nw, end = n_slots * (gw + 1) / nw, step = 1;
+    }
     uint32_t issued = 0, consumed = 0;
     int wpos = 0, c = 0;
     auto issue = [&]() __attribute__((always_inline)) {
-        if (next >= s1) return;
+        if (next >= end) return;
         const uint8_t *src = fm_uniform(buf + next * PROBE_SLOT) + lane * 16;
         const uint32_t slot = ring0 + (uint32_t)wpos * PROBE_SLOT;
 #pragma unroll
         for (int j = 0; j < 4; j++)
             __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(src + 1024 * j),
                                              (fm_lptr)(uintptr_t)(slot + 1024 * j), 16, 0, 0);
-        next += PROBE_WAVES;
+        next += step;
         wpos = wpos + 1 == PROBE_RING ? 0 : wpos + 1;
         issued++;
     };
@@ -57,15 +71,20 @@ __global__ __launch_bounds__(PROBE_WAVES * 64) void fm_stream_probe_k(const uint
 
 }  // namespace
 
-// reads nbytes (rounded down to whole 4 KB slots) of d_buf once
-extern "C" int fm_launch_stream_probe(const void *d_buf, size_t nbytes, unsigned int *d_sink, int n_cu,
-                                      hipStream_t st) {
+// reads nbytes (rounded down to whole 4 KB slots) of d_buf once, in the given pattern
+extern "C" int fm_launch_stream_probe(const void *d_buf, size_t nbytes, int pattern, unsigned int *d_sink,
+                                      int n_cu, hipStream_t st) {
     const size_t n_slots = nbytes / PROBE_SLOT;
-    if (!d_buf || n_slots == 0 || ((uintptr_t)d_buf & 15)) return FM_ERR_ARG;
+    if (!d_buf || n_slots == 0 || ((uintptr_t)d_buf & 15) || pattern < 0 || pattern > 2) return FM_ERR_ARG;
     const size_t sh = (size_t)PROBE_WAVES * PROBE_RING * PROBE_SLOT;
-    static FmLdsAttr attr;
-    if (!fm_dyn_lds_ready(attr, (const void *)fm_stream_probe_k, sh)) return FM_ERR_HIP;
-    hipLaunchKernelGGL(fm_stream_probe_k, dim3(n_cu), dim3(PROBE_WAVES * 64), sh, st,
-                       (const uint8_t *)d_buf, n_slots, d_sink);
+    static FmLdsAttr attr[3];
+    const void *fn = pattern == 0 ? (const void *)fm_stream_probe_k<0>
+                   : pattern == 1 ? (const void *)fm_stream_probe_k<1> : (const void *)fm_stream_probe_k<2>;
+    if (!fm_dyn_lds_ready(attr[pattern], fn, sh)) return FM_ERR_HIP;
+    const dim3 grid(n_cu), block(PROBE_WAVES * 64);
+    const uint8_t *b = (const uint8_t *)d_buf;
+    if (pattern == 0) hipLaunchKernelGGL(fm_stream_probe_k<0>, grid, block, sh, st, b, n_slots, d_sink);
+    else if (pattern == 1) hipLaunchKernelGGL(fm_stream_probe_k<1>, grid, block, sh, st, b, n_slots, d_sink);
+    else hipLaunchKernelGGL(fm_stream_probe_k<2>, grid, block, sh, st, b, n_slots, d_sink);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }

@@ -105,10 +105,12 @@ FM_API int fm_kernel_timing_read(fm_ctx *ctx, double *gate_up_ms, double *down_m
 
 /* Streaming probe: reads nbytes (whole 4 KB slots) of the device buffer d_buf once, with the
  * access structure of the expert kernels (one workgroup of eight waves per CU, LDS-direct
- * 16-byte loads into a ring, contiguous shares) and no arithmetic; asynchronous on the
- * context's stream.  Timed with fm_timer_start/stop it gives the rate the memory system
- * delivers to a kernel of that structure.  No counterpart in the reference. */
-FM_API int fm_stream_probe_dev(fm_ctx *ctx, const void *d_buf, size_t nbytes);
+ * 16-byte loads into a ring) and no arithmetic; asynchronous on the context's stream.
+ * pattern: 0 = slots dealt out over all waves of the chip (one dense window at any moment),
+ * 1 = a contiguous share per workgroup, its waves interleaved (the decode kernels' order),
+ * 2 = a contiguous share per wave.  Timed with fm_timer_start/stop it gives the rate the
+ * memory system delivers to a kernel of that structure.  No counterpart in the reference. */
+FM_API int fm_stream_probe_dev(fm_ctx *ctx, const void *d_buf, size_t nbytes, int pattern);
 
 /* ---------------------------------------------------------------- expert store, affine
  * Replaces the packed-expert files + pread/LRU machinery
