@@ -56,11 +56,14 @@ def build(force=False, verbose=False, extra_flags=(), lib=None):
                 print(out)
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
         subprocess.check_call(cmd)
-    host_src = os.path.join(HERE, "host", "finch_ops.c")
-    if not lib and os.path.exists(host_src) and (force or _stale(HOSTLIB, [host_src, os.path.join(HERE, "host", "finch_ops.h")])):
-        subprocess.check_call(["gcc", "-O2", "-std=c99", "-fPIC", "-shared", "-Wall",
+    host = os.path.join(HERE, "host")
+    host_src = [os.path.join(host, f) for f in ("finch_ops.c", "finch_files.c")]
+    host_hdr = [os.path.join(HERE, "..", "include", f) for f in ("finch_hip.h", "finch_ops.h", "finch_files.h")]
+    if not lib and (force or _stale(HOSTLIB, host_src + host_hdr)):
+        # -ffp-contract=off: the quantizer reproduces fp32 array arithmetic operation by operation
+        subprocess.check_call(["gcc", "-O2", "-std=c99", "-ffp-contract=off", "-fPIC", "-shared", "-Wall",
                                "-I", os.path.join(HERE, "..", "include"),
-                               "-o", HOSTLIB, host_src, "-L", HERE, "-lfinchhip",
+                               "-o", HOSTLIB] + host_src + ["-L", HERE, "-lfinchhip", "-lm",
                                "-Wl,-rpath,$ORIGIN"])
     return LIB
 

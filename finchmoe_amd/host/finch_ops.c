@@ -118,6 +118,14 @@ int finch_ops_last_status(void) { return g_status; }
 const char *finch_ops_last_error(void) { return g_err; }
 void finch_ops_set_scale_dtype(int d) { g_scale_dtype = d; }
 
+int finch_ops_make_resident(const void *W, const uint16_t *scales, const uint16_t *biases,
+                            int out_dim, int in_dim, int group_size, int bits) {
+    if (!g_ctx) return fail(FM_ERR_STATE, "finch_ops_make_resident");
+    fm_tensor t;
+    int rc = resident(W, scales, biases, out_dim, in_dim, group_size, bits, &t);
+    return rc ? fail(rc, "finch_ops_make_resident") : FM_OK;
+}
+
 void finch_ops_forget_tensor(const void *W) {
     slot *s = g_tab ? tab_find(W, 0) : NULL;
     if (s && s->t >= 0) {

@@ -56,6 +56,9 @@ void fast_batch_matvec(const float *x, uint32_t x_dim, BatchMatvecSpec *specs, i
 void fast_prefill_matvec(const uint32_t *W, const uint16_t *scales, const uint16_t *biases,
                          const float *x, float *out, int out_dim, int in_dim, int group_size,
                          int bits, int M);
+/* upload a tensor now rather than on its first use (a loader's warm-up) */
+int finch_ops_make_resident(const void *W, const uint16_t *scales, const uint16_t *biases,
+                            int out_dim, int in_dim, int group_size, int bits);
 /* forget the HBM copy of a tensor whose host memory is about to be reused */
 void finch_ops_forget_tensor(const void *W);
 

@@ -32,6 +32,20 @@ def test_library_exports_every_declared_symbol():
     assert sorted(L._signatures) == _declared()
 
 
+def test_host_library_exports_every_declared_symbol():
+    """libfinchops.so: every function include/finch_ops.h and include/finch_files.h declare."""
+    from finchmoe_amd import binding
+    binding.load()
+    L = C.CDLL(os.path.join(ROOT, "finchmoe_amd", "libfinchops.so"))
+    names = []
+    for h in ("finch_ops.h", "finch_files.h"):
+        text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", h)).read(), flags=re.S)
+        names += re.findall(r"^[a-z][A-Za-z0-9_ \*]*?\b([a-z][a-z0-9_]+)\s*\(", text, flags=re.M)
+    assert len(names) >= 45 and "fast_batch_matvec" in names and "finch_ops_open_gguf" in names
+    missing = [n for n in names if not hasattr(L, n)]
+    assert not missing, missing
+
+
 def test_status_strings():
     from finchmoe_amd import binding
     L = binding.load()
