@@ -220,6 +220,7 @@ int ensure_scratch(fm_ctx *c, int groups, int hidden, int inter) {
     if (c->d_eo) (void)hipFree(c->d_eo);
     if (c->d_counters) (void)hipFree(c->d_counters);
     if (c->dflags.set[0]) (void)hipFree(c->dflags.set[0]);
+    if (c->dflags.act_set[0]) (void)hipFree(c->dflags.act_set[0]);
     c->d_act = c->d_eo = nullptr;
     c->d_counters = nullptr;
     c->dflags = FmDecodeFlags{};
@@ -239,6 +240,17 @@ int ensure_scratch(fm_ctx *c, int groups, int hidden, int inter) {
         c->dflags.cap = (unsigned int)cap;
         c->dflags.err = c->d_err;
         c->dflags.spin_limit = c->wait_limit;
+    }
+    {   // three activation sets of the launch that sums in LDS, every element marked "not
+        // produced yet" (0xFFC5A3E1, FM_ACT_EMPTY of fm_decode.hip)
+        const size_t cap = (size_t)g * FM_MAX_K * in;
+        float *p = nullptr;
+        HIPCHK(c, hipMalloc((void **)&p, 3 * cap * sizeof(float)));
+        HIPCHK(c, hipMemsetD32Async((hipDeviceptr_t)p, (int)0xFFC5A3E1u, 3 * cap, c->stream));
+        c->dflags.act_set[0] = p;
+        c->dflags.act_set[1] = p + cap;
+        c->dflags.act_graph = p + 2 * cap;
+        c->dflags.act_cap = (unsigned int)cap;
     }
     c->cap_groups = g;
     c->cap_hidden = h;
@@ -338,7 +350,7 @@ extern "C" int fm_ctx_destroy(fm_ctx *c) {
         }
     if (c->h_err) (void)hipHostFree(c->h_err);
     void *ptrs[] = {c->d_layer_ptrs, c->d_gg_ptrs, c->d_act, c->d_eo, c->d_counters,
-                    c->dflags.set[0],
+                    c->dflags.set[0], c->dflags.act_set[0],
                     c->d_stage, c->d_ws, c->d_tail};
     if (c->h_stage) (void)hipHostFree(c->h_stage);
     for (void *p : ptrs)
@@ -549,7 +561,8 @@ extern "C" int fm_moe_decode_step_dev(fm_ctx *c, int layer0, int n_layers, const
     const bool split = c->split_phases || c->ktiming == 2;
     rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer0, 1, n_layers, d_x, d_idx, d_w,
                                  K, c->d_act, d_expert_out ? d_expert_out : c->d_eo, d_out,
-                                 split ? nullptr : &c->dflags, flags, c->n_cu, c->stream,
+                                 split ? nullptr : &c->dflags,
+                                 flags | (d_expert_out ? 0 : FM_INT_NO_EXPERT_OUT), c->n_cu, c->stream,
                                  c->ktiming ? c->kev : nullptr);
     if (rc) return fail(c, rc, "decode launch failed: %s", hipGetErrorString(hipGetLastError()));
     if (!split) c->sync_unchecked = true;
@@ -723,7 +736,7 @@ static int moe_prefill_any(fm_ctx *c, int layer, const void *d_X, bool x_bf16, c
     if (rc) return rc;
     rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer, 0, M, xf, d_idx, d_w, K,
                                  c->d_act, c->d_eo, d_out, c->split_phases ? nullptr : &c->dflags,
-                                 flags, c->n_cu, c->stream, nullptr);
+                                 flags | FM_INT_NO_EXPERT_OUT, c->n_cu, c->stream, nullptr);
     if (rc) return fail(c, rc, "prefill launch failed: %s", hipGetErrorString(hipGetLastError()));
     if (!c->split_phases) c->sync_unchecked = true;
     return FM_OK;

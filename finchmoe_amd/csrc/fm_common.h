@@ -33,7 +33,21 @@ struct FmDecodeFlags {
     unsigned int *err;
     unsigned int spin_limit;
     int always_graph_set;   // count in graph_set behind a clearing kernel even when not capturing
+    // Activation sets of the launch form that keeps the per-expert vectors in LDS
+    // (fm_moe_fused_rows): elements not yet produced hold a marker, so a set must be all
+    // markers when a launch starts.  Two sets alternate like the counters (a launch fills
+    // act_set[act_parity] and re-marks the act_used[act_parity ^ 1] floats the launch before it
+    // filled); act_graph belongs to captured launches, re-marked by a kernel recorded in front.
+    float *act_set[2];
+    float *act_graph;
+    unsigned int act_used[2];
+    unsigned int act_cap;   // floats per set; 0: this launch form is not available
+    int act_parity;
 };
+
+// internal launch flag (above the public FM_* bits): the caller has no use for the per-expert
+// vectors
+#define FM_INT_NO_EXPERT_OUT (1 << 16)
 
 // Geometry of the GGUF slabs of one layer (finchmoe/infer.m:1017-1022).
 struct FmGgufGeom {

@@ -700,6 +700,558 @@ void fm_moe_fused(DecodeArgs a, int n_pairs, FmFlags f) {
     }
 }
 
+// ======================================================================
+// The operator as one launch when the caller does not want the per-expert vectors and the
+// plain combine applies (no finite guard): nothing but `out` leaves the workgroup.
+//
+// Down phase by row blocks.  A row block is one wave step's rows (64/LPR_DOWN of them) of all
+// K experts of a layer; the row blocks are split over the workgroups, so
+// a workgroup owns whole output rows: it keeps the K partial vectors of its rows in LDS and
+// adds them up itself, w_k * down_k in slot order (the arithmetic of fm_combine_rows<false>),
+// when its part of a layer is finished.  The per-expert vectors are never written, there is
+// no combine phase, and nothing waits for the slowest workgroup of the grid.  A segment of
+// the down phase is a layer: the K activation images of its experts fill the LDS of the two
+// gate/up images.  Units of a part are handed out expert by expert, so a wave re-reads its
+// activation registers only when the expert changes.
+//
+// Activations between the phases.  A vector element that has not been produced yet holds
+// FM_ACT_EMPTY (a NaN that no arithmetic yields); the consumer polls each element it needs
+// until it holds something else.  No counters, so the producer never has to wait for its
+// stores (a wait for stores is a wait for every load in flight as well: it would empty the
+// ring).  Two activation sets alternate between launches: a launch fills the one it is given
+// and marks the part of the other that the launch before it filled as empty again.
+//
+// The split (see Fm2Stream::run): a workgroup's down rows lie in one layer, and its gate/up
+// units are sized so that every workgroup streams the same number of bytes; a gate/up share
+// touches at most two layers, whose images are both built before the stream starts, so the
+// only workgroup barrier of the steady state is the one between the phases.  The slowest
+// workgroup ends the kernel: a workgroup that changed layer more often than the others used
+// to be that one.
+//
+// Nothing in the steady state waits for vector memory except the ring's own waits: all
+// segment tables (blob pointers, router weights) are built before the first load of the ring,
+// LDS is accessed with explicit instructions (the compiler would order a visible LDS access
+// behind every LDS-direct load in flight), barriers likewise.
+// ======================================================================
+constexpr uint32_t FM_ACT_EMPTY = 0xFFC5A3E1u;
+constexpr int FM2_MAX_SEG = 12;         // segments of one workgroup's shares, all sub-phases
+constexpr int FM2_PART_BYTES = 12288;   // partial vectors of a part
+
+struct Fm2Seg {
+    const uint8_t *blob[FM_MAX_K];
+    float w[FM_MAX_K];       // router weight, 0 for an invalid expert index
+    uint32_t valid;          // bit k: slot k has a valid expert index
+    uint32_t next_unit;
+    uint32_t first, n;       // this workgroup's units of the segment
+    int layer;               // layer group (layer of a step, position of a chunk)
+    int pad;
+};
+
+struct Fm2Sync {
+    float *act_other;        // the activation set of the previous and of the next launch
+    unsigned int clear_n;    // floats of it to mark empty
+    unsigned int *err;       // host memory
+    unsigned int spin_limit;
+};
+
+template <int BITS, int LPR>
+constexpr size_t fm2_lds_bytes() {
+    return FmDma<BITS>::WG_BYTES + 2 * sizeof(FmActLds<LPR>) + FM2_MAX_SEG * sizeof(Fm2Seg) +
+           FM2_PART_BYTES;
+}
+
+__device__ __forceinline__ void fm_lds_w32(uint32_t addr, uint32_t v) {
+    asm volatile("ds_write_b32 %0, %1" ::"v"(addr), "v"(v) : "memory");
+}
+__device__ __forceinline__ uint32_t fm_lds_r32(uint32_t addr) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
+    return v;
+}
+// workgroup barrier that waits for this wave's LDS operations only (the compiler's own puts a
+// wait for every LDS-direct load in front)
+__device__ __forceinline__ void fm_wg_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// fm_read_act_lds with explicit instructions; img = LDS address of the image
+template <int LPR>
+__device__ __forceinline__ void fm_read_act_lds_x(uint32_t img, int lane, FmActRegs &ar) {
+    constexpr int NE = 4 * LPR, QS = NE * 16;
+    const int e = lane % NE;
+    const uint32_t a0 = img + (uint32_t)e * 16u;
+    const uint32_t as = img + 16u * QS + (uint32_t)(e >> 2) * 16u;
+    fm_u4 q[16], sm;
+    asm volatile("ds_read_b128 %0, %17\n\t"
+                 "ds_read_b128 %1, %17 offset:%c19\n\t"
+                 "ds_read_b128 %2, %17 offset:%c19*2\n\t"
+                 "ds_read_b128 %3, %17 offset:%c19*3\n\t"
+                 "ds_read_b128 %4, %17 offset:%c19*4\n\t"
+                 "ds_read_b128 %5, %17 offset:%c19*5\n\t"
+                 "ds_read_b128 %6, %17 offset:%c19*6\n\t"
+                 "ds_read_b128 %7, %17 offset:%c19*7\n\t"
+                 "ds_read_b128 %8, %17 offset:%c19*8\n\t"
+                 "ds_read_b128 %9, %17 offset:%c19*9\n\t"
+                 "ds_read_b128 %10, %17 offset:%c19*10\n\t"
+                 "ds_read_b128 %11, %17 offset:%c19*11\n\t"
+                 "ds_read_b128 %12, %17 offset:%c19*12\n\t"
+                 "ds_read_b128 %13, %17 offset:%c19*13\n\t"
+                 "ds_read_b128 %14, %17 offset:%c19*14\n\t"
+                 "ds_read_b128 %15, %17 offset:%c19*15\n\t"
+                 "ds_read_b128 %16, %18\n\t"
+                 "s_waitcnt lgkmcnt(0)"
+                 : "=&v"(q[0]), "=&v"(q[1]), "=&v"(q[2]), "=&v"(q[3]), "=&v"(q[4]), "=&v"(q[5]),
+                   "=&v"(q[6]), "=&v"(q[7]), "=&v"(q[8]), "=&v"(q[9]), "=&v"(q[10]), "=&v"(q[11]),
+                   "=&v"(q[12]), "=&v"(q[13]), "=&v"(q[14]), "=&v"(q[15]), "=&v"(sm)
+                 : "v"(a0), "v"(as), "n"(QS)
+                 : "memory");
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        ar.a[4 * i + 0] = q[i][0];
+        ar.a[4 * i + 1] = q[i][1];
+        ar.a[4 * i + 2] = q[i][2];
+        ar.a[4 * i + 3] = q[i][3];
+    }
+    ar.xsum[0] = __uint_as_float(sm[0]);
+    ar.xsum[1] = __uint_as_float(sm[1]);
+    ar.xoff[0] = __uint_as_float(sm[2]);
+    ar.xoff[1] = __uint_as_float(sm[3]);
+    ar.ones = fm_opaque(0x3F803F80u);
+}
+
+// fm_act_build for one (chunk, image) with explicit LDS writes: this wave's 64 lanes hold
+// the 64 register slots of chunk `ch` (xl, xh: the slot's two activations), img = LDS address
+template <int BITS, int LPR>
+__device__ __forceinline__ void fm2_build_chunk(float xl, float xh, const FmBuildSlot<BITS> &bs,
+                                                uint32_t img, int ch, bool on) {
+    constexpr int NE = 4 * LPR;
+    const int w = threadIdx.x & 63;
+    float vl = xl * bs.slo, vh = xh * bs.shi;
+    uint32_t l0 = __float_as_uint(vl) & 0xFFFF0000u, h0 = __float_as_uint(vh) & 0xFFFF0000u;
+    float rl = vl - __uint_as_float(l0), rh = vh - __uint_as_float(h0);
+    uint32_t l1 = __float_as_uint(rl) & 0xFFFF0000u, h1 = __float_as_uint(rh) & 0xFFFF0000u;
+    rl -= __uint_as_float(l1);
+    rh -= __uint_as_float(h1);
+    uint32_t l2 = __float_as_uint(rl), h2 = __float_as_uint(rh) & 0xFFFF0000u;
+    float xs = fm_group_sum<32>(xl + xh);
+    float xo = fm_group_sum<32>(vl + vh);
+    if (on) {
+        const uint32_t dst = img + (uint32_t)((((w >> 2) * NE + 4 * ch) * 4 + (w & 3)) * 4);
+        fm_lds_w32(dst, (l0 >> 16) | h0);
+        fm_lds_w32(dst + 16, (l1 >> 16) | h1);
+        fm_lds_w32(dst + 32, (l2 >> 16) | h2);
+        fm_lds_w32(dst + 48, 0u);
+        if ((w & 31) == 0) {
+            const uint32_t sp = img + (uint32_t)(16 * NE * 16 + ch * 16 + (w >> 5) * 4);
+            fm_lds_w32(sp, __float_as_uint(xs));
+            fm_lds_w32(sp + 8, __float_as_uint(xo));
+        }
+    }
+}
+
+#ifdef FM2_TIMING
+// timing aid of experimental builds: per wave, the 100 MHz clock at eight points of the kernel
+__device__ unsigned long long fm2_tlog[1024 * FM_NW * 8];
+#define FM2_T(I)                                                                          \
+    do {                                                                                  \
+        if ((threadIdx.x & 63) == 0 && blockIdx.x < 1024)                                 \
+            fm2_tlog[((size_t)blockIdx.x * FM_NW + (threadIdx.x >> 6)) * 8 + (I)] = wall_clock64(); \
+    } while (0)
+#else
+#define FM2_T(I) do {} while (0)
+#endif
+
+template <int BITS, int LPR_UP, bool FP16>
+struct Fm2Stream {
+    using D = FmDma<BITS>;
+    static constexpr int RING = D::RING;
+    static constexpr int LPR_DN = LPR_UP / 4;
+    static constexpr int RPS_UP = FM_WAVE / LPR_UP, RPS_DN = FM_WAVE / LPR_DN;
+    static constexpr int IMG_UP = (int)sizeof(FmActLds<LPR_UP>), IMG_DN = (int)sizeof(FmActLds<LPR_DN>);
+    static_assert(FM_MAX_K * IMG_DN <= 2 * IMG_UP, "the K down images use the two gate/up images");
+
+    const DecodeArgs &a;
+    const Fm2Sync &sy;
+    int lane, wave;
+    uint32_t ring0, img0, part0;
+    Fm2Seg *tab;
+    uint32_t gu_upp, dn_upp;
+    int n_up, n_seq;
+    uint32_t gu_wstep, gu_sstep, dn_wstep, dn_sstep;
+    // loader's phase (plain members assigned at the phase change, see FmOperatorStream)
+    bool l_gu;
+    uint32_t cur_wstep, cur_sstep, cur_w, cur_s, cur_b, d_w, d_s, d_b;
+    int lq, cq;
+    uint32_t l_first, l_n, l_nrb;
+    float l_inv;
+    int hn, wpos, c;
+    uint32_t tag_n, rsn, issued, consumed;
+    const uint8_t *blob_n;
+    bool dry;
+    FmBuildSlot<BITS> bslot;
+
+    __device__ __forceinline__ Fm2Stream(const DecodeArgs &a_, const Fm2Sync &sy_) : a(a_), sy(sy_) {
+        lane = threadIdx.x & 63;
+        wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const uint32_t lds0 = fm_lds_addr(fm_dyn_lds);
+        ring0 = lds0 + (uint32_t)wave * (RING * D::BYTES);
+        img0 = lds0 + D::WG_BYTES;
+        tab = reinterpret_cast<Fm2Seg *>(fm_dyn_lds + D::WG_BYTES + 2 * IMG_UP);
+        part0 = img0 + 2 * IMG_UP + FM2_MAX_SEG * (uint32_t)sizeof(Fm2Seg);
+        gu_upp = (uint32_t)(a.g.inter / RPS_UP);
+        dn_upp = (uint32_t)(a.g.hidden / RPS_DN);
+        gu_wstep = (uint32_t)(RPS_UP * (a.g.hidden * BITS / 8));
+        gu_sstep = (uint32_t)(RPS_UP * (a.g.hidden / 64) * 2);
+        dn_wstep = (uint32_t)(RPS_DN * (a.g.inter * BITS / 8));
+        dn_sstep = (uint32_t)(RPS_DN * (a.g.inter / 64) * 2);
+        d_w = a.g.up_w - a.g.gate_w;
+        d_s = a.g.up_s - a.g.gate_s;
+        d_b = a.g.up_b - a.g.gate_b;
+        lq = cq = 0;
+        l_first = l_n = l_nrb = 0;
+        l_inv = 0.0f;
+        hn = wpos = c = 0;
+        tag_n = rsn = issued = consumed = 0;
+        blob_n = nullptr;
+        dry = false;
+        l_gu = true;
+        bslot.init();
+    }
+
+    __device__ __forceinline__ void loader_enter(int q) {
+        if (l_gu && q >= n_up) {
+            l_gu = false;
+            cur_wstep = dn_wstep, cur_sstep = dn_sstep;
+            cur_w = a.g.down_w, cur_s = a.g.down_s, cur_b = a.g.down_b;
+        }
+        const uint32_t ta = fm_lds_addr(&tab[q].first);
+        l_first = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta));
+        l_n = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + 4));
+        if (!l_gu) {
+            l_nrb = l_n / (uint32_t)a.K;
+            l_first = l_first / (uint32_t)a.K;          // first row block of the part
+            l_inv = 1.0f / (float)(l_nrb ? l_nrb : 1u);
+        }
+    }
+
+    __device__ __forceinline__ void issue() {
+        if (dry) return;
+        if (!l_gu || hn == 0) {
+            uint32_t ul;
+            for (;;) {
+                ul = fm_claim_unit(&tab[lq].next_unit, lane);
+                if (ul < l_n) break;
+                if (lq + 1 < n_seq && lq == cq) {       // run on into the next segment
+                    lq++;
+                    loader_enter(lq);
+                    continue;
+                }
+                dry = true;
+                return;
+            }
+            uint32_t pn;
+            if (l_gu) {
+                const uint32_t uq = l_first + ul;
+                pn = uq / gu_upp;
+                rsn = uq - pn * gu_upp;
+            } else {
+                // expert by expert: unit ul = row block ul % nrb of expert ul / nrb
+                pn = (uint32_t)(((float)ul + 0.5f) * l_inv);
+                rsn = l_first + (ul - pn * l_nrb);
+            }
+            tag_n = ((uint32_t)(lq & 1) << 31) | (pn << 28) | ul;
+            const uint32_t ba = fm_lds_addr(&tab[lq].blob[pn]);
+            const uint32_t lo = __builtin_amdgcn_readfirstlane(fm_lds_r32(ba));
+            const uint32_t hi = __builtin_amdgcn_readfirstlane(fm_lds_r32(ba + 4));
+            blob_n = (const uint8_t *)(((uintptr_t)hi << 32) | lo);
+        }
+        const uint32_t slot = ring0 + (uint32_t)wpos * D::BYTES;
+        fm_slot_tag(slot + D::TAG, tag_n);
+        const uint8_t *b = blob_n + (size_t)rsn * cur_wstep;
+        const uint8_t *sb = blob_n + (size_t)rsn * cur_sstep;
+        const uint32_t second = (uint32_t)hn;
+        fm_dma_issue<BITS>(slot, b + cur_w + second * d_w, sb + cur_s + second * d_s,
+                           sb + cur_b + second * d_b, lane);
+        if (l_gu) hn ^= 1;
+        wpos = wpos + 1 == RING ? 0 : wpos + 1;
+        issued++;
+    }
+
+    template <int LPR>
+    __device__ __forceinline__ float take(uint32_t woff, uint32_t soff, const FmActRegs &ar) {
+        FmRowSlice<BITS> t;
+        if (issued - consumed == (uint32_t)RING) fm_dma_wait<D::LOADS *(RING - 1)>(false);
+        else fm_dma_wait<0>(true);
+        fm_dma_read<BITS>(ring0 + (uint32_t)c * D::BYTES, woff, soff, t);
+        consumed++;
+        c = c + 1 == RING ? 0 : c + 1;
+        issue();
+#ifdef FM2_NOCOMPUTE
+        return (float)((t.s ^ t.b ^ t.q[0][0] ^ t.q[1][1] ^ t.q[2][2]) & 3u) + 0.5f;
+#else
+        return fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(t, ar));
+#endif
+    }
+
+    __device__ __forceinline__ int seg_layer(int q) const {
+        return __builtin_amdgcn_readfirstlane((int)fm_lds_r32(fm_lds_addr(&tab[q].layer)));
+    }
+
+    // an activation produced in this launch: polled until it is there
+    __device__ __forceinline__ float act_get(const float *p) const {
+        unsigned int polls = 0;
+        for (;;) {
+            const float v = fm_ld_shared(p);
+            if (__float_as_uint(v) != FM_ACT_EMPTY) return v;
+            if (++polls > sy.spin_limit) {
+                __hip_atomic_store(sy.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                return 0.0f;
+            }
+            __builtin_amdgcn_s_sleep(8);
+        }
+    }
+
+    // w_k * partial_k over the part's rows, in slot order -> out (fm_combine_rows<false>)
+    __device__ __forceinline__ void reduce_part(int q) {
+        const int K = a.K;
+        const uint32_t ta = fm_lds_addr(&tab[q]);
+        const uint32_t first = fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, first));
+        const uint32_t n = fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, n));
+        float wk[FM_MAX_K];
+#pragma unroll
+        for (int k = 0; k < FM_MAX_K; k++)
+            wk[k] = k < K ? __uint_as_float(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, w) + 4u * k)) : 0.0f;
+        const int rows = (int)(n / (uint32_t)K) * RPS_DN;
+        const int l = seg_layer(q);
+        float *out = a.out + (size_t)l * a.g.hidden + (size_t)(first / (uint32_t)K) * RPS_DN;
+        for (int r = threadIdx.x; r < rows; r += FM_NW * 64) {
+            const int rbi = r / RPS_DN, ris = r - rbi * RPS_DN;
+            float acc = 0.0f;
+#pragma unroll
+            for (int k = 0; k < FM_MAX_K; k++)
+                if (k < K && wk[k] != 0.0f)
+                    acc += wk[k] * __uint_as_float(fm_lds_r32(part0 + 4u * (uint32_t)((rbi * K + k) * RPS_DN + ris)));
+            out[r] = (a.flags & FM_ACCUMULATE) ? out[r] + acc : acc;
+        }
+    }
+
+    __device__ __forceinline__ void run(int n_pairs) {
+        const int K = a.K, n_groups = n_pairs / K, G = gridDim.x, g = blockIdx.x;
+        FM2_T(0);
+        // The split.  Down: a workgroup's row blocks lie in ONE layer whenever there are at
+        // least as many workgroups as layers (layer l gets the workgroups g with g*L/G == l, its
+        // row blocks divided evenly among them), so the down phase has one segment and no
+        // workgroup pays for a change of layer that others do not have.  Gate/up: contiguous unit
+        // ranges sized so that gate/up + down bytes are the same for every workgroup (a
+        // workgroup with fewer down rows takes more gate/up units).
+        // (32-bit arithmetic: the launcher checks that slices x workgroups stays below 2^31)
+        const uint32_t Ku = (uint32_t)K, Gu = (uint32_t)G, Lu = (uint32_t)n_groups;
+        const uint32_t gu_segu = gu_upp * Ku, dn_segu = dn_upp * Ku;
+        const uint32_t gu_total = (uint32_t)n_pairs * gu_upp, rb_total = Lu * dn_upp;
+        const uint32_t s_total = 2u * gu_total + rb_total * Ku;     // slices of the whole operator
+        auto dn_start = [&](uint32_t gg) -> uint32_t {              // first row block of workgroup gg
+            if (gg >= Gu) return rb_total;
+            if (Gu < Lu) return rb_total * gg / Gu;
+            const uint32_t l = gg * Lu / Gu;
+            const uint32_t g_lo = (l * Gu + Lu - 1u) / Lu, g_hi = ((l + 1u) * Gu + Lu - 1u) / Lu;
+            return l * dn_upp + dn_upp * (gg - g_lo) / (g_hi - g_lo);
+        };
+        auto gu_start = [&](uint32_t gg, uint32_t dn0) -> uint32_t {   // first gate/up unit of workgroup gg
+            const uint32_t t = s_total * gg / Gu, d = dn0 * Ku;
+            const uint32_t u = t > d ? (t - d) / 2u : 0u;
+            return u > gu_total ? gu_total : u;
+        };
+        const uint32_t dn_rb0 = dn_start((uint32_t)g), dn_rb1 = dn_start((uint32_t)g + 1u);
+        const uint32_t gu_wg0 = gu_start((uint32_t)g, dn_rb0), gu_wg1 = gu_start((uint32_t)g + 1u, dn_rb1);
+        const uint32_t dn_wg0 = dn_rb0 * Ku, dn_wg1 = dn_rb1 * Ku;
+        const int gu_s0 = (int)(gu_wg0 / gu_segu), dn_s0 = (int)(dn_wg0 / dn_segu);
+        n_up = gu_wg1 > gu_wg0 ? (int)((gu_wg1 - 1u) / gu_segu) + 1 - gu_s0 : 0;
+        const int n_dn = dn_wg1 > dn_wg0 ? (int)((dn_wg1 - 1u) / dn_segu) + 1 - dn_s0 : 0;
+        n_seq = n_up + n_dn;
+        const int qq = threadIdx.x >> 3;        // the segment this thread looks up below
+        const bool mine = qq < n_seq;
+        const bool mine_gu = qq < n_up;
+        const uint32_t mine_s = (uint32_t)(mine_gu ? gu_s0 + qq : dn_s0 + (qq - n_up));
+        uint32_t mine_first, mine_n;
+        {
+            const uint32_t segu = mine_gu ? gu_segu : dn_segu, w0 = mine_gu ? gu_wg0 : dn_wg0, w1 = mine_gu ? gu_wg1 : dn_wg1;
+            const uint32_t lo = mine_s * segu > w0 ? mine_s * segu : w0;
+            const uint32_t hi = (mine_s + 1u) * segu < w1 ? (mine_s + 1u) * segu : w1;
+            mine_first = lo - mine_s * segu;
+            mine_n = hi > lo ? hi - lo : 0u;
+        }
+
+        // the other activation set becomes empty again (plain stores, nobody reads it now)
+        for (unsigned int i = blockIdx.x * blockDim.x + threadIdx.x; i < sy.clear_n; i += G * blockDim.x)
+            sy.act_other[i] = __uint_as_float(FM_ACT_EMPTY);
+        if (n_seq == 0) return;
+
+        // the first gate/up segment's input, then the tables of every segment: thread 8q + k
+        // looks up slot k of segment q (ordinary loads and LDS stores: nothing is in flight yet)
+        // (every thread loads, and the values are used unconditionally further down: a load
+        // whose result is still pending on some path of the control flow makes the compiler
+        // wait for every load in flight at the register's next use, in the middle of the stream)
+        FmActX<LPR_UP> xr0, xr1;
+        fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)(n_up > 0 ? gu_s0 : 0) * a.g.hidden, bslot, xr0);
+        fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)(n_up > 1 ? gu_s0 + 1 : 0) * a.g.hidden, bslot, xr1);
+        if (mine) {
+            const int k = threadIdx.x & 7;
+            const size_t sg = mine_s;                              // layer group of the segment
+            Fm2Seg &t = tab[qq];
+            bool ok = false;
+            if (k < K) {
+                const int e = a.idx[sg * K + k];
+                const float wv = a.w[sg * K + k];
+                ok = (unsigned)e < (unsigned)a.g.n_experts;
+                t.blob[k] = a.layer_ptrs[a.layer0 + (int)sg * a.layer_stride] + (size_t)(ok ? e : 0) * a.g.expert_size;
+                t.w[k] = ok ? wv : 0.0f;
+            }
+            const uint64_t m = __ballot(ok);
+            if (k == 0) {
+                t.valid = (uint32_t)(m >> (threadIdx.x & 56)) & 0xFFu;
+                t.next_unit = 0u;
+                t.first = mine_first;
+                t.n = mine_n;
+                t.layer = (int)sg;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < FmActX<LPR_UP>::NIT; i++)
+            asm volatile("" ::"v"(xr0.xl[i]), "v"(xr0.xh[i]), "v"(xr1.xl[i]), "v"(xr1.xh[i]));
+        if (n_up > 0) {
+            cur_wstep = gu_wstep, cur_sstep = gu_sstep;
+            cur_w = a.g.gate_w, cur_s = a.g.gate_s, cur_b = a.g.gate_b;
+            // the images of both gate/up segments, before anything of the ring is in flight: a
+            // wave then changes segment on its own, without a barrier
+            if (threadIdx.x < 256) {
+#pragma unroll
+                for (int i = 0; i < FmActX<LPR_UP>::NIT; i++) {
+                    const int chn = (threadIdx.x >> 6) + 4 * i;
+                    fm2_build_chunk<BITS, LPR_UP>(xr0.xl[i], xr0.xh[i], bslot, img0, chn, chn < LPR_UP);
+                    fm2_build_chunk<BITS, LPR_UP>(xr1.xl[i], xr1.xh[i], bslot, img0 + IMG_UP, chn, chn < LPR_UP && n_up > 1);
+                }
+            }
+        }
+        __syncthreads();
+        FM2_T(1);
+        loader_enter(0);
+#pragma unroll
+        for (int k = 0; k < RING; k++) issue();
+        FM2_T(2);
+
+        // ---------------------------------------------------------- gate/up
+        {
+            uint32_t woff, soff;
+            int ris, ch;
+            fm_unit_lane_offsets<BITS, LPR_UP>(lane, a.g.hidden * BITS / 8, (a.g.hidden / 64) * 2, woff,
+                                               soff, ris, ch);
+            for (; cq < n_up; cq++) {
+                const int s = seg_layer(cq);
+                const uint32_t img = img0 + (uint32_t)(cq & 1) * IMG_UP;
+                FmActRegs ar;
+                fm_read_act_lds_x<LPR_UP>(img, lane, ar);
+                const uint32_t ta = fm_lds_addr(&tab[cq]);
+                const uint32_t valid = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, valid)));
+                const uint32_t c_first = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, first)));
+                const size_t out0 = ((size_t)s * gu_segu + c_first) * RPS_UP + ris;
+                dry = false;
+                while (issued - consumed < (uint32_t)RING && !dry) issue();
+                while (consumed < issued) {
+                    const uint32_t tag = fm_slot_peek(ring0 + (uint32_t)c * D::BYTES + D::TAG);
+                    if ((tag >> 31) != (uint32_t)(cq & 1)) break;
+                    const uint32_t pc = (tag >> 28) & 7u, ul = tag & 0x0FFFFFFFu;
+                    const float gv = take<LPR_UP>(woff, soff, ar);
+#ifdef FM2_TIMING
+                    if (consumed == 1) FM2_T(3);
+#endif
+                    const float uv = take<LPR_UP>(woff, soff, ar);
+                    float v = fm_silu_mul(gv, uv);
+                    if (!((valid >> pc) & 1u)) v = 0.0f;
+                    if (ch == 0) fm_st_shared(a.act + out0 + (size_t)ul * RPS_UP, v);
+                }
+            }
+        }
+        FM2_T(4);
+        // ---------------------------------------------------------- down
+        {
+            uint32_t woff, soff;
+            int ris, ch;
+            fm_unit_lane_offsets<BITS, LPR_DN>(lane, a.g.inter * BITS / 8, (a.g.inter / 64) * 2, woff,
+                                               soff, ris, ch);
+            for (; cq < n_seq; cq++) {
+                const int l = seg_layer(cq);
+                fm_wg_barrier();                       // images and partial vectors are free
+                if (cq > n_up) reduce_part(cq - 1);
+                // the K activation vectors of the layer -> K images; wave slot (tid / 64) takes
+                // the (expert, chunk) combinations slot, slot + 8, ...
+                float xl[LPR_DN], xh[LPR_DN];
+#pragma unroll
+                for (int i = 0; i < LPR_DN; i++) {       // all loads first, polls where needed after
+                    const int cmb = (threadIdx.x >> 6) + FM_NW * i;
+                    const int k = cmb / LPR_DN, chn = cmb - k * LPR_DN;
+                    const float *src = a.act + ((size_t)l * K + (k < K ? k : 0)) * a.g.inter + chn * FM_CPL;
+                    xl[i] = fm_ld_shared(src + bslot.lo);
+                    xh[i] = fm_ld_shared(src + bslot.hi);
+                }
+#pragma unroll
+                for (int i = 0; i < LPR_DN; i++) {
+                    const int cmb = (threadIdx.x >> 6) + FM_NW * i;
+                    const int k = cmb / LPR_DN, chn = cmb - k * LPR_DN;
+                    const bool on = k < K;
+                    const float *src = a.act + ((size_t)l * K + (on ? k : 0)) * a.g.inter + chn * FM_CPL;
+                    if (__float_as_uint(xl[i]) == FM_ACT_EMPTY) xl[i] = act_get(src + bslot.lo);
+                    if (__float_as_uint(xh[i]) == FM_ACT_EMPTY) xh[i] = act_get(src + bslot.hi);
+                    fm2_build_chunk<BITS, LPR_DN>(xl[i], xh[i], bslot, img0 + (uint32_t)(on ? k : 0) * IMG_DN, chn, on);
+                }
+                fm_wg_barrier();
+                const uint32_t ta = fm_lds_addr(&tab[cq]);
+                const uint32_t valid = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, valid)));
+                const uint32_t c_nrb = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, n))) / (uint32_t)K;
+                FmActRegs ar;
+                uint32_t k_cur = 0xFFFFFFFFu;
+#ifdef FM2_TIMING
+                if (cq == n_up) FM2_T(5);
+#endif
+                dry = false;
+                while (issued - consumed < (uint32_t)RING && !dry) issue();
+                while (consumed < issued) {
+                    const uint32_t tag = fm_slot_peek(ring0 + (uint32_t)c * D::BYTES + D::TAG);
+                    if ((tag >> 31) != (uint32_t)(cq & 1)) break;
+                    const uint32_t pc = (tag >> 28) & 7u, ul = tag & 0x0FFFFFFFu;
+                    if (pc != k_cur) {
+                        fm_read_act_lds_x<LPR_DN>(img0 + pc * IMG_DN, lane, ar);
+                        k_cur = pc;
+                    }
+                    float v = take<LPR_DN>(woff, soff, ar);
+                    if (!((valid >> pc) & 1u)) v = 0.0f;
+                    const uint32_t rbi = ul - pc * c_nrb;
+                    if (ch == 0)
+                        fm_lds_w32(part0 + 4u * ((rbi * (uint32_t)K + pc) * RPS_DN + (uint32_t)ris), __float_as_uint(v));
+                }
+            }
+            FM2_T(6);
+            if (n_seq > n_up) {
+                fm_wg_barrier();
+                reduce_part(n_seq - 1);
+            }
+        }
+        FM2_T(7);
+    }
+};
+
+template <int BITS, int LPR_UP, bool FP16>
+__global__ __launch_bounds__(FM_NW * 64)
+void fm_moe_fused_rows(DecodeArgs a, int n_pairs, Fm2Sync sy) {
+    Fm2Stream<BITS, LPR_UP, FP16> st(a, sy);
+    st.run(n_pairs);
+}
+
+// fills n words with v (counters to zero, activations to FM_ACT_EMPTY)
+__global__ __launch_bounds__(256) void fm_fill_words(unsigned int *p, unsigned int n, unsigned int v) {
+    const unsigned int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
 __global__ __launch_bounds__(256) void fm_clear_counters(unsigned int *p, unsigned int n) {
     const unsigned int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0u;
@@ -761,14 +1313,79 @@ int launch_fused(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st, con
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 
+// The launch that keeps the per-expert vectors in LDS.  FM_ERR_UNSUPPORTED when the shape does
+// not fit its fixed tables (the caller then takes the launch with counters).
+template <int BITS, int LPR_UP, bool FP16>
+int launch_fused_rows(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st, const Fm2Sync &sy) {
+    auto kfn = fm_moe_fused_rows<BITS, LPR_UP, FP16>;
+    const size_t sh = fm2_lds_bytes<BITS, LPR_UP>();
+    static FmKernelSetup ks;
+    if (!fm_dyn_lds_ok(ks, (const void *)kfn, sh)) return FM_ERR_HIP;
+    const int dev = fm_current_device();
+    int per_cu = dev >= 0 ? ks.per_cu[dev] : 0;
+    if (per_cu == 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kfn, FM_NW * 64, sh) != hipSuccess)
+            per_cu = 0;
+        if (per_cu < 1) per_cu = -1;
+        if (dev >= 0) ks.per_cu[dev] = per_cu;
+    }
+    if (per_cu < 1) return FM_ERR_UNSUPPORTED;   // the grid could not be resident at once
+    constexpr int RPS_UP = FM_WAVE / LPR_UP, RPS_DN = FM_WAVE / (LPR_UP / 4);
+    const int n_groups = n_pairs / a.K;
+    const long gu_segu = (long)(a.g.inter / RPS_UP) * a.K, dn_rbs = a.g.hidden / RPS_DN;
+    const long up_units = (long)n_groups * gu_segu, rb_total = (long)n_groups * dn_rbs;
+    long wgs = n_cu;
+    const long small = up_units < rb_total * a.K ? up_units : rb_total * a.K;
+    if (small < FM_NW * wgs) wgs = (small + FM_NW - 1) / FM_NW;
+    if (wgs < 1) wgs = 1;
+    // the kernel's split (Fm2Stream::run): at most two gate/up segments, and the down segments
+    // and the row blocks of one part within the fixed tables
+    const long s_total = 2 * up_units + rb_total * a.K;
+    const long up_share = (s_total / wgs + 1) / 2 + 1;                  // upper bound, in units
+    if (up_share > gu_segu || s_total * wgs >= (1L << 31)) return FM_ERR_UNSUPPORTED;
+    long n_dn, part_rbs;
+    if (wgs >= n_groups) {
+        n_dn = 1;
+        part_rbs = (dn_rbs + wgs / n_groups - 1) / (wgs / n_groups);
+    } else {
+        const long rb_share = (rb_total + wgs - 1) / wgs;
+        n_dn = (rb_share - 1) / dn_rbs + 2;
+        part_rbs = rb_share < dn_rbs ? rb_share : dn_rbs;
+    }
+    if (2 + n_dn > FM2_MAX_SEG) return FM_ERR_UNSUPPORTED;
+    if (part_rbs * a.K * RPS_DN * 4 > FM2_PART_BYTES) return FM_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(FM_NW * 64), sh, st, a, n_pairs, sy);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
+
 template <int BITS, bool FP16>
 int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int n_cu,
-                    hipStream_t st, hipEvent_t *kev, const FmFlags *fl, bool *fused) {
+                    hipStream_t st, hipEvent_t *kev, const FmFlags *fl, bool *fused,
+                    const Fm2Sync *sy = nullptr, float *act_rows = nullptr, bool *rows = nullptr) {
     dim3 b(256);
     const int lpr_up = a.g.hidden / FM_CPL, lpr_down = a.g.inter / FM_CPL;
     const bool lds_up = lpr_up >= 4 && lpr_up <= 16, lds_down = lpr_down <= 16;
     if (!lds_down) return FM_ERR_UNSUPPORTED;
     if (kev) (void)hipEventRecord(kev[0], st);
+    if (sy && lds_up && lpr_down * 4 == lpr_up) {
+        DecodeArgs a2 = a;
+        a2.act = act_rows;
+        a2.expert_out = nullptr;
+        int rc = FM_ERR_UNSUPPORTED;
+        switch (lpr_up) {
+            case 4: rc = launch_fused_rows<BITS, 4, FP16>(a2, n_pairs, n_cu, st, *sy); break;
+            case 8: rc = launch_fused_rows<BITS, 8, FP16>(a2, n_pairs, n_cu, st, *sy); break;
+            case 16: rc = launch_fused_rows<BITS, 16, FP16>(a2, n_pairs, n_cu, st, *sy); break;
+        }
+        if (rc != FM_ERR_UNSUPPORTED) {
+            *rows = rc == FM_OK;
+            if (kev) {
+                (void)hipEventRecord(kev[1], st);
+                (void)hipEventRecord(kev[2], st);
+            }
+            return rc;
+        }
+    }
     if (fl && lds_up && lpr_down * 4 == lpr_up) {
         int rc = FM_ERR_UNSUPPORTED;
         switch (lpr_up) {
@@ -852,6 +1469,12 @@ int pick_rows_per_item(int rows, int n_pairs, int min_rows, int cap, int want) {
 
 }  // namespace
 
+#ifdef FM2_TIMING
+extern "C" __attribute__((visibility("default"))) int fm_debug_read_tlog(void *dst, size_t bytes) {
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(fm2_tlog), bytes);
+}
+#endif
+
 // Enqueue the operator for n_layers x K pairs (n_layers groups of K slots: the
 // layers of a decode step, or with layer_stride 0 the positions of a chunk).  Shapes are validated by the
 // caller (fm_api.cpp): hidden, inter multiples of 128 with a supported
@@ -914,12 +1537,44 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
         fl.spin_limit = df->spin_limit;
         flp = &fl;
     }
-    bool fused = false;
-#define FM_DEC(B, F) launch_decode_t<B, F>(a, n_pairs, rpi_up, n_cu, st, kev, flp, &fused)
+    // without per-expert vectors and without the finite guard: the launch that sums in LDS
+    Fm2Sync sy{};
+    const Fm2Sync *syp = nullptr;
+    float *act_rows = nullptr;
+    const unsigned int act_need = (unsigned int)n_pairs * (unsigned int)g->inter;
+    if (flp && (flags & FM_INT_NO_EXPERT_OUT) && !(flags & FM_GUARD) && df->act_cap >= act_need &&
+        df->act_set[0]) {
+        if (own_clear) {
+            if (df->act_graph) {
+                hipLaunchKernelGGL(fm_fill_words, dim3((act_need + 255) / 256), dim3(256), 0, st,
+                                   (unsigned int *)df->act_graph, act_need, FM_ACT_EMPTY);
+                act_rows = df->act_graph;
+                sy.act_other = df->act_graph;
+                sy.clear_n = 0u;
+            }
+        } else {
+            act_rows = df->act_set[df->act_parity];
+            sy.act_other = df->act_set[df->act_parity ^ 1];
+            sy.clear_n = df->act_used[df->act_parity ^ 1];
+        }
+        if (act_rows) {
+            sy.err = df->err;
+            sy.spin_limit = df->spin_limit;
+            syp = &sy;
+        }
+    }
+    a.flags = flags & ~FM_INT_NO_EXPERT_OUT;
+    bool fused = false, rows = false;
+#define FM_DEC(B, F) launch_decode_t<B, F>(a, n_pairs, rpi_up, n_cu, st, kev, flp, &fused, syp, act_rows, &rows)
     int rc = FM_ERR_UNSUPPORTED;
     if (g->bits == 3) rc = g->scale_fp16 ? FM_DEC(3, true) : FM_DEC(3, false);
     else if (g->bits == 4) rc = g->scale_fp16 ? FM_DEC(4, true) : FM_DEC(4, false);
 #undef FM_DEC
+    if (rows && !own_clear) {    // the set just filled is in use, the other one is all markers again
+        df->act_used[df->act_parity] = act_need;
+        df->act_used[df->act_parity ^ 1] = 0u;
+        df->act_parity ^= 1;
+    }
     if (fused && !own_clear) {   // the set just used is dirty, the other one is clean again
         df->used[df->parity] = need;
         df->used[df->parity ^ 1] = 0u;

@@ -339,3 +339,70 @@ def test_host_call_falls_back_to_separate_kernels(hip, orc, store3):
             assert_parity(eo, ref_eo, "fallback expert outputs")
     finally:
         hip.set_wait_limit(1 << 20)
+
+
+def test_row_sum_launch_equals_counter_launch(hip, orc, store3):
+    """Without a buffer for the per-expert vectors the operator takes the launch that sums the
+    experts in LDS: its result equals, bit for bit, the launch that writes the per-expert
+    vectors and combines them — for steps of different sizes in a row (the two activation
+    sets alternate and re-mark what the launch before filled), with the accumulate flag, with
+    K below 8, and with an expert index out of range."""
+    import torch
+    for seed, L, K, flags in ((31, 4, 8, 0), (32, 1, 8, 0), (33, 3, 8, fb.ACCUMULATE), (34, 4, 4, 0),
+                              (35, 2, 8, 0), (36, 4, 3, 0), (37, 4, 8, 0), (38, 1, 1, fb.ACCUMULATE)):
+        x, idx, w, (dx, di, dw) = _step_inputs(orc, seed, L, K)
+        if seed == 37:
+            idx[2, 5] = 99                                  # out of range: contributes zero
+            di = torch.from_numpy(idx).cuda()
+        base = torch.from_numpy(np.random.default_rng(seed).standard_normal((L, H)).astype(np.float32)).cuda()
+        want = base.clone()
+        deo = torch.zeros(L, K, H, device="cuda")
+        torch.cuda.synchronize()
+        hip.moe_decode_step_dev(0, L, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K,
+                                want.data_ptr(), deo.data_ptr(), flags)
+        hip.sync()
+        for rep in range(2):
+            got = base.clone()
+            torch.cuda.synchronize()
+            hip.moe_decode_step_dev(0, L, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K,
+                                    got.data_ptr(), None, flags)
+            hip.sync()
+            assert torch.equal(got, want), (seed, L, K, flags, rep)
+        l = L - 1
+        keep = (idx[l] >= 0) & (idx[l] < 12)
+        ref, _ = orc.moe_experts_forward(store3[l], x[l], idx[l][keep], w[l][keep], H, I, 3)
+        mine = want[l].cpu().numpy() - (base[l].cpu().numpy() if flags & fb.ACCUMULATE else 0)
+        assert rel_err(mine, ref) < 1e-3, (seed, rel_err(mine, ref))
+
+
+@pytest.mark.parametrize("h,i,bits,dtype", [(1024, 256, 3, "bf16"), (512, 128, 3, "bf16"), (1024, 256, 4, "fp16"),
+                                            (512, 128, 4, "bf16"), (2048, 512, 4, "bf16"), (2048, 512, 3, "fp16")])
+def test_row_sum_launch_other_shapes(orc, h, i, bits, dtype):
+    """The same equality where the lane maps differ (16/8/4 lanes per gate row, 4/2/1 per down
+    row), for 4-bit codes and FP16 scales, on a step of several layers."""
+    import torch
+    from finchmoe_amd import FinchHip
+    rng = np.random.default_rng(h + i + bits)
+    L, E, K = 3, 6, 4
+    blobs = [F.synth_expert_layer(rng, E, h, i, bits, dtype) for _ in range(L)]
+    ctx = FinchHip(0)
+    try:
+        sd = fb.SCALE_FP16 if dtype == "fp16" else fb.SCALE_BF16
+        ctx.experts_config(L, E, h, i, 64, bits, sd)
+        for l, b in enumerate(blobs):
+            ctx.experts_upload_layer(l, b)
+        x = rng.standard_normal((L, h)).astype(np.float32)
+        idx = np.stack([rng.permutation(E)[:K] for _ in range(L)]).astype(np.int32)
+        w = rng.random((L, K)).astype(np.float32)
+        dx, di, dw = (torch.from_numpy(a).cuda() for a in (x, idx, w))
+        want, got = torch.zeros(L, h, device="cuda"), torch.zeros(L, h, device="cuda")
+        deo = torch.zeros(L, K, h, device="cuda")
+        torch.cuda.synchronize()
+        ctx.moe_decode_step_dev(0, L, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K, want.data_ptr(), deo.data_ptr(), 0)
+        ctx.moe_decode_step_dev(0, L, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K, got.data_ptr(), None, 0)
+        ctx.sync()
+        assert torch.equal(got, want)
+        ref, _ = orc.moe_experts_forward(blobs[1], x[1], idx[1], w[1], h, i, bits, scale_dtype=sd)
+        assert_parity(got[1].cpu().numpy(), ref, "layer 1 %d/%d/%d" % (h, i, bits))
+    finally:
+        ctx.close()
