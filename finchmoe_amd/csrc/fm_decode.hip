@@ -851,11 +851,11 @@ __device__ __forceinline__ void fm2_build_chunk(float xl, float xh, const FmBuil
 
 #ifdef FM2_TIMING
 // timing aid of experimental builds: per wave, the 100 MHz clock at eight points of the kernel
-__device__ unsigned long long fm2_tlog[1024 * FM_NW * 8];
+__device__ unsigned long long fm2_tlog[1024 * FM_NW * 16];
 #define FM2_T(I)                                                                          \
     do {                                                                                  \
         if ((threadIdx.x & 63) == 0 && blockIdx.x < 1024)                                 \
-            fm2_tlog[((size_t)blockIdx.x * FM_NW + (threadIdx.x >> 6)) * 8 + (I)] = wall_clock64(); \
+            fm2_tlog[((size_t)blockIdx.x * FM_NW + (threadIdx.x >> 6)) * 16 + (I)] = wall_clock64(); \
     } while (0)
 #else
 #define FM2_T(I) do {} while (0)
@@ -1091,6 +1091,7 @@ struct Fm2Stream {
         // (every thread loads, and the values are used unconditionally further down: a load
         // whose result is still pending on some path of the control flow makes the compiler
         // wait for every load in flight at the register's next use, in the middle of the stream)
+        FM2_T(8);
         FmActX<LPR_UP> xr0, xr1;
         fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)(n_up > 0 ? gu_s0 : 0) * a.g.hidden, bslot, xr0);
         fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)(n_up > 1 ? gu_s0 + 1 : 0) * a.g.hidden, bslot, xr1);
@@ -1118,26 +1119,34 @@ struct Fm2Stream {
 #pragma unroll
         for (int i = 0; i < FmActX<LPR_UP>::NIT; i++)
             asm volatile("" ::"v"(xr0.xl[i]), "v"(xr0.xh[i]), "v"(xr1.xl[i]), "v"(xr1.xh[i]));
+        FM2_T(9);
         if (n_up > 0) {
             cur_wstep = gu_wstep, cur_sstep = gu_sstep;
             cur_w = a.g.gate_w, cur_s = a.g.gate_s, cur_b = a.g.gate_b;
-            // the images of both gate/up segments, before anything of the ring is in flight: a
-            // wave then changes segment on its own, without a barrier
-            if (threadIdx.x < 256) {
-#pragma unroll
-                for (int i = 0; i < FmActX<LPR_UP>::NIT; i++) {
-                    const int chn = (threadIdx.x >> 6) + 4 * i;
-                    fm2_build_chunk<BITS, LPR_UP>(xr0.xl[i], xr0.xh[i], bslot, img0, chn, chn < LPR_UP);
-                    fm2_build_chunk<BITS, LPR_UP>(xr1.xl[i], xr1.xh[i], bslot, img0 + IMG_UP, chn, chn < LPR_UP && n_up > 1);
-                }
-            }
         }
         __syncthreads();
         FM2_T(1);
         loader_enter(0);
-#pragma unroll
-        for (int k = 0; k < RING; k++) issue();
+        FM2_T(10);
+#pragma nounroll
+        for (int k = 0; k < RING; k++) {
+            issue();
+#ifdef FM2_TIMING
+            if (k == 0) FM2_T(11);
+#endif
+        }
         FM2_T(2);
+        // the images of both gate/up segments (from registers: no load is waited for here); a
+        // wave then changes segment on its own, without a barrier
+        if (n_up > 0 && threadIdx.x < 256) {
+#pragma unroll
+            for (int i = 0; i < FmActX<LPR_UP>::NIT; i++) {
+                const int chn = (threadIdx.x >> 6) + 4 * i;
+                fm2_build_chunk<BITS, LPR_UP>(xr0.xl[i], xr0.xh[i], bslot, img0, chn, chn < LPR_UP);
+                fm2_build_chunk<BITS, LPR_UP>(xr1.xl[i], xr1.xh[i], bslot, img0 + IMG_UP, chn, chn < LPR_UP && n_up > 1);
+            }
+        }
+        fm_wg_barrier();
 
         // ---------------------------------------------------------- gate/up
         {
