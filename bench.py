@@ -32,7 +32,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 peak
 # --pmc FETCH_SIZE (x2: calibrated against a 1 GiB copy) + WRITE_SIZE.  An OFFLINE constant
 # (hardware counters cannot be read from inside this process): the JSON line names the file
 # it comes from in roofline.traffic_source, and it is null for any other size.
-FUSED_TRAFFIC_BYTES_40L = int((218295.98 * 2 + 4186.4) * 1024)
+FUSED_TRAFFIC_BYTES_40L = int((218733.97 * 2 + 2237.57) * 1024)
 FUSED_TRAFFIC_SOURCE = "offline constant from profiles/decode_step_3bit_hbm_traffic.md (rocprofv3 --pmc), not measured in this run"
 
 H, I, E, K, L = 2048, 512, 256, 8, 40
@@ -220,7 +220,7 @@ def run_decode_step(args):
         "token_latency_us": {"mean": round(float(lat.mean()), 1), "p50": round(float(np.median(lat)), 1),
                              "p99": round(float(np.percentile(lat, 99)), 1)},
         "unique_experts_touched_in_256_tokens": uniq,
-        "roofline": {"bound": "hbm", "kernel": "fm_moe_fused<%d,16> (gate/up, down, combine in one launch)" % bits,
+        "roofline": {"bound": "hbm", "kernel": "fm_moe_fused_rows<%d,16> (gate/up, down and the sum over the experts in one launch)" % bits,
                      "achieved": round(bytes_step / (op_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(bytes_step / (op_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                      "traffic": FUSED_TRAFFIC_BYTES_40L if (n_layers, E, K, bits) == (40, 256, 8, 3) else None,
