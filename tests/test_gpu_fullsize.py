@@ -140,3 +140,91 @@ def test_full_chunk_4bit_equals_positions(orc):
         ctx.close()
         del blob
         torch.cuda.empty_cache()
+
+
+def test_full_step_without_expert_vectors_equals_with(full_store):
+    """At the benchmark's size the launch that sums the experts in LDS (no buffer for the
+    per-expert vectors) returns, bit for bit, what the launch with per-expert vectors and a
+    combine phase returns — also when it accumulates, and twice in a row (activation sets)."""
+    import torch
+    from finchmoe_amd import binding as fb
+    ctx, blob, lo, idx, w = full_store
+    x = torch.randn(L, H, device="cuda", generator=torch.Generator(device="cuda").manual_seed(9))
+    for tok, flags in ((0, 0), (1, fb.ACCUMULATE), (0, 0)):
+        d_idx, d_w = torch.from_numpy(idx[tok]).cuda(), torch.from_numpy(w[tok]).cuda()
+        base = torch.full((L, H), 0.25, device="cuda")
+        want, got = base.clone(), base.clone()
+        d_eo = torch.zeros(L, K, H, device="cuda")
+        torch.cuda.synchronize()
+        ctx.moe_decode_step_dev(0, L, x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, want.data_ptr(),
+                                d_eo.data_ptr(), flags)
+        ctx.moe_decode_step_dev(0, L, x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, got.data_ptr(),
+                                None, flags)
+        ctx.sync()
+        assert torch.isfinite(got).all() and torch.equal(got, want), (tok, flags)
+
+
+def test_full_gguf_step_equals_layer_calls_and_oracle(orc):
+    """The GGUF store at the benchmark's size (40 layers x 256 experts, Q4_K gate/up and Q6_K
+    down, 21.5 GB): the 40-layer step equals the 40 single-layer calls bit for bit, the weighted
+    sum equals the per-expert outputs combined in slot order, and the routed experts of three
+    layers equal the CPU oracle on their own bytes copied back."""
+    import torch
+    from bench import zipf_routing
+    from finchmoe_amd import FinchHip
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(5)
+    gsl, dsl = I * (H // 256) * 144, H * (I // 256) * 210      # bytes per expert: gate/up, down
+
+    def slab(nblocks, bsz, d_off, n_d):
+        t = torch.empty(nblocks, bsz, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
+        d = (torch.randn(nblocks, n_d, device=dev, generator=gen).abs_() * 0.002).to(torch.float16)
+        t[:, d_off:d_off + 2 * n_d] = d.view(torch.uint8)
+        return t
+
+    ctx = FinchHip(0)
+    keep = []
+    try:
+        ctx.gguf_config(L, E, H, I)
+        for l in range(L):
+            g = slab(E * I * (H // 256), 144, 0, 2)
+            u = slab(E * I * (H // 256), 144, 0, 2)
+            d = slab(E * H * (I // 256), 210, 208, 1)
+            keep.append((g, u, d))
+            ctx.gguf_adopt_layer(l, g.data_ptr(), g.numel(), u.data_ptr(), u.numel(), d.data_ptr(), d.numel())
+        idx, w = zipf_routing(np.random.default_rng(15), 1, L, E, K)
+        idx, w = idx[0], w[0]
+        x = np.random.default_rng(16).standard_normal((L, H)).astype(np.float32)
+        d_x, d_idx, d_w = (torch.from_numpy(a).cuda() for a in (x, idx, w))
+        d_out, d_eo = torch.zeros(L, H, device=dev), torch.zeros(L, K, H, device=dev)
+        torch.cuda.synchronize()
+        ctx.gguf_moe_decode_step_dev(0, L, d_x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K,
+                                     d_out.data_ptr(), d_eo.data_ptr())
+        ctx.sync()
+        out, eo = d_out.cpu().numpy(), d_eo.cpu().numpy()
+        assert np.isfinite(out).all() and np.abs(out).max() > 0
+        s_out, s_eo = torch.zeros(H, device=dev), torch.zeros(K, H, device=dev)
+        for l in range(L):
+            ctx.gguf_moe_decode_dev(l, d_x.data_ptr() + l * H * 4, d_idx.data_ptr() + l * K * 4,
+                                    d_w.data_ptr() + l * K * 4, K, s_out.data_ptr(), s_eo.data_ptr())
+            ctx.sync()
+            assert np.array_equal(s_out.cpu().numpy(), out[l]), l
+            assert np.array_equal(s_eo.cpu().numpy(), eo[l]), l
+            acc = np.zeros(H, np.float32)
+            for k in range(K):
+                acc = acc + w[l, k] * eo[l, k]
+            assert rel_err(out[l], acc) < 1e-6, l
+        for l in (0, 21, 39):
+            g, u, d = keep[l]
+            mg = np.concatenate([g.view(E, gsl)[int(e)].cpu().numpy() for e in idx[l]])
+            mu = np.concatenate([u.view(E, gsl)[int(e)].cpu().numpy() for e in idx[l]])
+            md = np.concatenate([d.view(E, dsl)[int(e)].cpu().numpy() for e in idx[l]])
+            ref, ref_eo = orc.moe_gguf_forward(mg, mu, md, x[l], np.arange(K, dtype=np.int32), w[l], H, I,
+                                               nthreads=8)
+            assert_parity(eo[l], ref_eo, "gguf expert_out layer %d" % l)
+            assert_parity(out[l], ref, "gguf layer %d" % l)
+    finally:
+        ctx.close()
+        del keep
+        torch.cuda.empty_cache()
