@@ -504,9 +504,10 @@ def run_moe_layer(args):
                                  [d_log.data_ptr(), d_seg.data_ptr(), d_sg.data_ptr(), d_su.data_ptr()])
             ctx.route_topk_dev(d_log.data_ptr(), E, K, d_seg.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(),
                                d_p.data_ptr())
-            ctx.moe_decode_dev(l, x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, d_moe.data_ptr(),
-                               d_eo.data_ptr())
-            ctx.layer_tail_dev(t_sd, h_mid.data_ptr(), d_eo.data_ptr(), d_p.data_ptr(), K, d_sg.data_ptr(),
+            # no buffer for the per-expert vectors: the experts' sum goes to d_moe, and the tail
+            # takes it as it is (K = 0 with a vector)
+            ctx.moe_decode_dev(l, x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, d_moe.data_ptr(), None)
+            ctx.layer_tail_dev(t_sd, h_mid.data_ptr(), d_moe.data_ptr(), d_p.data_ptr(), 0, d_sg.data_ptr(),
                                d_su.data_ptr(), nw.data_ptr(), 1e-6, hid[l & 1].data_ptr(), xin[l & 1].data_ptr())
 
     token()

@@ -13,12 +13,6 @@
 #include "fm_common.h"
 
 // ---- launchers implemented in the kernel files ------------------------------
-struct FmDenseSpec {
-    const uint8_t *W, *S, *B;
-    float *out;
-    int out_dim;
-    int first_item;
-};
 extern "C" {
 int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs, const FmExpertGeom *g,
                             int layer0, int layer_stride, int n_layers, const float *d_x,
@@ -27,6 +21,8 @@ int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs, const FmExpertGe
                             int n_cu, hipStream_t st, hipEvent_t *kev);
 int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
                     const float *d_x, int M, int n_cu, hipStream_t st);
+int fm_launch_dense_mixed(FmDenseSpec *specs, int n, int in_dim, int scale_fp16, const float *d_x,
+                          int n_cu, hipStream_t st);
 int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim, const float *d_x, int M,
                          hipStream_t st);
 int fm_launch_stream_probe(const void *d_buf, size_t nbytes, int pattern, unsigned int *d_sink,
@@ -876,6 +872,38 @@ static int matvec_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
     if (!ts || !d_x || !d_outs) return fail(c, FM_ERR_ARG, "null pointer");
     if (n < 1) return fail(c, FM_ERR_ARG, "n %d", n);
     DeviceGuard dg(c->device);
+    // One position, up to 8 small affine tensors of different code widths: one launch (each
+    // tensor's rows are computed as its own launch would; two launches would pay the start-up
+    // latency twice).  "Small": the whole batch is below the size from which a width's tensors
+    // take the streaming kernel.
+    if (M == 1 && n >= 2 && n <= 8) {
+        FmDenseSpec specs[8];
+        bool ok = true, mixed = false;
+        long rows = 0;
+        Tensor *t0 = get_tensor(c, ts[0]);
+        for (int k = 0; ok && k < n; k++) {
+            Tensor *t = get_tensor(c, ts[k]);
+            ok = t && t0 && !t->raw_bf16() && t->in_dim == t0->in_dim && t->scale_fp16 == t0->scale_fp16 &&
+                 t->group_size == 64 && d_outs[k] && (t->bits == 3 || t->bits == 4 || t->bits == 8);
+            if (!ok) break;
+            mixed = mixed || t->bits != t0->bits;
+            rows += t->out_dim;
+            specs[k].W = (const uint8_t *)t->W;
+            specs[k].S = (const uint8_t *)t->S;
+            specs[k].B = (const uint8_t *)t->B;
+            specs[k].out = d_outs[k];
+            specs[k].out_dim = t->out_dim;
+            specs[k].first_item = 0;
+            specs[k].bits = t->bits;
+        }
+        const int lpr = ok ? t0->in_dim / 128 : 0;
+        if (ok && mixed && lpr >= 1 && lpr <= 64 && rows * lpr / 64 < 8L * c->n_cu) {
+            int rc = fm_launch_dense_mixed(specs, n, t0->in_dim, t0->scale_fp16, d_x, c->n_cu, c->stream);
+            if (rc == FM_OK) return FM_OK;
+            if (rc != FM_ERR_UNSUPPORTED)
+                return fail(c, rc, "matvec launch failed: %s", hipGetErrorString(hipGetLastError()));
+        }
+    }
     // batches of up to 8 tensors with equal in_dim / bits / scale type
     int i = 0;
     while (i < n) {
@@ -897,6 +925,7 @@ static int matvec_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
             specs[m].out = d_outs[i];
             specs[m].out_dim = t->out_dim;
             specs[m].first_item = 0;
+            specs[m].bits = t->bits;
             m++;
             i++;
         }

@@ -49,6 +49,15 @@ struct FmDecodeFlags {
 // vectors
 #define FM_INT_NO_EXPERT_OUT (1 << 16)
 
+// One tensor of a dense GEMV launch (fm_dense.hip).
+struct FmDenseSpec {
+    const uint8_t *W, *S, *B;
+    float *out;
+    int out_dim;
+    int first_item;   // first workgroup of this tensor
+    int bits;         // code width (read by the launch of tensors of different widths only)
+};
+
 // Geometry of the GGUF slabs of one layer (finchmoe/infer.m:1017-1022).
 struct FmGgufGeom {
     int hidden, inter, n_experts;

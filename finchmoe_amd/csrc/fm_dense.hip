@@ -15,13 +15,6 @@
 
 #define FM_MAX_BATCH 8
 
-struct FmDenseSpec {
-    const uint8_t *W, *S, *B;
-    float *out;
-    int out_dim;
-    int first_item;   // first workgroup of this tensor
-};
-
 struct FmDenseArgs {
     FmDenseSpec spec[FM_MAX_BATCH];
     int n;
@@ -34,14 +27,19 @@ struct FmDenseArgs {
 
 namespace {
 
-template <int BITS, int LPR, bool FP16>
-__global__ __launch_bounds__(256) void fm_dense_gemv(FmDenseArgs a) {
-    constexpr int RPS = FM_WAVE / LPR;
-    constexpr int BPL = FmLaneBytes<BITS>::value;
+// the tensor a workgroup of the launch belongs to
+__device__ __forceinline__ int fm_dense_which(const FmDenseArgs &a) {
     int t = 0;
 #pragma unroll
     for (int i = 1; i < FM_MAX_BATCH; i++)
         if (i < a.n && (int)blockIdx.x >= a.spec[i].first_item) t = i;
+    return t;
+}
+
+template <int BITS, int LPR, bool FP16>
+__device__ __forceinline__ void fm_dense_gemv_rows(const FmDenseArgs &a, int t) {
+    constexpr int RPS = FM_WAVE / LPR;
+    constexpr int BPL = FmLaneBytes<BITS>::value;
     const FmDenseSpec sp = a.spec[t];
     const int chunk = blockIdx.x - sp.first_item;
     const int m = blockIdx.y;
@@ -83,6 +81,26 @@ __global__ __launch_bounds__(256) void fm_dense_gemv(FmDenseArgs a) {
         if (c == 0 && row <= last_row) out[row] = v;
         row += RPS;
         cur = next;
+    }
+}
+
+template <int BITS, int LPR, bool FP16>
+__global__ __launch_bounds__(256) void fm_dense_gemv(FmDenseArgs a) {
+    fm_dense_gemv_rows<BITS, LPR, FP16>(a, fm_dense_which(a));
+}
+
+// Tensors of different code widths in one launch (the routing batch of a layer: the 8-bit
+// router and the 4-bit shared-expert projections read the same x, finchmoe/infer.m:9285-9300;
+// two launches cost twice the start-up latency, which is most of a launch this small).  Every
+// workgroup runs the rows of one tensor with that tensor's arithmetic, exactly as the launch
+// of one width does.
+template <int LPR, bool FP16>
+__global__ __launch_bounds__(256) void fm_dense_gemv_mixed(FmDenseArgs a) {
+    const int t = fm_dense_which(a);
+    switch (a.spec[t].bits) {
+        case 3: fm_dense_gemv_rows<3, LPR, FP16>(a, t); break;
+        case 8: fm_dense_gemv_rows<8, LPR, FP16>(a, t); break;
+        default: fm_dense_gemv_rows<4, LPR, FP16>(a, t); break;
     }
 }
 
@@ -401,6 +419,53 @@ extern "C" int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim,
     const dim3 grid((rows + 3) / 4, M);
     if (vec) hipLaunchKernelGGL(fm_dense_bf16<true>, grid, dim3(256), 0, st, a, rows);
     else hipLaunchKernelGGL(fm_dense_bf16<false>, grid, dim3(256), 0, st, a, rows);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
+
+// Tensors of different widths (specs[i].bits in {3, 4, 8}), one position, plain kernel.
+extern "C" int fm_launch_dense_mixed(FmDenseSpec *specs, int n, int in_dim, int scale_fp16,
+                                     const float *d_x, int n_cu, hipStream_t st) {
+    if (n < 1 || n > FM_MAX_BATCH) return FM_ERR_ARG;
+    const int lpr = in_dim / FM_CPL;
+    if (lpr < 1 || lpr > 64 || (lpr & (lpr - 1)) || in_dim % FM_CPL) return FM_ERR_UNSUPPORTED;
+    const int min_rows = 4 * (FM_WAVE / lpr);
+    long total_rows = 0;
+    for (int i = 0; i < n; i++) {
+        if (specs[i].bits != 3 && specs[i].bits != 4 && specs[i].bits != 8) return FM_ERR_UNSUPPORTED;
+        total_rows += specs[i].out_dim;
+    }
+    int rpi = min_rows;     // as fm_launch_dense
+    while (rpi * 2 <= 8 * min_rows && (total_rows + rpi - 1) / rpi > 2L * n_cu) rpi *= 2;
+    FmDenseArgs a;
+    a.n = n;
+    a.in_dim = in_dim;
+    a.rows_per_item = rpi;
+    a.x = d_x;
+    a.out_stride = 0;
+    int items = 0;
+    for (int i = 0; i < n; i++) {
+        specs[i].first_item = items;
+        items += (specs[i].out_dim + rpi - 1) / rpi;
+        a.spec[i] = specs[i];
+    }
+    for (int i = n; i < FM_MAX_BATCH; i++) a.spec[i] = a.spec[0];
+    const dim3 grid(items), b(256);
+#define FM_DM(L)                                                                           \
+    do {                                                                                   \
+        if (scale_fp16) hipLaunchKernelGGL((fm_dense_gemv_mixed<L, true>), grid, b, 0, st, a);  \
+        else hipLaunchKernelGGL((fm_dense_gemv_mixed<L, false>), grid, b, 0, st, a);       \
+    } while (0)
+    switch (lpr) {
+        case 1: FM_DM(1); break;
+        case 2: FM_DM(2); break;
+        case 4: FM_DM(4); break;
+        case 8: FM_DM(8); break;
+        case 16: FM_DM(16); break;
+        case 32: FM_DM(32); break;
+        case 64: FM_DM(64); break;
+        default: return FM_ERR_UNSUPPORTED;
+    }
+#undef FM_DM
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 

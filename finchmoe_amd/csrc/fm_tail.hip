@@ -2,7 +2,7 @@
 // after the routed experts (finchmoe/infer.m:9608-9760), in one launch:
 //   shared expert   act = SwiGLU(shared_gate, shared_up)          (shaders.metal:1056-1068)
 //                   shared_out = down_proj(act), affine 4-bit      (infer.m:9629-9634)
-//   combine         hidden = h_mid + sum_k params[k] * expert_out[k]
+//   combine         hidden = h_mid + sum_k params[k] * expert_out[k]   (or the sum, ready-made)
 //                            + sigmoid(params[8]) * shared_out     (shaders.metal:2196-2231)
 //   next input      rms_norm(hidden) * bf16 weights of the next layer's input norm
 //                                                                  (shaders.metal:1134-1205)
@@ -48,6 +48,9 @@ __global__ __launch_bounds__(256) void fm_layer_tail(FmTailArgs a) {
         eo[k] = k < a.K ? a.expert_out[(size_t)k * a.hidden + row] : 0.0f;
         pw[k] = k < a.K ? a.params[k] : 0.0f;
     }
+    // K == 0 with a vector: the routed experts' sum is there already (fm_moe_decode_dev without
+    // a buffer for the per-expert vectors adds them up in the same slot order)
+    const float pre = (a.K == 0 && a.expert_out) ? a.expert_out[row] : 0.0f;
     const float hm = a.h_mid[row], score = a.params[8];
     for (int j = threadIdx.x; j < a.inter; j += blockDim.x)
         tail_act[j] = fm_silu_mul(a.shared_gate[j], a.shared_up[j]);
@@ -58,7 +61,7 @@ __global__ __launch_bounds__(256) void fm_layer_tail(FmTailArgs a) {
 
     float sq = 0.0f;
     if (c == 0) {
-        float moe = 0.0f;
+        float moe = pre;
 #pragma unroll
         for (int k = 0; k < FM_MAX_K; k++)
             if (k < a.K) moe += pw[k] * eo[k];

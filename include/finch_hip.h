@@ -235,6 +235,10 @@ FM_API int fm_route_topk_dev(fm_ctx *ctx, const float *d_logits, int n_experts, 
  *   params[10] = expert weights 0..7 (0 for an invalid slot), shared gate score
  *   at [8] (buf_combine_params), shared_gate / shared_up [shared_inter],
  *   next_norm_w[hidden] bf16 + next_input[hidden], both NULL for the last layer.
+ *   K == 0 with expert_out != NULL: expert_out is ONE vector [hidden], the routed experts'
+ *   weighted sum as fm_moe_decode_dev leaves it in `out` when it is called without a buffer
+ *   for the per-expert vectors (same slot order, same arithmetic: the results are identical,
+ *   and the expert launch is the faster one that never writes the K vectors).
  * hidden_out = h_mid + sum_k params[k]*expert_out[k] + sigmoid(params[8])*shared_out;
  * next_input = hidden_out / sqrt(mean(hidden_out^2) + eps) * next_norm_w.
  * All pointers device memory; asynchronous on the context's stream. */

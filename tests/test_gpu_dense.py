@@ -233,3 +233,25 @@ def test_raw_bf16_in_a_mixed_batch(hip, orc):
     assert_parity(o3, orc.dequant_matvec(c[1], c[2], c[3], x, 64, 2048, 4), "4-bit last")
     for t in (t4, tb, t4b):
         hip.tensor_release(t)
+
+
+def test_mixed_widths_in_one_batch_equal_separate_calls(hip, orc):
+    """The routing batch of a layer — 8-bit router and shared-gate score, 4-bit shared gate/up,
+    one x (finchmoe/infer.m:9285-9300) — goes out as one launch; every output equals, bit for
+    bit, the tensor's own call, and the oracle within the bar.  A 3-bit tensor joins too."""
+    rng = np.random.default_rng(77)
+    Hh = 2048
+    shapes = [(256, 8), (1, 8), (512, 4), (512, 4), (96, 3)]
+    tens, handles = [], []
+    for rows, bits in shapes:
+        t = F.synth_affine_tensor(rng, rows, Hh, bits)
+        tens.append(t)
+        handles.append(hip.tensor_register(t[1], t[2], t[3], rows, Hh, bits))
+    x = rng.standard_normal(Hh).astype(np.float32)
+    outs = hip.matvec_batch(handles, x, [r for r, _ in shapes])
+    for (rows, bits), t, h, got in zip(shapes, tens, handles, outs):
+        (alone,) = hip.matvec_batch([h], x, [rows])
+        assert np.array_equal(got, alone), (rows, bits)
+        assert_parity(got, orc.dequant_matvec(t[1], t[2], t[3], x, rows, Hh, bits), "%d rows at %d bits" % (rows, bits))
+    for h in handles:
+        hip.tensor_release(h)

@@ -39,7 +39,7 @@ def _run(hip, orc, rng, hidden, si, bits, K, dtype="bf16", with_norm=True, score
         d_hid.zero_()
         d_next.zero_()
         torch.cuda.synchronize()
-        hip.layer_tail_dev(t, dev[0].data_ptr(), dev[1].data_ptr(), dev[2].data_ptr(), K,
+        hip.layer_tail_dev(t, dev[0].data_ptr(), dev[1].data_ptr() if K else None, dev[2].data_ptr(), K,
                            dev[3].data_ptr(), dev[4].data_ptr(),
                            d_nw.data_ptr() if with_norm else None, 1e-6, d_hid.data_ptr(),
                            d_next.data_ptr() if with_norm else None)
@@ -202,5 +202,15 @@ def _moe_half(hip, orc):
     ref_h, ref_n = orc.layer_tail(*sdt[1:], h_mid, ref_eo, params, Kk, sg, su, nw)
     assert_parity(d_hid.cpu().numpy(), ref_h, "hidden")
     assert_parity(d_next.cpu().numpy(), ref_n, "next input")
+    # the shorter chain: no buffer for the per-expert vectors, the tail takes the experts' sum
+    # (K = 0 with a vector) — identical results
+    d_moe2 = torch.empty(Hh, device="cuda")
+    d_hid2, d_next2 = torch.empty(Hh, device="cuda"), torch.empty(Hh, device="cuda")
+    torch.cuda.synchronize()
+    hip.moe_decode_dev(0, d_x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), Kk, d_moe2.data_ptr(), None)
+    hip.layer_tail_dev(t_sd, d_hmid.data_ptr(), d_moe2.data_ptr(), d_p.data_ptr(), 0, d_sg.data_ptr(),
+                       d_su.data_ptr(), d_nw.data_ptr(), 1e-6, d_hid2.data_ptr(), d_next2.data_ptr())
+    hip.sync()
+    assert torch.equal(d_moe2, d_moe) and torch.equal(d_hid2, d_hid) and torch.equal(d_next2, d_next)
     for t in (t_gate, t_seg, t_sg, t_su, t_sd):
         hip.tensor_release(t)
