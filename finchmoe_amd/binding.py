@@ -62,6 +62,8 @@ def load():
         "fm_timer_stop": (i, [vp, C.POINTER(C.c_float)]),
         "fm_kernel_timing": (i, [vp, i]),
         "fm_set_wait_limit": (i, [vp, C.c_uint]),
+        "fm_reserve": (i, [vp, i, i, C.c_size_t]),
+        "fm_release_graphs": (i, [vp]),
         "fm_kernel_timing_read": (i, [vp, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i)]),
         "fm_stream_probe_dev": (i, [vp, vp, sz, i]),
         "fm_experts_config": (i, [vp, i, i, i, i, i, i, i]),
@@ -165,6 +167,13 @@ class FinchHip:
 
     def set_wait_limit(self, polls):
         self._chk(self.L.fm_set_wait_limit(self.h, C.c_uint(polls)))
+
+    def reserve(self, n_groups=0, M=0, workspace_bytes=0):
+        """Scratch for steps of n_groups layers / chunks of M positions, before capturing."""
+        self._chk(self.L.fm_reserve(self.h, n_groups, M, workspace_bytes))
+
+    def release_graphs(self):
+        self._chk(self.L.fm_release_graphs(self.h))
 
     def kernel_timing_read(self):
         a, b, n = C.c_double(), C.c_double(), C.c_int()

@@ -8,6 +8,7 @@
 
 #include <mutex>
 #include <string>
+#include <algorithm>
 #include <vector>
 
 #include "fm_common.h"
@@ -97,6 +98,8 @@ struct LayerBuf {
 
 }  // namespace
 
+#define FM_TAIL_PARTIALS 4096
+
 struct fm_ctx {
     int device = 0;
     int n_cu = 256;
@@ -109,6 +112,7 @@ struct fm_ctx {
     // dependency counters (allocated with the scratch)
     unsigned int *h_err = nullptr, *d_err = nullptr;
     FmDecodeFlags dflags{};
+    bool scratch_pinned = false;   // a call has been issued under stream capture
     unsigned int wait_limit = 1u << 20;
     bool split_phases = false;     // run the phases as separate kernels
     bool sync_unchecked = false;   // a fused launch has not had its error flag read yet
@@ -194,8 +198,28 @@ int ensure_stage(fm_ctx *c, size_t bytes) {
     return FM_OK;
 }
 
+// A graph captured from this context's stream has the scratch addresses of the moment baked in:
+// from the first call issued under capture on, the scratch buffers are pinned — a call that
+// would have to reallocate them is refused instead (FM_ERR_STATE), until fm_release_graphs().
+// Sizes are reserved before capturing with fm_reserve().
+bool note_capture(fm_ctx *c) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(c->stream, &cs);
+    const bool capturing = cs == hipStreamCaptureStatusActive;
+    if (capturing) c->scratch_pinned = true;
+    return capturing;
+}
+int refuse_growth(fm_ctx *c, const char *what) {
+    return fail(c, FM_ERR_STATE,
+                "%s would have to grow, but a captured graph holds the current addresses: call "
+                "fm_reserve() before capturing (or fm_release_graphs() once the graphs are gone)", what);
+}
+
 int ensure_ws(fm_ctx *c, size_t bytes) {
+    note_capture(c);
     if (c->ws_bytes >= bytes) return FM_OK;
+    if (c->scratch_pinned) return refuse_growth(c, "the workspace");
+    HIPCHK(c, hipStreamSynchronize(c->stream));    // queued work may still use the old one
     if (c->d_ws) HIPCHK(c, hipFree(c->d_ws));
     c->d_ws = nullptr;
     c->ws_bytes = 0;
@@ -206,8 +230,10 @@ int ensure_ws(fm_ctx *c, size_t bytes) {
 
 // scratch for `groups` groups (layers of a step, or positions of a chunk)
 int ensure_scratch(fm_ctx *c, int groups, int hidden, int inter) {
+    note_capture(c);
     if (groups <= c->cap_groups && hidden <= c->cap_hidden && inter <= c->cap_inter)
         return FM_OK;
+    if (c->scratch_pinned) return refuse_growth(c, "the expert scratch");
     int g = groups > c->cap_groups ? groups : c->cap_groups;
     int h = hidden > c->cap_hidden ? hidden : c->cap_hidden;
     int in = inter > c->cap_inter ? inter : c->cap_inter;
@@ -420,6 +446,42 @@ extern "C" int fm_set_wait_limit(fm_ctx *c, unsigned int polls) {
     if (!c) return FM_ERR_ARG;
     c->wait_limit = polls;
     c->dflags.spin_limit = polls;
+    return FM_OK;
+}
+
+// Scratch for steps of up to n_groups layers and chunks of up to M positions on the configured
+// stores, the layer tail's scratch, and at least workspace_bytes of workspace — so that no
+// later call of those sizes allocates (a precondition for capturing calls into a HIP graph).
+extern "C" int fm_reserve(fm_ctx *c, int n_groups, int M, size_t workspace_bytes) {
+    if (!c) return FM_ERR_ARG;
+    if (n_groups < 0 || M < 0) return fail(c, FM_ERR_ARG, "negative size");
+    DeviceGuard dg(c->device);
+    if (note_capture(c)) return fail(c, FM_ERR_STATE, "fm_reserve under stream capture");
+    const int groups = n_groups > M ? n_groups : M;   // small chunks run as groups of the decode kernels
+    int rc = FM_OK;
+    size_t ws = workspace_bytes;
+    if (c->aff_cfg) {
+        if (groups > 0 && (rc = ensure_scratch(c, groups, c->geom.hidden, c->geom.inter))) return rc;
+        if (M > 0) {
+            const size_t widen = (size_t)M * c->geom.hidden * sizeof(float);
+            const size_t a0 = fm_prefill_affine_ws_bytes(&c->geom, M, FM_MAX_K, 0);
+            const size_t a1 = fm_prefill_affine_ws_bytes(&c->geom, M, FM_MAX_K, 1);
+            ws = std::max(ws, std::max(widen, std::max(a0, a1)));
+        }
+    }
+    if (c->gguf_cfg && groups > 0 && (rc = ensure_scratch(c, groups, c->ggeom.hidden, c->ggeom.inter))) return rc;
+    if (ws && (rc = ensure_ws(c, ws))) return rc;
+    if (!c->d_tail) {
+        HIPCHK(c, hipMalloc((void **)&c->d_tail, (FM_TAIL_PARTIALS + 64) * sizeof(float)));
+        HIPCHK(c, hipMemsetAsync(c->d_tail, 0, (FM_TAIL_PARTIALS + 64) * sizeof(float), c->stream));
+    }
+    return FM_OK;
+}
+
+// The caller no longer replays any graph captured from this context: scratch may move again.
+extern "C" int fm_release_graphs(fm_ctx *c) {
+    if (!c) return FM_ERR_ARG;
+    c->scratch_pinned = false;
     return FM_OK;
 }
 
@@ -1076,7 +1138,6 @@ extern "C" int fm_route_topk_dev(fm_ctx *c, const float *d_logits, int n_experts
 // ============================================================================
 // layer tail
 // ============================================================================
-#define FM_TAIL_PARTIALS 4096
 
 extern "C" int fm_layer_tail_dev(fm_ctx *c, fm_tensor shared_down, const float *d_h_mid,
                                  const float *d_expert_out, const float *d_params, int K,
@@ -1099,6 +1160,7 @@ extern "C" int fm_layer_tail_dev(fm_ctx *c, fm_tensor shared_down, const float *
     if (t->out_dim / 4 > FM_TAIL_PARTIALS) return fail(c, FM_ERR_UNSUPPORTED, "hidden %d", t->out_dim);
     DeviceGuard dg(c->device);
     if (!c->d_tail) {
+        if (note_capture(c)) return refuse_growth(c, "the layer tail's scratch");
         HIPCHK(c, hipMalloc((void **)&c->d_tail, (FM_TAIL_PARTIALS + 64) * sizeof(float)));
         HIPCHK(c, hipMemsetAsync(c->d_tail, 0, (FM_TAIL_PARTIALS + 64) * sizeof(float), c->stream));
     }

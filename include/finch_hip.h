@@ -101,6 +101,17 @@ FM_API int fm_kernel_timing(fm_ctx *ctx, int mode);
  * counterpart in the reference (its kernels are separate Metal dispatches). */
 FM_API int fm_set_wait_limit(fm_ctx *ctx, unsigned int polls);
 /* sums in milliseconds since the last read, and the number of calls; resets */
+/* Calls captured into a HIP graph (hipStreamBeginCapture on fm_stream()).  A graph records the
+ * addresses of the context's scratch buffers, which grow on demand otherwise.  So: reserve
+ * first — scratch for steps of up to n_groups layers and chunks of up to M positions on the
+ * configured stores, the layer tail's scratch, at least workspace_bytes of workspace (dense
+ * prefill products) — then capture.  From the first call issued under capture on, a call that
+ * would have to grow a buffer returns FM_ERR_STATE instead of moving it under the graph's
+ * feet; fm_release_graphs() lifts that once no such graph will be replayed.  No counterpart in
+ * the reference (its command buffers are re-encoded per token). */
+FM_API int fm_reserve(fm_ctx *ctx, int n_groups, int M, size_t workspace_bytes);
+FM_API int fm_release_graphs(fm_ctx *ctx);
+
 FM_API int fm_kernel_timing_read(fm_ctx *ctx, double *gate_up_ms, double *down_ms, int *calls);
 
 /* Streaming probe: reads nbytes (whole 4 KB slots) of the device buffer d_buf once, with the

@@ -148,3 +148,46 @@ def test_moe_half_of_a_layer_replayed_from_graph():
         hip.hipGraphDestroy(graph)
     finally:
         ctx.close()
+
+
+def test_scratch_is_pinned_by_a_capture_and_reserved_beforehand():
+    """A graph holds the scratch addresses of its capture: sizes are reserved first
+    (fm_reserve), a later call that would have to grow the scratch is refused with a state
+    error instead of moving it, the graph still replays correctly, and fm_release_graphs lifts
+    the pin."""
+    import torch
+    from finchmoe_amd import FinchHip, FinchError
+    hip = _hip()
+    rng = np.random.default_rng(41)
+    ctx = FinchHip(0)
+    try:
+        ctx.experts_config(L, E, H, I, 64, 3, fb.SCALE_BF16)
+        for l in range(L):
+            ctx.experts_upload_layer(l, F.synth_expert_layer(rng, E, H, I, 3))
+        x = torch.from_numpy(rng.standard_normal((L, H)).astype(np.float32)).cuda()
+        idx = torch.from_numpy(np.stack([rng.permutation(E)[:K] for _ in range(L)]).astype(np.int32)).cuda()
+        w = torch.full((L, K), 1.0 / K, device="cuda")
+        d_out, d_ref = torch.zeros(L, H, device="cuda"), torch.zeros(L, H, device="cuda")
+        ctx.reserve(n_groups=2)                       # enough for steps of two layers
+        ctx.moe_decode_step_dev(0, 2, x.data_ptr(), idx.data_ptr(), w.data_ptr(), K, d_ref.data_ptr())
+        ctx.sync()
+        stream = C.c_void_p(ctx.stream())
+        graph, gexec = C.c_void_p(), C.c_void_p()
+        assert hip.hipStreamBeginCapture(stream, 2) == 0
+        ctx.moe_decode_step_dev(0, 2, x.data_ptr(), idx.data_ptr(), w.data_ptr(), K, d_out.data_ptr())
+        assert hip.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        with pytest.raises(FinchError) as e:          # six layers need more scratch than reserved
+            ctx.moe_decode_step_dev(0, L, x.data_ptr(), idx.data_ptr(), w.data_ptr(), K, d_ref.data_ptr())
+        assert e.value.status == fb.ERR_STATE and "fm_reserve" in str(e.value)
+        assert hip.hipGraphLaunch(gexec, stream) == 0
+        ctx.sync()
+        assert torch.equal(d_out[:2], d_ref[:2])
+        hip.hipGraphExecDestroy(gexec)
+        hip.hipGraphDestroy(graph)
+        ctx.release_graphs()
+        ctx.moe_decode_step_dev(0, L, x.data_ptr(), idx.data_ptr(), w.data_ptr(), K, d_out.data_ptr())
+        ctx.sync()
+        assert torch.isfinite(d_out).all() and torch.equal(d_out[:2], d_ref[:2])
+    finally:
+        ctx.close()
