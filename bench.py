@@ -450,8 +450,8 @@ def run_moe_layer(args):
     """The MoE half of every layer without a host round trip, one token per step: routing and
     shared-expert GEMVs (8-bit gate [256,2048] and shared-gate score, 4-bit shared gate/up
     [512,2048]) -> softmax/top-8 -> routed experts -> shared down + combine + residual + next
-    layer's norm (finchmoe/infer.m:9285-9760), layer l+1 reading what layer l wrote.  Four
-    launches per layer; with --graph the whole token is one captured HIP graph."""
+    layer's norm (finchmoe/infer.m:9285-9760), layer l+1 reading what layer l wrote.  Three
+    launches per layer (the GEMV batch's last workgroup routes); with --graph the whole token is one captured HIP graph."""
     import ctypes as C
     import torch
     from finchmoe_amd import FinchHip, formats
@@ -500,10 +500,9 @@ def run_moe_layer(args):
             t_gate, t_seg, t_sg, t_su, t_sd = layers[l]
             x = x0 if l == 0 else xin[(l - 1) & 1]
             h_mid = x0 if l == 0 else hid[(l - 1) & 1]
-            ctx.matvec_batch_dev([t_gate, t_seg, t_sg, t_su], x.data_ptr(),
-                                 [d_log.data_ptr(), d_seg.data_ptr(), d_sg.data_ptr(), d_su.data_ptr()])
-            ctx.route_topk_dev(d_log.data_ptr(), E, K, d_seg.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(),
-                               d_p.data_ptr())
+            ctx.matvec_batch_route_dev([t_gate, t_seg, t_sg, t_su], x.data_ptr(),
+                                       [d_log.data_ptr(), d_seg.data_ptr(), d_sg.data_ptr(), d_su.data_ptr()],
+                                       K, d_seg.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), d_p.data_ptr())
             # no buffer for the per-expert vectors: the experts' sum goes to d_moe, and the tail
             # takes it as it is (K = 0 with a vector)
             ctx.moe_decode_dev(l, x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, d_moe.data_ptr(), None)

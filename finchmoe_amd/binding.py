@@ -86,6 +86,7 @@ def load():
         "fm_matvec_prefill_dev": (i, [vp, i, vp, vp, i]),
         "fm_matvec_prefill": (i, [vp, i, vp, vp, i]),
         "fm_route_topk_dev": (i, [vp, vp, i, i, vp, vp, vp, vp]),
+        "fm_matvec_batch_route_dev": (i, [vp, C.POINTER(i), i, vp, C.POINTER(vp), i, vp, vp, vp, vp]),
         "fm_layer_tail_dev": (i, [vp, i, vp, vp, vp, i, vp, vp, vp, C.c_float, vp, vp]),
         "fm_gguf_config": (i, [vp, i, i, i, i, i, i, i]),
         "fm_gguf_upload_layer": (i, [vp, i, vp, sz, vp, sz, vp, sz]),
@@ -284,6 +285,14 @@ class FinchHip:
         ts = (C.c_int * n)(*tensors)
         ps = (C.c_void_p * n)(*d_outs)
         self._chk(self.L.fm_matvec_batch_dev(self.h, ts, n, d_x, ps))
+
+    def matvec_batch_route_dev(self, tensors, d_x, d_outs, K, d_seg_score, d_idx, d_w, d_params=None):
+        """matvec_batch_dev + route_topk_dev over tensors[0]'s outputs, one launch when it fits."""
+        n = len(tensors)
+        ts = (C.c_int * n)(*tensors)
+        ps = (C.c_void_p * n)(*d_outs)
+        self._chk(self.L.fm_matvec_batch_route_dev(self.h, ts, n, d_x, ps, K, d_seg_score, d_idx, d_w,
+                                                   d_params))
 
     def matvec_prefill(self, t, X, out_dim):
         X = _np(X, np.float32)

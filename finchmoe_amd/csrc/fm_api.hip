@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "fm_common.h"
+#include "fm_route.h"     // RouteArgs
 
 // ---- launchers implemented in the kernel files ------------------------------
 extern "C" {
@@ -23,7 +24,7 @@ int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs, const FmExpertGe
 int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
                     const float *d_x, int M, int n_cu, hipStream_t st);
 int fm_launch_dense_mixed(FmDenseSpec *specs, int n, int in_dim, int scale_fp16, const float *d_x,
-                          int n_cu, hipStream_t st);
+                          int n_cu, const RouteArgs *route, unsigned int *ticket, hipStream_t st);
 int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim, const float *d_x, int M,
                          hipStream_t st);
 int fm_launch_stream_probe(const void *d_buf, size_t nbytes, int pattern, unsigned int *d_sink,
@@ -930,7 +931,8 @@ extern "C" int fm_tensor_release(fm_ctx *c, fm_tensor t) {
 }
 
 static int matvec_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
-                      float *const *d_outs, int M) {
+                      float *const *d_outs, int M, const RouteArgs *route = nullptr,
+                      bool *routed = nullptr) {
     if (!ts || !d_x || !d_outs) return fail(c, FM_ERR_ARG, "null pointer");
     if (n < 1) return fail(c, FM_ERR_ARG, "n %d", n);
     DeviceGuard dg(c->device);
@@ -959,9 +961,14 @@ static int matvec_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
             specs[k].bits = t->bits;
         }
         const int lpr = ok ? t0->in_dim / 128 : 0;
-        if (ok && mixed && lpr >= 1 && lpr <= 64 && rows * lpr / 64 < 8L * c->n_cu) {
-            int rc = fm_launch_dense_mixed(specs, n, t0->in_dim, t0->scale_fp16, d_x, c->n_cu, c->stream);
-            if (rc == FM_OK) return FM_OK;
+        if (ok && (mixed || route) && lpr >= 1 && lpr <= 64 && rows * lpr / 64 < 8L * c->n_cu) {
+            unsigned int *ticket = route && c->d_tail ? (unsigned int *)(c->d_tail + FM_TAIL_PARTIALS) + 1 : nullptr;
+            int rc = fm_launch_dense_mixed(specs, n, t0->in_dim, t0->scale_fp16, d_x, c->n_cu,
+                                           ticket ? route : nullptr, ticket, c->stream);
+            if (rc == FM_OK) {
+                if (routed) *routed = ticket != nullptr;
+                return FM_OK;
+            }
             if (rc != FM_ERR_UNSUPPORTED)
                 return fail(c, rc, "matvec launch failed: %s", hipGetErrorString(hipGetLastError()));
         }
@@ -1004,6 +1011,31 @@ extern "C" int fm_matvec_batch_dev(fm_ctx *c, const fm_tensor *ts, int n, const 
                                    float *const *d_outs) {
     if (!c) return FM_ERR_ARG;
     return matvec_dev(c, ts, n, d_x, d_outs, 1);
+}
+
+static int ensure_tail_scratch(fm_ctx *c);
+
+// fm_matvec_batch_dev followed by fm_route_topk_dev over tensor 0's outputs, as ONE launch when
+// the batch is small enough for the plain kernel (the last workgroup to finish routes), else as
+// the two launches: the results are the same either way.
+extern "C" int fm_matvec_batch_route_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
+                                         float *const *d_outs, int K, const float *d_seg_score,
+                                         int32_t *d_idx, float *d_w, float *d_params) {
+    if (!c) return FM_ERR_ARG;
+    if (!ts || !d_outs || n < 1 || !d_idx || !d_w) return fail(c, FM_ERR_ARG, "null pointer");
+    Tensor *t0 = get_tensor(c, ts[0]);
+    if (!t0) return fail(c, FM_ERR_ARG, "bad tensor handle %d", ts[0]);
+    const int n_experts = t0->out_dim;
+    if (K < 1 || K > FM_MAX_K || K > n_experts)
+        return fail(c, FM_ERR_ARG, "K %d outside 1..min(%d, n_experts)", K, FM_MAX_K);
+    DeviceGuard dg(c->device);
+    int rc = ensure_tail_scratch(c);
+    if (rc) return rc;
+    const RouteArgs ra{d_outs[0], n_experts, K, d_seg_score, d_idx, d_w, d_params};
+    bool routed = false;
+    rc = matvec_dev(c, ts, n, d_x, d_outs, 1, &ra, &routed);
+    if (rc || routed) return rc;
+    return fm_route_topk_dev(c, d_outs[0], n_experts, K, d_seg_score, d_idx, d_w, d_params);
 }
 
 extern "C" size_t fm_prefill_dense_ws_bytes(int out_dim, int in_dim, int group_size, int bits, int M);
@@ -1139,6 +1171,15 @@ extern "C" int fm_route_topk_dev(fm_ctx *c, const float *d_logits, int n_experts
 // layer tail
 // ============================================================================
 
+// partial sums of the norm + the ticket words of the tail and of the fused routing
+static int ensure_tail_scratch(fm_ctx *c) {
+    if (c->d_tail) return FM_OK;
+    if (note_capture(c)) return refuse_growth(c, "the layer tail's scratch");
+    HIPCHK(c, hipMalloc((void **)&c->d_tail, (FM_TAIL_PARTIALS + 64) * sizeof(float)));
+    HIPCHK(c, hipMemsetAsync(c->d_tail, 0, (FM_TAIL_PARTIALS + 64) * sizeof(float), c->stream));
+    return FM_OK;
+}
+
 extern "C" int fm_layer_tail_dev(fm_ctx *c, fm_tensor shared_down, const float *d_h_mid,
                                  const float *d_expert_out, const float *d_params, int K,
                                  const float *d_shared_gate, const float *d_shared_up,
@@ -1159,11 +1200,8 @@ extern "C" int fm_layer_tail_dev(fm_ctx *c, fm_tensor shared_down, const float *
         return fail(c, FM_ERR_UNSUPPORTED, "shared down projection must be 3/4/8-bit, group size 64");
     if (t->out_dim / 4 > FM_TAIL_PARTIALS) return fail(c, FM_ERR_UNSUPPORTED, "hidden %d", t->out_dim);
     DeviceGuard dg(c->device);
-    if (!c->d_tail) {
-        if (note_capture(c)) return refuse_growth(c, "the layer tail's scratch");
-        HIPCHK(c, hipMalloc((void **)&c->d_tail, (FM_TAIL_PARTIALS + 64) * sizeof(float)));
-        HIPCHK(c, hipMemsetAsync(c->d_tail, 0, (FM_TAIL_PARTIALS + 64) * sizeof(float), c->stream));
-    }
+    int rc0 = ensure_tail_scratch(c);
+    if (rc0) return rc0;
     FmTailArgs a;
     a.W = (const uint8_t *)t->W;
     a.S = (const uint8_t *)t->S;

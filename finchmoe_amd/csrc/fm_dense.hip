@@ -10,6 +10,7 @@
 // contiguous in memory.
 #include "fm_mfma.h"
 #include "fm_ring.h"
+#include "fm_route.h"
 
 #include <type_traits>
 
@@ -23,6 +24,11 @@ struct FmDenseArgs {
     const float *x;      // [M][in_dim]
     size_t out_stride;   // elements between positions in every out (= out_dim of that tensor if 0)
     int unit_first[FM_MAX_BATCH + 1];   // streaming kernel: first wave step of every tensor
+    // fm_dense_gemv_mixed only: the token's routing over tensor 0's outputs, run by the
+    // workgroup that finishes last (route_ticket: a device word that is 0 between launches)
+    int route_on;
+    RouteArgs route;
+    unsigned int *route_ticket;
 };
 
 namespace {
@@ -47,7 +53,7 @@ __device__ __forceinline__ void fm_dense_gemv_rows(const FmDenseArgs &a, int t) 
     const int c = lane % LPR, r = lane / LPR;
     const int rows_per_wave = a.rows_per_item >> 2;
     const int row0 = chunk * a.rows_per_item + wave * rows_per_wave;
-    if (row0 >= sp.out_dim) return;
+    if (row0 >= sp.out_dim) return;          // (the wave comes back to its caller)
     int steps = rows_per_wave / RPS;
     {   // the last workgroup of a tensor may be short
         int left = (sp.out_dim - row0 + RPS - 1) / RPS;
@@ -78,7 +84,11 @@ __device__ __forceinline__ void fm_dense_gemv_rows(const FmDenseArgs &a, int t) 
                                 sp.B + ro * sb_row_bytes + (size_t)c * 4);
         }
         float v = fm_group_sum<LPR>(fm_lane_dot<BITS, FP16>(cur, xs, xsum0, xsum1));
-        if (c == 0 && row <= last_row) out[row] = v;
+        if (c == 0 && row <= last_row) {
+            // read later in this launch by another workgroup (the routing): stored at device scope
+            if (a.route_on) __hip_atomic_store(out + row, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else out[row] = v;
+        }
         row += RPS;
         cur = next;
     }
@@ -102,6 +112,22 @@ __global__ __launch_bounds__(256) void fm_dense_gemv_mixed(FmDenseArgs a) {
         case 8: fm_dense_gemv_rows<8, LPR, FP16>(a, t); break;
         default: fm_dense_gemv_rows<4, LPR, FP16>(a, t); break;
     }
+    if (!a.route_on) return;
+    // The routing (softmax, top-K, weights: fm_route.h) needs every logit: each workgroup takes
+    // a ticket once its rows are in memory, and the one that draws the last runs it — the
+    // pattern of the layer tail's norm (fm_tail.hip).
+    __shared__ float route_p[FM_ROUTE_MAX];
+    __shared__ unsigned int ticket;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's rows are in memory
+    __syncthreads();
+    if (threadIdx.x == 0)
+        ticket = __hip_atomic_fetch_add(a.route_ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket != gridDim.x - 1 || threadIdx.x >= 64) return;
+    __atomic_signal_fence(__ATOMIC_ACQUIRE);             // the loads below stay behind the ticket
+    fm_route_wave<true>(a.route, route_p);
+    if (threadIdx.x == 0)
+        __hip_atomic_store(a.route_ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ----------------------------------------------------------------------
@@ -406,6 +432,7 @@ extern "C" int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim,
     a.rows_per_item = 0;
     a.x = d_x;
     a.out_stride = 0;
+    a.route_on = 0;
     int rows = 0;
     bool vec = in_dim % 8 == 0 && ((uintptr_t)d_x & 15) == 0;
     for (int i = 0; i < n; i++) {
@@ -423,8 +450,11 @@ extern "C" int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim,
 }
 
 // Tensors of different widths (specs[i].bits in {3, 4, 8}), one position, plain kernel.
+// route (optional): the routing over specs[0]'s outputs in the same launch; ticket: a device word
+// that is zero between launches.
 extern "C" int fm_launch_dense_mixed(FmDenseSpec *specs, int n, int in_dim, int scale_fp16,
-                                     const float *d_x, int n_cu, hipStream_t st) {
+                                     const float *d_x, int n_cu, const RouteArgs *route,
+                                     unsigned int *ticket, hipStream_t st) {
     if (n < 1 || n > FM_MAX_BATCH) return FM_ERR_ARG;
     const int lpr = in_dim / FM_CPL;
     if (lpr < 1 || lpr > 64 || (lpr & (lpr - 1)) || in_dim % FM_CPL) return FM_ERR_UNSUPPORTED;
@@ -442,6 +472,7 @@ extern "C" int fm_launch_dense_mixed(FmDenseSpec *specs, int n, int in_dim, int 
     a.rows_per_item = rpi;
     a.x = d_x;
     a.out_stride = 0;
+    a.route_on = 0;
     int items = 0;
     for (int i = 0; i < n; i++) {
         specs[i].first_item = items;
@@ -449,6 +480,15 @@ extern "C" int fm_launch_dense_mixed(FmDenseSpec *specs, int n, int in_dim, int 
         a.spec[i] = specs[i];
     }
     for (int i = n; i < FM_MAX_BATCH; i++) a.spec[i] = a.spec[0];
+    a.route_on = 0;
+    if (route) {
+        if (!ticket || route->n < 1 || route->n > FM_ROUTE_MAX || route->K < 1 || route->K > FM_MAX_K ||
+            route->K > route->n || route->n != specs[0].out_dim)
+            return FM_ERR_UNSUPPORTED;
+        a.route_on = 1;
+        a.route = *route;
+        a.route_ticket = ticket;
+    }
     const dim3 grid(items), b(256);
 #define FM_DM(L)                                                                           \
     do {                                                                                   \
@@ -489,6 +529,7 @@ extern "C" int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, 
     a.rows_per_item = rpi;
     a.x = d_x;
     a.out_stride = 0;
+    a.route_on = 0;
     int items = 0;
     for (int i = 0; i < n; i++) {
         specs[i].first_item = items;

@@ -235,6 +235,16 @@ FM_API int fm_matvec_prefill(fm_ctx *ctx, fm_tensor t, const float *X, float *ou
 FM_API int fm_route_topk_dev(fm_ctx *ctx, const float *d_logits, int n_experts, int K,
                       const float *d_seg_score, int32_t *d_idx, float *d_w, float *d_params);
 
+/* fm_matvec_batch_dev followed by fm_route_topk_dev over tensor 0's outputs (the gate logits),
+ * as ONE launch when the batch is small enough for the plain GEMV kernel — the workgroup that
+ * finishes last routes — and as the two launches otherwise; same results either way.  The
+ * per-layer loop's first step: 8-bit mlp.gate + shared_expert_gate and the 4-bit shared
+ * gate/up projections on one x, then softmax/top-K (finchmoe/infer.m:9285-9300, 1794-1840).
+ * d_seg_score is normally d_outs[1]. */
+FM_API int fm_matvec_batch_route_dev(fm_ctx *ctx, const fm_tensor *tensors, int n, const float *d_x,
+                              float *const *d_outs, int K, const float *d_seg_score,
+                              int32_t *d_idx, float *d_w, float *d_params);
+
 /* ---------------------------------------------------------------- layer tail
  * Replaces the five dispatches the reference appends to a layer's expert command
  * buffer (finchmoe/infer.m:9608-9760): swiglu_fused on the shared expert's gate/up

@@ -212,5 +212,18 @@ def _moe_half(hip, orc):
                        d_su.data_ptr(), d_nw.data_ptr(), 1e-6, d_hid2.data_ptr(), d_next2.data_ptr())
     hip.sync()
     assert torch.equal(d_moe2, d_moe) and torch.equal(d_hid2, d_hid) and torch.equal(d_next2, d_next)
+    # and the first two launches as one (the GEMV batch's last workgroup routes): identical
+    keep = [t.clone() for t in (d_log, d_seg, d_sg, d_su, d_idx, d_w, d_p)]
+    for rep in range(3):       # the ticket word must come back to zero every time
+        for t in (d_log, d_seg, d_sg, d_su, d_w, d_p):
+            t.zero_()
+        d_idx.zero_()
+        torch.cuda.synchronize()
+        hip.matvec_batch_route_dev([t_gate, t_seg, t_sg, t_su], d_x.data_ptr(),
+                                   [d_log.data_ptr(), d_seg.data_ptr(), d_sg.data_ptr(), d_su.data_ptr()],
+                                   Kk, d_seg.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), d_p.data_ptr())
+        hip.sync()
+        for got, want in zip((d_log, d_seg, d_sg, d_su, d_idx, d_w, d_p), keep):
+            assert torch.equal(got, want), rep
     for t in (t_gate, t_seg, t_sg, t_su, t_sd):
         hip.tensor_release(t)
