@@ -22,7 +22,8 @@ int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs, const FmExpertGe
                             float *d_expert_out, float *d_out, FmDecodeFlags *df, int flags,
                             int n_cu, hipStream_t st, hipEvent_t *kev);
 int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
-                    const float *d_x, int M, int n_cu, hipStream_t st);
+                    const float *d_x, int M, int n_cu, hipStream_t st, const FmDenseSpec *riders,
+                    int n_riders, int *riders_done);
 int fm_launch_dense_mixed(FmDenseSpec *specs, int n, int in_dim, int scale_fp16, const float *d_x,
                           int n_cu, const RouteArgs *route, unsigned int *ticket, hipStream_t st);
 int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim, const float *d_x, int M,
@@ -998,11 +999,30 @@ static int matvec_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
             m++;
             i++;
         }
+        // up to two raw-BF16 tensors right behind an affine group can ride along in its launch
+        // (the b / a rows behind qkv / z, finchmoe/infer.m:8118-8122)
+        FmDenseSpec riders[2];
+        int n_riders = 0, riders_done = 0;
+        if (!t0->raw_bf16()) {
+            for (int k = i; k < n && n_riders < 2; k++) {
+                Tensor *t = get_tensor(c, ts[k]);
+                if (!t || !t->raw_bf16() || t->in_dim != t0->in_dim || !d_outs[k]) break;
+                riders[n_riders].W = (const uint8_t *)t->W;
+                riders[n_riders].S = riders[n_riders].B = nullptr;
+                riders[n_riders].out = d_outs[k];
+                riders[n_riders].out_dim = t->out_dim;
+                riders[n_riders].first_item = 0;
+                riders[n_riders].bits = 16;
+                n_riders++;
+            }
+        }
         int rc = t0->raw_bf16()
                      ? fm_launch_dense_bf16(specs, m, t0->in_dim, d_x, M, c->stream)
                      : fm_launch_dense(specs, m, t0->in_dim, t0->bits, t0->scale_fp16, d_x, M,
-                                       c->n_cu, c->stream);
+                                       c->n_cu, c->stream, n_riders ? riders : nullptr, n_riders,
+                                       &riders_done);
         if (rc) return fail(c, rc, "matvec launch failed: %s", hipGetErrorString(hipGetLastError()));
+        if (riders_done) i += n_riders;
     }
     return FM_OK;
 }

@@ -29,6 +29,11 @@ struct FmDenseArgs {
     int route_on;
     RouteArgs route;
     unsigned int *route_ticket;
+    // fm_dense_stream only: raw-BF16 tensors of a few rows that ride along (one row per wave,
+    // after the wave's share of the stream): rider r's rows are [rider_first[r], rider_first[r+1])
+    int n_riders;
+    FmDenseSpec rider[2];
+    int rider_first[3];
 };
 
 namespace {
@@ -128,6 +133,31 @@ __global__ __launch_bounds__(256) void fm_dense_gemv_mixed(FmDenseArgs a) {
     fm_route_wave<true>(a.route, route_p);
     if (threadIdx.x == 0)
         __hip_atomic_store(a.route_ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// one row of raw BF16 weights times x, by one wave (every lane receives the sum)
+template <bool VEC>
+__device__ __forceinline__ float fm_bf16_row(const uint16_t *w, const float *x, int in_dim, int lane) {
+    float acc = 0.0f;
+    if constexpr (VEC) {
+        for (int c = lane * 8; c < in_dim; c += 64 * 8) {
+            const uint4 q = *reinterpret_cast<const uint4 *>(w + c);
+            const float4 x0 = *reinterpret_cast<const float4 *>(x + c);
+            const float4 x1 = *reinterpret_cast<const float4 *>(x + c + 4);
+            acc = fmaf(fm_bf16_lo(q.x), x0.x, acc);
+            acc = fmaf(fm_bf16_hi(q.x), x0.y, acc);
+            acc = fmaf(fm_bf16_lo(q.y), x0.z, acc);
+            acc = fmaf(fm_bf16_hi(q.y), x0.w, acc);
+            acc = fmaf(fm_bf16_lo(q.z), x1.x, acc);
+            acc = fmaf(fm_bf16_hi(q.z), x1.y, acc);
+            acc = fmaf(fm_bf16_lo(q.w), x1.z, acc);
+            acc = fmaf(fm_bf16_hi(q.w), x1.w, acc);
+        }
+    } else {
+        for (int c = lane; c < in_dim; c += 64)
+            acc = fmaf(__uint_as_float((uint32_t)w[c] << 16), x[c], acc);
+    }
+    return fm_group_sum<64>(acc);
 }
 
 // ----------------------------------------------------------------------
@@ -306,6 +336,22 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
         if (ch == 0) w.out[(size_t)m * w.out_dim + w.row0 + ris] = v;
     }
     }
+    // riders: wave gw of the launch takes row gw of the raw-BF16 tensors (the in_proj_b /
+    // in_proj_a rows next to in_proj_qkv / in_proj_z: finchmoe/infer.m:8118-8122), so that the
+    // set is one launch
+    if (a.n_riders > 0) {
+        const int gw = (int)blockIdx.x * 8 + wave;
+        if (gw < a.rider_first[a.n_riders]) {
+            const int r = a.n_riders > 1 && gw >= a.rider_first[1] ? 1 : 0;
+            const FmDenseSpec sp = r ? a.rider[1] : a.rider[0];
+            const int row = gw - (r ? a.rider_first[1] : 0);
+            const uint16_t *w = reinterpret_cast<const uint16_t *>(sp.W) + (size_t)row * a.in_dim;
+            const float *x = a.x + (size_t)m * a.in_dim;
+            const bool vec = a.in_dim % 8 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0;
+            const float acc = vec ? fm_bf16_row<true>(w, x, a.in_dim, lane) : fm_bf16_row<false>(w, x, a.in_dim, lane);
+            if (lane == 0) sp.out[(size_t)m * sp.out_dim + row] = acc;
+        }
+    }
 #else
     (void)a;
     (void)total_units;
@@ -335,6 +381,7 @@ int launch_dense_stream_t(FmDenseArgs &a, int M, int n_cu, hipStream_t st) {
     if (units < 8L * n_cu) return FM_ERR_UNSUPPORTED;
     long wgs = n_cu;
     if (units < 8 * wgs) wgs = (units + 7) / 8;
+    if (a.n_riders > 0 && a.rider_first[a.n_riders] > 8 * wgs) a.n_riders = 0;   // one row per wave
     dim3 grid((unsigned)wgs, M);
 #define FM_DS(L, NS_)                                                                          \
     do {                                                                                       \
@@ -395,28 +442,8 @@ __global__ __launch_bounds__(256) void fm_dense_bf16(FmDenseArgs a, int total_ro
     const FmDenseSpec sp = a.spec[t];
     const int row = gr - a.unit_first[t];
     const int m = blockIdx.y;
-    const uint16_t *w = reinterpret_cast<const uint16_t *>(sp.W) + (size_t)row * a.in_dim;
-    const float *x = a.x + (size_t)m * a.in_dim;
-    float acc = 0.0f;
-    if constexpr (VEC) {
-        for (int c = lane * 8; c < a.in_dim; c += 64 * 8) {
-            const uint4 q = *reinterpret_cast<const uint4 *>(w + c);
-            const float4 x0 = *reinterpret_cast<const float4 *>(x + c);
-            const float4 x1 = *reinterpret_cast<const float4 *>(x + c + 4);
-            acc = fmaf(fm_bf16_lo(q.x), x0.x, acc);
-            acc = fmaf(fm_bf16_hi(q.x), x0.y, acc);
-            acc = fmaf(fm_bf16_lo(q.y), x0.z, acc);
-            acc = fmaf(fm_bf16_hi(q.y), x0.w, acc);
-            acc = fmaf(fm_bf16_lo(q.z), x1.x, acc);
-            acc = fmaf(fm_bf16_hi(q.z), x1.y, acc);
-            acc = fmaf(fm_bf16_lo(q.w), x1.z, acc);
-            acc = fmaf(fm_bf16_hi(q.w), x1.w, acc);
-        }
-    } else {
-        for (int c = lane; c < a.in_dim; c += 64)
-            acc = fmaf(__uint_as_float((uint32_t)w[c] << 16), x[c], acc);
-    }
-    acc = fm_group_sum<64>(acc);
+    const float acc = fm_bf16_row<VEC>(reinterpret_cast<const uint16_t *>(sp.W) + (size_t)row * a.in_dim,
+                                       a.x + (size_t)m * a.in_dim, a.in_dim, lane);
     if (lane == 0) sp.out[(size_t)m * sp.out_dim + row] = acc;
 }
 
@@ -433,6 +460,7 @@ extern "C" int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim,
     a.x = d_x;
     a.out_stride = 0;
     a.route_on = 0;
+    a.n_riders = 0;
     int rows = 0;
     bool vec = in_dim % 8 == 0 && ((uintptr_t)d_x & 15) == 0;
     for (int i = 0; i < n; i++) {
@@ -473,6 +501,7 @@ extern "C" int fm_launch_dense_mixed(FmDenseSpec *specs, int n, int in_dim, int 
     a.x = d_x;
     a.out_stride = 0;
     a.route_on = 0;
+    a.n_riders = 0;
     int items = 0;
     for (int i = 0; i < n; i++) {
         specs[i].first_item = items;
@@ -481,6 +510,7 @@ extern "C" int fm_launch_dense_mixed(FmDenseSpec *specs, int n, int in_dim, int 
     }
     for (int i = n; i < FM_MAX_BATCH; i++) a.spec[i] = a.spec[0];
     a.route_on = 0;
+    a.n_riders = 0;
     if (route) {
         if (!ticket || route->n < 1 || route->n > FM_ROUTE_MAX || route->K < 1 || route->K > FM_MAX_K ||
             route->K > route->n || route->n != specs[0].out_dim)
@@ -510,8 +540,12 @@ extern "C" int fm_launch_dense_mixed(FmDenseSpec *specs, int n, int in_dim, int 
 }
 
 // specs[i].first_item is filled here.  in_dim must be 128 * 2^j, j <= 6.
+// riders (optional, at most two): raw-BF16 tensors of a few rows computed in the same launch when
+// the streaming kernel takes it; *riders_done says whether they were.
 extern "C" int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
-                               const float *d_x, int M, int n_cu, hipStream_t st) {
+                               const float *d_x, int M, int n_cu, hipStream_t st,
+                               const FmDenseSpec *riders, int n_riders, int *riders_done) {
+    if (riders_done) *riders_done = 0;
     if (n < 1 || n > FM_MAX_BATCH || M < 1) return FM_ERR_ARG;
     const int lpr = in_dim / FM_CPL;
     if (lpr < 1 || lpr > 64 || (lpr & (lpr - 1)) || in_dim % FM_CPL) return FM_ERR_UNSUPPORTED;
@@ -530,6 +564,7 @@ extern "C" int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, 
     a.x = d_x;
     a.out_stride = 0;
     a.route_on = 0;
+    a.n_riders = 0;
     int items = 0;
     for (int i = 0; i < n; i++) {
         specs[i].first_item = items;
@@ -539,6 +574,18 @@ extern "C" int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, 
     for (int i = n; i < FM_MAX_BATCH; i++) a.spec[i] = a.spec[0];
     static const bool no_stream = getenv("FINCH_DENSE_VALU") != nullptr;
     if (!no_stream && (bits == 3 || bits == 4 || bits == 8)) {
+        if (riders && n_riders >= 1 && n_riders <= 2 && riders_done) {
+            a.n_riders = n_riders;
+            a.rider_first[0] = 0;
+            for (int i = 0; i < n_riders; i++) {
+                a.rider[i] = riders[i];
+                a.rider_first[i + 1] = a.rider_first[i] + riders[i].out_dim;
+            }
+            for (int i = n_riders; i < 2; i++) {
+                a.rider[i] = a.rider[0];
+                a.rider_first[i + 1] = a.rider_first[n_riders];
+            }
+        }
         int rc = FM_ERR_UNSUPPORTED;
         if (bits == 3) rc = scale_fp16 ? launch_dense_stream_t<3, true>(a, M, n_cu, st)
                                        : launch_dense_stream_t<3, false>(a, M, n_cu, st);
@@ -546,7 +593,11 @@ extern "C" int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, 
                                             : launch_dense_stream_t<8, false>(a, M, n_cu, st);
         else rc = scale_fp16 ? launch_dense_stream_t<4, true>(a, M, n_cu, st)
                              : launch_dense_stream_t<4, false>(a, M, n_cu, st);
-        if (rc != FM_ERR_UNSUPPORTED) return rc;
+        if (rc != FM_ERR_UNSUPPORTED) {
+            if (riders_done && rc == FM_OK) *riders_done = a.n_riders > 0;
+            return rc;
+        }
+        a.n_riders = 0;
     }
     switch (bits) {
         case 3: return scale_fp16 ? launch_dense_t<3, true>(a, items, M, st)

@@ -255,3 +255,31 @@ def test_mixed_widths_in_one_batch_equal_separate_calls(hip, orc):
         assert_parity(got, orc.dequant_matvec(t[1], t[2], t[3], x, rows, Hh, bits), "%d rows at %d bits" % (rows, bits))
     for h in handles:
         hip.tensor_release(h)
+
+
+def test_gdn_set_is_one_launch_with_riders(hip, orc):
+    """The reference's four-spec batch {qkv 8192, z 4096, b 32, a 32} on one x
+    (finchmoe/infer.m:8118-8122): the two raw-BF16 tensors ride along in the streaming launch
+    of the 4-bit ones.  Every output equals, bit for bit, what the launches without riders give,
+    and the oracle within the bar."""
+    rng = np.random.default_rng(78)
+    Hh = 2048
+    q4 = [F.synth_affine_tensor(rng, rows, Hh, 4) for rows in (8192, 4096)]
+    raw = [F.bf16_trunc(rng.standard_normal((32, Hh)).astype(np.float32) * np.float32(0.1)) for _ in range(2)]
+    hs = [hip.tensor_register(t[1], t[2], t[3], rows, Hh, 4) for t, rows in zip(q4, (8192, 4096))]
+    hs += [hip.tensor_register(w, None, None, 32, Hh) for w in raw]
+    dims = [8192, 4096, 32, 32]
+    x = rng.standard_normal(Hh).astype(np.float32)
+    outs = hip.matvec_batch(hs, x, dims)
+    # the 4-bit pair without riders (same kernel), the raw tensors on their own
+    for got, want in zip(outs[:2], hip.matvec_batch(hs[:2], x, dims[:2])):
+        assert np.array_equal(got, want)
+    for h, got in zip(hs[2:], outs[2:]):
+        (alone,) = hip.matvec_batch([h], x, [32])
+        assert np.array_equal(got, alone)
+    for t, rows, got in zip(q4, (8192, 4096), outs[:2]):
+        assert_parity(got, orc.dequant_matvec(t[1], t[2], t[3], x, rows, Hh, 4), "%d rows" % rows)
+    for w, got in zip(raw, outs[2:]):
+        assert_parity(got, orc.dequant_matvec(w, None, None, x, 32, Hh, 0), "raw BF16")
+    for h in hs:
+        hip.tensor_release(h)
