@@ -607,11 +607,12 @@ def run_gguf(args):
         keep.extend([g, u, d])
         ctx.gguf_adopt_layer(l, g.data_ptr(), g.numel(), u.data_ptr(), u.numel(), d.data_ptr(), d.numel())
     rng = np.random.default_rng(7)
-    tokens = 64
+    tokens = max(64, args.chunk) if args.workload == "gguf_chunk" else 64
     idx, w = zipf_routing(rng, tokens, n_layers, E, K)
     if args.workload == "gguf_chunk":
-        # the chunked-prefill variant of config 4: M positions of one layer per call (per-position
-        # products, as the reference runs them), the layer changes from call to call
+        # the chunked-prefill variant of config 4: M positions of one layer per call (grouped
+        # products from 32 positions on, per-position products below, as the reference runs
+        # them; FINCH_GGUF_NO_GROUP=1 forces the latter), the layer changes from call to call
         M = args.chunk if args.chunk <= tokens else 8
         c_idx = torch.from_numpy(np.ascontiguousarray(idx.transpose(1, 0, 2))).to(dev)   # [layer][token][k]
         c_w = torch.from_numpy(np.ascontiguousarray(w.transpose(1, 0, 2))).to(dev)
@@ -631,7 +632,7 @@ def run_gguf(args):
         return _finish({"event_ms_per_step": round(ev, 5)},
                        "GGUF Q4_K/Q6_K expert GEMV HBM GB/s, %d-position chunk of one layer" % M,
                        "config 4, chunk variant: %d positions x top-8 Zipf(1.1) on one of %d GGUF layers "
-                       "(Q4_K gate/up, Q6_K down), per-position products" % (M, n_layers),
+                       "(Q4_K gate/up, Q6_K down), %s products" % (M, n_layers, "grouped" if M >= 32 and not os.environ.get("FINCH_GGUF_NO_GROUP") else "per-position"),
                        M * K * (2 * gsl + dsl), ms, args)
     d_idx, d_w = torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)
     d_x = torch.randn(n_layers, H, device=dev)

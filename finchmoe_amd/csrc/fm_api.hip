@@ -1391,10 +1391,42 @@ extern "C" int fm_gguf_moe_decode_dev(fm_ctx *c, int layer, const float *d_x, co
     return gguf_decode_groups(c, layer, 1, 1, d_x, d_idx, d_w, K, d_out, d_expert_out, flags);
 }
 
+extern "C" size_t fm_prefill_gguf_ws_bytes(const FmGgufGeom *g, int M, int K);
+extern "C" int fm_launch_prefill_gguf(const uint8_t *d_gate, const uint8_t *d_up, const uint8_t *d_down,
+                                      const FmGgufGeom *g, const float *d_X, const int32_t *d_idx,
+                                      const float *d_w, int M, int K, float *d_out, void *d_ws,
+                                      size_t ws_bytes, int flags, hipStream_t st);
+
+// Chunks of FM_PREFILL_GEMM_MIN_M positions and more with at least four (position, slot) pairs
+// per expert take the grouped products (every routed
+// expert streamed once per group of its positions; prefill_chunk_cmd3_batch_general,
+// finchmoe/infer.m:10958-11059, streams it once per position) when the store is Q4_K gate/up
+// with Q6_K down; smaller chunks, other type combinations and the finite guard run the decode
+// kernels position by position.
 extern "C" int fm_gguf_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, const int32_t *d_idx,
                                        const float *d_w, int M, int K, float *d_out, int flags) {
     if (!c) return FM_ERR_ARG;
     if (M < 1) return fail(c, FM_ERR_ARG, "M %d", M);
+    static const bool no_group = getenv("FINCH_GGUF_NO_GROUP") != nullptr;
+    // (grouping pays from about four positions per expert on: measured at 256 experts, a chunk of
+    // 64 positions is faster position by position, 152 against 179 us, one of 512 is 2.7 times
+    // faster grouped)
+    if (c->gguf_cfg && M >= FM_PREFILL_GEMM_MIN_M && !(flags & FM_GUARD) && !no_group && d_X && d_idx &&
+        d_w && d_out && K >= 1 && K <= FM_MAX_K && (long)M * K >= 4L * c->ggeom.n_experts) {
+        const size_t ws = fm_prefill_gguf_ws_bytes(&c->ggeom, M, K);
+        if (ws) {
+            int rc = check_layers(c, c->g_gate, layer, 1);
+            if (rc) return rc;
+            DeviceGuard dg(c->device);
+            if ((rc = ensure_ws(c, ws))) return rc;
+            rc = fm_launch_prefill_gguf((const uint8_t *)c->g_gate[layer].ptr, (const uint8_t *)c->g_up[layer].ptr,
+                                        (const uint8_t *)c->g_down[layer].ptr, &c->ggeom, d_X, d_idx, d_w, M,
+                                        K, d_out, c->d_ws, c->ws_bytes, flags, c->stream);
+            if (rc == FM_OK) return FM_OK;
+            if (rc != FM_ERR_UNSUPPORTED)
+                return fail(c, rc, "GGUF prefill launch failed: %s", hipGetErrorString(hipGetLastError()));
+        }
+    }
     return gguf_decode_groups(c, layer, 0, M, d_X, d_idx, d_w, K, d_out, nullptr, flags);
 }
 
@@ -1404,7 +1436,7 @@ static int gguf_decode_fn(fm_ctx *c, int layer, const float *x, const int32_t *i
 }
 static int gguf_prefill_fn(fm_ctx *c, int layer, const float *x, const int32_t *idx,
                            const float *w, int M, int K, float *out, float *, int flags) {
-    return gguf_decode_groups(c, layer, 0, M, x, idx, w, K, out, nullptr, flags);
+    return fm_gguf_moe_prefill_dev(c, layer, x, idx, w, M, K, out, flags);
 }
 
 extern "C" int fm_gguf_moe_decode(fm_ctx *c, int layer, const float *x, const int32_t *idx,

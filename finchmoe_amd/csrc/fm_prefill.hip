@@ -79,6 +79,8 @@ struct PfArgs {
     PfItem *items_up, *items_dn;
     int *n_items_up, *n_items_dn;
     int tm_up, tm_dn;
+    // GGUF experts (fm_gq_gate_up / fm_gq_down): the layer's three slabs
+    const uint8_t *gq_gate, *gq_up, *gq_down;
 };
 
 enum { PF_GATE_UP = 0, PF_DOWN = 1, PF_DENSE = 2, PF_DENSE_TEAMS = 3 };
@@ -1583,6 +1585,248 @@ bool pf_dense_supported(int out_dim, int in_dim, int group_size, int bits) {
     return in_dim >= 2048 && in_dim % 2048 == 0 && in_dim <= 16384 && out_dim >= 64 && out_dim % 64 == 0;
 }
 
+// ======================================================================
+// GGUF experts (Q4_K gate/up, Q6_K down), chunks of many positions: grouped products.
+// Replaces the per-position pool kernels of prefill_chunk_cmd3_batch_general
+// (finchmoe/infer.m:10958-11059; finchmoe/shaders.metal:3460-3517, 3641-3712), which stream
+// every routed expert once per position, by one pass per (expert, group of its positions).
+//
+// One workgroup (8 waves) takes one item of fm_pf_group's lists — an expert and up to 8
+// (gate/up) or 16 (down) of its positions — stages the positions' activations in LDS in MFMA
+// operand form and walks the expert's rows, a wave per tile of 16 rows, codes straight from
+// memory into registers (a lane's bytes of a block are used by no other lane).
+//
+// Arithmetic.  A block format is affine per sub-block: Q4_K y = (d sc_j) q - dmin m_j over 32
+// values, Q6_K y = (d sc_g)(q - 32) over 16 (finchmoe/infer.m:1604-1657).  The codes go into
+// bf16 mantissas as 1 + q/128 (fm_mfma.h) — one V_AND_OR per two codes — so a product over a
+// sub-block is D' = sum x + sum q x / 128, exact products, fp32 sum; with xs = sum x from the
+// staging pass, sum y x = (128 d sc) D' - (128 d sc + dmin m) xs for Q4_K and
+// (128 d sc) D' - (160 d sc) xs for Q6_K, in fp32 on the accumulator registers.  fp32
+// activations are two bf16 pieces (16 significant bits): gate/up puts them in M rows p and
+// p + 8 of a 16x16x32 product, down runs two 16x16x16 products on one accumulator.
+// ======================================================================
+typedef short gq_s4 __attribute__((ext_vector_type(4)));
+constexpr int GQ_TM_UP = 8, GQ_TM_DN = 16;
+
+__device__ __forceinline__ uint32_t gq_hi(float v) { return __float_as_uint(v) >> 16; }
+__device__ __forceinline__ uint32_t gq_lo(float v) {
+    return __float_as_uint(v - __uint_as_float(__float_as_uint(v) & 0xFFFF0000u)) >> 16;
+}
+// what the two pieces of v add up to (what the products really multiply)
+__device__ __forceinline__ float gq_both(float v) {
+    const float h = __uint_as_float(__float_as_uint(v) & 0xFFFF0000u);
+    return h + __uint_as_float(__float_as_uint(v - h) & 0xFFFF0000u);
+}
+
+// (scale, min) pair j of a Q4_K block's 12 scale bytes s0 s1 s2 (finchmoe/infer.m:1595-1603)
+__device__ __forceinline__ void gq_scale_min(uint32_t s0, uint32_t s1, uint32_t s2, int j, float &sc, float &mn) {
+    uint32_t a, b;
+    if (j < 4) {
+        a = (s0 >> (8 * j)) & 63u;
+        b = (s1 >> (8 * j)) & 63u;
+    } else {
+        const int i = j - 4;
+        const uint32_t hi = (s2 >> (8 * i)) & 0xFFu;
+        a = (hi & 0xFu) | (((s0 >> (8 * i + 6)) & 3u) << 4);
+        b = (hi >> 4) | (((s1 >> (8 * i + 6)) & 3u) << 4);
+    }
+    sc = (float)a;
+    mn = (float)b;
+}
+
+// gate/up: Q4_K rows [inter][hidden/256 blocks of 144 B]; item = (expert, <= 8 positions)
+__global__ __launch_bounds__(512) void fm_gq_gate_up(PfArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    extern __shared__ __attribute__((aligned(16))) uint8_t gq_smem[];
+    const int it = blockIdx.x;
+    if (it >= *a.n_items_up) return;
+    const PfItem item = a.items_up[it];
+    const int H = a.g.hidden, I = a.g.inter, NKS = H / 32, NB = H / 256;
+    uint4 *img = reinterpret_cast<uint4 *>(gq_smem);                       // [NKS][64 lanes]
+    float *xs = reinterpret_cast<float *>(gq_smem + (size_t)NKS * 1024);   // [NKS][16 M rows]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 15, kb = lane >> 4;
+
+    // ---- stage: thread (position p, k steps ks, ks + 64, ...): hi pieces to M row p, lo to p + 8
+    {
+        const int p = threadIdx.x & 7;
+        const bool on = p < item.count;
+        const size_t m = on ? (size_t)(a.sorted[item.start + p] / a.K) : 0;
+        for (int ks = threadIdx.x >> 3; ks < NKS; ks += 64) {
+            float x[32];
+            const float4 *src = reinterpret_cast<const float4 *>(a.X + m * H + 32 * ks);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float4 v = on ? src[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                x[4 * i] = v.x, x[4 * i + 1] = v.y, x[4 * i + 2] = v.z, x[4 * i + 3] = v.w;
+            }
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 32; i++) sum += gq_both(x[i]);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                // k slots of lane group q: bytes 0 2 | 1 3 | 4 6 | 5 7 of its eight values
+                const float *v = x + 8 * q;
+                const uint4 hi = make_uint4(gq_hi(v[0]) | (gq_hi(v[2]) << 16), gq_hi(v[1]) | (gq_hi(v[3]) << 16),
+                                            gq_hi(v[4]) | (gq_hi(v[6]) << 16), gq_hi(v[5]) | (gq_hi(v[7]) << 16));
+                const uint4 lo = make_uint4(gq_lo(v[0]) | (gq_lo(v[2]) << 16), gq_lo(v[1]) | (gq_lo(v[3]) << 16),
+                                            gq_lo(v[4]) | (gq_lo(v[6]) << 16), gq_lo(v[5]) | (gq_lo(v[7]) << 16));
+                img[(size_t)ks * 64 + 16 * q + p] = hi;
+                img[(size_t)ks * 64 + 16 * q + p + 8] = lo;
+            }
+            xs[ks * 16 + p] = sum;
+            xs[ks * 16 + p + 8] = 0.0f;
+        }
+    }
+    __syncthreads();
+
+    const size_t row_bytes = (size_t)NB * 144;
+    const uint8_t *gbase = a.gq_gate + (size_t)item.expert * I * row_bytes;
+    const uint8_t *ubase = a.gq_up + (size_t)item.expert * I * row_bytes;
+    const uint32_t ones = fm_opaque(0x3F803F80u);
+    for (int tile = wave; tile < I / 16; tile += 8) {
+        const int row = tile * 16 + n;
+        const uint8_t *rp[2] = {gbase + (size_t)row * row_bytes, ubase + (size_t)row * row_bytes};
+        pfr_f4 acc[2] = {pfr_f4{0.0f, 0.0f, 0.0f, 0.0f}, pfr_f4{0.0f, 0.0f, 0.0f, 0.0f}};
+        for (int b = 0; b < NB; b++) {
+            uint4 hdr[2];
+            uint2 qs[2][4];
+#pragma unroll
+            for (int T = 0; T < 2; T++) {
+                const uint8_t *blk = rp[T] + (size_t)b * 144;
+                hdr[T] = *reinterpret_cast<const uint4 *>(blk);
+#pragma unroll
+                for (int c = 0; c < 4; c++) qs[T][c] = *reinterpret_cast<const uint2 *>(blk + 16 + 32 * c + 8 * kb);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int ks = b * 8 + j;
+                const uint4 av = img[(size_t)ks * 64 + lane];
+                const float4 xv = *reinterpret_cast<const float4 *>(xs + ks * 16 + 4 * kb);
+#pragma unroll
+                for (int T = 0; T < 2; T++) {
+                    const float d = fm_fp16_bits(hdr[T].x & 0xFFFFu), dmin = fm_fp16_bits(hdr[T].x >> 16);
+                    float sc, mn;
+                    gq_scale_min(hdr[T].y, hdr[T].z, hdr[T].w, j, sc, mn);
+                    const float c1 = 128.0f * (d * sc), c2 = c1 + dmin * mn;
+                    const uint2 w = qs[T][j >> 1];
+                    const int sh = (j & 1) * 4;
+                    const pfr_u4 bq = {((w.x >> sh) & 0x000F000Fu) | ones, ((w.x >> (sh + 8)) & 0x000F000Fu) | ones,
+                                       ((w.y >> sh) & 0x000F000Fu) | ones, ((w.y >> (sh + 8)) & 0x000F000Fu) | ones};
+                    const pfr_f4 D = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf8, av), __builtin_bit_cast(bf8, bq), pfr_f4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+                    acc[T][0] = fmaf(c1, D[0], fmaf(-c2, xv.x, acc[T][0]));
+                    acc[T][1] = fmaf(c1, D[1], fmaf(-c2, xv.y, acc[T][1]));
+                    acc[T][2] = fmaf(c1, D[2], fmaf(-c2, xv.z, acc[T][2]));
+                    acc[T][3] = fmaf(c1, D[3], fmaf(-c2, xv.w, acc[T][3]));
+                }
+            }
+        }
+        // M rows p and p + 8 (lanes kb and kb + 2) are the two pieces of position p
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float g = acc[0][i] + __shfl_xor(acc[0][i], 32);
+            const float u = acc[1][i] + __shfl_xor(acc[1][i], 32);
+            const int pos = 4 * kb + i;
+            if (kb < 2 && pos < item.count) a.act[(size_t)(item.start + pos) * I + row] = fm_silu_mul(g, u);
+        }
+    }
+#else
+    (void)a;
+#endif
+}
+
+// down: Q6_K rows [hidden][inter/256 blocks of 210 B]; item = (expert, <= 16 positions);
+// input a.act by sorted position, output a.eo by pair id
+__global__ __launch_bounds__(512) void fm_gq_down(PfArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    extern __shared__ __attribute__((aligned(16))) uint8_t gq_smem[];
+    __shared__ int pairs[GQ_TM_DN];
+    const int it = blockIdx.x;
+    if (it >= *a.n_items_dn) return;
+    const PfItem item = a.items_dn[it];
+    const int H = a.g.hidden, I = a.g.inter, NKS = I / 16, NB = I / 256;
+    uint2 *img_hi = reinterpret_cast<uint2 *>(gq_smem);                    // [NKS][64 lanes]
+    uint2 *img_lo = img_hi + (size_t)NKS * 64;
+    float *xs = reinterpret_cast<float *>(img_lo + (size_t)NKS * 64);      // [NKS][16 positions]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 15, kb = lane >> 4;
+    {
+        const int p = threadIdx.x & 15;
+        const bool on = p < item.count;
+        if (threadIdx.x < GQ_TM_DN) pairs[p] = on ? a.sorted[item.start + p] : 0;
+        const float *arow = a.act + (size_t)(item.start + (on ? p : 0)) * I;
+        for (int ks = threadIdx.x >> 4; ks < NKS; ks += 32) {
+            float x[16];
+            const float4 *src = reinterpret_cast<const float4 *>(arow + 16 * ks);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float4 v = on ? src[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                x[4 * i] = v.x, x[4 * i + 1] = v.y, x[4 * i + 2] = v.z, x[4 * i + 3] = v.w;
+            }
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) sum += gq_both(x[i]);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float *v = x + 4 * q;        // k slots: values 0 2 | 1 3 of the lane group's four
+                img_hi[(size_t)ks * 64 + 16 * q + p] = make_uint2(gq_hi(v[0]) | (gq_hi(v[2]) << 16), gq_hi(v[1]) | (gq_hi(v[3]) << 16));
+                img_lo[(size_t)ks * 64 + 16 * q + p] = make_uint2(gq_lo(v[0]) | (gq_lo(v[2]) << 16), gq_lo(v[1]) | (gq_lo(v[3]) << 16));
+            }
+            xs[ks * 16 + p] = sum;
+        }
+    }
+    __syncthreads();
+
+    const size_t row_bytes = (size_t)NB * 210;
+    const uint8_t *dbase = a.gq_down + (size_t)item.expert * H * row_bytes;
+    const uint32_t ones = fm_opaque(0x3F803F80u);
+    struct __attribute__((packed, aligned(2))) U32a2 { uint32_t v; };
+    struct __attribute__((packed, aligned(2))) U16a2 { uint16_t v; };
+    for (int tile = wave; tile < H / 16; tile += 8) {
+        const int row = tile * 16 + n;
+        const uint8_t *rp = dbase + (size_t)row * row_bytes;
+        pfr_f4 acc = pfr_f4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int b = 0; b < NB; b++) {
+            const uint8_t *blk = rp + (size_t)b * 210;
+            const float d = fm_fp16_bits(reinterpret_cast<const U16a2 *>(blk + 208)->v);
+            uint32_t scw[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) scw[i] = reinterpret_cast<const U32a2 *>(blk + 192 + 4 * i)->v;
+#pragma unroll
+            for (int g = 0; g < 16; g++) {
+                // group g: half h, quarter qt of the half (which nibble / which two qh bits),
+                // l = 16 (g & 1) + 4 kb .. + 3 (finchmoe/infer.m:1636-1657)
+                const int h = g >> 3, qt = (g >> 1) & 3, l = 16 * (g & 1) + 4 * kb;
+                const uint32_t wql = reinterpret_cast<const U32a2 *>(blk + 64 * h + 32 * (qt & 1) + l)->v;
+                const uint32_t wqh = reinterpret_cast<const U32a2 *>(blk + 128 + 32 * h + l)->v;
+                const uint32_t code = ((wql >> (4 * (qt >> 1))) & 0x0F0F0F0Fu) | (((wqh >> (2 * qt)) & 0x03030303u) << 4);
+                const uint2 bq = make_uint2((code & 0x00FF00FFu) | ones, ((code >> 8) & 0x00FF00FFu) | ones);
+                const int ks = b * 16 + g;
+                const uint2 ah = img_hi[(size_t)ks * 64 + lane], al = img_lo[(size_t)ks * 64 + lane];
+                const float4 xv = *reinterpret_cast<const float4 *>(xs + ks * 16 + 4 * kb);
+                pfr_f4 D = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(gq_s4, ah), __builtin_bit_cast(gq_s4, bq),
+                                                                    pfr_f4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+                D = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(gq_s4, al), __builtin_bit_cast(gq_s4, bq), D, 0, 0, 0);
+                const float sc = (float)(int)(int8_t)((scw[g >> 2] >> (8 * (g & 3))) & 0xFFu);
+                const float c1 = 128.0f * (d * sc), c2 = 160.0f * (d * sc);
+                acc[0] = fmaf(c1, D[0], fmaf(-c2, xv.x, acc[0]));
+                acc[1] = fmaf(c1, D[1], fmaf(-c2, xv.y, acc[1]));
+                acc[2] = fmaf(c1, D[2], fmaf(-c2, xv.z, acc[2]));
+                acc[3] = fmaf(c1, D[3], fmaf(-c2, xv.w, acc[3]));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int pos = 4 * kb + i;
+            if (pos < item.count) a.eo[(size_t)pairs[pos] * H + row] = acc[i];
+        }
+    }
+#else
+    (void)a;
+#endif
+}
+
 }  // namespace
 
 // Dense tensor against M positions on the same matrix-core kernel as the expert products
@@ -1670,6 +1914,63 @@ extern "C" int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGe
                             : pf_launch<4, true>(a, g, M, d_out, flags, n_cu, st);
     return g->bits == 3 ? pf_launch<3, false>(a, g, M, d_out, flags, n_cu, st)
                         : pf_launch<4, false>(a, g, M, d_out, flags, n_cu, st);
+}
+
+// ---- GGUF experts: grouped products of a chunk ----------------------------------------------
+static bool gq_supported(const FmGgufGeom *g) {
+    return g->gate_type == FM_GGML_Q4_K && g->up_type == FM_GGML_Q4_K && g->down_type == FM_GGML_Q6_K &&
+           g->n_experts <= PF_MAX_EXPERTS && g->hidden % 256 == 0 && g->inter % 256 == 0 &&
+           g->hidden <= 4096 && g->inter <= 4096;
+}
+
+extern "C" size_t fm_prefill_gguf_ws_bytes(const FmGgufGeom *g, int M, int K) {
+    if (!gq_supported(g) || M < 1 || K < 1) return 0;
+    const size_t n = (size_t)M * K;
+    return align256(n * 4) + align256((g->n_experts + n / GQ_TM_UP + 1) * sizeof(PfItem)) +
+           align256((g->n_experts + n / GQ_TM_DN + 1) * sizeof(PfItem)) + 256 +
+           align256(n * g->inter * 4) + align256(n * g->hidden * 4);
+}
+
+// d_gate / d_up / d_down: the layer's slabs.  FM_ERR_UNSUPPORTED: the caller runs the chunk
+// position by position.
+extern "C" int fm_launch_prefill_gguf(const uint8_t *d_gate, const uint8_t *d_up, const uint8_t *d_down,
+                                      const FmGgufGeom *g, const float *d_X, const int32_t *d_idx,
+                                      const float *d_w, int M, int K, float *d_out, void *d_ws,
+                                      size_t ws_bytes, int flags, hipStream_t st) {
+    if (!gq_supported(g)) return FM_ERR_UNSUPPORTED;
+    if (ws_bytes < fm_prefill_gguf_ws_bytes(g, M, K)) return FM_ERR_ARG;
+    const size_t n = (size_t)M * K;
+    char *ws = (char *)d_ws;
+    PfArgs a{};
+    a.g.hidden = g->hidden;
+    a.g.inter = g->inter;
+    a.g.n_experts = g->n_experts;
+    a.X = d_X;
+    a.idx = d_idx;
+    a.w = d_w;
+    a.M = M;
+    a.K = K;
+    a.tm_up = GQ_TM_UP;
+    a.tm_dn = GQ_TM_DN;
+    a.gq_gate = d_gate;
+    a.gq_up = d_up;
+    a.gq_down = d_down;
+    a.sorted = (int *)ws;                 ws += align256(n * 4);
+    a.items_up = (PfItem *)ws;            ws += align256((g->n_experts + n / GQ_TM_UP + 1) * sizeof(PfItem));
+    a.items_dn = (PfItem *)ws;            ws += align256((g->n_experts + n / GQ_TM_DN + 1) * sizeof(PfItem));
+    a.n_items_up = (int *)ws;
+    a.n_items_dn = (int *)ws + 1;         ws += 256;
+    a.act = (float *)ws;                  ws += align256(n * g->inter * 4);
+    a.eo = (float *)ws;
+    hipLaunchKernelGGL(fm_pf_group, dim3(1), dim3(1024), 0, st, a);
+    const size_t lds_up = (size_t)(g->hidden / 32) * (1024 + 64), lds_dn = (size_t)(g->inter / 16) * (1024 + 64);
+    static FmLdsAttr attr_up, attr_dn;
+    if (!fm_dyn_lds_ready(attr_up, (const void *)fm_gq_gate_up, 160 * 1024 - 1024)) return FM_ERR_HIP;
+    if (!fm_dyn_lds_ready(attr_dn, (const void *)fm_gq_down, 160 * 1024 - 1024)) return FM_ERR_HIP;
+    hipLaunchKernelGGL(fm_gq_gate_up, dim3((unsigned)(g->n_experts + n / GQ_TM_UP)), dim3(512), lds_up, st, a);
+    hipLaunchKernelGGL(fm_gq_down, dim3((unsigned)(g->n_experts + n / GQ_TM_DN)), dim3(512), lds_dn, st, a);
+    hipLaunchKernelGGL(fm_pf_combine, dim3(M, (g->hidden + 1023) / 1024), dim3(256), 0, st, a, d_out, flags);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 
 extern "C" int fm_launch_widen_bf16(const uint16_t *d_src, float *d_dst, size_t n, hipStream_t st) {

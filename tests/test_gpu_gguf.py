@@ -165,3 +165,41 @@ def test_gguf_streaming_shapes(orc, h, i, down_t, layers, K):
         assert not eo[0, K - 1].any()
     finally:
         ctx.close()
+
+
+@pytest.mark.parametrize("M,K,h,i,seed", [(40, 8, 2048, 512, 1), (97, 4, 1024, 256, 2), (32, 8, 512, 512, 3)])
+def test_gguf_chunk_grouped_products(orc, M, K, h, i, seed):
+    """Chunks of 32 positions and more on a Q4_K / Q4_K / Q6_K store take the grouped products
+    (an expert streamed once per group of its positions, prefill_chunk_cmd3_batch_general's
+    result, finchmoe/infer.m:10958-11059): every position equals its per-position call and the
+    oracle within the bar; skewed routing gives items of every size, an expert index outside the
+    store contributes nothing, the accumulate flag adds, and a repeat is bit-identical."""
+    from finchmoe_amd import FinchHip
+    rng = np.random.default_rng(seed)
+    Ee = 12
+    gate, up, down = F.synth_gguf_layer(rng, Ee, h, i)
+    ctx = FinchHip(0)
+    try:
+        ctx.gguf_config(1, Ee, h, i, (fb.Q4_K, fb.Q4_K, fb.Q6_K))
+        ctx.gguf_upload_layer(0, gate, up, down)
+        X = rng.standard_normal((M, h)).astype(np.float32)
+        # skewed: expert 0 in every position's set, the others random without repeats
+        idx = np.stack([np.concatenate([[0], 1 + rng.permutation(Ee - 1)[:K - 1]]) for _ in range(M)]).astype(np.int32)
+        w = rng.random((M, K)).astype(np.float32)
+        idx[5, K - 1] = Ee + 3                                 # outside the store
+        out = ctx.gguf_moe_prefill(0, X, idx, w)
+        assert np.isfinite(out).all()
+        assert np.array_equal(ctx.gguf_moe_prefill(0, X, idx, w), out)
+        for m in range(M):
+            keep = idx[m] < Ee
+            single, _ = ctx.gguf_moe_decode(0, X[m], idx[m][keep], w[m][keep])
+            assert rel_err(out[m], single) < 1e-3, (m, rel_err(out[m], single))
+        for m in (0, 5, M - 1):
+            keep = idx[m] < Ee
+            ref, _ = orc.moe_gguf_forward(gate, up, down, X[m], idx[m][keep], w[m][keep], h, i)
+            assert_parity(out[m], ref, "position %d" % m)
+        base = rng.standard_normal((M, h)).astype(np.float32)
+        acc = ctx.gguf_moe_prefill(0, X, idx, w, flags=fb.ACCUMULATE, out=base.copy())
+        assert rel_err(acc, base + out) < 1e-6
+    finally:
+        ctx.close()
