@@ -1,40 +1,37 @@
-// fm_prefill.hip — grouped chunked-prefill expert product on bf16 MFMA.
+// fm_prefill.hip — chunks of many positions on the matrix cores: the routed experts' products
+// grouped by expert (affine 3-/4-bit stores and GGUF Q4_K / Q6_K stores), and dense affine
+// tensors against M positions.
 //
 // The reference has no GEMM here: prefill_chunk_cmd3_encode (finchmoe/infer.m:
 // 10704-10765) runs the per-position GEMV chain for each of the M positions, so two
 // positions routed to the same expert read its weights twice.  This file groups
 // the M*K (position, slot) pairs by expert and multiplies each expert's weights
-// once against all of its positions.  Numerical contract: the per-position
-// result (fm_decode.hip) within the parity bar.
+// once against a group of its positions.  Numerical contract: the per-position
+// result (fm_decode.hip, fm_gguf.hip) within the parity bar.
 //
 // Why not "dequantize to bf16 and multiply": rounding (q*s + b) to bf16 misses
 // the bar (max relative error 1.8e-3 on the benchmark's weight distribution).
 // Instead
 //   * the CODES are the MFMA operand, as exact bf16 numbers 1 + q*2^t/128 (the
-//     mantissa trick of fm_mfma.h: one V_AND_OR_B32 per two codes; 4-bit codes: t = 0);
-//   * each quantization group (64 columns) is accumulated by its own MFMA chain
-//     and its scale is applied to the result in fp32: acc += s[row][g] * D_g;
-//   * activations are split hi + lo (two bf16 pieces, 16 significant bits); the
-//     pieces are extra M rows: M row j = hi piece of position j, row j+16 = lo piece,
-//     which land in registers i and i+8 of the same lane;
-//   * the bias term sum_g b[row][g] * xsum[pos][g] and the offset the "1 +" adds,
-//     sum_g s[row][g] * xoff[pos][g], are two small products over the group index,
-//     also on MFMA: the bf16 bits of b and s are operands as they are (FP16 ones are
-//     split into a bf16 head and tail first, pf_side_b).
+//     mantissa trick of fm_mfma.h: one V_AND_OR_B32 per two codes);
+//   * each quantization group is accumulated by its own MFMA chain and its scale is
+//     applied to the result in fp32: acc += s[row][g] * D_g;
+//   * fp32 activations are split hi + lo (two bf16 pieces, 16 significant bits), bf16
+//     activations are operands as they are;
+//   * the bias term sum_g b[row][g] * xsum[pos][g] and the offset the "1 +" adds are
+//     small products over the group index (affine stores: on MFMA as well, the bf16 bits
+//     of b and s being operands as they are; GGUF stores: in fp32 on the accumulators).
 //
-// V_MFMA_F32_32X32X16_BF16 with positions on M and weight rows on N: lane
-// (n = lane%32, h = lane/32) supplies 8 consecutive k of weight row n and holds
-// 16 results, all of weight row n — so a lane needs ONE scale per group.
-// A lane's codes for one group are half a group: 32 codes = 12 bytes (3-bit) or 16 bytes
-// (4-bit).  The kernels are instantiated for both widths.
-//
-// Work item = (expert, up to 16 of its positions).  Four kinds of kernel per chunk:
-//   fm_pf_sort         workgroup 0 groups the pairs by expert and cuts them into items; the
-//                      others turn X into MFMA operand registers (pf_prepare)
-//   fm_pf_gemm<false>  gate/up + SwiGLU for every item -> act (by sorted position)
-//   fm_pf_prepare_act  act -> operand registers
-//   fm_pf_gemm<true>   down for every item -> expert_out (by pair)
-//   fm_pf_combine      weighted sum in slot order
+// Kernels of a chunk of routed experts:
+//   fm_pf_group        one workgroup groups the pairs by expert and cuts every expert's
+//                      positions into items (two lists: gate/up and down items may differ
+//                      in size)
+//   fm_pf_rows<GATE_UP>, fm_pf_rows<DOWN>     affine stores: row-tile kernels, see below
+//   fm_gq_gate_up, fm_gq_down                 GGUF stores
+//   fm_pf_combine      weighted sum of a position's K expert outputs in slot order
+// Dense tensors: fm_pf_dense_prep (X -> operand registers, once per chunk) and fm_pf_gemm
+// (V_MFMA_F32_32X32X16_BF16, K split over the waves of a workgroup, partial tiles summed
+// through LDS).
 #include "fm_mfma.h"
 #include "fm_ring.h"
 
@@ -65,8 +62,6 @@ struct PfArgs {
     float *eo;         // [M*K][hidden], by pair id
     uint4 *xop;        // [M][hidden/64][k step 4][half 2][piece 2]: X as MFMA operand registers
     float2 *xsums;     // [M][hidden/64]: (xsum, xoff) of every group of every position
-    uint4 *aop;        // [M*K][inter/64][4][2][2]: act (by sorted position) in the same form
-    float2 *asums;     // [M*K][inter/64]
     // dense tensor (PF_DENSE): out[M][d_rows] = X[M][d_cols] * W^T, scales / biases d_sb bytes
     // behind / before W; one launch covers the 2048 columns of pass d_pass
     const uint8_t *d_w;
@@ -83,7 +78,7 @@ struct PfArgs {
     const uint8_t *gq_gate, *gq_up, *gq_down;
 };
 
-enum { PF_GATE_UP = 0, PF_DOWN = 1, PF_DENSE = 2, PF_DENSE_TEAMS = 3 };
+enum { PF_DENSE = 2, PF_DENSE_TEAMS = 3 };
 
 // ---- pairing of the 32 codes a lane holds for one group -------------------
 // Pair p fills k slots 2p (low half of the register, code lo(p) at mantissa bit tl(p)) and
@@ -149,9 +144,7 @@ __device__ __forceinline__ void pf_stage_pair(const float *x, uint32_t *hi, uint
 }
 
 // ---------------------------------------------------------------- kernels
-// pairs -> grouped by expert, cut into items of <= PF_TM positions.  One workgroup of
-// 1024 threads, one expert per thread for the two prefix sums.
-// X in the form the gate/up kernel multiplies with: per position, group, k step and column
+// X in the form the dense kernel multiplies with: per position, group, k step and column
 // half the four operand registers of the hi pieces and of the lo pieces (pf_stage_pair), and
 // per position and group the two sums the bias and offset terms need.  Done once per chunk:
 // a position is multiplied by K experts, and splitting it inside the multiply kernel cost a
@@ -203,70 +196,6 @@ __device__ __forceinline__ void pf_prepare(const float *src, int rows, int cols,
             dst[4 * k + 2 * h + 1] = regs[4 * k + 1];
         }
         if (h == 0) dst_sums[(size_t)m * NG + g] = make_float2(xs, xo);
-    }
-}
-
-// the SwiGLU outputs (by sorted position) as operand registers for the down product
-template <int BITS>
-__global__ __launch_bounds__(256) void fm_pf_prepare_act(PfArgs a) {
-    pf_prepare<BITS>(a.act, a.M * a.K, a.g.inter, a.aop, a.asums, (int)(blockIdx.x * blockDim.x + threadIdx.x));
-}
-
-// workgroup 0 sorts, the others prepare X
-template <int BITS>
-__global__ __launch_bounds__(1024) void fm_pf_sort(PfArgs a) {
-    __shared__ int hist[PF_MAX_EXPERTS], cursor[PF_MAX_EXPERTS], scan_a[PF_MAX_EXPERTS],
-        scan_b[PF_MAX_EXPERTS];
-    if (blockIdx.x > 0) {
-        pf_prepare<BITS>(a.X, a.M, a.g.hidden, a.xop, a.xsums, (int)((blockIdx.x - 1) * blockDim.x + threadIdx.x));
-        return;
-    }
-    const int E = a.g.n_experts, n = a.M * a.K, e = threadIdx.x;
-    hist[e] = 0;
-    __syncthreads();
-    for (int p = threadIdx.x; p < n; p += blockDim.x) {
-        int x = a.idx[p];
-        if ((unsigned)x < (unsigned)E) atomicAdd(&hist[x], 1);
-    }
-    __syncthreads();
-    const int cnt = e < E ? hist[e] : 0, nit = (cnt + PF_TM - 1) / PF_TM;
-    // inclusive scans of the pair counts and the item counts: inside each wave by lane
-    // shifts, the 16 wave totals by wave 0, two barriers in all
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    int sa = cnt, sb = nit;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int va = __shfl_up(sa, d), vb = __shfl_up(sb, d);
-        if (lane >= d) sa += va, sb += vb;
-    }
-    if (lane == 63) scan_a[wv] = sa, scan_b[wv] = sb;
-    __syncthreads();
-    if (wv == 0) {
-        int ta = lane < 16 ? scan_a[lane] : 0, tb = lane < 16 ? scan_b[lane] : 0;
-#pragma unroll
-        for (int d = 1; d < 16; d <<= 1) {
-            const int va = __shfl_up(ta, d), vb = __shfl_up(tb, d);
-            if (lane >= d) ta += va, tb += vb;
-        }
-        if (lane < 16) scan_a[lane] = ta, scan_b[lane] = tb;     // inclusive totals of waves 0..lane
-    }
-    __syncthreads();
-    if (wv > 0) sa += scan_a[wv - 1], sb += scan_b[wv - 1];
-    const int off = sa - cnt, ioff = sb - nit;
-    cursor[e] = off;
-    for (int s = 0; s < nit; s++) {
-        PfItem it;
-        it.expert = e;
-        it.start = off + s * PF_TM;
-        it.count = cnt - s * PF_TM < PF_TM ? cnt - s * PF_TM : PF_TM;
-        it.pad = 0;
-        a.items[ioff + s] = it;
-    }
-    if (e == 1023) *a.n_items = sb;
-    __syncthreads();
-    for (int p = threadIdx.x; p < n; p += blockDim.x) {
-        int x = a.idx[p];
-        if ((unsigned)x < (unsigned)E) a.sorted[atomicAdd(&cursor[x], 1)] = p;
     }
 }
 
@@ -350,28 +279,22 @@ __device__ __forceinline__ uint4 pf_side_b(uint32_t w0, uint32_t w1, int hh, uin
     }
 }
 
-// MODE PF_GATE_UP (DOWN = false): K = hidden is eight slabs, wave w owns slab w, all waves work on the
-//   same 32 rows; a step = the gate tile and the up tile of those rows; sum over eight waves,
-//   SwiGLU, act.
-// MODE PF_DOWN: K = inter is two slabs: the workgroup is four teams of two waves (slab = wave & 1),
-//   every team on its own 64 rows of a step's 256; a step = two row tiles per team; sum over
-//   the team's two waves, expert_out.  The activation operand comes from aop / asums
-//   (fm_pf_prepare_act), indexed by sorted position.
-// MODE PF_DENSE: one dense tensor against M positions, 2048 of its columns per launch (eight slabs
-//   as in gate/up; column pass d_pass adds to what the passes before it stored); an item is a
-//   block of 16 positions, a step = two row tiles (64 rows), the operand comes from xop.
-// MODE PF_DENSE_TEAMS: a dense tensor of 512 columns: the slabs and teams of PF_DOWN (a step =
-//   256 rows), operand and output as in PF_DENSE.
+// MODE PF_DENSE: one dense tensor against M positions, 2048 of its columns per launch (eight
+//   slabs, wave w owns slab w, all waves work on the same rows; column pass d_pass adds to what
+//   the passes before it stored); an item is a block of 16 positions, a step = two row tiles
+//   (64 rows), the partial tiles of the eight waves are summed through LDS; the operand comes
+//   from xop (fm_pf_dense_prep).
+// MODE PF_DENSE_TEAMS: a dense tensor of 512 columns: two slabs, the workgroup is four teams of
+//   two waves (slab = wave & 1), every team on its own 64 rows of a step's 256; operand and
+//   output as in PF_DENSE.
 template <int MODE, int BITS, bool FP16>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fm_pf_gemm(PfArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // (the host pass cannot allocate the registers of the asm blocks)
     using P = PfSlab<BITS>;
     constexpr int DW = PfCode<BITS>::DW;
-    // TEAMS: geometry of the down product; DTENSOR: operands of a dense tensor; DENSE / DOWN: the
-    // two pure forms
-    constexpr bool TEAMS = MODE == PF_DOWN || MODE == PF_DENSE_TEAMS;
-    constexpr bool DTENSOR = MODE == PF_DENSE || MODE == PF_DENSE_TEAMS;
-    constexpr bool DOWN = MODE == PF_DOWN, DENSE = MODE == PF_DENSE;
+    // TEAMS: 512 columns as two slabs, four teams of two waves; DENSE: 2048 columns per pass
+    constexpr bool TEAMS = MODE == PF_DENSE_TEAMS, DENSE = MODE == PF_DENSE;
+    static_assert(TEAMS || DENSE, "dense tensors only (the expert products are fm_pf_rows)");
     constexpr int GPW = P::GPW;
     constexpr int RING = P::RING;
     extern __shared__ __attribute__((aligned(16))) uint8_t pf2_smem[];
@@ -382,24 +305,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint32_t ring0 = lds0 + (uint32_t)wave * (RING * P::SLOT);
     const uint32_t red0 = lds0 + 8 * RING * P::SLOT;
     const int n_items = *a.n_items;
-    const int in_dim = DTENSOR ? a.d_cols : DOWN ? a.g.inter : a.g.hidden;
+    const int in_dim = a.d_cols;
     const int row_bytes = in_dim * BITS / 8, sb_bytes = (in_dim / 64) * 2;
     const int slab = DENSE ? wave + 8 * a.d_pass : TEAMS ? (wave & 1) : wave, team = TEAMS ? (wave >> 1) : 0;
-    const int n_steps = DENSE ? a.d_rows / 64 : DTENSOR ? a.d_rows / 256 : DOWN ? a.g.hidden / 256 : a.g.inter / 32;
+    const int n_steps = DENSE ? a.d_rows / 64 : a.d_rows / 256;
     const uint32_t ones = fm_opaque(0x3F803F80u);
     // region offsets of the first tile-matrix of a step (this team's), the distance to the
     // second one, rows per step
     // (byte offsets from the blob's — the dense tensor's W — first byte, modulo 2^64)
     const size_t team_w = 64u * team * row_bytes, team_sb = 64u * team * sb_bytes;
-    const size_t w_off0 = DTENSOR ? team_w : DOWN ? a.g.down_w + team_w : a.g.gate_w;
-    const size_t s_off0 = DTENSOR ? (size_t)a.d_s + team_sb : DOWN ? a.g.down_s + team_sb : a.g.gate_s;
-    const size_t b_off0 = DTENSOR ? (size_t)a.d_b + team_sb : DOWN ? a.g.down_b + team_sb : a.g.gate_b;
-    const uint32_t w_d = TEAMS || DENSE ? 32u * row_bytes : a.g.up_w - a.g.gate_w;
-    const uint32_t s_d = TEAMS || DENSE ? 32u * sb_bytes : a.g.up_s - a.g.gate_s;
-    const uint32_t b_d = TEAMS || DENSE ? 32u * sb_bytes : a.g.up_b - a.g.gate_b;
-    const uint32_t step_rows = DENSE ? 64u : TEAMS ? 256u : 32u;
-    const uint8_t *store = DTENSOR ? a.d_w : a.layer;        // what an item's "expert" indexes into
-    const size_t expert_size = DTENSOR ? 0 : a.g.expert_size;
+    const size_t w_off0 = team_w;
+    const size_t s_off0 = (size_t)a.d_s + team_sb;
+    const size_t b_off0 = (size_t)a.d_b + team_sb;
+    const uint32_t w_d = 32u * row_bytes;
+    const uint32_t s_d = 32u * sb_bytes;
+    const uint32_t b_d = 32u * sb_bytes;
+    const uint32_t step_rows = DENSE ? 64u : 256u;
+    const uint8_t *store = a.d_w;       // (an item's "expert" is 0: one tensor)
+    const size_t expert_size = 0;
     // this lane's pieces of a slot copy
     uint32_t coff[P::NQ];
     bool cvalid[P::NQ];
@@ -478,30 +401,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // costs one memory round trip (the operand registers) instead of a chain of three, each
     // of which would also drain the ring.
     PfItem item_next = PfItem{0, 0, 0, 0};
-    int pair_next = 0;              // pair id of this lane's position (divided by K when used)
-    int out_pairs_next[8];          // DOWN: pair ids of the eight positions this lane stores
-#pragma unroll
-    for (int i = 0; i < 8; i++) out_pairs_next[i] = 0;
-    if (t0 < t1) {
-        item_next = a.items[t0 / n_steps];
-        if constexpr (DOWN) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int tok = 8 * (i / 4) + 4 * hh + (i % 4);
-                if (tok < item_next.count) out_pairs_next[i] = a.sorted[item_next.start + tok];
-            }
-        } else if constexpr (!DTENSOR) {
-            if ((n & 15) < item_next.count) pair_next = a.sorted[item_next.start + (n & 15)];
-        }
-    }
+    if (t0 < t1) item_next = a.items[t0 / n_steps];
     for (int t = t0; t < t1;) {
         const int it = t / n_steps, s_begin = t - it * n_steps;
         const int s_end = t1 - t < n_steps - s_begin ? s_begin + (t1 - t) : n_steps;
         t += s_end - s_begin;
         const PfItem item = item_next;
-        int out_pairs[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) out_pairs[i] = out_pairs_next[i];
         const bool more = t < t1;                  // this workgroup goes on to item it + 1
         if (more) item_next = a.items[it + 1];
         // ---- this wave's share of the activation operand, straight into registers:
@@ -517,10 +422,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 // X was turned into operand registers once per chunk (pf_prepare): lane (m, hh)
                 // takes the hi (m < 16) or lo registers of its position, its groups, its half
                 const int piece = n < 16 ? 0 : 1;
-                const size_t m = !on ? 0 : DOWN || DTENSOR ? (size_t)(item.start + pos) : (size_t)(pair_next / a.K);
+                const size_t m = !on ? 0 : (size_t)(item.start + pos);
                 const int ng = in_dim / 64;
-                const uint4 *src = (DOWN ? a.aop : a.xop) + (m * ng + GPW * slab) * 16 + 2 * hh + piece;
-                const float2 *sm = (DOWN ? a.asums : a.xsums) + m * ng + GPW * slab;
+                const uint4 *src = a.xop + (m * ng + GPW * slab) * 16 + 2 * hh + piece;
+                const float2 *sm = a.xsums + m * ng + GPW * slab;
 #pragma unroll
                 for (int gi = 0; gi < GPW; gi++) {
 #pragma unroll
@@ -541,19 +446,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                         if (!on) t = fm_u4{0u, 0u, 0u, 0u};     // rows past the item's positions
                         A[gi][k] = __builtin_bit_cast(uint4, t);
                     }
-                // the next item has arrived with them: its position row, used at its start
-                // (no arithmetic on it here: that would wait for the load now)
-                if constexpr (DOWN) {
-#pragma unroll
-                    for (int i = 0; i < 8; i++) {
-                        const int tok = 8 * (i / 4) + 4 * hh + (i % 4);
-                        out_pairs_next[i] = 0;
-                        if (more && tok < item_next.count) out_pairs_next[i] = a.sorted[item_next.start + tok];
-                    }
-                } else if constexpr (!DTENSOR) {
-                    pair_next = 0;
-                    if (more && pos < item_next.count) pair_next = a.sorted[item_next.start + pos];
-                }
                 if (more) e_ahead = item_next.expert;     // the loader enters it during this item
             }
             // K slots of the bias/offset MFMAs: slot = 4*piece + group, one MFMA per term (xsum
@@ -726,16 +618,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     t0 += p[w2];
                     t1 += p[8 + w2];
                 }
-                if constexpr (DENSE) {
-                    // the two row tiles of the step; later column passes add to the earlier ones
-                    if (my_on) {
-                        float *o = a.d_out + (size_t)(item.start + my_pos) * a.d_rows + 64 * s + n;
-                        const bool add = a.d_pass > 0 || (a.d_flags & FM_ACCUMULATE);
-                        o[0] = add ? o[0] + t0 : t0;
-                        o[32] = add ? o[32] + t1 : t1;
-                    }
-                } else if (my_on) {
-                    a.act[(size_t)(item.start + my_pos) * a.g.inter + 32 * s + n] = fm_silu_mul(t0, t1);
+                // the two row tiles of the step; later column passes add to the earlier ones
+                if (my_on) {
+                    float *o = a.d_out + (size_t)(item.start + my_pos) * a.d_rows + 64 * s + n;
+                    const bool add = a.d_pass > 0 || (a.d_flags & FM_ACCUMULATE);
+                    o[0] = add ? o[0] + t0 : t0;
+                    o[32] = add ? o[32] + t1 : t1;
                 }
             } else {
                 // wave (team, j) sums tile j of its team over the team's two waves (slab 0, then
@@ -762,12 +650,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     const int tok = 8 * (i / 4) + 4 * hh + (i % 4);
                     if (tok < item.count) {
                         const float v = p[i] + p[8 + i];
-                        if constexpr (DTENSOR) {
-                            float *o = a.d_out + (size_t)(item.start + tok) * a.d_rows + row;
-                            *o = (a.d_flags & FM_ACCUMULATE) ? *o + v : v;
-                        } else {
-                            a.eo[(size_t)out_pairs[i] * a.g.hidden + row] = v;
-                        }
+                        float *o = a.d_out + (size_t)(item.start + tok) * a.d_rows + row;
+                        *o = (a.d_flags & FM_ACCUMULATE) ? *o + v : v;
                     }
                 }
             }
