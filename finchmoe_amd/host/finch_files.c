@@ -316,6 +316,14 @@ static double j_number(jcur *c) {
     return v;
 }
 
+/* a number that must be an integer in [lo, hi] (a double holds every file offset below 2^53
+ * exactly); anything else makes the manifest bad instead of being converted */
+static int64_t j_int(jcur *c, double lo, double hi) {
+    const double v = j_number(c);
+    if (!(v >= lo && v <= hi) || v != (double)(int64_t)v) { c->bad = 1; return 0; }
+    return (int64_t)v;
+}
+
 static void j_skip(jcur *c, int depth) {
     if (c->bad || depth > 64) { c->bad = 1; return; }
     int ch = j_peek(c);
@@ -410,10 +418,10 @@ static void parse_entry(jcur *c, dense_ent *e) {
     do {
         char *k = j_string(c);
         if (!k || !j_eat(c, ':')) { free(k); c->bad = 1; return; }
-        if (!strcmp(k, "offset")) { e->offset = (uint64_t)j_number(c); have |= 1; }
-        else if (!strcmp(k, "size")) { e->size = (uint64_t)j_number(c); have |= 2; }
-        else if (!strcmp(k, "bits") && j_peek(c) != 'n') e->bits = (int)j_number(c);
-        else if (!strcmp(k, "group_size") && j_peek(c) != 'n') e->group_size = (int)j_number(c);
+        if (!strcmp(k, "offset")) { e->offset = (uint64_t)j_int(c, 0.0, 9007199254740992.0); have |= 1; }
+        else if (!strcmp(k, "size")) { e->size = (uint64_t)j_int(c, 0.0, 9007199254740992.0); have |= 2; }
+        else if (!strcmp(k, "bits") && j_peek(c) != 'n') e->bits = (int)j_int(c, -2147483648.0, 2147483647.0);
+        else if (!strcmp(k, "group_size") && j_peek(c) != 'n') e->group_size = (int)j_int(c, -2147483648.0, 2147483647.0);
         else if (!strcmp(k, "dtype")) {
             char *d = j_string(c);
             if (d) { strncpy(e->dtype, d, sizeof e->dtype - 1); have |= 4; }
@@ -422,8 +430,8 @@ static void parse_entry(jcur *c, dense_ent *e) {
             if (!j_eat(c, '[')) c->bad = 1;
             else if (!j_eat(c, ']')) {
                 do {
-                    double v = j_number(c);
-                    if (e->ndim < 4) e->shape[e->ndim] = (int64_t)v;
+                    const int64_t v = j_int(c, -9007199254740992.0, 9007199254740992.0);
+                    if (e->ndim < 4) e->shape[e->ndim] = v;
                     e->ndim++;
                 } while (!c->bad && j_eat(c, ','));
                 if (!j_eat(c, ']')) c->bad = 1;
@@ -510,7 +518,9 @@ void finch_ops_close_dense(finch_dense *d) {
     if (!d) return;
     /* resident copies keyed by addresses inside the mapping must not outlive it */
     for (int i = 0; i < d->n; i++) {
-        if (d->map.p && !strcmp(d->ent[i].dtype, "U32")) finch_ops_forget_tensor(d->map.p + d->ent[i].offset);
+        /* (an entry that ends past the file made the open fail: its offset is not an address) */
+        if (d->map.p && d->ent[i].offset <= d->map.n && !strcmp(d->ent[i].dtype, "U32"))
+            finch_ops_forget_tensor(d->map.p + d->ent[i].offset);
         free(d->ent[i].name);
     }
     unmap_file(&d->map);
