@@ -40,20 +40,25 @@ static size_t hash_ptr(const void *p) {
     return (size_t)v;
 }
 
+/* NULL: no such key (insert == 0), or no memory for the table */
 static slot *tab_find(const void *key, int insert) {
+    if (!key) return NULL;               /* NULL marks an empty slot */
     if (!g_cap) {
+        g_tab = (slot *)calloc(1024, sizeof(slot));
+        if (!g_tab) return NULL;
         g_cap = 1024;
-        g_tab = (slot *)calloc(g_cap, sizeof(slot));
     }
     if (insert && (g_used + 1) * 2 > g_cap) {
+        slot *bigger = (slot *)calloc(2 * g_cap, sizeof(slot));
+        if (!bigger) return NULL;
         slot *old = g_tab;
-        size_t oc = g_cap;
-        g_cap *= 2;
-        g_tab = (slot *)calloc(g_cap, sizeof(slot));
+        const size_t oc = g_cap;
+        g_tab = bigger;
+        g_cap = 2 * oc;
         g_used = 0;
         for (size_t i = 0; i < oc; i++)
             if (old[i].key) {
-                slot *s = tab_find(old[i].key, 1);
+                slot *s = tab_find(old[i].key, 1);     /* cannot fail: the table is half empty */
                 *s = old[i];
             }
         free(old);
@@ -75,7 +80,9 @@ static int resident(const void *W, const void *S, const void *B, int out_dim, in
      * (infer.m:4491).  Normalised here so that the table compares like with like. */
     if (!S || !B) { S = B = NULL; bits = 16; }
     else if (bits == 0) bits = 4;
+    if (!W) return FM_ERR_ARG;
     slot *s = tab_find(W, 1);
+    if (!s) return FM_ERR_NOMEM;
     if (s->t >= 0 && (s->out_dim != out_dim || s->in_dim != in_dim || s->bits != bits)) {
         fm_tensor_release(g_ctx, s->t);   /* host memory was reused for another tensor */
         s->t = -1;
@@ -203,8 +210,12 @@ void fast_prefill_matvec(const uint32_t *W, const uint16_t *scales, const uint16
     fm_tensor t;
     int rc = resident(W, scales, biases, out_dim, in_dim, group_size, bits, &t);
     if (!rc) rc = fm_matvec_prefill(g_ctx, t, x, out, M);
-    if (rc) fail(rc, "fast_prefill_matvec");
-    else g_status = FM_OK;
+    if (rc) {
+        if (out && out_dim > 0 && M > 0) memset(out, 0, (size_t)M * (size_t)out_dim * sizeof(float));
+        fail(rc, "fast_prefill_matvec");
+    } else {
+        g_status = FM_OK;
+    }
 }
 
 int finch_ops_config_experts(int n_layers, int n_experts, int hidden, int inter, int bits) {

@@ -148,3 +148,23 @@ def test_manifest_reader_survives_damaged_files(driver, tmp_path):
         (d / ("m%03d.bin" % i)).write_bytes(blob if i % 7 else blob[:int(rng.integers(0, len(blob)))])
     res = _run(driver, "dense", d)
     assert int(res["files"]) == len(muts) + 1 and int(res["accepted"]) >= 1
+
+
+def test_host_layer_bookkeeping_under_sanitizers(tmp_path):
+    """finch_ops.c (the table from host weight pointers to resident tensors, the batch wrapper,
+    the error paths) compiled with tests/host_fuzz/ops_table_main.c around it: doubles of the C
+    ABI count registrations and releases; 60000 keys, reused pointers, failing registrations."""
+    if not shutil.which("gcc"):
+        pytest.skip("no host compiler")
+    out = str(tmp_path / "ops_table_main")
+    cmd = ["gcc", "-O1", "-g", "-std=gnu99", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+           "-static-libasan", "-I", os.path.join(ROOT, "include"),
+           os.path.join(ROOT, "tests", "host_fuzz", "ops_table_main.c"), "-lm", "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode and "static-libasan" in r.stderr:
+        cmd.remove("-static-libasan")
+        r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    r = subprocess.run([out], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.strip().splitlines()[-1].startswith("done "), \
+        (r.stdout[-500:], r.stderr[-2000:])
