@@ -806,6 +806,11 @@ def main():
         print("bench.py: unknown workload %r (have: %s)" % (args.workload, ", ".join(runners)),
               file=sys.stderr)
         sys.exit(2)
+    # the case by name before the GPU is touched: if a kernel faults, the box may take the
+    # output files with it and only the end of stderr comes back
+    print("bench.py: workload=%s chunk=%d bits=%d scale_dtype=%s x_dtype=%s steps=%d warmup=%d graph=%s"
+          % (args.workload, args.chunk, args.bits, args.scale_dtype, args.x_dtype, args.steps, args.warmup,
+             bool(args.graph)), file=sys.stderr, flush=True)
     res = runners[args.workload](args)
     print(json.dumps(res))
 

@@ -13,6 +13,13 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+def pytest_runtest_logstart(nodeid, location):
+    """Name every GPU test on stderr before it runs: a kernel fault can end the machine with
+    the run, and then the end of stderr is all that comes back."""
+    if "test_gpu_" in nodeid or "test_zz_" in nodeid or "on_gpu" in nodeid:
+        print("\n[gpu test] %s" % nodeid, file=sys.stderr, flush=True)
+
+
 @pytest.fixture(scope="session")
 def orc():
     """The CPU oracle (test infrastructure)."""
