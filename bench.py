@@ -101,11 +101,71 @@ def cpu_baseline_decode(blob_t, lo, idx, w, x, budget_s=12.0, bits=3, scale_dtyp
                 break
         return done, t_cpu
 
+    def ref_leg(budget, first):
+        """The same blocks through the reference's own compiled CPU functions
+        (oracle/_ref/libfm_ref.so: cpu_dequant_matvec x3, cpu_swiglu, cpu_vec_madd, called in the
+        order of the CPU expert loop, finchmoe/infer.m:10166-10195).  BF16 scales only (what the
+        reference's files hold).  None when the library did not travel with the tree."""
+        R = oracle.ref_lib()
+        if R is None or scale_dtype != 0:
+            return None
+        ofs = lo
+        g_out, u_out, act = (np.empty(I, np.float32) for _ in range(3))
+        e_out, moe = np.empty(H, np.float32), np.zeros(H, np.float32)
+        done, t_cpu = 0, 0.0
+        for (t, l) in samples[first:]:
+            experts = [np.ascontiguousarray(blob_t[l, int(e)].cpu().numpy()) for e in idx[t, l]]
+            xv = np.ascontiguousarray(x[l % x.shape[0]], np.float32)
+            wv = w[t, l]
+            moe[:] = 0.0
+            t0 = time.perf_counter()
+            for k, eb in enumerate(experts):
+                b = eb.ctypes.data
+                R.ref_cpu_dequant_matvec(b + ofs["gate_w"], b + ofs["gate_s"], b + ofs["gate_b"], xv.ctypes.data,
+                                         g_out.ctypes.data, I, H, 64, bits)
+                R.ref_cpu_dequant_matvec(b + ofs["up_w"], b + ofs["up_s"], b + ofs["up_b"], xv.ctypes.data,
+                                         u_out.ctypes.data, I, H, 64, bits)
+                R.ref_cpu_swiglu(g_out.ctypes.data, u_out.ctypes.data, act.ctypes.data, I)
+                R.ref_cpu_dequant_matvec(b + ofs["down_w"], b + ofs["down_s"], b + ofs["down_b"], act.ctypes.data,
+                                         e_out.ctypes.data, H, I, 64, bits)
+                R.ref_cpu_vec_madd(moe.ctypes.data, e_out.ctypes.data, float(wv[k]), H)
+            t_cpu += time.perf_counter() - t0
+            done += 1
+            if t_cpu >= budget:
+                break
+        return done, t_cpu, moe.copy(), (t, l)
+
     bytes_per_layer = len(idx[0, 0]) * es
+
+    def reference_result(port, ref):
+        if ref is None or ref[0] == 0:
+            return port
+        done_r, t_r, moe_ref, (t_last, l_last) = ref
+        # the last block once more through the port, outside the timing: the two legs must agree
+        mini = np.concatenate([blob_t[l_last, int(e)].cpu().numpy() for e in idx[t_last, l_last]])
+        moe_port, _ = oracle.moe_experts_forward(mini, x[l_last % x.shape[0]], np.arange(len(idx[t_last, l_last]), dtype=np.int32),
+                                                 w[t_last, l_last], H, I, bits, scale_dtype=scale_dtype)
+        same = bool(np.array_equal(moe_ref.view(np.uint32), moe_port.view(np.uint32)))
+        out = {
+            "value": round(done_r * bytes_per_layer / t_r / 1e9, 4),
+            "unit": "GB/s",
+            "cores": 1,
+            "kind": "reference",
+            "us_per_layer": round(t_r / done_r * 1e6, 1),
+            "sample": "%d (token, layer) expert blocks of the same workload (8 experts each, %.1f s of CPU "
+                      "time) through the reference's own cpu_dequant_matvec / cpu_swiglu / cpu_vec_madd "
+                      "(finchmoe/infer.m:1676-1881 compiled gcc -O2 into oracle/_ref/libfm_ref.so), called in "
+                      "the order of its CPU expert loop; host has %d logical CPUs" % (done_r, t_r, os.cpu_count()),
+            "equals_port_bit_for_bit": same,
+            "port": {k: port[k] for k in ("value", "unit", "cores", "us_per_layer", "sample")},
+            "rows_over_threads": port["rows_over_threads"],
+        }
+        return out
+
     done, t_cpu = leg(1, budget_s, 0)
     many = min(16, os.cpu_count() or 1)
     done_m, t_m = leg(many, min(3.0, budget_s / 4), done)
-    return {
+    port = {
         "value": round(done * bytes_per_layer / t_cpu / 1e9, 4),
         "unit": "GB/s",
         "cores": 1,
@@ -118,6 +178,11 @@ def cpu_baseline_decode(blob_t, lo, idx, w, x, budget_s=12.0, bits=3, scale_dtyp
                               "cores": many, "us_per_layer": round(t_m / done_m * 1e6, 1),
                               "sample": "%d further blocks, %.1f s" % (done_m, t_m)},
     }
+    try:
+        return reference_result(port, ref_leg(budget_s, done + done_m))
+    except Exception as exc:          # the reference leg must never cost the run its result
+        print("bench.py: reference CPU leg skipped: %r" % (exc,), file=sys.stderr)
+        return port
 
 
 def run_decode_step(args):

@@ -53,3 +53,32 @@ def test_zipf_routing_of_the_benchmark():
     # a fresh permutation per layer: the hot experts differ between layers
     hot = [int(np.bincount(idx[:, l].reshape(-1), minlength=256).argmax()) for l in range(3)]
     assert len(set(hot)) > 1
+
+
+def test_cpu_baseline_legs_on_a_small_store():
+    """bench.py's CPU leg on a store of 2 layers x 8 experts held in host memory: the port
+    (oracle) leg, and — where oracle/_ref has been built — the leg through the reference's own
+    compiled functions, which must reproduce the port's result bit for bit."""
+    import numpy as np
+    import torch
+    import bench
+    from finchmoe_amd import formats
+    from oracle import oracle
+    rng = np.random.default_rng(3)
+    lo = formats.expert_layout(bench.H, bench.I, 3)
+    Ls, E = 2, 8
+    blob = torch.from_numpy(np.stack([formats.synth_expert_layer(rng, E, bench.H, bench.I, 3).reshape(E, -1)
+                                      for _ in range(Ls)]))
+    idx = np.stack([[rng.permutation(E) for _ in range(Ls)] for _ in range(3)]).astype(np.int32)
+    w = rng.random((3, Ls, E)).astype(np.float32)
+    x = rng.standard_normal((Ls, bench.H)).astype(np.float32)
+    res = bench.cpu_baseline_decode(blob, lo, idx, w, x, budget_s=0.05, bits=3)
+    assert res["unit"] == "GB/s" and res["cores"] == 1 and res["value"] > 0 and "sample" in res
+    if oracle.ref_lib() is not None:
+        assert res["kind"] == "reference" and res["equals_port_bit_for_bit"] is True
+        assert res["port"]["value"] > 0
+    else:
+        assert res["kind"] == "port"
+    # FP16 scales: the reference's files hold none, the port leg stands alone
+    res16 = bench.cpu_baseline_decode(blob, lo, idx, w, x, budget_s=0.05, bits=3, scale_dtype=1)
+    assert res16["kind"] == "port"
