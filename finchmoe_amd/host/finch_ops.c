@@ -278,6 +278,26 @@ int moe_experts_forward_chunk(int layer_idx, const float *h_post, const int *exp
     return 1;
 }
 
+int moe_experts_forward_chunk_bf16(int layer_idx, const uint16_t *h_post_bf16, const int *expert_indices,
+                                   const float *expert_weights, int M, int K, float *moe_out) {
+    if (!g_ctx) { fail(FM_ERR_STATE, "moe_experts_forward_chunk_bf16"); return 0; }
+    int rc = fm_moe_prefill_bf16(g_ctx, layer_idx, h_post_bf16, expert_indices, expert_weights, M, K,
+                                 moe_out, FM_ACCUMULATE);
+    if (rc) { fail(rc, "moe_experts_forward_chunk_bf16"); return 0; }
+    g_status = FM_OK;
+    return 1;
+}
+
+int gpu_gguf_experts_forward_chunk(int layer_idx, const float *h_post, const int *expert_indices,
+                                   const float *expert_weights, int M, int K, float *moe_out) {
+    if (!g_ctx) { fail(FM_ERR_STATE, "gpu_gguf_experts_forward_chunk"); return 0; }
+    int rc = fm_gguf_moe_prefill(g_ctx, layer_idx, h_post, expert_indices, expert_weights, M, K,
+                                 moe_out, FM_ACCUMULATE);
+    if (rc) { fail(rc, "gpu_gguf_experts_forward_chunk"); return 0; }
+    g_status = FM_OK;
+    return 1;
+}
+
 /* ---- routing (finchmoe/infer.m:1794-1840): runs on the host in the reference too ---- */
 void cpu_softmax(float *x, int dim) {
     float mx = x[0];

@@ -84,6 +84,15 @@ int gpu_gguf_experts_forward(int layer_idx, const float *h_post, const int *expe
 int moe_experts_forward_chunk(int layer_idx, const float *h_post, const int *expert_indices,
                               const float *expert_weights, int M, int K, float *moe_out);
 
+/* the same chunk with the positions as BF16 bits (an engine that keeps its residual stream in
+ * bf16; the reference's prefill buffers are fp32, infer.m:10704-10765) */
+int moe_experts_forward_chunk_bf16(int layer_idx, const uint16_t *h_post_bf16, const int *expert_indices,
+                                   const float *expert_weights, int M, int K, float *moe_out);
+/* chunk of M positions on the GGUF store (prefill_chunk_cmd3_batch_general, infer.m:10958-11059:
+ * the *_pool_prefill kernels once per position; here grouped by expert from 32 positions on) */
+int gpu_gguf_experts_forward_chunk(int layer_idx, const float *h_post, const int *expert_indices,
+                                   const float *expert_weights, int M, int K, float *moe_out);
+
 /* routing runs on the CPU in the reference (finchmoe/infer.m:1794-1840, 9285-9289) */
 void cpu_softmax(float *x, int dim);
 void cpu_topk(const float *scores, int dim, int K, int *indices, float *values);

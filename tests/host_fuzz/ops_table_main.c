@@ -68,6 +68,9 @@ int fm_moe_decode(fm_ctx *c, int l, const float *x, const int32_t *i, const floa
 int fm_gguf_moe_decode(fm_ctx *c, int l, const float *x, const int32_t *i, const float *w, int K, float *o, float *e, int f) { (void)c; (void)l; (void)x; (void)i; (void)w; (void)K; (void)e; (void)f; o[0] = 4.0f; return FM_OK; }
 int fm_moe_prefill(fm_ctx *c, int l, const float *X, const int32_t *i, const float *w, int M, int K, float *o, int f) { (void)c; (void)l; (void)X; (void)i; (void)w; (void)M; (void)K; (void)f; o[0] = 5.0f; return FM_OK; }
 
+int fm_moe_prefill_bf16(fm_ctx *c, int l, const uint16_t *X, const int32_t *i, const float *w, int M, int K, float *o, int f) { (void)c; (void)l; (void)X; (void)i; (void)w; (void)M; (void)K; o[0] = f == FM_ACCUMULATE ? 6.0f : -1.0f; return l < 0 ? FM_ERR_ARG : FM_OK; }
+int fm_gguf_moe_prefill(fm_ctx *c, int l, const float *X, const int32_t *i, const float *w, int M, int K, float *o, int f) { (void)c; (void)l; (void)X; (void)i; (void)w; (void)M; (void)K; o[0] = f == FM_ACCUMULATE ? 7.0f : -1.0f; return l < 0 ? FM_ERR_ARG : FM_OK; }
+
 #define CHECK(cond) do { if (!(cond)) { printf("FAILED line %d: %s\n", __LINE__, #cond); return 1; } } while (0)
 
 int main(void) {
@@ -138,6 +141,17 @@ int main(void) {
     fail_register_after = -1;
     fast_dequant_matvec(&arena[60300], sb, sb, x, out, 4, 64, 64, 4);
     CHECK(finch_ops_last_status() == FM_OK && out[0] == 1.0f);
+
+    /* the chunk wrappers: 1 / 0 like the reference's expert functions, accumulate flag passed on */
+    {
+        uint16_t xb[64] = {0};
+        int idx[8] = {0};
+        float w8[8] = {0};
+        CHECK(moe_experts_forward_chunk_bf16(0, xb, idx, w8, 1, 8, out) == 1 && out[0] == 6.0f);
+        CHECK(gpu_gguf_experts_forward_chunk(0, x, idx, w8, 1, 8, out) == 1 && out[0] == 7.0f);
+        CHECK(moe_experts_forward_chunk_bf16(-1, xb, idx, w8, 1, 8, out) == 0 && finch_ops_last_status() == FM_ERR_ARG);
+        CHECK(gpu_gguf_experts_forward_chunk(-1, x, idx, w8, 1, 8, out) == 0 && finch_ops_last_status() == FM_ERR_ARG);
+    }
 
     finch_ops_shutdown();
     finch_ops_shutdown();
