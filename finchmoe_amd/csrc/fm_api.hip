@@ -101,6 +101,8 @@ struct LayerBuf {
 }  // namespace
 
 #define FM_TAIL_PARTIALS 4096
+// positions of one chunk: the chunk kernels index pairs x hidden in 32 bits
+#define FM_MAX_CHUNK 65535
 
 struct fm_ctx {
     int device = 0;
@@ -690,7 +692,7 @@ static int moe_host_call(fm_ctx *c, moe_dev_fn fn, int hidden, int layer, const 
                          const int32_t *idx, const float *w, int M, int K, float *out,
                          float *expert_out, int flags, size_t x_elem = 4) {
     if (!x || !idx || !w || !out) return fail(c, FM_ERR_ARG, "null pointer");
-    if (M < 1) return fail(c, FM_ERR_ARG, "M %d", M);
+    if (M < 1 || M > FM_MAX_CHUNK) return fail(c, FM_ERR_ARG, "M %d outside 1..%d", M, FM_MAX_CHUNK);
     if (K < 1 || K > FM_MAX_K) return fail(c, FM_ERR_ARG, "K %d outside 1..%d", K, FM_MAX_K);
     DeviceGuard dg(c->device);
     size_t nx = (size_t)M * hidden * 4, ni = (size_t)M * K * 4, ne = (size_t)M * K * hidden * 4;
@@ -759,7 +761,7 @@ static int moe_prefill_any(fm_ctx *c, int layer, const void *d_X, bool x_bf16, c
     if (!c) return FM_ERR_ARG;
     if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
     if (!d_X || !d_idx || !d_w || !d_out) return fail(c, FM_ERR_ARG, "null pointer");
-    if (M < 1) return fail(c, FM_ERR_ARG, "M %d", M);
+    if (M < 1 || M > FM_MAX_CHUNK) return fail(c, FM_ERR_ARG, "M %d outside 1..%d", M, FM_MAX_CHUNK);
     if (K < 1 || K > FM_MAX_K) return fail(c, FM_ERR_ARG, "K %d outside 1..%d", K, FM_MAX_K);
     if (((uintptr_t)d_X | (uintptr_t)d_out) & 15)
         return fail(c, FM_ERR_ARG, "X / out not 16-byte aligned");
@@ -1406,7 +1408,7 @@ extern "C" int fm_launch_prefill_gguf(const uint8_t *d_gate, const uint8_t *d_up
 extern "C" int fm_gguf_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, const int32_t *d_idx,
                                        const float *d_w, int M, int K, float *d_out, int flags) {
     if (!c) return FM_ERR_ARG;
-    if (M < 1) return fail(c, FM_ERR_ARG, "M %d", M);
+    if (M < 1 || M > FM_MAX_CHUNK) return fail(c, FM_ERR_ARG, "M %d outside 1..%d", M, FM_MAX_CHUNK);
     static const bool no_group = getenv("FINCH_GGUF_NO_GROUP") != nullptr;
     // (grouping pays from about four positions per expert on: measured at 256 experts, a chunk of
     // 64 positions is faster position by position, 152 against 179 us, one of 512 is 2.7 times

@@ -175,7 +175,7 @@ FM_API int fm_moe_decode_step_noalloc_dev(fm_ctx *ctx, int layer0, int n_layers,
  * (finchmoe/infer.m:10704-11059): M positions, each with its own top-K.
  *   X[M][hidden] fp32, idx[M][K], w[M][K], out[M][hidden] fp32; X and out 16-byte
  *   aligned (fp32 vectors are read and written four at a time throughout the library).
- * Result contract: the same as fm_moe_decode per position. */
+ * Result contract: the same as fm_moe_decode per position.  1 <= M <= 65535. */
 FM_API int fm_moe_prefill_dev(fm_ctx *ctx, int layer, const float *d_X, const int32_t *d_idx,
                        const float *d_w, int M, int K, float *d_out, int flags);
 FM_API int fm_moe_prefill(fm_ctx *ctx, int layer, const float *X, const int32_t *idx,
