@@ -15,6 +15,16 @@
 //   down    (in 512):   4 lanes x 48 B = one 192-byte row, 16 rows per step
 // The scales (and biases) of those rows are contiguous too — [rows][groups]
 // 16-bit, two groups per lane = one dword per lane.
+//
+// What the file holds, in order: the three plain kernels above (fm_gate_up_swiglu, fm_down,
+// fm_combine: any shape, registers only); the streaming forms of the first two
+// (fm_gate_up_swiglu_lds, fm_down_lds: weight ring in LDS filled by LDS-direct loads, inner
+// product on the matrix cores); fm_moe_fused, the three phases as one persistent launch with
+// dependency counters per vector (the form that keeps the per-expert vectors and the finite
+// guard); fm_moe_fused_rows, the launch that sums a row block's experts in LDS and writes only
+// the layer's output (the default when nobody asks for the per-expert vectors); the launchers.
+// All of them add the K experts of a row in slot order with the same arithmetic, so their
+// results are equal bit for bit.
 #include "fm_mfma.h"
 #include "fm_ring.h"
 

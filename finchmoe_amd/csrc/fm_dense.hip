@@ -8,6 +8,13 @@
 // Same lane mapping as the expert kernels: a lane owns 128 columns, LPR =
 // in_dim/128 lanes share a row, a wave step covers 64/LPR rows that are
 // contiguous in memory.
+//
+// Kernels: fm_dense_gemv (one workgroup per row tile, vector-ALU unpack: small launches),
+// fm_dense_stream (one workgroup per CU, weight ring in LDS, matrix cores: launches with a wave
+// step for every wave of the chip; up to two raw-BF16 tensors of a few rows can ride along at
+// its end), fm_dense_gemv_mixed (tensors of different code widths in one launch, optionally with
+// the token's routing done by the workgroup that finishes last), fm_dense_bf16 (unquantized
+// BF16 tensors, cpu_dequant_matvec with scales == NULL, finchmoe/infer.m:1689-1701).
 #include "fm_mfma.h"
 #include "fm_ring.h"
 #include "fm_route.h"
