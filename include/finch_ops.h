@@ -7,8 +7,10 @@
  * stay resident.
  *
  * Differences from the reference, all deliberate:
- *   - nothing aborts: a failed call leaves its output untouched and records a
- *     status readable with finch_ops_last_status() / finch_ops_last_error()
+ *   - nothing aborts: a failed matvec call fills its output with zeros (the call sites
+ *     take a void result and go on to read it), a failed expert call returns 0 and
+ *     leaves moe_out as it was, and both record a status readable with
+ *     finch_ops_last_status() / finch_ops_last_error()
  *     (the reference abort()s on a BF16 tensor reaching a 4-bit kernel,
  *     infer.m:2879-2885, and falls back to the CPU elsewhere; there is no CPU
  *     fallback here)

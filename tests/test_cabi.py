@@ -76,3 +76,24 @@ def test_product_does_not_import_oracle():
             if f.endswith((".py", ".c", ".h", ".hip", ".cpp")):
                 text = open(os.path.join(dirpath, f), errors="ignore").read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+
+
+def test_integration_example_compiles_and_links(tmp_path):
+    """examples/engine_moe_layer.c — the reference's call sites written against the two host
+    headers — compiles as strict C99 and links against the built libraries; without a GPU it
+    ends with the library's error, not a crash."""
+    import shutil
+    import subprocess
+    if not shutil.which("gcc"):
+        pytest.skip("no host compiler")
+    libdir = os.path.join(ROOT, "finchmoe_amd")
+    out = str(tmp_path / "engine_moe_layer")
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror",
+                        "-I", os.path.join(ROOT, "include"), os.path.join(ROOT, "examples", "engine_moe_layer.c"),
+                        "-L", libdir, "-lfinchops", "-lfinchhip", "-lm", "-Wl,-rpath," + libdir, "-o", out],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    import torch
+    if not torch.cuda.is_available():
+        r = subprocess.run([out, str(tmp_path)], capture_output=True, text=True, timeout=120)
+        assert r.returncode == 1 and "finch_ops_init" in r.stderr
