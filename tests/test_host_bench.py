@@ -82,3 +82,20 @@ def test_cpu_baseline_legs_on_a_small_store():
     # FP16 scales: the reference's files hold none, the port leg stands alone
     res16 = bench.cpu_baseline_decode(blob, lo, idx, w, x, budget_s=0.05, bits=3, scale_dtype=1)
     assert res16["kind"] == "port"
+
+
+def test_workloads_of_the_unexplained_fault_need_to_be_asked_for():
+    """Workloads that were part of the run that ended in an unexplained GPU fault start only
+    with FINCH_BENCH_UNVERIFIED=1; the default workload and the chunked prefill are not among
+    them."""
+    env = {k: v for k, v in os.environ.items() if k != "FINCH_BENCH_UNVERIFIED"}
+    for extra in (["--workload", "gdn"], ["--workload", "gguf"], ["--bits", "4"], ["--workload", "gguf_chunk", "--chunk", "8"]):
+        r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--no-cpu", *extra], capture_output=True,
+                           text=True, timeout=300, env=env)
+        assert r.returncode == 4 and "FINCH_BENCH_UNVERIFIED" in r.stderr and r.stdout.strip() == "", extra
+    import torch
+    if not torch.cuda.is_available():
+        for extra in ([], ["--workload", "prefill"], ["--workload", "gguf_chunk", "--chunk", "512"]):
+            r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--no-cpu", *extra],
+                               capture_output=True, text=True, timeout=300, env=env)
+            assert r.returncode == 3, extra          # past the gate: stopped by the missing GPU
