@@ -54,7 +54,9 @@ static void quantize_group(const float *p, int n, float maxv, uint8_t *q, uint16
         volatile float d = p[i] - lo;
         volatile float t = d / scale;
         float r = rintf(t);               /* round half to even, as numpy.round */
-        if (r < 0.0f) r = 0.0f;
+        /* (a NaN — only from non-finite weights, whose quantization numpy leaves to the
+         * platform's float-to-integer cast as well — becomes code 0 instead of a cast of NaN) */
+        if (!(r >= 0.0f)) r = 0.0f;
         if (r > maxv) r = maxv;
         q[i] = (uint8_t)r;
     }

@@ -8,9 +8,13 @@
  *
  *   fuzz_files_main dense <dir>    every *.json in <dir> with the same-named .bin
  *   fuzz_files_main gguf  <dir>    every *.gguf in <dir>
+ *   fuzz_files_main quant -        the quantizer on tensors salted with NaN, infinities, the largest
+ *                                  and the smallest floats and constant groups: error codes or codes,
+ *                                  never a conversion the C standard leaves undefined
  * Prints one line per file before it is opened, and a summary; exit code 0 unless a
  * sanitizer aborts the process. */
 #include <dirent.h>
+#include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -110,8 +114,37 @@ static int run_gguf(const char *path) {
     return 1;
 }
 
+static int run_quant(void) {
+    enum { OD = 4, ID = 128 };
+    static float w[OD * ID];
+    static uint8_t packed[OD * ID];
+    uint16_t s[OD * ID / 64], b[OD * ID / 64];
+    const float specials[] = {NAN, INFINITY, -INFINITY, 3.4e38f, -3.4e38f, 1e-45f, 0.0f, -0.0f};
+    const int widths[] = {2, 3, 4, 8};
+    unsigned seed = 1;
+    int calls = 0;
+    for (int bi = 0; bi < 4; bi++)
+        for (int t = 0; t < 2000; t++) {
+            for (int i = 0; i < OD * ID; i++) {
+                seed = seed * 1664525u + 1013904223u;
+                w[i] = (float)((int)((seed >> 8) % 2001u) - 1000) / 500.0f;
+            }
+            for (int k = 0; k < t % 7; k++) {
+                seed = seed * 1664525u + 1013904223u;
+                w[(seed >> 8) % (OD * ID)] = specials[(seed >> 20) % 8];
+            }
+            if (t % 11 == 0)
+                for (int i = 0; i < 64; i++) w[i] = 1.5f;            /* a constant group: the scale clamps */
+            if (finch_quantize_affine_pack(w, OD, ID, 64, widths[bi], packed, s, b) == 0) calls++;
+            touch(packed, (size_t)OD * ID * (size_t)widths[bi] / 8);
+        }
+    printf("done files=%d accepted=%d touched=%lu\n", 8000, calls, g_touched);
+    return 0;
+}
+
 int main(int argc, char **argv) {
     if (argc != 3) return 2;
+    if (strcmp(argv[1], "quant") == 0) return run_quant();
     const int dense = strcmp(argv[1], "dense") == 0;
     DIR *dir = opendir(argv[2]);
     if (!dir) return 2;

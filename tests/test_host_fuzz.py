@@ -150,6 +150,15 @@ def test_manifest_reader_survives_damaged_files(driver, tmp_path):
     assert int(res["files"]) == len(muts) + 1 and int(res["accepted"]) >= 1
 
 
+def test_quantizer_on_non_finite_and_extreme_weights(driver, tmp_path):
+    """NaN, infinities, the largest floats and constant groups through the C quantizer under
+    the sanitizers (float-to-integer conversions included): every call returns and packs."""
+    env = dict(os.environ, UBSAN_OPTIONS="print_stacktrace=1:halt_on_error=1:exitcode=98")
+    r = subprocess.run([driver, "quant", "-"], capture_output=True, text=True, timeout=300, env=env)
+    assert r.returncode == 0, r.stderr[-3000:]
+    assert r.stdout.strip().endswith(tuple("0123456789")) and "accepted=8000" in r.stdout
+
+
 def test_host_layer_bookkeeping_under_sanitizers(tmp_path):
     """finch_ops.c (the table from host weight pointers to resident tensors, the batch wrapper,
     the error paths) compiled with tests/host_fuzz/ops_table_main.c around it: doubles of the C
