@@ -112,7 +112,10 @@ def test_gguf_reader_survives_damaged_files(driver, tmp_path):
     dir_len = head + 2048
     for i, m in enumerate(_mutations(rng, base[:dir_len], 360, structural)):
         (d / ("m%03d.gguf" % i)).write_bytes(m + base[dir_len:] if i % 6 != 2 else m)
-    res = _run(driver, "gguf", d)
+    try:
+        res = _run(driver, "gguf", d)
+    finally:
+        shutil.rmtree(d, ignore_errors=True)       # a few hundred MB of damaged copies
     assert int(res["files"]) == 361 and int(res["accepted"]) >= 1
 
 
@@ -146,7 +149,10 @@ def test_manifest_reader_survives_damaged_files(driver, tmp_path):
         (d / ("m%03d.json" % i)).write_bytes(m)
         # mostly the intact data file; sometimes a shortened or an empty one
         (d / ("m%03d.bin" % i)).write_bytes(blob if i % 7 else blob[:int(rng.integers(0, len(blob)))])
-    res = _run(driver, "dense", d)
+    try:
+        res = _run(driver, "dense", d)
+    finally:
+        shutil.rmtree(d, ignore_errors=True)
     assert int(res["files"]) == len(muts) + 1 and int(res["accepted"]) >= 1
 
 
