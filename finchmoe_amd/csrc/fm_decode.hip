@@ -25,6 +25,7 @@
 // the layer's output (the default when nobody asks for the per-expert vectors); the launchers.
 // All of them add the K experts of a row in slot order with the same arithmetic, so their
 // results are equal bit for bit.
+#include "fm_index.h"
 #include "fm_mfma.h"
 #include "fm_ring.h"
 
@@ -292,8 +293,9 @@ struct FmOperatorStream {
     // geometry of the two phases: units per pair / per segment, this workgroup's
     // units and segments, bytes per unit in the code and in the scale/bias regions
     uint32_t gu_upp, dn_upp;
-    long gu_segu, dn_segu, gu_wg0, gu_wg1, dn_wg0, dn_wg1;
-    int gu_s0, dn_s0, n_up, n_seq;
+    Fm1Split sp;            // this workgroup's shares of both phases (fm_index.h)
+    long gu_segu, dn_segu;
+    int n_up, n_seq;
     uint32_t gu_wstep, gu_sstep, dn_wstep, dn_sstep;
     // Loader's current phase: bytes per unit, region offsets of a unit's first
     // slice, and how far the second slice (up after gate) lies behind it.  Kept
@@ -302,7 +304,6 @@ struct FmOperatorStream {
     // whole object in private memory.
     bool l_gu;
     uint32_t cur_wstep, cur_sstep, cur_w, cur_s, cur_b, d_w, d_s, d_b;
-    int dn_adj;             // dn_s0 - gu_s0 - n_up
     // loader / multiply state
     int lq, cq;             // segment of the loader / of the multiply
     uint32_t l_first, l_n;
@@ -328,20 +329,13 @@ struct FmOperatorStream {
         dn_segu = (long)dn_upp;
         const long gu_total = DO_UP ? (long)n_pairs * gu_upp : 0;
         const long dn_total = DO_DOWN ? (long)n_pairs * dn_upp : 0;
-        gu_wg0 = gu_total * blockIdx.x / gridDim.x;
-        gu_wg1 = gu_total * (blockIdx.x + 1) / gridDim.x;
-        dn_wg0 = dn_total * blockIdx.x / gridDim.x;
-        dn_wg1 = dn_total * (blockIdx.x + 1) / gridDim.x;
-        gu_s0 = (int)(gu_wg0 / gu_segu);
-        dn_s0 = (int)(dn_wg0 / dn_segu);
-        n_up = gu_wg1 > gu_wg0 ? (int)((gu_wg1 - 1) / gu_segu) + 1 - gu_s0 : 0;
-        const int n_dn = dn_wg1 > dn_wg0 ? (int)((dn_wg1 - 1) / dn_segu) + 1 - dn_s0 : 0;
-        n_seq = n_up + n_dn;
+        sp = fm1_split(gu_total, dn_total, gu_segu, dn_segu, blockIdx.x, gridDim.x);
+        n_up = sp.n_up;
+        n_seq = sp.n_up + sp.n_dn;
         gu_wstep = (uint32_t)(RPS_UP * (a.g.hidden * BITS / 8));
         gu_sstep = (uint32_t)(RPS_UP * (a.g.hidden / 64) * 2);
         dn_wstep = (uint32_t)(RPS_DN * (a.g.inter * BITS / 8));
         dn_sstep = (uint32_t)(RPS_DN * (a.g.inter / 64) * 2);
-        dn_adj = dn_s0 - gu_s0 - n_up;
         d_w = a.g.up_w - a.g.gate_w;
         d_s = a.g.up_s - a.g.gate_s;
         d_b = a.g.up_b - a.g.gate_b;
@@ -369,20 +363,11 @@ struct FmOperatorStream {
     }
     // segment number q of the sequence -> phase and segment of that phase
     __device__ __forceinline__ bool seq_gu(int q) const { return q < n_up; }
-    __device__ __forceinline__ int seq_seg(int q) const {
-        return gu_s0 + q + (q < n_up ? 0 : dn_adj);
-    }
+    __device__ __forceinline__ int seq_seg(int q) const { return fm1_seg(sp, q); }
     // this workgroup's part of it: first unit (inside the segment) and count
     template <bool GU>
     __device__ __forceinline__ void seq_part(int q, uint32_t &first, uint32_t &n) const {
-        const long s = seq_seg(q);
-        long segu, w0, w1;
-        if constexpr (GU) segu = gu_segu, w0 = gu_wg0, w1 = gu_wg1;
-        else segu = dn_segu, w0 = dn_wg0, w1 = dn_wg1;
-        const long lo = s * segu > w0 ? s * segu : w0;
-        const long hi = (s + 1) * segu < w1 ? (s + 1) * segu : w1;
-        first = (uint32_t)(lo - s * segu);
-        n = (uint32_t)(hi - lo);
+        fm1_part(sp, q, GU, &first, &n);
     }
     // the loader enters segment q
     __device__ __forceinline__ void loader_enter(int q) {
@@ -744,8 +729,8 @@ void fm_moe_fused(DecodeArgs a, int n_pairs, FmFlags f) {
 // behind every LDS-direct load in flight), barriers likewise.
 // ======================================================================
 constexpr uint32_t FM_ACT_EMPTY = 0xFFC5A3E1u;
-constexpr int FM2_MAX_SEG = 12;         // segments of one workgroup's shares, all sub-phases
-constexpr int FM2_PART_BYTES = 12288;   // partial vectors of a part
+// FM2_MAX_SEG segments of one workgroup's shares and FM2_PART_BYTES of partial vectors of a part:
+// fm_index.h
 
 struct Fm2Seg {
     const uint8_t *blob[FM_MAX_K];
@@ -859,17 +844,6 @@ __device__ __forceinline__ void fm2_build_chunk(float xl, float xh, const FmBuil
     }
 }
 
-#ifdef FM2_TIMING
-// timing aid of experimental builds: per wave, the 100 MHz clock at eight points of the kernel
-__device__ unsigned long long fm2_tlog[1024 * FM_NW * 16];
-#define FM2_T(I)                                                                          \
-    do {                                                                                  \
-        if ((threadIdx.x & 63) == 0 && blockIdx.x < 1024)                                 \
-            fm2_tlog[((size_t)blockIdx.x * FM_NW + (threadIdx.x >> 6)) * 16 + (I)] = wall_clock64(); \
-    } while (0)
-#else
-#define FM2_T(I) do {} while (0)
-#endif
 
 template <int BITS, int LPR_UP, bool FP16>
 struct Fm2Stream {
@@ -960,15 +934,8 @@ struct Fm2Stream {
                 return;
             }
             uint32_t pn;
-            if (l_gu) {
-                const uint32_t uq = l_first + ul;
-                pn = uq / gu_upp;
-                rsn = uq - pn * gu_upp;
-            } else {
-                // expert by expert: unit ul = row block ul % nrb of expert ul / nrb
-                pn = (uint32_t)(((float)ul + 0.5f) * l_inv);
-                rsn = l_first + (ul - pn * l_nrb);
-            }
+            if (l_gu) fm2_gu_unit(l_first, ul, gu_upp, &pn, &rsn);
+            else fm2_dn_unit(l_first, l_nrb, l_inv, ul, &pn, &rsn);     // expert by expert
             tag_n = ((uint32_t)(lq & 1) << 31) | (pn << 28) | ul;
             const uint32_t ba = fm_lds_addr(&tab[lq].blob[pn]);
             const uint32_t lo = __builtin_amdgcn_readfirstlane(fm_lds_r32(ba));
@@ -996,11 +963,7 @@ struct Fm2Stream {
         consumed++;
         c = c + 1 == RING ? 0 : c + 1;
         issue();
-#ifdef FM2_NOCOMPUTE
-        return (float)((t.s ^ t.b ^ t.q[0][0] ^ t.q[1][1] ^ t.q[2][2]) & 3u) + 0.5f;
-#else
         return fm_chunk_sum<LPR>(fm_lane_dot_mfma<BITS, FP16>(t, ar));
-#endif
     }
 
     __device__ __forceinline__ int seg_layer(int q) const {
@@ -1047,7 +1010,6 @@ struct Fm2Stream {
 
     __device__ __forceinline__ void run(int n_pairs) {
         const int K = a.K, n_groups = n_pairs / K, G = gridDim.x, g = blockIdx.x;
-        FM2_T(0);
         // The split.  Down: a workgroup's row blocks lie in ONE layer whenever there are at
         // least as many workgroups as layers (layer l gets the workgroups g with g*L/G == l, its
         // row blocks divided evenly among them), so the down phase has one segment and no
@@ -1055,41 +1017,16 @@ struct Fm2Stream {
         // ranges sized so that gate/up + down bytes are the same for every workgroup (a
         // workgroup with fewer down rows takes more gate/up units).
         // (32-bit arithmetic: the launcher checks that slices x workgroups stays below 2^31)
-        const uint32_t Ku = (uint32_t)K, Gu = (uint32_t)G, Lu = (uint32_t)n_groups;
-        const uint32_t gu_segu = gu_upp * Ku, dn_segu = dn_upp * Ku;
-        const uint32_t gu_total = (uint32_t)n_pairs * gu_upp, rb_total = Lu * dn_upp;
-        const uint32_t s_total = 2u * gu_total + rb_total * Ku;     // slices of the whole operator
-        auto dn_start = [&](uint32_t gg) -> uint32_t {              // first row block of workgroup gg
-            if (gg >= Gu) return rb_total;
-            if (Gu < Lu) return rb_total * gg / Gu;
-            const uint32_t l = gg * Lu / Gu;
-            const uint32_t g_lo = (l * Gu + Lu - 1u) / Lu, g_hi = ((l + 1u) * Gu + Lu - 1u) / Lu;
-            return l * dn_upp + dn_upp * (gg - g_lo) / (g_hi - g_lo);
-        };
-        auto gu_start = [&](uint32_t gg, uint32_t dn0) -> uint32_t {   // first gate/up unit of workgroup gg
-            const uint32_t t = s_total * gg / Gu, d = dn0 * Ku;
-            const uint32_t u = t > d ? (t - d) / 2u : 0u;
-            return u > gu_total ? gu_total : u;
-        };
-        const uint32_t dn_rb0 = dn_start((uint32_t)g), dn_rb1 = dn_start((uint32_t)g + 1u);
-        const uint32_t gu_wg0 = gu_start((uint32_t)g, dn_rb0), gu_wg1 = gu_start((uint32_t)g + 1u, dn_rb1);
-        const uint32_t dn_wg0 = dn_rb0 * Ku, dn_wg1 = dn_rb1 * Ku;
-        const int gu_s0 = (int)(gu_wg0 / gu_segu), dn_s0 = (int)(dn_wg0 / dn_segu);
-        n_up = gu_wg1 > gu_wg0 ? (int)((gu_wg1 - 1u) / gu_segu) + 1 - gu_s0 : 0;
-        const int n_dn = dn_wg1 > dn_wg0 ? (int)((dn_wg1 - 1u) / dn_segu) + 1 - dn_s0 : 0;
-        n_seq = n_up + n_dn;
+        const Fm2Dims dm = fm2_dims(n_pairs, K, G, a.g.inter, a.g.hidden, LPR_UP);
+        const Fm2Split sp = fm2_split(dm, (uint32_t)g);
+        const uint32_t gu_segu = dm.gu_segu;
+        const int gu_s0 = sp.gu_s0;
+        n_up = sp.n_up;
+        n_seq = sp.n_up + sp.n_dn;
         const int qq = threadIdx.x >> 3;        // the segment this thread looks up below
         const bool mine = qq < n_seq;
-        const bool mine_gu = qq < n_up;
-        const uint32_t mine_s = (uint32_t)(mine_gu ? gu_s0 + qq : dn_s0 + (qq - n_up));
-        uint32_t mine_first, mine_n;
-        {
-            const uint32_t segu = mine_gu ? gu_segu : dn_segu, w0 = mine_gu ? gu_wg0 : dn_wg0, w1 = mine_gu ? gu_wg1 : dn_wg1;
-            const uint32_t lo = mine_s * segu > w0 ? mine_s * segu : w0;
-            const uint32_t hi = (mine_s + 1u) * segu < w1 ? (mine_s + 1u) * segu : w1;
-            mine_first = lo - mine_s * segu;
-            mine_n = hi > lo ? hi - lo : 0u;
-        }
+        const Fm2Part mp = fm2_part(dm, sp, mine ? qq : 0);
+        const uint32_t mine_s = mp.seg, mine_first = mp.first, mine_n = mp.n;
 
         // the other activation set becomes empty again (plain stores, nobody reads it now)
         for (unsigned int i = blockIdx.x * blockDim.x + threadIdx.x; i < sy.clear_n; i += G * blockDim.x)
@@ -1101,7 +1038,6 @@ struct Fm2Stream {
         // (every thread loads, and the values are used unconditionally further down: a load
         // whose result is still pending on some path of the control flow makes the compiler
         // wait for every load in flight at the register's next use, in the middle of the stream)
-        FM2_T(8);
         FmActX<LPR_UP> xr0, xr1;
         fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)(n_up > 0 ? gu_s0 : 0) * a.g.hidden, bslot, xr0);
         fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)(n_up > 1 ? gu_s0 + 1 : 0) * a.g.hidden, bslot, xr1);
@@ -1129,23 +1065,16 @@ struct Fm2Stream {
 #pragma unroll
         for (int i = 0; i < FmActX<LPR_UP>::NIT; i++)
             asm volatile("" ::"v"(xr0.xl[i]), "v"(xr0.xh[i]), "v"(xr1.xl[i]), "v"(xr1.xh[i]));
-        FM2_T(9);
         if (n_up > 0) {
             cur_wstep = gu_wstep, cur_sstep = gu_sstep;
             cur_w = a.g.gate_w, cur_s = a.g.gate_s, cur_b = a.g.gate_b;
         }
         __syncthreads();
-        FM2_T(1);
         loader_enter(0);
-        FM2_T(10);
 #pragma nounroll
         for (int k = 0; k < RING; k++) {
             issue();
-#ifdef FM2_TIMING
-            if (k == 0) FM2_T(11);
-#endif
         }
-        FM2_T(2);
         // the images of both gate/up segments (from registers: no load is waited for here); a
         // wave then changes segment on its own, without a barrier
         if (n_up > 0 && threadIdx.x < 256) {
@@ -1180,9 +1109,6 @@ struct Fm2Stream {
                     if ((tag >> 31) != (uint32_t)(cq & 1)) break;
                     const uint32_t pc = (tag >> 28) & 7u, ul = tag & 0x0FFFFFFFu;
                     const float gv = take<LPR_UP>(woff, soff, ar);
-#ifdef FM2_TIMING
-                    if (consumed == 1) FM2_T(3);
-#endif
                     const float uv = take<LPR_UP>(woff, soff, ar);
                     float v = fm_silu_mul(gv, uv);
                     if (!((valid >> pc) & 1u)) v = 0.0f;
@@ -1190,7 +1116,6 @@ struct Fm2Stream {
                 }
             }
         }
-        FM2_T(4);
         // ---------------------------------------------------------- down
         {
             uint32_t woff, soff;
@@ -1228,9 +1153,6 @@ struct Fm2Stream {
                 const uint32_t c_nrb = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, n))) / (uint32_t)K;
                 FmActRegs ar;
                 uint32_t k_cur = 0xFFFFFFFFu;
-#ifdef FM2_TIMING
-                if (cq == n_up) FM2_T(5);
-#endif
                 dry = false;
                 while (issued - consumed < (uint32_t)RING && !dry) issue();
                 while (consumed < issued) {
@@ -1248,13 +1170,11 @@ struct Fm2Stream {
                         fm_lds_w32(part0 + 4u * ((rbi * (uint32_t)K + pc) * RPS_DN + (uint32_t)ris), __float_as_uint(v));
                 }
             }
-            FM2_T(6);
             if (n_seq > n_up) {
                 fm_wg_barrier();
                 reduce_part(n_seq - 1);
             }
         }
-        FM2_T(7);
     }
 };
 
@@ -1296,11 +1216,8 @@ bool fm_dyn_lds_ok(FmKernelSetup &ks, const void *fn, size_t bytes) {
 // workgroups of a streaming launch: one per CU (LDS budget), fewer when there
 // are not enough units to give every wave `per_wave` of them
 dim3 fm_stream_grid(long units, int n_cu, int per_wave) {
-    long wgs = (long)n_cu;
-    const long need = (long)FM_NW * per_wave;
-    if (units < need * wgs) wgs = (units + need - 1) / need;
-    if (wgs < 1) wgs = 1;
-    return dim3((unsigned)wgs);
+    static_assert(FM_NW == 8, "fm_stream_wgs counts eight waves per workgroup");
+    return dim3((unsigned)fm_stream_wgs(units, n_cu, per_wave));
 }
 
 // One fused launch.  Returns FM_ERR_UNSUPPORTED when the grid cannot be made
@@ -1324,10 +1241,7 @@ int launch_fused(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st, con
     per_cu = 1;
     const long up_units = (long)n_pairs * (a.g.inter / (FM_WAVE / LPR_UP));
     const long down_units = (long)n_pairs * (a.g.hidden / (FM_WAVE / (LPR_UP / 4)));
-    long wgs = (long)n_cu * per_cu;
-    const long small = up_units < down_units ? up_units : down_units;
-    if (small < FM_NW * wgs) wgs = (small + FM_NW - 1) / FM_NW;
-    if (wgs < 1) wgs = 1;
+    const long wgs = fm1_fused_wgs(up_units, down_units, n_cu);
     hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(FM_NW * 64), sh, st, a, n_pairs, f);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
@@ -1349,30 +1263,11 @@ int launch_fused_rows(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st
         if (dev >= 0) ks.per_cu[dev] = per_cu;
     }
     if (per_cu < 1) return FM_ERR_UNSUPPORTED;   // the grid could not be resident at once
-    constexpr int RPS_UP = FM_WAVE / LPR_UP, RPS_DN = FM_WAVE / (LPR_UP / 4);
-    const int n_groups = n_pairs / a.K;
-    const long gu_segu = (long)(a.g.inter / RPS_UP) * a.K, dn_rbs = a.g.hidden / RPS_DN;
-    const long up_units = (long)n_groups * gu_segu, rb_total = (long)n_groups * dn_rbs;
-    long wgs = n_cu;
-    const long small = up_units < rb_total * a.K ? up_units : rb_total * a.K;
-    if (small < FM_NW * wgs) wgs = (small + FM_NW - 1) / FM_NW;
-    if (wgs < 1) wgs = 1;
     // the kernel's split (Fm2Stream::run): at most two gate/up segments, and the down segments
     // and the row blocks of one part within the fixed tables
-    const long s_total = 2 * up_units + rb_total * a.K;
-    const long up_share = (s_total / wgs + 1) / 2 + 1;                  // upper bound, in units
-    if (up_share > gu_segu || s_total * wgs >= (1L << 31)) return FM_ERR_UNSUPPORTED;
-    long n_dn, part_rbs;
-    if (wgs >= n_groups) {
-        n_dn = 1;
-        part_rbs = (dn_rbs + wgs / n_groups - 1) / (wgs / n_groups);
-    } else {
-        const long rb_share = (rb_total + wgs - 1) / wgs;
-        n_dn = (rb_share - 1) / dn_rbs + 2;
-        part_rbs = rb_share < dn_rbs ? rb_share : dn_rbs;
-    }
-    if (2 + n_dn > FM2_MAX_SEG) return FM_ERR_UNSUPPORTED;
-    if (part_rbs * a.K * RPS_DN * 4 > FM2_PART_BYTES) return FM_ERR_UNSUPPORTED;
+    const Fm2Plan plan = fm2_plan(n_pairs, a.K, a.g.inter, a.g.hidden, LPR_UP, n_cu);
+    if (!plan.ok) return FM_ERR_UNSUPPORTED;
+    const long wgs = plan.wgs;
     hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(FM_NW * 64), sh, st, a, n_pairs, sy);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
@@ -1488,11 +1383,6 @@ int pick_rows_per_item(int rows, int n_pairs, int min_rows, int cap, int want) {
 
 }  // namespace
 
-#ifdef FM2_TIMING
-extern "C" __attribute__((visibility("default"))) int fm_debug_read_tlog(void *dst, size_t bytes) {
-    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(fm2_tlog), bytes);
-}
-#endif
 
 // Enqueue the operator for n_layers x K pairs (n_layers groups of K slots: the
 // layers of a decode step, or with layer_stride 0 the positions of a chunk).  Shapes are validated by the

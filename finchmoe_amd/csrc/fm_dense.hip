@@ -63,20 +63,15 @@ __device__ __forceinline__ void fm_dense_gemv_rows(const FmDenseArgs &a, int t) 
     const int m = blockIdx.y;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int c = lane % LPR, r = lane / LPR;
-    const int rows_per_wave = a.rows_per_item >> 2;
-    const int row0 = chunk * a.rows_per_item + wave * rows_per_wave;
-    if (row0 >= sp.out_dim) return;          // (the wave comes back to its caller)
-    int steps = rows_per_wave / RPS;
-    {   // the last workgroup of a tensor may be short
-        int left = (sp.out_dim - row0 + RPS - 1) / RPS;
-        if (left < steps) steps = left;
-    }
+    const FmGemvWave gw = fm_gemv_wave(chunk, wave, a.rows_per_item, LPR, sp.out_dim);
+    const int row0 = gw.row0, steps = gw.steps;
+    if (steps == 0) return;                  // (the wave comes back to its caller)
     const int row_bytes = a.in_dim * BITS / 8;
     const int sb_row_bytes = (a.in_dim / 64) * 2;
     const int last_row = sp.out_dim - 1;
     // rows past the end (only when out_dim is not a multiple of 64/LPR) re-read
     // the last row and are not stored
-    auto rowc = [&](int row) { return row < last_row ? row : last_row; };
+    auto rowc = [&](int row) { return fm_gemv_row_clamp(row, sp.out_dim); };
     int row = row0 + r;
     FmRowSlice<BITS> cur, next;
     {
@@ -208,9 +203,9 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
     const uint32_t ring0 = fm_lds_addr(fm_dense_lds) + (uint32_t)wave * (RING * SL::BYTES);
     FmActLds<LPR> *img = reinterpret_cast<FmActLds<LPR> *>(fm_dense_lds + FmDenseRing<BITS>::BYTES);
     const int row_bytes = NS * SLAB_ROW_BYTES, sb_row_bytes = NS * SLAB_SB;
-    const long wg0 = (long)total_units * blockIdx.x / gridDim.x,
-               wg1 = (long)total_units * (blockIdx.x + 1) / gridDim.x;
-    const uint32_t n_units = (uint32_t)(wg1 - wg0);
+    const FmRange wg = fm_share(total_units, blockIdx.x, gridDim.x);
+    const long wg0 = wg.lo;
+    const uint32_t n_units = (uint32_t)(wg.hi - wg.lo);
     // The launch is a chain of memory round trips; the activations' is started first so
     // that it runs beside the counter set-up and the first weight loads instead of after them.
     typedef typename std::conditional<BITS == 8, FmBuildSlot<4>, FmBuildSlot<BITS>>::type BuildSlot;
@@ -238,10 +233,11 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
     };
     auto locate = [&](long u) __attribute__((always_inline)) {
         Where w{a.spec[0].W, a.spec[0].S, a.spec[0].B, a.spec[0].out, 0, a.spec[0].out_dim};
+        const int t = fm_dense_unit_tensor(a.unit_first, a.n, u);
         int first = 0;
 #pragma unroll
         for (int i = 1; i < FM_MAX_BATCH; i++)
-            if (i < a.n && u >= a.unit_first[i]) {
+            if (i == t) {
                 w.W = a.spec[i].W, w.S = a.spec[i].S, w.B = a.spec[i].B, w.out = a.spec[i].out;
                 w.out_dim = a.spec[i].out_dim;
                 first = a.unit_first[i];
@@ -278,9 +274,9 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
 #pragma unroll
             for (int i = 0; i < RPS; i++)
                 __builtin_amdgcn_global_load_lds(
-                    (fm_gptr)(uintptr_t)(wp + (size_t)i * row_bytes + kn * SLAB_ROW_BYTES + lane * 16),
+                    (fm_gptr)(uintptr_t)(wp + fm_dense_slab_woff(i, kn, lane, row_bytes, SLAB_ROW_BYTES)),
                     (fm_lptr)(uintptr_t)(slot + 1024 * i), 16, 0, 0);
-            const uint32_t so = (uint32_t)((lane >> 4) * sb_row_bytes + kn * SLAB_SB + (lane & 15) * 4);
+            const uint32_t so = fm_dense_slab_sboff(kn, lane, sb_row_bytes, SLAB_SB);
             __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(sp + so),
                                              (fm_lptr)(uintptr_t)(slot + SL::WBYTES), 4, 0, 0);
             __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(bp + so),
@@ -347,11 +343,10 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
     // in_proj_a rows next to in_proj_qkv / in_proj_z: finchmoe/infer.m:8118-8122), so that the
     // set is one launch
     if (a.n_riders > 0) {
-        const int gw = (int)blockIdx.x * 8 + wave;
-        if (gw < a.rider_first[a.n_riders]) {
-            const int r = a.n_riders > 1 && gw >= a.rider_first[1] ? 1 : 0;
+        int row = 0;
+        const int r = fm_dense_rider_of(a.rider_first, a.n_riders, (int)blockIdx.x * 8 + wave, &row);
+        if (r >= 0) {
             const FmDenseSpec sp = r ? a.rider[1] : a.rider[0];
-            const int row = gw - (r ? a.rider_first[1] : 0);
             const uint16_t *w = reinterpret_cast<const uint16_t *>(sp.W) + (size_t)row * a.in_dim;
             const float *x = a.x + (size_t)m * a.in_dim;
             const bool vec = a.in_dim % 8 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0;
@@ -368,26 +363,18 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
 // launches the streaming kernel when the shapes allow it; FM_ERR_UNSUPPORTED otherwise
 template <int BITS, bool FP16>
 int launch_dense_stream_t(FmDenseArgs &a, int M, int n_cu, hipStream_t st) {
-    const int lpr_full = a.in_dim / FM_CPL;
-    const int ns = lpr_full == 32 ? 2 : 1, lpr = lpr_full / ns;
-    if (!(lpr == 4 || lpr == 8 || lpr == 16) || (ns == 2 && BITS != 4)) return FM_ERR_UNSUPPORTED;
     if (BITS == 8 && ((uintptr_t)a.x & 15)) return FM_ERR_UNSUPPORTED;
-    const int rps = FM_WAVE / lpr;
-    int units = 0;
-    for (int i = 0; i < a.n; i++) {
-        if (a.spec[i].out_dim % rps) return FM_ERR_UNSUPPORTED;
-        a.unit_first[i] = units;
-        units += a.spec[i].out_dim / rps;
-    }
-    for (int i = a.n; i <= FM_MAX_BATCH; i++) a.unit_first[i] = units;
-    // Worth it only when every wave of the chip gets a unit: below that the launch is a
-    // chain of latencies either way, and the plain kernel's chain is shorter (measured:
-    // 2048 rows of 4096 columns take 6.0 us there and 12.4 us here).
+    int out_dims[FM_MAX_BATCH];
+    for (int i = 0; i < a.n; i++) out_dims[i] = a.spec[i].out_dim;
     // (decided by the tensor shapes alone, so that M positions and one position take the same
-    // kernel and stay bitwise equal)
-    if (units < 8L * n_cu) return FM_ERR_UNSUPPORTED;
-    long wgs = n_cu;
-    if (units < 8 * wgs) wgs = (units + 7) / 8;
+    // kernel and stay bitwise equal; worth it only when every wave of the chip gets a unit: below
+    // that the launch is a chain of latencies either way, and the plain kernel's chain is shorter —
+    // 2048 rows of 4096 columns take 6.0 us there and 12.4 us here)
+    const FmDensePlan plan = fm_dense_stream_plan(out_dims, a.n, a.in_dim, BITS, n_cu);
+    if (!plan.ok) return FM_ERR_UNSUPPORTED;
+    for (int i = 0; i <= FM_MAX_BATCH; i++) a.unit_first[i] = plan.unit_first[i];
+    const int ns = plan.ns, lpr = plan.lpr, units = plan.units;
+    const long wgs = plan.wgs;
     if (a.n_riders > 0 && a.rider_first[a.n_riders] > 8 * wgs) a.n_riders = 0;   // one row per wave
     dim3 grid((unsigned)wgs, M);
 #define FM_DS(L, NS_)                                                                          \
@@ -493,14 +480,12 @@ extern "C" int fm_launch_dense_mixed(FmDenseSpec *specs, int n, int in_dim, int 
     if (n < 1 || n > FM_MAX_BATCH) return FM_ERR_ARG;
     const int lpr = in_dim / FM_CPL;
     if (lpr < 1 || lpr > 64 || (lpr & (lpr - 1)) || in_dim % FM_CPL) return FM_ERR_UNSUPPORTED;
-    const int min_rows = 4 * (FM_WAVE / lpr);
     long total_rows = 0;
     for (int i = 0; i < n; i++) {
         if (specs[i].bits != 3 && specs[i].bits != 4 && specs[i].bits != 8) return FM_ERR_UNSUPPORTED;
         total_rows += specs[i].out_dim;
     }
-    int rpi = min_rows;     // as fm_launch_dense
-    while (rpi * 2 <= 8 * min_rows && (total_rows + rpi - 1) / rpi > 2L * n_cu) rpi *= 2;
+    const int rpi = fm_gemv_rows_per_item(total_rows, 1, lpr, n_cu);     // as fm_launch_dense
     FmDenseArgs a;
     a.n = n;
     a.in_dim = in_dim;
@@ -556,14 +541,12 @@ extern "C" int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, 
     if (n < 1 || n > FM_MAX_BATCH || M < 1) return FM_ERR_ARG;
     const int lpr = in_dim / FM_CPL;
     if (lpr < 1 || lpr > 64 || (lpr & (lpr - 1)) || in_dim % FM_CPL) return FM_ERR_UNSUPPORTED;
-    const int min_rows = 4 * (FM_WAVE / lpr);
     long total_rows = 0;
     for (int i = 0; i < n; i++) total_rows += specs[i].out_dim;
     // Rows per workgroup: the register budget keeps two workgroups per CU resident, and a
     // launch that needs a second round of workgroups pays its start-up latencies twice —
     // so grow the tile until the launch fits in one round (or the tile is 8 steps deep).
-    int rpi = min_rows;
-    while (rpi * 2 <= 8 * min_rows && (total_rows * M + rpi - 1) / rpi > 2L * n_cu) rpi *= 2;
+    const int rpi = fm_gemv_rows_per_item(total_rows, M, lpr, n_cu);
     FmDenseArgs a;
     a.n = n;
     a.in_dim = in_dim;

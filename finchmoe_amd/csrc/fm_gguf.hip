@@ -30,6 +30,7 @@
 // Q6_K blocks are only 2-byte aligned (210 = 2 mod 4).  The loads below are
 // plain multi-dword loads at that alignment, which gfx950 serves in its
 // unaligned-access mode.
+#include "fm_index.h"
 #include "fm_mfma.h"
 #include "fm_ring.h"
 
@@ -678,22 +679,13 @@ constexpr size_t gg_stream_lds() {
 
 extern __shared__ __attribute__((aligned(16))) uint8_t fm_gguf_lds[];
 
-// u / d for u < 2^31 without the division sequence: with l = ceil(log2 d),
-// mul = ceil(2^(31 + l) / d) fits 32 bits and floor(u * mul / 2^(31 + l)) is exact.
-struct GgDiv {
-    uint32_t mul, shift, d;
-    __device__ __forceinline__ uint32_t operator()(uint32_t u) const {
-        return d == 1u ? u : __umulhi(u, mul) >> shift;
-    }
+// u / d without the division sequence (fm_index.h), callable
+struct GgDiv : FmDiv {
+    __device__ __forceinline__ uint32_t operator()(uint32_t u) const { return fm_div(*this, u); }
 };
 inline GgDiv gg_div_make(uint32_t d) {
-    GgDiv r{0u, 0u, d};
-    if (d > 1u) {
-        uint32_t l = 0;
-        while ((1ull << l) < d) l++;
-        r.mul = (uint32_t)(((1ull << (31 + l)) + d - 1) / d);
-        r.shift = l - 1;
-    }
+    GgDiv r;
+    static_cast<FmDiv &>(r) = fm_div_make(d);
     return r;
 }
 
@@ -734,8 +726,8 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
     const uint32_t ring0 = fm_lds_addr(fm_gguf_lds) + (uint32_t)wave * (RING * SLOT);
     Image *img = reinterpret_cast<Image *>(fm_gguf_lds + 8 * RING * SLOT);
     const uint32_t img0 = fm_lds_addr(img);
-    const long wg0 = (long)total_units * blockIdx.x / gridDim.x,
-               wg1 = (long)total_units * (blockIdx.x + 1) / gridDim.x;
+    const FmRange wg = fm_share(total_units, blockIdx.x, gridDim.x);
+    const long wg0 = wg.lo, wg1 = wg.hi;
     const uint32_t n_units = (uint32_t)(wg1 - wg0);
     if (n_units == 0) return;
     const int in_dim = GU ? a.g.hidden : a.g.inter;
@@ -875,22 +867,12 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
 template <int KIND, bool GU>
 int gg_launch_stream(const GgufArgs &a, int n_pairs, int n_cu, hipStream_t st) {
     const int in_dim = GU ? a.g.hidden : a.g.inter, rows = GU ? a.g.inter : a.g.hidden;
-    const int per_lane = KIND == GG_Q6 ? 64 : 128;
-    const int lpr = in_dim / per_lane;
-    if (in_dim % per_lane || !(lpr == 4 || lpr == 8 || lpr == 16)) return FM_ERR_UNSUPPORTED;
-    const int rps = FM_WAVE / lpr;
-    if (rows % rps) return FM_ERR_UNSUPPORTED;
-    const int upp = rows / rps;
-    const long total = (long)n_pairs * upp;
-    if (total >= (1L << 31)) return FM_ERR_UNSUPPORTED;
-    // a workgroup holds the images of 2 layers (gate/up) or 3 pairs (down): keep its share
-    // of the units within that span
-    const long upv = GU ? (long)upp * a.K : upp, max_share = upv * ((GU ? 2 : 3) - 1);
-    long wgs = n_cu;
-    if (total < 8 * wgs) wgs = (total + 7) / 8;
-    if ((total + wgs - 1) / wgs > max_share) wgs = (total + max_share - 1) / max_share;
-    // every share must be <= max_share: shares differ by at most one unit
-    while (wgs < total && (total + wgs - 1) / wgs > max_share) wgs++;
+    // a workgroup holds the images of 2 layers (gate/up) or 3 pairs (down): the plan keeps its
+    // share of the units within that span
+    const FmGgPlan plan = fm_gg_plan(n_pairs, a.K, in_dim, rows, KIND == GG_Q6, GU, n_cu);
+    if (!plan.ok) return FM_ERR_UNSUPPORTED;
+    const int lpr = plan.lpr, upp = plan.upp;
+    const long total = plan.total, wgs = plan.wgs;
 #define GG_ST(L)                                                                               \
     do {                                                                                       \
         auto kfn = fm_gguf_stream<KIND, L, GU>;                                                \

@@ -32,6 +32,7 @@
 // Dense tensors: fm_pf_dense_prep (X -> operand registers, once per chunk) and fm_pf_gemm
 // (V_MFMA_F32_32X32X16_BF16, K split over the waves of a workgroup, partial tiles summed
 // through LDS).
+#include "fm_index.h"
 #include "fm_mfma.h"
 #include "fm_ring.h"
 
@@ -43,7 +44,7 @@ typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef const __attribute__((address_space(1))) uint8_t *gptr;
 
-#define PF_TM 16          // positions per item
+#define PF_TM FM_PF_TM    // positions per item
 #define PF_MAX_EXPERTS 1024
 
 struct PfItem { int expert, start, count, pad; };
@@ -167,7 +168,8 @@ template <int BITS>
 __device__ __forceinline__ void pf_prepare(const float *src, int rows, int cols, uint4 *dst_op,
                                            float2 *dst_sums, int task) {
     const int NG = cols / 64;
-    const int h = task & 1, g = (task >> 1) % NG, m = task / (2 * NG);
+    const FmPfPrepTask pt = fm_pf_prep_task(task, NG);
+    const int h = pt.h, g = pt.g, m = pt.m;
     const bool on = m < rows;
     float x[32];
     if (on) {
@@ -189,11 +191,10 @@ __device__ __forceinline__ void pf_prepare(const float *src, int rows, int cols,
     xs += fm_dpp<0xB1>(xs);
     xo += fm_dpp<0xB1>(xo);
     if (on) {
-        uint4 *dst = dst_op + ((size_t)m * NG + g) * 16;
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            dst[4 * k + 2 * h] = regs[4 * k];
-            dst[4 * k + 2 * h + 1] = regs[4 * k + 1];
+            dst_op[fm_pf_xop_index((size_t)m, NG, g, k, h, 0)] = regs[4 * k];
+            dst_op[fm_pf_xop_index((size_t)m, NG, g, k, h, 1)] = regs[4 * k + 1];
         }
         if (h == 0) dst_sums[(size_t)m * NG + g] = make_float2(xs, xo);
     }
@@ -222,23 +223,25 @@ __device__ __forceinline__ void pf_prepare(const float *src, int rows, int cols,
 // ======================================================================
 template <int BITS>
 struct PfSlab {
+    static constexpr FmPfSlab G = fm_pf_slab(BITS);     // shared with the host-side bounds walk
     static constexpr int GPW = 4;                       // groups per wave
-    static constexpr int CB = 8 * BITS * GPW;           // code bytes of a row inside the slab: 96 / 128
+    static constexpr int CB = G.cb;                     // code bytes of a row inside the slab: 96 / 128
     static constexpr int PS = 16;                       // bytes a lane copies per load
-    static constexpr int RP = CB / PS;                  // pieces per row: 6 / 8
+    static constexpr int RP = G.rp;                     // pieces per row: 6 / 8
     // a row takes one piece slot more in LDS (it stays empty): with 96- or 128-byte rows the
     // 128-bit reads of neighbouring rows would hit the same banks
-    static constexpr int RS = RP + 1;                   // piece slots per row in LDS: 7 / 9
-    static constexpr int PIECES = 32 * RS;              // piece slots of a tile-matrix: 224 / 288
-    static constexpr int NQ = (PIECES + 63) / 64;       // LDS-direct loads for the codes
-    static constexpr int LDS_CODE = PIECES * PS;        // 3584 / 4608
-    static constexpr int SLOT = LDS_CODE + 512;         // + scales 256 + biases 256
+    static constexpr int RS = G.rs;                     // piece slots per row in LDS: 7 / 9
+    static constexpr int PIECES = G.pieces;             // piece slots of a tile-matrix: 224 / 288
+    static constexpr int NQ = G.nq;                     // LDS-direct loads for the codes
+    static constexpr int LDS_CODE = G.lds_code;         // 3584 / 4608
+    static constexpr int SLOT = G.slot;                 // + scales 256 + biases 256
     static constexpr int LOADS = NQ + 2;
     static constexpr int RED_BYTES = 2 * 2 * 8 * 8 * 64 * 4;   // [buffer][matrix][wave][reg][lane]
     // what is left of the 160 KB for the eight waves' rings: 3 slots of 4096 B / 2 of 5120 B
-    static constexpr int RING = (160 * 1024 - RED_BYTES) / (8 * SLOT);
-    static constexpr int LDS_BYTES = 8 * RING * SLOT + RED_BYTES;
+    static constexpr int RING = G.ring;
+    static constexpr int LDS_BYTES = G.lds_bytes;
     static_assert(RING >= 2, "a ring needs a slot in flight beside the one being multiplied");
+    static_assert(LDS_BYTES == 8 * RING * SLOT + RED_BYTES && LDS_BYTES <= 160 * 1024, "LDS layout");
 };
 
 // three bf16 pieces (bit patterns) of v, the last one truncated
@@ -313,14 +316,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // region offsets of the first tile-matrix of a step (this team's), the distance to the
     // second one, rows per step
     // (byte offsets from the blob's — the dense tensor's W — first byte, modulo 2^64)
-    const size_t team_w = 64u * team * row_bytes, team_sb = 64u * team * sb_bytes;
-    const size_t w_off0 = team_w;
-    const size_t s_off0 = (size_t)a.d_s + team_sb;
-    const size_t b_off0 = (size_t)a.d_b + team_sb;
-    const uint32_t w_d = 32u * row_bytes;
-    const uint32_t s_d = 32u * sb_bytes;
-    const uint32_t b_d = 32u * sb_bytes;
-    const uint32_t step_rows = DENSE ? 64u : 256u;
+    const size_t s_off0 = (size_t)a.d_s, b_off0 = (size_t)a.d_b;
     const uint8_t *store = a.d_w;       // (an item's "expert" is 0: one tensor)
     const size_t expert_size = 0;
     // this lane's pieces of a slot copy
@@ -328,14 +324,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     bool cvalid[P::NQ];
 #pragma unroll
     for (int j = 0; j < P::NQ; j++) {
-        const int q = 64 * j + lane;
-        const int row = q / P::RS, piece = q - row * P::RS;
-        cvalid[j] = q < P::PIECES && piece < P::RP;
-        coff[j] = (uint32_t)(row * row_bytes + P::CB * slab + P::PS * piece);
+        int v;
+        coff[j] = fm_pf_piece_off(P::G, j, lane, row_bytes, slab, &v);
+        cvalid[j] = v != 0;
     }
     // scales / biases of the slab: 2*GPW bytes per row, fetched as whole dwords
-    const int sb_slab = (2 * GPW * slab) & ~3;
-    const uint32_t soff = (uint32_t)((lane >> 1) * sb_bytes + sb_slab + 4 * (lane & 1));
+    const uint32_t soff = fm_pf_sb_off(lane, sb_bytes, slab);
 
     // ---- this workgroup's share of the launch: steps [t0, t1) of the sequence
     // (item, step), items in order — every workgroup gets the same number of steps
@@ -344,10 +338,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // Workgroups are dealt out to the eight XCDs in turn and every XCD has an L2 of its own:
     // workgroup b takes share (b % 8) * (grid / 8) + b / 8, so that neighbouring shares — the
     // items of one expert — run behind the same L2 and its weights come from HBM once.
-    const long T = (long)n_items * n_steps;
-    const unsigned int share = gridDim.x % 8u == 0u ? (blockIdx.x % 8u) * (gridDim.x / 8u) + blockIdx.x / 8u
-                                                    : blockIdx.x;
-    const int t0 = (int)(T * share / gridDim.x), t1 = (int)(T * (share + 1) / gridDim.x);
+    const FmRange tr = fm_share((long)n_items * n_steps, fm_xcd_share(blockIdx.x, gridDim.x), gridDim.x);
+    const int t0 = (int)tr.lo, t1 = (int)tr.hi;
 
     // ---- loader: tile-matrices of the share, in order
     int l_t = t0, l_it = t0 / n_steps, l_mat = 0, wpos = 0;
@@ -365,10 +357,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     auto issue = [&]() __attribute__((always_inline)) {
         if (l_done) return;
         const uint32_t slot = ring0 + (uint32_t)wpos * P::SLOT;
-        const size_t row0 = (size_t)l_s * step_rows;
-        const uint8_t *wb = l_blob + (w_off0 + (l_mat ? w_d : 0u) + row0 * row_bytes);
-        const uint8_t *sb = l_blob + (s_off0 + (l_mat ? s_d : 0u) + row0 * sb_bytes);
-        const uint8_t *bb = l_blob + (b_off0 + (l_mat ? b_d : 0u) + row0 * sb_bytes);
+        const size_t row0 = fm_pf_dense_row(l_s, l_mat, team, TEAMS);
+        const uint8_t *wb = l_blob + row0 * row_bytes;
+        const uint8_t *sb = l_blob + (s_off0 + row0 * sb_bytes);
+        const uint8_t *bb = l_blob + (b_off0 + row0 * sb_bytes);
 #pragma unroll
         for (int j = 0; j < P::NQ; j++)
             if (cvalid[j])
@@ -424,12 +416,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 const int piece = n < 16 ? 0 : 1;
                 const size_t m = !on ? 0 : (size_t)(item.start + pos);
                 const int ng = in_dim / 64;
-                const uint4 *src = a.xop + (m * ng + GPW * slab) * 16 + 2 * hh + piece;
                 const float2 *sm = a.xsums + m * ng + GPW * slab;
 #pragma unroll
                 for (int gi = 0; gi < GPW; gi++) {
 #pragma unroll
-                    for (int k = 0; k < 4; k++) A[gi][k] = src[16 * gi + 4 * k];
+                    for (int k = 0; k < 4; k++)
+                        A[gi][k] = a.xop[fm_pf_xop_index(m, ng, GPW * slab + gi, k, hh, piece)];
                     const float2 v = sm[gi];
                     xs[gi] = on ? v.x : 0.0f;
                     xo[gi] = on ? v.y : 0.0f;
@@ -1441,14 +1433,12 @@ int pf_launch_dense(PfArgs a, int n_cu, bool prepare, hipStream_t st) {
     const int prep_tasks = a.M * (a.d_cols / 64) * 2;
     if (prepare)
         hipLaunchKernelGGL(fm_pf_dense_prep<BITS>, dim3(1 + (prep_tasks + 1023) / 1024), dim3(1024), 0, st, a);
-    const long steps = (long)((a.M + PF_TM - 1) / PF_TM) * (a.d_rows / 64);
-    const int grid = steps < n_cu ? (int)steps : n_cu;
+    const int grid = fm_pf_dense_grid(a.M, a.d_rows, 0, n_cu).grid;
     constexpr int LDS = PfSlab<BITS>::LDS_BYTES;
     static FmLdsAttr attr;
     if (!fm_dyn_lds_ready(attr, (const void *)fm_pf_gemm<PF_DENSE, BITS, FP16>, LDS)) return FM_ERR_HIP;
     if (a.d_cols == 512) {       // two slabs: the teams of the down product, 256 rows per step
-        const long tsteps = (long)((a.M + PF_TM - 1) / PF_TM) * (a.d_rows / 256);
-        const int tgrid = tsteps < n_cu ? (int)tsteps : n_cu;
+        const int tgrid = fm_pf_dense_grid(a.M, a.d_rows, 1, n_cu).grid;
         static FmLdsAttr attr_t;
         if (!fm_dyn_lds_ready(attr_t, (const void *)fm_pf_gemm<PF_DENSE_TEAMS, BITS, FP16>, LDS)) return FM_ERR_HIP;
         hipLaunchKernelGGL((fm_pf_gemm<PF_DENSE_TEAMS, BITS, FP16>), dim3(tgrid), dim3(512), LDS, st, a);
@@ -1717,9 +1707,8 @@ __global__ __launch_bounds__(512) void fm_gq_down(PfArgs a) {
 // (gpu_encode_prefill_matvec, finchmoe/infer.m:3672: the reference runs M matvecs).
 extern "C" size_t fm_prefill_dense_ws_bytes(int out_dim, int in_dim, int group_size, int bits, int M) {
     if (!pf_dense_supported(out_dim, in_dim, group_size, bits) || M < 1) return 0;
-    return align256(((size_t)M / PF_TM + 1) * sizeof(PfItem)) + 256 +
-           align256((size_t)M * (in_dim / 64) * 16 * sizeof(uint4)) +
-           align256((size_t)M * (in_dim / 64) * sizeof(float2));
+    static_assert(sizeof(PfItem) == 16 && sizeof(uint4) == 16 && sizeof(float2) == 8, "sizes of fm_pf_dense_ws");
+    return fm_pf_dense_ws(M, in_dim).total;
 }
 
 extern "C" int fm_launch_prefill_dense(const void *d_W, const void *d_S, const void *d_B, int out_dim,
@@ -1735,10 +1724,11 @@ extern "C" int fm_launch_prefill_dense(const void *d_W, const void *d_S, const v
     a.X = d_X;
     a.M = M;
     a.K = 1;
-    a.items = (PfItem *)ws;               ws += align256(((size_t)M / PF_TM + 1) * sizeof(PfItem));
-    a.n_items = (int *)ws;                ws += 256;
-    a.xop = (uint4 *)ws;                  ws += align256((size_t)M * (in_dim / 64) * 16 * sizeof(uint4));
-    a.xsums = (float2 *)ws;
+    const FmPfDenseWs lay = fm_pf_dense_ws(M, in_dim);
+    a.items = (PfItem *)(ws + lay.items);
+    a.n_items = (int *)(ws + lay.n_items);
+    a.xop = (uint4 *)(ws + lay.xop);
+    a.xsums = (float2 *)(ws + lay.xsums);
     a.d_w = (const uint8_t *)d_W;
     a.d_s = (const uint8_t *)d_S - (const uint8_t *)d_W;
     a.d_b = (const uint8_t *)d_B - (const uint8_t *)d_W;

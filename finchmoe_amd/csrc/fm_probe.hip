@@ -6,6 +6,7 @@
 // best; the decode kernels are priced against the published peak and compared with this.
 // No counterpart in the reference (a measurement aid, like its --timing accumulators,
 // finchmoe/infer.m:281-298).
+#include "fm_index.h"
 #include "fm_ring.h"
 
 namespace {
@@ -28,15 +29,9 @@ __global__ __launch_bounds__(PROBE_WAVES * 64) void fm_stream_probe_k(const uint
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t ring0 = fm_lds_addr(fm_probe_lds) + (uint32_t)wave * (PROBE_RING * PROBE_SLOT);
-    const size_t gw = (size_t)blockIdx.x * PROBE_WAVES + wave, nw = (size_t)gridDim.x * PROBE_WAVES;
-    size_t next, end, step;
-    if constexpr (PATTERN == 0) {
-        next = gw, end = n_slots, step = nw;
-    } else if constexpr (PATTERN == 1) {
-        next = n_slots * blockIdx.x / gridDim.x + wave, end = n_slots * (blockIdx.x + 1) / gridDim.x, step = PROBE_WAVES;
-    } else {
-        next = n_slots * gw / nw, end = n_slots * (gw + 1) / nw, step = 1;
-    }
+    const FmProbeWalk pw = fm_probe_walk(PATTERN, n_slots, blockIdx.x, gridDim.x, wave, PROBE_WAVES);
+    size_t next = pw.next;
+    const size_t end = pw.end, step = pw.step;
     uint32_t issued = 0, consumed = 0;
     int wpos = 0, c = 0;
     auto issue = [&]() __attribute__((always_inline)) {

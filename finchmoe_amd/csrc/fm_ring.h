@@ -11,6 +11,7 @@
 // the consumers wait and read with explicit instructions.
 #pragma once
 
+#include "fm_index.h"
 #include "fm_unpack.h"
 
 #if defined(__HIPCC__)
@@ -58,12 +59,8 @@ template <int BITS, int LPR>
 __device__ __forceinline__ void fm_unit_lane_offsets(int lane, int row_bytes, int sb_row_bytes,
                                                      uint32_t &woff, uint32_t &soff,
                                                      int &row_in_step, int &ch) {
-    const int j = lane & 3;
-    ch = (lane >> 2) % LPR;
-    const int rq = lane / (4 * LPR);
-    row_in_step = 4 * rq + j;
-    woff = (uint32_t)(row_in_step * row_bytes + ch * FmLaneBytes<BITS>::value);
-    soff = (uint32_t)(row_in_step * sb_row_bytes + ch * 4);
+    const FmUnitLane u = fm_unit_lane(lane, LPR, FmLaneBytes<BITS>::value, row_bytes, sb_row_bytes);
+    woff = u.woff, soff = u.soff, row_in_step = u.row_in_step, ch = u.ch;
 }
 
 template <int BITS, int I>

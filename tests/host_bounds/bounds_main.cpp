@@ -1,0 +1,626 @@
+// bounds_main.cpp — host-side walk of the kernels' memory accesses.
+//
+// The kernels of finchmoe_amd/csrc form every global address as  base + f(workgroup, wave, lane,
+// unit)  with f taken from fm_index.h.  This program includes the same header, takes the grid the
+// launcher would take, enumerates every (workgroup, unit, lane, load instruction) of a launch and
+// checks each byte range against the size of the buffer it indexes — the sizes bench.py and the
+// GPU tests allocate.  For the streaming kernels it also checks that the ranges tile the weights
+// exactly once (a wrong split shows up as a gap or an overlap even when it stays in bounds).
+// LDS offsets (ring slots, segment tables, partial vectors, images) are checked against the
+// kernels' LDS sizes.  Built with -fsanitize=address,undefined by tests/test_host_bounds.py; no
+// GPU, no HIP.
+//
+// What is NOT shared with the kernels and therefore restated here: the order in which a
+// workgroup's waves claim units (irrelevant for bounds: every unit of a share is claimed exactly
+// once, by fm_claim_unit's counter), the LDS-direct load helpers' fixed per-lane pattern
+// (lane * 16 + 1024 * j for codes, lane * 4 for scales and biases: fm_ring.h), and the activation
+// staging patterns (fm_mfma.h), which index inside one input vector.
+#include "../../finchmoe_amd/csrc/fm_index.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+static int g_fail = 0;
+static std::string g_case;
+
+#define CHECK(cond, ...)                                                  \
+    do {                                                                  \
+        if (!(cond)) {                                                    \
+            if (g_fail < 20) {                                            \
+                std::fprintf(stderr, "FAIL [%s] %s: ", g_case.c_str(), #cond); \
+                std::fprintf(stderr, __VA_ARGS__);                        \
+                std::fprintf(stderr, "\n");                               \
+            }                                                             \
+            g_fail++;                                                     \
+        }                                                                 \
+    } while (0)
+
+// a buffer of `size` bytes; touch() checks a range; with `cover` every byte counts how often a
+// read touched it (for the once-only tiling check; granularity = `gran` bytes)
+struct Region {
+    std::string name;
+    size_t size = 0;
+    size_t gran = 0;
+    std::vector<uint8_t> count;
+    size_t lo = (size_t)-1, hi = 0;
+    unsigned long touches = 0;
+    Region(const char *n, size_t sz, size_t g = 0) : name(n), size(sz), gran(g) {
+        if (gran) count.assign((size + gran - 1) / gran, 0);
+    }
+    void touch(size_t off, size_t len, const char *what) {
+        touches++;
+        if (off > size || len > size - off) {
+            CHECK(false, "%s: %s offset %zu + %zu outside %zu bytes", name.c_str(), what, off, len, size);
+            return;
+        }
+        if (off < lo) lo = off;
+        if (off + len > hi) hi = off + len;
+        if (gran) {
+            CHECK(off % gran == 0 && len % gran == 0, "%s: %s range %zu+%zu not on the %zu-byte grid", name.c_str(),
+                  what, off, len, gran);
+            for (size_t i = off / gran; i < (off + len) / gran; i++)
+                if (count[i] < 255) count[i]++;
+        }
+    }
+    // every grid cell of [a, b) touched exactly once
+    void expect_once(size_t a, size_t b) {
+        size_t bad = 0, first_bad = 0;
+        for (size_t i = a / gran; i < b / gran; i++)
+            if (count[i] != 1) {
+                if (!bad) first_bad = i;
+                bad++;
+            }
+        CHECK(bad == 0, "%s: %zu cells of [%zu, %zu) not read exactly once (first at byte %zu, count %d)",
+              name.c_str(), bad, a, b, first_bad * gran, (int)count[first_bad]);
+    }
+    void expect_untouched(size_t a, size_t b) {
+        for (size_t i = a / gran; i < b / gran; i++)
+            if (count[i] != 0) {
+                CHECK(false, "%s: byte %zu read although outside the operands", name.c_str(), i * gran);
+                return;
+            }
+    }
+};
+
+static const int N_CU = 256;
+
+// the LDS-direct copy of one GEMV unit (fm_dma_issue): NQ loads of 64 lanes x 16 bytes for the
+// codes, one load of 64 x 4 bytes each for scales and biases
+static void unit_dma(Region &W, size_t w0, Region &S, size_t s0, Region &B, size_t b0, int bits) {
+    const int nq = fm_lane_bytes(bits) / 16;
+    for (int lane = 0; lane < 64; lane++) {
+        for (int j = 0; j < nq; j++) W.touch(w0 + (size_t)lane * 16 + 1024 * (size_t)j, 16, "unit codes");
+        S.touch(s0 + (size_t)lane * 4, 4, "unit scales");
+        B.touch(b0 + (size_t)lane * 4, 4, "unit biases");
+    }
+}
+
+// ------------------------------------------------------------------------------------ probe
+static void walk_probe(size_t nbytes, int pattern) {
+    g_case = "stream_probe pattern " + std::to_string(pattern) + " bytes " + std::to_string(nbytes);
+    const size_t n_slots = nbytes / 4096;
+    Region buf("probe buffer", nbytes, 4096);
+    const int G = N_CU, ring = 4, slot = 4096;
+    for (int b = 0; b < G; b++)
+        for (int wave = 0; wave < 8; wave++) {
+            FmProbeWalk w = fm_probe_walk(pattern, n_slots, b, G, wave, 8);
+            for (size_t s = w.next; s < w.end; s += w.step) buf.touch(s * 4096, 4096, "slot");
+            // ring in LDS: wave * ring * slot + wpos * slot + 1024 j + 16 lane + 16
+            CHECK((size_t)wave * ring * slot + (ring - 1) * slot + 3 * 1024 + 63 * 16 + 16 <= (size_t)8 * ring * slot, "ring");
+        }
+    buf.expect_once(0, n_slots * 4096);
+    std::printf("ok  %-58s %zu slots\n", g_case.c_str(), n_slots);
+}
+
+// ------------------------------------------------------------------------------------ dense
+struct DenseT {
+    int out_dim, bits;      // bits 16: raw bf16
+};
+
+static void walk_dense_batch(const char *name, const std::vector<DenseT> &ts, int in_dim, int M,
+                             const std::vector<int> &rider_rows) {
+    g_case = std::string("dense ") + name;
+    const int n = (int)ts.size(), bits = ts[0].bits;
+    const int row_bytes = in_dim * bits / 8, sb_row = (in_dim / 64) * 2;
+    std::vector<Region> W, S, B, O;
+    int out_dims[8];
+    long total_rows = 0;
+    for (int i = 0; i < n; i++) {
+        out_dims[i] = ts[i].out_dim;
+        total_rows += ts[i].out_dim;
+        W.emplace_back("W", (size_t)ts[i].out_dim * in_dim * ts[i].bits / 8, 16);
+        S.emplace_back("S", (size_t)ts[i].out_dim * sb_row, 4);
+        B.emplace_back("B", (size_t)ts[i].out_dim * sb_row, 4);
+        O.emplace_back("out", (size_t)M * ts[i].out_dim * 4, 4);
+    }
+    Region X("x", (size_t)M * in_dim * 4);
+    bool same = true;
+    for (auto &t : ts) same = same && t.bits == bits;
+    const FmDensePlan plan = same ? fm_dense_stream_plan(out_dims, n, in_dim, bits, N_CU) : FmDensePlan{};
+    if (same && plan.ok) {
+        const int lpr = plan.lpr, ns = plan.ns, rps = plan.rps;
+        const int slab_row = lpr * fm_lane_bytes(bits), slab_sb = 4 * lpr;
+        CHECK(ns == 1 || (slab_row == 1024 && rps == fm_lane_bytes(bits) / 16), "one load per row and slab");
+        const int ring = bits == 3 ? 4 : (bits == 8 ? 2 : 3);
+        const size_t slot_bytes = 64 * (size_t)fm_lane_bytes(bits) + 512 + 16;
+        const size_t lds = 8 * ring * slot_bytes + (bits == 8 ? 0 : (size_t)ns * (16 * 4 * lpr * 16 + lpr * 16));
+        CHECK(lds + 16 <= 160 * 1024, "LDS %zu", lds);
+        int riders_first[3] = {0, 0, 0};
+        int n_riders = (int)rider_rows.size();
+        for (int i = 0; i < n_riders; i++) riders_first[i + 1] = riders_first[i] + rider_rows[i];
+        for (int i = n_riders; i < 2; i++) riders_first[i + 1] = riders_first[n_riders];
+        if (n_riders > 0 && riders_first[n_riders] > 8 * plan.wgs) n_riders = 0;
+        std::vector<Region> RW, RO;
+        for (int i = 0; i < n_riders; i++) {
+            RW.emplace_back("rider W", (size_t)rider_rows[i] * in_dim * 2, 2);
+            RO.emplace_back("rider out", (size_t)M * rider_rows[i] * 4, 4);
+        }
+        for (int m = 0; m < M; m++)
+            for (int b = 0; b < plan.wgs; b++) {
+                const FmRange wg = fm_share(plan.units, b, plan.wgs);
+                CHECK(wg.hi - wg.lo >= 8 || plan.units < 8L * plan.wgs, "share of %ld units", wg.hi - wg.lo);
+                for (long u = wg.lo; u < wg.hi; u++) {
+                    const int t = fm_dense_unit_tensor(plan.unit_first, n, u);
+                    const int row0 = (int)(u - plan.unit_first[t]) * rps;
+                    CHECK(row0 >= 0 && row0 + rps <= ts[t].out_dim, "unit %ld row0 %d", u, row0);
+                    if (m == 0) {
+                        if (ns == 1) {
+                            unit_dma(W[t], (size_t)row0 * row_bytes, S[t], (size_t)row0 * sb_row, B[t],
+                                     (size_t)row0 * sb_row, bits);
+                        } else {
+                            for (int kn = 0; kn < ns; kn++)
+                                for (int lane = 0; lane < 64; lane++) {
+                                    for (int i = 0; i < rps; i++)
+                                        W[t].touch((size_t)row0 * row_bytes + fm_dense_slab_woff(i, kn, lane, row_bytes, slab_row), 16,
+                                                   "slab codes");
+                                    const uint32_t so = fm_dense_slab_sboff(kn, lane, sb_row, slab_sb);
+                                    S[t].touch((size_t)row0 * sb_row + so, 4, "slab scales");
+                                    B[t].touch((size_t)row0 * sb_row + so, 4, "slab biases");
+                                }
+                        }
+                    }
+                    for (int lane = 0; lane < 64; lane++) {
+                        const FmUnitLane ul = fm_unit_lane(lane, lpr, fm_lane_bytes(bits), slab_row, slab_sb);
+                        // the lane's reads back out of the slot
+                        CHECK(ul.woff + (uint32_t)fm_lane_bytes(bits) <= 64u * fm_lane_bytes(bits), "woff");
+                        CHECK(ul.soff + 4 <= 256, "soff");
+                        if (ul.ch == 0) O[t].touch(((size_t)m * ts[t].out_dim + row0 + ul.row_in_step) * 4, 4, "out");
+                    }
+                }
+                for (int wave = 0; wave < 8 && n_riders; wave++) {
+                    int row = 0;
+                    const int r = fm_dense_rider_of(riders_first, n_riders, b * 8 + wave, &row);
+                    if (r < 0) continue;
+                    if (m == 0) RW[r].touch((size_t)row * in_dim * 2, (size_t)in_dim * 2, "rider row");
+                    RO[r].touch(((size_t)m * rider_rows[r] + row) * 4, 4, "rider out");
+                }
+            }
+        for (int i = 0; i < n; i++) {
+            W[i].expect_once(0, W[i].size);
+            S[i].expect_once(0, S[i].size);
+            B[i].expect_once(0, B[i].size);
+            O[i].expect_once(0, O[i].size);
+        }
+        for (int i = 0; i < n_riders; i++) RW[i].expect_once(0, RW[i].size), RO[i].expect_once(0, RO[i].size);
+        std::printf("ok  %-58s stream: %d units over %d workgroups, ns %d\n", g_case.c_str(), plan.units, plan.wgs, ns);
+        return;
+    }
+    // plain kernel (also the launch of tensors of different widths): a workgroup per row tile
+    const int lpr = in_dim / FM_CPL;
+    const int rpi = fm_gemv_rows_per_item(total_rows, same ? M : 1, lpr, N_CU);
+    const int rps = FM_WAVE / lpr;
+    for (int t = 0; t < n; t++) {
+        const int tb = ts[t].bits, bpl = fm_lane_bytes(tb), rb = in_dim * tb / 8;
+        const int items = (ts[t].out_dim + rpi - 1) / rpi;
+        for (int m = 0; m < M; m++)
+            for (int chunk = 0; chunk < items; chunk++)
+                for (int wave = 0; wave < 4; wave++) {
+                    const FmGemvWave gw = fm_gemv_wave(chunk, wave, rpi, lpr, ts[t].out_dim);
+                    for (int it = 0; it < gw.steps; it++)
+                        for (int lane = 0; lane < 64; lane++) {
+                            const int c = lane % lpr, r = lane / lpr;
+                            const int row = gw.row0 + it * rps + r;
+                            const size_t ro = (size_t)fm_gemv_row_clamp(row, ts[t].out_dim);
+                            // (clamped rows re-read the last row: no once-only check on W here)
+                            Region w1("W", W[t].size), s1("S", S[t].size);
+                            w1.touch(ro * rb + (size_t)c * bpl, bpl, "row slice");
+                            s1.touch(ro * sb_row + (size_t)c * 4, 4, "row scale");
+                            X.touch(((size_t)m * in_dim + (size_t)c * FM_CPL) * 4, FM_CPL * 4, "x chunk");
+                            if (c == 0 && row <= ts[t].out_dim - 1) O[t].touch(((size_t)m * ts[t].out_dim + row) * 4, 4, "out");
+                        }
+                }
+        O[t].expect_once(0, O[t].size);
+    }
+    std::printf("ok  %-58s plain kernel: %d rows per workgroup\n", g_case.c_str(), rpi);
+}
+
+// --------------------------------------------------------------------- dense against M positions
+static void walk_pf_dense(int out_dim, int in_dim, int bits, int M) {
+    g_case = "prefill dense " + std::to_string(out_dim) + "x" + std::to_string(in_dim) + " " + std::to_string(bits) +
+             "-bit M=" + std::to_string(M);
+    const bool teams = in_dim == 512;
+    const FmPfSlab sl = fm_pf_slab(bits);
+    CHECK(sl.ring >= 2 && sl.lds_bytes <= 160 * 1024, "LDS %d ring %d", sl.lds_bytes, sl.ring);
+    const int row_bytes = in_dim * bits / 8, sb_bytes = (in_dim / 64) * 2, ng = in_dim / 64;
+    const FmPfDenseWs ws = fm_pf_dense_ws(M, in_dim);
+    Region WS("workspace", ws.total);
+    Region Wt("W", (size_t)out_dim * row_bytes, 16), St("S", (size_t)out_dim * sb_bytes, 4), Bt("B", (size_t)out_dim * sb_bytes, 4);
+    Region X("X", (size_t)M * in_dim * 4, 4), Out("out", (size_t)M * out_dim * 4);
+    Region Xop("xop", (size_t)M * ng * 16 * 16, 16), Xs("xsums", (size_t)M * ng * 8, 8);
+    // carve-up: every part inside the workspace, in order, not overlapping
+    CHECK(ws.items + ((size_t)(M + 15) / 16) * 16 <= ws.n_items, "items part");
+    CHECK(ws.n_items + 4 <= ws.xop && ws.xop + Xop.size <= ws.xsums && ws.xsums + Xs.size <= ws.total, "carve-up");
+    // ---- fm_pf_dense_prep: block 0 writes the items, blocks 1.. prepare X
+    const int n_items = (M + FM_PF_TM - 1) / FM_PF_TM;
+    const int prep_tasks = M * ng * 2, prep_blocks = (prep_tasks + 1023) / 1024;
+    for (int t = 0; t < prep_blocks * 1024; t++) {
+        const FmPfPrepTask pt = fm_pf_prep_task(t, ng);
+        if (pt.m >= M) continue;
+        X.touch(((size_t)pt.m * in_dim + 64 * pt.g + 32 * pt.h) * 4, 32 * 4, "prep x");
+        for (int k = 0; k < 4; k++)
+            for (int p = 0; p < 2; p++) Xop.touch(fm_pf_xop_index(pt.m, ng, pt.g, k, pt.h, p) * 16, 16, "prep xop");
+        if (pt.h == 0) Xs.touch(((size_t)pt.m * ng + pt.g) * 8, 8, "prep xsums");
+    }
+    X.expect_once(0, X.size);
+    Xop.expect_once(0, Xop.size);
+    Xs.expect_once(0, Xs.size);
+    // ---- fm_pf_gemm
+    const FmPfDenseGrid gr = fm_pf_dense_grid(M, out_dim, teams, N_CU);
+    CHECK(gr.items == n_items, "items");
+    const int passes = teams ? 1 : in_dim / 2048;
+    const long T = (long)n_items * gr.n_steps;
+    std::vector<uint8_t> seen(T, 0);
+    for (int pass = 0; pass < passes; pass++) {
+        Region Wp("W (pass)", Wt.size, 16);
+        for (int b = 0; b < gr.grid; b++) {
+            const FmRange tr = fm_share(T, fm_xcd_share(b, gr.grid), gr.grid);
+            for (long t = tr.lo; t < tr.hi; t++) {
+                const int it = (int)(t / gr.n_steps), s = (int)(t - (long)it * gr.n_steps);
+                CHECK(it < n_items, "item %d", it);
+                if (pass == 0) seen[t]++;
+                const int start = it * FM_PF_TM, count = M - start < FM_PF_TM ? M - start : FM_PF_TM;
+                for (int wave = 0; wave < 8; wave++) {
+                    const int slab = teams ? (wave & 1) : wave + 8 * pass, team = teams ? (wave >> 1) : 0;
+                    CHECK(4 * slab + 3 < ng, "slab %d of %d groups", slab, ng);
+                    for (int mat = 0; mat < 2; mat++) {
+                        const size_t row0 = fm_pf_dense_row(s, mat, team, teams);
+                        CHECK(row0 + 32 <= (size_t)out_dim, "tile rows %zu", row0);
+                        for (int lane = 0; lane < 64; lane++) {
+                            for (int j = 0; j < sl.nq; j++) {
+                                int valid;
+                                const uint32_t co = fm_pf_piece_off(sl, j, lane, row_bytes, slab, &valid);
+                                if (!valid) continue;
+                                Wp.touch(row0 * row_bytes + co, 16, "slab piece");
+                                CHECK((size_t)64 * 16 * j + 16 * lane + 16 <= (size_t)sl.lds_code, "piece slot in LDS");
+                            }
+                            const uint32_t so = fm_pf_sb_off(lane, sb_bytes, slab);
+                            St.touch(row0 * sb_bytes + so, 4, "slab scales");
+                            Bt.touch(row0 * sb_bytes + so, 4, "slab biases");
+                        }
+                    }
+                    // operand registers of the item's positions (rows past the item read position 0)
+                    for (int lane = 0; lane < 64; lane++) {
+                        const int n = lane & 31, hh = lane >> 5, pos = n & 15, piece = n < 16 ? 0 : 1;
+                        const size_t m = pos < count ? (size_t)(start + pos) : 0;
+                        for (int gi = 0; gi < 4; gi++) {
+                            for (int k = 0; k < 4; k++) {
+                                Region xo("xop", Xop.size);
+                                xo.touch(fm_pf_xop_index(m, ng, 4 * slab + gi, k, hh, piece) * 16, 16, "xop read");
+                            }
+                            Region xs("xsums", Xs.size);
+                            xs.touch((m * ng + 4 * slab + gi) * 8, 8, "xsums read");
+                        }
+                        // results
+                        if (!teams) {
+                            const int my_pos = 8 * (wave >> 2) + 4 * hh + (wave & 3);
+                            if (my_pos < count) {
+                                Out.touch(((size_t)(start + my_pos) * out_dim + 64 * s + n) * 4, 4, "out");
+                                Out.touch(((size_t)(start + my_pos) * out_dim + 64 * s + n + 32) * 4, 4, "out");
+                            }
+                        } else {
+                            const int j = wave & 1, row = 256 * s + 64 * team + 32 * j + n;
+                            for (int i = 0; i < 8; i++) {
+                                const int tok = 8 * (i / 4) + 4 * hh + (i % 4);
+                                if (tok < count) Out.touch(((size_t)(start + tok) * out_dim + row) * 4, 4, "out");
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        // a pass reads the pass's columns of every row once for every item
+        (void)Wp;
+    }
+    for (long t = 0; t < T; t++) CHECK(seen[t] == 1, "step %ld taken %d times", t, (int)seen[t]);
+    CHECK(Out.lo == 0 && Out.hi == Out.size, "output range %zu..%zu of %zu", Out.lo, Out.hi, Out.size);
+    std::printf("ok  %-58s %d items x %d steps over %d workgroups, %d passes\n", g_case.c_str(), n_items, gr.n_steps,
+                gr.grid, passes);
+}
+
+// ------------------------------------------------------------------------- affine expert geometry
+struct Geom {
+    int hidden, inter, bits;
+    size_t gate_w, gate_s, gate_b, up_w, up_s, up_b, down_w, down_s, down_b, expert_size;
+};
+static Geom geom(int hidden, int inter, int bits) {
+    Geom g{};
+    g.hidden = hidden, g.inter = inter, g.bits = bits;
+    const size_t gu_w = (size_t)inter * hidden * bits / 8, gu_s = (size_t)inter * (hidden / 64) * 2;
+    const size_t d_w = (size_t)hidden * inter * bits / 8, d_s = (size_t)hidden * (inter / 64) * 2;
+    size_t o = 0;
+    g.gate_w = o; o += gu_w; g.gate_s = o; o += gu_s; g.gate_b = o; o += gu_s;
+    g.up_w = o;   o += gu_w; g.up_s = o;   o += gu_s; g.up_b = o;   o += gu_s;
+    g.down_w = o; o += d_w;  g.down_s = o; o += d_s;  g.down_b = o; o += d_s;
+    g.expert_size = o;
+    return g;
+}
+
+// fm_moe_fused_rows: n_groups layer groups (layers of a step / positions of a chunk) x K slots.
+// Every pair gets an expert blob of its own here, so "read exactly once" is checked per pair.
+static void walk_fused_rows(int n_groups, int K, int hidden, int inter, int bits) {
+    g_case = "fused rows " + std::to_string(n_groups) + " groups x " + std::to_string(K) + ", " + std::to_string(bits) + "-bit";
+    const Geom g = geom(hidden, inter, bits);
+    const int lpr_up = hidden / FM_CPL, lpr_dn = lpr_up / 4, n_pairs = n_groups * K;
+    CHECK(inter / FM_CPL == lpr_dn, "widths");
+    const int rps_up = FM_WAVE / lpr_up, rps_dn = FM_WAVE / lpr_dn;
+    const Fm2Plan plan = fm2_plan(n_pairs, K, inter, hidden, lpr_up, N_CU);
+    if (!plan.ok) {
+        std::printf("--  %-58s not taken by this launch form\n", g_case.c_str());
+        return;
+    }
+    const int G = plan.wgs;
+    const Fm2Dims dm = fm2_dims(n_pairs, K, G, inter, hidden, lpr_up);
+    const uint32_t gu_wstep = rps_up * (hidden * bits / 8), gu_sstep = rps_up * (hidden / 64) * 2;
+    const uint32_t dn_wstep = rps_dn * (inter * bits / 8), dn_sstep = rps_dn * (inter / 64) * 2;
+    // LDS: rings | two gate/up images | segment tables | partial vectors
+    const int ring = bits == 3 ? 4 : 3;
+    const size_t slot = 64 * (size_t)fm_lane_bytes(bits) + 512 + 16;
+    const size_t img_up = (size_t)16 * 4 * lpr_up * 16 + lpr_up * 16, img_dn = (size_t)16 * 4 * lpr_dn * 16 + lpr_dn * 16;
+    const size_t seg_bytes = 8 * 8 + 8 * 4 + 6 * 4;
+    const size_t lds = 8 * ring * slot + 2 * img_up + FM2_MAX_SEG * seg_bytes + FM2_PART_BYTES;
+    CHECK(lds <= 160 * 1024, "LDS %zu", lds);
+    CHECK((size_t)FM_MAX_K * img_dn <= 2 * img_up, "down images in the gate/up images");
+    std::vector<Region> blob;
+    blob.reserve(n_pairs);
+    for (int p = 0; p < n_pairs; p++) blob.emplace_back("expert blob", g.expert_size, 4);
+    Region act("act", (size_t)n_pairs * inter * 4, 4), out("out", (size_t)n_groups * hidden * 4, 4);
+    Region X("x", (size_t)n_groups * hidden * 4), idx("idx", (size_t)n_pairs * 4);
+    int max_seq = 0;
+    size_t max_bytes = 0, min_bytes = (size_t)-1;
+    for (int gi = 0; gi < G; gi++) {
+        const Fm2Split sp = fm2_split(dm, gi);
+        const int n_seq = sp.n_up + sp.n_dn;
+        if (n_seq > max_seq) max_seq = n_seq;
+        CHECK(sp.n_up <= 2, "workgroup %d: %d gate/up segments", gi, sp.n_up);
+        CHECK(n_seq <= FM2_MAX_SEG && n_seq <= 64, "workgroup %d: %d segments", gi, n_seq);
+        // the two input vectors loaded up front
+        if (sp.n_up > 0) X.touch((size_t)sp.gu_s0 * hidden * 4, (size_t)hidden * 4, "x of the first segment");
+        if (sp.n_up > 1) X.touch((size_t)(sp.gu_s0 + 1) * hidden * 4, (size_t)hidden * 4, "x of the second segment");
+        size_t bytes = 0;
+        for (int qq = 0; qq < n_seq; qq++) {
+            const Fm2Part pt = fm2_part(dm, sp, qq);
+            CHECK(pt.seg < (uint32_t)n_groups, "segment %u", pt.seg);
+            for (int k = 0; k < K; k++) idx.touch(((size_t)pt.seg * K + k) * 4, 4, "idx");
+            if (pt.gu) {
+                for (uint32_t ul = 0; ul < pt.n; ul++) {
+                    uint32_t pn, rsn;
+                    fm2_gu_unit(pt.first, ul, dm.gu_upp, &pn, &rsn);
+                    CHECK(pn < (uint32_t)K && rsn < dm.gu_upp, "gate/up unit %u -> slot %u step %u", ul, pn, rsn);
+                    if (pn >= (uint32_t)K) continue;
+                    Region &bl = blob[pt.seg * K + pn];
+                    for (int second = 0; second < 2; second++)
+                        unit_dma(bl, (size_t)rsn * gu_wstep + (second ? g.up_w : g.gate_w), bl,
+                                 (size_t)rsn * gu_sstep + (second ? g.up_s : g.gate_s), bl,
+                                 (size_t)rsn * gu_sstep + (second ? g.up_b : g.gate_b), bits);
+                    bytes += 2 * (64 * (size_t)fm_lane_bytes(bits) + 512);
+                    for (int lane = 0; lane < 64; lane++) {
+                        const FmUnitLane ulr = fm_unit_lane(lane, lpr_up, fm_lane_bytes(bits), hidden * bits / 8, (hidden / 64) * 2);
+                        if (ulr.ch == 0)
+                            act.touch((((size_t)pt.seg * dm.gu_segu + pt.first) * rps_up + ulr.row_in_step + (size_t)ul * rps_up) * 4, 4, "act");
+                    }
+                }
+            } else {
+                CHECK(pt.first % K == 0 && pt.n % K == 0, "down part %u + %u not whole row blocks", pt.first, pt.n);
+                const uint32_t rb_first = pt.first / K, nrb = pt.n / K;
+                const float inv = 1.0f / (float)(nrb ? nrb : 1u);
+                CHECK((size_t)nrb * K * rps_dn * 4 <= FM2_PART_BYTES, "partial vectors of %u row blocks", nrb);
+                for (uint32_t ul = 0; ul < pt.n; ul++) {
+                    uint32_t pn, rsn;
+                    fm2_dn_unit(rb_first, nrb, inv, ul, &pn, &rsn);
+                    CHECK(pn == ul / nrb && rsn == rb_first + ul % nrb, "down unit %u -> slot %u block %u", ul, pn, rsn);
+                    CHECK(pn < (uint32_t)K && rsn < dm.dn_upp, "down unit %u -> slot %u block %u", ul, pn, rsn);
+                    if (pn >= (uint32_t)K) continue;
+                    Region &bl = blob[pt.seg * K + pn];
+                    unit_dma(bl, (size_t)rsn * dn_wstep + g.down_w, bl, (size_t)rsn * dn_sstep + g.down_s, bl,
+                             (size_t)rsn * dn_sstep + g.down_b, bits);
+                    bytes += 64 * (size_t)fm_lane_bytes(bits) + 512;
+                    const uint32_t rbi = ul - pn * nrb;
+                    for (int ris = 0; ris < rps_dn; ris++)
+                        CHECK(4u * ((rbi * K + pn) * rps_dn + ris) + 4 <= FM2_PART_BYTES, "partial slot");
+                }
+                // activations of the layer's K experts, and the part's rows of out
+                Region a1("act", act.size);
+                a1.touch((size_t)pt.seg * K * inter * 4, (size_t)K * inter * 4, "act of the layer");
+                const int rows = (int)nrb * rps_dn;
+                out.touch(((size_t)pt.seg * hidden + (size_t)rb_first * rps_dn) * 4, (size_t)rows * 4, "out rows");
+            }
+        }
+        if (bytes > max_bytes) max_bytes = bytes;
+        if (bytes < min_bytes) min_bytes = bytes;
+    }
+    for (int p = 0; p < n_pairs; p++) blob[p].expect_once(0, g.expert_size);
+    act.expect_once(0, act.size);
+    out.expect_once(0, out.size);
+    std::printf("ok  %-58s %d workgroups, <= %d segments, bytes per workgroup %zu..%zu\n", g_case.c_str(), G, max_seq,
+                min_bytes, max_bytes);
+}
+
+// the streaming phases with per-phase proportional shares: fm_gate_up_swiglu_lds / fm_down_lds as
+// separate launches (per_wave 2) and fm_moe_fused (both phases in one grid)
+static void walk_phases(int n_groups, int K, int hidden, int inter, int bits, bool fused) {
+    g_case = std::string(fused ? "fused (counters) " : "split phases ") + std::to_string(n_groups) + " groups x " +
+             std::to_string(K) + ", " + std::to_string(bits) + "-bit";
+    const Geom g = geom(hidden, inter, bits);
+    const int lpr_up = hidden / FM_CPL, lpr_dn = inter / FM_CPL, n_pairs = n_groups * K;
+    const int rps_up = FM_WAVE / lpr_up, rps_dn = FM_WAVE / lpr_dn;
+    const long gu_upp = inter / rps_up, dn_upp = hidden / rps_dn;
+    const long gu_total = (long)n_pairs * gu_upp, dn_total = (long)n_pairs * dn_upp;
+    const uint32_t gu_wstep = rps_up * (hidden * bits / 8), gu_sstep = rps_up * (hidden / 64) * 2;
+    const uint32_t dn_wstep = rps_dn * (inter * bits / 8), dn_sstep = rps_dn * (inter / 64) * 2;
+    std::vector<Region> blob;
+    blob.reserve(n_pairs);
+    for (int p = 0; p < n_pairs; p++) blob.emplace_back("expert blob", g.expert_size, 4);
+    Region act("act", (size_t)n_pairs * inter * 4, 4), eo("expert_out", (size_t)n_pairs * hidden * 4, 4);
+    for (int phase = 0; phase < 2; phase++) {
+        const bool up = phase == 0;
+        const long G = fused ? fm1_fused_wgs(gu_total, dn_total, N_CU) : fm_stream_wgs(up ? gu_total : dn_total, N_CU, 2);
+        for (long b = 0; b < G; b++) {
+            const Fm1Split sp = fm1_split(fused || up ? gu_total : 0, fused || !up ? dn_total : 0, gu_upp * K, dn_upp, (unsigned)b, (unsigned)G);
+            const int q0 = up ? 0 : sp.n_up, q1 = up ? sp.n_up : sp.n_up + sp.n_dn;
+            for (int q = q0; q < q1; q++) {
+                const int seg = fm1_seg(sp, q);
+                uint32_t first, n;
+                fm1_part(sp, q, up, &first, &n);
+                CHECK(seg >= 0 && seg < (up ? n_groups : n_pairs), "segment %d", seg);
+                for (uint32_t ul = 0; ul < n; ul++) {
+                    const uint32_t uq = first + ul;
+                    const uint32_t pn = up ? uq / (uint32_t)gu_upp : 0u, rsn = uq - pn * (uint32_t)gu_upp;
+                    CHECK(pn < (uint32_t)K && rsn < (uint32_t)(up ? gu_upp : dn_upp), "unit %u -> slot %u step %u", ul, pn, rsn);
+                    if (pn >= (uint32_t)K) continue;
+                    Region &bl = blob[up ? seg * K + pn : seg];
+                    if (up) {
+                        for (int second = 0; second < 2; second++)
+                            unit_dma(bl, (size_t)rsn * gu_wstep + (second ? g.up_w : g.gate_w), bl,
+                                     (size_t)rsn * gu_sstep + (second ? g.up_s : g.gate_s), bl,
+                                     (size_t)rsn * gu_sstep + (second ? g.up_b : g.gate_b), bits);
+                        for (int ris = 0; ris < rps_up; ris++)
+                            act.touch((((size_t)seg * gu_upp * K + first) * rps_up + ris + (size_t)ul * rps_up) * 4, 4, "act");
+                    } else {
+                        unit_dma(bl, (size_t)rsn * dn_wstep + g.down_w, bl, (size_t)rsn * dn_sstep + g.down_s, bl,
+                                 (size_t)rsn * dn_sstep + g.down_b, bits);
+                        for (int ris = 0; ris < rps_dn; ris++)
+                            eo.touch((((size_t)seg * dn_upp + first) * rps_dn + ris + (size_t)ul * rps_dn) * 4, 4, "expert_out");
+                    }
+                }
+            }
+        }
+    }
+    for (int p = 0; p < n_pairs; p++) blob[p].expect_once(0, g.expert_size);
+    act.expect_once(0, act.size);
+    eo.expect_once(0, eo.size);
+    std::printf("ok  %-58s\n", g_case.c_str());
+}
+
+// ----------------------------------------------------------------------------- GGUF streaming
+static void walk_gguf_stream(int n_groups, int K, int hidden, int inter, bool gu) {
+    const bool q6 = !gu;
+    g_case = std::string("gguf stream ") + (gu ? "gate/up Q4_K " : "down Q6_K ") + std::to_string(n_groups) + " groups x " + std::to_string(K);
+    const int n_pairs = n_groups * K, in_dim = gu ? hidden : inter, rows = gu ? inter : hidden;
+    const FmGgPlan pl = fm_gg_plan(n_pairs, K, in_dim, rows, q6, gu, N_CU);
+    if (!pl.ok) {
+        std::printf("--  %-58s not taken by the streaming kernel\n", g_case.c_str());
+        return;
+    }
+    const size_t slab = (size_t)rows * pl.row_bytes;       // one expert's rows of one matrix
+    CHECK((size_t)pl.upp * pl.slot_data == slab, "slices tile the expert");
+    const int ring = q6 ? 5 : 3, nreg = q6 ? 32 : 64;
+    const size_t img = (size_t)(nreg / 4) * 4 * pl.lpr * 16 + pl.lpr * 16;
+    const size_t lds = (size_t)8 * ring * (pl.slot_data + 16) + pl.n_img * img + pl.n_pair * 32 + 16;
+    CHECK(lds <= 160 * 1024, "LDS %zu", lds);
+    std::vector<Region> m0, m1;
+    for (int p = 0; p < n_pairs; p++) {
+        m0.emplace_back(gu ? "gate rows" : "down rows", slab, 2);
+        if (gu) m1.emplace_back("up rows", slab, 2);
+    }
+    Region outv(gu ? "act" : "expert_out", (size_t)n_pairs * rows * 4, 4);
+    const FmDiv by_upp = fm_div_make(pl.upp), by_k = fm_div_make(K);
+    for (int b = 0; b < pl.wgs; b++) {
+        const FmRange wg = fm_share(pl.total, b, pl.wgs);
+        if (wg.hi == wg.lo) continue;
+        const uint32_t pair0 = fm_div(by_upp, (uint32_t)wg.lo), pair_last = fm_div(by_upp, (uint32_t)wg.hi - 1u);
+        CHECK(pair0 == wg.lo / pl.upp && pair_last == (wg.hi - 1) / pl.upp, "division by multiply-shift");
+        CHECK(pair_last - pair0 < (uint32_t)pl.n_pair, "workgroup %d touches %u pairs", b, pair_last - pair0 + 1);
+        const uint32_t vid0 = gu ? fm_div(by_k, pair0) : pair0, vid1 = gu ? fm_div(by_k, pair_last) : pair_last;
+        CHECK(vid1 - vid0 < (uint32_t)pl.n_img, "workgroup %d needs %u images", b, vid1 - vid0 + 1);
+        for (long u = wg.lo; u < wg.hi; u++) {
+            const uint32_t pair = fm_div(by_upp, (uint32_t)u), step = (uint32_t)u - pair * by_upp.d;
+            CHECK(pair == u / pl.upp && pair < (uint32_t)n_pairs && step < (uint32_t)pl.upp, "unit %ld", u);
+            for (int kn = 0; kn < (gu ? 2 : 1); kn++) {
+                Region &r = kn ? m1[pair] : m0[pair];
+                for (int lane = 0; lane < 64; lane++)
+                    for (int i = 0; i * 1024 < pl.slot_data; i++)
+                        if (i * 1024 + lane * 16 < pl.slot_data) {
+                            // the last load of a slice may be partial in bytes as well: 16 bytes per
+                            // lane must still end inside the slice
+                            CHECK(i * 1024 + lane * 16 + 16 <= pl.slot_data, "load %d lane %d runs over the slice", i, lane);
+                            r.touch((size_t)step * pl.slot_data + (size_t)i * 1024 + (size_t)lane * 16, 16, "slice");
+                        }
+            }
+            for (int ris = 0; ris < pl.rps; ris++) outv.touch(((size_t)pair * rows + step * pl.rps + ris) * 4, 4, "result");
+        }
+    }
+    for (int p = 0; p < n_pairs; p++) {
+        m0[p].expect_once(0, slab);
+        if (gu) m1[p].expect_once(0, slab);
+    }
+    outv.expect_once(0, outv.size);
+    std::printf("ok  %-58s %ld units over %d workgroups\n", g_case.c_str(), pl.total, pl.wgs);
+}
+
+int main() {
+    // ---- the probes of bench.py --workload stream_probe (2 GiB) and of the decode profile (440 MB)
+    for (int pattern = 0; pattern < 3; pattern++) {
+        walk_probe((size_t)2 << 30, pattern);
+        walk_probe(440401920, pattern);
+        walk_probe(4096 * 3 + 100, pattern);
+    }
+    // ---- config 1 (bench.py --workload gdn): qkv + z in one launch, out_proj on its own
+    walk_dense_batch("gdn in_proj qkv+z 4-bit", {{8192, 4}, {4096, 4}}, 2048, 1, {});
+    walk_dense_batch("gdn in_proj qkv+z with riders b, a", {{8192, 4}, {4096, 4}}, 2048, 1, {32, 32});
+    walk_dense_batch("gdn out_proj 2048x4096 4-bit", {{2048, 4}}, 4096, 1, {});
+    walk_dense_batch("8192x4096 4-bit (two column slabs)", {{8192, 4}}, 4096, 1, {});
+    walk_dense_batch("lm_head 248320x2048 8-bit", {{248320, 8}}, 2048, 1, {});
+    walk_dense_batch("routing batch, mixed widths", {{256, 8}, {1, 8}, {512, 4}, {512, 4}}, 2048, 1, {});
+    walk_dense_batch("3-bit 12288x2048", {{12288, 3}}, 2048, 1, {});
+    walk_dense_batch("ragged 4-bit 1000x1024 x 3 positions", {{1000, 4}}, 1024, 3, {});
+    walk_dense_batch("qkv+z per position, 5 positions", {{8192, 4}, {4096, 4}}, 2048, 5, {});
+    // ---- config 1 against M positions (bench.py --workload gdn_prefill)
+    for (int M : {16, 100, 512, 513}) {
+        walk_pf_dense(8192, 2048, 4, M);
+        walk_pf_dense(4096, 2048, 4, M);
+        walk_pf_dense(2048, 4096, 4, M);
+        walk_pf_dense(2048, 512, 4, M);
+    }
+    walk_pf_dense(2048, 2048, 3, 512);
+    walk_pf_dense(512, 512, 3, 64);
+    // ---- routed experts: the decode step (config 2, and its 4-bit form), one layer per call
+    // (config 0), chunks below 32 positions (config 3 at chunk 8)
+    for (int bits : {3, 4}) {
+        walk_fused_rows(40, 8, 2048, 512, bits);
+        walk_fused_rows(1, 8, 2048, 512, bits);
+        walk_fused_rows(8, 8, 2048, 512, bits);
+        walk_fused_rows(31, 8, 2048, 512, bits);
+        walk_fused_rows(3, 5, 2048, 512, bits);
+        walk_fused_rows(40, 8, 1024, 256, bits);
+        walk_phases(40, 8, 2048, 512, bits, false);
+        walk_phases(40, 8, 2048, 512, bits, true);
+        walk_phases(1, 8, 2048, 512, bits, false);
+        walk_phases(1, 8, 2048, 512, bits, true);
+    }
+    walk_fused_rows(64, 8, 2048, 512, 3);
+    walk_fused_rows(300, 8, 2048, 512, 3);
+    // ---- config 4: GGUF step, one layer, chunk of 8 positions
+    for (int groups : {40, 1, 8}) {
+        walk_gguf_stream(groups, 8, 2048, 512, true);
+        walk_gguf_stream(groups, 8, 2048, 512, false);
+    }
+    if (g_fail) {
+        std::fprintf(stderr, "%d checks failed\n", g_fail);
+        return 1;
+    }
+    std::printf("all address ranges inside their buffers\n");
+    return 0;
+}
