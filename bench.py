@@ -990,7 +990,9 @@ def run_stream_probe(args):
     ctx = FinchHip(0)
     torch.cuda.synchronize()
     rates = {}
-    for pattern, name in ((1, "contiguous_share_per_workgroup"), (2, "contiguous_share_per_wave"), (0, "dense")):
+    for pattern, name in ((1, "contiguous_share_per_workgroup"), (2, "contiguous_share_per_wave"),
+                          (3, "groups_of_4_workgroups_interleaved"), (4, "groups_of_8_workgroups_interleaved"),
+                          (5, "groups_of_8_workgroups_of_one_xcd_interleaved"), (0, "dense")):
         def step(t, pattern=pattern):
             ctx.stream_probe_dev(bufs[t & 1].data_ptr(), n, pattern)
         ms, ev = _timed(ctx, step, args)

@@ -43,6 +43,10 @@ int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t *const *d_
                           int flags, int n_cu, hipStream_t st, hipEvent_t *kev);
 int fm_launch_gguf_matvec(const uint8_t *d_W, int ggml_type, const float *d_x, float *d_out,
                           int out_dim, int in_dim, int n_cu, hipStream_t st);
+int fm_launch_gguf_dense(const uint8_t *d_W, int ggml_type, const float *d_x, float *d_out, int out_dim,
+                         int in_dim, int n_cu, hipStream_t st);
+int fm_launch_embed_rows_gguf(const void *W, int rows, int in_dim, int ggml_type, const int32_t *d_ids,
+                              int n, float *d_out, hipStream_t st);
 int fm_launch_prefill_affine(const uint8_t *d_layer, const FmExpertGeom *g, const void *d_X,
                              int x_bf16, const int32_t *d_idx, const float *d_w, int M, int K,
                              float *d_out, void *d_ws, size_t ws_bytes, int flags, int n_cu,
@@ -86,11 +90,17 @@ int noalloc_lookup(int device, unsigned char **out) {
 // (cpu_dequant_matvec's scales == NULL branch, finchmoe/infer.m:1689-1701)
 constexpr int FM_BITS_RAW_BF16 = 16;
 
+// `bits` of a GGUF block-format tensor, the reference's own convention for cpu_dequant_matvec
+// and BatchMatvecSpec (finchmoe/infer.m:1684-1688): 10 = Q4_K, 11 = Q6_K
+constexpr int FM_BITS_GGUF_Q4K = 10, FM_BITS_GGUF_Q6K = 11;
+
 struct Tensor {
     bool used = false, owned = false;
     void *W = nullptr, *S = nullptr, *B = nullptr;
     int out_dim = 0, in_dim = 0, group_size = 0, bits = 0, scale_fp16 = 0;
     bool raw_bf16() const { return bits == FM_BITS_RAW_BF16; }
+    bool gguf() const { return bits == FM_BITS_GGUF_Q4K || bits == FM_BITS_GGUF_Q6K; }
+    int ggml_type() const { return bits == FM_BITS_GGUF_Q4K ? FM_GGML_Q4_K : FM_GGML_Q6_K; }
 };
 
 struct LayerBuf {
@@ -513,8 +523,8 @@ static int ktiming_collect(fm_ctx *c) {
 
 extern "C" int fm_stream_probe_dev(fm_ctx *c, const void *d_buf, size_t nbytes, int pattern) {
     if (!c) return FM_ERR_ARG;
-    if (!d_buf || nbytes < 4096 || ((uintptr_t)d_buf & 15) || pattern < 0 || pattern > 2)
-        return fail(c, FM_ERR_ARG, "stream probe: a 16-byte aligned buffer of 4 KB or more, pattern 0..2");
+    if (!d_buf || nbytes < 4096 || ((uintptr_t)d_buf & 15) || pattern < 0 || pattern > 5)
+        return fail(c, FM_ERR_ARG, "stream probe: a 16-byte aligned buffer of 4 KB or more, pattern 0..5");
     DeviceGuard dg(c->device);
     int rc = fm_launch_stream_probe(d_buf, nbytes, pattern, nullptr, c->n_cu, c->stream);
     if (rc) return fail(c, rc, "stream probe launch failed: %s", hipGetErrorString(hipGetLastError()));
@@ -851,10 +861,12 @@ static int tensor_add(fm_ctx *c, const void *W, const void *S, const void *B, in
     if (out_dim < 1 || in_dim < 1) return fail(c, FM_ERR_ARG, "non-positive dimension");
     // scales == NULL or biases == NULL: an unquantized BF16 weight, as in cpu_dequant_matvec
     // (finchmoe/infer.m:1689); `bits` and `group_size` say nothing about it then
-    const bool raw = !S || !B;
-    if (raw && (bits == 10 || bits == 11))
-        return fail(c, FM_ERR_ARG, "GGUF tensors (bits 10/11) go through fm_gguf_matvec");
-    if (!raw) {
+    // bits 10 / 11: a GGUF Q4_K / Q6_K tensor (block rows, no separate scales: S and B are ignored)
+    const bool gguf = bits == FM_BITS_GGUF_Q4K || bits == FM_BITS_GGUF_Q6K;
+    const bool raw = !gguf && (!S || !B);
+    if (gguf && (in_dim < 256 || in_dim % 256 || in_dim > 16384))
+        return fail(c, FM_ERR_UNSUPPORTED, "GGUF tensor in_dim %d: need a multiple of 256 up to 16384", in_dim);
+    if (!raw && !gguf) {
         if (bits == 0) bits = 4;   // BatchMatvecSpec default, finchmoe/infer.m:4491
         if (group_size != 64) return fail(c, FM_ERR_UNSUPPORTED, "group_size %d (only 64)", group_size);
         if (bits != 3 && bits != 4 && bits != 8)
@@ -872,19 +884,21 @@ static int tensor_add(fm_ctx *c, const void *W, const void *S, const void *B, in
     t.in_dim = in_dim;
     t.group_size = group_size;
     t.bits = raw ? FM_BITS_RAW_BF16 : bits;
-    t.scale_fp16 = !raw && scale_dtype == FM_SCALE_FP16;
-    size_t wb = (size_t)out_dim * in_dim * t.bits / 8, sb = (size_t)out_dim * (in_dim / 64) * 2;
+    t.scale_fp16 = !raw && !gguf && scale_dtype == FM_SCALE_FP16;
+    const bool plain = raw || gguf;        // W only
+    size_t wb = gguf ? (size_t)out_dim * gguf_row_bytes(in_dim, t.ggml_type()) : (size_t)out_dim * in_dim * t.bits / 8;
+    size_t sb = (size_t)out_dim * (in_dim / 64) * 2;
     if (adopt) {
-        if (((uintptr_t)W & (raw ? 1 : 15)) || (!raw && (((uintptr_t)S & 3) || ((uintptr_t)B & 3))))
+        if (((uintptr_t)W & (raw ? 1 : 15)) || (!plain && (((uintptr_t)S & 3) || ((uintptr_t)B & 3))))
             return fail(c, FM_ERR_ARG, "device tensor not aligned (W 16, S/B 4 bytes; raw BF16 2)");
         t.W = const_cast<void *>(W);
-        t.S = raw ? nullptr : const_cast<void *>(S);
-        t.B = raw ? nullptr : const_cast<void *>(B);
+        t.S = plain ? nullptr : const_cast<void *>(S);
+        t.B = plain ? nullptr : const_cast<void *>(B);
     } else {
         t.owned = true;
         HIPCHK(c, hipMalloc(&t.W, wb));
         HIPCHK(c, hipMemcpy(t.W, W, wb, hipMemcpyHostToDevice));
-        if (!raw) {
+        if (!plain) {
             HIPCHK(c, hipMalloc(&t.S, sb));
             HIPCHK(c, hipMalloc(&t.B, sb));
             HIPCHK(c, hipMemcpy(t.S, S, sb, hipMemcpyHostToDevice));
@@ -950,7 +964,7 @@ static int matvec_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
         Tensor *t0 = get_tensor(c, ts[0]);
         for (int k = 0; ok && k < n; k++) {
             Tensor *t = get_tensor(c, ts[k]);
-            ok = t && t0 && !t->raw_bf16() && t->in_dim == t0->in_dim && t->scale_fp16 == t0->scale_fp16 &&
+            ok = t && t0 && !t->raw_bf16() && !t->gguf() && t->in_dim == t0->in_dim && t->scale_fp16 == t0->scale_fp16 &&
                  t->group_size == 64 && d_outs[k] && (t->bits == 3 || t->bits == 4 || t->bits == 8);
             if (!ok) break;
             mixed = mixed || t->bits != t0->bits;
@@ -981,6 +995,18 @@ static int matvec_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
     while (i < n) {
         Tensor *t0 = get_tensor(c, ts[i]);
         if (!t0) return fail(c, FM_ERR_ARG, "bad tensor handle %d", ts[i]);
+        if (t0->gguf()) {
+            // a block-format tensor is a launch of its own (one per position)
+            if (!d_outs[i]) return fail(c, FM_ERR_ARG, "null output %d", i);
+            for (int pos = 0; pos < M; pos++) {
+                int rc = fm_launch_gguf_dense((const uint8_t *)t0->W, t0->ggml_type(), d_x + (size_t)pos * t0->in_dim,
+                                              d_outs[i] + (size_t)pos * t0->out_dim, t0->out_dim, t0->in_dim,
+                                              c->n_cu, c->stream);
+                if (rc) return fail(c, rc, "GGUF matvec launch failed: %s", hipGetErrorString(hipGetLastError()));
+            }
+            i++;
+            continue;
+        }
         FmDenseSpec specs[8];
         int m = 0;
         while (i < n && m < 8) {
@@ -1091,7 +1117,7 @@ extern "C" int fm_matvec_prefill_batch_dev(fm_ctx *c, const fm_tensor *ts, int n
         Tensor *p = get_tensor(c, ts[i]);
         if (!d_outs[i]) return fail(c, FM_ERR_ARG, "null output %d", i);
         size_t ws = 0;
-        if (!no_gemm && !p->raw_bf16() && M >= FM_DENSE_GEMM_MIN_M && ((uintptr_t)d_X & 15) == 0 && ((uintptr_t)d_outs[i] & 3) == 0)
+        if (!no_gemm && !p->raw_bf16() && !p->gguf() && M >= FM_DENSE_GEMM_MIN_M && ((uintptr_t)d_X & 15) == 0 && ((uintptr_t)d_outs[i] & 3) == 0)
             ws = fm_prefill_dense_ws_bytes(p->out_dim, p->in_dim, p->group_size, p->bits, M);
         if (ws) {
             DeviceGuard dg(c->device);
@@ -1218,7 +1244,7 @@ extern "C" int fm_layer_tail_dev(fm_ctx *c, fm_tensor shared_down, const float *
         return fail(c, FM_ERR_ARG, "next input and its norm weights go together");
     if (((uintptr_t)d_shared_gate | (uintptr_t)d_shared_up) & 3)
         return fail(c, FM_ERR_ARG, "vector not 4-byte aligned");
-    if (t->raw_bf16() || t->group_size != 64)
+    if (t->raw_bf16() || t->gguf() || t->group_size != 64)
         return fail(c, FM_ERR_UNSUPPORTED, "shared down projection must be 3/4/8-bit, group size 64");
     if (t->out_dim / 4 > FM_TAIL_PARTIALS) return fail(c, FM_ERR_UNSUPPORTED, "hidden %d", t->out_dim);
     DeviceGuard dg(c->device);
@@ -1532,6 +1558,11 @@ extern "C" int fm_dequant_tensor(fm_ctx *c, fm_tensor t, uint8_t *codes, float *
     if (!p) return fail(c, FM_ERR_ARG, "bad tensor handle %d", t);
     if (p->raw_bf16()) return fail(c, FM_ERR_UNSUPPORTED, "tensor %d is raw BF16: nothing to dequantize", t);
     DeviceGuard dg(c->device);
+    if (p->gguf()) {        // block formats have no integer codes or fp16 form here: fp32 values only
+        if (codes || w_f16) return fail(c, FM_ERR_UNSUPPORTED, "GGUF tensor %d: fp32 weights only", t);
+        return dequant_common(c, p->W, nullptr, nullptr, p->out_dim, p->in_dim, 0, 0, p->ggml_type(), nullptr,
+                              w_f32, nullptr);
+    }
     return dequant_common(c, p->W, p->S, p->B, p->out_dim, p->in_dim, p->bits, p->scale_fp16, 0,
                           codes, w_f32, w_f16);
 }
@@ -1549,6 +1580,12 @@ extern "C" int fm_embed_lookup_dev(fm_ctx *c, fm_tensor t, const int32_t *d_toke
     if (n_tokens < 1) return fail(c, FM_ERR_ARG, "n_tokens %d", n_tokens);
     if (p->raw_bf16()) return fail(c, FM_ERR_UNSUPPORTED, "embedding lookup needs a quantized tensor");
     DeviceGuard dg(c->device);
+    if (p->gguf()) {
+        int rc = fm_launch_embed_rows_gguf(p->W, p->out_dim, p->in_dim, p->ggml_type(), d_token_ids, n_tokens,
+                                           d_out, c->stream);
+        if (rc) return fail(c, rc, "embedding lookup launch failed: %s", hipGetErrorString(hipGetLastError()));
+        return FM_OK;
+    }
     int rc = fm_launch_embed_rows(p->W, p->S, p->B, p->out_dim, p->in_dim, p->group_size, p->bits,
                                   p->scale_fp16, d_token_ids, n_tokens, d_out, c->stream);
     if (rc) return fail(c, rc, "embedding lookup launch failed: %s", hipGetErrorString(hipGetLastError()));

@@ -78,36 +78,51 @@ __device__ __forceinline__ void scale_min_k4(int j, const uint8_t *s, int &sc, i
     }
 }
 
+// fp32 value of element `col` of a Q4_K / Q6_K row (finchmoe/infer.m:1604-1657)
+__device__ __forceinline__ float fm_gguf_elem(const uint8_t *row, int col, int ggml_type) {
+    const int bsz = ggml_type == FM_GGML_Q4_K ? 144 : 210;
+    const uint8_t *blk = row + (size_t)(col >> 8) * bsz;
+    const int e = col & 255;
+    if (ggml_type == FM_GGML_Q4_K) {
+        float d = fm_fp16_bits(blk[0] | (blk[1] << 8));
+        float dmin = fm_fp16_bits(blk[2] | (blk[3] << 8));
+        int chunk = e >> 6, high = (e >> 5) & 1, l = e & 31;
+        int sc, m;
+        scale_min_k4(2 * chunk + high, blk + 4, sc, m);
+        int nib = (blk[16 + 32 * chunk + l] >> (4 * high)) & 0xF;
+        float d1 = d * (float)sc, m1 = dmin * (float)m;
+        return d1 * (float)nib - m1;
+    }
+    float d = fm_fp16_bits(blk[208] | (blk[209] << 8));
+    int half = e >> 7, vi = e & 127;
+    int nib = (blk[64 * half + (vi & 63)] >> (4 * (vi >> 6))) & 0xF;
+    int hi2 = (blk[128 + 32 * half + (vi & 31)] >> (2 * ((vi >> 5) & 3))) & 3;
+    int sc = (int)(int8_t)blk[192 + 8 * half + (vi >> 4)];
+    int q = (nib | (hi2 << 4)) - 32;
+    return d * (float)sc * (float)q;
+}
+
 __global__ void fm_dequant_gguf_k(const uint8_t *W, int out_dim, int in_dim, int ggml_type,
                                   float *w32) {
     size_t n = (size_t)out_dim * in_dim;
-    const int bsz = ggml_type == FM_GGML_Q4_K ? 144 : 210;
+    const size_t row_bytes = (size_t)(in_dim / 256) * (ggml_type == FM_GGML_Q4_K ? 144 : 210);
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
          i += (size_t)gridDim.x * blockDim.x) {
         int r = (int)(i / in_dim), col = (int)(i % in_dim);
-        const uint8_t *blk = W + ((size_t)r * (in_dim / 256) + (col >> 8)) * bsz;
-        int e = col & 255;
-        float w;
-        if (ggml_type == FM_GGML_Q4_K) {
-            float d = fm_fp16_bits(blk[0] | (blk[1] << 8));
-            float dmin = fm_fp16_bits(blk[2] | (blk[3] << 8));
-            int chunk = e >> 6, high = (e >> 5) & 1, l = e & 31;
-            int sc, m;
-            scale_min_k4(2 * chunk + high, blk + 4, sc, m);
-            int nib = (blk[16 + 32 * chunk + l] >> (4 * high)) & 0xF;
-            float d1 = d * (float)sc, m1 = dmin * (float)m;
-            w = d1 * (float)nib - m1;
-        } else {
-            float d = fm_fp16_bits(blk[208] | (blk[209] << 8));
-            int half = e >> 7, vi = e & 127;
-            int nib = (blk[64 * half + (vi & 63)] >> (4 * (vi >> 6))) & 0xF;
-            int hi2 = (blk[128 + 32 * half + (vi & 31)] >> (2 * ((vi >> 5) & 3))) & 3;
-            int sc = (int)(int8_t)blk[192 + 8 * half + (vi >> 4)];
-            int q = (nib | (hi2 << 4)) - 32;
-            w = d * (float)sc * (float)q;
-        }
-        w32[i] = w;
+        w32[i] = fm_gguf_elem(W + (size_t)r * row_bytes, col, ggml_type);
     }
+}
+
+// Embedding lookup in a Q4_K / Q6_K tensor: out[i] = dequantized row ids[i], one workgroup per
+// id (embed_lookup's block-format branch, finchmoe/infer.m:5675-5683: gguf_dequant_row of the
+// token's row); an id outside the tensor gives zeros.
+__global__ __launch_bounds__(256) void fm_embed_rows_gguf_k(const uint8_t *W, int rows, int in_dim,
+                                                            int ggml_type, const int32_t *ids, float *out) {
+    const int r = ids[blockIdx.x];
+    const size_t row_bytes = (size_t)(in_dim / 256) * (ggml_type == FM_GGML_Q4_K ? 144 : 210);
+    float *o = out + (size_t)blockIdx.x * in_dim;
+    for (int col = threadIdx.x; col < in_dim; col += blockDim.x)
+        o[col] = (unsigned)r < (unsigned)rows ? fm_gguf_elem(W + (size_t)r * row_bytes, col, ggml_type) : 0.0f;
 }
 
 }  // namespace
@@ -141,5 +156,12 @@ extern "C" int fm_launch_dequant_gguf(const void *W, int out_dim, int in_dim, in
     if (blocks > 65535) blocks = 65535;
     hipLaunchKernelGGL(fm_dequant_gguf_k, dim3(blocks), dim3(256), 0, st, (const uint8_t *)W,
                        out_dim, in_dim, ggml_type, w32);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
+
+extern "C" int fm_launch_embed_rows_gguf(const void *W, int rows, int in_dim, int ggml_type,
+                                         const int32_t *d_ids, int n, float *d_out, hipStream_t st) {
+    hipLaunchKernelGGL(fm_embed_rows_gguf_k, dim3(n), dim3(256), 0, st, (const uint8_t *)W, rows, in_dim,
+                       ggml_type, d_ids, d_out);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }

@@ -47,6 +47,9 @@ struct GgufArgs {
     const float *w;
     float *act, *expert_out, *out;
     int rows_per_item, items_per_pair, flags;
+    // one dense tensor instead of an expert store (fm_launch_gguf_dense): its rows start here,
+    // there is one "pair", and the index and pointer tables are not read
+    const uint8_t *direct;
 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -405,6 +408,42 @@ __global__ __launch_bounds__(256) void fm_gguf_matvec_k(const uint8_t *W, const 
     if (lane == 0) out[row] = acc;
 }
 
+// The same product for rows of HPR <= 64 half blocks (in_dim = 128 * HPR, HPR a power of two): HPR
+// adjacent lanes share a row, a wave step covers 64 / HPR rows, and a lane keeps its 128
+// activations in registers over the `steps` row steps of its wave — every lane works whatever the
+// row length (a vocabulary projection of 2048 columns keeps a quarter of the lanes busy in the
+// kernel above).  Rows past out_dim are not loaded and not stored.
+template <bool Q6, int HPR>
+__global__ __launch_bounds__(256) void fm_gguf_matvec_rows_k(const uint8_t *W, const float *x, float *out,
+                                                             int out_dim, int steps) {
+    constexpr int RPW = FM_WAVE / HPR;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int hb = lane % HPR, rr = lane / HPR;
+    const size_t row_bytes = (size_t)(HPR / 2) * (Q6 ? 210 : 144);
+    float xs[128], xsum[8];
+    if constexpr (Q6) q6_load_x(x + hb * 128, xs, xsum);
+    else q4_load_x(x + hb * 128, xs, xsum);
+    const long row0 = ((long)blockIdx.x * 4 + wave) * RPW * steps;
+    for (int s = 0; s < steps; s++) {
+        const long row = row0 + (long)s * RPW + rr;
+        float acc = 0.0f;
+        if (row < out_dim) {
+            const uint8_t *blk = W + (size_t)row * row_bytes + (size_t)(hb >> 1) * (Q6 ? 210 : 144);
+            if constexpr (Q6) {
+                Q6Half t;
+                q6_load(t, blk, hb & 1);
+                acc = q6_half_dot(t, xs, xsum);
+            } else {
+                Q4Half t;
+                q4_load(t, blk, hb & 1);
+                acc = q4_half_dot(t, hb & 1, xs, xsum);
+            }
+        }
+        acc = fm_group_sum<HPR>(acc);
+        if (hb == 0 && row < out_dim) out[row] = acc;
+    }
+}
+
 // ---------------------------------------------------------------- streaming kernels
 // The large launches take the form of the affine decode kernels: one workgroup of
 // eight waves per CU, each wave keeps a ring of slices in LDS filled by LDS-direct
@@ -742,12 +781,16 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
     if (threadIdx.x == 0) next_unit = 0u;
     if (threadIdx.x <= pair_last - pair0 && threadIdx.x < NPAIR) {
         const uint32_t pair = pair0 + threadIdx.x;
-        int e = a.idx[pair];
+        const bool direct = !GU && a.direct != nullptr;
+        int e = direct ? 0 : a.idx[pair];
         const bool ok = (unsigned)e < (unsigned)a.g.n_experts;
         if (!ok) e = 0;                                  // stream something valid, store zeros
         const int li = a.layer0 + (int)by_k(pair) * a.layer_stride;
         GgPairEntry pe;
-        if constexpr (GU) {
+        if (direct) {
+            pe.first = (uint64_t)(uintptr_t)a.direct;
+            pe.second = 0;
+        } else if constexpr (GU) {
             const uint8_t *g = a.gate[li] + (size_t)e * a.g.gate_slab;
             pe.first = (uint64_t)(uintptr_t)g;
             pe.second = (int64_t)((a.up[li] + (size_t)e * a.g.up_slab) - g);
@@ -906,6 +949,7 @@ extern "C" int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t
                                      float *d_expert_out, float *d_out, unsigned int *, int flags,
                                      int n_cu, hipStream_t st, hipEvent_t *kev) {
     GgufArgs a;
+    a.direct = nullptr;
     a.gate = d_gate;
     a.up = d_up;
     a.down = d_down;
@@ -978,10 +1022,59 @@ extern "C" int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t
 
 extern "C" int fm_launch_gguf_matvec(const uint8_t *d_W, int ggml_type, const float *d_x,
                                      float *d_out, int out_dim, int in_dim, int, hipStream_t st) {
+    const bool q6 = ggml_type == FM_GGML_Q6_K;
+    const int hpr = in_dim / 128;
+    // rows of up to 64 half blocks: 64 / hpr rows per wave step, a few steps per wave
+    if (in_dim % 256 == 0 && hpr >= 2 && hpr <= 64 && (hpr & (hpr - 1)) == 0 && ((uintptr_t)d_x & 15) == 0) {
+        const int rpw = FM_WAVE / hpr;
+        int steps = 1;
+        while (steps < 8 && (long)out_dim > 4L * rpw * steps * 2048) steps *= 2;
+        const dim3 grid((unsigned)((out_dim + 4 * rpw * steps - 1) / (4 * rpw * steps))), b(256);
+#define GG_MV(H)                                                                                          \
+    do {                                                                                                  \
+        if (q6) hipLaunchKernelGGL((fm_gguf_matvec_rows_k<true, H>), grid, b, 0, st, d_W, d_x, d_out, out_dim, steps);  \
+        else hipLaunchKernelGGL((fm_gguf_matvec_rows_k<false, H>), grid, b, 0, st, d_W, d_x, d_out, out_dim, steps);    \
+    } while (0)
+        switch (hpr) {
+            case 2: GG_MV(2); break;
+            case 4: GG_MV(4); break;
+            case 8: GG_MV(8); break;
+            case 16: GG_MV(16); break;
+            case 32: GG_MV(32); break;
+            default: GG_MV(64); break;
+        }
+#undef GG_MV
+        return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+    }
     dim3 grid((out_dim + 3) / 4), b(256);
-    if (ggml_type == FM_GGML_Q6_K)
-        hipLaunchKernelGGL(fm_gguf_matvec_k<true>, grid, b, 0, st, d_W, d_x, d_out, out_dim, in_dim);
-    else
-        hipLaunchKernelGGL(fm_gguf_matvec_k<false>, grid, b, 0, st, d_W, d_x, d_out, out_dim, in_dim);
+    if (q6) hipLaunchKernelGGL(fm_gguf_matvec_k<true>, grid, b, 0, st, d_W, d_x, d_out, out_dim, in_dim);
+    else hipLaunchKernelGGL(fm_gguf_matvec_k<false>, grid, b, 0, st, d_W, d_x, d_out, out_dim, in_dim);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
+
+// One dense Q4_K / Q6_K tensor [out_dim][in_dim] times x (the vocabulary projection and the
+// other block-format tensors of a GGUF model: lm_head_forward's block branch,
+// finchmoe/infer.m:5738-5746; cpu_dequant_matvec with bits 10 / 11, finchmoe/infer.m:1684-1688).
+// Shapes the streaming kernel covers (a lane per 128 Q4_K / 64 Q6_K values, 4 to 16 lanes per
+// row, rows a multiple of the wave step, 16-byte aligned rows) take it — the tensor is its one
+// "expert" —, the others the plain kernel.
+extern "C" int fm_launch_gguf_dense(const uint8_t *d_W, int ggml_type, const float *d_x, float *d_out,
+                                    int out_dim, int in_dim, int n_cu, hipStream_t st) {
+    if (ggml_type != FM_GGML_Q4_K && ggml_type != FM_GGML_Q6_K) return FM_ERR_UNSUPPORTED;
+    if (out_dim < 1 || in_dim < 256 || in_dim % 256) return FM_ERR_UNSUPPORTED;
+    static const bool no_stream = getenv("FINCH_GGUF_VALU") != nullptr;
+    const bool q6 = ggml_type == FM_GGML_Q6_K;
+    if (!no_stream && ((uintptr_t)d_W & 15) == 0) {
+        GgufArgs a{};
+        a.g.hidden = out_dim;          // the down phase's names: rows = hidden, columns = inter
+        a.g.inter = in_dim;
+        a.g.n_experts = 1;
+        a.K = 1;
+        a.act = const_cast<float *>(d_x);
+        a.expert_out = d_out;
+        a.direct = d_W;
+        const int rc = q6 ? gg_launch_stream<GG_Q6, false>(a, 1, n_cu, st) : gg_launch_stream<GG_Q4, false>(a, 1, n_cu, st);
+        if (rc != FM_ERR_UNSUPPORTED) return rc;
+    }
+    return fm_launch_gguf_matvec(d_W, ggml_type, d_x, d_out, out_dim, in_dim, n_cu, st);
 }

@@ -91,8 +91,25 @@ FM_HD FmProbeWalk fm_probe_walk(int pattern, size_t n_slots, unsigned int b, uns
         w.next = gw, w.end = n_slots, w.step = nw;
     } else if (pattern == 1) {
         w.next = n_slots * b / G + wave, w.end = n_slots * (b + 1) / G, w.step = (size_t)waves_per_wg;
-    } else {
+    } else if (pattern == 2) {
         w.next = n_slots * gw / nw, w.end = n_slots * (gw + 1) / nw, w.step = 1;
+    } else {
+        // groups of `gs` workgroups share a contiguous region, its slots dealt out to the group's
+        // waves in turn (3: four consecutive workgroups, 4: eight consecutive workgroups — they sit
+        // on different XCDs —, 5: eight workgroups of one XCD, b % 8 equal)
+        const unsigned int gs = pattern == 3 ? 4u : 8u;
+        unsigned int grp, member;
+        if (pattern == 5 && G % 64u == 0u) {
+            const unsigned int xcd = b % 8u, k = b / 8u;        // k-th workgroup of its XCD
+            grp = xcd * (G / 64u) + k / 8u, member = k % 8u;
+        } else {
+            grp = b / gs, member = b % gs;
+        }
+        const unsigned int n_grp = (G + gs - 1u) / gs;
+        const unsigned int members = grp + 1u < n_grp || G % gs == 0u ? gs : G % gs;
+        w.next = n_slots * grp / n_grp + (size_t)member * waves_per_wg + wave;
+        w.end = n_slots * (grp + 1u) / n_grp;
+        w.step = (size_t)members * waves_per_wg;
     }
     return w;
 }

@@ -23,6 +23,8 @@ extern __shared__ __attribute__((aligned(16))) uint8_t fm_probe_lds[];
 //   1  every workgroup a contiguous share, its eight waves interleaved over it (the order of
 //      the expert decode kernels)
 //   2  every wave a contiguous share
+//   3, 4, 5  groups of 4 / 8 / 8 workgroups share a contiguous region whose slots go to the
+//      group's waves in turn (5: the eight workgroups of a group sit on one XCD)
 template <int PATTERN>
 __global__ __launch_bounds__(PROBE_WAVES * 64) void fm_stream_probe_k(const uint8_t *buf, size_t n_slots,
                                                                       unsigned int *sink) {
@@ -70,16 +72,15 @@ __global__ __launch_bounds__(PROBE_WAVES * 64) void fm_stream_probe_k(const uint
 extern "C" int fm_launch_stream_probe(const void *d_buf, size_t nbytes, int pattern, unsigned int *d_sink,
                                       int n_cu, hipStream_t st) {
     const size_t n_slots = nbytes / PROBE_SLOT;
-    if (!d_buf || n_slots == 0 || ((uintptr_t)d_buf & 15) || pattern < 0 || pattern > 2) return FM_ERR_ARG;
+    if (!d_buf || n_slots == 0 || ((uintptr_t)d_buf & 15) || pattern < 0 || pattern > 5) return FM_ERR_ARG;
     const size_t sh = (size_t)PROBE_WAVES * PROBE_RING * PROBE_SLOT;
-    static FmLdsAttr attr[3];
-    const void *fn = pattern == 0 ? (const void *)fm_stream_probe_k<0>
-                   : pattern == 1 ? (const void *)fm_stream_probe_k<1> : (const void *)fm_stream_probe_k<2>;
-    if (!fm_dyn_lds_ready(attr[pattern], fn, sh)) return FM_ERR_HIP;
+    static FmLdsAttr attr[6];
+    typedef void (*probe_fn)(const uint8_t *, size_t, unsigned int *);
+    static const probe_fn fns[6] = {fm_stream_probe_k<0>, fm_stream_probe_k<1>, fm_stream_probe_k<2>,
+                                    fm_stream_probe_k<3>, fm_stream_probe_k<4>, fm_stream_probe_k<5>};
+    if (!fm_dyn_lds_ready(attr[pattern], (const void *)fns[pattern], sh)) return FM_ERR_HIP;
     const dim3 grid(n_cu), block(PROBE_WAVES * 64);
     const uint8_t *b = (const uint8_t *)d_buf;
-    if (pattern == 0) hipLaunchKernelGGL(fm_stream_probe_k<0>, grid, block, sh, st, b, n_slots, d_sink);
-    else if (pattern == 1) hipLaunchKernelGGL(fm_stream_probe_k<1>, grid, block, sh, st, b, n_slots, d_sink);
-    else hipLaunchKernelGGL(fm_stream_probe_k<2>, grid, block, sh, st, b, n_slots, d_sink);
+    hipLaunchKernelGGL(fns[pattern], grid, block, sh, st, b, n_slots, d_sink);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }

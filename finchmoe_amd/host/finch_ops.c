@@ -76,9 +76,11 @@ static slot *tab_find(const void *key, int insert) {
 
 static int resident(const void *W, const void *S, const void *B, int out_dim, int in_dim,
                     int group_size, int bits, fm_tensor *t) {
-    /* scales == NULL: an unquantized BF16 tensor (infer.m:1689); otherwise bits 0 means 4
-     * (infer.m:4491).  Normalised here so that the table compares like with like. */
-    if (!S || !B) { S = B = NULL; bits = 16; }
+    /* bits 10 / 11: a GGUF Q4_K / Q6_K tensor, which carries no scales (infer.m:1684-1688,
+     * 3378-3388); scales == NULL otherwise: an unquantized BF16 tensor (infer.m:1689); bits 0
+     * means 4 (infer.m:4491).  Normalised here so that the table compares like with like. */
+    if (bits == 10 || bits == 11) S = B = NULL;
+    else if (!S || !B) { S = B = NULL; bits = 16; }
     else if (bits == 0) bits = 4;
     if (!W) return FM_ERR_ARG;
     slot *s = tab_find(W, 1);
@@ -145,18 +147,13 @@ void fast_dequant_matvec(const uint32_t *W, const uint16_t *scales, const uint16
                          const float *x, float *out, int out_dim, int in_dim, int group_size,
                          int bits) {
     if (!g_ctx) { fail(FM_ERR_STATE, "fast_dequant_matvec"); return; }
-    int rc;
-    if ((!scales || !biases) && (bits == 10 || bits == 11)) {
-        /* GGUF tensors carry no scales (infer.m:3378-3388) */
-        rc = fm_gguf_matvec(g_ctx, W, bits == 10 ? FM_GGML_Q4_K : FM_GGML_Q6_K, x, out, out_dim, in_dim);
-    } else {
-        /* quantized, or scales == NULL: raw BF16 [out_dim][in_dim] (infer.m:1689-1701) */
-        fm_tensor t;
-        rc = resident(W, scales, biases, out_dim, in_dim, group_size, bits, &t);
-        if (!rc) {
-            float *outs[1] = {out};
-            rc = fm_matvec_batch(g_ctx, &t, 1, x, outs);
-        }
+    /* quantized; bits 10 / 11: GGUF block rows (infer.m:3378-3388); scales == NULL otherwise: raw
+     * BF16 [out_dim][in_dim] (infer.m:1689-1701).  The tensor stays resident after its first use. */
+    fm_tensor t;
+    int rc = resident(W, scales, biases, out_dim, in_dim, group_size, bits, &t);
+    if (!rc) {
+        float *outs[1] = {out};
+        rc = fm_matvec_batch(g_ctx, &t, 1, x, outs);
     }
     if (rc) {
         /* the reference's call sites take a void result: never leave `out` uninitialised */
@@ -183,11 +180,6 @@ void fast_batch_matvec(const float *x, uint32_t x_dim, BatchMatvecSpec *specs, i
         if (specs[i].in_dim != x_dim) {
             rc = FM_ERR_ARG;
             what = "fast_batch_matvec (in_dim != x_dim)";
-        } else if ((!specs[i].scales || !specs[i].biases) && (specs[i].bits == 10 || specs[i].bits == 11)) {
-            /* a GGUF spec has no batched kernel: the reference keeps such batches on its CPU
-             * path too (infer.m:4481-4483); issue it as a single fast_dequant_matvec */
-            rc = FM_ERR_UNSUPPORTED;
-            what = "fast_batch_matvec (GGUF spec: use fast_dequant_matvec)";
         } else {
             rc = resident(specs[i].W, specs[i].scales, specs[i].biases, (int)specs[i].out_dim,
                           (int)specs[i].in_dim, (int)specs[i].group_size, specs[i].bits, &ts[i]);

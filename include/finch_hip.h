@@ -195,7 +195,13 @@ FM_API int fm_moe_prefill_bf16(fm_ctx *ctx, int layer, const uint16_t *X, const 
  * gpu_encode_prefill_matvec (finchmoe/infer.m:3369, 3401-3411, 4477, 3672;
  * kernels dequant_matvec_4bit_v3 and _prefill, shaders.metal:374-463, 2460-2529).
  * W: u32 [out_dim][in_dim*bits/32] (bits 4 or 8) or bytes [out_dim][in_dim*3/8]
- * (bits 3); S, B: 16-bit [out_dim][in_dim/group_size]. */
+ * (bits 3); S, B: 16-bit [out_dim][in_dim/group_size].
+ * S == NULL or B == NULL: an unquantized BF16 tensor [out_dim][in_dim] (cpu_dequant_matvec's
+ * raw branch, finchmoe/infer.m:1689-1701).
+ * bits 10 / 11 (the reference's own codes, finchmoe/infer.m:1684-1688, 3378-3388): a GGUF Q4_K /
+ * Q6_K tensor, rows of in_dim/256 blocks of 144 / 210 bytes, S and B ignored — the vocabulary
+ * projection and embedding of a GGUF model (lm_head_forward and embed_lookup,
+ * finchmoe/infer.m:5738-5746, 5675-5683).  in_dim a multiple of 256. */
 typedef int fm_tensor;   /* handle >= 0 */
 FM_API int fm_tensor_register(fm_ctx *ctx, const void *W, const void *S, const void *B,
                        int out_dim, int in_dim, int group_size, int bits,
@@ -303,9 +309,11 @@ FM_API int fm_gguf_matvec(fm_ctx *ctx, const void *W, int ggml_type, const float
                    int out_dim, int in_dim);
 
 /* ---------------------------------------------------------------- embedding lookup
- * embed_lookup(wf, token_id, out) (finchmoe/infer.m:5664-5722, the 4-/8-bit branch): row
- * token_id of a registered affine tensor [vocab][hidden], dequantized to fp32 —
- * out[j] = (float)code * scale + bias, the same value fm_dequant_tensor gives for that row.
+ * embed_lookup(wf, token_id, out) (finchmoe/infer.m:5664-5722): row token_id of a registered
+ * tensor [vocab][hidden], dequantized to fp32.  Affine tensors (the 4-/8-bit branch):
+ * out[j] = (float)code * scale + bias; GGUF tensors registered with bits 10 / 11 (the
+ * block-format branch, finchmoe/infer.m:5675-5683): gguf_dequant_row of the token's row.  Either
+ * way the same value fm_dequant_tensor gives for that row.
  * The _dev form takes n ids from device memory (one row each, out [n][in_dim], asynchronous
  * on the context's stream); an id outside the tensor gives a row of zeros. */
 FM_API int fm_embed_lookup_dev(fm_ctx *ctx, fm_tensor t, const int32_t *d_token_ids, int n_tokens,

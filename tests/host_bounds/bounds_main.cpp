@@ -515,9 +515,11 @@ static void walk_phases(int n_groups, int K, int hidden, int inter, int bits, bo
 }
 
 // ----------------------------------------------------------------------------- GGUF streaming
-static void walk_gguf_stream(int n_groups, int K, int hidden, int inter, bool gu) {
-    const bool q6 = !gu;
-    g_case = std::string("gguf stream ") + (gu ? "gate/up Q4_K " : "down Q6_K ") + std::to_string(n_groups) + " groups x " + std::to_string(K);
+static void walk_gguf_stream(int n_groups, int K, int hidden, int inter, bool gu, int down_q6 = 1,
+                             const char *label = nullptr) {
+    const bool q6 = !gu && down_q6;
+    g_case = label ? std::string("gguf dense ") + label
+                   : std::string("gguf stream ") + (gu ? "gate/up Q4_K " : "down Q6_K ") + std::to_string(n_groups) + " groups x " + std::to_string(K);
     const int n_pairs = n_groups * K, in_dim = gu ? hidden : inter, rows = gu ? inter : hidden;
     const FmGgPlan pl = fm_gg_plan(n_pairs, K, in_dim, rows, q6, gu, N_CU);
     if (!pl.ok) {
@@ -572,7 +574,7 @@ static void walk_gguf_stream(int n_groups, int K, int hidden, int inter, bool gu
 
 int main() {
     // ---- the probes of bench.py --workload stream_probe (2 GiB) and of the decode profile (440 MB)
-    for (int pattern = 0; pattern < 3; pattern++) {
+    for (int pattern = 0; pattern < 6; pattern++) {
         walk_probe((size_t)2 << 30, pattern);
         walk_probe(440401920, pattern);
         walk_probe(4096 * 3 + 100, pattern);
@@ -617,6 +619,13 @@ int main() {
         walk_gguf_stream(groups, 8, 2048, 512, true);
         walk_gguf_stream(groups, 8, 2048, 512, false);
     }
+    // ---- one dense GGUF tensor as the streaming kernel's single "expert" (rows = hidden, columns =
+    // inter in the down phase's names): the vocabulary projection at Q4_K, and smaller shapes
+    walk_gguf_stream(1, 1, 248320, 2048, false, 0, "Q4_K 248320x2048");
+    walk_gguf_stream(1, 1, 248320, 1024, false, 1, "Q6_K 248320x1024");
+    walk_gguf_stream(1, 1, 4096, 2048, false, 0, "Q4_K 4096x2048");
+    walk_gguf_stream(1, 1, 4096, 1024, false, 1, "Q6_K 4096x1024");
+    walk_gguf_stream(1, 1, 1024, 2048, false, 1, "Q6_K 1024x2048 (rows-per-wave kernel)");
     if (g_fail) {
         std::fprintf(stderr, "%d checks failed\n", g_fail);
         return 1;

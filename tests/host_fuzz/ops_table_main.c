@@ -26,7 +26,7 @@ int fm_tensor_register(fm_ctx *c, const void *W, const void *S, const void *B, i
     (void)c; (void)S; (void)B; (void)group_size; (void)scale_dtype;
     if (!W || out_dim < 1 || in_dim < 1) return FM_ERR_ARG;
     if ((S == NULL) != (B == NULL)) { bad++; return FM_ERR_ARG; }     /* the wrapper normalises this */
-    if (!S && bits != 16) { bad++; return FM_ERR_ARG; }
+    if (!S && bits != 16 && bits != 10 && bits != 11) { bad++; return FM_ERR_ARG; }   /* raw BF16 or GGUF */
     if (fail_register_after >= 0 && n_reg >= fail_register_after) return FM_ERR_NOMEM;
     if (n_reg >= MAXT) return FM_ERR_NOMEM;
     live[n_reg] = 1;
@@ -120,16 +120,22 @@ int main(void) {
     fast_batch_matvec(x, 64, sp, 3);
     CHECK(finch_ops_last_status() == FM_ERR_ARG && n_batch == batches && out[0] == 0.0f && out[64] == 0.0f && out[128] == 0.0f);
     sp[1].in_dim = 64;
-    sp[2].scales = NULL; sp[2].bits = 10;                   /* a GGUF spec inside a batch */
+    sp[2].scales = NULL; sp[2].bits = 10;                   /* a GGUF spec inside a batch: a resident tensor like the others */
+    out[128] = 9.0f;
     fast_batch_matvec(x, 64, sp, 3);
-    CHECK(finch_ops_last_status() == FM_ERR_UNSUPPORTED && n_batch == batches);
+    CHECK(finch_ops_last_status() == FM_OK && n_batch == batches + 1 && out[128] == 1.0f);
     fast_batch_matvec(x, 64, sp, 0);
     CHECK(finch_ops_last_status() == FM_ERR_ARG);
     fast_batch_matvec(x, 64, sp, 65);
     CHECK(finch_ops_last_status() == FM_ERR_ARG);
-    /* a GGUF tensor on its own goes to the GGUF matvec */
-    fast_dequant_matvec(&arena[60200], NULL, NULL, x, out, 4, 256, 64, 11);
-    CHECK(finch_ops_last_status() == FM_OK && out[0] == 2.0f);
+    /* a GGUF tensor on its own is registered once (bits 11, no scales) and stays resident */
+    {
+        const int regs = n_reg;
+        fast_dequant_matvec(&arena[60200], NULL, NULL, x, out, 4, 256, 64, 11);
+        CHECK(finch_ops_last_status() == FM_OK && out[0] == 1.0f && n_reg == regs + 1);
+        fast_dequant_matvec(&arena[60200], NULL, NULL, x, out, 4, 256, 64, 11);
+        CHECK(finch_ops_last_status() == FM_OK && n_reg == regs + 1);
+    }
     /* registration failing inside the library: an error, zeros, the slot stays usable */
     fail_register_after = n_reg;
     out[0] = 9.0f;

@@ -105,6 +105,82 @@ def test_full_chunk_equals_positions(full_store, orc):
     assert_parity(out[m], ref, "position %d" % m)
 
 
+def test_full_chunk_bf16_entry_equals_positions(full_store, orc):
+    """The same 512-position chunk handed over as bf16 bits (fm_moe_prefill_bf16: 16 positions per
+    gate/up item, one matrix-core operand per value — the entry bench.py's prefill workload
+    times): equal to the fp32 entry on the widened values within the bar, to per-position calls,
+    and to the oracle on one position; a repeat is bit-identical."""
+    import torch
+    from bench import zipf_routing
+    ctx, blob, lo, _, _ = full_store
+    M, layer = 512, 5
+    rng = np.random.default_rng(18)
+    idx, w = zipf_routing(rng, M, 1, E, K)
+    idx, w = np.ascontiguousarray(idx[:, 0]), np.ascontiguousarray(w[:, 0])
+    Xb = torch.randn(M, H).to(torch.bfloat16)
+    X = Xb.to(torch.float32).numpy()
+    bits = Xb.view(torch.int16).numpy().view(np.uint16)
+    out = ctx.moe_prefill_bf16(layer, bits, idx, w)
+    assert np.isfinite(out).all()
+    assert np.array_equal(ctx.moe_prefill_bf16(layer, bits, idx, w), out)
+    wide = ctx.moe_prefill(layer, X, idx, w)
+    for m in list(range(0, M, 29)) + [M - 1]:
+        assert rel_err(out[m], wide[m]) < 1e-3 and cosine(out[m], wide[m]) > 0.99999, m
+        single, _ = ctx.moe_decode(layer, X[m], idx[m], w[m])
+        assert rel_err(out[m], single) < 1e-3 and cosine(out[m], single) > 0.99999, m
+    m = 77
+    mini = np.concatenate([blob[layer, int(e)].cpu().numpy() for e in idx[m]])
+    ref, _ = orc.moe_experts_forward(mini, X[m], np.arange(K, dtype=np.int32), w[m], H, I, 3, nthreads=8)
+    assert_parity(out[m], ref, "position %d" % m)
+
+
+def test_lm_head_8bit_full_size(orc):
+    """The 8-bit vocabulary projection at its real size, 248320 x 2048 (the streaming kernel of
+    bench.py's lm_head workload): a few thousand sampled rows against the oracle, all outputs
+    finite, and embedding rows bit for bit."""
+    import torch
+    from finchmoe_amd import FinchHip
+    V, D = 248320, 2048
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(11)
+    W = torch.empty(V * D, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
+    s = torch.randn(V * (D // 64), device=dev, generator=gen).abs_() * (0.02 / 127.5)
+    S = (s.view(torch.int32) >> 16).to(torch.int16)
+    B = ((s * -127.5).view(torch.int32) >> 16).to(torch.int16)
+    x = torch.randn(D, device=dev, generator=gen)
+    out = torch.empty(V, device=dev)
+    torch.cuda.synchronize()
+    ctx = FinchHip(0)
+    try:
+        t = ctx.tensor_adopt(W.data_ptr(), S.data_ptr(), B.data_ptr(), V, D, 8)
+        ctx.matvec_batch_dev([t], x.data_ptr(), [out.data_ptr()])
+        ctx.sync()
+        got = out.cpu().numpy()
+        assert np.isfinite(got).all()
+        rng = np.random.default_rng(6)
+        rows = np.unique(np.concatenate([rng.integers(0, V, 3000), [0, 1, 2, 3, V - 4, V - 3, V - 2, V - 1]]))
+        sel = torch.from_numpy(rows).to(dev)
+        Wh = W.view(V, D)[sel].cpu().numpy()
+        Sh = S.view(V, D // 64)[sel].cpu().numpy().view(np.uint16)
+        Bh = B.view(V, D // 64)[sel].cpu().numpy().view(np.uint16)
+        ref = orc.dequant_matvec(Wh.reshape(-1), Sh.reshape(-1), Bh.reshape(-1), x.cpu().numpy(), len(rows), D, 8)
+        assert_parity(got[rows], ref, "sampled rows of the 8-bit vocabulary projection")
+        ids = torch.tensor([5, V - 1], dtype=torch.int32, device=dev)
+        emb = torch.empty(2, D, device=dev)
+        ctx.embed_lookup_dev(t, ids.data_ptr(), 2, emb.data_ptr())
+        ctx.sync()
+        for i, tok in enumerate((5, V - 1)):
+            k = int(np.searchsorted(rows, tok)) if tok in rows else None
+            Wr = W.view(V, D)[tok].cpu().numpy()
+            Sr = S.view(V, D // 64)[tok].cpu().numpy().view(np.uint16)
+            Br = B.view(V, D // 64)[tok].cpu().numpy().view(np.uint16)
+            _, w32 = orc.dequant_affine(Wr, Sr, Br, 1, D, 8)
+            assert np.array_equal(emb[i].cpu().numpy().view(np.uint32), w32[0].view(np.uint32)), (tok, k)
+    finally:
+        ctx.close()
+
+
 def test_full_chunk_4bit_equals_positions(orc):
     """The same 512-position chunk on one layer of 256 4-bit experts (453 MB): the grouped
     product against per-position calls, and one position against the oracle."""

@@ -203,3 +203,81 @@ def test_gguf_chunk_grouped_products(orc, M, K, h, i, seed):
         assert rel_err(acc, base + out) < 1e-6
     finally:
         ctx.close()
+
+
+@pytest.mark.parametrize("gtype,out_dim,in_dim", [(12, 4096, 2048), (14, 4096, 1024), (14, 1024, 2048),
+                                                  (12, 515, 512), (14, 100, 256), (12, 64, 4096)])
+def test_gguf_dense_tensor_resident_matvec_and_embedding(hip, orc, gtype, out_dim, in_dim):
+    """A Q4_K / Q6_K tensor registered with the reference's bits 10 / 11: fp32 values and the
+    embedding rows bit for bit the oracle's gguf_dequant_row, the matvec within the bar (the
+    streaming kernel where the shape allows it, the rows-per-wave kernel otherwise), also for
+    several positions."""
+    rng = np.random.default_rng(3 * out_dim + in_dim + gtype)
+    W = F.synth_gguf_tensor(rng, out_dim, in_dim, gtype)
+    bits = 10 if gtype == 12 else 11
+    t = hip.tensor_register(W, None, None, out_dim, in_dim, bits=bits)
+    try:
+        ref_w = orc.gguf_dequant(W, out_dim, in_dim, gtype)
+        if out_dim * in_dim <= 1 << 22:
+            w32 = np.empty((out_dim, in_dim), np.float32)
+            hip._chk(hip.L.fm_dequant_tensor(hip.h, t, None, w32.ctypes.data, None))
+            assert np.array_equal(w32.view(np.uint32), ref_w.view(np.uint32))
+        for tok in (0, out_dim - 1, out_dim // 3):
+            row = hip.embed_lookup(t, tok, in_dim)
+            assert np.array_equal(row.view(np.uint32), ref_w[tok].view(np.uint32))
+        assert not hip.embed_lookup(t, out_dim, in_dim).any()          # outside the tensor: zeros
+        x = rng.standard_normal(in_dim).astype(np.float32)
+        ref = orc.dequant_matvec(W, None, None, x, out_dim, in_dim, bits)
+        (got,) = hip.matvec_batch([t], x, [out_dim])
+        assert_parity(got, ref, "resident GGUF matvec")
+        X = rng.standard_normal((3, in_dim)).astype(np.float32)
+        outs = hip.matvec_prefill(t, X, out_dim)
+        for m in range(3):
+            assert_parity(outs[m], orc.dequant_matvec(W, None, None, X[m], out_dim, in_dim, bits), "position %d" % m)
+    finally:
+        hip.tensor_release(t)
+
+
+@pytest.mark.parametrize("gtype", [12, 14])
+def test_gguf_vocabulary_projection_full_size(orc, gtype):
+    """The vocabulary projection of a GGUF model at its real size, 248320 x 2048 (Q4_K: the
+    streaming kernel; Q6_K: the rows-per-wave kernel): a few thousand sampled rows against the
+    oracle, every output finite, and rows sampled from the embedding lookup bit for bit."""
+    import torch
+    from finchmoe_amd import FinchHip
+    V, D = 248320, 2048
+    rb = F.gguf_row_bytes(D, gtype)
+    bsz = 144 if gtype == 12 else 210
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(17 + gtype)
+    Wd = torch.empty(V * (D // 256), bsz, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
+    n_d, d_off = (2, 0) if gtype == 12 else (1, 208)
+    d = (torch.randn(V * (D // 256), n_d, device=dev, generator=gen).abs_() * 0.002).to(torch.float16)
+    Wd[:, d_off:d_off + 2 * n_d] = d.view(torch.uint8)
+    x = torch.randn(D, device=dev, generator=gen)
+    out = torch.empty(V, device=dev)
+    torch.cuda.synchronize()
+    ctx = FinchHip(0)
+    try:
+        t = ctx.tensor_adopt(Wd.data_ptr(), None, None, V, D, bits=10 if gtype == 12 else 11)
+        ctx.matvec_batch_dev([t], x.data_ptr(), [out.data_ptr()])
+        ctx.sync()
+        got = out.cpu().numpy()
+        assert np.isfinite(got).all()
+        rng = np.random.default_rng(5)
+        rows = np.unique(np.concatenate([rng.integers(0, V, 3000), [0, 1, 2, 3, V - 4, V - 3, V - 2, V - 1]]))
+        Wh = Wd.view(V, rb)[torch.from_numpy(rows).to(dev)].cpu().numpy()
+        xh = x.cpu().numpy()
+        ref = orc.dequant_matvec(Wh.reshape(-1), None, None, xh, len(rows), D, 10 if gtype == 12 else 11)
+        assert_parity(got[rows], ref, "sampled rows of the vocabulary projection")
+        ids = torch.tensor([0, 777, V - 1], dtype=torch.int32, device=dev)
+        emb = torch.empty(3, D, device=dev)
+        ctx.embed_lookup_dev(t, ids.data_ptr(), 3, emb.data_ptr())
+        ctx.sync()
+        for i, tok in enumerate((0, 777, V - 1)):
+            rowb = Wd.view(V, rb)[tok].cpu().numpy()
+            assert np.array_equal(emb[i].cpu().numpy().view(np.uint32),
+                                  orc.gguf_dequant(rowb, 1, D, gtype)[0].view(np.uint32))
+    finally:
+        ctx.close()
