@@ -221,11 +221,11 @@ def cpu_baseline_dense(tensors, xs, budget_s=12.0, what="weight set"):
             x = np.ascontiguousarray(xs[xi], np.float32)
             out = np.empty(od, np.float32)
             t0 = time.perf_counter()
+            sp, bp = (None, None) if bits in (10, 11) else (S.ctypes.data, B.ctypes.data)
             if R is not None:
-                R.ref_cpu_dequant_matvec(W.ctypes.data, S.ctypes.data, B.ctypes.data, x.ctypes.data, out.ctypes.data,
-                                         od, idim, 64, bits)
+                R.ref_cpu_dequant_matvec(W.ctypes.data, sp, bp, x.ctypes.data, out.ctypes.data, od, idim, 64, bits)
             else:
-                oracle.dequant_matvec(W, S, B, x, od, idim, bits)
+                oracle.dequant_matvec(W, None if sp is None else S, None if bp is None else B, x, od, idim, bits)
             spent += time.perf_counter() - t0
         return spent
 
@@ -563,8 +563,9 @@ def run_gdn(args):
 
 
 def run_lm_head(args):
-    """Next row after the expert path: the 8-bit [vocab 248320, 2048] output projection
-    (finchmoe/infer.m:5728-5760), batch 1, three weight sets cycled (1.6 GB)."""
+    """Next row after the expert path: the [vocab 248320, 2048] output projection, batch 1, three
+    weight sets cycled: 8-bit affine (finchmoe/infer.m:5728-5760) or, with --lm-format q4k / q6k,
+    the GGUF block formats of a GGUF model's output.weight (finchmoe/infer.m:5738-5746)."""
     import torch
     from finchmoe_amd import FinchHip
     dev = torch.device("cuda:0")
@@ -573,13 +574,22 @@ def run_lm_head(args):
     gen.manual_seed(11)
     V, D = 248320, 2048
     keep, sets = [], []
+    fmt = args.lm_format
     for _ in range(3):
-        W = torch.empty(V * D, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
-        s = torch.randn(V * (D // 64), device=dev, generator=gen).abs_() * (0.02 / 127.5)
-        b = s * -127.5
-        S, B = _bf16_trunc_bits(s), _bf16_trunc_bits(b)
-        keep.extend([W, S, B])
-        sets.append(ctx.tensor_adopt(W.data_ptr(), S.data_ptr(), B.data_ptr(), V, D, 8))
+        if fmt == "affine8":
+            W = torch.empty(V * D, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
+            s = torch.randn(V * (D // 64), device=dev, generator=gen).abs_() * (0.02 / 127.5)
+            b = s * -127.5
+            S, B = _bf16_trunc_bits(s), _bf16_trunc_bits(b)
+            keep.extend([W, S, B])
+            sets.append(ctx.tensor_adopt(W.data_ptr(), S.data_ptr(), B.data_ptr(), V, D, 8))
+        else:
+            bsz, n_d, d_off, bits = (144, 2, 0, 10) if fmt == "q4k" else (210, 1, 208, 11)
+            W = torch.empty(V * (D // 256), bsz, dtype=torch.uint8, device=dev).random_(0, 256, generator=gen)
+            d = (torch.randn(V * (D // 256), n_d, device=dev, generator=gen).abs_() * 0.002).to(torch.float16)
+            W[:, d_off:d_off + 2 * n_d] = d.view(torch.uint8)
+            keep.append(W)
+            sets.append(ctx.tensor_adopt(W.data_ptr(), None, None, V, D, bits))
     d_x = torch.randn(D, device=dev)
     d_o = torch.empty(V, device=dev)
     torch.cuda.synchronize()
@@ -589,19 +599,29 @@ def run_lm_head(args):
 
     ms, ev = _timed(ctx, step, args)
     assert torch.isfinite(d_o).all()
-    bytes_set = V * D + 2 * V * (D // 64) * 2
-    res = {"event_ms_per_step": round(ev, 5),
-           "roofline": _roofline_hbm("fm_dense_stream<8,16,1>", bytes_set, ev * 1e3)}
+    if fmt == "affine8":
+        bytes_set = V * D + 2 * V * (D // 64) * 2
+        kernel = "fm_dense_stream<8,16,1>"
+    else:
+        bytes_set = V * (D // 256) * (144 if fmt == "q4k" else 210)
+        kernel = "fm_gguf_stream<Q4_K,16,down> on one dense tensor" if fmt == "q4k" else "fm_gguf_matvec_rows_k<Q6_K,16>"
+    res = {"event_ms_per_step": round(ev, 5), "roofline": _roofline_hbm(kernel, bytes_set, ev * 1e3)}
     if not args.no_cpu:
         # a bounded sample: the first 8192 rows of a set (the per-row arithmetic does not depend on the row)
         rows = 8192
-        sub = [[(keep[3 * i][:rows * D], keep[3 * i + 1][:rows * (D // 64)], keep[3 * i + 2][:rows * (D // 64)], rows, D, 8, 0)]
-               for i in range(3)]
+        if fmt == "affine8":
+            sub = [[(keep[3 * i][:rows * D], keep[3 * i + 1][:rows * (D // 64)], keep[3 * i + 2][:rows * (D // 64)], rows, D, 8, 0)]
+                   for i in range(3)]
+        else:
+            empty = torch.empty(0, dtype=torch.int16)
+            sub = [[(keep[i][:rows * (D // 256)].reshape(-1), empty, empty, rows, D, 10 if fmt == "q4k" else 11, 0)]
+                   for i in range(3)]
         res["cpu_baseline"] = cpu_baseline_dense(sub, [d_x.cpu().numpy()], args.cpu_seconds,
                                                  "%d-row slice of the projection" % rows)
     ctx.close()
-    return _finish(res, "8-bit output projection GEMV HBM GB/s", "lm_head 2048->248320, 8-bit g64, "
-                   "batch 1, 3 weight sets cycled", bytes_set, ms, args)
+    return _finish(res, "%s output projection GEMV HBM GB/s" % {"affine8": "8-bit", "q4k": "GGUF Q4_K", "q6k": "GGUF Q6_K"}[fmt],
+                   "lm_head 2048->248320, %s, batch 1, 3 weight sets cycled" % {"affine8": "8-bit g64", "q4k": "Q4_K", "q6k": "Q6_K"}[fmt],
+                   bytes_set, ms, args)
 
 
 def run_layer_tail(args):
@@ -835,10 +855,15 @@ def run_gguf(args):
         ms, ev = _timed(ctx, cstep, args)
         assert torch.isfinite(c_out).all()
         grouped = M >= 32 and not os.environ.get("FINCH_GGUF_NO_GROUP")
+        # grouped products read an expert once per group of its positions: priced on the distinct
+        # experts of a chunk; per-position products stream every routed expert once per position
+        uniq = float(np.mean([len(set(idx[:M, l].reshape(-1).tolist())) for l in range(n_layers)]))
+        rbytes = uniq * (2 * gsl + dsl) if grouped else M * K * (2 * gsl + dsl)
         cres = {"event_ms_per_step": round(ev, 5),
-                "roofline": _roofline_hbm("fm_gq_gate_up + fm_gq_down + fm_pf_combine (grouped products)" if grouped else
+                "roofline": _roofline_hbm("fm_gq_gate_up + fm_gq_down + fm_pf_combine (grouped products; bytes of the "
+                                          "chunk's distinct experts)" if grouped else
                                           "fm_gguf_stream<Q4_K gate/up> + fm_gguf_stream<Q6_K down> + fm_gguf_combine "
-                                          "(one group per position)", M * K * (2 * gsl + dsl), ev * 1e3, 4 if grouped else 3)}
+                                          "(one group per position)", rbytes, ev * 1e3, 4 if grouped else 3)}
         if grouped:
             flops = 2.0 * M * K * 3 * H * I
             cres["tflops"] = round(flops / (ev * 1e-3) / 1e12, 2)
@@ -910,6 +935,13 @@ def run_prefill(args):
         ctx.experts_adopt_layer(l, blob[l].data_ptr(), E * es)
     rng = np.random.default_rng(7)
     idx, w = zipf_routing(rng, M, nl, E, K)          # [M, nl, K]
+    if args.prefill_experts:
+        # profile buckets: uniform routing over the first N experts (N = 16: 256 positions per
+        # expert of a 512-position chunk, every item full; N = 256 with --chunk 128: 4 per expert)
+        n_e = max(K, min(E, args.prefill_experts))
+        for t in range(M):
+            for l in range(nl):
+                idx[t, l] = rng.permutation(n_e)[:K]
     idx = np.ascontiguousarray(idx.transpose(1, 0, 2))
     w = np.ascontiguousarray(w.transpose(1, 0, 2))
     d_idx, d_w = torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)
@@ -992,7 +1024,9 @@ def run_stream_probe(args):
     rates = {}
     for pattern, name in ((1, "contiguous_share_per_workgroup"), (2, "contiguous_share_per_wave"),
                           (3, "groups_of_4_workgroups_interleaved"), (4, "groups_of_8_workgroups_interleaved"),
-                          (5, "groups_of_8_workgroups_of_one_xcd_interleaved"), (0, "dense")):
+                          (5, "groups_of_8_workgroups_of_one_xcd_interleaved"),
+                          (6, "contiguous_share_per_workgroup_neighbours_on_one_xcd"),
+                          (7, "groups_of_4_workgroups_of_one_xcd_interleaved"), (0, "dense")):
         def step(t, pattern=pattern):
             ctx.stream_probe_dev(bufs[t & 1].data_ptr(), n, pattern)
         ms, ev = _timed(ctx, step, args)
@@ -1034,6 +1068,11 @@ def main():
                     help="untimed busy period before the warmup steps (clock ramp)")
     ap.add_argument("--graph", action="store_true",
                     help="moe_layer workload: replay the token from a captured HIP graph")
+    ap.add_argument("--prefill-experts", type=int, default=0,
+                    help="prefill workload: route uniformly over the first N experts instead of Zipf over all "
+                         "(profile buckets: all items full / all items small)")
+    ap.add_argument("--lm-format", default="affine8", choices=("affine8", "q4k", "q6k"),
+                    help="lm_head workload: 8-bit affine, or the GGUF block formats")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()

@@ -25,6 +25,7 @@ extern __shared__ __attribute__((aligned(16))) uint8_t fm_probe_lds[];
 //   2  every wave a contiguous share
 //   3, 4, 5  groups of 4 / 8 / 8 workgroups share a contiguous region whose slots go to the
 //      group's waves in turn (5: the eight workgroups of a group sit on one XCD)
+//   6  as 1 with neighbouring shares on one XCD;  7  groups of 4 workgroups of one XCD
 template <int PATTERN>
 __global__ __launch_bounds__(PROBE_WAVES * 64) void fm_stream_probe_k(const uint8_t *buf, size_t n_slots,
                                                                       unsigned int *sink) {
@@ -72,12 +73,13 @@ __global__ __launch_bounds__(PROBE_WAVES * 64) void fm_stream_probe_k(const uint
 extern "C" int fm_launch_stream_probe(const void *d_buf, size_t nbytes, int pattern, unsigned int *d_sink,
                                       int n_cu, hipStream_t st) {
     const size_t n_slots = nbytes / PROBE_SLOT;
-    if (!d_buf || n_slots == 0 || ((uintptr_t)d_buf & 15) || pattern < 0 || pattern > 5) return FM_ERR_ARG;
+    if (!d_buf || n_slots == 0 || ((uintptr_t)d_buf & 15) || pattern < 0 || pattern > 7) return FM_ERR_ARG;
     const size_t sh = (size_t)PROBE_WAVES * PROBE_RING * PROBE_SLOT;
-    static FmLdsAttr attr[6];
+    static FmLdsAttr attr[8];
     typedef void (*probe_fn)(const uint8_t *, size_t, unsigned int *);
-    static const probe_fn fns[6] = {fm_stream_probe_k<0>, fm_stream_probe_k<1>, fm_stream_probe_k<2>,
-                                    fm_stream_probe_k<3>, fm_stream_probe_k<4>, fm_stream_probe_k<5>};
+    static const probe_fn fns[8] = {fm_stream_probe_k<0>, fm_stream_probe_k<1>, fm_stream_probe_k<2>,
+                                    fm_stream_probe_k<3>, fm_stream_probe_k<4>, fm_stream_probe_k<5>,
+                                    fm_stream_probe_k<6>, fm_stream_probe_k<7>};
     if (!fm_dyn_lds_ready(attr[pattern], (const void *)fns[pattern], sh)) return FM_ERR_HIP;
     const dim3 grid(n_cu), block(PROBE_WAVES * 64);
     const uint8_t *b = (const uint8_t *)d_buf;
