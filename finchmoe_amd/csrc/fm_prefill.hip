@@ -946,13 +946,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint8_t *l_w = nullptr, *l_sb = nullptr;
     // SREG: scales and biases of the task the loader has entered, requested with four loads of
     // one contiguous KB each — lane (n, kb) gets the 16 bytes (eight groups) 16 kb of its rows —
-    // in front of the task's first slot: once that slot has landed, so have they.  nsc: the
-    // task being loaded, csc: the task being multiplied; [tile 0 s, tile 0 b, tile 1 s, tile 1 b].
-    pfr_u4 nsc[4], csc[4];
+    // in front of the task's first slot: once that slot has landed, so have they.  They land in
+    // v[240:255], which the statements name themselves: a value that is still in flight must
+    // never sit in a register the compiler allocates, because the compiler may move such a
+    // value to another register (at a loop's back edge, say) before the wait that makes it
+    // valid.  The kernel's own values stay far below v240 (the allocator fills registers from
+    // v0 upwards; a host test reads the compiled kernel and checks that nothing else names
+    // these sixteen).  csc: the landed copy of the task being multiplied, [tile 0 s, tile 0 b,
+    // tile 1 s, tile 1 b], taken behind that wait.
+    pfr_u4 csc[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) nsc[i] = csc[i] = pfr_u4{0u, 0u, 0u, 0u};
+    for (int i = 0; i < 4; i++) csc[i] = pfr_u4{0u, 0u, 0u, 0u};
     const uint32_t sc_lane = (uint32_t)(n * sb_bytes + 16 * kb);
-    int sc_round = R0;            // the round nsc was requested for
+    int sc_round = R0;            // the round whose scales were requested last
     auto loader_enter = [&]() __attribute__((always_inline)) {
         const int it = l_r / RPI, t = (l_r - it * RPI) * 8 + wave;
         const int e = __builtin_amdgcn_readlane(ev, it - it0);
@@ -962,11 +968,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         l_sb = fm_uniform(blob + r0 * sb_bytes);
         if constexpr (P::SREG) {
             const uint8_t *p0 = l_sb + a.g.gate_s, *p1 = l_sb + a.g.gate_b, *p2 = l_sb + a.g.up_s, *p3 = l_sb + a.g.up_b;
-            asm volatile("global_load_dwordx4 %0, %4, %5\n\tglobal_load_dwordx4 %1, %4, %6\n\t"
-                         "global_load_dwordx4 %2, %4, %7\n\tglobal_load_dwordx4 %3, %4, %8"
-                         : "=&v"(nsc[0]), "=&v"(nsc[1]), "=&v"(nsc[2]), "=&v"(nsc[3])
+            asm volatile("global_load_dwordx4 v[240:243], %0, %1\n\tglobal_load_dwordx4 v[244:247], %0, %2\n\t"
+                         "global_load_dwordx4 v[248:251], %0, %3\n\tglobal_load_dwordx4 v[252:255], %0, %4"
+                         :
                          : "v"(sc_lane), "s"(p0), "s"(p1), "s"(p2), "s"(p3)
-                         : "memory");
+                         : "memory", "v240", "v241", "v242", "v243", "v244", "v245", "v246", "v247", "v248", "v249",
+                           "v250", "v251", "v252", "v253", "v254", "v255");
             sc_round = l_r;
         }
     };
@@ -1129,8 +1136,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             uint2 q[2][4];
             if constexpr (P::SREG) {
                 if (s == 0) {          // the task's first slot is there, and so are its scales
+                    uint32_t t[16];
+                    asm volatile("v_mov_b32 %0, v240\n\tv_mov_b32 %1, v241\n\t"
+                                 "v_mov_b32 %2, v242\n\tv_mov_b32 %3, v243\n\t"
+                                 "v_mov_b32 %4, v244\n\tv_mov_b32 %5, v245\n\t"
+                                 "v_mov_b32 %6, v246\n\tv_mov_b32 %7, v247\n\t"
+                                 "v_mov_b32 %8, v248\n\tv_mov_b32 %9, v249\n\t"
+                                 "v_mov_b32 %10, v250\n\tv_mov_b32 %11, v251\n\t"
+                                 "v_mov_b32 %12, v252\n\tv_mov_b32 %13, v253\n\t"
+                                 "v_mov_b32 %14, v254\n\tv_mov_b32 %15, v255"
+                                 : "=v"(t[0]), "=v"(t[1]), "=v"(t[2]), "=v"(t[3]), "=v"(t[4]), "=v"(t[5]), "=v"(t[6]),
+                                   "=v"(t[7]), "=v"(t[8]), "=v"(t[9]), "=v"(t[10]), "=v"(t[11]), "=v"(t[12]),
+                                   "=v"(t[13]), "=v"(t[14]), "=v"(t[15])
+                                 :
+                                 : "memory");
 #pragma unroll
-                    for (int i = 0; i < 4; i++) csc[i] = nsc[i];
+                    for (int i = 0; i < 4; i++) csc[i] = pfr_u4{t[4 * i], t[4 * i + 1], t[4 * i + 2], t[4 * i + 3]};
                 }
                 // the slab's four groups are one dword pair of the lanes kb = s / 2
                 const uint32_t src = 4u * (uint32_t)(n + 16 * (s >> 1));

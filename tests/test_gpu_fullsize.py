@@ -28,6 +28,7 @@ def full_store():
     blob = torch.empty(L, E, es, dtype=torch.uint8, device=dev)
     for l in range(L):
         fill_affine_layer(blob[l], lo, 3, gen)
+    torch.cuda.synchronize()       # the context's stream does not wait for torch's
     ctx = FinchHip(0)
     ctx.experts_config(L, E, H, I, 64, 3, 0)
     for l in range(L):
@@ -194,6 +195,7 @@ def test_full_chunk_4bit_equals_positions(orc):
     gen.manual_seed(77)
     blob = torch.empty(1, E, es, dtype=torch.uint8, device=dev)
     fill_affine_layer(blob[0], lo, 4, gen)
+    torch.cuda.synchronize()       # the context's stream does not wait for torch's
     ctx = FinchHip(0)
     try:
         ctx.experts_config(1, E, H, I, 64, 4, 0)
