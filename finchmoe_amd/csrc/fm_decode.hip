@@ -739,7 +739,7 @@ struct Fm2Seg {
     uint32_t next_unit;
     uint32_t first, n;       // this workgroup's units of the segment
     int layer;               // layer group (layer of a step, position of a chunk)
-    uint32_t stride;         // distance between its units (fm2_part, fm_index.h)
+    int pad;
 };
 
 struct Fm2Sync {
@@ -866,9 +866,8 @@ struct Fm2Stream {
     bool l_gu;
     uint32_t cur_wstep, cur_sstep, cur_w, cur_s, cur_b, d_w, d_s, d_b;
     int lq, cq;
-    uint32_t l_first, l_n, l_nrb, l_stride;
+    uint32_t l_first, l_n, l_nrb;
     float l_inv;
-    int gu_l0;              // layer of gate/up image 0
     int hn, wpos, c;
     uint32_t tag_n, rsn, issued, consumed;
     const uint8_t *blob_n;
@@ -894,9 +893,7 @@ struct Fm2Stream {
         d_b = a.g.up_b - a.g.gate_b;
         lq = cq = 0;
         l_first = l_n = l_nrb = 0;
-        l_stride = 1u;
         l_inv = 0.0f;
-        gu_l0 = 0;
         hn = wpos = c = 0;
         tag_n = rsn = issued = consumed = 0;
         blob_n = nullptr;
@@ -914,9 +911,6 @@ struct Fm2Stream {
         const uint32_t ta = fm_lds_addr(&tab[q].first);
         l_first = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta));
         l_n = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + 4));
-        l_stride = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + 12));
-        static_assert(offsetof(Fm2Seg, n) == offsetof(Fm2Seg, first) + 4 &&
-                      offsetof(Fm2Seg, stride) == offsetof(Fm2Seg, first) + 12, "table layout");
         if (!l_gu) {
             l_nrb = l_n / (uint32_t)a.K;
             l_first = l_first / (uint32_t)a.K;          // first row block of the part
@@ -940,8 +934,8 @@ struct Fm2Stream {
                 return;
             }
             uint32_t pn;
-            if (l_gu) fm2_gu_unit(l_first, l_stride, ul, gu_upp, &pn, &rsn);
-            else fm2_dn_unit(l_first, l_stride, l_nrb, l_inv, ul, &pn, &rsn);     // expert by expert
+            if (l_gu) fm2_gu_unit(l_first, ul, gu_upp, &pn, &rsn);
+            else fm2_dn_unit(l_first, l_nrb, l_inv, ul, &pn, &rsn);     // expert by expert
             tag_n = ((uint32_t)(lq & 1) << 31) | (pn << 28) | ul;
             const uint32_t ba = fm_lds_addr(&tab[lq].blob[pn]);
             const uint32_t lo = __builtin_amdgcn_readfirstlane(fm_lds_r32(ba));
@@ -996,24 +990,21 @@ struct Fm2Stream {
         const uint32_t ta = fm_lds_addr(&tab[q]);
         const uint32_t first = fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, first));
         const uint32_t n = fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, n));
-        const int stride = (int)fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, stride));
         float wk[FM_MAX_K];
 #pragma unroll
         for (int k = 0; k < FM_MAX_K; k++)
             wk[k] = k < K ? __uint_as_float(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, w) + 4u * k)) : 0.0f;
         const int rows = (int)(n / (uint32_t)K) * RPS_DN;
         const int l = seg_layer(q);
-        // the part's row block rbi is row block first / K + stride * rbi of the layer
         float *out = a.out + (size_t)l * a.g.hidden + (size_t)(first / (uint32_t)K) * RPS_DN;
         for (int r = threadIdx.x; r < rows; r += FM_NW * 64) {
             const int rbi = r / RPS_DN, ris = r - rbi * RPS_DN;
-            const int orow = stride * rbi * RPS_DN + ris;
             float acc = 0.0f;
 #pragma unroll
             for (int k = 0; k < FM_MAX_K; k++)
                 if (k < K && wk[k] != 0.0f)
                     acc += wk[k] * __uint_as_float(fm_lds_r32(part0 + 4u * (uint32_t)((rbi * K + k) * RPS_DN + ris)));
-            out[orow] = (a.flags & FM_ACCUMULATE) ? out[orow] + acc : acc;
+            out[r] = (a.flags & FM_ACCUMULATE) ? out[r] + acc : acc;
         }
     }
 
@@ -1029,7 +1020,7 @@ struct Fm2Stream {
         const Fm2Dims dm = fm2_dims(n_pairs, K, G, a.g.inter, a.g.hidden, LPR_UP);
         const Fm2Split sp = fm2_split(dm, (uint32_t)g);
         const uint32_t gu_segu = dm.gu_segu;
-        gu_l0 = (int)sp.gu_l0;
+        const int gu_s0 = sp.gu_s0;
         n_up = sp.n_up;
         n_seq = sp.n_up + sp.n_dn;
         const int qq = threadIdx.x >> 3;        // the segment this thread looks up below
@@ -1048,8 +1039,8 @@ struct Fm2Stream {
         // whose result is still pending on some path of the control flow makes the compiler
         // wait for every load in flight at the register's next use, in the middle of the stream)
         FmActX<LPR_UP> xr0, xr1;
-        fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)(n_up > 0 ? gu_l0 : 0) * a.g.hidden, bslot, xr0);
-        fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)(n_up > 0 && sp.gu_two ? gu_l0 + 1 : 0) * a.g.hidden, bslot, xr1);
+        fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)(n_up > 0 ? gu_s0 : 0) * a.g.hidden, bslot, xr0);
+        fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)(n_up > 1 ? gu_s0 + 1 : 0) * a.g.hidden, bslot, xr1);
         if (mine) {
             const int k = threadIdx.x & 7;
             const size_t sg = mine_s;                              // layer group of the segment
@@ -1069,7 +1060,6 @@ struct Fm2Stream {
                 t.first = mine_first;
                 t.n = mine_n;
                 t.layer = (int)sg;
-                t.stride = mp.stride;
             }
         }
 #pragma unroll
@@ -1092,7 +1082,7 @@ struct Fm2Stream {
             for (int i = 0; i < FmActX<LPR_UP>::NIT; i++) {
                 const int chn = (threadIdx.x >> 6) + 4 * i;
                 fm2_build_chunk<BITS, LPR_UP>(xr0.xl[i], xr0.xh[i], bslot, img0, chn, chn < LPR_UP);
-                fm2_build_chunk<BITS, LPR_UP>(xr1.xl[i], xr1.xh[i], bslot, img0 + IMG_UP, chn, chn < LPR_UP && sp.gu_two);
+                fm2_build_chunk<BITS, LPR_UP>(xr1.xl[i], xr1.xh[i], bslot, img0 + IMG_UP, chn, chn < LPR_UP && n_up > 1);
             }
         }
         fm_wg_barrier();
@@ -1105,13 +1095,12 @@ struct Fm2Stream {
                                                soff, ris, ch);
             for (; cq < n_up; cq++) {
                 const int s = seg_layer(cq);
-                const uint32_t img = img0 + (uint32_t)(s - gu_l0) * IMG_UP;      // image of the segment's layer
+                const uint32_t img = img0 + (uint32_t)(cq & 1) * IMG_UP;
                 FmActRegs ar;
                 fm_read_act_lds_x<LPR_UP>(img, lane, ar);
                 const uint32_t ta = fm_lds_addr(&tab[cq]);
                 const uint32_t valid = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, valid)));
                 const uint32_t c_first = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, first)));
-                const uint32_t c_stride = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, stride)));
                 const size_t out0 = ((size_t)s * gu_segu + c_first) * RPS_UP + ris;
                 dry = false;
                 while (issued - consumed < (uint32_t)RING && !dry) issue();
@@ -1123,7 +1112,7 @@ struct Fm2Stream {
                     const float uv = take<LPR_UP>(woff, soff, ar);
                     float v = fm_silu_mul(gv, uv);
                     if (!((valid >> pc) & 1u)) v = 0.0f;
-                    if (ch == 0) fm_st_shared(a.act + out0 + (size_t)(ul * c_stride) * RPS_UP, v);
+                    if (ch == 0) fm_st_shared(a.act + out0 + (size_t)ul * RPS_UP, v);
                 }
             }
         }

@@ -379,158 +379,68 @@ FM_HD Fm2Dims fm2_dims(int n_pairs, int K, int G, int inter, int hidden, int lpr
     d.s_total = 2u * d.gu_total + d.rb_total * d.K;
     return d;
 }
-// Down phase.  With at least as many workgroups as layers a workgroup's row blocks lie in ONE layer:
-// layer l belongs to the workgroups g with g * L / G == l, and its row blocks are dealt out to them
-// in turn (workgroup j of n takes row blocks j, j + n, ...), so that the layer's workgroups read
-// its experts side by side.  Otherwise (more layers than workgroups) every workgroup takes a
-// contiguous run of row blocks.
-struct Fm2Down {
-    int interleaved;
-    uint32_t layer, rb0, nrb, stride;   // interleaved: row blocks rb0 + stride * i, i < nrb, of `layer`
-    uint32_t wg0, wg1;                  // contiguous: units (row block * K + slot) [wg0, wg1)
-};
-FM_HD Fm2Down fm2_down(const Fm2Dims &d, uint32_t gg) {
-    Fm2Down w;
-    w.interleaved = d.G >= d.L;
-    w.layer = w.rb0 = w.nrb = 0u, w.stride = 1u, w.wg0 = w.wg1 = 0u;
-    if (gg >= d.G) return w;
-    if (!w.interleaved) {
-        w.wg0 = (d.rb_total * gg / d.G) * d.K;
-        w.wg1 = (d.rb_total * (gg + 1u) / d.G) * d.K;
-        return w;
-    }
-    w.layer = gg * d.L / d.G;
-    const uint32_t g_lo = (w.layer * d.G + d.L - 1u) / d.L, g_hi = ((w.layer + 1u) * d.G + d.L - 1u) / d.L;
-    w.stride = g_hi - g_lo;
-    w.rb0 = gg - g_lo;
-    w.nrb = w.rb0 < d.dn_upp ? (d.dn_upp - w.rb0 + w.stride - 1u) / w.stride : 0u;
-    return w;
-}
-// row blocks of the workgroups before gg (what the gate/up split balances against)
+// first down row block of workgroup gg: a workgroup's row blocks lie in ONE layer whenever there
+// are at least as many workgroups as layers
 FM_HD uint32_t fm2_dn_start(const Fm2Dims &d, uint32_t gg) {
     if (gg >= d.G) return d.rb_total;
     if (d.G < d.L) return d.rb_total * gg / d.G;
     const uint32_t l = gg * d.L / d.G;
     const uint32_t g_lo = (l * d.G + d.L - 1u) / d.L, g_hi = ((l + 1u) * d.G + d.L - 1u) / d.L;
-    const uint32_t n = g_hi - g_lo, j = gg - g_lo, q = d.dn_upp / n, r = d.dn_upp % n;
-    return l * d.dn_upp + j * q + (j < r ? j : r);
+    return l * d.dn_upp + d.dn_upp * (gg - g_lo) / (g_hi - g_lo);
 }
-// first gate/up unit of workgroup gg's share (dn0 = row blocks of the workgroups before it): sized
-// so that gate/up + down slices are the same for every workgroup
+// first gate/up unit of workgroup gg (dn0 = its first down row block): sized so that gate/up +
+// down slices are the same for every workgroup
 FM_HD uint32_t fm2_gu_start(const Fm2Dims &d, uint32_t gg, uint32_t dn0) {
     const uint32_t t = d.s_total * gg / d.G, dd = dn0 * d.K;
     const uint32_t u = t > dd ? (t - dd) / 2u : 0u;
     return u > d.gu_total ? d.gu_total : u;
 }
-FM_HD uint32_t fm2_gu_begin(const Fm2Dims &d, uint32_t gg) {
-    return gg >= d.G ? d.gu_total : fm2_gu_start(d, gg, fm2_dn_start(d, gg));
-}
-// Gate/up phase.  Groups of FM2_GROUP workgroups (neighbours behind one XCD's L2) share the
-// contiguous unit range their byte-balanced shares add up to, and its units are dealt out to the
-// members in turn — at any moment a group reads one window of an expert instead of four distant
-// ones (measured with the stream probe: 71.7 us against 75.3 us for 440 MB).  Member j takes
-// units r0 + j + members * i for i < cmin (cmin = the smallest share of the group) and then a
-// contiguous run of the remaining units, as many as its own share exceeds cmin.  A group whose
-// range is longer than a layer keeps contiguous shares (its units would touch more than the two
-// layers a workgroup holds images for).
-#define FM2_GROUP 4
 struct Fm2Split {
-    uint32_t g;                 // logical workgroup: neighbours sit on one XCD
-    uint32_t a0, na, sa;        // dealt-out run: units a0 + sa * i, i < na
-    uint32_t b0, nb;            // contiguous run: units b0 + i, i < nb
-    uint32_t gu_l0;             // first layer the group's range touches (image 0; image 1 = the next)
-    int gu_two;                 // the range touches a second layer
-    int na_seg, nb_seg;         // layers the two runs cross
-    Fm2Down dn;
-    int n_up, n_dn;             // segments of each phase
+    uint32_t gu_wg0, gu_wg1, dn_wg0, dn_wg1;    // unit ranges (down: row block * K)
+    int gu_s0, dn_s0, n_up, n_dn;               // first segment and segment count of each phase
 };
-FM_HD Fm2Split fm2_split(const Fm2Dims &d, uint32_t block) {
+FM_HD Fm2Split fm2_split(const Fm2Dims &d, uint32_t g) {
     Fm2Split s;
-    s.g = fm_xcd_share(block, d.G);
-    const uint32_t m0 = s.g - s.g % FM2_GROUP;
-    const uint32_t members = d.G - m0 < FM2_GROUP ? d.G - m0 : FM2_GROUP;
-    const uint32_t r0 = fm2_gu_begin(d, m0), r1 = fm2_gu_begin(d, m0 + members);
-    const uint32_t own0 = fm2_gu_begin(d, s.g), own1 = fm2_gu_begin(d, s.g + 1u);
-    if (members > 1u && r1 - r0 <= d.gu_segu) {
-        uint32_t cmin = 0xFFFFFFFFu, before = 0u;
-        for (uint32_t k = 0; k < members; k++) {
-            const uint32_t c = fm2_gu_begin(d, m0 + k + 1u) - fm2_gu_begin(d, m0 + k);
-            if (c < cmin) cmin = c;
-        }
-        for (uint32_t k = 0; k < s.g - m0; k++)
-            before += fm2_gu_begin(d, m0 + k + 1u) - fm2_gu_begin(d, m0 + k) - cmin;
-        s.a0 = r0 + (s.g - m0), s.na = cmin, s.sa = members;
-        s.b0 = r0 + members * cmin + before, s.nb = own1 - own0 - cmin;
-        s.gu_l0 = r0 / d.gu_segu;
-        s.gu_two = r1 > r0 && (r1 - 1u) / d.gu_segu > s.gu_l0;
-    } else {
-        s.a0 = own0, s.na = own1 - own0, s.sa = 1u;
-        s.b0 = own1, s.nb = 0u;
-        s.gu_l0 = own0 / d.gu_segu;
-        s.gu_two = own1 > own0 && (own1 - 1u) / d.gu_segu > s.gu_l0;
-    }
-    s.na_seg = s.na ? (int)((s.a0 + s.sa * (s.na - 1u)) / d.gu_segu - s.a0 / d.gu_segu) + 1 : 0;
-    s.nb_seg = s.nb ? (int)((s.b0 + s.nb - 1u) / d.gu_segu - s.b0 / d.gu_segu) + 1 : 0;
-    s.n_up = s.na_seg + s.nb_seg;
-    s.dn = fm2_down(d, s.g);
-    if (s.dn.interleaved) s.n_dn = s.dn.nrb ? 1 : 0;
-    else s.n_dn = s.dn.wg1 > s.dn.wg0 ? (int)((s.dn.wg1 - 1u) / d.dn_segu - s.dn.wg0 / d.dn_segu) + 1 : 0;
+    const uint32_t dn_rb0 = fm2_dn_start(d, g), dn_rb1 = fm2_dn_start(d, g + 1u);
+    s.gu_wg0 = fm2_gu_start(d, g, dn_rb0);
+    s.gu_wg1 = fm2_gu_start(d, g + 1u, dn_rb1);
+    s.dn_wg0 = dn_rb0 * d.K;
+    s.dn_wg1 = dn_rb1 * d.K;
+    s.gu_s0 = (int)(s.gu_wg0 / d.gu_segu);
+    s.dn_s0 = (int)(s.dn_wg0 / d.dn_segu);
+    s.n_up = s.gu_wg1 > s.gu_wg0 ? (int)((s.gu_wg1 - 1u) / d.gu_segu) + 1 - s.gu_s0 : 0;
+    s.n_dn = s.dn_wg1 > s.dn_wg0 ? (int)((s.dn_wg1 - 1u) / d.dn_segu) + 1 - s.dn_s0 : 0;
     return s;
 }
 // segment qq of the workgroup's sequence (gate/up segments first): layer group, first unit inside
-// the layer, unit count, distance between the units.  Gate/up unit i of the segment is unit
-// first + stride * i of the layer (slot-major); down unit ul is row block first / K + stride * (ul
-// % (n / K)) of slot ul / (n / K).
+// the segment, unit count
 struct Fm2Part {
-    uint32_t seg, first, n, stride;
+    uint32_t seg, first, n;
     int gu;
 };
-// the units of run (u0, count, step) that lie in layer `l`
-FM_HD void fm2_run_in_layer(uint32_t u0, uint32_t count, uint32_t step, uint32_t l, uint32_t segu, uint32_t *first,
-                            uint32_t *n) {
-    const uint32_t lo = l * segu, hi = lo + segu;
-    const uint32_t i_lo = lo > u0 ? (lo - u0 + step - 1u) / step : 0u;
-    uint32_t i_hi = hi > u0 ? (hi - u0 + step - 1u) / step : 0u;
-    if (i_hi > count) i_hi = count;
-    *n = i_hi > i_lo ? i_hi - i_lo : 0u;
-    *first = u0 + step * i_lo - lo;
-}
 FM_HD Fm2Part fm2_part(const Fm2Dims &d, const Fm2Split &s, int qq) {
     Fm2Part p;
     p.gu = qq < s.n_up;
-    p.stride = 1u;
-    if (p.gu) {
-        if (qq < s.na_seg) {
-            p.seg = s.a0 / d.gu_segu + (uint32_t)qq;
-            p.stride = s.sa;
-            fm2_run_in_layer(s.a0, s.na, s.sa, p.seg, d.gu_segu, &p.first, &p.n);
-        } else {
-            p.seg = s.b0 / d.gu_segu + (uint32_t)(qq - s.na_seg);
-            fm2_run_in_layer(s.b0, s.nb, 1u, p.seg, d.gu_segu, &p.first, &p.n);
-        }
-    } else if (s.dn.interleaved) {
-        p.seg = s.dn.layer;
-        p.first = s.dn.rb0 * d.K;
-        p.n = s.dn.nrb * d.K;
-        p.stride = s.dn.stride;
-    } else {
-        p.seg = s.dn.wg0 / d.dn_segu + (uint32_t)(qq - s.n_up);
-        fm2_run_in_layer(s.dn.wg0, s.dn.wg1 - s.dn.wg0, 1u, p.seg, d.dn_segu, &p.first, &p.n);
-    }
+    p.seg = (uint32_t)(p.gu ? s.gu_s0 + qq : s.dn_s0 + (qq - s.n_up));
+    const uint32_t segu = p.gu ? d.gu_segu : d.dn_segu, w0 = p.gu ? s.gu_wg0 : s.dn_wg0,
+                   w1 = p.gu ? s.gu_wg1 : s.dn_wg1;
+    const uint32_t lo = p.seg * segu > w0 ? p.seg * segu : w0;
+    const uint32_t hi = (p.seg + 1u) * segu < w1 ? (p.seg + 1u) * segu : w1;
+    p.first = lo - p.seg * segu;
+    p.n = hi > lo ? hi - lo : 0u;
     return p;
 }
 // claimed unit ul of a gate/up part: slot pn of the layer and row step rsn of its expert
-FM_HD void fm2_gu_unit(uint32_t first, uint32_t stride, uint32_t ul, uint32_t gu_upp, uint32_t *pn, uint32_t *rsn) {
-    const uint32_t uq = first + stride * ul;
+FM_HD void fm2_gu_unit(uint32_t first, uint32_t ul, uint32_t gu_upp, uint32_t *pn, uint32_t *rsn) {
+    const uint32_t uq = first + ul;
     *pn = uq / gu_upp;
     *rsn = uq - *pn * gu_upp;
 }
-// claimed unit ul of a down part of nrb row blocks rb_first + stride * i (expert by expert: unit
-// ul = the part's row block ul % nrb of slot ul / nrb); inv = 1 / nrb in fp32
-FM_HD void fm2_dn_unit(uint32_t rb_first, uint32_t stride, uint32_t nrb, float inv, uint32_t ul, uint32_t *pn,
-                       uint32_t *rsn) {
+// claimed unit ul of a down part of nrb row blocks starting at row block rb_first (expert by
+// expert: unit ul = row block ul % nrb of slot ul / nrb); inv = 1 / nrb in fp32
+FM_HD void fm2_dn_unit(uint32_t rb_first, uint32_t nrb, float inv, uint32_t ul, uint32_t *pn, uint32_t *rsn) {
     *pn = (uint32_t)(((float)ul + 0.5f) * inv);
-    *rsn = rb_first + stride * (ul - *pn * nrb);
+    *rsn = rb_first + (ul - *pn * nrb);
 }
 // the launcher's decision: workgroups, and whether the shape fits the kernel's fixed tables
 struct Fm2Plan {
@@ -562,7 +472,7 @@ FM_HD Fm2Plan fm2_plan(int n_pairs, int K, int inter, int hidden, int lpr_up, in
         n_dn = (rb_share - 1) / dn_rbs + 2;
         part_rbs = rb_share < dn_rbs ? rb_share : dn_rbs;
     }
-    if (4 + n_dn > FM2_MAX_SEG) return p;      // up to four gate/up segments: two runs x two layers
+    if (2 + n_dn > FM2_MAX_SEG) return p;
     if (part_rbs * K * rps_dn * 4 > FM2_PART_BYTES) return p;
     p.ok = 1;
     return p;

@@ -390,30 +390,24 @@ static void walk_fused_rows(int n_groups, int K, int hidden, int inter, int bits
     Region X("x", (size_t)n_groups * hidden * 4), idx("idx", (size_t)n_pairs * 4);
     int max_seq = 0;
     size_t max_bytes = 0, min_bytes = (size_t)-1;
-    std::vector<uint8_t> logical(G, 0);
     for (int gi = 0; gi < G; gi++) {
         const Fm2Split sp = fm2_split(dm, gi);
-        CHECK(sp.g < (uint32_t)G && !logical[sp.g], "logical workgroup %u taken twice", sp.g);
-        if (sp.g < (uint32_t)G) logical[sp.g] = 1;
         const int n_seq = sp.n_up + sp.n_dn;
         if (n_seq > max_seq) max_seq = n_seq;
-        CHECK(sp.n_up <= 4, "workgroup %d: %d gate/up segments", gi, sp.n_up);
+        CHECK(sp.n_up <= 2, "workgroup %d: %d gate/up segments", gi, sp.n_up);
         CHECK(n_seq <= FM2_MAX_SEG && n_seq <= 64, "workgroup %d: %d segments", gi, n_seq);
-        // the two input vectors loaded up front: images 0 and 1 = layers gu_l0 and gu_l0 + 1
-        if (sp.n_up > 0) X.touch((size_t)sp.gu_l0 * hidden * 4, (size_t)hidden * 4, "x of image 0");
-        if (sp.n_up > 0 && sp.gu_two) X.touch((size_t)(sp.gu_l0 + 1) * hidden * 4, (size_t)hidden * 4, "x of image 1");
+        // the two input vectors loaded up front
+        if (sp.n_up > 0) X.touch((size_t)sp.gu_s0 * hidden * 4, (size_t)hidden * 4, "x of the first segment");
+        if (sp.n_up > 1) X.touch((size_t)(sp.gu_s0 + 1) * hidden * 4, (size_t)hidden * 4, "x of the second segment");
         size_t bytes = 0;
         for (int qq = 0; qq < n_seq; qq++) {
             const Fm2Part pt = fm2_part(dm, sp, qq);
             CHECK(pt.seg < (uint32_t)n_groups, "segment %u", pt.seg);
-            if (pt.seg >= (uint32_t)n_groups) continue;
             for (int k = 0; k < K; k++) idx.touch(((size_t)pt.seg * K + k) * 4, 4, "idx");
             if (pt.gu) {
-                CHECK(pt.seg == sp.gu_l0 || (pt.seg == sp.gu_l0 + 1 && sp.gu_two), "segment of layer %u has no image (first layer %u)",
-                      pt.seg, sp.gu_l0);
                 for (uint32_t ul = 0; ul < pt.n; ul++) {
                     uint32_t pn, rsn;
-                    fm2_gu_unit(pt.first, pt.stride, ul, dm.gu_upp, &pn, &rsn);
+                    fm2_gu_unit(pt.first, ul, dm.gu_upp, &pn, &rsn);
                     CHECK(pn < (uint32_t)K && rsn < dm.gu_upp, "gate/up unit %u -> slot %u step %u", ul, pn, rsn);
                     if (pn >= (uint32_t)K) continue;
                     Region &bl = blob[pt.seg * K + pn];
@@ -425,8 +419,7 @@ static void walk_fused_rows(int n_groups, int K, int hidden, int inter, int bits
                     for (int lane = 0; lane < 64; lane++) {
                         const FmUnitLane ulr = fm_unit_lane(lane, lpr_up, fm_lane_bytes(bits), hidden * bits / 8, (hidden / 64) * 2);
                         if (ulr.ch == 0)
-                            act.touch((((size_t)pt.seg * dm.gu_segu + pt.first) * rps_up + ulr.row_in_step +
-                                       (size_t)(ul * pt.stride) * rps_up) * 4, 4, "act");
+                            act.touch((((size_t)pt.seg * dm.gu_segu + pt.first) * rps_up + ulr.row_in_step + (size_t)ul * rps_up) * 4, 4, "act");
                     }
                 }
             } else {
@@ -436,10 +429,10 @@ static void walk_fused_rows(int n_groups, int K, int hidden, int inter, int bits
                 CHECK((size_t)nrb * K * rps_dn * 4 <= FM2_PART_BYTES, "partial vectors of %u row blocks", nrb);
                 for (uint32_t ul = 0; ul < pt.n; ul++) {
                     uint32_t pn, rsn;
-                    fm2_dn_unit(rb_first, pt.stride, nrb, inv, ul, &pn, &rsn);
-                    CHECK(pn == ul / nrb && rsn == rb_first + pt.stride * (ul % nrb), "down unit %u -> slot %u block %u", ul, pn, rsn);
+                    fm2_dn_unit(rb_first, nrb, inv, ul, &pn, &rsn);
+                    CHECK(pn == ul / nrb && rsn == rb_first + ul % nrb, "down unit %u -> slot %u block %u", ul, pn, rsn);
                     CHECK(pn < (uint32_t)K && rsn < dm.dn_upp, "down unit %u -> slot %u block %u", ul, pn, rsn);
-                    if (pn >= (uint32_t)K || rsn >= dm.dn_upp) continue;
+                    if (pn >= (uint32_t)K) continue;
                     Region &bl = blob[pt.seg * K + pn];
                     unit_dma(bl, (size_t)rsn * dn_wstep + g.down_w, bl, (size_t)rsn * dn_sstep + g.down_s, bl,
                              (size_t)rsn * dn_sstep + g.down_b, bits);
@@ -448,15 +441,11 @@ static void walk_fused_rows(int n_groups, int K, int hidden, int inter, int bits
                     for (int ris = 0; ris < rps_dn; ris++)
                         CHECK(4u * ((rbi * K + pn) * rps_dn + ris) + 4 <= FM2_PART_BYTES, "partial slot");
                 }
-                // activations of the layer's K experts, and the part's rows of out (reduce_part)
+                // activations of the layer's K experts, and the part's rows of out
                 Region a1("act", act.size);
                 a1.touch((size_t)pt.seg * K * inter * 4, (size_t)K * inter * 4, "act of the layer");
                 const int rows = (int)nrb * rps_dn;
-                for (int r = 0; r < rows; r++) {
-                    const int rbi = r / rps_dn, ris = r - rbi * rps_dn;
-                    out.touch(((size_t)pt.seg * hidden + (size_t)rb_first * rps_dn + (size_t)pt.stride * rbi * rps_dn + ris) * 4, 4,
-                              "out row");
-                }
+                out.touch(((size_t)pt.seg * hidden + (size_t)rb_first * rps_dn) * 4, (size_t)rows * 4, "out rows");
             }
         }
         if (bytes > max_bytes) max_bytes = bytes;
@@ -475,53 +464,49 @@ static void sweep_fused_rows() {
     g_case = "fused rows, sweep of shapes";
     int taken = 0;
     for (int lpr_up : {4, 8, 16})
-        for (int inter_mul : {1, 2})
-            for (int n_groups : {1, 2, 3, 5, 8, 13, 31, 40, 41, 47, 64, 100})
-                for (int K : {1, 2, 5, 8})
-                    for (int n_cu : {256, 240, 104, 30}) {
-                        const int hidden = 128 * lpr_up, inter = (hidden / 4) * inter_mul;
-                        if (inter / FM_CPL != lpr_up / 4 && inter_mul == 1) continue;
-                        if (inter_mul == 2) continue;       // the kernel covers inter = hidden / 4 only
-                        const int n_pairs = n_groups * K;
-                        const Fm2Plan plan = fm2_plan(n_pairs, K, inter, hidden, lpr_up, n_cu);
-                        if (!plan.ok) continue;
-                        taken++;
-                        const int rps_dn = FM_WAVE / (lpr_up / 4);
-                        const Fm2Dims dm = fm2_dims(n_pairs, K, plan.wgs, inter, hidden, lpr_up);
-                        std::vector<uint8_t> gu(dm.gu_total, 0), dn((size_t)dm.rb_total * K, 0);
-                        for (int b = 0; b < plan.wgs; b++) {
-                            const Fm2Split sp = fm2_split(dm, b);
-                            CHECK(sp.n_up <= 4 && sp.n_up + sp.n_dn <= FM2_MAX_SEG, "%d groups K %d lpr %d cu %d: segments %d + %d",
-                                  n_groups, K, lpr_up, n_cu, sp.n_up, sp.n_dn);
-                            for (int qq = 0; qq < sp.n_up + sp.n_dn; qq++) {
-                                const Fm2Part pt = fm2_part(dm, sp, qq);
-                                if (pt.gu) {
-                                    CHECK(pt.seg == sp.gu_l0 || (pt.seg == sp.gu_l0 + 1 && sp.gu_two), "image of layer %u", pt.seg);
-                                    for (uint32_t ul = 0; ul < pt.n; ul++) {
-                                        const size_t u = (size_t)pt.seg * dm.gu_segu + pt.first + (size_t)pt.stride * ul;
-                                        CHECK(pt.first + pt.stride * ul < dm.gu_segu && u < gu.size(), "gate/up unit");
-                                        if (u < gu.size()) gu[u]++;
-                                    }
-                                } else {
-                                    const uint32_t rb_first = pt.first / K, nrb = pt.n / K;
-                                    CHECK(pt.first % K == 0 && pt.n % K == 0 && (size_t)nrb * K * rps_dn * 4 <= FM2_PART_BYTES,
-                                          "%d groups K %d lpr %d cu %d: part of %u row blocks", n_groups, K, lpr_up, n_cu, nrb);
-                                    const float inv = 1.0f / (float)(nrb ? nrb : 1u);
-                                    for (uint32_t ul = 0; ul < pt.n; ul++) {
-                                        uint32_t pn, rsn;
-                                        fm2_dn_unit(rb_first, pt.stride, nrb, inv, ul, &pn, &rsn);
-                                        CHECK(pn < (uint32_t)K && rsn < dm.dn_upp, "down unit");
-                                        const size_t u = ((size_t)pt.seg * dm.dn_upp + rsn) * K + pn;
-                                        if (pn < (uint32_t)K && rsn < dm.dn_upp) dn[u]++;
-                                    }
+        for (int n_groups : {1, 2, 3, 5, 8, 13, 31, 40, 41, 47, 64, 100})
+            for (int K : {1, 2, 5, 8})
+                for (int n_cu : {256, 240, 104, 30}) {
+                    const int hidden = 128 * lpr_up, inter = hidden / 4;     // the kernel covers inter = hidden / 4
+                    const int n_pairs = n_groups * K;
+                    const Fm2Plan plan = fm2_plan(n_pairs, K, inter, hidden, lpr_up, n_cu);
+                    if (!plan.ok) continue;
+                    taken++;
+                    const int rps_dn = FM_WAVE / (lpr_up / 4);
+                    const Fm2Dims dm = fm2_dims(n_pairs, K, plan.wgs, inter, hidden, lpr_up);
+                    std::vector<uint8_t> gu(dm.gu_total, 0), dn((size_t)dm.rb_total * K, 0);
+                    for (int b = 0; b < plan.wgs; b++) {
+                        const Fm2Split sp = fm2_split(dm, b);
+                        CHECK(sp.n_up <= 2 && sp.n_up + sp.n_dn <= FM2_MAX_SEG, "%d groups K %d lpr %d cu %d: segments %d + %d",
+                              n_groups, K, lpr_up, n_cu, sp.n_up, sp.n_dn);
+                        for (int qq = 0; qq < sp.n_up + sp.n_dn; qq++) {
+                            const Fm2Part pt = fm2_part(dm, sp, qq);
+                            if (pt.gu) {
+                                for (uint32_t ul = 0; ul < pt.n; ul++) {
+                                    const size_t u = (size_t)pt.seg * dm.gu_segu + pt.first + ul;
+                                    CHECK(pt.first + ul < dm.gu_segu && u < gu.size(), "gate/up unit");
+                                    if (u < gu.size()) gu[u]++;
+                                }
+                            } else {
+                                const uint32_t rb_first = pt.first / K, nrb = pt.n / K;
+                                CHECK(pt.first % K == 0 && pt.n % K == 0 && (size_t)nrb * K * rps_dn * 4 <= FM2_PART_BYTES,
+                                      "%d groups K %d lpr %d cu %d: part of %u row blocks", n_groups, K, lpr_up, n_cu, nrb);
+                                const float inv = 1.0f / (float)(nrb ? nrb : 1u);
+                                for (uint32_t ul = 0; ul < pt.n; ul++) {
+                                    uint32_t pn, rsn;
+                                    fm2_dn_unit(rb_first, nrb, inv, ul, &pn, &rsn);
+                                    CHECK(pn < (uint32_t)K && rsn < dm.dn_upp, "down unit");
+                                    const size_t u = ((size_t)pt.seg * dm.dn_upp + rsn) * K + pn;
+                                    if (pn < (uint32_t)K && rsn < dm.dn_upp) dn[u]++;
                                 }
                             }
                         }
-                        size_t bad = 0;
-                        for (uint8_t c : gu) bad += c != 1;
-                        for (uint8_t c : dn) bad += c != 1;
-                        CHECK(bad == 0, "%d groups K %d lpr %d cu %d: %zu units not handed out exactly once", n_groups, K, lpr_up, n_cu, bad);
                     }
+                    size_t bad = 0;
+                    for (uint8_t c : gu) bad += c != 1;
+                    for (uint8_t c : dn) bad += c != 1;
+                    CHECK(bad == 0, "%d groups K %d lpr %d cu %d: %zu units not handed out exactly once", n_groups, K, lpr_up, n_cu, bad);
+                }
     std::printf("ok  %-58s %d shapes taken by this launch form\n", g_case.c_str(), taken);
 }
 

@@ -39,20 +39,21 @@ def test_every_access_of_the_benchmark_launches_is_inside_its_buffer(walker):
                  "fused rows 40 groups x 8, 3-bit", "fused rows 40 groups x 8, 4-bit",
                  "fused rows 1 groups x 8, 3-bit", "split phases 40 groups x 8, 4-bit",
                  "fused (counters) 40 groups x 8, 4-bit", "gguf stream gate/up Q4_K 40 groups x 8",
-                 "gguf stream down Q6_K 40 groups x 8", "gguf stream down Q6_K 8 groups x 8"):
+                 "gguf stream down Q6_K 40 groups x 8", "gguf stream down Q6_K 8 groups x 8",
+                 "fused rows, sweep of shapes"):
         assert ("ok  " + case) in r.stdout or ("ok  dense " + case) in r.stdout, case
 
 
 def test_the_walk_notices_a_wrong_split(walker, tmp_path):
-    """The same program with one index function broken on purpose (the first unit of every part that
-    lies in layer 1 shifted by one: a gap, an overlap and a row step past the expert's last) must
+    """The same program with one index function broken on purpose (the first unit of a workgroup's
+    second segment shifted by one: a gap, an overlap and a row step past the expert's last) must
     fail: a check that cannot fail proves nothing."""
     hdr = open(os.path.join(ROOT, "finchmoe_amd", "csrc", "fm_index.h")).read()
-    needle = "*first = u0 + step * i_lo - lo;"
+    needle = "p.first = lo - p.seg * segu;"
     assert needle in hdr
     bad_dir = tmp_path / "finchmoe_amd" / "csrc"
     bad_dir.mkdir(parents=True)
-    (bad_dir / "fm_index.h").write_text(hdr.replace(needle, "*first = u0 + step * i_lo - lo + (l == 1u);"))
+    (bad_dir / "fm_index.h").write_text(hdr.replace(needle, "p.first = lo - p.seg * segu + (qq == 1);"))
     tdir = tmp_path / "tests" / "host_bounds"
     tdir.mkdir(parents=True)
     (tdir / "bounds_main.cpp").write_text(open(SRC).read())
