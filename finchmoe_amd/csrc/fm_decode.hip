@@ -860,6 +860,7 @@ struct Fm2Stream {
     uint32_t ring0, img0, part0;
     Fm2Seg *tab;
     uint32_t gu_upp, dn_upp;
+    FmDiv by_gu_upp, by_K;
     int n_up, n_seq;
     uint32_t gu_wstep, gu_sstep, dn_wstep, dn_sstep;
     // loader's phase (plain members assigned at the phase change, see FmOperatorStream)
@@ -912,8 +913,8 @@ struct Fm2Stream {
         l_first = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta));
         l_n = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + 4));
         if (!l_gu) {
-            l_nrb = l_n / (uint32_t)a.K;
-            l_first = l_first / (uint32_t)a.K;          // first row block of the part
+            l_nrb = fm_div(by_K, l_n);
+            l_first = fm_div(by_K, l_first);            // first row block of the part
             l_inv = 1.0f / (float)(l_nrb ? l_nrb : 1u);
         }
     }
@@ -934,7 +935,7 @@ struct Fm2Stream {
                 return;
             }
             uint32_t pn;
-            if (l_gu) fm2_gu_unit(l_first, ul, gu_upp, &pn, &rsn);
+            if (l_gu) fm2_gu_unit(l_first, ul, by_gu_upp, &pn, &rsn);
             else fm2_dn_unit(l_first, l_nrb, l_inv, ul, &pn, &rsn);     // expert by expert
             tag_n = ((uint32_t)(lq & 1) << 31) | (pn << 28) | ul;
             const uint32_t ba = fm_lds_addr(&tab[lq].blob[pn]);
@@ -994,9 +995,9 @@ struct Fm2Stream {
 #pragma unroll
         for (int k = 0; k < FM_MAX_K; k++)
             wk[k] = k < K ? __uint_as_float(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, w) + 4u * k)) : 0.0f;
-        const int rows = (int)(n / (uint32_t)K) * RPS_DN;
+        const int rows = (int)fm_div(by_K, n) * RPS_DN;
         const int l = seg_layer(q);
-        float *out = a.out + (size_t)l * a.g.hidden + (size_t)(first / (uint32_t)K) * RPS_DN;
+        float *out = a.out + (size_t)l * a.g.hidden + (size_t)fm_div(by_K, first) * RPS_DN;
         for (int r = threadIdx.x; r < rows; r += FM_NW * 64) {
             const int rbi = r / RPS_DN, ris = r - rbi * RPS_DN;
             float acc = 0.0f;
@@ -1008,8 +1009,9 @@ struct Fm2Stream {
         }
     }
 
-    __device__ __forceinline__ void run(int n_pairs) {
-        const int K = a.K, n_groups = n_pairs / K, G = gridDim.x, g = blockIdx.x;
+    // dm: the launch's dimensions with their divisions prepared (fm2_dims on the host)
+    __device__ __forceinline__ void run(const Fm2Dims &dm) {
+        const int K = a.K, G = gridDim.x, g = blockIdx.x;
         // The split.  Down: a workgroup's row blocks lie in ONE layer whenever there are at
         // least as many workgroups as layers (layer l gets the workgroups g with g*L/G == l, its
         // row blocks divided evenly among them), so the down phase has one segment and no
@@ -1017,7 +1019,7 @@ struct Fm2Stream {
         // ranges sized so that gate/up + down bytes are the same for every workgroup (a
         // workgroup with fewer down rows takes more gate/up units).
         // (32-bit arithmetic: the launcher checks that slices x workgroups stays below 2^31)
-        const Fm2Dims dm = fm2_dims(n_pairs, K, G, a.g.inter, a.g.hidden, LPR_UP);
+        by_gu_upp = dm.by_gu_upp, by_K = dm.by_K;
         const Fm2Split sp = fm2_split(dm, (uint32_t)g);
         const uint32_t gu_segu = dm.gu_segu;
         const int gu_s0 = sp.gu_s0;
@@ -1150,7 +1152,7 @@ struct Fm2Stream {
                 fm_wg_barrier();
                 const uint32_t ta = fm_lds_addr(&tab[cq]);
                 const uint32_t valid = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, valid)));
-                const uint32_t c_nrb = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, n))) / (uint32_t)K;
+                const uint32_t c_nrb = fm_div(by_K, __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(Fm2Seg, n))));
                 FmActRegs ar;
                 uint32_t k_cur = 0xFFFFFFFFu;
                 dry = false;
@@ -1180,9 +1182,9 @@ struct Fm2Stream {
 
 template <int BITS, int LPR_UP, bool FP16>
 __global__ __launch_bounds__(FM_NW * 64)
-void fm_moe_fused_rows(DecodeArgs a, int n_pairs, Fm2Sync sy) {
+void fm_moe_fused_rows(DecodeArgs a, Fm2Dims dm, Fm2Sync sy) {
     Fm2Stream<BITS, LPR_UP, FP16> st(a, sy);
-    st.run(n_pairs);
+    st.run(dm);
 }
 
 // fills n words with v (counters to zero, activations to FM_ACT_EMPTY)
@@ -1268,7 +1270,8 @@ int launch_fused_rows(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st
     const Fm2Plan plan = fm2_plan(n_pairs, a.K, a.g.inter, a.g.hidden, LPR_UP, n_cu);
     if (!plan.ok) return FM_ERR_UNSUPPORTED;
     const long wgs = plan.wgs;
-    hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(FM_NW * 64), sh, st, a, n_pairs, sy);
+    const Fm2Dims dm = fm2_dims(n_pairs, a.K, (int)wgs, a.g.inter, a.g.hidden, LPR_UP);
+    hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(FM_NW * 64), sh, st, a, dm, sy);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 

@@ -356,15 +356,44 @@ FM_HD long fm1_fused_wgs(long up_units, long down_units, int n_cu) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// u / d for u < 2^31 without the division sequence: with l = ceil(log2 d),
+// mul = ceil(2^(31 + l) / d) fits 32 bits and floor(u * mul / 2^(31 + l)) is exact.
+struct FmDiv {
+    uint32_t mul, shift, d;
+};
+FM_HD FmDiv fm_div_make(uint32_t d) {
+    FmDiv r;
+    r.mul = 0u, r.shift = 0u, r.d = d;
+    if (d > 1u) {
+        uint32_t l = 0;
+        while ((1ull << l) < d) l++;
+        r.mul = (uint32_t)(((1ull << (31 + l)) + d - 1) / d);
+        r.shift = l - 1;
+    }
+    return r;
+}
+FM_HD uint32_t fm_div(const FmDiv &v, uint32_t u) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return v.d == 1u ? u : __umulhi(u, v.mul) >> v.shift;
+#else
+    return v.d == 1u ? u : (uint32_t)(((uint64_t)u * v.mul) >> 32) >> v.shift;
+#endif
+}
+// ---------------------------------------------------------------------------------------------
 // routed-expert decode, the launch that sums the experts in LDS (fm_moe_fused_rows)
 // ---------------------------------------------------------------------------------------------
 #define FM2_MAX_SEG 12          // segments of one workgroup's shares
 #define FM2_PART_BYTES 12288    // partial vectors of a part
+// The launcher works these out on the host and hands them to the kernel by value: the divisions a
+// workgroup needs for its split are then multiplications (seventeen division sequences on eight
+// waves were 1.4 us in front of the first load).
 struct Fm2Dims {
     uint32_t K, G, L;           // slots, workgroups, layer groups
     uint32_t gu_upp, dn_upp;    // gate/up units per pair, down row blocks per layer
     uint32_t gu_segu, dn_segu;  // units per segment: a layer's K experts
     uint32_t gu_total, rb_total, s_total;
+    uint32_t wq;                // G / L: a layer has wq or wq + 1 workgroups (G >= L)
+    FmDiv by_G, by_L, by_K, by_gu_upp, by_gu_segu, by_dn_segu, by_wq, by_wq1;
 };
 FM_HD Fm2Dims fm2_dims(int n_pairs, int K, int G, int inter, int hidden, int lpr_up) {
     Fm2Dims d;
@@ -377,21 +406,28 @@ FM_HD Fm2Dims fm2_dims(int n_pairs, int K, int G, int inter, int hidden, int lpr
     d.gu_total = (uint32_t)n_pairs * d.gu_upp;
     d.rb_total = d.L * d.dn_upp;
     d.s_total = 2u * d.gu_total + d.rb_total * d.K;
+    d.wq = d.L ? d.G / d.L : 0u;
+    d.by_G = fm_div_make(d.G), d.by_L = fm_div_make(d.L ? d.L : 1u), d.by_K = fm_div_make(d.K);
+    d.by_gu_upp = fm_div_make(d.gu_upp ? d.gu_upp : 1u);
+    d.by_gu_segu = fm_div_make(d.gu_segu ? d.gu_segu : 1u), d.by_dn_segu = fm_div_make(d.dn_segu ? d.dn_segu : 1u);
+    d.by_wq = fm_div_make(d.wq ? d.wq : 1u), d.by_wq1 = fm_div_make(d.wq + 1u);
     return d;
 }
 // first down row block of workgroup gg: a workgroup's row blocks lie in ONE layer whenever there
 // are at least as many workgroups as layers
 FM_HD uint32_t fm2_dn_start(const Fm2Dims &d, uint32_t gg) {
     if (gg >= d.G) return d.rb_total;
-    if (d.G < d.L) return d.rb_total * gg / d.G;
-    const uint32_t l = gg * d.L / d.G;
-    const uint32_t g_lo = (l * d.G + d.L - 1u) / d.L, g_hi = ((l + 1u) * d.G + d.L - 1u) / d.L;
-    return l * d.dn_upp + d.dn_upp * (gg - g_lo) / (g_hi - g_lo);
+    if (d.G < d.L) return fm_div(d.by_G, d.rb_total * gg);
+    const uint32_t l = fm_div(d.by_G, gg * d.L);
+    const uint32_t g_lo = fm_div(d.by_L, l * d.G + d.L - 1u), g_hi = fm_div(d.by_L, (l + 1u) * d.G + d.L - 1u);
+    // the layer's workgroups: wq or wq + 1 of them
+    const uint32_t n = g_hi - g_lo, v = d.dn_upp * (gg - g_lo);
+    return l * d.dn_upp + (n == d.wq ? fm_div(d.by_wq, v) : fm_div(d.by_wq1, v));
 }
 // first gate/up unit of workgroup gg (dn0 = its first down row block): sized so that gate/up +
 // down slices are the same for every workgroup
 FM_HD uint32_t fm2_gu_start(const Fm2Dims &d, uint32_t gg, uint32_t dn0) {
-    const uint32_t t = d.s_total * gg / d.G, dd = dn0 * d.K;
+    const uint32_t t = fm_div(d.by_G, d.s_total * gg), dd = dn0 * d.K;
     const uint32_t u = t > dd ? (t - dd) / 2u : 0u;
     return u > d.gu_total ? d.gu_total : u;
 }
@@ -406,10 +442,10 @@ FM_HD Fm2Split fm2_split(const Fm2Dims &d, uint32_t g) {
     s.gu_wg1 = fm2_gu_start(d, g + 1u, dn_rb1);
     s.dn_wg0 = dn_rb0 * d.K;
     s.dn_wg1 = dn_rb1 * d.K;
-    s.gu_s0 = (int)(s.gu_wg0 / d.gu_segu);
-    s.dn_s0 = (int)(s.dn_wg0 / d.dn_segu);
-    s.n_up = s.gu_wg1 > s.gu_wg0 ? (int)((s.gu_wg1 - 1u) / d.gu_segu) + 1 - s.gu_s0 : 0;
-    s.n_dn = s.dn_wg1 > s.dn_wg0 ? (int)((s.dn_wg1 - 1u) / d.dn_segu) + 1 - s.dn_s0 : 0;
+    s.gu_s0 = (int)fm_div(d.by_gu_segu, s.gu_wg0);
+    s.dn_s0 = (int)fm_div(d.by_dn_segu, s.dn_wg0);
+    s.n_up = s.gu_wg1 > s.gu_wg0 ? (int)fm_div(d.by_gu_segu, s.gu_wg1 - 1u) + 1 - s.gu_s0 : 0;
+    s.n_dn = s.dn_wg1 > s.dn_wg0 ? (int)fm_div(d.by_dn_segu, s.dn_wg1 - 1u) + 1 - s.dn_s0 : 0;
     return s;
 }
 // segment qq of the workgroup's sequence (gate/up segments first): layer group, first unit inside
@@ -431,10 +467,10 @@ FM_HD Fm2Part fm2_part(const Fm2Dims &d, const Fm2Split &s, int qq) {
     return p;
 }
 // claimed unit ul of a gate/up part: slot pn of the layer and row step rsn of its expert
-FM_HD void fm2_gu_unit(uint32_t first, uint32_t ul, uint32_t gu_upp, uint32_t *pn, uint32_t *rsn) {
+FM_HD void fm2_gu_unit(uint32_t first, uint32_t ul, const FmDiv &by_gu_upp, uint32_t *pn, uint32_t *rsn) {
     const uint32_t uq = first + ul;
-    *pn = uq / gu_upp;
-    *rsn = uq - *pn * gu_upp;
+    *pn = fm_div(by_gu_upp, uq);
+    *rsn = uq - *pn * by_gu_upp.d;
 }
 // claimed unit ul of a down part of nrb row blocks starting at row block rb_first (expert by
 // expert: unit ul = row block ul % nrb of slot ul / nrb); inv = 1 / nrb in fp32
@@ -481,29 +517,6 @@ FM_HD Fm2Plan fm2_plan(int n_pairs, int K, int inter, int hidden, int lpr_up, in
 // ---------------------------------------------------------------------------------------------
 // GGUF experts, streaming kernels (fm_gguf_stream)
 // ---------------------------------------------------------------------------------------------
-// u / d for u < 2^31 without the division sequence: with l = ceil(log2 d),
-// mul = ceil(2^(31 + l) / d) fits 32 bits and floor(u * mul / 2^(31 + l)) is exact.
-struct FmDiv {
-    uint32_t mul, shift, d;
-};
-FM_HD FmDiv fm_div_make(uint32_t d) {
-    FmDiv r;
-    r.mul = 0u, r.shift = 0u, r.d = d;
-    if (d > 1u) {
-        uint32_t l = 0;
-        while ((1ull << l) < d) l++;
-        r.mul = (uint32_t)(((1ull << (31 + l)) + d - 1) / d);
-        r.shift = l - 1;
-    }
-    return r;
-}
-FM_HD uint32_t fm_div(const FmDiv &v, uint32_t u) {
-#if defined(__HIP_DEVICE_COMPILE__)
-    return v.d == 1u ? u : __umulhi(u, v.mul) >> v.shift;
-#else
-    return v.d == 1u ? u : (uint32_t)(((uint64_t)u * v.mul) >> 32) >> v.shift;
-#endif
-}
 struct FmGgPlan {
     int ok, lpr, rps, upp, wgs;
     long total;

@@ -390,6 +390,24 @@ static void walk_fused_rows(int n_groups, int K, int hidden, int inter, int bits
     Region X("x", (size_t)n_groups * hidden * 4), idx("idx", (size_t)n_pairs * 4);
     int max_seq = 0;
     size_t max_bytes = 0, min_bytes = (size_t)-1;
+    for (int gi = 0; gi <= G; gi++) {
+        // the prepared divisions against plain ones
+        const uint32_t ug = (uint32_t)gi;
+        uint32_t dn_ref;
+        if (ug >= dm.G) dn_ref = dm.rb_total;
+        else if (dm.G < dm.L) dn_ref = dm.rb_total * ug / dm.G;
+        else {
+            const uint32_t l = ug * dm.L / dm.G;
+            const uint32_t g_lo = (l * dm.G + dm.L - 1u) / dm.L, g_hi = ((l + 1u) * dm.G + dm.L - 1u) / dm.L;
+            CHECK(g_hi - g_lo == dm.wq || g_hi - g_lo == dm.wq + 1u, "layer %u has %u workgroups", l, g_hi - g_lo);
+            dn_ref = l * dm.dn_upp + dm.dn_upp * (ug - g_lo) / (g_hi - g_lo);
+        }
+        CHECK(fm2_dn_start(dm, ug) == dn_ref, "first down row block of workgroup %d", gi);
+        const uint32_t t = dm.s_total * ug / dm.G, dd = dn_ref * dm.K;
+        uint32_t gu_ref = t > dd ? (t - dd) / 2u : 0u;
+        if (gu_ref > dm.gu_total) gu_ref = dm.gu_total;
+        CHECK(fm2_gu_start(dm, ug, dn_ref) == gu_ref, "first gate/up unit of workgroup %d", gi);
+    }
     for (int gi = 0; gi < G; gi++) {
         const Fm2Split sp = fm2_split(dm, gi);
         const int n_seq = sp.n_up + sp.n_dn;
@@ -407,7 +425,7 @@ static void walk_fused_rows(int n_groups, int K, int hidden, int inter, int bits
             if (pt.gu) {
                 for (uint32_t ul = 0; ul < pt.n; ul++) {
                     uint32_t pn, rsn;
-                    fm2_gu_unit(pt.first, ul, dm.gu_upp, &pn, &rsn);
+                    fm2_gu_unit(pt.first, ul, dm.by_gu_upp, &pn, &rsn);
                     CHECK(pn < (uint32_t)K && rsn < dm.gu_upp, "gate/up unit %u -> slot %u step %u", ul, pn, rsn);
                     if (pn >= (uint32_t)K) continue;
                     Region &bl = blob[pt.seg * K + pn];
