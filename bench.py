@@ -32,7 +32,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 peak
 # --pmc FETCH_SIZE (x2: calibrated against a 1 GiB copy) + WRITE_SIZE.  An OFFLINE constant
 # (hardware counters cannot be read from inside this process): the JSON line names the file
 # it comes from in roofline.traffic_source, and it is null for any other size.
-FUSED_TRAFFIC_BYTES_40L = int((218733.97 * 2 + 2237.57) * 1024)
+FUSED_TRAFFIC_BYTES_40L = int((218685.2 * 2 + 2237.6) * 1024)
 FUSED_TRAFFIC_SOURCE = "offline constant from profiles/decode_step_3bit_hbm_traffic.md (rocprofv3 --pmc), not measured in this run"
 
 H, I, E, K, L = 2048, 512, 256, 8, 40
