@@ -28,6 +28,8 @@ int fm_launch_dense_mixed(FmDenseSpec *specs, int n, int in_dim, int scale_fp16,
                           int n_cu, const RouteArgs *route, unsigned int *ticket, hipStream_t st);
 int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim, const float *d_x, int M,
                          hipStream_t st);
+int fm_launch_dense_lowbit(const FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
+                           const float *d_x, int M, hipStream_t st);
 int fm_launch_stream_probe(const void *d_buf, size_t nbytes, int pattern, unsigned int *d_sink,
                            int n_cu, hipStream_t st);
 int fm_launch_dequant_affine(const void *W, const void *S, const void *B, int out_dim,
@@ -869,12 +871,15 @@ static int tensor_add(fm_ctx *c, const void *W, const void *S, const void *B, in
     if (!raw && !gguf) {
         if (bits == 0) bits = 4;   // BatchMatvecSpec default, finchmoe/infer.m:4491
         if (group_size != 64) return fail(c, FM_ERR_UNSUPPORTED, "group_size %d (only 64)", group_size);
-        if (bits != 3 && bits != 4 && bits != 8)
-            return fail(c, FM_ERR_UNSUPPORTED, "tensor bits %d (3, 4 or 8)", bits);
+        if (bits != 1 && bits != 2 && bits != 3 && bits != 4 && bits != 8)
+            return fail(c, FM_ERR_UNSUPPORTED, "tensor bits %d (1, 2, 3, 4 or 8)", bits);
         if (scale_dtype != FM_SCALE_BF16 && scale_dtype != FM_SCALE_FP16)
             return fail(c, FM_ERR_ARG, "scale_dtype %d", scale_dtype);
         int lpr = in_dim / 128;
-        if (in_dim % 128 || !pow2(lpr) || lpr > 64)
+        if (bits <= 2) {         // the legacy widths: a kernel of their own, any multiple of a group
+            if (in_dim % 64 || in_dim > 16384)
+                return fail(c, FM_ERR_UNSUPPORTED, "in_dim %d: need a multiple of 64 up to 16384", in_dim);
+        } else if (in_dim % 128 || !pow2(lpr) || lpr > 64)
             return fail(c, FM_ERR_UNSUPPORTED, "in_dim %d: need 128*2^j, j<=6", in_dim);
     }
     DeviceGuard dg(c->device);
@@ -1031,7 +1036,7 @@ static int matvec_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
         // (the b / a rows behind qkv / z, finchmoe/infer.m:8118-8122)
         FmDenseSpec riders[2];
         int n_riders = 0, riders_done = 0;
-        if (!t0->raw_bf16()) {
+        if (!t0->raw_bf16() && t0->bits > 2) {
             for (int k = i; k < n && n_riders < 2; k++) {
                 Tensor *t = get_tensor(c, ts[k]);
                 if (!t || !t->raw_bf16() || t->in_dim != t0->in_dim || !d_outs[k]) break;
@@ -1046,6 +1051,8 @@ static int matvec_dev(fm_ctx *c, const fm_tensor *ts, int n, const float *d_x,
         }
         int rc = t0->raw_bf16()
                      ? fm_launch_dense_bf16(specs, m, t0->in_dim, d_x, M, c->stream)
+                 : t0->bits <= 2
+                     ? fm_launch_dense_lowbit(specs, m, t0->in_dim, t0->bits, t0->scale_fp16, d_x, M, c->stream)
                      : fm_launch_dense(specs, m, t0->in_dim, t0->bits, t0->scale_fp16, d_x, M,
                                        c->n_cu, c->stream, n_riders ? riders : nullptr, n_riders,
                                        &riders_done);
@@ -1244,7 +1251,7 @@ extern "C" int fm_layer_tail_dev(fm_ctx *c, fm_tensor shared_down, const float *
         return fail(c, FM_ERR_ARG, "next input and its norm weights go together");
     if (((uintptr_t)d_shared_gate | (uintptr_t)d_shared_up) & 3)
         return fail(c, FM_ERR_ARG, "vector not 4-byte aligned");
-    if (t->raw_bf16() || t->gguf() || t->group_size != 64)
+    if (t->raw_bf16() || t->gguf() || t->bits <= 2 || t->group_size != 64)
         return fail(c, FM_ERR_UNSUPPORTED, "shared down projection must be 3/4/8-bit, group size 64");
     if (t->out_dim / 4 > FM_TAIL_PARTIALS) return fail(c, FM_ERR_UNSUPPORTED, "hidden %d", t->out_dim);
     DeviceGuard dg(c->device);

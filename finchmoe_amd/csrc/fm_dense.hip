@@ -441,7 +441,83 @@ __global__ __launch_bounds__(256) void fm_dense_bf16(FmDenseArgs a, int total_ro
     if (lane == 0) sp.out[(size_t)m * sp.out_dim + row] = acc;
 }
 
+// ----------------------------------------------------------------------
+// 1- and 2-bit affine tensors (cpu_dequant_matvec's generic branch, finchmoe/infer.m:1734-1760:
+// 32 / 16 codes per little-endian u32, LSB first; the legacy widths of the reference's tensor
+// boundary, in none of its benchmark configurations).  One wave per row: a lane takes whole
+// words (a word never straddles a group of 64), per word s * sum(q x) + b * sum(x) in fp32, sum
+// over the wave.
+// ----------------------------------------------------------------------
+template <int BITS, bool FP16>
+__global__ __launch_bounds__(256) void fm_dense_lowbit(FmDenseArgs a, int total_rows) {
+    constexpr int VPU = 32 / BITS;
+    const int lane = threadIdx.x & 63;
+    const int gr = blockIdx.x * 4 + (threadIdx.x >> 6);   // row of the launch (wave-uniform)
+    if (gr >= total_rows) return;
+    int t = 0;
+#pragma unroll
+    for (int i = 1; i < FM_MAX_BATCH; i++)
+        if (i < a.n && gr >= a.unit_first[i]) t = i;
+    const FmDenseSpec sp = a.spec[t];
+    const int row = gr - a.unit_first[t];
+    const int m = blockIdx.y;
+    const int words = a.in_dim / VPU, ng = a.in_dim / 64;
+    const uint32_t *w = reinterpret_cast<const uint32_t *>(sp.W) + (size_t)row * words;
+    const uint16_t *S = reinterpret_cast<const uint16_t *>(sp.S) + (size_t)row * ng;
+    const uint16_t *B = reinterpret_cast<const uint16_t *>(sp.B) + (size_t)row * ng;
+    const float *x = a.x + (size_t)m * a.in_dim;
+    float acc = 0.0f;
+    for (int wi = lane; wi < words; wi += 64) {
+        const uint32_t q = w[wi];
+        const int col0 = wi * VPU, g = col0 >> 6;
+        const float sc = FP16 ? fm_fp16_bits(S[g]) : fm_bf16_lo(S[g]);
+        const float bs = FP16 ? fm_fp16_bits(B[g]) : fm_bf16_lo(B[g]);
+        float dq = 0.0f, dx = 0.0f;
+#pragma unroll
+        for (int j = 0; j < VPU; j++) {
+            const float xv = x[col0 + j];
+            dq = fmaf((float)((q >> (j * BITS)) & ((1u << BITS) - 1u)), xv, dq);
+            dx += xv;
+        }
+        acc = fmaf(sc, dq, fmaf(bs, dx, acc));
+    }
+    acc = fm_group_sum<64>(acc);
+    if (lane == 0) sp.out[(size_t)m * sp.out_dim + row] = acc;
+}
+
 }  // namespace
+
+// n 1- or 2-bit affine tensors [out_dim][in_dim] (in_dim a multiple of 64) sharing x[M][in_dim]
+extern "C" int fm_launch_dense_lowbit(const FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
+                                      const float *d_x, int M, hipStream_t st) {
+    if (n < 1 || n > FM_MAX_BATCH || M < 1 || in_dim < 64 || in_dim % 64 || (bits != 1 && bits != 2))
+        return FM_ERR_ARG;
+    FmDenseArgs a;
+    a.n = n;
+    a.in_dim = in_dim;
+    a.rows_per_item = 0;
+    a.x = d_x;
+    a.out_stride = 0;
+    a.route_on = 0;
+    a.n_riders = 0;
+    int rows = 0;
+    for (int i = 0; i < n; i++) {
+        a.spec[i] = specs[i];
+        a.unit_first[i] = rows;
+        rows += specs[i].out_dim;
+    }
+    for (int i = n; i < FM_MAX_BATCH; i++) a.spec[i] = a.spec[0];
+    for (int i = n; i <= FM_MAX_BATCH; i++) a.unit_first[i] = rows;
+    const dim3 grid((rows + 3) / 4, M);
+    if (bits == 1) {
+        if (scale_fp16) hipLaunchKernelGGL((fm_dense_lowbit<1, true>), grid, dim3(256), 0, st, a, rows);
+        else hipLaunchKernelGGL((fm_dense_lowbit<1, false>), grid, dim3(256), 0, st, a, rows);
+    } else {
+        if (scale_fp16) hipLaunchKernelGGL((fm_dense_lowbit<2, true>), grid, dim3(256), 0, st, a, rows);
+        else hipLaunchKernelGGL((fm_dense_lowbit<2, false>), grid, dim3(256), 0, st, a, rows);
+    }
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
 
 // n raw-BF16 tensors [out_dim][in_dim] sharing x[M][in_dim]; specs[i].S / .B are unused.
 extern "C" int fm_launch_dense_bf16(const FmDenseSpec *specs, int n, int in_dim, const float *d_x,

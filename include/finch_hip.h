@@ -194,8 +194,11 @@ FM_API int fm_moe_prefill_bf16(fm_ctx *ctx, int layer, const uint16_t *X, const 
  * Replaces fast_dequant_matvec / BatchMatvecSpec + fast_batch_matvec /
  * gpu_encode_prefill_matvec (finchmoe/infer.m:3369, 3401-3411, 4477, 3672;
  * kernels dequant_matvec_4bit_v3 and _prefill, shaders.metal:374-463, 2460-2529).
- * W: u32 [out_dim][in_dim*bits/32] (bits 4 or 8) or bytes [out_dim][in_dim*3/8]
- * (bits 3); S, B: 16-bit [out_dim][in_dim/group_size].
+ * W: u32 [out_dim][in_dim*bits/32] (bits 1, 2, 4 or 8; LSB first) or bytes
+ * [out_dim][in_dim*3/8] (bits 3); S, B: 16-bit [out_dim][in_dim/group_size].  in_dim:
+ * 128 * 2^j up to 8192 for bits 3, 4, 8; any multiple of 64 up to 16384 for the legacy widths
+ * 1 and 2 (cpu_dequant_matvec's generic branch, finchmoe/infer.m:1734-1760), which run a plain
+ * kernel of their own and are not accepted by fm_layer_tail_dev.
  * S == NULL or B == NULL: an unquantized BF16 tensor [out_dim][in_dim] (cpu_dequant_matvec's
  * raw branch, finchmoe/infer.m:1689-1701).
  * bits 10 / 11 (the reference's own codes, finchmoe/infer.m:1684-1688, 3378-3388): a GGUF Q4_K /

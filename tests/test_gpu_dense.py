@@ -37,10 +37,12 @@ def test_gdn_projections_4bit(hip, orc):
 
 @pytest.mark.parametrize("bits,dtype,out_dim,in_dim", [
     (4, "bf16", 32, 2048), (4, "fp16", 100, 512), (8, "bf16", 256, 2048), (3, "bf16", 77, 1024),
-    (4, "bf16", 5, 128), (8, "fp16", 33, 256), (4, "bf16", 64, 8192)])
+    (4, "bf16", 5, 128), (8, "fp16", 33, 256), (4, "bf16", 64, 8192),
+    (2, "bf16", 77, 1024), (2, "fp16", 100, 4096), (1, "bf16", 33, 192), (1, "fp16", 256, 2048), (2, "bf16", 3, 64)])
 def test_matvec_shapes_and_widths(hip, orc, bits, dtype, out_dim, in_dim):
-    """Ragged out_dim, small and large in_dim, every packing width, both scale types;
-    codes and weights bit-exact, outputs within tolerance."""
+    """Ragged out_dim, small and large in_dim, every packing width (the legacy 1- and 2-bit
+    widths of cpu_dequant_matvec, infer.m:1734, included), both scale types; codes and weights
+    bit-exact, outputs within tolerance."""
     rng = np.random.default_rng(out_dim * 31 + in_dim + bits)
     t, (codes, W, S, B, sd) = _tensor(hip, rng, out_dim, in_dim, bits, dtype)
     gc, gw, gh = hip.dequant_tensor(t, out_dim, in_dim)
@@ -91,6 +93,29 @@ def test_matvec_prefill_positions(hip, orc):
         assert np.array_equal(out[m], single)
         assert_parity(out[m], orc.dequant_matvec(W, S, B, X[m], 512, 2048, 4), "pos %d" % m)
     hip.tensor_release(t)
+
+
+def test_low_widths_in_a_batch_and_over_positions(hip, orc):
+    """2-bit tensors in one batch with a 4-bit one (separate launches, one call), and a 1-bit
+    tensor against several positions: each position equals the single call bitwise."""
+    rng = np.random.default_rng(40)
+    t2a, a = _tensor(hip, rng, 96, 1024, 2)
+    t2b, b = _tensor(hip, rng, 40, 1024, 2)
+    t4, c4 = _tensor(hip, rng, 64, 1024, 4)
+    x = rng.standard_normal(1024).astype(np.float32)
+    oa, ob, o4 = hip.matvec_batch([t2a, t2b, t4], x, [96, 40, 64])
+    assert_parity(oa, orc.dequant_matvec(a[1], a[2], a[3], x, 96, 1024, 2), "2-bit a")
+    assert_parity(ob, orc.dequant_matvec(b[1], b[2], b[3], x, 40, 1024, 2), "2-bit b")
+    assert_parity(o4, orc.dequant_matvec(c4[1], c4[2], c4[3], x, 64, 1024, 4), "4-bit")
+    t1, d = _tensor(hip, rng, 50, 512, 1)
+    X = rng.standard_normal((20, 512)).astype(np.float32)
+    out = hip.matvec_prefill(t1, X, 50)
+    for m in (0, 7, 19):
+        (one,) = hip.matvec_batch([t1], X[m], [50])
+        assert np.array_equal(out[m], one)
+        assert_parity(out[m], orc.dequant_matvec(d[1], d[2], d[3], X[m], 50, 512, 1), "1-bit position %d" % m)
+    for t in (t2a, t2b, t4, t1):
+        hip.tensor_release(t)
 
 
 def test_mixed_batch_and_errors(hip, orc):
