@@ -838,8 +838,9 @@ def run_gguf(args):
     if args.workload == "gguf_chunk":
         # the chunked-prefill variant of config 4: M positions of one layer per call (grouped
         # products from 32 positions on, per-position products below, as the reference runs
-        # them; FINCH_GGUF_NO_GROUP=1 forces the latter), the layer changes from call to call
+        # them; --forms per-position forces the latter), the layer changes from call to call
         M = args.chunk if args.chunk <= tokens else 8
+        per_position = "per-position" in args.forms
         c_idx = torch.from_numpy(np.ascontiguousarray(idx.transpose(1, 0, 2))).to(dev)   # [layer][token][k]
         c_w = torch.from_numpy(np.ascontiguousarray(w.transpose(1, 0, 2))).to(dev)
         c_x = torch.randn(M, H, device=dev)
@@ -854,7 +855,7 @@ def run_gguf(args):
 
         ms, ev = _timed(ctx, cstep, args)
         assert torch.isfinite(c_out).all()
-        grouped = M >= 32 and not os.environ.get("FINCH_GGUF_NO_GROUP")
+        grouped = M >= 32 and not per_position
         # grouped products read an expert once per group of its positions: priced on the distinct
         # experts of a chunk; per-position products stream every routed expert once per position
         uniq = float(np.mean([len(set(idx[:M, l].reshape(-1).tolist())) for l in range(n_layers)]))
@@ -875,7 +876,7 @@ def run_gguf(args):
         return _finish(cres,
                        "GGUF Q4_K/Q6_K expert GEMV HBM GB/s, %d-position chunk of one layer" % M,
                        "config 4, chunk variant: %d positions x top-8 Zipf(1.1) on one of %d GGUF layers "
-                       "(Q4_K gate/up, Q6_K down), %s products" % (M, n_layers, "grouped" if M >= 32 and not os.environ.get("FINCH_GGUF_NO_GROUP") else "per-position"),
+                       "(Q4_K gate/up, Q6_K down), %s products" % (M, n_layers, "grouped" if M >= 32 and not per_position else "per-position"),
                        M * K * (2 * gsl + dsl), ms, args)
     d_idx, d_w = torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)
     d_x = torch.randn(n_layers, H, device=dev)
@@ -1073,6 +1074,9 @@ def main():
                          "(profile buckets: all items full / all items small)")
     ap.add_argument("--lm-format", default="affine8", choices=("affine8", "q4k", "q6k"),
                     help="lm_head workload: 8-bit affine, or the GGUF block formats")
+    ap.add_argument("--forms", default="", help="comma-separated overrides of the library's kernel choice for A/B "
+                    "runs: plain-dense, plain-gguf (the non-streaming kernels), per-position (no dense GEMM, "
+                    "no grouped GGUF products for chunks)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
@@ -1106,7 +1110,23 @@ def main():
     print("bench.py: workload=%s chunk=%d bits=%d scale_dtype=%s x_dtype=%s steps=%d warmup=%d graph=%s"
           % (args.workload, args.chunk, args.bits, args.scale_dtype, args.x_dtype, args.steps, args.warmup,
              bool(args.graph)), file=sys.stderr, flush=True)
+    args.forms = [f for f in args.forms.split(",") if f]
+    if args.forms:
+        from finchmoe_amd import binding as fb
+        known = {"plain-dense": fb.FORM_PLAIN_DENSE, "plain-gguf": fb.FORM_PLAIN_GGUF,
+                 "per-position": fb.FORM_NO_DENSE_GEMM | fb.FORM_NO_GGUF_GROUP}
+        bad = [f for f in args.forms if f not in known]
+        if bad:
+            print("bench.py: unknown --forms %s (have: %s)" % (bad, ", ".join(known)), file=sys.stderr)
+            sys.exit(2)
+        flags = 0
+        for f in args.forms:
+            flags |= known[f]
+        rc = fb.load().fm_set_kernel_forms(flags)
+        assert rc == 0, rc
     res = runners[args.workload](args)
+    if args.forms:
+        res.setdefault("config", {})["kernel_forms"] = args.forms
     print(json.dumps(res))
 
 

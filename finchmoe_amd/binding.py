@@ -13,6 +13,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
 OK, ERR_ARG, ERR_HIP, ERR_STATE, ERR_UNSUPPORTED, ERR_NOMEM = 0, -1, -2, -3, -4, -5
+FORM_PLAIN_DENSE, FORM_PLAIN_GGUF, FORM_NO_DENSE_GEMM, FORM_NO_GGUF_GROUP = 1, 2, 4, 8
 SCALE_BF16, SCALE_FP16 = 0, 1
 Q4_K, Q6_K = 12, 14
 ACCUMULATE, GUARD = 1, 2
@@ -62,6 +63,7 @@ def load():
         "fm_timer_stop": (i, [vp, C.POINTER(C.c_float)]),
         "fm_kernel_timing": (i, [vp, i]),
         "fm_set_wait_limit": (i, [vp, C.c_uint]),
+        "fm_set_kernel_forms": (i, [C.c_uint]),
         "fm_reserve": (i, [vp, i, i, C.c_size_t]),
         "fm_release_graphs": (i, [vp]),
         "fm_kernel_timing_read": (i, [vp, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(i)]),
@@ -168,6 +170,10 @@ class FinchHip:
 
     def set_wait_limit(self, polls):
         self._chk(self.L.fm_set_wait_limit(self.h, C.c_uint(polls)))
+
+    def set_kernel_forms(self, forms):
+        """Process-wide override of the kernel choice (FORM_* flags; 0 = default)."""
+        self._chk(self.L.fm_set_kernel_forms(C.c_uint(forms)))
 
     def reserve(self, n_groups=0, M=0, workspace_bytes=0):
         """Scratch for steps of n_groups layers / chunks of M positions, before capturing."""

@@ -332,6 +332,15 @@ size_t gguf_row_bytes(int in_dim, int type) {
 // ============================================================================
 // context
 // ============================================================================
+unsigned int fm_kernel_forms = 0;
+
+extern "C" int fm_set_kernel_forms(unsigned int forms) {
+    if (forms & ~(unsigned)(FM_FORM_PLAIN_DENSE | FM_FORM_PLAIN_GGUF | FM_FORM_NO_DENSE_GEMM | FM_FORM_NO_GGUF_GROUP))
+        return FM_ERR_ARG;
+    fm_kernel_forms = forms;
+    return FM_OK;
+}
+
 extern "C" int fm_ctx_create(int device, fm_ctx **out) {
     if (!out) return FM_ERR_ARG;
     *out = nullptr;
@@ -1111,7 +1120,7 @@ extern "C" int fm_matvec_prefill_batch_dev(fm_ctx *c, const fm_tensor *ts, int n
     if (!ts || !d_X || !d_outs) return fail(c, FM_ERR_ARG, "null pointer");
     if (n < 1 || n > 64) return fail(c, FM_ERR_ARG, "n %d outside 1..64", n);
     if (M < 1 || M > 65535) return fail(c, FM_ERR_ARG, "M %d outside 1..65535", M);
-    static const bool no_gemm = getenv("FINCH_DENSE_NO_GEMM") != nullptr;
+    const bool no_gemm = (fm_kernel_forms & FM_FORM_NO_DENSE_GEMM) != 0;
     int prepared_bits = 0, prepared_in = 0;
     for (int i = 0; i < n; i++) {   // one X for all: the tensors must agree on its width
         Tensor *p = get_tensor(c, ts[i]), *p0 = get_tensor(c, ts[0]);
@@ -1442,7 +1451,7 @@ extern "C" int fm_gguf_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, c
                                        const float *d_w, int M, int K, float *d_out, int flags) {
     if (!c) return FM_ERR_ARG;
     if (M < 1 || M > FM_MAX_CHUNK) return fail(c, FM_ERR_ARG, "M %d outside 1..%d", M, FM_MAX_CHUNK);
-    static const bool no_group = getenv("FINCH_GGUF_NO_GROUP") != nullptr;
+    const bool no_group = (fm_kernel_forms & FM_FORM_NO_GGUF_GROUP) != 0;
     // (grouping pays from about four positions per expert on: measured at 256 experts, a chunk of
     // 64 positions is faster position by position, 152 against 179 us, one of 512 is 2.7 times
     // faster grouped)

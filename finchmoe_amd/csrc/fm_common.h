@@ -126,3 +126,7 @@ __device__ __forceinline__ float fm_silu_mul(float g, float u) {
 }
 
 #endif  // __HIPCC__
+
+// Which form of a kernel the launchers pick where two exist (fm_set_kernel_forms): 0 = the
+// default choice.  Process-wide; read by the launchers on the host only.
+extern unsigned int fm_kernel_forms;

@@ -638,7 +638,7 @@ extern "C" int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, 
         a.spec[i] = specs[i];
     }
     for (int i = n; i < FM_MAX_BATCH; i++) a.spec[i] = a.spec[0];
-    static const bool no_stream = getenv("FINCH_DENSE_VALU") != nullptr;
+    const bool no_stream = (fm_kernel_forms & FM_FORM_PLAIN_DENSE) != 0;
     if (!no_stream && (bits == 3 || bits == 4 || bits == 8)) {
         if (riders && n_riders >= 1 && n_riders <= 2 && riders_done) {
             a.n_riders = n_riders;

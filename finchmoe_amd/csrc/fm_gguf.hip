@@ -978,7 +978,7 @@ extern "C" int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t
     a2.rows_per_item = pick_rpi(g->hidden, n_pairs, min_down, 256, 4 * n_cu);
     a2.items_per_pair = g->hidden / a2.rows_per_item;
     if (kev) (void)hipEventRecord(kev[0], st);
-    static const bool no_stream = getenv("FINCH_GGUF_VALU") != nullptr;
+    const bool no_stream = (fm_kernel_forms & FM_FORM_PLAIN_GGUF) != 0;
     int rc_up = FM_ERR_UNSUPPORTED;
     if (!no_stream) rc_up = gg_launch_stream<GG_Q4, true>(a, n_pairs, n_cu, st);
     if (rc_up != FM_OK && rc_up != FM_ERR_UNSUPPORTED) return rc_up;
@@ -1062,7 +1062,7 @@ extern "C" int fm_launch_gguf_dense(const uint8_t *d_W, int ggml_type, const flo
                                     int out_dim, int in_dim, int n_cu, hipStream_t st) {
     if (ggml_type != FM_GGML_Q4_K && ggml_type != FM_GGML_Q6_K) return FM_ERR_UNSUPPORTED;
     if (out_dim < 1 || in_dim < 256 || in_dim % 256) return FM_ERR_UNSUPPORTED;
-    static const bool no_stream = getenv("FINCH_GGUF_VALU") != nullptr;
+    const bool no_stream = (fm_kernel_forms & FM_FORM_PLAIN_GGUF) != 0;
     const bool q6 = ggml_type == FM_GGML_Q6_K;
     if (!no_stream && ((uintptr_t)d_W & 15) == 0) {
         GgufArgs a{};

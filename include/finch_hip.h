@@ -100,6 +100,15 @@ FM_API int fm_kernel_timing(fm_ctx *ctx, int mode);
  * fm_sync / host-pointer call returns FM_ERR_HIP ("results are invalid").  No
  * counterpart in the reference (its kernels are separate Metal dispatches). */
 FM_API int fm_set_wait_limit(fm_ctx *ctx, unsigned int polls);
+/* Where the library has two forms of a kernel it picks one by shape.  For A/B measurements
+ * (and for callers that want the forms whose results are bitwise those of the one-position
+ * call) the choice can be overridden, process-wide; 0 restores the default.  No counterpart
+ * in the reference. */
+#define FM_FORM_PLAIN_DENSE 1u     /* dense affine GEMV: the plain kernel for every shape */
+#define FM_FORM_PLAIN_GGUF 2u      /* GGUF experts and tensors: the plain kernels for every shape */
+#define FM_FORM_NO_DENSE_GEMM 4u   /* fm_matvec_prefill*: one GEMV per position for every M */
+#define FM_FORM_NO_GGUF_GROUP 8u   /* fm_gguf_moe_prefill*: the per-position kernels for every M */
+FM_API int fm_set_kernel_forms(unsigned int forms);
 /* sums in milliseconds since the last read, and the number of calls; resets */
 /* Calls captured into a HIP graph (hipStreamBeginCapture on fm_stream()).  A graph records the
  * addresses of the context's scratch buffers, which grow on demand otherwise.  So: reserve

@@ -118,6 +118,35 @@ def test_low_widths_in_a_batch_and_over_positions(hip, orc):
         hip.tensor_release(t)
 
 
+def test_kernel_forms_override(hip, orc):
+    """fm_set_kernel_forms: the plain kernel for a shape that streams by default agrees with the
+    oracle too; with the dense GEMM switched off a 40-position call equals the one-position
+    calls bitwise; unknown flags are refused; 0 restores the default."""
+    from finchmoe_amd import FinchError
+    rng = np.random.default_rng(41)
+    t, (codes, W, S, B, sd) = _tensor(hip, rng, 8192, 2048, 4)
+    X = rng.standard_normal((40, 2048)).astype(np.float32)
+    ref = orc.dequant_matvec(W, S, B, X[0], 8192, 2048, 4, nthreads=8)
+    (dflt,) = hip.matvec_batch([t], X[0], [8192])
+    try:
+        hip.set_kernel_forms(fb.FORM_PLAIN_DENSE)
+        (plain,) = hip.matvec_batch([t], X[0], [8192])
+        assert_parity(plain, ref, "plain kernel")
+        hip.set_kernel_forms(fb.FORM_NO_DENSE_GEMM)
+        out = hip.matvec_prefill(t, X, 8192)
+        for m in (0, 17, 39):
+            (one,) = hip.matvec_batch([t], X[m], [8192])
+            assert np.array_equal(out[m], one), m
+        with pytest.raises(FinchError):
+            hip.set_kernel_forms(1 << 9)
+    finally:
+        hip.set_kernel_forms(0)
+    (again,) = hip.matvec_batch([t], X[0], [8192])
+    assert np.array_equal(again, dflt)
+    assert_parity(dflt, ref, "streaming kernel")
+    hip.tensor_release(t)
+
+
 def test_mixed_batch_and_errors(hip, orc):
     rng = np.random.default_rng(4)
     t4, a = _tensor(hip, rng, 64, 2048, 4)
