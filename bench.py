@@ -714,6 +714,9 @@ def run_moe_layer(args):
     nw = torch.ones(H, device=dev).to(torch.bfloat16)
     torch.cuda.synchronize()
 
+    # --forms three-launches: experts and tail as two launches (the form a captured graph takes)
+    three = "three-launches" in args.forms or bool(args.graph)
+
     def token():
         for l in range(n_layers):
             t_gate, t_seg, t_sg, t_su, t_sd = layers[l]
@@ -722,11 +725,17 @@ def run_moe_layer(args):
             ctx.matvec_batch_route_dev([t_gate, t_seg, t_sg, t_su], x.data_ptr(),
                                        [d_log.data_ptr(), d_seg.data_ptr(), d_sg.data_ptr(), d_su.data_ptr()],
                                        K, d_seg.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), d_p.data_ptr())
-            # no buffer for the per-expert vectors: the experts' sum goes to d_moe, and the tail
-            # takes it as it is (K = 0 with a vector)
-            ctx.moe_decode_dev(l, x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, d_moe.data_ptr(), None)
-            ctx.layer_tail_dev(t_sd, h_mid.data_ptr(), d_moe.data_ptr(), d_p.data_ptr(), 0, d_sg.data_ptr(),
-                               d_su.data_ptr(), nw.data_ptr(), 1e-6, hid[l & 1].data_ptr(), xin[l & 1].data_ptr())
+            if three:
+                # no buffer for the per-expert vectors: the experts' sum goes to d_moe, and the tail
+                # takes it as it is (K = 0 with a vector)
+                ctx.moe_decode_dev(l, x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, d_moe.data_ptr(), None)
+                ctx.layer_tail_dev(t_sd, h_mid.data_ptr(), d_moe.data_ptr(), d_p.data_ptr(), 0, d_sg.data_ptr(),
+                                   d_su.data_ptr(), nw.data_ptr(), 1e-6, hid[l & 1].data_ptr(), xin[l & 1].data_ptr())
+            else:
+                # the experts and the tail in one launch (bit for bit the two calls above)
+                ctx.moe_decode_tail_dev(l, x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, t_sd, h_mid.data_ptr(),
+                                        d_p.data_ptr(), d_sg.data_ptr(), d_su.data_ptr(), nw.data_ptr(), 1e-6,
+                                        hid[l & 1].data_ptr(), xin[l & 1].data_ptr())
 
     token()
     ctx.sync()
@@ -744,11 +753,14 @@ def run_moe_layer(args):
     ms, ev = _timed(ctx, step, args)
     ctx.sync()
     assert torch.equal(xin[(n_layers - 1) & 1], ref)      # same inputs, same result on every step
-    res = {"us_per_layer": round(ms * 1e3 / n_layers, 2), "launches_per_layer": 3,
+    nl_launch = 3 if three else 2
+    res = {"us_per_layer": round(ms * 1e3 / n_layers, 2), "launches_per_layer": nl_launch,
            "graph": bool(args.graph), "event_ms_per_step": round(ev, 5),
-           "roofline": _roofline_hbm("fm_dense_gemv_mixed + fm_moe_fused_rows<3,16> + fm_layer_tail per layer "
-                                     "(three dependent launches, latency-bound)", n_layers * K * es + dense_bytes,
-                                     ev * 1e3, 3 * n_layers)}
+           "roofline": _roofline_hbm(("fm_dense_gemv_mixed + fm_moe_fused_rows<3,16> + fm_layer_tail per layer "
+                                      "(three dependent launches, latency-bound)") if three else
+                                     ("fm_dense_gemv_mixed + fm_moe_fused_rows_tail<3,16> per layer "
+                                      "(two dependent launches, latency-bound)"), n_layers * K * es + dense_bytes,
+                                     ev * 1e3, nl_launch * n_layers)}
     ctx.close()
     return _finish(res, "MoE half of a layer on the device, GB/s over a %d-layer token" % n_layers,
                    "routing + shared-expert GEMVs, top-8, routed 3-bit experts (router-chosen), shared "
@@ -1076,7 +1088,7 @@ def main():
                     help="lm_head workload: 8-bit affine, or the GGUF block formats")
     ap.add_argument("--forms", default="", help="comma-separated overrides of the library's kernel choice for A/B "
                     "runs: plain-dense, plain-gguf (the non-streaming kernels), per-position (no dense GEMM, "
-                    "no grouped GGUF products for chunks)")
+                    "no grouped GGUF products for chunks), three-launches (moe_layer: experts and tail apart)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
@@ -1114,7 +1126,7 @@ def main():
     if args.forms:
         from finchmoe_amd import binding as fb
         known = {"plain-dense": fb.FORM_PLAIN_DENSE, "plain-gguf": fb.FORM_PLAIN_GGUF,
-                 "per-position": fb.FORM_NO_DENSE_GEMM | fb.FORM_NO_GGUF_GROUP}
+                 "per-position": fb.FORM_NO_DENSE_GEMM | fb.FORM_NO_GGUF_GROUP, "three-launches": 0}
         bad = [f for f in args.forms if f not in known]
         if bad:
             print("bench.py: unknown --forms %s (have: %s)" % (bad, ", ".join(known)), file=sys.stderr)

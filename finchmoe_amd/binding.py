@@ -90,6 +90,7 @@ def load():
         "fm_route_topk_dev": (i, [vp, vp, i, i, vp, vp, vp, vp]),
         "fm_matvec_batch_route_dev": (i, [vp, C.POINTER(i), i, vp, C.POINTER(vp), i, vp, vp, vp, vp]),
         "fm_layer_tail_dev": (i, [vp, i, vp, vp, vp, i, vp, vp, vp, C.c_float, vp, vp]),
+        "fm_moe_decode_tail_dev": (i, [vp, i, vp, vp, vp, i, i, vp, vp, vp, vp, vp, C.c_float, vp, vp]),
         "fm_gguf_config": (i, [vp, i, i, i, i, i, i, i]),
         "fm_gguf_upload_layer": (i, [vp, i, vp, sz, vp, sz, vp, sz]),
         "fm_gguf_adopt_layer": (i, [vp, i, vp, sz, vp, sz, vp, sz]),
@@ -326,6 +327,13 @@ class FinchHip:
         self._chk(self.L.fm_layer_tail_dev(self.h, shared_down, d_h_mid, d_eo, d_params, K,
                                            d_shared_gate, d_shared_up, d_next_norm_w, eps,
                                            d_hidden_out, d_next_input))
+
+    def moe_decode_tail_dev(self, layer, d_x, d_idx, d_w, K, shared_down, d_h_mid, d_params, d_shared_gate,
+                            d_shared_up, d_next_norm_w, eps, d_hidden_out, d_next_input):
+        """one layer's routed experts and its tail in one launch (all device pointers)"""
+        self._chk(self.L.fm_moe_decode_tail_dev(self.h, layer, d_x, d_idx, d_w, K, shared_down, d_h_mid, d_params,
+                                                d_shared_gate, d_shared_up, d_next_norm_w, eps, d_hidden_out,
+                                                d_next_input))
 
     def gguf_config(self, n_layers, n_experts, hidden=2048, inter=512,
                     types=(Q4_K, Q4_K, Q6_K)):

@@ -20,7 +20,7 @@ int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs, const FmExpertGe
                             int layer0, int layer_stride, int n_layers, const float *d_x,
                             const int32_t *d_idx, const float *d_w, int K, float *d_act,
                             float *d_expert_out, float *d_out, FmDecodeFlags *df, int flags,
-                            int n_cu, hipStream_t st, hipEvent_t *kev);
+                            int n_cu, hipStream_t st, hipEvent_t *kev, const FmTailArgs *tail);
 int fm_launch_dense(FmDenseSpec *specs, int n, int in_dim, int bits, int scale_fp16,
                     const float *d_x, int M, int n_cu, hipStream_t st, const FmDenseSpec *riders,
                     int n_riders, int *riders_done);
@@ -113,6 +113,7 @@ struct LayerBuf {
 }  // namespace
 
 #define FM_TAIL_PARTIALS 4096
+#define FM_TAIL_VECTOR 16384
 // positions of one chunk: the chunk kernels index pairs x hidden in 32 bits
 #define FM_MAX_CHUNK 65535
 
@@ -281,7 +282,8 @@ int ensure_scratch(fm_ctx *c, int groups, int hidden, int inter) {
     }
     {   // three activation sets of the launch that sums in LDS, every element marked "not
         // produced yet" (0xFFC5A3E1, FM_ACT_EMPTY of fm_decode.hip)
-        const size_t cap = (size_t)g * FM_MAX_K * in;
+        // (+ hidden: the per-row-block sums of squares of the launch that takes the layer tail along)
+        const size_t cap = (size_t)g * FM_MAX_K * in + (size_t)h;
         float *p = nullptr;
         HIPCHK(c, hipMalloc((void **)&p, 3 * cap * sizeof(float)));
         HIPCHK(c, hipMemsetD32Async((hipDeviceptr_t)p, (int)0xFFC5A3E1u, 3 * cap, c->stream));
@@ -497,7 +499,7 @@ extern "C" int fm_reserve(fm_ctx *c, int n_groups, int M, size_t workspace_bytes
     if (c->gguf_cfg && groups > 0 && (rc = ensure_scratch(c, groups, c->ggeom.hidden, c->ggeom.inter))) return rc;
     if (ws && (rc = ensure_ws(c, ws))) return rc;
     if (!c->d_tail) {
-        HIPCHK(c, hipMalloc((void **)&c->d_tail, (FM_TAIL_PARTIALS + 64) * sizeof(float)));
+        HIPCHK(c, hipMalloc((void **)&c->d_tail, (FM_TAIL_PARTIALS + 64 + FM_TAIL_VECTOR) * sizeof(float)));
         HIPCHK(c, hipMemsetAsync(c->d_tail, 0, (FM_TAIL_PARTIALS + 64) * sizeof(float), c->stream));
     }
     return FM_OK;
@@ -646,7 +648,7 @@ extern "C" int fm_moe_decode_step_dev(fm_ctx *c, int layer0, int n_layers, const
                                  K, c->d_act, d_expert_out ? d_expert_out : c->d_eo, d_out,
                                  split ? nullptr : &c->dflags,
                                  flags | (d_expert_out ? 0 : FM_INT_NO_EXPERT_OUT), c->n_cu, c->stream,
-                                 c->ktiming ? c->kev : nullptr);
+                                 c->ktiming ? c->kev : nullptr, nullptr);
     if (rc) return fail(c, rc, "decode launch failed: %s", hipGetErrorString(hipGetLastError()));
     if (!split) c->sync_unchecked = true;
     if (c->ktiming) return ktiming_collect(c);
@@ -696,7 +698,7 @@ extern "C" int fm_moe_decode_step_noalloc_dev(fm_ctx *c, int layer0, int n_layer
     rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer0, 1, n_layers, d_x, d_idx, d_w,
                                  K, (float *)s, (float *)(s + act_b), d_out,
                                  c->split_phases ? nullptr : &df, flags, c->n_cu, c->stream,
-                                 nullptr);
+                                 nullptr, nullptr);
     if (rc) return fail(c, rc, "decode launch failed: %s", hipGetErrorString(hipGetLastError()));
     if (!c->split_phases) c->sync_unchecked = true;
     return FM_OK;
@@ -819,7 +821,7 @@ static int moe_prefill_any(fm_ctx *c, int layer, const void *d_X, bool x_bf16, c
     if (rc) return rc;
     rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer, 0, M, xf, d_idx, d_w, K,
                                  c->d_act, c->d_eo, d_out, c->split_phases ? nullptr : &c->dflags,
-                                 flags | FM_INT_NO_EXPERT_OUT, c->n_cu, c->stream, nullptr);
+                                 flags | FM_INT_NO_EXPERT_OUT, c->n_cu, c->stream, nullptr, nullptr);
     if (rc) return fail(c, rc, "prefill launch failed: %s", hipGetErrorString(hipGetLastError()));
     if (!c->split_phases) c->sync_unchecked = true;
     return FM_OK;
@@ -1239,7 +1241,9 @@ extern "C" int fm_route_topk_dev(fm_ctx *c, const float *d_logits, int n_experts
 static int ensure_tail_scratch(fm_ctx *c) {
     if (c->d_tail) return FM_OK;
     if (note_capture(c)) return refuse_growth(c, "the layer tail's scratch");
-    HIPCHK(c, hipMalloc((void **)&c->d_tail, (FM_TAIL_PARTIALS + 64) * sizeof(float)));
+    // partial sums | ticket words | one vector of up to FM_TAIL_VECTOR floats (the experts' sum
+    // between the two launches of fm_moe_decode_tail_dev when it runs as two)
+    HIPCHK(c, hipMalloc((void **)&c->d_tail, (FM_TAIL_PARTIALS + 64 + FM_TAIL_VECTOR) * sizeof(float)));
     HIPCHK(c, hipMemsetAsync(c->d_tail, 0, (FM_TAIL_PARTIALS + 64) * sizeof(float), c->stream));
     return FM_OK;
 }
@@ -1288,6 +1292,72 @@ extern "C" int fm_layer_tail_dev(fm_ctx *c, fm_tensor shared_down, const float *
     if (rc) return fail(c, rc, "layer tail: shape [%d, %d] at %d bits has no kernel", t->out_dim,
                         t->in_dim, t->bits);
     return FM_OK;
+}
+
+// One layer's routed experts and the layer's tail in one launch: fm_moe_decode_dev (without the
+// per-expert vectors) followed by fm_layer_tail_dev in its K = 0 form, bit for bit.  Shapes the
+// one-launch kernel does not cover (and calls under stream capture) run as those two launches.
+extern "C" int fm_moe_decode_tail_dev(fm_ctx *c, int layer, const float *d_x, const int32_t *d_idx,
+                                      const float *d_w, int K, fm_tensor shared_down, const float *d_h_mid,
+                                      const float *d_params, const float *d_shared_gate,
+                                      const float *d_shared_up, const uint16_t *d_next_norm_w, float eps,
+                                      float *d_hidden_out, float *d_next_input) {
+    if (!c) return FM_ERR_ARG;
+    if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
+    Tensor *t = get_tensor(c, shared_down);
+    if (!t) return fail(c, FM_ERR_ARG, "bad tensor handle %d", shared_down);
+    if (!d_x || !d_idx || !d_w || !d_h_mid || !d_params || !d_shared_gate || !d_shared_up || !d_hidden_out)
+        return fail(c, FM_ERR_ARG, "null pointer");
+    if (K < 1 || K > FM_MAX_K) return fail(c, FM_ERR_ARG, "K %d outside 1..%d", K, FM_MAX_K);
+    if ((d_next_input != nullptr) != (d_next_norm_w != nullptr))
+        return fail(c, FM_ERR_ARG, "next input and its norm weights go together");
+    if (((uintptr_t)d_shared_gate | (uintptr_t)d_shared_up) & 3)
+        return fail(c, FM_ERR_ARG, "vector not 4-byte aligned");
+    int rc = check_layers(c, c->layers, layer, 1);
+    if (rc) return rc;
+    DeviceGuard dg(c->device);
+    rc = ensure_scratch(c, 1, c->geom.hidden, c->geom.inter);
+    if (rc) return rc;
+    rc = ensure_tail_scratch(c);
+    if (rc) return rc;
+    const bool one_launch = !c->split_phases && !c->ktiming && t->bits == 4 && !t->raw_bf16() && !t->gguf() &&
+                            t->group_size == 64 && t->out_dim == c->geom.hidden && t->in_dim == c->geom.inter;
+    if (one_launch) {
+        FmTailArgs a{};
+        a.W = (const uint8_t *)t->W;
+        a.S = (const uint8_t *)t->S;
+        a.B = (const uint8_t *)t->B;
+        a.hidden = t->out_dim;
+        a.inter = t->in_dim;
+        a.K = 0;
+        a.h_mid = d_h_mid;
+        a.expert_out = nullptr;
+        a.params = d_params;
+        a.shared_gate = d_shared_gate;
+        a.shared_up = d_shared_up;
+        a.norm_w = d_next_norm_w;
+        a.eps = eps;
+        a.hidden_out = d_hidden_out;
+        a.next_in = d_next_input;
+        a.partial = c->d_tail;
+        a.counter = (unsigned int *)(c->d_tail + FM_TAIL_PARTIALS);
+        a.scale_fp16 = t->scale_fp16;
+        rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer, 1, 1, d_x, d_idx, d_w, K, c->d_act, c->d_eo,
+                                     d_hidden_out, &c->dflags, FM_INT_NO_EXPERT_OUT, c->n_cu, c->stream, nullptr, &a);
+        if (rc == FM_OK) {
+            c->sync_unchecked = true;
+            return FM_OK;
+        }
+        if (rc != FM_ERR_UNSUPPORTED)
+            return fail(c, rc, "decode + tail launch failed: %s", hipGetErrorString(hipGetLastError()));
+    }
+    // two launches: the experts' sum crosses in a vector of the tail's scratch
+    if (c->geom.hidden > FM_TAIL_VECTOR) return fail(c, FM_ERR_UNSUPPORTED, "hidden %d", c->geom.hidden);
+    float *d_sum = c->d_tail + FM_TAIL_PARTIALS + 64;
+    rc = fm_moe_decode_step_dev(c, layer, 1, d_x, d_idx, d_w, K, d_sum, nullptr, 0);
+    if (rc) return rc;
+    return fm_layer_tail_dev(c, shared_down, d_h_mid, d_sum, d_params, 0, d_shared_gate, d_shared_up,
+                             d_next_norm_w, eps, d_hidden_out, d_next_input);
 }
 
 // ============================================================================

@@ -77,6 +77,7 @@ struct FmTailArgs {
     float *hidden_out, *next_in;
     float *partial;
     unsigned int *counter;
+    int scale_fp16;          // scale type of W's groups (the launch with the experts in front only)
 };
 
 // ---------------------------------------------------------------- device helpers

@@ -1009,8 +1009,13 @@ struct Fm2Stream {
         }
     }
 
-    // dm: the launch's dimensions with their divisions prepared (fm2_dims on the host)
-    __device__ __forceinline__ void run(const Fm2Dims &dm) {
+    // dm: the launch's dimensions with their divisions prepared (fm2_dims on the host).
+    // TAIL (one layer, one down part per workgroup): the layer's tail in the same launch — the
+    // workgroup that owns rows of the experts' sum also runs those rows of the shared expert's
+    // down projection and writes hidden = h_mid + sum + sigmoid(score) * shared; the workgroup
+    // that finishes last normalises (fm_layer_tail's arithmetic, operation for operation).
+    template <bool TAIL>
+    __device__ __forceinline__ void run(const Fm2Dims &dm, const FmTailArgs *tp) {
         const int K = a.K, G = gridDim.x, g = blockIdx.x;
         // The split.  Down: a workgroup's row blocks lie in ONE layer whenever there are at
         // least as many workgroups as layers (layer l gets the workgroups g with g*L/G == l, its
@@ -1063,6 +1068,32 @@ struct Fm2Stream {
                 t.n = mine_n;
                 t.layer = (int)sg;
             }
+        }
+        // TAIL: what the tail needs from memory is requested here too (the shared expert's codes
+        // for this workgroup's rows stay in registers until the experts are done)
+        FmRowSlice<4> tw;
+        float t_hm = 0.0f, t_score = 0.0f;
+        uint32_t t_nw = 0u;
+        int t_row0 = 0, t_nrb = 0;
+        Fm2TailLds tl{};
+        if constexpr (TAIL) {
+            t_nrb = (int)fm_div(dm.by_K, sp.dn_wg1 - sp.dn_wg0);
+            t_row0 = (int)fm_div(dm.by_K, sp.dn_wg0) * RPS_DN;
+            tl = fm2_tail_lds(t_nrb, K, RPS_DN, tp->inter, tp->hidden);
+            const int tw_row = t_row0 + (wave < t_nrb ? wave : 0) * RPS_DN + lane / LPR_DN, tc = lane % LPR_DN;
+            const int trb = tp->inter / 2, tsb = (tp->inter / 64) * 2;
+            fm_load_slice<4>(tw, tp->W + (size_t)tw_row * trb + (size_t)tc * 64, tp->S + (size_t)tw_row * tsb + (size_t)tc * 4,
+                             tp->B + (size_t)tw_row * tsb + (size_t)tc * 4);
+            const int rows = t_nrb * RPS_DN, tr = (int)threadIdx.x < rows ? (int)threadIdx.x : (rows > 0 ? rows - 1 : 0);
+            t_hm = tp->h_mid[t_row0 + tr];
+            t_score = tp->params[8];
+            t_nw = tp->next_in ? (uint32_t)tp->norm_w[t_row0 + tr] : 0u;
+            const int tj = (int)threadIdx.x < tp->inter ? (int)threadIdx.x : tp->inter - 1;
+            const float tact = fm_silu_mul(tp->shared_gate[tj], tp->shared_up[tj]);
+            if ((int)threadIdx.x < tp->inter) fm_lds_w32(part0 + tl.act + 4u * (uint32_t)tj, __float_as_uint(tact));
+#pragma unroll
+            for (int i = 0; i < FmRowSlice<4>::NQ; i++) asm volatile("" ::"v"(tw.q[i]));
+            asm volatile("" ::"v"(tw.s), "v"(tw.b), "v"(t_hm), "v"(t_score), "v"(t_nw));
         }
 #pragma unroll
         for (int i = 0; i < FmActX<LPR_UP>::NIT; i++)
@@ -1174,8 +1205,92 @@ struct Fm2Stream {
             }
             if (n_seq > n_up) {
                 fm_wg_barrier();
-                reduce_part(n_seq - 1);
+                if constexpr (TAIL) tail_part(n_seq - 1, *tp, tw, t_hm, t_score, t_nw, t_row0, t_nrb, tl);
+                else reduce_part(n_seq - 1);
             }
+        }
+    }
+
+    // The tail for the rows of part q (the workgroup's only down part).  The rings are empty by now.
+    __device__ __forceinline__ void tail_part(int q, const FmTailArgs &ta, const FmRowSlice<4> &tw, float hm,
+                                              float score, uint32_t nw, int row0, int nrb, const Fm2TailLds &tl) {
+        const int K = a.K;
+        const int r_in = lane / LPR_DN, tc = lane % LPR_DN;
+        // the shared expert's down projection for these rows: fm_layer_tail's lane map and arithmetic
+        if (wave < nrb) {
+            float xs[FM_CPL], xsum0, xsum1;
+            const uint8_t *part_mem = fm_dyn_lds + D::WG_BYTES + 2 * IMG_UP + FM2_MAX_SEG * sizeof(Fm2Seg);
+            fm_load_x<4>(reinterpret_cast<const float *>(part_mem + tl.act) + tc * FM_CPL, xs, xsum0, xsum1);
+            const float d = ta.scale_fp16 ? fm_lane_dot<4, true>(tw, xs, xsum0, xsum1)
+                                          : fm_lane_dot<4, false>(tw, xs, xsum0, xsum1);
+            const float so = fm_group_sum<LPR_DN>(d);
+            if (tc == 0) fm_lds_w32(part0 + tl.so + 4u * (uint32_t)(wave * RPS_DN + r_in), __float_as_uint(so));
+        }
+        fm_wg_barrier();
+        const uint32_t tq = fm_lds_addr(&tab[q]);
+        float wk[FM_MAX_K];
+#pragma unroll
+        for (int k = 0; k < FM_MAX_K; k++)
+            wk[k] = k < K ? __uint_as_float(fm_lds_r32(tq + (uint32_t)offsetof(Fm2Seg, w) + 4u * k)) : 0.0f;
+        const int rows = nrb * RPS_DN;
+        const bool mine = (int)threadIdx.x < rows;
+        float hv = 0.0f;
+        if (mine) {
+            const int r = threadIdx.x, rbi = r / RPS_DN, ris = r - rbi * RPS_DN;
+            float acc = 0.0f;
+#pragma unroll
+            for (int k = 0; k < FM_MAX_K; k++)
+                if (k < K && wk[k] != 0.0f)
+                    acc += wk[k] * __uint_as_float(fm_lds_r32(part0 + 4u * (uint32_t)((rbi * K + k) * RPS_DN + ris)));
+            const float shared_out = __uint_as_float(fm_lds_r32(part0 + tl.so + 4u * (uint32_t)r));
+            const float moe = acc;
+            const float shared_gate = 1.0f / (1.0f + expf(-score));
+            hv = hm + moe + shared_gate * shared_out;
+            fm_st_shared(ta.hidden_out + row0 + r, hv);
+            fm_lds_w32(part0 + tl.so + 4u * (uint32_t)r, __float_as_uint(hv));    // (its shared_out is used up)
+        }
+        if (!ta.next_in) return;
+        // The norm needs the sum of squares over all rows.  fm_layer_tail adds them per wave of 16
+        // rows (lane 4 r holds row r's square), per workgroup of four such waves, then over the
+        // workgroups in order; a row block here is one such wave.  Every workgroup publishes its
+        // row blocks' sums (a word that holds the not-yet-produced marker until then), gathers all
+        // of them, adds them in that order and normalises its own rows: nothing waits for a last
+        // workgroup, and no ticket is drawn.
+        fm_wg_barrier();
+        if (wave < nrb) {
+            const float v = tc == 0 ? __uint_as_float(fm_lds_r32(part0 + tl.so + 4u * (uint32_t)(wave * RPS_DN + r_in))) : 0.0f;
+            const float sq = fm_group_sum<64>(v * v);
+            if (lane == 0) fm_st_shared(ta.partial + row0 / RPS_DN + wave, sq);
+        }
+        const int n_vw = ta.hidden / RPS_DN;
+        for (int v = threadIdx.x; v < n_vw; v += FM_NW * 64)
+            fm_lds_w32(part0 + tl.red + 4u * (uint32_t)v, __float_as_uint(act_get(ta.partial + v)));
+        fm_wg_barrier();
+        if (wave == 0) {
+            float sum_sq = 0.0f;
+            for (int b0 = 0; b0 < n_vw / 4; b0 += 64) {
+                const int b = b0 + lane;
+                float p = 0.0f;
+                if (b < n_vw / 4) {
+                    const uint32_t ra = part0 + tl.red + 16u * (uint32_t)b;
+                    uint2 q01, q23;
+                    asm volatile("ds_read2_b32 %0, %2 offset1:1\n\tds_read2_b32 %1, %2 offset0:2 offset1:3\n\ts_waitcnt lgkmcnt(0)"
+                                 : "=&v"(q01), "=&v"(q23)
+                                 : "v"(ra)
+                                 : "memory");
+                    p = ((__uint_as_float(q01.x) + __uint_as_float(q01.y)) + __uint_as_float(q23.x)) + __uint_as_float(q23.y);
+                }
+                const int nb = n_vw / 4 - b0 < 64 ? n_vw / 4 - b0 : 64;
+                for (int i = 0; i < nb; i++) sum_sq += __shfl(p, i);
+            }
+            if (lane == 0) fm_lds_w32(part0 + tl.word, __float_as_uint(sum_sq));
+        }
+        fm_wg_barrier();
+        const float sum_sq = __uint_as_float(fm_lds_r32(part0 + tl.word));
+        const float inv_rms = 1.0f / sqrtf(sum_sq / (float)ta.hidden + ta.eps);   // infer.m:1771-1772
+        if (mine) {
+            const int row = row0 + (int)threadIdx.x;
+            ta.next_in[row] = hv * inv_rms * __uint_as_float(nw << 16);
         }
     }
 };
@@ -1184,7 +1299,15 @@ template <int BITS, int LPR_UP, bool FP16>
 __global__ __launch_bounds__(FM_NW * 64)
 void fm_moe_fused_rows(DecodeArgs a, Fm2Dims dm, Fm2Sync sy) {
     Fm2Stream<BITS, LPR_UP, FP16> st(a, sy);
-    st.run(dm);
+    st.template run<false>(dm, nullptr);
+}
+
+// one layer's experts with the layer's tail behind them (Fm2Stream::run<true>)
+template <int BITS, int LPR_UP, bool FP16>
+__global__ __launch_bounds__(FM_NW * 64)
+void fm_moe_fused_rows_tail(DecodeArgs a, Fm2Dims dm, Fm2Sync sy, FmTailArgs ta) {
+    Fm2Stream<BITS, LPR_UP, FP16> st(a, sy);
+    st.template run<true>(dm, &ta);
 }
 
 // fills n words with v (counters to zero, activations to FM_ACT_EMPTY)
@@ -1251,6 +1374,37 @@ int launch_fused(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st, con
 // The launch that keeps the per-expert vectors in LDS.  FM_ERR_UNSUPPORTED when the shape does
 // not fit its fixed tables (the caller then takes the launch with counters).
 template <int BITS, int LPR_UP, bool FP16>
+int launch_fused_rows_tail(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st, const Fm2Sync &sy,
+                           const FmTailArgs &ta) {
+    auto kfn = fm_moe_fused_rows_tail<BITS, LPR_UP, FP16>;
+    const size_t sh = fm2_lds_bytes<BITS, LPR_UP>();
+    static FmKernelSetup ks;
+    if (!fm_dyn_lds_ok(ks, (const void *)kfn, sh)) return FM_ERR_HIP;
+    const int dev = fm_current_device();
+    int per_cu = dev >= 0 ? ks.per_cu[dev] : 0;
+    if (per_cu == 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kfn, FM_NW * 64, sh) != hipSuccess)
+            per_cu = 0;
+        if (per_cu < 1) per_cu = -1;
+        if (dev >= 0) ks.per_cu[dev] = per_cu;
+    }
+    if (per_cu < 1) return FM_ERR_UNSUPPORTED;
+    // one layer; the shared expert's down projection has the experts' down shape (its rows are
+    // the rows of the experts' sum, its wave step their row block), 4-bit; every workgroup owns
+    // at least one row block and the tail's tables fit beside its partial vectors
+    if (n_pairs != a.K || ta.hidden != a.g.hidden || ta.inter != a.g.inter || ta.K != 0) return FM_ERR_UNSUPPORTED;
+    const Fm2Plan plan = fm2_plan(n_pairs, a.K, a.g.inter, a.g.hidden, LPR_UP, n_cu);
+    if (!plan.ok) return FM_ERR_UNSUPPORTED;
+    const int rps_dn = FM_WAVE / (LPR_UP / 4), dn_rbs = a.g.hidden / rps_dn;
+    if (plan.wgs > dn_rbs) return FM_ERR_UNSUPPORTED;
+    const int nrb_max = (dn_rbs + plan.wgs - 1) / plan.wgs;
+    if (!fm2_tail_lds(nrb_max, a.K, rps_dn, ta.inter, ta.hidden).ok) return FM_ERR_UNSUPPORTED;
+    const Fm2Dims dm = fm2_dims(n_pairs, a.K, plan.wgs, a.g.inter, a.g.hidden, LPR_UP);
+    hipLaunchKernelGGL(kfn, dim3((unsigned)plan.wgs), dim3(FM_NW * 64), sh, st, a, dm, sy, ta);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
+
+template <int BITS, int LPR_UP, bool FP16>
 int launch_fused_rows(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st, const Fm2Sync &sy) {
     auto kfn = fm_moe_fused_rows<BITS, LPR_UP, FP16>;
     const size_t sh = fm2_lds_bytes<BITS, LPR_UP>();
@@ -1278,11 +1432,26 @@ int launch_fused_rows(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st
 template <int BITS, bool FP16>
 int launch_decode_t(const DecodeArgs &a, int n_pairs, int rpi_up, int n_cu,
                     hipStream_t st, hipEvent_t *kev, const FmFlags *fl, bool *fused,
-                    const Fm2Sync *sy = nullptr, float *act_rows = nullptr, bool *rows = nullptr) {
+                    const Fm2Sync *sy = nullptr, float *act_rows = nullptr, bool *rows = nullptr,
+                    const FmTailArgs *tail = nullptr) {
     dim3 b(256);
     const int lpr_up = a.g.hidden / FM_CPL, lpr_down = a.g.inter / FM_CPL;
     const bool lds_up = lpr_up >= 4 && lpr_up <= 16, lds_down = lpr_down <= 16;
     if (!lds_down) return FM_ERR_UNSUPPORTED;
+    if (tail) {      // only the launch that sums the experts itself can take the tail along
+        if (!(sy && lds_up && lpr_down * 4 == lpr_up)) return FM_ERR_UNSUPPORTED;
+        DecodeArgs a2 = a;
+        a2.act = act_rows;
+        a2.expert_out = nullptr;
+        int rc = FM_ERR_UNSUPPORTED;
+        switch (lpr_up) {
+            case 4: rc = launch_fused_rows_tail<BITS, 4, FP16>(a2, n_pairs, n_cu, st, *sy, *tail); break;
+            case 8: rc = launch_fused_rows_tail<BITS, 8, FP16>(a2, n_pairs, n_cu, st, *sy, *tail); break;
+            case 16: rc = launch_fused_rows_tail<BITS, 16, FP16>(a2, n_pairs, n_cu, st, *sy, *tail); break;
+        }
+        if (rows) *rows = rc == FM_OK;
+        return rc;
+    }
     if (kev) (void)hipEventRecord(kev[0], st);
     if (sy && lds_up && lpr_down * 4 == lpr_up) {
         DecodeArgs a2 = a;
@@ -1397,7 +1566,7 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
                                        const float *d_w, int K, float *d_act,
                                        float *d_expert_out, float *d_out,
                                        FmDecodeFlags *df, int flags, int n_cu,
-                                       hipStream_t st, hipEvent_t *kev) {
+                                       hipStream_t st, hipEvent_t *kev, const FmTailArgs *tail) {
     DecodeArgs a;
     a.layer_ptrs = d_layer_ptrs;
     a.g = *g;
@@ -1433,6 +1602,7 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     // (the entry point that allocates nothing has one counter set only: it takes the graph's
     // route whether or not the stream is capturing)
     const bool own_clear = captured || (df && df->always_graph_set);
+    if (tail && (own_clear || !df)) return FM_ERR_UNSUPPORTED;    // (the caller chains the two launches)
     if (df && (df->set[0] || df->always_graph_set) && need <= df->cap) {
         if (own_clear) {
             hipLaunchKernelGGL(fm_clear_counters, dim3((need + 255) / 256), dim3(256), 0, st,
@@ -1453,7 +1623,8 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     Fm2Sync sy{};
     const Fm2Sync *syp = nullptr;
     float *act_rows = nullptr;
-    const unsigned int act_need = (unsigned int)n_pairs * (unsigned int)g->inter;
+    // (with the tail along: one more vector for the row blocks' sums of squares, behind the activations)
+    const unsigned int act_need = (unsigned int)n_pairs * (unsigned int)g->inter + (tail ? (unsigned int)g->hidden : 0u);
     if (flp && (flags & FM_INT_NO_EXPERT_OUT) && !(flags & FM_GUARD) && df->act_cap >= act_need &&
         df->act_set[0]) {
         if (own_clear) {
@@ -1477,7 +1648,14 @@ extern "C" int fm_launch_decode_affine(const uint8_t *const *d_layer_ptrs,
     }
     a.flags = flags & ~FM_INT_NO_EXPERT_OUT;
     bool fused = false, rows = false;
-#define FM_DEC(B, F) launch_decode_t<B, F>(a, n_pairs, rpi_up, n_cu, st, kev, flp, &fused, syp, act_rows, &rows)
+    FmTailArgs tail_args{};
+    if (tail) {
+        if (!syp) return FM_ERR_UNSUPPORTED;      // (the caller chains the two launches)
+        tail_args = *tail;
+        tail_args.partial = act_rows + (size_t)n_pairs * g->inter;
+        tail = &tail_args;
+    }
+#define FM_DEC(B, F) launch_decode_t<B, F>(a, n_pairs, rpi_up, n_cu, st, kev, flp, &fused, syp, act_rows, &rows, tail)
     int rc = FM_ERR_UNSUPPORTED;
     if (g->bits == 3) rc = g->scale_fp16 ? FM_DEC(3, true) : FM_DEC(3, false);
     else if (g->bits == 4) rc = g->scale_fp16 ? FM_DEC(4, true) : FM_DEC(4, false);

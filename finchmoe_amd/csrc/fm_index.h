@@ -478,6 +478,23 @@ FM_HD void fm2_dn_unit(uint32_t rb_first, uint32_t nrb, float inv, uint32_t ul, 
     *pn = (uint32_t)(((float)ul + 0.5f) * inv);
     *rsn = rb_first + (ul - *pn * nrb);
 }
+// The layer tail behind the experts in the same launch keeps three small tables in the part of
+// LDS the partial vectors leave free: the shared expert's results for the workgroup's rows, the
+// shared expert's activations, and the per-wave sums of the norm.  nrb = row blocks of the
+// workgroup's (one) down part.
+struct Fm2TailLds {
+    int ok;
+    uint32_t so, act, red, word;     // byte offsets inside the partial-vector area
+};
+FM_HD Fm2TailLds fm2_tail_lds(int nrb, int K, int rps_dn, int shared_inter, int hidden) {
+    Fm2TailLds t;
+    t.so = (uint32_t)(nrb * K * rps_dn * 4);                 // behind the partial vectors
+    t.act = (t.so + (uint32_t)(nrb * rps_dn * 4) + 15u) & ~15u;
+    t.red = t.act + (uint32_t)shared_inter * 4u;
+    t.word = t.red + (uint32_t)(hidden / rps_dn) * 4u;
+    t.ok = nrb >= 1 && nrb <= 8 && shared_inter <= 512 && t.word + 16u <= FM2_PART_BYTES;
+    return t;
+}
 // the launcher's decision: workgroups, and whether the shape fits the kernel's fixed tables
 struct Fm2Plan {
     int ok, wgs;

@@ -287,6 +287,21 @@ FM_API int fm_layer_tail_dev(fm_ctx *ctx, fm_tensor shared_down, const float *d_
                       const uint16_t *d_next_norm_w, float eps, float *d_hidden_out,
                       float *d_next_input);
 
+/* The routed experts of one layer and the layer tail in ONE launch — the reference's CMD3 command
+ * buffer from the expert dispatches to the next layer's norm (finchmoe/infer.m:9608-9760):
+ * fm_moe_decode_dev(ctx, layer, d_x, d_idx, d_w, K, sum, NULL, 0) followed by
+ * fm_layer_tail_dev(ctx, shared_down, d_h_mid, sum, d_params, 0, ...), with identical results
+ * bit for bit.  d_params: only [8] (the shared-expert gate score) is read; the experts' weights are
+ * d_w.  One launch when shared_down is 4-bit with the experts' down shape (the workgroup that
+ * owns rows of the experts' sum runs the same rows of the shared projection, and the workgroup
+ * that finishes last normalises); other shapes, split-phase mode and calls under stream capture
+ * run as the two launches. */
+FM_API int fm_moe_decode_tail_dev(fm_ctx *ctx, int layer, const float *d_x, const int32_t *d_idx,
+                           const float *d_w, int K, fm_tensor shared_down, const float *d_h_mid,
+                           const float *d_params, const float *d_shared_gate,
+                           const float *d_shared_up, const uint16_t *d_next_norm_w, float eps,
+                           float *d_hidden_out, float *d_next_input);
+
 /* ---------------------------------------------------------------- GGUF expert store
  * Replaces GgufExpertInfo + the slab copies of gpu_gguf_experts_forward
  * (finchmoe/infer.m:1017-1022, 3239-3290).  gate/up/down are the stacked

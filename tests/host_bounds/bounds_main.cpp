@@ -683,6 +683,33 @@ int main() {
         walk_phases(1, 8, 2048, 512, bits, true);
     }
     sweep_fused_rows();
+    {   // the one-layer launch with the layer tail along: its three tables beside the partial vectors
+        g_case = "fused rows + tail, LDS tables";
+        for (int K : {1, 5, 8})
+            for (int lpr_up : {4, 8, 16}) {
+                const int hidden = 128 * lpr_up, inter = hidden / 4, rps_dn = FM_WAVE / (lpr_up / 4);
+                const Fm2Plan plan = fm2_plan(K, K, inter, hidden, lpr_up, N_CU);
+                if (!plan.ok) continue;
+                const int dn_rbs = hidden / rps_dn;
+                if (plan.wgs > dn_rbs) continue;                  // (the launcher refuses these)
+                const int nrb = (dn_rbs + plan.wgs - 1) / plan.wgs;
+                const Fm2TailLds t = fm2_tail_lds(nrb, K, rps_dn, inter, hidden);
+                if (!t.ok) continue;
+                CHECK(t.so >= (uint32_t)(nrb * K * rps_dn * 4), "shared results over the partial vectors");
+                CHECK(t.act >= t.so + (uint32_t)(nrb * rps_dn * 4) && t.act % 16 == 0, "activations over the shared results");
+                CHECK(t.red >= t.act + (uint32_t)inter * 4, "sums over the activations");
+                CHECK(t.word >= t.red + (uint32_t)(hidden / rps_dn) * 4 && t.word + 4 <= FM2_PART_BYTES, "word outside the area");
+                // every workgroup owns at least one row block, at most nrb
+                const Fm2Dims dm = fm2_dims(K, K, plan.wgs, inter, hidden, lpr_up);
+                for (int b = 0; b < plan.wgs; b++) {
+                    const Fm2Split sp = fm2_split(dm, b);
+                    const uint32_t n = (sp.dn_wg1 - sp.dn_wg0) / K;
+                    CHECK(sp.n_dn == 1 && n >= 1 && n <= (uint32_t)nrb, "workgroup %d owns %u row blocks (at most %d)", b, n, nrb);
+                    CHECK((sp.dn_wg0 / K + n) * rps_dn <= (uint32_t)hidden, "rows past the layer");
+                }
+            }
+        std::printf("ok  %-58s\n", g_case.c_str());
+    }
     walk_fused_rows(64, 8, 2048, 512, 3);
     walk_fused_rows(300, 8, 2048, 512, 3);
     // ---- config 4: GGUF step, one layer, chunk of 8 positions

@@ -225,5 +225,45 @@ def _moe_half(hip, orc):
         hip.sync()
         for got, want in zip((d_log, d_seg, d_sg, d_su, d_idx, d_w, d_p), keep):
             assert torch.equal(got, want), rep
+    # the experts and the tail as ONE launch (the reference's CMD3 from the expert dispatches to
+    # the next layer's norm): bit for bit the two launches above, several times in a row (the
+    # activation sets alternate and the ticket word must come back to zero), also between other
+    # decode calls, and in the last layer's form (no next input)
+    for rep in range(4):
+        d_hid3 = torch.full((Hh,), 3.0, device="cuda")
+        d_next3 = torch.full((Hh,), 5.0, device="cuda")
+        torch.cuda.synchronize()
+        hip.moe_decode_tail_dev(0, d_x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), Kk, t_sd, d_hmid.data_ptr(),
+                                d_p.data_ptr(), d_sg.data_ptr(), d_su.data_ptr(), d_nw.data_ptr(), 1e-6,
+                                d_hid3.data_ptr(), d_next3.data_ptr())
+        hip.sync()
+        assert torch.equal(d_hid3, d_hid), rep
+        assert torch.equal(d_next3, d_next), rep
+        if rep == 1:
+            hip.moe_decode_dev(0, d_x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), Kk, d_moe2.data_ptr(), None)
+            hip.sync()
+            assert torch.equal(d_moe2, d_moe)
+    d_hid4 = torch.full((Hh,), 3.0, device="cuda")
+    torch.cuda.synchronize()
+    hip.moe_decode_tail_dev(0, d_x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), Kk, t_sd, d_hmid.data_ptr(),
+                            d_p.data_ptr(), d_sg.data_ptr(), d_su.data_ptr(), None, 1e-6, d_hid4.data_ptr(), None)
+    hip.sync()
+    assert torch.equal(d_hid4, d_hid)
+    # fewer slots than eight, and a slot with an index outside the store (weight 0 upstream)
+    idx5 = d_idx.clone()
+    idx5[2] = Ee + 7
+    for kk, ix in ((5, d_idx), (Kk, idx5)):
+        d_sum = torch.empty(Hh, device="cuda")
+        d_ha, d_na = torch.empty(Hh, device="cuda"), torch.empty(Hh, device="cuda")
+        d_hb, d_nb = torch.empty(Hh, device="cuda"), torch.empty(Hh, device="cuda")
+        torch.cuda.synchronize()
+        hip.moe_decode_dev(0, d_x.data_ptr(), ix.data_ptr(), d_w.data_ptr(), kk, d_sum.data_ptr(), None)
+        hip.layer_tail_dev(t_sd, d_hmid.data_ptr(), d_sum.data_ptr(), d_p.data_ptr(), 0, d_sg.data_ptr(),
+                           d_su.data_ptr(), d_nw.data_ptr(), 1e-6, d_ha.data_ptr(), d_na.data_ptr())
+        hip.moe_decode_tail_dev(0, d_x.data_ptr(), ix.data_ptr(), d_w.data_ptr(), kk, t_sd, d_hmid.data_ptr(),
+                                d_p.data_ptr(), d_sg.data_ptr(), d_su.data_ptr(), d_nw.data_ptr(), 1e-6,
+                                d_hb.data_ptr(), d_nb.data_ptr())
+        hip.sync()
+        assert torch.equal(d_hb, d_ha) and torch.equal(d_nb, d_na), kk
     for t in (t_gate, t_seg, t_sg, t_su, t_sd):
         hip.tensor_release(t)

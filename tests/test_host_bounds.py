@@ -40,7 +40,7 @@ def test_every_access_of_the_benchmark_launches_is_inside_its_buffer(walker):
                  "fused rows 1 groups x 8, 3-bit", "split phases 40 groups x 8, 4-bit",
                  "fused (counters) 40 groups x 8, 4-bit", "gguf stream gate/up Q4_K 40 groups x 8",
                  "gguf stream down Q6_K 40 groups x 8", "gguf stream down Q6_K 8 groups x 8",
-                 "fused rows, sweep of shapes"):
+                 "fused rows, sweep of shapes", "fused rows + tail, LDS tables"):
         assert ("ok  " + case) in r.stdout or ("ok  dense " + case) in r.stdout, case
 
 
