@@ -722,6 +722,13 @@ def run_moe_layer(args):
             t_gate, t_seg, t_sg, t_su, t_sd = layers[l]
             x = x0 if l == 0 else xin[(l - 1) & 1]
             h_mid = x0 if l == 0 else hid[(l - 1) & 1]
+            if not three:
+                # two launches: the routing batch; routing + experts + tail (bit for bit the three below)
+                ctx.moe_layer_dev(l, [t_gate, t_seg, t_sg, t_su], x.data_ptr(), K, t_sd, h_mid.data_ptr(),
+                                  nw.data_ptr(), 1e-6, d_log.data_ptr(), d_seg.data_ptr(), d_sg.data_ptr(),
+                                  d_su.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), d_p.data_ptr(),
+                                  hid[l & 1].data_ptr(), xin[l & 1].data_ptr())
+                continue
             ctx.matvec_batch_route_dev([t_gate, t_seg, t_sg, t_su], x.data_ptr(),
                                        [d_log.data_ptr(), d_seg.data_ptr(), d_sg.data_ptr(), d_su.data_ptr()],
                                        K, d_seg.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), d_p.data_ptr())
@@ -758,7 +765,7 @@ def run_moe_layer(args):
            "graph": bool(args.graph), "event_ms_per_step": round(ev, 5),
            "roofline": _roofline_hbm(("fm_dense_gemv_mixed + fm_moe_fused_rows<3,16> + fm_layer_tail per layer "
                                       "(three dependent launches, latency-bound)") if three else
-                                     ("fm_dense_gemv_mixed + fm_moe_fused_rows_tail<3,16> per layer "
+                                     ("fm_dense_gemv_mixed + fm_moe_fused_rows_tail<3,16> (routing, experts, tail) per layer "
                                       "(two dependent launches, latency-bound)"), n_layers * K * es + dense_bytes,
                                      ev * 1e3, nl_launch * n_layers)}
     ctx.close()

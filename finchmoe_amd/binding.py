@@ -91,6 +91,7 @@ def load():
         "fm_matvec_batch_route_dev": (i, [vp, C.POINTER(i), i, vp, C.POINTER(vp), i, vp, vp, vp, vp]),
         "fm_layer_tail_dev": (i, [vp, i, vp, vp, vp, i, vp, vp, vp, C.c_float, vp, vp]),
         "fm_moe_decode_tail_dev": (i, [vp, i, vp, vp, vp, i, i, vp, vp, vp, vp, vp, C.c_float, vp, vp]),
+        "fm_moe_layer_dev": (i, [vp, i, C.POINTER(i), vp, i, i, vp, vp, C.c_float, vp, vp, vp, vp, vp, vp, vp, vp, vp]),
         "fm_gguf_config": (i, [vp, i, i, i, i, i, i, i]),
         "fm_gguf_upload_layer": (i, [vp, i, vp, sz, vp, sz, vp, sz]),
         "fm_gguf_adopt_layer": (i, [vp, i, vp, sz, vp, sz, vp, sz]),
@@ -334,6 +335,14 @@ class FinchHip:
         self._chk(self.L.fm_moe_decode_tail_dev(self.h, layer, d_x, d_idx, d_w, K, shared_down, d_h_mid, d_params,
                                                 d_shared_gate, d_shared_up, d_next_norm_w, eps, d_hidden_out,
                                                 d_next_input))
+
+    def moe_layer_dev(self, layer, route_tensors, d_x, K, shared_down, d_h_mid, d_next_norm_w, eps, d_logits,
+                      d_seg, d_shared_gate, d_shared_up, d_idx, d_w, d_params, d_hidden_out, d_next_input):
+        """the MoE half of a layer: routing batch, then routing + experts + tail in one launch"""
+        ts = (C.c_int * 4)(*route_tensors)
+        self._chk(self.L.fm_moe_layer_dev(self.h, layer, ts, d_x, K, shared_down, d_h_mid, d_next_norm_w, eps,
+                                          d_logits, d_seg, d_shared_gate, d_shared_up, d_idx, d_w, d_params,
+                                          d_hidden_out, d_next_input))
 
     def gguf_config(self, n_layers, n_experts, hidden=2048, inter=512,
                     types=(Q4_K, Q4_K, Q6_K)):

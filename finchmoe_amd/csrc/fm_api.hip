@@ -1297,12 +1297,12 @@ extern "C" int fm_layer_tail_dev(fm_ctx *c, fm_tensor shared_down, const float *
 // One layer's routed experts and the layer's tail in one launch: fm_moe_decode_dev (without the
 // per-expert vectors) followed by fm_layer_tail_dev in its K = 0 form, bit for bit.  Shapes the
 // one-launch kernel does not cover (and calls under stream capture) run as those two launches.
-extern "C" int fm_moe_decode_tail_dev(fm_ctx *c, int layer, const float *d_x, const int32_t *d_idx,
-                                      const float *d_w, int K, fm_tensor shared_down, const float *d_h_mid,
-                                      const float *d_params, const float *d_shared_gate,
-                                      const float *d_shared_up, const uint16_t *d_next_norm_w, float eps,
-                                      float *d_hidden_out, float *d_next_input) {
-    if (!c) return FM_ERR_ARG;
+// route: the token's routing (fm_route_topk_dev) at the start of the same launch, over logits
+// that an earlier launch left in memory; d_idx / d_w / d_params are then outputs.
+static int decode_tail(fm_ctx *c, int layer, const float *d_x, const int32_t *d_idx, const float *d_w, int K,
+                       fm_tensor shared_down, const float *d_h_mid, const float *d_params,
+                       const float *d_shared_gate, const float *d_shared_up, const uint16_t *d_next_norm_w,
+                       float eps, float *d_hidden_out, float *d_next_input, const RouteArgs *route) {
     if (!c->aff_cfg) return fail(c, FM_ERR_STATE, "experts store not configured");
     Tensor *t = get_tensor(c, shared_down);
     if (!t) return fail(c, FM_ERR_ARG, "bad tensor handle %d", shared_down);
@@ -1342,6 +1342,14 @@ extern "C" int fm_moe_decode_tail_dev(fm_ctx *c, int layer, const float *d_x, co
         a.partial = c->d_tail;
         a.counter = (unsigned int *)(c->d_tail + FM_TAIL_PARTIALS);
         a.scale_fp16 = t->scale_fp16;
+        if (route) {
+            a.route_logits = route->logits;
+            a.route_n = route->n;
+            a.route_seg = route->seg_score;
+            a.route_idx = route->idx;
+            a.route_w = route->w;
+            a.route_params = route->params;
+        }
         rc = fm_launch_decode_affine(c->d_layer_ptrs, &c->geom, layer, 1, 1, d_x, d_idx, d_w, K, c->d_act, c->d_eo,
                                      d_hidden_out, &c->dflags, FM_INT_NO_EXPERT_OUT, c->n_cu, c->stream, nullptr, &a);
         if (rc == FM_OK) {
@@ -1351,13 +1359,53 @@ extern "C" int fm_moe_decode_tail_dev(fm_ctx *c, int layer, const float *d_x, co
         if (rc != FM_ERR_UNSUPPORTED)
             return fail(c, rc, "decode + tail launch failed: %s", hipGetErrorString(hipGetLastError()));
     }
-    // two launches: the experts' sum crosses in a vector of the tail's scratch
+    // separate launches: the routing if it was asked for, the experts (their sum crosses in a
+    // vector of the tail's scratch), the tail
+    if (route) {
+        rc = fm_route_topk_dev(c, route->logits, route->n, K, route->seg_score, route->idx, route->w, route->params);
+        if (rc) return rc;
+    }
     if (c->geom.hidden > FM_TAIL_VECTOR) return fail(c, FM_ERR_UNSUPPORTED, "hidden %d", c->geom.hidden);
     float *d_sum = c->d_tail + FM_TAIL_PARTIALS + 64;
     rc = fm_moe_decode_step_dev(c, layer, 1, d_x, d_idx, d_w, K, d_sum, nullptr, 0);
     if (rc) return rc;
     return fm_layer_tail_dev(c, shared_down, d_h_mid, d_sum, d_params, 0, d_shared_gate, d_shared_up,
                              d_next_norm_w, eps, d_hidden_out, d_next_input);
+}
+
+extern "C" int fm_moe_decode_tail_dev(fm_ctx *c, int layer, const float *d_x, const int32_t *d_idx,
+                                      const float *d_w, int K, fm_tensor shared_down, const float *d_h_mid,
+                                      const float *d_params, const float *d_shared_gate,
+                                      const float *d_shared_up, const uint16_t *d_next_norm_w, float eps,
+                                      float *d_hidden_out, float *d_next_input) {
+    if (!c) return FM_ERR_ARG;
+    return decode_tail(c, layer, d_x, d_idx, d_w, K, shared_down, d_h_mid, d_params, d_shared_gate, d_shared_up,
+                       d_next_norm_w, eps, d_hidden_out, d_next_input, nullptr);
+}
+
+// The MoE half of a layer in two launches: the routing batch (gate logits, the shared expert's
+// gate score and gate / up projections: fm_matvec_batch_dev over route_tensors[0..3], all from
+// d_x), then the routing, the routed experts and the tail in one.  Identical to
+// fm_matvec_batch_route_dev + fm_moe_decode_dev + fm_layer_tail_dev.
+extern "C" int fm_moe_layer_dev(fm_ctx *c, int layer, const fm_tensor *route_tensors, const float *d_x, int K,
+                                fm_tensor shared_down, const float *d_h_mid, const uint16_t *d_next_norm_w,
+                                float eps, float *d_logits, float *d_seg_score, float *d_shared_gate,
+                                float *d_shared_up, int32_t *d_idx, float *d_w, float *d_params,
+                                float *d_hidden_out, float *d_next_input) {
+    if (!c) return FM_ERR_ARG;
+    if (!route_tensors || !d_logits || !d_seg_score || !d_shared_gate || !d_shared_up || !d_idx || !d_w || !d_params)
+        return fail(c, FM_ERR_ARG, "null pointer");
+    Tensor *t0 = get_tensor(c, route_tensors[0]);
+    if (!t0) return fail(c, FM_ERR_ARG, "bad tensor handle %d", route_tensors[0]);
+    const int n_experts = t0->out_dim;
+    if (K < 1 || K > FM_MAX_K || K > n_experts)
+        return fail(c, FM_ERR_ARG, "K %d outside 1..min(%d, n_experts)", K, FM_MAX_K);
+    float *outs[4] = {d_logits, d_seg_score, d_shared_gate, d_shared_up};
+    int rc = matvec_dev(c, route_tensors, 4, d_x, outs, 1);
+    if (rc) return rc;
+    const RouteArgs ra{d_logits, n_experts, K, d_seg_score, d_idx, d_w, d_params};
+    return decode_tail(c, layer, d_x, d_idx, d_w, K, shared_down, d_h_mid, d_params, d_shared_gate, d_shared_up,
+                       d_next_norm_w, eps, d_hidden_out, d_next_input, &ra);
 }
 
 // ============================================================================

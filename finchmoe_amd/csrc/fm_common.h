@@ -78,6 +78,14 @@ struct FmTailArgs {
     float *partial;
     unsigned int *counter;
     int scale_fp16;          // scale type of W's groups (the launch with the experts in front only)
+    // the launch with the experts in front, optionally: the token's routing at its start (every
+    // workgroup runs it on the gate logits a launch before it left in memory) instead of expert
+    // indices and weights handed in; the results also go to route_idx / route_w / route_params
+    const float *route_logits;
+    int route_n;
+    const float *route_seg;
+    int32_t *route_idx;
+    float *route_w, *route_params;
 };
 
 // ---------------------------------------------------------------- device helpers

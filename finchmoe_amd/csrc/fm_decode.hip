@@ -28,6 +28,7 @@
 #include "fm_index.h"
 #include "fm_mfma.h"
 #include "fm_ring.h"
+#include "fm_route.h"
 
 #include <type_traits>
 
@@ -1048,14 +1049,41 @@ struct Fm2Stream {
         FmActX<LPR_UP> xr0, xr1;
         fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)(n_up > 0 ? gu_s0 : 0) * a.g.hidden, bslot, xr0);
         fm_act_load<BITS, LPR_UP, false>(a.x + (size_t)(n_up > 1 ? gu_s0 + 1 : 0) * a.g.hidden, bslot, xr1);
+        // TAIL with the routing inside: wave 0 of every workgroup routes the token (the same wave
+        // function as the routing kernel, on the same logits: the same indices and weights
+        // everywhere), into LDS; workgroup 0 also leaves them in memory for the caller
+        const int32_t *idx_src = a.idx;
+        const float *w_src = a.w;
+        if constexpr (TAIL) {
+            if (tp->route_logits) {
+                uint8_t *part_mem = fm_dyn_lds + D::WG_BYTES + 2 * IMG_UP + FM2_MAX_SEG * sizeof(Fm2Seg);
+                int32_t *r_idx = reinterpret_cast<int32_t *>(part_mem + FM2_PART_BYTES - FM2_ROUTE_WORDS);
+                float *r_w = reinterpret_cast<float *>(part_mem + FM2_PART_BYTES - FM2_ROUTE_WORDS + 32);
+                float *r_par = reinterpret_cast<float *>(part_mem + FM2_PART_BYTES - FM2_ROUTE_WORDS + 64);
+                if (wave == 0) {
+                    const RouteArgs ra{tp->route_logits, tp->route_n, K, tp->route_seg, r_idx, r_w, r_par};
+                    fm_route_wave<false>(ra, reinterpret_cast<float *>(part_mem));
+                    if (blockIdx.x == 0) {
+                        if (lane < K) {
+                            tp->route_idx[lane] = r_idx[lane];
+                            tp->route_w[lane] = r_w[lane];
+                        }
+                        if (tp->route_params && lane < 10) tp->route_params[lane] = r_par[lane];
+                    }
+                }
+                __syncthreads();
+                idx_src = r_idx;
+                w_src = r_w;
+            }
+        }
         if (mine) {
             const int k = threadIdx.x & 7;
             const size_t sg = mine_s;                              // layer group of the segment
             Fm2Seg &t = tab[qq];
             bool ok = false;
             if (k < K) {
-                const int e = a.idx[sg * K + k];
-                const float wv = a.w[sg * K + k];
+                const int e = idx_src[sg * K + k];
+                const float wv = w_src[sg * K + k];
                 ok = (unsigned)e < (unsigned)a.g.n_experts;
                 t.blob[k] = a.layer_ptrs[a.layer0 + (int)sg * a.layer_stride] + (size_t)(ok ? e : 0) * a.g.expert_size;
                 t.w[k] = ok ? wv : 0.0f;
@@ -1086,7 +1114,7 @@ struct Fm2Stream {
                              tp->B + (size_t)tw_row * tsb + (size_t)tc * 4);
             const int rows = t_nrb * RPS_DN, tr = (int)threadIdx.x < rows ? (int)threadIdx.x : (rows > 0 ? rows - 1 : 0);
             t_hm = tp->h_mid[t_row0 + tr];
-            t_score = tp->params[8];
+            t_score = tp->route_logits ? (tp->route_seg ? *tp->route_seg : 0.0f) : tp->params[8];
             t_nw = tp->next_in ? (uint32_t)tp->norm_w[t_row0 + tr] : 0u;
             const int tj = (int)threadIdx.x < tp->inter ? (int)threadIdx.x : tp->inter - 1;
             const float tact = fm_silu_mul(tp->shared_gate[tj], tp->shared_up[tj]);
@@ -1393,6 +1421,7 @@ int launch_fused_rows_tail(const DecodeArgs &a, int n_pairs, int n_cu, hipStream
     // the rows of the experts' sum, its wave step their row block), 4-bit; every workgroup owns
     // at least one row block and the tail's tables fit beside its partial vectors
     if (n_pairs != a.K || ta.hidden != a.g.hidden || ta.inter != a.g.inter || ta.K != 0) return FM_ERR_UNSUPPORTED;
+    if (ta.route_logits && (!fm2_route_fits(ta.route_n) || ta.route_n > FM_ROUTE_MAX || a.K > ta.route_n)) return FM_ERR_UNSUPPORTED;
     const Fm2Plan plan = fm2_plan(n_pairs, a.K, a.g.inter, a.g.hidden, LPR_UP, n_cu);
     if (!plan.ok) return FM_ERR_UNSUPPORTED;
     const int rps_dn = FM_WAVE / (LPR_UP / 4), dn_rbs = a.g.hidden / rps_dn;

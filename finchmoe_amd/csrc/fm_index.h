@@ -486,13 +486,18 @@ struct Fm2TailLds {
     int ok;
     uint32_t so, act, red, word;     // byte offsets inside the partial-vector area
 };
+// (the routing at the launch's start uses the area before any of this: n softmax values from its
+// first byte, and indices / weights / params in its last FM2_ROUTE_WORDS bytes, which stay until
+// the segment tables are built)
+#define FM2_ROUTE_WORDS 128
+FM_HD int fm2_route_fits(int n) { return n >= 1 && (size_t)n * 4 + FM2_ROUTE_WORDS <= FM2_PART_BYTES; }
 FM_HD Fm2TailLds fm2_tail_lds(int nrb, int K, int rps_dn, int shared_inter, int hidden) {
     Fm2TailLds t;
     t.so = (uint32_t)(nrb * K * rps_dn * 4);                 // behind the partial vectors
     t.act = (t.so + (uint32_t)(nrb * rps_dn * 4) + 15u) & ~15u;
     t.red = t.act + (uint32_t)shared_inter * 4u;
     t.word = t.red + (uint32_t)(hidden / rps_dn) * 4u;
-    t.ok = nrb >= 1 && nrb <= 8 && shared_inter <= 512 && t.word + 16u <= FM2_PART_BYTES;
+    t.ok = nrb >= 1 && nrb <= 8 && shared_inter <= 512 && t.word + 16u <= FM2_PART_BYTES - FM2_ROUTE_WORDS;
     return t;
 }
 // the launcher's decision: workgroups, and whether the shape fits the kernel's fixed tables

@@ -302,6 +302,23 @@ FM_API int fm_moe_decode_tail_dev(fm_ctx *ctx, int layer, const float *d_x, cons
                            const float *d_shared_up, const uint16_t *d_next_norm_w, float eps,
                            float *d_hidden_out, float *d_next_input);
 
+/* The MoE half of a layer (finchmoe/infer.m:9285-9760: routing_batch_fused, the CPU routing,
+ * CMD3) in two launches and without a host round trip:
+ *   route_tensors[4] = router gate [n_experts][hidden] (8-bit upstream), shared-expert gate
+ *   [1][hidden], shared expert's gate and up projections [inter][hidden] — all multiplied with
+ *   d_x in the first launch (fm_matvec_batch_dev), results in d_logits, d_seg_score,
+ *   d_shared_gate, d_shared_up;
+ *   second launch: softmax + top-K + normalisation of the logits (every workgroup runs the
+ *   routing wave on them; d_idx, d_w, d_params[10] receive the result), the routed experts of
+ *   `layer` on d_x, and the layer tail as fm_moe_decode_tail_dev.
+ * Identical to fm_matvec_batch_route_dev + fm_moe_decode_dev + fm_layer_tail_dev (K = 0 form);
+ * shapes the one-launch kernel does not cover run as those launches. */
+FM_API int fm_moe_layer_dev(fm_ctx *ctx, int layer, const fm_tensor *route_tensors, const float *d_x, int K,
+                     fm_tensor shared_down, const float *d_h_mid, const uint16_t *d_next_norm_w,
+                     float eps, float *d_logits, float *d_seg_score, float *d_shared_gate,
+                     float *d_shared_up, int32_t *d_idx, float *d_w, float *d_params,
+                     float *d_hidden_out, float *d_next_input);
+
 /* ---------------------------------------------------------------- GGUF expert store
  * Replaces GgufExpertInfo + the slab copies of gpu_gguf_experts_forward
  * (finchmoe/infer.m:1017-1022, 3239-3290).  gate/up/down are the stacked

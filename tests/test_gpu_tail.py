@@ -249,6 +249,23 @@ def _moe_half(hip, orc):
                             d_p.data_ptr(), d_sg.data_ptr(), d_su.data_ptr(), None, 1e-6, d_hid4.data_ptr(), None)
     hip.sync()
     assert torch.equal(d_hid4, d_hid)
+    # the whole MoE half in two launches (routing batch; routing + experts + tail): every
+    # intermediate and both results bit for bit the chain above, three times in a row
+    for rep in range(3):
+        o_log, o_seg = torch.zeros(Ee, device="cuda"), torch.zeros(1, device="cuda")
+        o_sg, o_su = torch.zeros(Ii, device="cuda"), torch.zeros(Ii, device="cuda")
+        o_idx = torch.zeros(Kk, dtype=torch.int32, device="cuda")
+        o_w, o_p = torch.zeros(Kk, device="cuda"), torch.full((10,), 9.0, device="cuda")
+        o_hid, o_next = torch.zeros(Hh, device="cuda"), torch.zeros(Hh, device="cuda")
+        torch.cuda.synchronize()
+        hip.moe_layer_dev(0, [t_gate, t_seg, t_sg, t_su], d_x.data_ptr(), Kk, t_sd, d_hmid.data_ptr(),
+                          d_nw.data_ptr(), 1e-6, o_log.data_ptr(), o_seg.data_ptr(), o_sg.data_ptr(),
+                          o_su.data_ptr(), o_idx.data_ptr(), o_w.data_ptr(), o_p.data_ptr(), o_hid.data_ptr(),
+                          o_next.data_ptr())
+        hip.sync()
+        for got, want in zip((o_log, o_seg, o_sg, o_su, o_idx, o_w, o_p), keep):
+            assert torch.equal(got, want), rep
+        assert torch.equal(o_hid, d_hid) and torch.equal(o_next, d_next), rep
     # fewer slots than eight, and a slot with an index outside the store (weight 0 upstream)
     idx5 = d_idx.clone()
     idx5[2] = Ee + 7
