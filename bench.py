@@ -915,13 +915,19 @@ def run_gguf(args):
     k1, k2, n = ctx.kernel_timing_read()
     ctx.kernel_timing(0)
     assert torch.isfinite(d_out).all()
-    res = {"kernels_us": {"fm_gguf_gate_up": round(k1 / n * 1e3, 2),
-                          "fm_gguf_down+combine": round(k2 / n * 1e3, 2)},
+    phases = any(f in args.forms for f in ("gguf-phases", "plain-gguf"))
+    res = {"kernels_us": {"fm_gguf_gate_up (as three launches)": round(k1 / n * 1e3, 2),
+                          "fm_gguf_down+combine (as three launches)": round(k2 / n * 1e3, 2)},
            "event_ms_per_step": round(ev, 5), "us_per_layer": round(ms * 1e3 / n_layers, 3),
-           "tokens_per_s": round(1e3 / ms, 1),
-           # the dominant kernel: the Q4_K gate/up stream (its own events, isolated launches)
-           "roofline": _roofline_hbm("fm_gguf_stream<Q4_K,16,gate/up> (first of the step's three launches)",
-                                     n_layers * K * 2 * gsl, k1 / n * 1e3)}
+           "tokens_per_s": round(1e3 / ms, 1), "launches_per_step": 3 if phases else 1}
+    if phases:
+        # the dominant kernel: the Q4_K gate/up stream (its own events, isolated launches)
+        res["roofline"] = _roofline_hbm("fm_gguf_stream<Q4_K,16,gate/up> (first of the step's three launches)",
+                                        n_layers * K * 2 * gsl, k1 / n * 1e3)
+    else:
+        # the step is one launch: HIP events around the timed region on the library's stream
+        res["roofline"] = _roofline_hbm("fm_gguf_fused_rows<Q6_K,16,8> (the step's one launch)",
+                                        n_layers * K * (2 * gsl + dsl), ev * 1e3)
     res["roofline"]["step"] = {"bytes": n_layers * K * (2 * gsl + dsl), "us": round(ev * 1e3, 2),
                                "frac": round(n_layers * K * (2 * gsl + dsl) / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     if not args.no_cpu:
@@ -1133,7 +1139,8 @@ def main():
     if args.forms:
         from finchmoe_amd import binding as fb
         known = {"plain-dense": fb.FORM_PLAIN_DENSE, "plain-gguf": fb.FORM_PLAIN_GGUF,
-                 "per-position": fb.FORM_NO_DENSE_GEMM | fb.FORM_NO_GGUF_GROUP, "three-launches": 0}
+                 "per-position": fb.FORM_NO_DENSE_GEMM | fb.FORM_NO_GGUF_GROUP, "three-launches": 0,
+                 "gguf-phases": fb.FORM_GGUF_PHASES}
         bad = [f for f in args.forms if f not in known]
         if bad:
             print("bench.py: unknown --forms %s (have: %s)" % (bad, ", ".join(known)), file=sys.stderr)

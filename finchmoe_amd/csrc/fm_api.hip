@@ -41,7 +41,7 @@ int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t *const *d_
                           const uint8_t *const *d_down, const FmGgufGeom *g, int layer0,
                           int layer_stride, int n_layers, const float *d_x,
                           const int32_t *d_idx, const float *d_w, int K, float *d_act,
-                          float *d_expert_out, float *d_out, unsigned int *d_counters,
+                          float *d_expert_out, float *d_out, FmDecodeFlags *df,
                           int flags, int n_cu, hipStream_t st, hipEvent_t *kev);
 int fm_launch_gguf_matvec(const uint8_t *d_W, int ggml_type, const float *d_x, float *d_out,
                           int out_dim, int in_dim, int n_cu, hipStream_t st);
@@ -337,7 +337,8 @@ size_t gguf_row_bytes(int in_dim, int type) {
 unsigned int fm_kernel_forms = 0;
 
 extern "C" int fm_set_kernel_forms(unsigned int forms) {
-    if (forms & ~(unsigned)(FM_FORM_PLAIN_DENSE | FM_FORM_PLAIN_GGUF | FM_FORM_NO_DENSE_GEMM | FM_FORM_NO_GGUF_GROUP))
+    if (forms & ~(unsigned)(FM_FORM_PLAIN_DENSE | FM_FORM_PLAIN_GGUF | FM_FORM_NO_DENSE_GEMM | FM_FORM_NO_GGUF_GROUP |
+                           FM_FORM_GGUF_PHASES))
         return FM_ERR_ARG;
     fm_kernel_forms = forms;
     return FM_OK;
@@ -1531,9 +1532,12 @@ static int gguf_decode_groups(fm_ctx *c, int layer0, int layer_stride, int group
     rc = fm_launch_decode_gguf(c->d_gg_ptrs, c->d_gg_ptrs + c->g_layers,
                                c->d_gg_ptrs + 2 * (size_t)c->g_layers, &c->ggeom, layer0,
                                layer_stride, groups, d_x, d_idx, d_w, K, c->d_act,
-                               d_expert_out ? d_expert_out : c->d_eo, d_out, c->d_counters, flags,
+                               d_expert_out ? d_expert_out : c->d_eo, d_out,
+                               c->split_phases ? nullptr : &c->dflags,
+                               flags | (d_expert_out ? 0 : FM_INT_NO_EXPERT_OUT),
                                c->n_cu, c->stream, c->ktiming ? c->kev : nullptr);
     if (rc) return fail(c, rc, "GGUF decode launch failed: %s", hipGetErrorString(hipGetLastError()));
+    if (!c->split_phases) c->sync_unchecked = true;     // (the one-launch form may have run: its waits are bounded)
     if (c->ktiming) return ktiming_collect(c);
     return FM_OK;
 }

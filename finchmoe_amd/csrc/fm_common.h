@@ -45,6 +45,16 @@ struct FmDecodeFlags {
     int act_parity;
 };
 
+// What an element of an activation set holds until its producer has stored it (a NaN that no
+// arithmetic yields), and the part of a launch's arguments that concerns the sets.
+#define FM_ACT_EMPTY 0xFFC5A3E1u
+struct Fm2Sync {
+    float *act_other;        // the activation set of the previous and of the next launch
+    unsigned int clear_n;    // floats of it to mark empty
+    unsigned int *err;       // host memory
+    unsigned int spin_limit;
+};
+
 // internal launch flag (above the public FM_* bits): the caller has no use for the per-expert
 // vectors
 #define FM_INT_NO_EXPERT_OUT (1 << 16)

@@ -54,17 +54,6 @@ struct DecodeArgs {
     int flags;
 };
 
-// The intermediate vectors (act, expert_out) are written by one phase and read
-// by the next, possibly inside one launch and from a CU behind another L2.
-// They are stored and loaded as device-scope relaxed atomics: such accesses are
-// performed at the level all CUs share, so a consumer that starts after the
-// producer's stores have completed sees them without any cache maintenance.
-__device__ __forceinline__ void fm_st_shared(float *p, float v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float fm_ld_shared(const float *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
 // ---------------------------------------------------------------- kernel 1
 template <int BITS, int LPR, bool FP16>
@@ -729,7 +718,7 @@ void fm_moe_fused(DecodeArgs a, int n_pairs, FmFlags f) {
 // LDS is accessed with explicit instructions (the compiler would order a visible LDS access
 // behind every LDS-direct load in flight), barriers likewise.
 // ======================================================================
-constexpr uint32_t FM_ACT_EMPTY = 0xFFC5A3E1u;
+// (FM_ACT_EMPTY and Fm2Sync: fm_common.h)
 // FM2_MAX_SEG segments of one workgroup's shares and FM2_PART_BYTES of partial vectors of a part:
 // fm_index.h
 
@@ -743,32 +732,13 @@ struct Fm2Seg {
     int pad;
 };
 
-struct Fm2Sync {
-    float *act_other;        // the activation set of the previous and of the next launch
-    unsigned int clear_n;    // floats of it to mark empty
-    unsigned int *err;       // host memory
-    unsigned int spin_limit;
-};
-
 template <int BITS, int LPR>
 constexpr size_t fm2_lds_bytes() {
     return FmDma<BITS>::WG_BYTES + 2 * sizeof(FmActLds<LPR>) + FM2_MAX_SEG * sizeof(Fm2Seg) +
            FM2_PART_BYTES;
 }
 
-__device__ __forceinline__ void fm_lds_w32(uint32_t addr, uint32_t v) {
-    asm volatile("ds_write_b32 %0, %1" ::"v"(addr), "v"(v) : "memory");
-}
-__device__ __forceinline__ uint32_t fm_lds_r32(uint32_t addr) {
-    uint32_t v;
-    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
-    return v;
-}
-// workgroup barrier that waits for this wave's LDS operations only (the compiler's own puts a
-// wait for every LDS-direct load in front)
-__device__ __forceinline__ void fm_wg_barrier() {
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
+// (fm_lds_w32 / fm_lds_r32 / fm_wg_barrier: fm_ring.h)
 
 // fm_read_act_lds with explicit instructions; img = LDS address of the image
 template <int LPR>

@@ -906,6 +906,478 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
 #endif
 }
 
+// ======================================================================
+// The operator as one launch when the caller does not want the per-expert vectors and the
+// plain combine applies: the form of fm_moe_fused_rows (fm_decode.hip) for block formats.
+//
+// Gate/up: contiguous ranges of units (a unit = the gate slice and the up slice of a wave step),
+// SwiGLU, activations stored at device scope into a set whose elements hold FM_ACT_EMPTY until
+// then.  Down by row blocks: a row block is one wave step's rows of all K experts of a layer; a
+// workgroup owns whole output rows of ONE layer (fm2_split), polls that layer's K activation
+// vectors into K images, keeps the K partial vectors of its rows in LDS and adds them up itself,
+// w_k * down_k in slot order — fm_gguf_combine<false>'s arithmetic.  No per-expert vectors, no
+// combine launch, nobody waits for the slowest workgroup of the grid.  The shares are sized so
+// that every workgroup streams the same number of bytes.
+//
+// A gate/up slice and a down slice differ in size, so the ring changes geometry between the
+// phases: the loader does not run on from the last gate/up unit into the down phase; a wave
+// refills its ring with down slices as soon as it has consumed its last gate/up slice, before
+// the workgroup's barrier and the polls.
+// ======================================================================
+struct __attribute__((aligned(16))) GgSeg {
+    uint64_t first[FM_MAX_K];      // gate (or down) rows of slot k's expert
+    int64_t second[FM_MAX_K];      // up rows - gate rows
+    float w[FM_MAX_K];             // router weight, 0 for an invalid expert index
+    uint32_t valid;                // bit k: slot k has a valid expert index
+    uint32_t next_unit;
+    uint32_t first_unit, n;        // this workgroup's units of the segment
+    int layer;                     // layer group
+    int pad[3];
+};
+static_assert(sizeof(GgSeg) == FM_GG2_SEG_BYTES, "segment table entry");
+
+template <int DN_KIND, int LPR_UP, int LPR_DN>
+struct GgFused {
+    using GU = GgLane<GG_Q4, LPR_UP>;
+    using GD = GgLane<DN_KIND, LPR_DN>;
+    using LaneD = typename GgLaneOps<DN_KIND>::Lane;
+    using DataD = typename GgLaneOps<DN_KIND>::Data;
+    using ImageU = GgImage<GU::NREG, LPR_UP>;
+    using ImageD = GgImage<GD::NREG, LPR_DN>;
+    static constexpr int RPS_UP = FM_WAVE / LPR_UP, RPS_DN = FM_WAVE / LPR_DN;
+    static constexpr int RING_UP = FM_GG2_RING_UP, RING_DN = DN_KIND == GG_Q6 ? 4 : 3;
+    static constexpr int SLOT_UP = GU::SLOT_DATA + 16, SLOT_DN = GD::SLOT_DATA + 16;
+    static constexpr int LOADS_UP = (GU::SLOT_DATA + 1023) / 1024, LOADS_DN = (GD::SLOT_DATA + 1023) / 1024;
+    static constexpr int RING_BYTES = RING_UP * SLOT_UP > RING_DN * SLOT_DN ? RING_UP * SLOT_UP : RING_DN * SLOT_DN;
+    static constexpr int IMG_UP = (int)sizeof(ImageU), IMG_DN = (int)sizeof(ImageD);
+    static constexpr int IMG_BYTES = 2 * IMG_UP > FM_MAX_K * IMG_DN ? 2 * IMG_UP : FM_MAX_K * IMG_DN;
+    static constexpr int LDS_BYTES = 8 * RING_BYTES + IMG_BYTES + FM2_MAX_SEG * (int)sizeof(GgSeg) + FM2_PART_BYTES;
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+
+    const GgufArgs &a;
+    const Fm2Sync &sy;
+    int lane, wave;
+    uint32_t ring0, img0, part0;
+    GgSeg *tab;
+    FmDiv by_gu_upp, by_K;
+    int n_up, n_seq;
+    // loader
+    bool l_gu, dry;
+    int lq, cq, hn, wpos, c;
+    uint32_t l_first, l_n, l_nrb, tag_n, issued, consumed;
+    float l_inv;
+    const uint8_t *src_n;
+    ptrdiff_t second_n;
+    uint32_t ones;
+
+    __device__ __forceinline__ GgFused(const GgufArgs &a_, const Fm2Sync &sy_) : a(a_), sy(sy_) {
+        lane = threadIdx.x & 63;
+        wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const uint32_t lds0 = fm_lds_addr(fm_gguf_lds);
+        ring0 = lds0 + (uint32_t)wave * RING_BYTES;
+        img0 = lds0 + 8u * RING_BYTES;
+        tab = reinterpret_cast<GgSeg *>(fm_gguf_lds + 8 * RING_BYTES + IMG_BYTES);
+        part0 = img0 + (uint32_t)IMG_BYTES + FM2_MAX_SEG * (uint32_t)sizeof(GgSeg);
+        l_gu = true, dry = false;
+        lq = cq = hn = wpos = c = 0;
+        l_first = l_n = l_nrb = tag_n = issued = consumed = 0u;
+        l_inv = 0.0f;
+        src_n = nullptr;
+        second_n = 0;
+        ones = fm_opaque(0x3F803F80u);
+    }
+
+    __device__ __forceinline__ void loader_enter(int q) {
+        const uint32_t ta = fm_lds_addr(&tab[q].first_unit);
+        l_first = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta));
+        l_n = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + 4));
+        if (!l_gu) {
+            l_nrb = fm_div(by_K, l_n);
+            l_first = fm_div(by_K, l_first);            // first row block of the part
+            l_inv = 1.0f / (float)(l_nrb ? l_nrb : 1u);
+        }
+    }
+
+    // the next slice of the loader's phase into the ring's write position
+    template <bool GATE_UP>
+    __device__ __forceinline__ void issue() {
+        constexpr int RING = GATE_UP ? RING_UP : RING_DN, SLOT = GATE_UP ? SLOT_UP : SLOT_DN;
+        constexpr int DATA = GATE_UP ? GU::SLOT_DATA : GD::SLOT_DATA;
+        if (dry) return;
+        if (!GATE_UP || hn == 0) {
+            uint32_t ul;
+            const int q_end = GATE_UP ? n_up : n_seq;
+            for (;;) {
+                ul = fm_claim_unit(&tab[lq].next_unit, lane);
+                if (ul < l_n) break;
+                if (lq + 1 < q_end && lq == cq) {       // run on into the next segment of the phase
+                    lq++;
+                    loader_enter(lq);
+                    continue;
+                }
+                dry = true;
+                return;
+            }
+            uint32_t pn, rsn;
+            if (GATE_UP) fm2_gu_unit(l_first, ul, by_gu_upp, &pn, &rsn);
+            else fm2_dn_unit(l_first, l_nrb, l_inv, ul, &pn, &rsn);     // expert by expert
+            tag_n = ((uint32_t)(lq & 1) << 31) | (pn << 28) | ul;
+            const uint32_t fa = fm_lds_addr(&tab[lq].first[pn]);
+            const uint32_t lo = __builtin_amdgcn_readfirstlane(fm_lds_r32(fa));
+            const uint32_t hi = __builtin_amdgcn_readfirstlane(fm_lds_r32(fa + 4));
+            src_n = (const uint8_t *)(((uintptr_t)hi << 32) | lo) + (size_t)rsn * DATA;
+            if (GATE_UP) {
+                const uint32_t sa = fm_lds_addr(&tab[lq].second[pn]);
+                const uint32_t slo = __builtin_amdgcn_readfirstlane(fm_lds_r32(sa));
+                const uint32_t shi = __builtin_amdgcn_readfirstlane(fm_lds_r32(sa + 4));
+                second_n = (ptrdiff_t)(((uint64_t)shi << 32) | slo);
+            }
+        }
+        const uint32_t slot = ring0 + (uint32_t)wpos * SLOT;
+        fm_slot_tag(slot + DATA, tag_n);
+        const uint8_t *src = src_n + (GATE_UP ? (ptrdiff_t)hn * second_n : (ptrdiff_t)0) + lane * 16;
+        gg_dma<DATA, 0>(slot, src, lane);
+        if (GATE_UP) hn ^= 1;
+        wpos = wpos + 1 == RING ? 0 : wpos + 1;
+        issued++;
+    }
+
+    // The next slice out of the ring into registers, its tag, and the slot handed back to the
+    // loader at once.  The consumer fetches a slice before it multiplies the one fetched before,
+    // so a slice that lands while the wave is busy does not keep its slot (measured: no
+    // difference against fetching and multiplying in turn; the launch is bound by the stream).
+    __device__ __forceinline__ uint32_t fetch_up(const GgQ4Lane &ln, Q4Half &t) {
+        if (issued - consumed == (uint32_t)RING_UP) fm_dma_wait<LOADS_UP *(RING_UP - 1)>(false);
+        else fm_dma_wait<0>(true);
+        const uint32_t slot = ring0 + (uint32_t)c * SLOT_UP;
+        const fm_u4 tag = ln.read(slot, slot + GU::SLOT_DATA, t);
+        consumed++;
+        c = c + 1 == RING_UP ? 0 : c + 1;
+        issue<true>();
+        return __builtin_amdgcn_readfirstlane(tag[0]);
+    }
+    __device__ __forceinline__ uint32_t fetch_dn(const LaneD &ln, DataD &t) {
+        if (issued - consumed == (uint32_t)RING_DN) fm_dma_wait<LOADS_DN *(RING_DN - 1)>(false);
+        else fm_dma_wait<0>(true);
+        const uint32_t slot = ring0 + (uint32_t)c * SLOT_DN;
+        const fm_u4 tag = ln.read(slot, slot + GD::SLOT_DATA, t);
+        consumed++;
+        c = c + 1 == RING_DN ? 0 : c + 1;
+        issue<false>();
+        return __builtin_amdgcn_readfirstlane(tag[0]);
+    }
+
+    __device__ __forceinline__ int seg_layer(int q) const {
+        return __builtin_amdgcn_readfirstlane((int)fm_lds_r32(fm_lds_addr(&tab[q].layer)));
+    }
+
+    // an activation produced in this launch: polled until it is there
+    __device__ __forceinline__ float act_get(const float *p) const {
+        unsigned int polls = 0;
+        for (;;) {
+            const float v = fm_ld_shared(p);
+            if (__float_as_uint(v) != FM_ACT_EMPTY) return v;
+            if (++polls > sy.spin_limit) {
+                __hip_atomic_store(sy.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                return 0.0f;
+            }
+            __builtin_amdgcn_s_sleep(8);
+        }
+    }
+
+    // w_k * partial_k over the part's rows, in slot order -> out
+    __device__ __forceinline__ void reduce_part(int q) {
+        const int K = a.K;
+        const uint32_t ta = fm_lds_addr(&tab[q]);
+        const uint32_t first = fm_lds_r32(ta + (uint32_t)offsetof(GgSeg, first_unit));
+        const uint32_t n = fm_lds_r32(ta + (uint32_t)offsetof(GgSeg, n));
+        float wk[FM_MAX_K];
+#pragma unroll
+        for (int k = 0; k < FM_MAX_K; k++)
+            wk[k] = k < K ? __uint_as_float(fm_lds_r32(ta + (uint32_t)offsetof(GgSeg, w) + 4u * k)) : 0.0f;
+        const int rows = (int)fm_div(by_K, n) * RPS_DN;
+        const int l = seg_layer(q);
+        float *out = a.out + (size_t)l * a.g.hidden + (size_t)fm_div(by_K, first) * RPS_DN;
+        for (int r = threadIdx.x; r < rows; r += 512) {
+            const int rbi = r / RPS_DN, ris = r - rbi * RPS_DN;
+            float acc = 0.0f;
+#pragma unroll
+            for (int k = 0; k < FM_MAX_K; k++)
+                if (k < K && wk[k] != 0.0f)
+                    acc += wk[k] * __uint_as_float(fm_lds_r32(part0 + 4u * (uint32_t)((rbi * K + k) * RPS_DN + ris)));
+            out[r] = (a.flags & FM_ACCUMULATE) ? out[r] + acc : acc;
+        }
+    }
+
+    // The K activation vectors of layer l -> K down images.  Thread t takes the (image, chunk,
+    // register) combinations t, t + 512, ...: all loads first, polls where needed after.
+    __device__ __forceinline__ void build_down_images(int l) {
+        constexpr int NREG = GD::NREG, PER = LPR_DN * NREG, NE = 4 * LPR_DN;
+        constexpr int NIT = FM_MAX_K * PER / 512;
+        static_assert(FM_MAX_K * PER % 512 == 0 && PER % 64 == 0, "whole waves per image");
+        const int K = a.K;
+        float xl[NIT], xh[NIT];
+#pragma unroll
+        for (int i = 0; i < NIT; i++) {
+            const int it = (int)threadIdx.x + 512 * i;
+            const int k = it / PER, rem = it - k * PER, ch = rem / NREG, r = rem - ch * NREG;
+            const int lo = 32 * (r >> 4) + 4 * ((r & 15) >> 1) + (r & 1);
+            const float *src = a.act + ((size_t)l * K + (k < K ? k : 0)) * a.g.inter;
+            xl[i] = fm_ld_shared(src + GD::col(ch, lo));
+            xh[i] = fm_ld_shared(src + GD::col(ch, lo + 2));
+        }
+#pragma unroll
+        for (int i = 0; i < NIT; i++) {
+            const int it = (int)threadIdx.x + 512 * i;
+            const int k = it / PER, rem = it - k * PER, ch = rem / NREG, r = rem - ch * NREG;
+            const int lo = 32 * (r >> 4) + 4 * ((r & 15) >> 1) + (r & 1);
+            const bool on = k < K;
+            const float *src = a.act + ((size_t)l * K + (on ? k : 0)) * a.g.inter;
+            if (__float_as_uint(xl[i]) == FM_ACT_EMPTY) xl[i] = act_get(src + GD::col(ch, lo));
+            if (__float_as_uint(xh[i]) == FM_ACT_EMPTY) xh[i] = act_get(src + GD::col(ch, lo + 2));
+            // gg_build_image's arithmetic with explicit LDS writes
+            const float vl = xl[i] * 128.0f, vh = xh[i] * 128.0f;
+            const uint32_t l0 = __float_as_uint(vl) & 0xFFFF0000u, h0 = __float_as_uint(vh) & 0xFFFF0000u;
+            float rl = vl - __uint_as_float(l0), rh = vh - __uint_as_float(h0);
+            const uint32_t l1 = __float_as_uint(rl) & 0xFFFF0000u, h1 = __float_as_uint(rh) & 0xFFFF0000u;
+            rl -= __uint_as_float(l1);
+            rh -= __uint_as_float(h1);
+            const uint32_t l2 = __float_as_uint(rl), h2 = __float_as_uint(rh) & 0xFFFF0000u;
+            const float gs = fm_group_sum<GD::GROUP_REGS>(xl[i] + xh[i]);
+            if (on) {
+                const uint32_t img = img0 + (uint32_t)k * IMG_DN;
+                const uint32_t dst = img + (uint32_t)((((r >> 2) * NE + 4 * ch) * 4 + (r & 3)) * 4);
+                fm_lds_w32(dst, (l0 >> 16) | h0);
+                fm_lds_w32(dst + 16, (l1 >> 16) | h1);
+                fm_lds_w32(dst + 32, (l2 >> 16) | h2);
+                fm_lds_w32(dst + 48, 0u);
+                if (r % GD::GROUP_REGS == 0)
+                    fm_lds_w32(img + (uint32_t)((NREG / 4) * NE * 16 + ch * 16 + (r / GD::GROUP_REGS) * 4),
+                               __float_as_uint(gs));
+            }
+        }
+    }
+
+    __device__ __forceinline__ void run(const Fm2Dims &dm) {
+        const int K = a.K, G = gridDim.x, g = blockIdx.x;
+        by_gu_upp = dm.by_gu_upp, by_K = dm.by_K;
+        const Fm2Split sp = fm2_split(dm, (uint32_t)g);
+        const uint32_t gu_segu = dm.gu_segu;
+        n_up = sp.n_up;
+        n_seq = sp.n_up + sp.n_dn;
+        const int qq = threadIdx.x >> 3;        // the segment this thread looks up below
+        const bool mine = qq < n_seq;
+        const Fm2Part mp = fm2_part(dm, sp, mine ? qq : 0);
+
+        // the other activation set becomes empty again (plain stores, nobody reads it now)
+        for (unsigned int i = blockIdx.x * blockDim.x + threadIdx.x; i < sy.clear_n; i += G * blockDim.x)
+            sy.act_other[i] = __uint_as_float(FM_ACT_EMPTY);
+        if (n_seq == 0) return;
+
+        // the tables of every segment: thread 8q + k looks up slot k of segment q
+        if (mine) {
+            const int k = threadIdx.x & 7;
+            const size_t sg = mp.seg;
+            GgSeg &t = tab[qq];
+            bool ok = false;
+            if (k < K) {
+                int e = a.idx[sg * K + k];
+                const float wv = a.w[sg * K + k];
+                ok = (unsigned)e < (unsigned)a.g.n_experts;
+                if (!ok) e = 0;                          // stream something valid, count zeros
+                const int li = a.layer0 + (int)sg * a.layer_stride;
+                if (mp.gu) {
+                    const uint8_t *gp = a.gate[li] + (size_t)e * a.g.gate_slab;
+                    t.first[k] = (uint64_t)(uintptr_t)gp;
+                    t.second[k] = (int64_t)((a.up[li] + (size_t)e * a.g.up_slab) - gp);
+                } else {
+                    t.first[k] = (uint64_t)(uintptr_t)(a.down[li] + (size_t)e * a.g.down_slab);
+                    t.second[k] = 0;
+                }
+                t.w[k] = ok ? wv : 0.0f;
+            }
+            const uint64_t m = __ballot(ok);
+            if (k == 0) {
+                t.valid = (uint32_t)(m >> (threadIdx.x & 56)) & 0xFFu;
+                t.next_unit = 0u;
+                t.first_unit = mp.first;
+                t.n = mp.n;
+                t.layer = (int)sg;
+            }
+        }
+        __syncthreads();
+
+        const int j = lane & 3;
+        // ---------------------------------------------------------- gate/up
+        if (n_up > 0) {
+            loader_enter(0);
+#pragma nounroll
+            for (int k = 0; k < RING_UP; k++) issue<true>();
+            // the images of both gate/up segments; a wave then changes segment on its own
+            ImageU *img = reinterpret_cast<ImageU *>(fm_gguf_lds + 8 * RING_BYTES);
+            for (int v = 0; v < n_up && v < 2; v++)
+                gg_build_image<GG_Q4, LPR_UP>(a.x + (size_t)(sp.gu_s0 + v) * a.g.hidden, img[v]);
+            __syncthreads();
+
+            const int ch = (lane >> 2) % LPR_UP, ris = 4 * (lane / (4 * LPR_UP)) + j;
+            GgQ4Lane ln;
+            ln.template init<LPR_UP>(ris, ch);
+            Q4Half ta_, tb_;                  // gate slice of the unit in hand, its up slice
+            uint32_t tag_a = 0u;
+            bool have = false;
+            for (; cq < n_up; cq++) {
+                const int s = seg_layer(cq);
+                GgAct<GU::NREG> ar;
+                gg_read_image<GU::NREG>(img0 + (uint32_t)(cq & 1) * IMG_UP, 4 * LPR_UP, lane, ar);
+                const uint32_t ta = fm_lds_addr(&tab[cq]);
+                const uint32_t valid = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(GgSeg, valid)));
+                const uint32_t c_first = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(GgSeg, first_unit)));
+                const size_t out0 = ((size_t)s * gu_segu + c_first) * RPS_UP + ris;
+                dry = false;
+                while (issued - consumed < (uint32_t)RING_UP && !dry) issue<true>();
+                if (!have && consumed < issued) {
+                    tag_a = fetch_up(ln, ta_);
+                    have = true;
+                }
+                while (have) {
+                    if ((tag_a >> 31) != (uint32_t)(cq & 1)) break;      // the next segment's: it waits in the registers
+                    const uint32_t pc = (tag_a >> 28) & 7u, ul = tag_a & 0x0FFFFFFFu;
+                    (void)fetch_up(ln, tb_);                             // (the up slice follows its gate slice)
+                    const float gv = fm_chunk_sum<LPR_UP>(ln.dot(ta_, ar, ones));
+                    have = consumed < issued;
+                    if (have) tag_a = fetch_up(ln, ta_);
+                    const float uv = fm_chunk_sum<LPR_UP>(ln.dot(tb_, ar, ones));
+                    float v = fm_silu_mul(gv, uv);
+                    if (!((valid >> pc) & 1u)) v = 0.0f;
+                    if (ch == 0) fm_st_shared(a.act + out0 + (size_t)ul * RPS_UP, v);
+                }
+            }
+        }
+        // ---------------------------------------------------------- down
+        if (n_seq > n_up) {
+            // the ring is empty: its geometry changes
+            l_gu = false;
+            dry = false;
+            hn = wpos = c = 0;
+            issued = consumed = 0u;
+            lq = cq = n_up;
+            loader_enter(lq);
+#pragma nounroll
+            for (int k = 0; k < RING_DN; k++) issue<false>();
+
+            const int ch = (lane >> 2) % LPR_DN, ris = 4 * (lane / (4 * LPR_DN)) + j;
+            LaneD ln;
+            ln.template init<LPR_DN>(ris, ch);
+            DataD td0, td1;                   // the slice in hand and the one fetched behind it
+            uint32_t tag_d = 0u;
+            bool have_d = false;
+            for (; cq < n_seq; cq++) {
+                const int l = seg_layer(cq);
+                fm_wg_barrier();                       // images and partial vectors are free
+                if (cq > n_up) reduce_part(cq - 1);
+                build_down_images(l);
+                fm_wg_barrier();
+                const uint32_t ta = fm_lds_addr(&tab[cq]);
+                const uint32_t valid = __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(GgSeg, valid)));
+                const uint32_t c_nrb = fm_div(by_K, __builtin_amdgcn_readfirstlane(fm_lds_r32(ta + (uint32_t)offsetof(GgSeg, n))));
+                GgAct<GD::NREG> ar;
+                uint32_t k_cur = 0xFFFFFFFFu;
+                dry = false;
+                while (issued - consumed < (uint32_t)RING_DN && !dry) issue<false>();
+                if (!have_d && consumed < issued) {
+                    tag_d = fetch_dn(ln, td0);
+                    have_d = true;
+                }
+                // one slice of this segment out of t (tag tg): image of its expert, product, partial vector
+                auto one = [&](const DataD &t, uint32_t tg) __attribute__((always_inline)) {
+                    const uint32_t pc = (tg >> 28) & 7u, ul = tg & 0x0FFFFFFFu;
+                    if (pc != k_cur) {
+                        gg_read_image<GD::NREG>(img0 + pc * (uint32_t)IMG_DN, 4 * LPR_DN, lane, ar);
+                        k_cur = pc;
+                    }
+                    float v = fm_chunk_sum<LPR_DN>(ln.dot(t, ar, ones));
+                    if (!((valid >> pc) & 1u)) v = 0.0f;
+                    const uint32_t rbi = ul - pc * c_nrb;
+                    if (ch == 0)
+                        fm_lds_w32(part0 + 4u * ((rbi * (uint32_t)K + pc) * RPS_DN + (uint32_t)ris), __float_as_uint(v));
+                };
+                while (have_d) {
+                    if ((tag_d >> 31) != (uint32_t)(cq & 1)) break;      // the next segment's: it waits in td0
+                    const bool more = consumed < issued;
+                    uint32_t tag_n = 0u;
+                    if (more) tag_n = fetch_dn(ln, td1);
+                    one(td0, tag_d);
+                    if (!more) {
+                        have_d = false;
+                        break;
+                    }
+                    if ((tag_n >> 31) != (uint32_t)(cq & 1)) {           // (once per segment at most)
+                        td0 = td1;
+                        tag_d = tag_n;
+                        break;
+                    }
+                    have_d = consumed < issued;
+                    if (have_d) tag_d = fetch_dn(ln, td0);
+                    one(td1, tag_n);
+                }
+            }
+            fm_wg_barrier();
+            reduce_part(n_seq - 1);
+        }
+    }
+};
+
+template <int DN_KIND, int LPR_UP, int LPR_DN>
+__global__ __launch_bounds__(512) void fm_gguf_fused_rows(GgufArgs a, Fm2Dims dm, Fm2Sync sy) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    GgFused<DN_KIND, LPR_UP, LPR_DN> st(a, sy);
+    st.run(dm);
+#else
+    (void)a;
+    (void)dm;
+    (void)sy;
+#endif
+}
+
+// One launch for the whole operator; FM_ERR_UNSUPPORTED when the shape has no instance or the
+// grid could not be resident at once (every workgroup may wait for another's activations).
+template <int DN_KIND, int LPR_UP, int LPR_DN>
+int gg_launch_fused_t(const GgufArgs &a, int n_pairs, const FmGg2Plan &plan, hipStream_t st, const Fm2Sync &sy) {
+    using F = GgFused<DN_KIND, LPR_UP, LPR_DN>;
+    auto kfn = fm_gguf_fused_rows<DN_KIND, LPR_UP, LPR_DN>;
+    if ((uint32_t)F::LDS_BYTES != plan.lds_bytes || (uint32_t)F::RING_BYTES != plan.ring_bytes ||
+        (uint32_t)F::IMG_BYTES != plan.img_bytes || F::RING_DN != plan.ring_dn)
+        return FM_ERR_UNSUPPORTED;                     // (the plan and the kernel disagree: never expected)
+    static FmLdsAttr attr;
+    static int per_cu[64] = {};
+    if (!fm_dyn_lds_ready(attr, (const void *)kfn, (size_t)F::LDS_BYTES)) return FM_ERR_HIP;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    const bool known = dev >= 0 && dev < 64;
+    int pc = known ? per_cu[dev] : 0;
+    if (pc == 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&pc, kfn, 512, (size_t)F::LDS_BYTES) != hipSuccess) pc = 0;
+        if (pc < 1) pc = -1;
+        if (known) per_cu[dev] = pc;
+    }
+    if (pc < 1) return FM_ERR_UNSUPPORTED;
+    const Fm2Dims dm = fm2_dims_units(n_pairs, a.K, plan.wgs, plan.gu_upp, plan.dn_upp, plan.gu_wt, plan.dn_wt);
+    hipLaunchKernelGGL(kfn, dim3((unsigned)plan.wgs), dim3(512), (size_t)F::LDS_BYTES, st, a, dm, sy);
+    return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+}
+
+int gg_launch_fused(const GgufArgs &a, int n_pairs, int n_cu, hipStream_t st, const Fm2Sync &sy) {
+    if (a.g.gate_type != FM_GGML_Q4_K || a.g.up_type != FM_GGML_Q4_K) return FM_ERR_UNSUPPORTED;
+    const bool q6 = a.g.down_type == FM_GGML_Q6_K;
+    if (!q6 && a.g.down_type != FM_GGML_Q4_K) return FM_ERR_UNSUPPORTED;
+    const FmGg2Plan plan = fm_gg2_plan(n_pairs, a.K, a.g.hidden, a.g.inter, q6 ? 1 : 0, n_cu);
+    if (!plan.ok || plan.wgs > n_cu) return FM_ERR_UNSUPPORTED;
+    if (q6 && plan.lpr_up == 16 && plan.lpr_dn == 8) return gg_launch_fused_t<GG_Q6, 16, 8>(a, n_pairs, plan, st, sy);
+    if (q6 && plan.lpr_up == 8 && plan.lpr_dn == 4) return gg_launch_fused_t<GG_Q6, 8, 4>(a, n_pairs, plan, st, sy);
+    if (!q6 && plan.lpr_up == 8 && plan.lpr_dn == 4) return gg_launch_fused_t<GG_Q4, 8, 4>(a, n_pairs, plan, st, sy);
+    return FM_ERR_UNSUPPORTED;
+}
+
 // launch of one streaming phase; FM_ERR_UNSUPPORTED when the shape has no instance
 template <int KIND, bool GU>
 int gg_launch_stream(const GgufArgs &a, int n_pairs, int n_cu, hipStream_t st) {
@@ -946,7 +1418,7 @@ extern "C" int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t
                                      const uint8_t *const *d_down, const FmGgufGeom *g, int layer0,
                                      int layer_stride, int n_layers, const float *d_x,
                                      const int32_t *d_idx, const float *d_w, int K, float *d_act,
-                                     float *d_expert_out, float *d_out, unsigned int *, int flags,
+                                     float *d_expert_out, float *d_out, FmDecodeFlags *df, int flags,
                                      int n_cu, hipStream_t st, hipEvent_t *kev) {
     GgufArgs a;
     a.direct = nullptr;
@@ -963,8 +1435,36 @@ extern "C" int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t
     a.act = d_act;
     a.expert_out = d_expert_out;
     a.out = d_out;
-    a.flags = flags;
+    a.flags = flags & ~FM_INT_NO_EXPERT_OUT;
     const int n_pairs = n_layers * K;
+    // Without per-expert vectors, without the finite guard and outside a graph capture: one launch
+    // (the activation sets alternate between launches exactly as for the affine experts; a
+    // captured launch would need the graph's set and a fill kernel in front, and takes the three
+    // kernels instead).
+    const bool phases = (fm_kernel_forms & (FM_FORM_PLAIN_GGUF | FM_FORM_GGUF_PHASES)) != 0;
+    const unsigned int act_need = (unsigned int)n_pairs * (unsigned int)g->inter;
+    if (!phases && !kev && df && (flags & FM_INT_NO_EXPERT_OUT) && !(flags & FM_GUARD) && df->act_set[0] &&
+        df->act_cap >= act_need && !df->always_graph_set) {
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        (void)hipStreamIsCapturing(st, &capture);
+        if (capture == hipStreamCaptureStatusNone) {
+            Fm2Sync sy{};
+            sy.act_other = df->act_set[df->act_parity ^ 1];
+            sy.clear_n = df->act_used[df->act_parity ^ 1];
+            sy.err = df->err;
+            sy.spin_limit = df->spin_limit;
+            GgufArgs af = a;
+            af.act = df->act_set[df->act_parity];
+            const int rc = gg_launch_fused(af, n_pairs, n_cu, st, sy);
+            if (rc == FM_OK) {     // the set just filled is in use, the other one is all markers again
+                df->act_used[df->act_parity] = act_need;
+                df->act_used[df->act_parity ^ 1] = 0u;
+                df->act_parity ^= 1;
+                return FM_OK;
+            }
+            if (rc != FM_ERR_UNSUPPORTED) return rc;
+        }
+    }
     const int lpr_up = g->hidden / 128, lpr_down = g->inter / 128;
     auto pow2 = [](int v) { return v > 0 && (v & (v - 1)) == 0; };
     if (!pow2(lpr_up) || !pow2(lpr_down) || lpr_up < 2 || lpr_up > 64 || lpr_down < 2 || lpr_down > 64)

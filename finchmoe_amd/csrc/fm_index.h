@@ -393,25 +393,34 @@ struct Fm2Dims {
     uint32_t gu_segu, dn_segu;  // units per segment: a layer's K experts
     uint32_t gu_total, rb_total, s_total;
     uint32_t wq;                // G / L: a layer has wq or wq + 1 workgroups (G >= L)
-    FmDiv by_G, by_L, by_K, by_gu_upp, by_gu_segu, by_dn_segu, by_wq, by_wq1;
+    uint32_t gu_wt, dn_wt;      // what a gate/up unit and a (row block, slot) weigh in the balance
+    FmDiv by_G, by_L, by_K, by_gu_upp, by_gu_segu, by_dn_segu, by_wq, by_wq1, by_gu_wt;
 };
-FM_HD Fm2Dims fm2_dims(int n_pairs, int K, int G, int inter, int hidden, int lpr_up) {
+// gu_upp gate/up units per pair, dn_upp down row blocks per layer; a gate/up unit streams gu_wt
+// and a down unit dn_wt of some common measure of bytes (affine experts: two slices and one)
+FM_HD Fm2Dims fm2_dims_units(int n_pairs, int K, int G, uint32_t gu_upp, uint32_t dn_upp, uint32_t gu_wt,
+                             uint32_t dn_wt) {
     Fm2Dims d;
-    const int rps_up = FM_WAVE / lpr_up, rps_dn = FM_WAVE / (lpr_up / 4);
     d.K = (uint32_t)K, d.G = (uint32_t)G, d.L = (uint32_t)(n_pairs / K);
-    d.gu_upp = (uint32_t)(inter / rps_up);
-    d.dn_upp = (uint32_t)(hidden / rps_dn);
+    d.gu_upp = gu_upp;
+    d.dn_upp = dn_upp;
+    d.gu_wt = gu_wt, d.dn_wt = dn_wt;
     d.gu_segu = d.gu_upp * d.K;
     d.dn_segu = d.dn_upp * d.K;
     d.gu_total = (uint32_t)n_pairs * d.gu_upp;
     d.rb_total = d.L * d.dn_upp;
-    d.s_total = 2u * d.gu_total + d.rb_total * d.K;
+    d.s_total = gu_wt * d.gu_total + dn_wt * d.rb_total * d.K;
     d.wq = d.L ? d.G / d.L : 0u;
     d.by_G = fm_div_make(d.G), d.by_L = fm_div_make(d.L ? d.L : 1u), d.by_K = fm_div_make(d.K);
     d.by_gu_upp = fm_div_make(d.gu_upp ? d.gu_upp : 1u);
     d.by_gu_segu = fm_div_make(d.gu_segu ? d.gu_segu : 1u), d.by_dn_segu = fm_div_make(d.dn_segu ? d.dn_segu : 1u);
     d.by_wq = fm_div_make(d.wq ? d.wq : 1u), d.by_wq1 = fm_div_make(d.wq + 1u);
+    d.by_gu_wt = fm_div_make(gu_wt ? gu_wt : 1u);
     return d;
+}
+FM_HD Fm2Dims fm2_dims(int n_pairs, int K, int G, int inter, int hidden, int lpr_up) {
+    const int rps_up = FM_WAVE / lpr_up, rps_dn = FM_WAVE / (lpr_up / 4);
+    return fm2_dims_units(n_pairs, K, G, (uint32_t)(inter / rps_up), (uint32_t)(hidden / rps_dn), 2u, 1u);
 }
 // first down row block of workgroup gg: a workgroup's row blocks lie in ONE layer whenever there
 // are at least as many workgroups as layers
@@ -427,8 +436,8 @@ FM_HD uint32_t fm2_dn_start(const Fm2Dims &d, uint32_t gg) {
 // first gate/up unit of workgroup gg (dn0 = its first down row block): sized so that gate/up +
 // down slices are the same for every workgroup
 FM_HD uint32_t fm2_gu_start(const Fm2Dims &d, uint32_t gg, uint32_t dn0) {
-    const uint32_t t = fm_div(d.by_G, d.s_total * gg), dd = dn0 * d.K;
-    const uint32_t u = t > dd ? (t - dd) / 2u : 0u;
+    const uint32_t t = fm_div(d.by_G, d.s_total * gg), dd = dn0 * d.K * d.dn_wt;
+    const uint32_t u = t > dd ? fm_div(d.by_gu_wt, t - dd) : 0u;
     return u > d.gu_total ? d.gu_total : u;
 }
 struct Fm2Split {
@@ -504,12 +513,14 @@ FM_HD Fm2TailLds fm2_tail_lds(int nrb, int K, int rps_dn, int shared_inter, int 
 struct Fm2Plan {
     int ok, wgs;
 };
-FM_HD Fm2Plan fm2_plan(int n_pairs, int K, int inter, int hidden, int lpr_up, int n_cu) {
+FM_HD Fm2Plan fm2_plan_units(int n_pairs, int K, long gu_upp, long dn_rbs, int rps_dn, long gu_wt, long dn_wt,
+                             int n_cu) {
     Fm2Plan p;
     p.ok = 0;
-    const int rps_up = FM_WAVE / lpr_up, rps_dn = FM_WAVE / (lpr_up / 4);
+    p.wgs = 0;
+    if (K < 1 || gu_upp < 1 || dn_rbs < 1 || gu_wt < 1 || dn_wt < 1) return p;
     const int n_groups = n_pairs / K;
-    const long gu_segu = (long)(inter / rps_up) * K, dn_rbs = hidden / rps_dn;
+    const long gu_segu = gu_upp * K;
     const long up_units = (long)n_groups * gu_segu, rb_total = (long)n_groups * dn_rbs;
     long wgs = n_cu;
     const long small = up_units < rb_total * K ? up_units : rb_total * K;
@@ -518,8 +529,8 @@ FM_HD Fm2Plan fm2_plan(int n_pairs, int K, int inter, int hidden, int lpr_up, in
     p.wgs = (int)wgs;
     // at most two gate/up segments, and the down segments and the row blocks of one part within
     // the fixed tables
-    const long s_total = 2 * up_units + rb_total * K;
-    const long up_share = (s_total / wgs + 1) / 2 + 1;                  // upper bound, in units
+    const long s_total = gu_wt * up_units + dn_wt * rb_total * K;
+    const long up_share = (s_total / wgs + 1) / gu_wt + 1;              // upper bound, in units
     if (up_share > gu_segu || s_total * wgs >= (1L << 31)) return p;
     long n_dn, part_rbs;
     if (wgs >= n_groups) {
@@ -534,6 +545,10 @@ FM_HD Fm2Plan fm2_plan(int n_pairs, int K, int inter, int hidden, int lpr_up, in
     if (part_rbs * K * rps_dn * 4 > FM2_PART_BYTES) return p;
     p.ok = 1;
     return p;
+}
+FM_HD Fm2Plan fm2_plan(int n_pairs, int K, int inter, int hidden, int lpr_up, int n_cu) {
+    const int rps_up = FM_WAVE / lpr_up, rps_dn = FM_WAVE / (lpr_up / 4);
+    return fm2_plan_units(n_pairs, K, inter / rps_up, hidden / rps_dn, rps_dn, 2, 1, n_cu);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -571,6 +586,71 @@ FM_HD FmGgPlan fm_gg_plan(int n_pairs, int K, int in_dim, int rows, int q6, int 
     if ((p.total + wgs - 1) / wgs > max_share) wgs = (p.total + max_share - 1) / max_share;
     while (wgs < p.total && (p.total + wgs - 1) / wgs > max_share) wgs++;
     p.wgs = (int)wgs;
+    p.ok = 1;
+    return p;
+}
+
+// The GGUF experts as one launch (fm_gguf_fused_rows): the split of fm_moe_fused_rows with a
+// gate/up unit = the gate and the up slice of a wave step (Q4_K) and a down unit = the slice of
+// one row block of one expert (Q6_K or Q4_K), weighed by their bytes.  LDS: eight rings (three
+// gate/up slots or ring_dn down slots each, whichever is larger) | two gate/up images or K down
+// images | segment tables | partial vectors.
+#define FM_GG2_RING_UP 3
+#define FM_GG2_SEG_BYTES 192
+struct FmGg2Plan {
+    int ok, wgs;
+    int lpr_up, lpr_dn, rps_up, rps_dn, ring_dn;
+    uint32_t gu_upp, dn_upp, gu_wt, dn_wt;
+    uint32_t slot_up, slot_dn;        // bytes of a slice (without the 16-byte trailer)
+    uint32_t ring_bytes, img_up, img_dn, img_bytes, lds_bytes;
+};
+FM_HD uint32_t fm_gcd(uint32_t a, uint32_t b) {
+    while (b) {
+        const uint32_t t = a % b;
+        a = b;
+        b = t;
+    }
+    return a;
+}
+FM_HD FmGg2Plan fm_gg2_plan(int n_pairs, int K, int hidden, int inter, int down_q6, int n_cu) {
+    FmGg2Plan p;
+    p.ok = 0, p.wgs = 0;
+    p.lpr_up = hidden / 128;
+    p.lpr_dn = inter / (down_q6 ? 64 : 128);
+    p.rps_up = p.rps_dn = 0;
+    p.ring_dn = down_q6 ? 4 : 3;
+    p.gu_upp = p.dn_upp = p.gu_wt = p.dn_wt = 0u;
+    p.slot_up = p.slot_dn = p.ring_bytes = p.img_up = p.img_dn = p.img_bytes = p.lds_bytes = 0u;
+    if (K < 1 || K > FM_MAX_K || n_pairs < K || n_pairs % K) return p;
+    if (hidden % 256 || inter % 256) return p;
+    if (!(p.lpr_up == 4 || p.lpr_up == 8 || p.lpr_up == 16)) return p;
+    if (!(p.lpr_dn == 4 || p.lpr_dn == 8 || p.lpr_dn == 16)) return p;
+    p.rps_up = FM_WAVE / p.lpr_up, p.rps_dn = FM_WAVE / p.lpr_dn;
+    if (inter % p.rps_up || hidden % p.rps_dn) return p;
+    p.gu_upp = (uint32_t)(inter / p.rps_up);
+    p.dn_upp = (uint32_t)(hidden / p.rps_dn);
+    p.slot_up = (uint32_t)(p.rps_up * (p.lpr_up / 2) * 144);
+    p.slot_dn = (uint32_t)(down_q6 ? p.rps_dn * (p.lpr_dn / 4) * 210 : p.rps_dn * (p.lpr_dn / 2) * 144);
+    const uint32_t r_up = FM_GG2_RING_UP * (p.slot_up + 16u), r_dn = (uint32_t)p.ring_dn * (p.slot_dn + 16u);
+    p.ring_bytes = r_up > r_dn ? r_up : r_dn;
+    const uint32_t nreg_dn = down_q6 ? 32u : 64u;
+    p.img_up = 16u * (4u * p.lpr_up) * 16u + (uint32_t)p.lpr_up * 16u;
+    p.img_dn = (nreg_dn / 4u) * (4u * p.lpr_dn) * 16u + (uint32_t)p.lpr_dn * 16u;
+    p.img_bytes = 2u * p.img_up > FM_MAX_K * p.img_dn ? 2u * p.img_up : FM_MAX_K * p.img_dn;
+    p.lds_bytes = 8u * p.ring_bytes + p.img_bytes + FM2_MAX_SEG * FM_GG2_SEG_BYTES + FM2_PART_BYTES;
+    if (p.lds_bytes > 160u * 1024u) return p;
+    // weights of the balance: bytes over their greatest common divisor, halved while the
+    // kernel's 32-bit products would not hold them (the balance then is approximate)
+    const uint32_t gdiv = fm_gcd(2u * p.slot_up, p.slot_dn);
+    p.gu_wt = 2u * p.slot_up / gdiv, p.dn_wt = p.slot_dn / gdiv;
+    for (;;) {
+        const Fm2Plan q = fm2_plan_units(n_pairs, K, p.gu_upp, p.dn_upp, p.rps_dn, p.gu_wt, p.dn_wt, n_cu);
+        p.wgs = q.wgs;
+        if (q.ok) break;
+        const long s_total = (long)p.gu_wt * n_pairs * p.gu_upp + (long)p.dn_wt * n_pairs * p.dn_upp;
+        if (s_total * (q.wgs > 0 ? q.wgs : 1) < (1L << 31) || (p.gu_wt <= 2u && p.dn_wt <= 1u)) return p;
+        p.gu_wt = (p.gu_wt + 1u) / 2u, p.dn_wt = (p.dn_wt + 1u) / 2u;
+    }
     p.ok = 1;
     return p;
 }

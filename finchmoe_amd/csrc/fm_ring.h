@@ -161,6 +161,34 @@ __device__ __forceinline__ uint32_t fm_slot_peek(uint32_t slot_tag_addr) {
 }
 
 
+// The intermediate vectors (act, expert_out) are written by one phase and read
+// by the next, possibly inside one launch and from a CU behind another L2.
+// They are stored and loaded as device-scope relaxed atomics: such accesses are
+// performed at the level all CUs share, so a consumer that starts after the
+// producer's stores have completed sees them without any cache maintenance.
+__device__ __forceinline__ void fm_st_shared(float *p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float fm_ld_shared(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// LDS words with explicit instructions (the compiler would order a visible LDS access behind
+// every LDS-direct load in flight)
+__device__ __forceinline__ void fm_lds_w32(uint32_t addr, uint32_t v) {
+    asm volatile("ds_write_b32 %0, %1" ::"v"(addr), "v"(v) : "memory");
+}
+__device__ __forceinline__ uint32_t fm_lds_r32(uint32_t addr) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
+    return v;
+}
+// workgroup barrier that waits for this wave's LDS operations only (the compiler's own puts a
+// wait for every LDS-direct load in front)
+__device__ __forceinline__ void fm_wg_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // Host side: raise a kernel's dynamic LDS limit above the 64 KB default, once per
 // kernel and device (the attribute belongs to a device's copy of the kernel, and the
 // runtime call costs more host time than a launch).

@@ -403,8 +403,9 @@ static void walk_fused_rows(int n_groups, int K, int hidden, int inter, int bits
             dn_ref = l * dm.dn_upp + dm.dn_upp * (ug - g_lo) / (g_hi - g_lo);
         }
         CHECK(fm2_dn_start(dm, ug) == dn_ref, "first down row block of workgroup %d", gi);
-        const uint32_t t = dm.s_total * ug / dm.G, dd = dn_ref * dm.K;
-        uint32_t gu_ref = t > dd ? (t - dd) / 2u : 0u;
+        const uint32_t t = dm.s_total * ug / dm.G, dd = dn_ref * dm.K * dm.dn_wt;
+        CHECK(dm.gu_wt == 2u && dm.dn_wt == 1u, "affine experts: two slices per gate/up unit, one per down unit");
+        uint32_t gu_ref = t > dd ? (t - dd) / dm.gu_wt : 0u;
         if (gu_ref > dm.gu_total) gu_ref = dm.gu_total;
         CHECK(fm2_gu_start(dm, ug, dn_ref) == gu_ref, "first gate/up unit of workgroup %d", gi);
     }
@@ -642,6 +643,157 @@ static void walk_gguf_stream(int n_groups, int K, int hidden, int inter, bool gu
     std::printf("ok  %-58s %ld units over %d workgroups\n", g_case.c_str(), pl.total, pl.wgs);
 }
 
+
+// fm_gguf_fused_rows: the GGUF experts as one launch.  Every pair gets slabs of its own here, so
+// "read exactly once" is checked per pair and matrix.
+static void walk_gguf_fused(int n_groups, int K, int hidden, int inter, int down_q6) {
+    g_case = std::string("gguf fused rows ") + (down_q6 ? "Q6_K" : "Q4_K") + " down, " + std::to_string(n_groups) + " groups x " +
+             std::to_string(K) + ", " + std::to_string(hidden) + "x" + std::to_string(inter);
+    const int n_pairs = n_groups * K;
+    const FmGg2Plan pl = fm_gg2_plan(n_pairs, K, hidden, inter, down_q6, N_CU);
+    if (!pl.ok) {
+        std::printf("--  %-58s not taken by this launch form\n", g_case.c_str());
+        return;
+    }
+    const int G = pl.wgs;
+    CHECK(G >= 1 && G <= N_CU, "%d workgroups", G);
+    const Fm2Dims dm = fm2_dims_units(n_pairs, K, G, pl.gu_upp, pl.dn_upp, pl.gu_wt, pl.dn_wt);
+    CHECK((uint64_t)dm.s_total * (uint64_t)G < (1ull << 31), "32-bit products");
+    const size_t gu_row = (size_t)(hidden / 256) * 144, dn_row = (size_t)(inter / 256) * (down_q6 ? 210 : 144);
+    const size_t gu_slab = (size_t)inter * gu_row, dn_slab = (size_t)hidden * dn_row;
+    CHECK((size_t)pl.gu_upp * pl.slot_up == gu_slab && (size_t)pl.dn_upp * pl.slot_dn == dn_slab, "slices tile the expert");
+    // LDS: rings | images | segment tables | partial vectors
+    CHECK(FM_GG2_RING_UP * (pl.slot_up + 16) <= pl.ring_bytes && (uint32_t)pl.ring_dn * (pl.slot_dn + 16) <= pl.ring_bytes,
+          "ring slots inside a wave's ring");
+    CHECK(2 * pl.img_up <= pl.img_bytes && FM_MAX_K * pl.img_dn <= pl.img_bytes, "images");
+    CHECK(pl.lds_bytes == 8 * pl.ring_bytes + pl.img_bytes + FM2_MAX_SEG * FM_GG2_SEG_BYTES + FM2_PART_BYTES &&
+              pl.lds_bytes <= 160 * 1024, "LDS %u", pl.lds_bytes);
+    {   // the image writes of the down phase: thread t, item t + 512 i
+        const int nreg = down_q6 ? 32 : 64, per = pl.lpr_dn * nreg, ne = 4 * pl.lpr_dn, grp = down_q6 ? 8 : 16;
+        CHECK(FM_MAX_K * per % 512 == 0 && per % 64 == 0, "whole waves per image");
+        std::vector<uint8_t> cols((size_t)inter, 0);
+        for (int it = 0; it < per; it++) {
+            const int ch = it / nreg, r = it % nreg, lo = 32 * (r >> 4) + 4 * ((r & 15) >> 1) + (r & 1);
+            for (int d = 0; d < 3; d += 2) {
+                const int v = lo + d;
+                const int col = down_q6 ? 128 * (ch >> 1) + 32 * (ch & 1) + (v < 32 ? v : v + 32) : 128 * ch + v;
+                CHECK(col >= 0 && col < inter, "image column %d", col);
+                if (col >= 0 && col < inter) cols[col]++;
+            }
+            const size_t dst = (size_t)((((r >> 2) * ne + 4 * ch) * 4 + (r & 3)) * 4);
+            CHECK(dst + 48 + 4 <= (size_t)(nreg / 4) * ne * 16, "image register of chunk %d", ch);
+            const size_t sum = (size_t)(nreg / 4) * ne * 16 + ch * 16 + (r / grp) * 4;
+            CHECK(sum + 4 <= pl.img_dn, "image sums");
+        }
+        for (int c = 0; c < inter; c++) CHECK(cols[c] == 1, "activation column %d polled %d times", c, (int)cols[c]);
+    }
+    std::vector<Region> gate, up, down;
+    for (int p = 0; p < n_pairs; p++) {
+        gate.emplace_back("gate rows", gu_slab, 16);
+        up.emplace_back("up rows", gu_slab, 16);
+        down.emplace_back("down rows", dn_slab, 16);
+    }
+    Region act("act", (size_t)n_pairs * inter * 4, 4), out("out", (size_t)n_groups * hidden * 4, 4);
+    Region X("x", (size_t)n_groups * hidden * 4), idx("idx", (size_t)n_pairs * 4);
+    auto slice = [&](Region &r, size_t off, uint32_t data) {
+        for (int lane = 0; lane < 64; lane++)
+            for (uint32_t i = 0; i * 1024 < data; i++)
+                if (i * 1024 + lane * 16 < data) {
+                    CHECK(i * 1024 + lane * 16 + 16 <= data, "load %u lane %d runs over the slice", i, lane);
+                    r.touch(off + (size_t)i * 1024 + (size_t)lane * 16, 16, "slice");
+                }
+    };
+    for (int gi = 0; gi <= G; gi++) {     // the prepared divisions against plain ones
+        const uint32_t ug = (uint32_t)gi;
+        uint32_t dn_ref;
+        if (ug >= dm.G) dn_ref = dm.rb_total;
+        else if (dm.G < dm.L) dn_ref = dm.rb_total * ug / dm.G;
+        else {
+            const uint32_t l = ug * dm.L / dm.G;
+            const uint32_t g_lo = (l * dm.G + dm.L - 1u) / dm.L, g_hi = ((l + 1u) * dm.G + dm.L - 1u) / dm.L;
+            dn_ref = l * dm.dn_upp + dm.dn_upp * (ug - g_lo) / (g_hi - g_lo);
+        }
+        CHECK(fm2_dn_start(dm, ug) == dn_ref, "first down row block of workgroup %d", gi);
+        const uint32_t t = (uint32_t)((uint64_t)dm.s_total * ug / dm.G), dd = dn_ref * dm.K * dm.dn_wt;
+        uint32_t gu_ref = t > dd ? (t - dd) / dm.gu_wt : 0u;
+        if (gu_ref > dm.gu_total) gu_ref = dm.gu_total;
+        CHECK(fm2_gu_start(dm, ug, dn_ref) == gu_ref, "first gate/up unit of workgroup %d", gi);
+    }
+    int max_seq = 0;
+    size_t max_bytes = 0, min_bytes = (size_t)-1;
+    uint32_t gu_prev = 0;
+    for (int gi = 0; gi < G; gi++) {
+        const Fm2Split sp = fm2_split(dm, gi);
+        CHECK(sp.gu_wg0 == gu_prev && sp.gu_wg1 >= sp.gu_wg0, "gate/up shares of workgroup %d follow on", gi);
+        gu_prev = sp.gu_wg1;
+        const int n_seq = sp.n_up + sp.n_dn;
+        if (n_seq > max_seq) max_seq = n_seq;
+        CHECK(sp.n_up <= 2, "workgroup %d: %d gate/up segments", gi, sp.n_up);
+        CHECK(n_seq <= FM2_MAX_SEG && n_seq <= 64, "workgroup %d: %d segments", gi, n_seq);
+        for (int v = 0; v < sp.n_up && v < 2; v++)
+            X.touch((size_t)(sp.gu_s0 + v) * hidden * 4, (size_t)hidden * 4, "x of a gate/up segment");
+        size_t bytes = 0;
+        for (int qq = 0; qq < n_seq; qq++) {
+            const Fm2Part pt = fm2_part(dm, sp, qq);
+            CHECK(pt.seg < (uint32_t)n_groups, "segment %u", pt.seg);
+            for (int k = 0; k < K; k++) idx.touch(((size_t)pt.seg * K + k) * 4, 4, "idx");
+            if (pt.gu) {
+                for (uint32_t ul = 0; ul < pt.n; ul++) {
+                    uint32_t pn, rsn;
+                    fm2_gu_unit(pt.first, ul, dm.by_gu_upp, &pn, &rsn);
+                    CHECK(pn < (uint32_t)K && rsn < dm.gu_upp, "gate/up unit %u -> slot %u step %u", ul, pn, rsn);
+                    CHECK(ul < (1u << 28), "unit number in the tag");
+                    if (pn >= (uint32_t)K) continue;
+                    slice(gate[pt.seg * K + pn], (size_t)rsn * pl.slot_up, pl.slot_up);
+                    slice(up[pt.seg * K + pn], (size_t)rsn * pl.slot_up, pl.slot_up);
+                    bytes += 2 * (size_t)pl.slot_up;
+                    for (int lane = 0; lane < 64; lane++) {
+                        const int j = lane & 3, ch = (lane >> 2) % pl.lpr_up, ris = 4 * (lane / (4 * pl.lpr_up)) + j;
+                        CHECK(ris < pl.rps_up, "row in step %d", ris);
+                        if (ch == 0)
+                            act.touch((((size_t)pt.seg * dm.gu_segu + pt.first) * pl.rps_up + ris + (size_t)ul * pl.rps_up) * 4, 4, "act");
+                    }
+                }
+            } else {
+                CHECK(pt.first % K == 0 && pt.n % K == 0, "down part %u + %u not whole row blocks", pt.first, pt.n);
+                const uint32_t rb_first = pt.first / K, nrb = pt.n / K;
+                const float inv = 1.0f / (float)(nrb ? nrb : 1u);
+                CHECK((size_t)nrb * K * pl.rps_dn * 4 <= FM2_PART_BYTES, "partial vectors of %u row blocks", nrb);
+                for (uint32_t ul = 0; ul < pt.n; ul++) {
+                    uint32_t pn, rsn;
+                    fm2_dn_unit(rb_first, nrb, inv, ul, &pn, &rsn);
+                    CHECK(pn == ul / nrb && rsn == rb_first + ul % nrb, "down unit %u -> slot %u block %u", ul, pn, rsn);
+                    CHECK(pn < (uint32_t)K && rsn < dm.dn_upp, "down unit %u -> slot %u block %u", ul, pn, rsn);
+                    if (pn >= (uint32_t)K) continue;
+                    slice(down[pt.seg * K + pn], (size_t)rsn * pl.slot_dn, pl.slot_dn);
+                    bytes += pl.slot_dn;
+                    const uint32_t rbi = ul - pn * nrb;
+                    for (int lane = 0; lane < 64; lane++) {
+                        const int j = lane & 3, ris = 4 * (lane / (4 * pl.lpr_dn)) + j;
+                        CHECK(ris < pl.rps_dn, "row in step %d", ris);
+                        CHECK(4u * ((rbi * K + pn) * pl.rps_dn + ris) + 4 <= FM2_PART_BYTES, "partial slot");
+                    }
+                }
+                Region a1("act", act.size);
+                a1.touch((size_t)pt.seg * K * inter * 4, (size_t)K * inter * 4, "act of the layer");
+                out.touch(((size_t)pt.seg * hidden + (size_t)rb_first * pl.rps_dn) * 4, (size_t)nrb * pl.rps_dn * 4, "out rows");
+            }
+        }
+        if (bytes > max_bytes) max_bytes = bytes;
+        if (bytes < min_bytes) min_bytes = bytes;
+    }
+    CHECK(gu_prev == dm.gu_total, "gate/up units handed out: %u of %u", gu_prev, dm.gu_total);
+    for (int p = 0; p < n_pairs; p++) {
+        gate[p].expect_once(0, gu_slab);
+        up[p].expect_once(0, gu_slab);
+        down[p].expect_once(0, dn_slab);
+    }
+    act.expect_once(0, act.size);
+    out.expect_once(0, out.size);
+    std::printf("ok  %-58s %d workgroups, <= %d segments, weights %u:%u, bytes per workgroup %zu..%zu\n", g_case.c_str(), G,
+                max_seq, pl.gu_wt, pl.dn_wt, min_bytes, max_bytes);
+}
+
 int main() {
     // ---- the probes of bench.py --workload stream_probe (2 GiB) and of the decode profile (440 MB)
     for (int pattern = 0; pattern < 8; pattern++) {
@@ -717,6 +869,16 @@ int main() {
         walk_gguf_stream(groups, 8, 2048, 512, true);
         walk_gguf_stream(groups, 8, 2048, 512, false);
     }
+    // ---- the GGUF experts as one launch: the step, one layer, the tests' shapes
+    for (int groups : {40, 1, 2, 3, 8, 31, 64})
+        walk_gguf_fused(groups, 8, 2048, 512, 1);
+    walk_gguf_fused(3, 5, 2048, 512, 1);
+    walk_gguf_fused(2, 8, 1024, 256, 1);
+    walk_gguf_fused(40, 8, 1024, 256, 1);
+    walk_gguf_fused(3, 8, 1024, 512, 0);
+    walk_gguf_fused(1, 2, 2048, 2048, 0);
+    walk_gguf_fused(1, 4, 512, 1024, 1);
+    walk_gguf_fused(300, 8, 2048, 512, 1);
     // ---- one dense GGUF tensor as the streaming kernel's single "expert" (rows = hidden, columns =
     // inter in the down phase's names): the vocabulary projection at Q4_K, and smaller shapes
     walk_gguf_stream(1, 1, 248320, 2048, false, 0, "Q4_K 248320x2048");

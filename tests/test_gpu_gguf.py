@@ -167,6 +167,56 @@ def test_gguf_streaming_shapes(orc, h, i, down_t, layers, K):
         ctx.close()
 
 
+@pytest.mark.parametrize("h,i,down_t,layers,K", [(2048, 512, 14, 3, 8), (2048, 512, 14, 1, 5), (1024, 256, 14, 2, 8),
+                                                 (1024, 512, 12, 3, 8)])
+def test_gguf_one_launch_equals_three(orc, h, i, down_t, layers, K):
+    """A caller that does not ask for the per-expert vectors gets the operator as one launch
+    (gate/up, down by row blocks, slot-order sum in LDS).  Bit for bit the three launches (the same
+    lane arithmetic and the same order of the sum), three calls in a row (the activation sets
+    alternate and are re-marked), accumulation into out, an expert index outside the store; and
+    within the bar of the oracle."""
+    import torch
+    from finchmoe_amd import FinchHip
+    rng = np.random.default_rng(3 * h + i + down_t + K)
+    e = 12
+    store = [F.synth_gguf_layer(rng, e, h, i, (12, 12, down_t)) for _ in range(layers)]
+    ctx = FinchHip(0)
+    try:
+        ctx.gguf_config(layers, e, h, i, (fb.Q4_K, fb.Q4_K, down_t))
+        for l, (g, u, d) in enumerate(store):
+            ctx.gguf_upload_layer(l, g, u, d)
+        for rep in range(3):
+            x = rng.standard_normal((layers, h)).astype(np.float32)
+            idx = np.stack([rng.permutation(e)[:K] for _ in range(layers)]).astype(np.int32)
+            w = np.stack([orc.normalize_weights(rng.random(K).astype(np.float32)) for _ in range(layers)])
+            if rep == 1:
+                idx[0, K - 1] = e + 3
+            base = rng.standard_normal((layers, h)).astype(np.float32) if rep == 2 else np.zeros((layers, h), np.float32)
+            flags = fb.ACCUMULATE if rep == 2 else 0
+            dx, di, dw = (torch.from_numpy(a).cuda() for a in (x, idx, w))
+            d_one, d_three = torch.from_numpy(base).cuda(), torch.from_numpy(base).cuda()
+            torch.cuda.synchronize()
+            ctx.gguf_moe_decode_step_dev(0, layers, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K, d_one.data_ptr(),
+                                         None, flags)
+            ctx.sync()
+            try:
+                ctx.set_kernel_forms(fb.FORM_GGUF_PHASES)
+                ctx.gguf_moe_decode_step_dev(0, layers, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K,
+                                             d_three.data_ptr(), None, flags)
+                ctx.sync()
+            finally:
+                ctx.set_kernel_forms(0)
+            one, three = d_one.cpu().numpy(), d_three.cpu().numpy()
+            assert np.array_equal(one.view(np.uint32), three.view(np.uint32)), rep
+            for l in range(layers):
+                ok = (idx[l] >= 0) & (idx[l] < e)
+                ref, _ = orc.moe_gguf_forward(*store[l], x[l], np.where(ok, idx[l], 0).astype(np.int32),
+                                              np.where(ok, w[l], 0).astype(np.float32), h, i, types=(12, 12, down_t))
+                assert_parity(one[l], base[l].astype(np.float64) + ref, "layer %d call %d" % (l, rep))
+    finally:
+        ctx.close()
+
+
 @pytest.mark.parametrize("M,K,h,i,seed", [(40, 8, 2048, 512, 1), (97, 4, 1024, 256, 2), (32, 8, 512, 512, 3)])
 def test_gguf_chunk_grouped_products(orc, M, K, h, i, seed):
     """Chunks of 32 positions and more on a Q4_K / Q4_K / Q6_K store take the grouped products

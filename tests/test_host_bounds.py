@@ -4,7 +4,8 @@ tests/host_bounds/bounds_main.cpp includes finchmoe_amd/csrc/fm_index.h — the 
 take their share / unit / lane arithmetic from — and walks every (workgroup, unit, lane, load) of
 the launches that bench.py and the GPU tests make, at their exact sizes (the 40 x 256 decode step
 at 3 and 4 bits, one layer per call, the GatedDeltaNet projections for one and for 512 positions,
-the vocabulary projection, the GGUF step and chunk, the stream probe), against the sizes of the
+the vocabulary projection, the GGUF step — as three launches and as one — and chunk, the stream
+probe), against the sizes of the
 buffers those callers allocate; for the streaming kernels it also checks that the weights are read
 exactly once.  Built with the address and undefined-behaviour sanitizers.  No GPU.
 """
@@ -40,7 +41,9 @@ def test_every_access_of_the_benchmark_launches_is_inside_its_buffer(walker):
                  "fused rows 1 groups x 8, 3-bit", "split phases 40 groups x 8, 4-bit",
                  "fused (counters) 40 groups x 8, 4-bit", "gguf stream gate/up Q4_K 40 groups x 8",
                  "gguf stream down Q6_K 40 groups x 8", "gguf stream down Q6_K 8 groups x 8",
-                 "fused rows, sweep of shapes", "fused rows + tail, LDS tables"):
+                 "fused rows, sweep of shapes", "fused rows + tail, LDS tables",
+                 "gguf fused rows Q6_K down, 40 groups x 8, 2048x512", "gguf fused rows Q6_K down, 1 groups x 8, 2048x512",
+                 "gguf fused rows Q4_K down, 3 groups x 8, 1024x512"):
         assert ("ok  " + case) in r.stdout or ("ok  dense " + case) in r.stdout, case
 
 
