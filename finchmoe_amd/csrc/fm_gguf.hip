@@ -473,7 +473,11 @@ __global__ __launch_bounds__(256) void fm_gguf_matvec_rows_k(const uint8_t *W, c
 // Register r of a chunk (both formats) pairs local values
 //   lo(r) = 32 (r / 16) + 4 ((r % 16) / 2) + r % 2   and   hi(r) = lo(r) + 2,
 // accumulator group = r / 16 (Q4_K sub-block of 32) or r / 8 (Q6_K scale group of 16).
-enum { GG_Q4 = 0, GG_Q6 = 1 };
+//
+// Q6_K rows of 2048 values (GG_Q6W: the vocabulary projection of a 2048-wide model) have 32
+// such chunks: the 16-lanes-per-row map with two chunks per lane, c and c + 16 (1024 values and
+// four blocks further on), a slice of four whole rows = 6720 B, two slices per ring.
+enum { GG_Q4 = 0, GG_Q6 = 1, GG_Q6W = 2 };
 
 template <int KIND, int LPR>
 struct GgLane;
@@ -492,9 +496,22 @@ struct GgLane<GG_Q6, LPR> {
     __device__ static int col(int c, int v) { return 128 * (c >> 1) + 32 * (c & 1) + (v < 32 ? v : v + 32); }
 };
 
+template <>
+struct GgLane<GG_Q6W, 16> {
+    static constexpr int NREG = 32, GROUP_REGS = 8;
+    static constexpr int ROW_BYTES = 8 * 210;
+    static constexpr int SLOT_DATA = 4 * ROW_BYTES;                    // 6720
+    __device__ static int col(int c, int v) { return GgLane<GG_Q6, 16>::col(c, v); }
+};
+// chunks an activation image holds per row (= lanes per row, except where a lane owns two)
+template <int KIND, int LPR>
+struct GgImgLpr {
+    static constexpr int value = KIND == GG_Q6W ? 2 * LPR : LPR;
+};
+
 template <int KIND, bool GU>
 struct GgRing {
-    static constexpr int value = KIND == GG_Q6 ? 5 : 3;
+    static constexpr int value = KIND == GG_Q6W ? 2 : KIND == GG_Q6 ? 5 : 3;
 };
 
 // activation image of one input vector: register quad q of entry e = 4*chunk + piece,
@@ -510,9 +527,10 @@ struct GgAct {
     float xsum[4];
 };
 
-template <int KIND, int LPR>
-__device__ __forceinline__ void gg_build_image(const float *x, GgImage<GgLane<KIND, LPR>::NREG, LPR> &L) {
-    using G = GgLane<KIND, LPR>;
+// (LPR = chunks per row of the image; LL = the lane map's lanes per row, which names the format's constants)
+template <int KIND, int LPR, int LL = LPR>
+__device__ __forceinline__ void gg_build_image(const float *x, GgImage<GgLane<KIND, LL>::NREG, LPR> &L) {
+    using G = GgLane<KIND, LL>;
     constexpr int NE = 4 * LPR;
     uint32_t *flat = reinterpret_cast<uint32_t *>(L.a);
     for (int it = threadIdx.x; it < LPR * G::NREG; it += blockDim.x) {
@@ -539,8 +557,9 @@ __device__ __forceinline__ void gg_build_image(const float *x, GgImage<GgLane<KI
 // a lane's activation registers out of an image, while LDS-direct loads are in flight
 // (explicit reads: see fm_ring.h)
 template <int NREG>
-__device__ __forceinline__ void gg_read_image(uint32_t img_addr, int n_entries, int lane, GgAct<NREG> &ar) {
-    const int e = lane % n_entries;
+__device__ __forceinline__ void gg_read_image(uint32_t img_addr, int n_entries, int lane, GgAct<NREG> &ar,
+                                              int entry0 = 0) {
+    const int e = lane % n_entries + entry0;
     uint32_t addr = img_addr + (uint32_t)e * 16u;
     const uint32_t stride = (uint32_t)n_entries * 16u;
 #pragma unroll
@@ -631,8 +650,11 @@ struct GgQ6Lane {
     uint32_t ql_off, qh_off, sc_off, d_off, sh_l, sh_h;
     template <int LPR>
     __device__ __forceinline__ void init(int row_in_step, int ch) {
+        init_rows(row_in_step, ch, GgLane<GG_Q6, LPR>::ROW_BYTES);
+    }
+    __device__ __forceinline__ void init_rows(int row_in_step, int ch, int row_bytes) {
         const int hf = (ch >> 1) & 1, sd = ch & 1;
-        const uint32_t blk = (uint32_t)(row_in_step * GgLane<GG_Q6, LPR>::ROW_BYTES + (ch >> 2) * 210);
+        const uint32_t blk = (uint32_t)(row_in_step * row_bytes + (ch >> 2) * 210);
         const uint32_t ql = blk + 64u * hf + 32u * sd, qh = blk + 128u + 32u * hf;
         ql_off = ql & ~3u;
         qh_off = qh & ~3u;
@@ -705,15 +727,33 @@ __device__ __forceinline__ void gg_dma(uint32_t slot, const uint8_t *src, int la
     }
 }
 
+// ---- Q6_K lane of a 2048-value row: chunks ch and ch + 16 of the row
+struct GgQ6WData {
+    GgQ6Data p[2];
+};
+struct GgQ6WLane {
+    GgQ6Lane l[2];
+    template <int LPR>
+    __device__ __forceinline__ void init(int row_in_step, int ch) {
+        l[0].init_rows(row_in_step, ch, GgLane<GG_Q6W, 16>::ROW_BYTES);
+        l[1].init_rows(row_in_step, ch + 16, GgLane<GG_Q6W, 16>::ROW_BYTES);
+    }
+    __device__ __forceinline__ fm_u4 read(uint32_t slot, uint32_t tag_addr, GgQ6WData &t) const {
+        (void)l[0].read(slot, tag_addr, t.p[0]);
+        return l[1].read(slot, tag_addr, t.p[1]);
+    }
+};
+
 template <int KIND> struct GgLaneOps;
 template <> struct GgLaneOps<GG_Q4> { using Lane = GgQ4Lane; using Data = Q4Half; };
 template <> struct GgLaneOps<GG_Q6> { using Lane = GgQ6Lane; using Data = GgQ6Data; };
+template <> struct GgLaneOps<GG_Q6W> { using Lane = GgQ6WLane; using Data = GgQ6WData; };
 
 template <int KIND, int LPR, bool GU>
 constexpr size_t gg_stream_lds() {
     using G = GgLane<KIND, LPR>;
     return (size_t)8 * GgRing<KIND, GU>::value * (G::SLOT_DATA + 16) +
-           (GU ? 2 : 3) * sizeof(GgImage<G::NREG, LPR>);
+           (GU ? 2 : 3) * sizeof(GgImage<G::NREG, GgImgLpr<KIND, LPR>::value>);
 }
 
 extern __shared__ __attribute__((aligned(16))) uint8_t fm_gguf_lds[];
@@ -752,9 +792,12 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
     using G = GgLane<KIND, LPR>;
     using Lane = typename GgLaneOps<KIND>::Lane;
     using Data = typename GgLaneOps<KIND>::Data;
-    using Image = GgImage<G::NREG, LPR>;
+    constexpr bool WIDE = KIND == GG_Q6W;
+    constexpr int ILPR = GgImgLpr<KIND, LPR>::value;
+    using Image = GgImage<G::NREG, ILPR>;
     constexpr int RPS = FM_WAVE / LPR, NS = GU ? 2 : 1, NIMG = GU ? 2 : 3;
     constexpr int RING = GgRing<KIND, GU>::value;
+    static_assert(!(WIDE && GU), "the two-chunk lane map is a down / dense-tensor form");
     constexpr int SLOT = G::SLOT_DATA + 16, TAG = G::SLOT_DATA, LOADS = (G::SLOT_DATA + 1023) / 1024;
     // pairs a workgroup's share can touch: it spans at most NIMG - 1 input vectors' worth
     constexpr int NPAIR = GU ? FM_MAX_K + 1 : NIMG;
@@ -859,10 +902,10 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
 
     // the images of every input vector this workgroup's units touch
     for (int v = 0; v < n_img && v < NIMG; v++)
-        gg_build_image<KIND, LPR>(xbase + (size_t)(vid0 + v) * in_dim, img[v]);
+        gg_build_image<KIND, ILPR, LPR>(xbase + (size_t)(vid0 + v) * in_dim, img[v]);
     __syncthreads();
 
-    GgAct<G::NREG> ar;
+    GgAct<G::NREG> ar, ar2;        // (ar2: the second chunk of a lane that owns two)
     uint32_t cur_image = ~0u;
     const uint32_t ones = fm_opaque(0x3F803F80u);
     int c = 0;
@@ -882,11 +925,14 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
             if (k == 0) {
                 const uint32_t image = __builtin_amdgcn_readfirstlane(tag[3]);
                 if (image != cur_image) {
-                    gg_read_image<G::NREG>(img0 + image * (uint32_t)sizeof(Image), 4 * LPR, lane, ar);
+                    gg_read_image<G::NREG>(img0 + image * (uint32_t)sizeof(Image), 4 * ILPR, lane, ar);
+                    if constexpr (WIDE)
+                        gg_read_image<G::NREG>(img0 + image * (uint32_t)sizeof(Image), 4 * ILPR, lane, ar2, 4 * LPR);
                     cur_image = image;
                 }
             }
-            v[k] = fm_chunk_sum<LPR>(ln.dot(t, ar, ones));
+            if constexpr (WIDE) v[k] = fm_chunk_sum<LPR>(ln.l[0].dot(t.p[0], ar, ones) + ln.l[1].dot(t.p[1], ar2, ones));
+            else v[k] = fm_chunk_sum<LPR>(ln.dot(t, ar, ones));
         }
         const uint32_t pair = __builtin_amdgcn_readfirstlane(tag[1]);
         const uint32_t step = __builtin_amdgcn_readfirstlane(tag[2]);
@@ -1388,21 +1434,29 @@ int gg_launch_stream(const GgufArgs &a, int n_pairs, int n_cu, hipStream_t st) {
     if (!plan.ok) return FM_ERR_UNSUPPORTED;
     const int lpr = plan.lpr, upp = plan.upp;
     const long total = plan.total, wgs = plan.wgs;
-#define GG_ST(L)                                                                               \
+#define GG_STK(KK, L)                                                                          \
     do {                                                                                       \
-        auto kfn = fm_gguf_stream<KIND, L, GU>;                                                \
-        const size_t sh = gg_stream_lds<KIND, L, GU>();                                        \
+        auto kfn = fm_gguf_stream<KK, L, GU>;                                                  \
+        const size_t sh = gg_stream_lds<KK, L, GU>();                                          \
         static FmLdsAttr attr;                                                                 \
         if (!fm_dyn_lds_ready(attr, (const void *)kfn, sh)) return FM_ERR_HIP;                 \
         hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(512), sh, st, a, (int)total,            \
                            gg_div_make((uint32_t)upp), gg_div_make((uint32_t)a.K));   \
     } while (0)
+#define GG_ST(L) GG_STK(KIND, L)
+    if constexpr (KIND == GG_Q6 && !GU) {
+        if (plan.wide) {
+            GG_STK(GG_Q6W, 16);
+            return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
+        }
+    }
     switch (lpr) {
         case 4: GG_ST(4); break;
         case 8: GG_ST(8); break;
         default: GG_ST(16); break;
     }
 #undef GG_ST
+#undef GG_STK
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 

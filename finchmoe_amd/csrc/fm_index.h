@@ -560,6 +560,8 @@ struct FmGgPlan {
     int slot_data;      // bytes of a slice = the rows of a wave step as they lie in memory
     int row_bytes;
     int n_img, n_pair;  // images / pair entries a workgroup keeps
+    int wide;           // Q6_K rows of 2048 values: a lane owns two 64-value pieces, 1024 values apart
+    int ring;           // slices per wave's ring
 };
 // q6: Q6_K (a lane owns 64 values) else Q4_K (128); gu: gate and up rows of a unit
 FM_HD FmGgPlan fm_gg_plan(int n_pairs, int K, int in_dim, int rows, int q6, int gu, int n_cu) {
@@ -567,11 +569,13 @@ FM_HD FmGgPlan fm_gg_plan(int n_pairs, int K, int in_dim, int rows, int q6, int 
     p.ok = 0;
     p.wgs = 0, p.total = 0;
     const int per_lane = q6 ? 64 : 128;
-    p.lpr = in_dim / per_lane;
+    p.wide = q6 && !gu && in_dim == 2048;
+    p.lpr = p.wide ? 16 : in_dim / per_lane;
     p.rps = p.lpr > 0 ? FM_WAVE / p.lpr : 0;
     p.upp = p.rps > 0 ? rows / p.rps : 0;
-    p.row_bytes = q6 ? (p.lpr / 4) * 210 : (p.lpr / 2) * 144;
+    p.row_bytes = q6 ? (in_dim / 256) * 210 : (p.lpr / 2) * 144;
     p.slot_data = p.rps * p.row_bytes;
+    p.ring = p.wide ? 2 : q6 ? 5 : 3;
     p.n_img = gu ? 2 : 3;
     p.n_pair = gu ? FM_MAX_K + 1 : 3;
     if (in_dim % per_lane || !(p.lpr == 4 || p.lpr == 8 || p.lpr == 16)) return p;

@@ -599,8 +599,31 @@ static void walk_gguf_stream(int n_groups, int K, int hidden, int inter, bool gu
     }
     const size_t slab = (size_t)rows * pl.row_bytes;       // one expert's rows of one matrix
     CHECK((size_t)pl.upp * pl.slot_data == slab, "slices tile the expert");
-    const int ring = q6 ? 5 : 3, nreg = q6 ? 32 : 64;
-    const size_t img = (size_t)(nreg / 4) * 4 * pl.lpr * 16 + pl.lpr * 16;
+    const int ring = pl.ring, nreg = q6 ? 32 : 64, img_lpr = pl.wide ? 2 * pl.lpr : pl.lpr;
+    CHECK(ring == (pl.wide ? 2 : q6 ? 5 : 3), "ring of %d slices", ring);
+    CHECK(pl.row_bytes == (q6 ? (in_dim / 256) * 210 : (in_dim / 256) * 144), "row of %d bytes", pl.row_bytes);
+    const size_t img = (size_t)(nreg / 4) * 4 * img_lpr * 16 + img_lpr * 16;
+    if (q6) {   // every column of the row is some lane's: chunk c (and c + 16 where a lane owns two), value v
+        std::vector<uint8_t> seen((size_t)in_dim, 0);
+        for (int lane = 0; lane < 64; lane++) {
+            const int j = lane & 3, ch = (lane >> 2) % pl.lpr, ris = 4 * (lane / (4 * pl.lpr)) + j;
+            CHECK(ris < pl.rps, "row in step %d", ris);
+            if (ris != 0) continue;
+            for (int pass = 0; pass < (pl.wide ? 2 : 1); pass++) {
+                const int c = ch + 16 * pass;
+                CHECK(4 * c + 3 < 4 * img_lpr, "image entry of chunk %d", c);
+                // bytes of the lane's piece inside its row: ql [64 hf + 32 sd, +32) and qh [128 + 32 hf, +32) of block c / 4
+                const int hf = (c >> 1) & 1, sd = c & 1, blk = (c >> 2) * 210;
+                CHECK(blk + 210 <= pl.row_bytes && blk + 64 * hf + 32 * sd + 36 <= pl.row_bytes + 2, "piece of chunk %d", c);
+                for (int v = 0; v < 64; v++) {
+                    const int col = 128 * (c >> 1) + 32 * (c & 1) + (v < 32 ? v : v + 32);
+                    CHECK(col < in_dim, "column %d", col);
+                    if (col < in_dim) seen[col]++;
+                }
+            }
+        }
+        for (int c = 0; c < in_dim; c++) CHECK(seen[c] == 1, "column %d owned %d times", c, (int)seen[c]);
+    }
     const size_t lds = (size_t)8 * ring * (pl.slot_data + 16) + pl.n_img * img + pl.n_pair * 32 + 16;
     CHECK(lds <= 160 * 1024, "LDS %zu", lds);
     std::vector<Region> m0, m1;
@@ -885,7 +908,9 @@ int main() {
     walk_gguf_stream(1, 1, 248320, 1024, false, 1, "Q6_K 248320x1024");
     walk_gguf_stream(1, 1, 4096, 2048, false, 0, "Q4_K 4096x2048");
     walk_gguf_stream(1, 1, 4096, 1024, false, 1, "Q6_K 4096x1024");
-    walk_gguf_stream(1, 1, 1024, 2048, false, 1, "Q6_K 1024x2048 (rows-per-wave kernel)");
+    walk_gguf_stream(1, 1, 1024, 2048, false, 1, "Q6_K 1024x2048 (two chunks per lane)");
+    walk_gguf_stream(1, 1, 248320, 2048, false, 1, "Q6_K 248320x2048 (two chunks per lane)");
+    walk_gguf_stream(2, 4, 512, 2048, false, 1, nullptr);
     if (g_fail) {
         std::fprintf(stderr, "%d checks failed\n", g_fail);
         return 1;
