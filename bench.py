@@ -874,7 +874,7 @@ def run_gguf(args):
 
         ms, ev = _timed(ctx, cstep, args)
         assert torch.isfinite(c_out).all()
-        grouped = M >= 32 and not per_position
+        grouped = M >= 32 and M * K >= 2 * E and not per_position      # the library's own condition
         # grouped products read an expert once per group of its positions: priced on the distinct
         # experts of a chunk; per-position products stream every routed expert once per position
         uniq = float(np.mean([len(set(idx[:M, l].reshape(-1).tolist())) for l in range(n_layers)]))
@@ -895,7 +895,7 @@ def run_gguf(args):
         return _finish(cres,
                        "GGUF Q4_K/Q6_K expert GEMV HBM GB/s, %d-position chunk of one layer" % M,
                        "config 4, chunk variant: %d positions x top-8 Zipf(1.1) on one of %d GGUF layers "
-                       "(Q4_K gate/up, Q6_K down), %s products" % (M, n_layers, "grouped" if M >= 32 and not per_position else "per-position"),
+                       "(Q4_K gate/up, Q6_K down), %s products" % (M, n_layers, "grouped" if grouped else "per-position"),
                        M * K * (2 * gsl + dsl), ms, args)
     d_idx, d_w = torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)
     d_x = torch.randn(n_layers, H, device=dev)

@@ -1561,9 +1561,9 @@ extern "C" size_t fm_prefill_gguf_ws_bytes(const FmGgufGeom *g, int M, int K);
 extern "C" int fm_launch_prefill_gguf(const uint8_t *d_gate, const uint8_t *d_up, const uint8_t *d_down,
                                       const FmGgufGeom *g, const float *d_X, const int32_t *d_idx,
                                       const float *d_w, int M, int K, float *d_out, void *d_ws,
-                                      size_t ws_bytes, int flags, hipStream_t st);
+                                      size_t ws_bytes, int flags, int n_cu, hipStream_t st);
 
-// Chunks of FM_PREFILL_GEMM_MIN_M positions and more with at least four (position, slot) pairs
+// Chunks of FM_PREFILL_GEMM_MIN_M positions and more with at least two (position, slot) pairs
 // per expert take the grouped products (every routed
 // expert streamed once per group of its positions; prefill_chunk_cmd3_batch_general,
 // finchmoe/infer.m:10958-11059, streams it once per position) when the store is Q4_K gate/up
@@ -1574,11 +1574,11 @@ extern "C" int fm_gguf_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, c
     if (!c) return FM_ERR_ARG;
     if (M < 1 || M > FM_MAX_CHUNK) return fail(c, FM_ERR_ARG, "M %d outside 1..%d", M, FM_MAX_CHUNK);
     const bool no_group = (fm_kernel_forms & FM_FORM_NO_GGUF_GROUP) != 0;
-    // (grouping pays from about four positions per expert on: measured at 256 experts, a chunk of
-    // 64 positions is faster position by position, 152 against 179 us, one of 512 is 2.7 times
-    // faster grouped)
+    // (grouping pays from two (position, slot) pairs per expert on: measured at 256 experts, chunks of
+    // 64 / 96 / 128 / 512 positions take 134 / 150 / 172 / 295 us grouped and 152 / 242 / 281 / 1050 us
+    // position by position; at 32 positions, one pair per expert, both stream every expert once)
     if (c->gguf_cfg && M >= FM_PREFILL_GEMM_MIN_M && !(flags & FM_GUARD) && !no_group && d_X && d_idx &&
-        d_w && d_out && K >= 1 && K <= FM_MAX_K && (long)M * K >= 4L * c->ggeom.n_experts) {
+        d_w && d_out && K >= 1 && K <= FM_MAX_K && (long)M * K >= 2L * c->ggeom.n_experts) {
         const size_t ws = fm_prefill_gguf_ws_bytes(&c->ggeom, M, K);
         if (ws) {
             int rc = check_layers(c, c->g_gate, layer, 1);
@@ -1587,7 +1587,7 @@ extern "C" int fm_gguf_moe_prefill_dev(fm_ctx *c, int layer, const float *d_X, c
             if ((rc = ensure_ws(c, ws))) return rc;
             rc = fm_launch_prefill_gguf((const uint8_t *)c->g_gate[layer].ptr, (const uint8_t *)c->g_up[layer].ptr,
                                         (const uint8_t *)c->g_down[layer].ptr, &c->ggeom, d_X, d_idx, d_w, M,
-                                        K, d_out, c->d_ws, c->ws_bytes, flags, c->stream);
+                                        K, d_out, c->d_ws, c->ws_bytes, flags, c->n_cu, c->stream);
             if (rc == FM_OK) return FM_OK;
             if (rc != FM_ERR_UNSUPPORTED)
                 return fail(c, rc, "GGUF prefill launch failed: %s", hipGetErrorString(hipGetLastError()));

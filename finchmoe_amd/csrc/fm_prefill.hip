@@ -1501,7 +1501,9 @@ bool pf_dense_supported(int out_dim, int in_dim, int group_size, int bits) {
 // p + 8 of a 16x16x32 product, down runs two 16x16x16 products on one accumulator.
 // ======================================================================
 typedef short gq_s4 __attribute__((ext_vector_type(4)));
-constexpr int GQ_TM_UP = 8, GQ_TM_DN = 16;
+constexpr int GQ_TM_DN = 16;
+// positions of a gate/up item: 16 where the two images of 16 positions fit in LDS, else 8
+static inline int gq_tm_up(const FmGgufGeom *g) { return g->hidden <= 2048 ? 16 : 8; }
 
 __device__ __forceinline__ uint32_t gq_hi(float v) { return __float_as_uint(v) >> 16; }
 __device__ __forceinline__ uint32_t gq_lo(float v) {
@@ -1529,101 +1531,164 @@ __device__ __forceinline__ void gq_scale_min(uint32_t s0, uint32_t s1, uint32_t 
     mn = (float)b;
 }
 
-// gate/up: Q4_K rows [inter][hidden/256 blocks of 144 B]; item = (expert, <= 8 positions)
+// gate/up: Q4_K rows [inter][hidden/256 blocks of 144 B]; item = (expert, <= TM positions).
+// TM = 8: the two bf16 pieces of position p in M rows p and p + 8 of one product.  TM = 16 (rows
+// of at most 2048 values: the two images are 128 KB): a product per piece on one accumulator —
+// twice the matrix instructions per item, but an expert with many positions is streamed and
+// unpacked half as often.  A lane's bytes of the next block are requested before the block in
+// hand is multiplied.
+struct GqUpBlock {
+    uint4 hdr[2];
+    uint2 qs[2][4];
+};
+__device__ __forceinline__ void gq_up_load(GqUpBlock &k, const uint8_t *const rp[2], int b, int kb) {
+#pragma unroll
+    for (int T = 0; T < 2; T++) {
+        const uint8_t *blk = rp[T] + (size_t)b * 144;
+        k.hdr[T] = *reinterpret_cast<const uint4 *>(blk);
+#pragma unroll
+        for (int c = 0; c < 4; c++) k.qs[T][c] = *reinterpret_cast<const uint2 *>(blk + 16 + 32 * c + 8 * kb);
+    }
+}
+// A workgroup's share of the launch: units u0 .. u1 of n_items * per_item, a unit = (item, group of
+// eight 16-row tiles, one per wave).  Contiguous shares: a workgroup stages an item's positions
+// when its units change item — once or twice more than its share of the items.
+struct GqShare {
+    int u0, u1;
+};
+__device__ __forceinline__ GqShare gq_share(int n_items, int per_item) {
+    const long total = (long)n_items * per_item;
+    GqShare s;
+    s.u0 = (int)(total * blockIdx.x / gridDim.x);
+    s.u1 = (int)(total * (blockIdx.x + 1) / gridDim.x);
+    return s;
+}
+
+template <int TM>
 __global__ __launch_bounds__(512) void fm_gq_gate_up(PfArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)
     extern __shared__ __attribute__((aligned(16))) uint8_t gq_smem[];
-    const int it = blockIdx.x;
-    if (it >= *a.n_items_up) return;
-    const PfItem item = a.items_up[it];
+    constexpr bool TWO = TM == 16;
     const int H = a.g.hidden, I = a.g.inter, NKS = H / 32, NB = H / 256;
-    uint4 *img = reinterpret_cast<uint4 *>(gq_smem);                       // [NKS][64 lanes]
-    float *xs = reinterpret_cast<float *>(gq_smem + (size_t)NKS * 1024);   // [NKS][16 M rows]
+    const int tiles = I / 16, per_item = (tiles + 7) / 8;
+    const GqShare sh_ = gq_share(*a.n_items_up, per_item);
+    uint4 *img = reinterpret_cast<uint4 *>(gq_smem);                       // [NKS][64 lanes] (TWO: the hi pieces)
+    uint4 *img_lo = img + (size_t)NKS * 64;                                // TWO only
+    float *xs = reinterpret_cast<float *>(gq_smem + (size_t)NKS * 1024 * (TWO ? 2 : 1));   // [NKS][16 M rows]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, kb = lane >> 4;
-
-    // ---- stage: thread (position p, k steps ks, ks + 64, ...): hi pieces to M row p, lo to p + 8
-    {
-        const int p = threadIdx.x & 7;
-        const bool on = p < item.count;
-        const size_t m = on ? (size_t)(a.sorted[item.start + p] / a.K) : 0;
-        for (int ks = threadIdx.x >> 3; ks < NKS; ks += 64) {
-            float x[32];
-            const float4 *src = reinterpret_cast<const float4 *>(a.X + m * H + 32 * ks);
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const float4 v = on ? src[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                x[4 * i] = v.x, x[4 * i + 1] = v.y, x[4 * i + 2] = v.z, x[4 * i + 3] = v.w;
-            }
-            float sum = 0.0f;
-#pragma unroll
-            for (int i = 0; i < 32; i++) sum += gq_both(x[i]);
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                // k slots of lane group q: bytes 0 2 | 1 3 | 4 6 | 5 7 of its eight values
-                const float *v = x + 8 * q;
-                const uint4 hi = make_uint4(gq_hi(v[0]) | (gq_hi(v[2]) << 16), gq_hi(v[1]) | (gq_hi(v[3]) << 16),
-                                            gq_hi(v[4]) | (gq_hi(v[6]) << 16), gq_hi(v[5]) | (gq_hi(v[7]) << 16));
-                const uint4 lo = make_uint4(gq_lo(v[0]) | (gq_lo(v[2]) << 16), gq_lo(v[1]) | (gq_lo(v[3]) << 16),
-                                            gq_lo(v[4]) | (gq_lo(v[6]) << 16), gq_lo(v[5]) | (gq_lo(v[7]) << 16));
-                img[(size_t)ks * 64 + 16 * q + p] = hi;
-                img[(size_t)ks * 64 + 16 * q + p + 8] = lo;
-            }
-            xs[ks * 16 + p] = sum;
-            xs[ks * 16 + p + 8] = 0.0f;
-        }
-    }
-    __syncthreads();
-
     const size_t row_bytes = (size_t)NB * 144;
-    const uint8_t *gbase = a.gq_gate + (size_t)item.expert * I * row_bytes;
-    const uint8_t *ubase = a.gq_up + (size_t)item.expert * I * row_bytes;
     const uint32_t ones = fm_opaque(0x3F803F80u);
-    for (int tile = wave; tile < I / 16; tile += 8) {
+    int cur_item = -1;
+    const int n_items = *a.n_items_up;
+    PfItem item{0, 0, 0, 0}, item_next{0, 0, 0, 0};
+    GqUpBlock pre;                           // the first block of this wave's next tile, requested a tile ahead
+    bool pre_ok = false;
+    for (int u = sh_.u0; u < sh_.u1; u++) {
+        const int it = u / per_item, part = u - it * per_item;
+        if (it != cur_item) {
+            cur_item = it;
+            item = a.items_up[it];
+            item_next = a.items_up[it + 1 < n_items ? it + 1 : it];
+            __syncthreads();                 // every wave is done with the images of the item before
+            // ---- stage: thread (position p, k steps ks, ks + 512 / TM, ...)
+            const int p = threadIdx.x & (TM - 1);
+            const bool on = p < item.count;
+            const size_t m = on ? (size_t)(a.sorted[item.start + p] / a.K) : 0;
+            for (int ks = threadIdx.x / TM; ks < NKS; ks += 512 / TM) {
+                float x[32];
+                const float4 *src = reinterpret_cast<const float4 *>(a.X + m * H + 32 * ks);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float4 v = on ? src[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                    x[4 * i] = v.x, x[4 * i + 1] = v.y, x[4 * i + 2] = v.z, x[4 * i + 3] = v.w;
+                }
+                float sum = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 32; i++) sum += gq_both(x[i]);
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    // k slots of lane group q: bytes 0 2 | 1 3 | 4 6 | 5 7 of its eight values
+                    const float *v = x + 8 * q;
+                    const uint4 hi = make_uint4(gq_hi(v[0]) | (gq_hi(v[2]) << 16), gq_hi(v[1]) | (gq_hi(v[3]) << 16),
+                                                gq_hi(v[4]) | (gq_hi(v[6]) << 16), gq_hi(v[5]) | (gq_hi(v[7]) << 16));
+                    const uint4 lo = make_uint4(gq_lo(v[0]) | (gq_lo(v[2]) << 16), gq_lo(v[1]) | (gq_lo(v[3]) << 16),
+                                                gq_lo(v[4]) | (gq_lo(v[6]) << 16), gq_lo(v[5]) | (gq_lo(v[7]) << 16));
+                    img[(size_t)ks * 64 + 16 * q + p] = hi;
+                    if constexpr (TWO) img_lo[(size_t)ks * 64 + 16 * q + p] = lo;
+                    else img[(size_t)ks * 64 + 16 * q + p + 8] = lo;
+                }
+                xs[ks * 16 + p] = sum;
+                if constexpr (!TWO) xs[ks * 16 + p + 8] = 0.0f;
+            }
+            __syncthreads();
+        }
+        const int tile = part * 8 + wave;
+        if (tile >= tiles) continue;
+        const uint8_t *gbase = a.gq_gate + (size_t)item.expert * I * row_bytes;
+        const uint8_t *ubase = a.gq_up + (size_t)item.expert * I * row_bytes;
         const int row = tile * 16 + n;
-        const uint8_t *rp[2] = {gbase + (size_t)row * row_bytes, ubase + (size_t)row * row_bytes};
+        const uint8_t *const rp[2] = {gbase + (size_t)row * row_bytes, ubase + (size_t)row * row_bytes};
         pfr_f4 acc[2] = {pfr_f4{0.0f, 0.0f, 0.0f, 0.0f}, pfr_f4{0.0f, 0.0f, 0.0f, 0.0f}};
+        GqUpBlock cur;
+        if (pre_ok) cur = pre;
+        else gq_up_load(cur, rp, 0, kb);
+        pre_ok = false;
         for (int b = 0; b < NB; b++) {
-            uint4 hdr[2];
-            uint2 qs[2][4];
-#pragma unroll
-            for (int T = 0; T < 2; T++) {
-                const uint8_t *blk = rp[T] + (size_t)b * 144;
-                hdr[T] = *reinterpret_cast<const uint4 *>(blk);
-#pragma unroll
-                for (int c = 0; c < 4; c++) qs[T][c] = *reinterpret_cast<const uint2 *>(blk + 16 + 32 * c + 8 * kb);
+            GqUpBlock nxt = cur;
+            if (b + 1 < NB) {
+                gq_up_load(nxt, rp, b + 1, kb);
+            } else if (u + 1 < sh_.u1) {
+                const int it2 = (u + 1) / per_item, tile2 = (u + 1 - it2 * per_item) * 8 + wave;
+                if (tile2 < tiles) {
+                    const int e2 = it2 == cur_item ? item.expert : item_next.expert;
+                    const size_t r2 = ((size_t)e2 * I + (size_t)tile2 * 16 + n) * row_bytes;
+                    const uint8_t *const rp2[2] = {a.gq_gate + r2, a.gq_up + r2};
+                    gq_up_load(nxt, rp2, 0, kb);
+                    pre_ok = true;
+                }
             }
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 const int ks = b * 8 + j;
                 const uint4 av = img[(size_t)ks * 64 + lane];
+                uint4 al = av;
+                if constexpr (TWO) al = img_lo[(size_t)ks * 64 + lane];
                 const float4 xv = *reinterpret_cast<const float4 *>(xs + ks * 16 + 4 * kb);
 #pragma unroll
                 for (int T = 0; T < 2; T++) {
-                    const float d = fm_fp16_bits(hdr[T].x & 0xFFFFu), dmin = fm_fp16_bits(hdr[T].x >> 16);
+                    const float d = fm_fp16_bits(cur.hdr[T].x & 0xFFFFu), dmin = fm_fp16_bits(cur.hdr[T].x >> 16);
                     float sc, mn;
-                    gq_scale_min(hdr[T].y, hdr[T].z, hdr[T].w, j, sc, mn);
+                    gq_scale_min(cur.hdr[T].y, cur.hdr[T].z, cur.hdr[T].w, j, sc, mn);
                     const float c1 = 128.0f * (d * sc), c2 = c1 + dmin * mn;
-                    const uint2 w = qs[T][j >> 1];
+                    const uint2 w = cur.qs[T][j >> 1];
                     const int sh = (j & 1) * 4;
                     const pfr_u4 bq = {((w.x >> sh) & 0x000F000Fu) | ones, ((w.x >> (sh + 8)) & 0x000F000Fu) | ones,
                                        ((w.y >> sh) & 0x000F000Fu) | ones, ((w.y >> (sh + 8)) & 0x000F000Fu) | ones};
-                    const pfr_f4 D = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    pfr_f4 D = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                         __builtin_bit_cast(bf8, av), __builtin_bit_cast(bf8, bq), pfr_f4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+                    if constexpr (TWO)
+                        D = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8, al), __builtin_bit_cast(bf8, bq), D, 0, 0, 0);
                     acc[T][0] = fmaf(c1, D[0], fmaf(-c2, xv.x, acc[T][0]));
                     acc[T][1] = fmaf(c1, D[1], fmaf(-c2, xv.y, acc[T][1]));
                     acc[T][2] = fmaf(c1, D[2], fmaf(-c2, xv.z, acc[T][2]));
                     acc[T][3] = fmaf(c1, D[3], fmaf(-c2, xv.w, acc[T][3]));
                 }
             }
+            cur = nxt;
         }
-        // M rows p and p + 8 (lanes kb and kb + 2) are the two pieces of position p
+        pre = cur;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float g = acc[0][i] + __shfl_xor(acc[0][i], 32);
-            const float u = acc[1][i] + __shfl_xor(acc[1][i], 32);
             const int pos = 4 * kb + i;
-            if (kb < 2 && pos < item.count) a.act[(size_t)(item.start + pos) * I + row] = fm_silu_mul(g, u);
+            if constexpr (TWO) {
+                if (pos < item.count) a.act[(size_t)(item.start + pos) * I + row] = fm_silu_mul(acc[0][i], acc[1][i]);
+            } else {
+                // M rows p and p + 8 (lanes kb and kb + 2) are the two pieces of position p
+                const float g = acc[0][i] + __shfl_xor(acc[0][i], 32);
+                const float u_ = acc[1][i] + __shfl_xor(acc[1][i], 32);
+                if (kb < 2 && pos < item.count) a.act[(size_t)(item.start + pos) * I + row] = fm_silu_mul(g, u_);
+            }
         }
     }
 #else
@@ -1632,84 +1697,169 @@ __global__ __launch_bounds__(512) void fm_gq_gate_up(PfArgs a) {
 }
 
 // down: Q6_K rows [hidden][inter/256 blocks of 210 B]; item = (expert, <= 16 positions);
-// input a.act by sorted position, output a.eo by pair id
+// input a.act by sorted position, output a.eo by pair id.  Shares of units as in gate/up; a
+// lane's words of the next block are requested before the block in hand is multiplied.
+struct GqDnBlock {
+    uint32_t ql[8], qh[4], scw[4], d;      // ql[4 h + 2 (qt & 1) + (g & 1)], qh[2 h + (g & 1)]
+};
+__device__ __forceinline__ void gq_dn_load(GqDnBlock &k, const uint8_t *blk, int kb) {
+    struct __attribute__((packed, aligned(2))) U32a2 { uint32_t v; };
+    struct __attribute__((packed, aligned(2))) U16a2 { uint16_t v; };
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int o = 0; o < 2; o++) {
+            const int l = 16 * o + 4 * kb;
+#pragma unroll
+            for (int q1 = 0; q1 < 2; q1++) k.ql[4 * h + 2 * q1 + o] = reinterpret_cast<const U32a2 *>(blk + 64 * h + 32 * q1 + l)->v;
+            k.qh[2 * h + o] = reinterpret_cast<const U32a2 *>(blk + 128 + 32 * h + l)->v;
+        }
+#pragma unroll
+    for (int i = 0; i < 4; i++) k.scw[i] = reinterpret_cast<const U32a2 *>(blk + 192 + 4 * i)->v;
+    k.d = reinterpret_cast<const U16a2 *>(blk + 208)->v;
+}
+// one block of one 16-row tile: the lane's words in `cur`, acc += its share of sum y x
+__device__ __forceinline__ void gq_dn_block(const GqDnBlock &cur, int b, int lane, int kb, uint32_t ones,
+                                            const uint2 *img_hi, const uint2 *img_lo, const uint2 *xsi, pfr_f4 &acc) {
+    const float d = fm_fp16_bits(cur.d);
+    {   // - 160 d sum_g sc_g xs_g: the block's 16 scales (exact in bf16) times the groups' sums of x,
+        // this lane's k slots = groups 4 kb .. 4 kb + 3 = the bytes of scw[kb]
+        const uint32_t w = kb == 0 ? cur.scw[0] : kb == 1 ? cur.scw[1] : kb == 2 ? cur.scw[2] : cur.scw[3];
+        const uint32_t b0 = __float_as_uint((float)(int)(int8_t)(w & 0xFFu)) >> 16;
+        const uint32_t b1 = __float_as_uint((float)(int)(int8_t)((w >> 8) & 0xFFu)) & 0xFFFF0000u;
+        const uint32_t b2 = __float_as_uint((float)(int)(int8_t)((w >> 16) & 0xFFu)) >> 16;
+        const uint32_t b3 = __float_as_uint((float)(int)(int8_t)(w >> 24)) & 0xFFFF0000u;
+        const uint2 bs = make_uint2(b0 | b1, b2 | b3);
+        const uint2 *xp = xsi + (size_t)b * 3 * 64 + lane;
+        pfr_f4 E = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(gq_s4, xp[0]), __builtin_bit_cast(gq_s4, bs),
+                                                            pfr_f4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+        E = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(gq_s4, xp[64]), __builtin_bit_cast(gq_s4, bs), E, 0, 0, 0);
+        E = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(gq_s4, xp[128]), __builtin_bit_cast(gq_s4, bs), E, 0, 0, 0);
+        const float c2 = -160.0f * d;
+        acc[0] = fmaf(c2, E[0], acc[0]);
+        acc[1] = fmaf(c2, E[1], acc[1]);
+        acc[2] = fmaf(c2, E[2], acc[2]);
+        acc[3] = fmaf(c2, E[3], acc[3]);
+    }
+#pragma unroll
+    for (int g = 0; g < 16; g++) {
+        // group g: half h, quarter qt of the half (which nibble / which two qh bits),
+        // l = 16 (g & 1) + 4 kb .. + 3 (finchmoe/infer.m:1636-1657)
+        const int h = g >> 3, qt = (g >> 1) & 3;
+        const uint32_t wql = cur.ql[4 * h + 2 * (qt & 1) + (g & 1)];
+        const uint32_t wqh = cur.qh[2 * h + (g & 1)];
+        const uint32_t code = ((wql >> (4 * (qt >> 1))) & 0x0F0F0F0Fu) | (((wqh >> (2 * qt)) & 0x03030303u) << 4);
+        const uint2 bq = make_uint2((code & 0x00FF00FFu) | ones, ((code >> 8) & 0x00FF00FFu) | ones);
+        const int ks = b * 16 + g;
+        const uint2 ah = img_hi[(size_t)ks * 64 + lane], al = img_lo[(size_t)ks * 64 + lane];
+        pfr_f4 D = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(gq_s4, ah), __builtin_bit_cast(gq_s4, bq),
+                                                            pfr_f4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+        D = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(gq_s4, al), __builtin_bit_cast(gq_s4, bq), D, 0, 0, 0);
+        const float sc = (float)(int)(int8_t)((cur.scw[g >> 2] >> (8 * (g & 3))) & 0xFFu);
+        const float c1 = 128.0f * (d * sc);
+        acc[0] = fmaf(c1, D[0], acc[0]);
+        acc[1] = fmaf(c1, D[1], acc[1]);
+        acc[2] = fmaf(c1, D[2], acc[2]);
+        acc[3] = fmaf(c1, D[3], acc[3]);
+    }
+}
+
+// (A form that copied a tile's 16 whole rows — one contiguous run — into a per-wave LDS buffer with
+// 16-byte loads and picked the words out of LDS was slower, 146 against 124 us: the loads are not
+// what bounds this kernel.)
 __global__ __launch_bounds__(512) void fm_gq_down(PfArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)
     extern __shared__ __attribute__((aligned(16))) uint8_t gq_smem[];
     __shared__ int pairs[GQ_TM_DN];
-    const int it = blockIdx.x;
-    if (it >= *a.n_items_dn) return;
-    const PfItem item = a.items_dn[it];
+    constexpr int NW = 8, NT = NW * 64;
     const int H = a.g.hidden, I = a.g.inter, NKS = I / 16, NB = I / 256;
+    const int tiles = H / 16, per_item = (tiles + NW - 1) / NW;
+    const GqShare sh_ = gq_share(*a.n_items_dn, per_item);
     uint2 *img_hi = reinterpret_cast<uint2 *>(gq_smem);                    // [NKS][64 lanes]
     uint2 *img_lo = img_hi + (size_t)NKS * 64;
-    float *xs = reinterpret_cast<float *>(img_lo + (size_t)NKS * 64);      // [NKS][16 positions]
+    // the sums of x over each scale group, as three bf16 pieces (exactly the fp32 sum) in the
+    // operand form of a 16x16x16 product over a block's 16 groups: [NB][3 pieces][64 lanes]
+    uint2 *xsi = img_lo + (size_t)NKS * 64;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, kb = lane >> 4;
-    {
-        const int p = threadIdx.x & 15;
-        const bool on = p < item.count;
-        if (threadIdx.x < GQ_TM_DN) pairs[p] = on ? a.sorted[item.start + p] : 0;
-        const float *arow = a.act + (size_t)(item.start + (on ? p : 0)) * I;
-        for (int ks = threadIdx.x >> 4; ks < NKS; ks += 32) {
-            float x[16];
-            const float4 *src = reinterpret_cast<const float4 *>(arow + 16 * ks);
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float4 v = on ? src[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                x[4 * i] = v.x, x[4 * i + 1] = v.y, x[4 * i + 2] = v.z, x[4 * i + 3] = v.w;
-            }
-            float sum = 0.0f;
-#pragma unroll
-            for (int i = 0; i < 16; i++) sum += gq_both(x[i]);
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const float *v = x + 4 * q;        // k slots: values 0 2 | 1 3 of the lane group's four
-                img_hi[(size_t)ks * 64 + 16 * q + p] = make_uint2(gq_hi(v[0]) | (gq_hi(v[2]) << 16), gq_hi(v[1]) | (gq_hi(v[3]) << 16));
-                img_lo[(size_t)ks * 64 + 16 * q + p] = make_uint2(gq_lo(v[0]) | (gq_lo(v[2]) << 16), gq_lo(v[1]) | (gq_lo(v[3]) << 16));
-            }
-            xs[ks * 16 + p] = sum;
-        }
-    }
-    __syncthreads();
-
     const size_t row_bytes = (size_t)NB * 210;
-    const uint8_t *dbase = a.gq_down + (size_t)item.expert * H * row_bytes;
     const uint32_t ones = fm_opaque(0x3F803F80u);
-    struct __attribute__((packed, aligned(2))) U32a2 { uint32_t v; };
-    struct __attribute__((packed, aligned(2))) U16a2 { uint16_t v; };
-    for (int tile = wave; tile < H / 16; tile += 8) {
-        const int row = tile * 16 + n;
-        const uint8_t *rp = dbase + (size_t)row * row_bytes;
-        pfr_f4 acc = pfr_f4{0.0f, 0.0f, 0.0f, 0.0f};
-        for (int b = 0; b < NB; b++) {
-            const uint8_t *blk = rp + (size_t)b * 210;
-            const float d = fm_fp16_bits(reinterpret_cast<const U16a2 *>(blk + 208)->v);
-            uint32_t scw[4];
+    int cur_item = -1;
+    const int n_items = *a.n_items_dn;
+    PfItem item{0, 0, 0, 0}, item_next{0, 0, 0, 0};
+    GqDnBlock pre;                           // the first block of this wave's next tile, requested a tile ahead
+    bool pre_ok = false;
+    for (int u = sh_.u0; u < sh_.u1; u++) {
+        const int it = u / per_item, part = u - it * per_item;
+        if (it != cur_item) {
+            cur_item = it;
+            item = a.items_dn[it];
+            item_next = a.items_dn[it + 1 < n_items ? it + 1 : it];
+            __syncthreads();                 // every wave is done with the images and pair ids of the item before
+            const int p = threadIdx.x & 15;
+            const bool on = p < item.count;
+            if (threadIdx.x < GQ_TM_DN) pairs[p] = on ? a.sorted[item.start + p] : 0;
+            const float *arow = a.act + (size_t)(item.start + (on ? p : 0)) * I;
+            for (int ks = threadIdx.x >> 4; ks < NKS; ks += NT / 16) {
+                float x[16];
+                const float4 *src = reinterpret_cast<const float4 *>(arow + 16 * ks);
 #pragma unroll
-            for (int i = 0; i < 4; i++) scw[i] = reinterpret_cast<const U32a2 *>(blk + 192 + 4 * i)->v;
+                for (int i = 0; i < 4; i++) {
+                    const float4 v = on ? src[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                    x[4 * i] = v.x, x[4 * i + 1] = v.y, x[4 * i + 2] = v.z, x[4 * i + 3] = v.w;
+                }
+                float sum = 0.0f;
 #pragma unroll
-            for (int g = 0; g < 16; g++) {
-                // group g: half h, quarter qt of the half (which nibble / which two qh bits),
-                // l = 16 (g & 1) + 4 kb .. + 3 (finchmoe/infer.m:1636-1657)
-                const int h = g >> 3, qt = (g >> 1) & 3, l = 16 * (g & 1) + 4 * kb;
-                const uint32_t wql = reinterpret_cast<const U32a2 *>(blk + 64 * h + 32 * (qt & 1) + l)->v;
-                const uint32_t wqh = reinterpret_cast<const U32a2 *>(blk + 128 + 32 * h + l)->v;
-                const uint32_t code = ((wql >> (4 * (qt >> 1))) & 0x0F0F0F0Fu) | (((wqh >> (2 * qt)) & 0x03030303u) << 4);
-                const uint2 bq = make_uint2((code & 0x00FF00FFu) | ones, ((code >> 8) & 0x00FF00FFu) | ones);
-                const int ks = b * 16 + g;
-                const uint2 ah = img_hi[(size_t)ks * 64 + lane], al = img_lo[(size_t)ks * 64 + lane];
-                const float4 xv = *reinterpret_cast<const float4 *>(xs + ks * 16 + 4 * kb);
-                pfr_f4 D = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(gq_s4, ah), __builtin_bit_cast(gq_s4, bq),
-                                                                    pfr_f4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
-                D = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(gq_s4, al), __builtin_bit_cast(gq_s4, bq), D, 0, 0, 0);
-                const float sc = (float)(int)(int8_t)((scw[g >> 2] >> (8 * (g & 3))) & 0xFFu);
-                const float c1 = 128.0f * (d * sc), c2 = 160.0f * (d * sc);
-                acc[0] = fmaf(c1, D[0], fmaf(-c2, xv.x, acc[0]));
-                acc[1] = fmaf(c1, D[1], fmaf(-c2, xv.y, acc[1]));
-                acc[2] = fmaf(c1, D[2], fmaf(-c2, xv.z, acc[2]));
-                acc[3] = fmaf(c1, D[3], fmaf(-c2, xv.w, acc[3]));
+                for (int i = 0; i < 16; i++) sum += gq_both(x[i]);
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float *v = x + 4 * q;        // k slots: values 0 2 | 1 3 of the lane group's four
+                    img_hi[(size_t)ks * 64 + 16 * q + p] = make_uint2(gq_hi(v[0]) | (gq_hi(v[2]) << 16), gq_hi(v[1]) | (gq_hi(v[3]) << 16));
+                    img_lo[(size_t)ks * 64 + 16 * q + p] = make_uint2(gq_lo(v[0]) | (gq_lo(v[2]) << 16), gq_lo(v[1]) | (gq_lo(v[3]) << 16));
+                }
+                // group ks = 16 b + 4 kq + i: k slot i of lane (p, kq) of block b
+                const uint32_t s0 = __float_as_uint(sum) & 0xFFFF0000u;
+                const float r1 = sum - __uint_as_float(s0);
+                const uint32_t s1 = __float_as_uint(r1) & 0xFFFF0000u;
+                const uint32_t s2 = __float_as_uint(r1 - __uint_as_float(s1));
+                uint16_t *dst = reinterpret_cast<uint16_t *>(xsi + ((size_t)(ks >> 4) * 3) * 64 + 16 * ((ks >> 2) & 3) + p) + (ks & 3);
+                dst[0] = (uint16_t)(s0 >> 16);
+                dst[64 * 4] = (uint16_t)(s1 >> 16);
+                dst[2 * 64 * 4] = (uint16_t)(s2 >> 16);
             }
+            __syncthreads();
+        }
+        const int tile = part * NW + wave;
+        if (tile >= tiles) continue;
+        const int row = tile * 16 + n;
+        // the wave's tile of the next unit, if it has one
+        const uint8_t *next_src = nullptr;
+        if (u + 1 < sh_.u1) {
+            const int it2 = (u + 1) / per_item, tile2 = (u + 1 - it2 * per_item) * NW + wave;
+            if (tile2 < tiles) {
+                const int e2 = it2 == cur_item ? item.expert : item_next.expert;
+                next_src = a.gq_down + ((size_t)e2 * H + (size_t)tile2 * 16) * row_bytes;
+            }
+        }
+        pfr_f4 acc = pfr_f4{0.0f, 0.0f, 0.0f, 0.0f};
+        {
+            const uint8_t *rp = a.gq_down + ((size_t)item.expert * H + row) * row_bytes;
+            GqDnBlock cur;
+            if (pre_ok) cur = pre;
+            else gq_dn_load(cur, rp, kb);
+            pre_ok = false;
+            for (int b = 0; b < NB; b++) {
+                GqDnBlock nxt = cur;
+                if (b + 1 < NB) {
+                    gq_dn_load(nxt, rp + (size_t)(b + 1) * 210, kb);
+                } else if (next_src) {
+                    gq_dn_load(nxt, next_src + (size_t)n * row_bytes, kb);
+                    pre_ok = true;
+                }
+                gq_dn_block(cur, b, lane, kb, ones, img_hi, img_lo, xsi, acc);
+                cur = nxt;
+            }
+            pre = cur;
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -1821,7 +1971,7 @@ static bool gq_supported(const FmGgufGeom *g) {
 extern "C" size_t fm_prefill_gguf_ws_bytes(const FmGgufGeom *g, int M, int K) {
     if (!gq_supported(g) || M < 1 || K < 1) return 0;
     const size_t n = (size_t)M * K;
-    return align256(n * 4) + align256((g->n_experts + n / GQ_TM_UP + 1) * sizeof(PfItem)) +
+    return align256(n * 4) + align256((g->n_experts + n / gq_tm_up(g) + 1) * sizeof(PfItem)) +
            align256((g->n_experts + n / GQ_TM_DN + 1) * sizeof(PfItem)) + 256 +
            align256(n * g->inter * 4) + align256(n * g->hidden * 4);
 }
@@ -1831,7 +1981,7 @@ extern "C" size_t fm_prefill_gguf_ws_bytes(const FmGgufGeom *g, int M, int K) {
 extern "C" int fm_launch_prefill_gguf(const uint8_t *d_gate, const uint8_t *d_up, const uint8_t *d_down,
                                       const FmGgufGeom *g, const float *d_X, const int32_t *d_idx,
                                       const float *d_w, int M, int K, float *d_out, void *d_ws,
-                                      size_t ws_bytes, int flags, hipStream_t st) {
+                                      size_t ws_bytes, int flags, int n_cu, hipStream_t st) {
     if (!gq_supported(g)) return FM_ERR_UNSUPPORTED;
     if (ws_bytes < fm_prefill_gguf_ws_bytes(g, M, K)) return FM_ERR_ARG;
     const size_t n = (size_t)M * K;
@@ -1845,25 +1995,31 @@ extern "C" int fm_launch_prefill_gguf(const uint8_t *d_gate, const uint8_t *d_up
     a.w = d_w;
     a.M = M;
     a.K = K;
-    a.tm_up = GQ_TM_UP;
+    a.tm_up = gq_tm_up(g);
     a.tm_dn = GQ_TM_DN;
     a.gq_gate = d_gate;
     a.gq_up = d_up;
     a.gq_down = d_down;
     a.sorted = (int *)ws;                 ws += align256(n * 4);
-    a.items_up = (PfItem *)ws;            ws += align256((g->n_experts + n / GQ_TM_UP + 1) * sizeof(PfItem));
+    a.items_up = (PfItem *)ws;            ws += align256((g->n_experts + n / a.tm_up + 1) * sizeof(PfItem));
     a.items_dn = (PfItem *)ws;            ws += align256((g->n_experts + n / GQ_TM_DN + 1) * sizeof(PfItem));
     a.n_items_up = (int *)ws;
     a.n_items_dn = (int *)ws + 1;         ws += 256;
     a.act = (float *)ws;                  ws += align256(n * g->inter * 4);
     a.eo = (float *)ws;
+    const bool two = a.tm_up == 16;
+    const size_t lds_up = (size_t)(g->hidden / 32) * ((two ? 2048 : 1024) + 64), lds_dn = (size_t)(g->inter / 16) * 1024 + (size_t)(g->inter / 256) * 1536;
+    if (lds_up > 160 * 1024 - 1024 || lds_dn > 160 * 1024 - 1024) return FM_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(fm_pf_group, dim3(1), dim3(1024), 0, st, a);
-    const size_t lds_up = (size_t)(g->hidden / 32) * (1024 + 64), lds_dn = (size_t)(g->inter / 16) * (1024 + 64);
-    static FmLdsAttr attr_up, attr_dn;
-    if (!fm_dyn_lds_ready(attr_up, (const void *)fm_gq_gate_up, 160 * 1024 - 1024)) return FM_ERR_HIP;
+    static FmLdsAttr attr_up8, attr_up16, attr_dn;
+    if (!fm_dyn_lds_ready(attr_up8, (const void *)fm_gq_gate_up<8>, 160 * 1024 - 1024)) return FM_ERR_HIP;
+    if (!fm_dyn_lds_ready(attr_up16, (const void *)fm_gq_gate_up<16>, 160 * 1024 - 1024)) return FM_ERR_HIP;
     if (!fm_dyn_lds_ready(attr_dn, (const void *)fm_gq_down, 160 * 1024 - 1024)) return FM_ERR_HIP;
-    hipLaunchKernelGGL(fm_gq_gate_up, dim3((unsigned)(g->n_experts + n / GQ_TM_UP)), dim3(512), lds_up, st, a);
-    hipLaunchKernelGGL(fm_gq_down, dim3((unsigned)(g->n_experts + n / GQ_TM_DN)), dim3(512), lds_dn, st, a);
+    // persistent grids: one workgroup per CU for gate/up (its images fill most of the LDS), two for down
+    const dim3 grid_up((unsigned)(n_cu > 0 ? n_cu : 256)), grid_dn((unsigned)(2 * (n_cu > 0 ? n_cu : 256)));
+    if (two) hipLaunchKernelGGL(fm_gq_gate_up<16>, grid_up, dim3(512), lds_up, st, a);
+    else hipLaunchKernelGGL(fm_gq_gate_up<8>, grid_up, dim3(512), lds_up, st, a);
+    hipLaunchKernelGGL(fm_gq_down, grid_dn, dim3(512), lds_dn, st, a);
     hipLaunchKernelGGL(fm_pf_combine, dim3(M, (g->hidden + 1023) / 1024), dim3(256), 0, st, a, d_out, flags);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }

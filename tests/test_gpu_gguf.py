@@ -217,7 +217,8 @@ def test_gguf_one_launch_equals_three(orc, h, i, down_t, layers, K):
         ctx.close()
 
 
-@pytest.mark.parametrize("M,K,h,i,seed", [(40, 8, 2048, 512, 1), (97, 4, 1024, 256, 2), (32, 8, 512, 512, 3)])
+@pytest.mark.parametrize("M,K,h,i,seed", [(40, 8, 2048, 512, 1), (97, 4, 1024, 256, 2), (32, 8, 512, 512, 3),
+                                          (36, 4, 4096, 256, 4)])
 def test_gguf_chunk_grouped_products(orc, M, K, h, i, seed):
     """Chunks of 32 positions and more on a Q4_K / Q4_K / Q6_K store take the grouped products
     (an expert streamed once per group of its positions, prefill_chunk_cmd3_batch_general's
