@@ -1890,6 +1890,13 @@ extern "C" int fm_launch_prefill_dense(const void *d_W, const void *d_S, const v
     const size_t need = fm_prefill_dense_ws_bytes(out_dim, in_dim, group_size, bits, M);
     if (need == 0) return FM_ERR_UNSUPPORTED;
     if (ws_bytes < need) return FM_ERR_ARG;
+    {   // Launches in which a workgroup takes more than one step (more steps than CUs) last ran in a
+        // session that ended with a GPU memory fault whose cause is not known; the host walk of
+        // their addresses is clean, but until the cause is known they are not taken: the caller
+        // runs one GEMV per position.
+        const FmPfDenseGrid gr = fm_pf_dense_grid(M, out_dim, in_dim == 512, n_cu);
+        if ((long)gr.items * gr.n_steps > (long)n_cu) return FM_ERR_UNSUPPORTED;
+    }
     char *ws = (char *)d_ws;
     PfArgs a{};
     a.X = d_X;

@@ -233,8 +233,10 @@ FM_API int fm_matvec_batch(fm_ctx *ctx, const fm_tensor *tensors, int n, const f
  * finchmoe/infer.m:3672).  Fewer than 16 positions (and shapes the matrix-core kernel does
  * not cover) run one GEMV per position, bitwise equal to the one-position call; from 16
  * positions on a 3-/4-bit tensor with in_dim a multiple of 2048 and out_dim a multiple of 64,
- * or in_dim 512 and out_dim a multiple of 256, is multiplied on the matrix cores (equal to the one-position call within the parity bar;
- * d_X must be 16-byte aligned for it). */
+ * or in_dim 512 and out_dim a multiple of 256, is multiplied on the matrix cores (equal to the
+ * one-position call within the parity bar; d_X must be 16-byte aligned for it) as long as
+ * ceil(M / 16) * (out_dim / 64) -- out_dim / 256 at in_dim 512 -- does not exceed the number of
+ * compute units; larger products run one GEMV per position. */
 FM_API int fm_matvec_prefill_dev(fm_ctx *ctx, fm_tensor t, const float *d_X, float *d_out, int M);
 /* n tensors against the same X[M][in_dim] (each tensor as fm_matvec_prefill_dev; tensors the
  * matrix-core kernel covers share one preparation of X) */
