@@ -34,6 +34,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 peak
 # it comes from in roofline.traffic_source, and it is null for any other size.
 FUSED_TRAFFIC_BYTES_40L = int((218685.2 * 2 + 2237.6) * 1024)
 FUSED_TRAFFIC_SOURCE = "offline constant from profiles/decode_step_3bit_hbm_traffic.md (rocprofv3 --pmc), not measured in this run"
+# the same for the one-launch GGUF step (fm_gguf_fused_rows at 40 x 256, top-8)
+GGUF_FUSED_TRAFFIC_BYTES_40L = int((322728.2 * 2 + 2148.6) * 1024)
+GGUF_FUSED_TRAFFIC_SOURCE = "offline constant from profiles/gguf_step_and_gdn_kernel_trace.md (rocprofv3 --pmc), not measured in this run"
 
 H, I, E, K, L = 2048, 512, 256, 8, 40
 
@@ -928,6 +931,9 @@ def run_gguf(args):
         # the step is one launch: HIP events around the timed region on the library's stream
         res["roofline"] = _roofline_hbm("fm_gguf_fused_rows<Q6_K,16,8> (the step's one launch)",
                                         n_layers * K * (2 * gsl + dsl), ev * 1e3)
+        if (n_layers, E, K) == (40, 256, 8):
+            res["roofline"]["traffic"] = GGUF_FUSED_TRAFFIC_BYTES_40L
+            res["roofline"]["traffic_source"] = GGUF_FUSED_TRAFFIC_SOURCE
     res["roofline"]["step"] = {"bytes": n_layers * K * (2 * gsl + dsl), "us": round(ev * 1e3, 2),
                                "frac": round(n_layers * K * (2 * gsl + dsl) / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     if not args.no_cpu:
