@@ -1054,7 +1054,10 @@ def run_stream_probe(args):
     ctx = FinchHip(0)
     torch.cuda.synchronize()
     rates = {}
-    for pattern, name in ((1, "contiguous_share_per_workgroup"), (2, "contiguous_share_per_wave"),
+    # patterns 0..7 read with the non-temporal hint the decode kernels give their weight loads,
+    # 8 + p is walk p with ordinary caching
+    for pattern, name in ((9, "contiguous_share_per_workgroup_ordinary_caching"), (8, "dense_ordinary_caching"),
+                          (1, "contiguous_share_per_workgroup"), (2, "contiguous_share_per_wave"),
                           (3, "groups_of_4_workgroups_interleaved"), (4, "groups_of_8_workgroups_interleaved"),
                           (5, "groups_of_8_workgroups_of_one_xcd_interleaved"),
                           (6, "contiguous_share_per_workgroup_neighbours_on_one_xcd"),
@@ -1065,7 +1068,7 @@ def run_stream_probe(args):
         rates[name] = round(n / (ev * 1e-3) / 1e9, 1)
     ctx.close()
     res = {"event_ms_per_step": round(ev, 5), "GBps_by_pattern": rates,
-           "roofline": {"bound": "hbm", "kernel": "fm_stream_probe_k<0> (dense order)", "achieved": rates["dense"],
+           "roofline": {"bound": "hbm", "kernel": "fm_stream_probe_k<0, non-temporal> (dense order)", "achieved": rates["dense"],
                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(rates["dense"] / HBM_PEAK_GBS, 4),
                         "traffic": None, "bytes_per_launch": n, "us_per_launch": round(ev * 1e3, 2)}}
     return _finish(res, "streaming read GB/s of the probe kernel", "stream probe: %d bytes read once per step, "

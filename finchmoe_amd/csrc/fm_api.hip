@@ -537,8 +537,8 @@ static int ktiming_collect(fm_ctx *c) {
 
 extern "C" int fm_stream_probe_dev(fm_ctx *c, const void *d_buf, size_t nbytes, int pattern) {
     if (!c) return FM_ERR_ARG;
-    if (!d_buf || nbytes < 4096 || ((uintptr_t)d_buf & 15) || pattern < 0 || pattern > 7)
-        return fail(c, FM_ERR_ARG, "stream probe: a 16-byte aligned buffer of 4 KB or more, pattern 0..7");
+    if (!d_buf || nbytes < 4096 || ((uintptr_t)d_buf & 15) || pattern < 0 || pattern > 15)
+        return fail(c, FM_ERR_ARG, "stream probe: a 16-byte aligned buffer of 4 KB or more, pattern 0..15");
     DeviceGuard dg(c->device);
     int rc = fm_launch_stream_probe(d_buf, nbytes, pattern, nullptr, c->n_cu, c->stream);
     if (rc) return fail(c, rc, "stream probe launch failed: %s", hipGetErrorString(hipGetLastError()));

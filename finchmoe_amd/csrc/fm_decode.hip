@@ -301,6 +301,7 @@ struct FmOperatorStream {
     uint32_t tag_n, rsn, issued, consumed;
     const uint8_t *blob_n;
     bool dry;               // nothing more to hand out for now
+    bool once;              // every expert byte is read once in this launch (fm_ring.h, FM_AUX_ONCE)
     Raw raw_next;           // of segment cq + 2
     FmBuildSlot<BITS> bslot;
 
@@ -342,6 +343,8 @@ struct FmOperatorStream {
         tag_n = rsn = issued = consumed = 0;
         blob_n = nullptr;
         dry = false;
+        // layers of a step have stores of their own; the positions of a chunk share one layer's experts
+        once = a.layer_stride != 0 || n_pairs == a.K;
         raw_next = Raw{0, nullptr};
         bslot.init();
     }
@@ -427,7 +430,7 @@ struct FmOperatorStream {
         const uint8_t *b = blob_n + (size_t)rsn * cur_wstep;
         const uint8_t *sb = blob_n + (size_t)rsn * cur_sstep;
         const uint32_t second = (uint32_t)hn;                     // 1: the up rows of a unit
-        fm_dma_issue<BITS>(slot, b + cur_w + second * d_w, sb + cur_s + second * d_s,
+        fm_dma_issue_as<BITS>(once, slot, b + cur_w + second * d_w, sb + cur_s + second * d_s,
                            sb + cur_b + second * d_b, lane);
         if (l_gu) hn ^= 1;
         wpos = wpos + 1 == RING ? 0 : wpos + 1;
@@ -844,6 +847,7 @@ struct Fm2Stream {
     uint32_t tag_n, rsn, issued, consumed;
     const uint8_t *blob_n;
     bool dry;
+    bool once;              // every expert byte is read once in this launch (fm_ring.h, FM_AUX_ONCE)
     FmBuildSlot<BITS> bslot;
 
     __device__ __forceinline__ Fm2Stream(const DecodeArgs &a_, const Fm2Sync &sy_) : a(a_), sy(sy_) {
@@ -870,6 +874,7 @@ struct Fm2Stream {
         tag_n = rsn = issued = consumed = 0;
         blob_n = nullptr;
         dry = false;
+        once = a.layer_stride != 0;      // (one group: run() says so, it knows the number of groups)
         l_gu = true;
         bslot.init();
     }
@@ -919,7 +924,7 @@ struct Fm2Stream {
         const uint8_t *b = blob_n + (size_t)rsn * cur_wstep;
         const uint8_t *sb = blob_n + (size_t)rsn * cur_sstep;
         const uint32_t second = (uint32_t)hn;
-        fm_dma_issue<BITS>(slot, b + cur_w + second * d_w, sb + cur_s + second * d_s,
+        fm_dma_issue_as<BITS>(once, slot, b + cur_w + second * d_w, sb + cur_s + second * d_s,
                            sb + cur_b + second * d_b, lane);
         if (l_gu) hn ^= 1;
         wpos = wpos + 1 == RING ? 0 : wpos + 1;
@@ -996,6 +1001,7 @@ struct Fm2Stream {
         // workgroup with fewer down rows takes more gate/up units).
         // (32-bit arithmetic: the launcher checks that slices x workgroups stays below 2^31)
         by_gu_upp = dm.by_gu_upp, by_K = dm.by_K;
+        if (dm.L == 1u) once = true;
         const Fm2Split sp = fm2_split(dm, (uint32_t)g);
         const uint32_t gu_segu = dm.gu_segu;
         const int gu_s0 = sp.gu_s0;

@@ -251,6 +251,9 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
     uint32_t issued = 0, consumed = 0, tag_n = 0;
     const uint8_t *wp = nullptr, *sp = nullptr, *bp = nullptr;
     bool dry = false;
+    // one position: every weight byte is read once (fm_ring.h, FM_AUX_ONCE); with more positions
+    // (gridDim.y) each of them reads the tensors again
+    const bool once = gridDim.y == 1;
     auto issue = [&]() __attribute__((always_inline)) {
         if (dry) return;
         if (kn == 0) {
@@ -268,19 +271,23 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
         const uint32_t slot = ring0 + (uint32_t)wpos * SL::BYTES;
         fm_slot_tag(slot + SL::TAG, tag_n);
         if constexpr (NS == 1) {
-            fm_dma_issue<BITS>(slot, wp, sp, bp, lane);
+            fm_dma_issue_as<BITS>(once, slot, wp, sp, bp, lane);
         } else {
             // slab kn of the unit's rows: one 1 KB run per row, 64 B of scales / biases per row
-#pragma unroll
-            for (int i = 0; i < RPS; i++)
-                __builtin_amdgcn_global_load_lds(
-                    (fm_gptr)(uintptr_t)(wp + fm_dense_slab_woff(i, kn, lane, row_bytes, SLAB_ROW_BYTES)),
-                    (fm_lptr)(uintptr_t)(slot + 1024 * i), 16, 0, 0);
             const uint32_t so = fm_dense_slab_sboff(kn, lane, sb_row_bytes, SLAB_SB);
-            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(sp + so),
-                                             (fm_lptr)(uintptr_t)(slot + SL::WBYTES), 4, 0, 0);
-            __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(bp + so),
-                                             (fm_lptr)(uintptr_t)(slot + SL::WBYTES + 256), 4, 0, 0);
+#define FM_DENSE_SLAB_LOADS(AUX)                                                                        \
+    do {                                                                                                \
+        _Pragma("unroll") for (int i = 0; i < RPS; i++) __builtin_amdgcn_global_load_lds(               \
+            (fm_gptr)(uintptr_t)(wp + fm_dense_slab_woff(i, kn, lane, row_bytes, SLAB_ROW_BYTES)),      \
+            (fm_lptr)(uintptr_t)(slot + 1024 * i), 16, 0, AUX);                                         \
+        __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(sp + so),                                 \
+                                         (fm_lptr)(uintptr_t)(slot + SL::WBYTES), 4, 0, AUX);           \
+        __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(bp + so),                                 \
+                                         (fm_lptr)(uintptr_t)(slot + SL::WBYTES + 256), 4, 0, AUX);     \
+    } while (0)
+            if (once) FM_DENSE_SLAB_LOADS(FM_AUX_ONCE);
+            else FM_DENSE_SLAB_LOADS(FM_AUX_KEEP);
+#undef FM_DENSE_SLAB_LOADS
         }
         kn = kn + 1 == NS ? 0 : kn + 1;
         wpos = wpos + 1 == RING ? 0 : wpos + 1;

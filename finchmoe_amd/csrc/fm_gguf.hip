@@ -714,7 +714,7 @@ struct GgQ6Lane {
 
 // BYTES of a slice, 16 per lane and load; the last load is partial.  The
 // instruction offset moves the global and the LDS address alike.
-template <int BYTES, int I>
+template <int BYTES, int I, int AUX = FM_AUX_KEEP>
 __device__ __forceinline__ void gg_dma(uint32_t slot, const uint8_t *src, int lane) {
     if constexpr (I * 1024 < BYTES) {
         // (the offset field holds -4096..4095: from the fifth load on it starts again from
@@ -722,8 +722,8 @@ __device__ __forceinline__ void gg_dma(uint32_t slot, const uint8_t *src, int la
         constexpr int BASE = (I / 4) * 4096, IMM = (I % 4) * 1024;
         if (I * 1024 + lane * 16 < BYTES)
             __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(src + BASE),
-                                             (fm_lptr)(uintptr_t)(slot + BASE), 16, IMM, 0);
-        gg_dma<BYTES, I + 1>(slot, src, lane);
+                                             (fm_lptr)(uintptr_t)(slot + BASE), 16, IMM, AUX);
+        gg_dma<BYTES, I + 1, AUX>(slot, src, lane);
     }
 }
 
@@ -812,6 +812,9 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
     const long wg0 = wg.lo, wg1 = wg.hi;
     const uint32_t n_units = (uint32_t)(wg1 - wg0);
     if (n_units == 0) return;
+    // a dense tensor, the layers of a step, one layer: every byte is read once (fm_ring.h,
+    // FM_AUX_ONCE); the positions of a chunk share one layer's experts
+    const bool once = a.direct != nullptr || a.layer_stride != 0 || total_units == (int)(by_upp.d * by_k.d);
     const int in_dim = GU ? a.g.hidden : a.g.inter;
     // input vector of a pair: its layer's x (gate/up) or its own act (down)
     auto vector_of = [&](uint32_t pair) __attribute__((always_inline)) {
@@ -892,7 +895,8 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
             asm volatile("ds_write_b128 %0, %1" ::"v"(ta), "v"(tv) : "memory");
         }
         const uint8_t *src = p0 + (ptrdiff_t)kn * p_second + lane * 16;
-        gg_dma<G::SLOT_DATA, 0>(slot, src, lane);
+        if (once) gg_dma<G::SLOT_DATA, 0, FM_AUX_ONCE>(slot, src, lane);
+        else gg_dma<G::SLOT_DATA, 0, FM_AUX_KEEP>(slot, src, lane);
         kn = kn + 1 == NS ? 0 : kn + 1;
         wpos = wpos + 1 == RING ? 0 : wpos + 1;
         issued++;
@@ -1009,6 +1013,7 @@ struct GgFused {
     int n_up, n_seq;
     // loader
     bool l_gu, dry;
+    bool once;              // every expert byte is read once in this launch (fm_ring.h, FM_AUX_ONCE)
     int lq, cq, hn, wpos, c;
     uint32_t l_first, l_n, l_nrb, tag_n, issued, consumed;
     float l_inv;
@@ -1025,6 +1030,7 @@ struct GgFused {
         tab = reinterpret_cast<GgSeg *>(fm_gguf_lds + 8 * RING_BYTES + IMG_BYTES);
         part0 = img0 + (uint32_t)IMG_BYTES + FM2_MAX_SEG * (uint32_t)sizeof(GgSeg);
         l_gu = true, dry = false;
+        once = a.layer_stride != 0;
         lq = cq = hn = wpos = c = 0;
         l_first = l_n = l_nrb = tag_n = issued = consumed = 0u;
         l_inv = 0.0f;
@@ -1082,7 +1088,8 @@ struct GgFused {
         const uint32_t slot = ring0 + (uint32_t)wpos * SLOT;
         fm_slot_tag(slot + DATA, tag_n);
         const uint8_t *src = src_n + (GATE_UP ? (ptrdiff_t)hn * second_n : (ptrdiff_t)0) + lane * 16;
-        gg_dma<DATA, 0>(slot, src, lane);
+        if (once) gg_dma<DATA, 0, FM_AUX_ONCE>(slot, src, lane);
+        else gg_dma<DATA, 0, FM_AUX_KEEP>(slot, src, lane);
         if (GATE_UP) hn ^= 1;
         wpos = wpos + 1 == RING ? 0 : wpos + 1;
         issued++;
@@ -1207,6 +1214,7 @@ struct GgFused {
     __device__ __forceinline__ void run(const Fm2Dims &dm) {
         const int K = a.K, G = gridDim.x, g = blockIdx.x;
         by_gu_upp = dm.by_gu_upp, by_K = dm.by_K;
+        if (dm.L == 1u) once = true;
         const Fm2Split sp = fm2_split(dm, (uint32_t)g);
         const uint32_t gu_segu = dm.gu_segu;
         n_up = sp.n_up;

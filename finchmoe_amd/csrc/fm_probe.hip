@@ -26,7 +26,9 @@ extern __shared__ __attribute__((aligned(16))) uint8_t fm_probe_lds[];
 //   3, 4, 5  groups of 4 / 8 / 8 workgroups share a contiguous region whose slots go to the
 //      group's waves in turn (5: the eight workgroups of a group sit on one XCD)
 //   6  as 1 with neighbouring shares on one XCD;  7  groups of 4 workgroups of one XCD
-template <int PATTERN>
+// AUX: the loads' cache policy — FM_AUX_ONCE as the decode kernels read weights (fm_ring.h), or
+// FM_AUX_KEEP, ordinary caching (patterns 8..15 = 0..7 with it).
+template <int PATTERN, int AUX>
 __global__ __launch_bounds__(PROBE_WAVES * 64) void fm_stream_probe_k(const uint8_t *buf, size_t n_slots,
                                                                       unsigned int *sink) {
     const int lane = threadIdx.x & 63;
@@ -44,7 +46,7 @@ __global__ __launch_bounds__(PROBE_WAVES * 64) void fm_stream_probe_k(const uint
 #pragma unroll
         for (int j = 0; j < 4; j++)
             __builtin_amdgcn_global_load_lds((fm_gptr)(uintptr_t)(src + 1024 * j),
-                                             (fm_lptr)(uintptr_t)(slot + 1024 * j), 16, 0, 0);
+                                             (fm_lptr)(uintptr_t)(slot + 1024 * j), 16, 0, AUX);
         next += step;
         wpos = wpos + 1 == PROBE_RING ? 0 : wpos + 1;
         issued++;
@@ -70,16 +72,19 @@ __global__ __launch_bounds__(PROBE_WAVES * 64) void fm_stream_probe_k(const uint
 }  // namespace
 
 // reads nbytes (rounded down to whole 4 KB slots) of d_buf once, in the given pattern
+// (0..7 with the non-temporal hint, 8..15 the same walks with ordinary caching)
 extern "C" int fm_launch_stream_probe(const void *d_buf, size_t nbytes, int pattern, unsigned int *d_sink,
                                       int n_cu, hipStream_t st) {
     const size_t n_slots = nbytes / PROBE_SLOT;
-    if (!d_buf || n_slots == 0 || ((uintptr_t)d_buf & 15) || pattern < 0 || pattern > 7) return FM_ERR_ARG;
+    if (!d_buf || n_slots == 0 || ((uintptr_t)d_buf & 15) || pattern < 0 || pattern > 15) return FM_ERR_ARG;
     const size_t sh = (size_t)PROBE_WAVES * PROBE_RING * PROBE_SLOT;
-    static FmLdsAttr attr[8];
+    static FmLdsAttr attr[16];
     typedef void (*probe_fn)(const uint8_t *, size_t, unsigned int *);
-    static const probe_fn fns[8] = {fm_stream_probe_k<0>, fm_stream_probe_k<1>, fm_stream_probe_k<2>,
-                                    fm_stream_probe_k<3>, fm_stream_probe_k<4>, fm_stream_probe_k<5>,
-                                    fm_stream_probe_k<6>, fm_stream_probe_k<7>};
+#define FM_PROBE_FNS(AUX)                                                                                  \
+    fm_stream_probe_k<0, AUX>, fm_stream_probe_k<1, AUX>, fm_stream_probe_k<2, AUX>, fm_stream_probe_k<3, AUX>, \
+        fm_stream_probe_k<4, AUX>, fm_stream_probe_k<5, AUX>, fm_stream_probe_k<6, AUX>, fm_stream_probe_k<7, AUX>
+    static const probe_fn fns[16] = {FM_PROBE_FNS(FM_AUX_ONCE), FM_PROBE_FNS(FM_AUX_KEEP)};
+#undef FM_PROBE_FNS
     if (!fm_dyn_lds_ready(attr[pattern], (const void *)fns[pattern], sh)) return FM_ERR_HIP;
     const dim3 grid(n_cu), block(PROBE_WAVES * 64);
     const uint8_t *b = (const uint8_t *)d_buf;

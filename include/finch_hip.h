@@ -129,7 +129,9 @@ FM_API int fm_kernel_timing_read(fm_ctx *ctx, double *gate_up_ms, double *down_m
  * 16-byte loads into a ring) and no arithmetic; asynchronous on the context's stream.
  * pattern: 0 = slots dealt out over all waves of the chip (one dense window at any moment),
  * 1 = a contiguous share per workgroup, its waves interleaved (the decode kernels' order),
- * 2 = a contiguous share per wave.  Timed with fm_timer_start/stop it gives the rate the
+ * 2 = a contiguous share per wave (3..7: groups of workgroups in turn).  The loads carry the
+ * non-temporal hint the decode kernels use for weights that a launch reads once; pattern + 8 is
+ * the same walk with ordinary caching.  Timed with fm_timer_start/stop it gives the rate the
  * memory system delivers to a kernel of that structure.  No counterpart in the reference. */
 FM_API int fm_stream_probe_dev(fm_ctx *ctx, const void *d_buf, size_t nbytes, int pattern);
 
