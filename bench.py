@@ -32,10 +32,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 peak
 # --pmc FETCH_SIZE (x2: calibrated against a 1 GiB copy) + WRITE_SIZE.  An OFFLINE constant
 # (hardware counters cannot be read from inside this process): the JSON line names the file
 # it comes from in roofline.traffic_source, and it is null for any other size.
-FUSED_TRAFFIC_BYTES_40L = int((218685.2 * 2 + 2237.6) * 1024)
+FUSED_TRAFFIC_BYTES_40L = int((218576.5 * 2 + 2237.6) * 1024)
 FUSED_TRAFFIC_SOURCE = "offline constant from profiles/decode_step_3bit_hbm_traffic.md (rocprofv3 --pmc), not measured in this run"
 # the same for the one-launch GGUF step (fm_gguf_fused_rows at 40 x 256, top-8)
-GGUF_FUSED_TRAFFIC_BYTES_40L = int((322728.2 * 2 + 2148.6) * 1024)
+GGUF_FUSED_TRAFFIC_BYTES_40L = int((322526.7 * 2 + 2148.6) * 1024)
 GGUF_FUSED_TRAFFIC_SOURCE = "offline constant from profiles/gguf_step_and_gdn_kernel_trace.md (rocprofv3 --pmc), not measured in this run"
 
 H, I, E, K, L = 2048, 512, 256, 8, 40
@@ -918,7 +918,8 @@ def run_gguf(args):
     k1, k2, n = ctx.kernel_timing_read()
     ctx.kernel_timing(0)
     assert torch.isfinite(d_out).all()
-    phases = any(f in args.forms for f in ("gguf-phases", "plain-gguf"))
+    # (the library's own choice: one launch up to 32 layers, three streaming launches beyond)
+    phases = any(f in args.forms for f in ("gguf-phases", "plain-gguf")) or (n_layers > 32 and "gguf-one-launch" not in args.forms)
     res = {"kernels_us": {"fm_gguf_gate_up (as three launches)": round(k1 / n * 1e3, 2),
                           "fm_gguf_down+combine (as three launches)": round(k2 / n * 1e3, 2)},
            "event_ms_per_step": round(ev, 5), "us_per_layer": round(ms * 1e3 / n_layers, 3),
@@ -1149,7 +1150,7 @@ def main():
         from finchmoe_amd import binding as fb
         known = {"plain-dense": fb.FORM_PLAIN_DENSE, "plain-gguf": fb.FORM_PLAIN_GGUF,
                  "per-position": fb.FORM_NO_DENSE_GEMM | fb.FORM_NO_GGUF_GROUP, "three-launches": 0,
-                 "gguf-phases": fb.FORM_GGUF_PHASES}
+                 "gguf-phases": fb.FORM_GGUF_PHASES, "gguf-one-launch": fb.FORM_GGUF_ONE_LAUNCH}
         bad = [f for f in args.forms if f not in known]
         if bad:
             print("bench.py: unknown --forms %s (have: %s)" % (bad, ", ".join(known)), file=sys.stderr)

@@ -14,6 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 
 OK, ERR_ARG, ERR_HIP, ERR_STATE, ERR_UNSUPPORTED, ERR_NOMEM = 0, -1, -2, -3, -4, -5
 FORM_PLAIN_DENSE, FORM_PLAIN_GGUF, FORM_NO_DENSE_GEMM, FORM_NO_GGUF_GROUP, FORM_GGUF_PHASES = 1, 2, 4, 8, 16
+FORM_GGUF_ONE_LAUNCH = 32
 SCALE_BF16, SCALE_FP16 = 0, 1
 Q4_K, Q6_K = 12, 14
 ACCUMULATE, GUARD = 1, 2

@@ -338,7 +338,7 @@ unsigned int fm_kernel_forms = 0;
 
 extern "C" int fm_set_kernel_forms(unsigned int forms) {
     if (forms & ~(unsigned)(FM_FORM_PLAIN_DENSE | FM_FORM_PLAIN_GGUF | FM_FORM_NO_DENSE_GEMM | FM_FORM_NO_GGUF_GROUP |
-                           FM_FORM_GGUF_PHASES))
+                           FM_FORM_GGUF_PHASES | FM_FORM_GGUF_ONE_LAUNCH))
         return FM_ERR_ARG;
     fm_kernel_forms = forms;
     return FM_OK;

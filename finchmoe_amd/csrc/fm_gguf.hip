@@ -1503,7 +1503,12 @@ extern "C" int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t
     // (the activation sets alternate between launches exactly as for the affine experts; a
     // captured launch would need the graph's set and a fill kernel in front, and takes the three
     // kernels instead).
-    const bool phases = (fm_kernel_forms & (FM_FORM_PLAIN_GGUF | FM_FORM_GGUF_PHASES)) != 0;
+    // (With the non-temporal loads the three streaming launches are the faster form of a long step:
+    // 40 layers x 8 take 119.4 us as three and 121.3 us as one; up to 32 layers, for one layer and
+    // for the positions of a chunk the one launch wins, 98.0 / 56.3 / 16.9 against 98.5 / 58.4 /
+    // 19.7 us at 32 / 16 / 2 layers.)
+    const bool phases = (fm_kernel_forms & (FM_FORM_PLAIN_GGUF | FM_FORM_GGUF_PHASES)) != 0 ||
+                        (n_layers > 32 && !(fm_kernel_forms & FM_FORM_GGUF_ONE_LAUNCH));
     const unsigned int act_need = (unsigned int)n_pairs * (unsigned int)g->inter;
     if (!phases && !kev && df && (flags & FM_INT_NO_EXPERT_OUT) && !(flags & FM_GUARD) && df->act_set[0] &&
         df->act_cap >= act_need && !df->always_graph_set) {

@@ -282,13 +282,24 @@ def test_full_gguf_step_equals_layer_calls_and_oracle(orc):
         ctx.sync()
         out, eo = d_out.cpu().numpy(), d_eo.cpu().numpy()
         assert np.isfinite(out).all() and np.abs(out).max() > 0
-        # the same step without the per-expert vectors: one launch, the same bits, twice
-        for _ in range(2):
-            d_one = torch.zeros(L, H, device=dev)
-            torch.cuda.synchronize()
-            ctx.gguf_moe_decode_step_dev(0, L, d_x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, d_one.data_ptr())
-            ctx.sync()
-            assert np.array_equal(d_one.cpu().numpy().view(np.uint32), out.view(np.uint32))
+        # the same step without the per-expert vectors as one launch (the library's own choice for
+        # more than 32 layers is the three launches): the same bits, twice
+        from finchmoe_amd import binding as fb
+        try:
+            ctx.set_kernel_forms(fb.FORM_GGUF_ONE_LAUNCH)
+            for _ in range(2):
+                d_one = torch.zeros(L, H, device=dev)
+                torch.cuda.synchronize()
+                ctx.gguf_moe_decode_step_dev(0, L, d_x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, d_one.data_ptr())
+                ctx.sync()
+                assert np.array_equal(d_one.cpu().numpy().view(np.uint32), out.view(np.uint32))
+        finally:
+            ctx.set_kernel_forms(0)
+        d_dflt = torch.zeros(L, H, device=dev)
+        torch.cuda.synchronize()
+        ctx.gguf_moe_decode_step_dev(0, L, d_x.data_ptr(), d_idx.data_ptr(), d_w.data_ptr(), K, d_dflt.data_ptr())
+        ctx.sync()
+        assert np.array_equal(d_dflt.cpu().numpy().view(np.uint32), out.view(np.uint32))
         s_out, s_eo = torch.zeros(H, device=dev), torch.zeros(K, H, device=dev)
         for l in range(L):
             ctx.gguf_moe_decode_dev(l, d_x.data_ptr() + l * H * 4, d_idx.data_ptr() + l * K * 4,
