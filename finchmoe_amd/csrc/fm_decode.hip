@@ -34,8 +34,13 @@
 
 namespace {
 
-// waves per workgroup of the streaming kernels: one workgroup per CU, two waves per SIMD
-constexpr int FM_NW = 8;
+// Waves per workgroup of the streaming kernels: one workgroup per CU, three waves per SIMD (the
+// kernels need up to 160 vector registers, so three is the most), each with a ring of two
+// slices.  Measured on the 40-layer step with the non-temporal loads: 8 waves with rings of 4 /
+// 3 / 2 slices 86.3 / 86.3 / 84.7 us — the ring's depth buys nothing, the memory pipeline takes
+// fewer requests than the rings hold — and 12 waves with rings of 2, the same LDS, 82.5 us: a
+// third wave per SIMD covers part of what the multiply of the other two leaves uncovered.
+constexpr int FM_NW = 12;
 
 struct DecodeArgs {
     const uint8_t *const *layer_ptrs;   // [n_layers] device pointers to layer blobs
@@ -202,11 +207,15 @@ __global__ __launch_bounds__(256) void fm_combine(DecodeArgs a) {
 // the dependence between a load into LDS and the consumer's LDS read, so both
 // the wait and the read are explicit.
 // ======================================================================
-template <int BITS>
+// (the one-layer launch that takes the layer tail along keeps eight waves: it is bound by its
+// chain of round trips, not by the stream, and with the tail's registers held across the
+// experts it does not fit the 168 registers that twelve waves leave a lane)
+constexpr int FM_NW_TAIL = 8;
+template <int BITS, int NW = FM_NW>
 struct FmDma : FmSlot<BITS> {
     // the workgroup's rings must fit in 160 KB of LDS next to the activation image
-    static constexpr int RING = BITS == 3 ? 4 : 3;
-    static constexpr int WG_BYTES = FM_NW * RING * FmSlot<BITS>::BYTES;
+    static constexpr int RING = 2;
+    static constexpr int WG_BYTES = NW * RING * FmSlot<BITS>::BYTES;
 };
 
 // Dynamic LDS of the streaming kernels: ring [FM_NW][RING] slots, then the
@@ -735,9 +744,9 @@ struct Fm2Seg {
     int pad;
 };
 
-template <int BITS, int LPR>
+template <int BITS, int LPR, int NW = FM_NW>
 constexpr size_t fm2_lds_bytes() {
-    return FmDma<BITS>::WG_BYTES + 2 * sizeof(FmActLds<LPR>) + FM2_MAX_SEG * sizeof(Fm2Seg) +
+    return FmDma<BITS, NW>::WG_BYTES + 2 * sizeof(FmActLds<LPR>) + FM2_MAX_SEG * sizeof(Fm2Seg) +
            FM2_PART_BYTES;
 }
 
@@ -819,9 +828,9 @@ __device__ __forceinline__ void fm2_build_chunk(float xl, float xh, const FmBuil
 }
 
 
-template <int BITS, int LPR_UP, bool FP16>
+template <int BITS, int LPR_UP, bool FP16, int NW = FM_NW>
 struct Fm2Stream {
-    using D = FmDma<BITS>;
+    using D = FmDma<BITS, NW>;
     static constexpr int RING = D::RING;
     static constexpr int LPR_DN = LPR_UP / 4;
     static constexpr int RPS_UP = FM_WAVE / LPR_UP, RPS_DN = FM_WAVE / LPR_DN;
@@ -974,7 +983,7 @@ struct Fm2Stream {
         const int rows = (int)fm_div(by_K, n) * RPS_DN;
         const int l = seg_layer(q);
         float *out = a.out + (size_t)l * a.g.hidden + (size_t)fm_div(by_K, first) * RPS_DN;
-        for (int r = threadIdx.x; r < rows; r += FM_NW * 64) {
+        for (int r = threadIdx.x; r < rows; r += NW * 64) {
             const int rbi = r / RPS_DN, ris = r - rbi * RPS_DN;
             float acc = 0.0f;
 #pragma unroll
@@ -1168,7 +1177,7 @@ struct Fm2Stream {
                 float xl[LPR_DN], xh[LPR_DN];
 #pragma unroll
                 for (int i = 0; i < LPR_DN; i++) {       // all loads first, polls where needed after
-                    const int cmb = (threadIdx.x >> 6) + FM_NW * i;
+                    const int cmb = (threadIdx.x >> 6) + NW * i;
                     const int k = cmb / LPR_DN, chn = cmb - k * LPR_DN;
                     const float *src = a.act + ((size_t)l * K + (k < K ? k : 0)) * a.g.inter + chn * FM_CPL;
                     xl[i] = fm_ld_shared(src + bslot.lo);
@@ -1176,7 +1185,7 @@ struct Fm2Stream {
                 }
 #pragma unroll
                 for (int i = 0; i < LPR_DN; i++) {
-                    const int cmb = (threadIdx.x >> 6) + FM_NW * i;
+                    const int cmb = (threadIdx.x >> 6) + NW * i;
                     const int k = cmb / LPR_DN, chn = cmb - k * LPR_DN;
                     const bool on = k < K;
                     const float *src = a.act + ((size_t)l * K + (on ? k : 0)) * a.g.inter + chn * FM_CPL;
@@ -1267,7 +1276,7 @@ struct Fm2Stream {
             if (lane == 0) fm_st_shared(ta.partial + row0 / RPS_DN + wave, sq);
         }
         const int n_vw = ta.hidden / RPS_DN;
-        for (int v = threadIdx.x; v < n_vw; v += FM_NW * 64)
+        for (int v = threadIdx.x; v < n_vw; v += NW * 64)
             fm_lds_w32(part0 + tl.red + 4u * (uint32_t)v, __float_as_uint(act_get(ta.partial + v)));
         fm_wg_barrier();
         if (wave == 0) {
@@ -1308,9 +1317,9 @@ void fm_moe_fused_rows(DecodeArgs a, Fm2Dims dm, Fm2Sync sy) {
 
 // one layer's experts with the layer's tail behind them (Fm2Stream::run<true>)
 template <int BITS, int LPR_UP, bool FP16>
-__global__ __launch_bounds__(FM_NW * 64)
+__global__ __launch_bounds__(FM_NW_TAIL * 64)
 void fm_moe_fused_rows_tail(DecodeArgs a, Fm2Dims dm, Fm2Sync sy, FmTailArgs ta) {
-    Fm2Stream<BITS, LPR_UP, FP16> st(a, sy);
+    Fm2Stream<BITS, LPR_UP, FP16, FM_NW_TAIL> st(a, sy);
     st.template run<true>(dm, &ta);
 }
 
@@ -1345,8 +1354,7 @@ bool fm_dyn_lds_ok(FmKernelSetup &ks, const void *fn, size_t bytes) {
 // workgroups of a streaming launch: one per CU (LDS budget), fewer when there
 // are not enough units to give every wave `per_wave` of them
 dim3 fm_stream_grid(long units, int n_cu, int per_wave) {
-    static_assert(FM_NW == 8, "fm_stream_wgs counts eight waves per workgroup");
-    return dim3((unsigned)fm_stream_wgs(units, n_cu, per_wave));
+    return dim3((unsigned)fm_stream_wgs(units, n_cu, per_wave, FM_NW));
 }
 
 // One fused launch.  Returns FM_ERR_UNSUPPORTED when the grid cannot be made
@@ -1381,13 +1389,13 @@ template <int BITS, int LPR_UP, bool FP16>
 int launch_fused_rows_tail(const DecodeArgs &a, int n_pairs, int n_cu, hipStream_t st, const Fm2Sync &sy,
                            const FmTailArgs &ta) {
     auto kfn = fm_moe_fused_rows_tail<BITS, LPR_UP, FP16>;
-    const size_t sh = fm2_lds_bytes<BITS, LPR_UP>();
+    const size_t sh = fm2_lds_bytes<BITS, LPR_UP, FM_NW_TAIL>();
     static FmKernelSetup ks;
     if (!fm_dyn_lds_ok(ks, (const void *)kfn, sh)) return FM_ERR_HIP;
     const int dev = fm_current_device();
     int per_cu = dev >= 0 ? ks.per_cu[dev] : 0;
     if (per_cu == 0) {
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kfn, FM_NW * 64, sh) != hipSuccess)
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kfn, FM_NW_TAIL * 64, sh) != hipSuccess)
             per_cu = 0;
         if (per_cu < 1) per_cu = -1;
         if (dev >= 0) ks.per_cu[dev] = per_cu;
@@ -1405,7 +1413,7 @@ int launch_fused_rows_tail(const DecodeArgs &a, int n_pairs, int n_cu, hipStream
     const int nrb_max = (dn_rbs + plan.wgs - 1) / plan.wgs;
     if (!fm2_tail_lds(nrb_max, a.K, rps_dn, ta.inter, ta.hidden).ok) return FM_ERR_UNSUPPORTED;
     const Fm2Dims dm = fm2_dims(n_pairs, a.K, plan.wgs, a.g.inter, a.g.hidden, LPR_UP);
-    hipLaunchKernelGGL(kfn, dim3((unsigned)plan.wgs), dim3(FM_NW * 64), sh, st, a, dm, sy, ta);
+    hipLaunchKernelGGL(kfn, dim3((unsigned)plan.wgs), dim3(FM_NW_TAIL * 64), sh, st, a, dm, sy, ta);
     return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_HIP;
 }
 

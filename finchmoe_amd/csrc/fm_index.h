@@ -339,9 +339,9 @@ FM_HD void fm1_part(const Fm1Split &s, int q, int gu, uint32_t *first, uint32_t 
 }
 // workgroups of a streaming launch: one per CU, fewer when there are not enough units to give
 // every wave `per_wave` of them
-FM_HD long fm_stream_wgs(long units, int n_cu, int per_wave) {
+FM_HD long fm_stream_wgs(long units, int n_cu, int per_wave, int n_waves = 8) {
     long wgs = (long)n_cu;
-    const long need = 8L * per_wave;
+    const long need = (long)n_waves * per_wave;
     if (units < need * wgs) wgs = (units + need - 1) / need;
     if (wgs < 1) wgs = 1;
     return wgs;

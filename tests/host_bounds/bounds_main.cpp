@@ -376,11 +376,11 @@ static void walk_fused_rows(int n_groups, int K, int hidden, int inter, int bits
     const uint32_t gu_wstep = rps_up * (hidden * bits / 8), gu_sstep = rps_up * (hidden / 64) * 2;
     const uint32_t dn_wstep = rps_dn * (inter * bits / 8), dn_sstep = rps_dn * (inter / 64) * 2;
     // LDS: rings | two gate/up images | segment tables | partial vectors
-    const int ring = bits == 3 ? 4 : 3;
+    const int ring = 2, n_waves = 12;          // fm_decode.hip: FM_NW, FmDma::RING
     const size_t slot = 64 * (size_t)fm_lane_bytes(bits) + 512 + 16;
     const size_t img_up = (size_t)16 * 4 * lpr_up * 16 + lpr_up * 16, img_dn = (size_t)16 * 4 * lpr_dn * 16 + lpr_dn * 16;
     const size_t seg_bytes = 8 * 8 + 8 * 4 + 6 * 4;
-    const size_t lds = 8 * ring * slot + 2 * img_up + FM2_MAX_SEG * seg_bytes + FM2_PART_BYTES;
+    const size_t lds = (size_t)n_waves * ring * slot + 2 * img_up + FM2_MAX_SEG * seg_bytes + FM2_PART_BYTES;
     CHECK(lds <= 160 * 1024, "LDS %zu", lds);
     CHECK((size_t)FM_MAX_K * img_dn <= 2 * img_up, "down images in the gate/up images");
     std::vector<Region> blob;
@@ -547,7 +547,7 @@ static void walk_phases(int n_groups, int K, int hidden, int inter, int bits, bo
     Region act("act", (size_t)n_pairs * inter * 4, 4), eo("expert_out", (size_t)n_pairs * hidden * 4, 4);
     for (int phase = 0; phase < 2; phase++) {
         const bool up = phase == 0;
-        const long G = fused ? fm1_fused_wgs(gu_total, dn_total, N_CU) : fm_stream_wgs(up ? gu_total : dn_total, N_CU, 2);
+        const long G = fused ? fm1_fused_wgs(gu_total, dn_total, N_CU) : fm_stream_wgs(up ? gu_total : dn_total, N_CU, 2, 12);
         for (long b = 0; b < G; b++) {
             const Fm1Split sp = fm1_split(fused || up ? gu_total : 0, fused || !up ? dn_total : 0, gu_upp * K, dn_upp, (unsigned)b, (unsigned)G);
             const int q0 = up ? 0 : sp.n_up, q1 = up ? sp.n_up : sp.n_up + sp.n_dn;
