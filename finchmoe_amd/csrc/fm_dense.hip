@@ -166,33 +166,34 @@ __device__ __forceinline__ float fm_bf16_row(const uint16_t *w, const float *x, 
 // Streaming form (3-, 4- and 8-bit, in_dim up to 2048, or 4096 at 4 bits): the
 // structure of the expert kernels (fm_decode.hip) without segments.  All wave
 // steps ("units", 64/LPR rows) of all tensors of the launch form one sequence;
-// workgroup g (8 waves, one per CU) takes [U*g/G, U*(g+1)/G), its waves claim
+// workgroup g (12 waves, or 8 for the two forms that need the registers; one per CU) takes
+// [U*g/G, U*(g+1)/G), its waves claim
 // units from an LDS counter, copy their bytes into a per-wave ring in LDS with
-// LDS-direct loads (three or four units in flight, no destination registers)
+// LDS-direct loads (two units in flight per wave, no destination registers)
 // and multiply on the matrix cores against the activation registers, which the
 // workgroup builds once.  in_dim = 4096 is two slabs of 2048 columns: a unit is
 // two slices, each against its own activation registers, summed in slab order.
 // 8-bit (the vocabulary projection, finchmoe/infer.m:5728-5760): same ring, two
 // 8 KB units in flight per wave, multiply on the vector ALU.
 // ----------------------------------------------------------------------
-template <int BITS>
+template <int BITS, int NS>
 struct FmDenseRing {
-    static constexpr int RING = BITS == 3 ? 4 : (BITS == 8 ? 2 : 3);
-    static constexpr int BYTES = 8 * RING * FmSlot<BITS>::BYTES;
+    static constexpr int RING = FM_DENSE_RING, NW = FM_DENSE_NW(BITS, NS);
+    static constexpr int BYTES = NW * RING * FmSlot<BITS>::BYTES;
 };
 
 template <int BITS, int LPR, int NS>
 constexpr size_t fm_dense_stream_lds() {
-    return FmDenseRing<BITS>::BYTES + (BITS == 8 ? 0 : NS * sizeof(FmActLds<LPR>));
+    return FmDenseRing<BITS, NS>::BYTES + (BITS == 8 ? 0 : NS * sizeof(FmActLds<LPR>));
 }
 
 extern __shared__ __attribute__((aligned(16))) uint8_t fm_dense_lds[];
 
 template <int BITS, int LPR, int NS, bool FP16>
-__global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_units) {
+__global__ __launch_bounds__(FM_DENSE_NW(BITS, NS) * 64) void fm_dense_stream(FmDenseArgs a, int total_units) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using SL = FmSlot<BITS>;
-    constexpr int RPS = FM_WAVE / LPR, RING = FmDenseRing<BITS>::RING;
+    constexpr int RPS = FM_WAVE / LPR, RING = FmDenseRing<BITS, NS>::RING;
     constexpr int SLAB_COLS = FM_CPL * LPR;
     constexpr int SLAB_ROW_BYTES = LPR * FmLaneBytes<BITS>::value, SLAB_SB = 4 * LPR;
     static_assert(NS == 1 || (SLAB_ROW_BYTES == 1024 && RPS == SL::NQ), "one load per row and slab");
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int m = blockIdx.y;
     const uint32_t ring0 = fm_lds_addr(fm_dense_lds) + (uint32_t)wave * (RING * SL::BYTES);
-    FmActLds<LPR> *img = reinterpret_cast<FmActLds<LPR> *>(fm_dense_lds + FmDenseRing<BITS>::BYTES);
+    FmActLds<LPR> *img = reinterpret_cast<FmActLds<LPR> *>(fm_dense_lds + FmDenseRing<BITS, NS>::BYTES);
     const int row_bytes = NS * SLAB_ROW_BYTES, sb_row_bytes = NS * SLAB_SB;
     const FmRange wg = fm_share(total_units, blockIdx.x, gridDim.x);
     const long wg0 = wg.lo;
@@ -351,7 +352,7 @@ __global__ __launch_bounds__(512) void fm_dense_stream(FmDenseArgs a, int total_
     // set is one launch
     if (a.n_riders > 0) {
         int row = 0;
-        const int r = fm_dense_rider_of(a.rider_first, a.n_riders, (int)blockIdx.x * 8 + wave, &row);
+        const int r = fm_dense_rider_of(a.rider_first, a.n_riders, (int)blockIdx.x * FM_DENSE_NW(BITS, NS) + wave, &row);
         if (r >= 0) {
             const FmDenseSpec sp = r ? a.rider[1] : a.rider[0];
             const uint16_t *w = reinterpret_cast<const uint16_t *>(sp.W) + (size_t)row * a.in_dim;
@@ -382,7 +383,7 @@ int launch_dense_stream_t(FmDenseArgs &a, int M, int n_cu, hipStream_t st) {
     for (int i = 0; i <= FM_MAX_BATCH; i++) a.unit_first[i] = plan.unit_first[i];
     const int ns = plan.ns, lpr = plan.lpr, units = plan.units;
     const long wgs = plan.wgs;
-    if (a.n_riders > 0 && a.rider_first[a.n_riders] > 8 * wgs) a.n_riders = 0;   // one row per wave
+    if (a.n_riders > 0 && a.rider_first[a.n_riders] > plan.nw * wgs) a.n_riders = 0;   // one row per wave
     dim3 grid((unsigned)wgs, M);
 #define FM_DS(L, NS_)                                                                          \
     do {                                                                                       \
@@ -390,7 +391,7 @@ int launch_dense_stream_t(FmDenseArgs &a, int M, int n_cu, hipStream_t st) {
         const size_t sh = fm_dense_stream_lds<BITS, L, NS_>();                                 \
         static FmLdsAttr attr;                                                                 \
         if (!fm_dyn_lds_ready(attr, (const void *)kfn, sh)) return FM_ERR_HIP;                 \
-        hipLaunchKernelGGL(kfn, grid, dim3(512), sh, st, a, units);                            \
+        hipLaunchKernelGGL(kfn, grid, dim3(FM_DENSE_NW(BITS, NS_) * 64), sh, st, a, units);    \
     } while (0)
     if (ns == 2) {
         if constexpr (BITS == 4) FM_DS(16, 2);

@@ -511,7 +511,7 @@ struct GgImgLpr {
 
 template <int KIND, bool GU>
 struct GgRing {
-    static constexpr int value = KIND == GG_Q6W ? 2 : KIND == GG_Q6 ? 5 : 3;
+    static constexpr int value = FM_GG_RING;
 };
 
 // activation image of one input vector: register quad q of entry e = 4*chunk + piece,
@@ -752,7 +752,7 @@ template <> struct GgLaneOps<GG_Q6W> { using Lane = GgQ6WLane; using Data = GgQ6
 template <int KIND, int LPR, bool GU>
 constexpr size_t gg_stream_lds() {
     using G = GgLane<KIND, LPR>;
-    return (size_t)8 * GgRing<KIND, GU>::value * (G::SLOT_DATA + 16) +
+    return (size_t)FM_GG_NW(KIND == GG_Q6W) * GgRing<KIND, GU>::value * (G::SLOT_DATA + 16) +
            (GU ? 2 : 3) * sizeof(GgImage<G::NREG, GgImgLpr<KIND, LPR>::value>);
 }
 
@@ -786,7 +786,7 @@ struct GgUnit {
 // Units (wave steps) of the launch are numbered pair-major, by_upp divides by the units per pair,
 // by_k by K.
 template <int KIND, int LPR, bool GU>
-__global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_units, GgDiv by_upp,
+__global__ __launch_bounds__(FM_GG_NW(KIND == GG_Q6W) * 64) void fm_gguf_stream(GgufArgs a, int total_units, GgDiv by_upp,
                                                       GgDiv by_k) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using G = GgLane<KIND, LPR>;
@@ -806,7 +806,7 @@ __global__ __launch_bounds__(512) void fm_gguf_stream(GgufArgs a, int total_unit
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t ring0 = fm_lds_addr(fm_gguf_lds) + (uint32_t)wave * (RING * SLOT);
-    Image *img = reinterpret_cast<Image *>(fm_gguf_lds + 8 * RING * SLOT);
+    Image *img = reinterpret_cast<Image *>(fm_gguf_lds + FM_GG_NW(WIDE) * RING * SLOT);
     const uint32_t img0 = fm_lds_addr(img);
     const FmRange wg = fm_share(total_units, blockIdx.x, gridDim.x);
     const long wg0 = wg.lo, wg1 = wg.hi;
@@ -1448,7 +1448,7 @@ int gg_launch_stream(const GgufArgs &a, int n_pairs, int n_cu, hipStream_t st) {
         const size_t sh = gg_stream_lds<KK, L, GU>();                                          \
         static FmLdsAttr attr;                                                                 \
         if (!fm_dyn_lds_ready(attr, (const void *)kfn, sh)) return FM_ERR_HIP;                 \
-        hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(512), sh, st, a, (int)total,            \
+        hipLaunchKernelGGL(kfn, dim3((unsigned)wgs), dim3(FM_GG_NW(KK == GG_Q6W) * 64), sh, st, a, (int)total, \
                            gg_div_make((uint32_t)upp), gg_div_make((uint32_t)a.K));   \
     } while (0)
 #define GG_ST(L) GG_STK(KIND, L)

@@ -127,12 +127,19 @@ struct FmDensePlan {
     int lpr, ns, rps;   // lanes per row and slab, column slabs, rows per unit
     int units;          // wave steps of the launch
     int wgs;            // workgroups (grid.x)
+    int nw;             // waves per workgroup
     int unit_first[FM_IDX_MAX_BATCH + 1];
 };
+// waves of a streaming workgroup and slices per wave's ring (fm_dense_stream): three waves per
+// SIMD where the registers allow it (the 8-bit form and the two-slab form need more than a third
+// of a SIMD's file)
+#define FM_DENSE_NW(bits, ns) (((bits) == 8 || (ns) == 2) ? 8 : 12)
+#define FM_DENSE_RING 2
 FM_HD FmDensePlan fm_dense_stream_plan(const int *out_dims, int n, int in_dim, int bits, int n_cu) {
     FmDensePlan p;
     p.ok = 0;
     p.units = p.wgs = 0;
+    p.nw = 8;
     const int lpr_full = in_dim / FM_CPL;
     p.ns = lpr_full == 32 ? 2 : 1;
     p.lpr = lpr_full / p.ns;
@@ -151,7 +158,8 @@ FM_HD FmDensePlan fm_dense_stream_plan(const int *out_dims, int n, int in_dim, i
     // worth it only when every wave of the chip gets a unit
     if ((long)units < 8L * n_cu) return p;
     long wgs = n_cu;
-    if (units < 8 * wgs) wgs = (units + 7) / 8;
+    p.nw = FM_DENSE_NW(bits, p.ns);
+    if (units < p.nw * wgs) wgs = (units + p.nw - 1) / p.nw;
     p.wgs = (int)wgs;
     p.ok = 1;
     return p;
@@ -562,7 +570,13 @@ struct FmGgPlan {
     int n_img, n_pair;  // images / pair entries a workgroup keeps
     int wide;           // Q6_K rows of 2048 values: a lane owns two 64-value pieces, 1024 values apart
     int ring;           // slices per wave's ring
+    int nw;             // waves per workgroup
 };
+// waves of a streaming workgroup and slices per wave's ring (fm_gguf_stream): three waves per SIMD
+// with two slices in flight each read faster than two waves with rings of three to five; the
+// slices of the wide Q6_K rows (6720 B) leave room for two waves per SIMD
+#define FM_GG_NW(wide) ((wide) ? 8 : 12)
+#define FM_GG_RING 2
 // q6: Q6_K (a lane owns 64 values) else Q4_K (128); gu: gate and up rows of a unit
 FM_HD FmGgPlan fm_gg_plan(int n_pairs, int K, int in_dim, int rows, int q6, int gu, int n_cu) {
     FmGgPlan p;
@@ -570,12 +584,13 @@ FM_HD FmGgPlan fm_gg_plan(int n_pairs, int K, int in_dim, int rows, int q6, int 
     p.wgs = 0, p.total = 0;
     const int per_lane = q6 ? 64 : 128;
     p.wide = q6 && !gu && in_dim == 2048;
+    p.nw = FM_GG_NW(p.wide);
     p.lpr = p.wide ? 16 : in_dim / per_lane;
     p.rps = p.lpr > 0 ? FM_WAVE / p.lpr : 0;
     p.upp = p.rps > 0 ? rows / p.rps : 0;
     p.row_bytes = q6 ? (in_dim / 256) * 210 : (p.lpr / 2) * 144;
     p.slot_data = p.rps * p.row_bytes;
-    p.ring = p.wide ? 2 : q6 ? 5 : 3;
+    p.ring = FM_GG_RING;
     p.n_img = gu ? 2 : 3;
     p.n_pair = gu ? FM_MAX_K + 1 : 3;
     if (in_dim % per_lane || !(p.lpr == 4 || p.lpr == 8 || p.lpr == 16)) return p;
@@ -586,7 +601,7 @@ FM_HD FmGgPlan fm_gg_plan(int n_pairs, int K, int in_dim, int rows, int q6, int 
     // units within that span
     const long upv = gu ? (long)p.upp * K : p.upp, max_share = upv * (p.n_img - 1);
     long wgs = n_cu;
-    if (p.total < 8 * wgs) wgs = (p.total + 7) / 8;
+    if (p.total < p.nw * wgs) wgs = (p.total + p.nw - 1) / p.nw;
     if ((p.total + wgs - 1) / wgs > max_share) wgs = (p.total + max_share - 1) / max_share;
     while (wgs < p.total && (p.total + wgs - 1) / wgs > max_share) wgs++;
     p.wgs = (int)wgs;

@@ -144,15 +144,15 @@ static void walk_dense_batch(const char *name, const std::vector<DenseT> &ts, in
         const int lpr = plan.lpr, ns = plan.ns, rps = plan.rps;
         const int slab_row = lpr * fm_lane_bytes(bits), slab_sb = 4 * lpr;
         CHECK(ns == 1 || (slab_row == 1024 && rps == fm_lane_bytes(bits) / 16), "one load per row and slab");
-        const int ring = bits == 3 ? 4 : (bits == 8 ? 2 : 3);
+        const int ring = FM_DENSE_RING;
         const size_t slot_bytes = 64 * (size_t)fm_lane_bytes(bits) + 512 + 16;
-        const size_t lds = 8 * ring * slot_bytes + (bits == 8 ? 0 : (size_t)ns * (16 * 4 * lpr * 16 + lpr * 16));
+        const size_t lds = (size_t)plan.nw * ring * slot_bytes + (bits == 8 ? 0 : (size_t)ns * (16 * 4 * lpr * 16 + lpr * 16));
         CHECK(lds + 16 <= 160 * 1024, "LDS %zu", lds);
         int riders_first[3] = {0, 0, 0};
         int n_riders = (int)rider_rows.size();
         for (int i = 0; i < n_riders; i++) riders_first[i + 1] = riders_first[i] + rider_rows[i];
         for (int i = n_riders; i < 2; i++) riders_first[i + 1] = riders_first[n_riders];
-        if (n_riders > 0 && riders_first[n_riders] > 8 * plan.wgs) n_riders = 0;
+        if (n_riders > 0 && riders_first[n_riders] > plan.nw * plan.wgs) n_riders = 0;
         std::vector<Region> RW, RO;
         for (int i = 0; i < n_riders; i++) {
             RW.emplace_back("rider W", (size_t)rider_rows[i] * in_dim * 2, 2);
@@ -161,7 +161,7 @@ static void walk_dense_batch(const char *name, const std::vector<DenseT> &ts, in
         for (int m = 0; m < M; m++)
             for (int b = 0; b < plan.wgs; b++) {
                 const FmRange wg = fm_share(plan.units, b, plan.wgs);
-                CHECK(wg.hi - wg.lo >= 8 || plan.units < 8L * plan.wgs, "share of %ld units", wg.hi - wg.lo);
+                CHECK(wg.hi - wg.lo >= 8, "share of %ld units", wg.hi - wg.lo);
                 for (long u = wg.lo; u < wg.hi; u++) {
                     const int t = fm_dense_unit_tensor(plan.unit_first, n, u);
                     const int row0 = (int)(u - plan.unit_first[t]) * rps;
@@ -190,9 +190,9 @@ static void walk_dense_batch(const char *name, const std::vector<DenseT> &ts, in
                         if (ul.ch == 0) O[t].touch(((size_t)m * ts[t].out_dim + row0 + ul.row_in_step) * 4, 4, "out");
                     }
                 }
-                for (int wave = 0; wave < 8 && n_riders; wave++) {
+                for (int wave = 0; wave < plan.nw && n_riders; wave++) {
                     int row = 0;
-                    const int r = fm_dense_rider_of(riders_first, n_riders, b * 8 + wave, &row);
+                    const int r = fm_dense_rider_of(riders_first, n_riders, b * plan.nw + wave, &row);
                     if (r < 0) continue;
                     if (m == 0) RW[r].touch((size_t)row * in_dim * 2, (size_t)in_dim * 2, "rider row");
                     RO[r].touch(((size_t)m * rider_rows[r] + row) * 4, 4, "rider out");
@@ -600,7 +600,7 @@ static void walk_gguf_stream(int n_groups, int K, int hidden, int inter, bool gu
     const size_t slab = (size_t)rows * pl.row_bytes;       // one expert's rows of one matrix
     CHECK((size_t)pl.upp * pl.slot_data == slab, "slices tile the expert");
     const int ring = pl.ring, nreg = q6 ? 32 : 64, img_lpr = pl.wide ? 2 * pl.lpr : pl.lpr;
-    CHECK(ring == (pl.wide ? 2 : q6 ? 5 : 3), "ring of %d slices", ring);
+    CHECK(ring == FM_GG_RING, "ring of %d slices", ring);
     CHECK(pl.row_bytes == (q6 ? (in_dim / 256) * 210 : (in_dim / 256) * 144), "row of %d bytes", pl.row_bytes);
     const size_t img = (size_t)(nreg / 4) * 4 * img_lpr * 16 + img_lpr * 16;
     if (q6) {   // every column of the row is some lane's: chunk c (and c + 16 where a lane owns two), value v
@@ -624,7 +624,7 @@ static void walk_gguf_stream(int n_groups, int K, int hidden, int inter, bool gu
         }
         for (int c = 0; c < in_dim; c++) CHECK(seen[c] == 1, "column %d owned %d times", c, (int)seen[c]);
     }
-    const size_t lds = (size_t)8 * ring * (pl.slot_data + 16) + pl.n_img * img + pl.n_pair * 32 + 16;
+    const size_t lds = (size_t)pl.nw * ring * (pl.slot_data + 16) + pl.n_img * img + pl.n_pair * 32 + 16;
     CHECK(lds <= 160 * 1024, "LDS %zu", lds);
     std::vector<Region> m0, m1;
     for (int p = 0; p < n_pairs; p++) {
