@@ -32,10 +32,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 peak
 # --pmc FETCH_SIZE (x2: calibrated against a 1 GiB copy) + WRITE_SIZE.  An OFFLINE constant
 # (hardware counters cannot be read from inside this process): the JSON line names the file
 # it comes from in roofline.traffic_source, and it is null for any other size.
-FUSED_TRAFFIC_BYTES_40L = int((218576.5 * 2 + 2237.6) * 1024)
+FUSED_TRAFFIC_BYTES_40L = int((218752.1 * 2 + 2237.6) * 1024)
 FUSED_TRAFFIC_SOURCE = "offline constant from profiles/decode_step_3bit_hbm_traffic.md (rocprofv3 --pmc), not measured in this run"
 # the same for the one-launch GGUF step (fm_gguf_fused_rows at 40 x 256, top-8)
-GGUF_FUSED_TRAFFIC_BYTES_40L = int((322526.7 * 2 + 2148.6) * 1024)
+GGUF_FUSED_TRAFFIC_BYTES_40L = int((322575.7 * 2 + 2148.6) * 1024)
 GGUF_FUSED_TRAFFIC_SOURCE = "offline constant from profiles/gguf_step_and_gdn_kernel_trace.md (rocprofv3 --pmc), not measured in this run"
 
 H, I, E, K, L = 2048, 512, 256, 8, 40
