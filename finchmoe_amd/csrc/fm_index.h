@@ -80,6 +80,9 @@ FM_HD FmUnitLane fm_unit_lane(int lane, int lpr, int lane_bytes, int row_bytes, 
 // ---------------------------------------------------------------------------------------------
 // stream probe (fm_probe.hip): which 4 KB slots a wave reads
 // ---------------------------------------------------------------------------------------------
+// (waves per workgroup and slots per wave's ring: the decode kernels' twelve and two)
+#define FM_PROBE_WAVES 12
+#define FM_PROBE_RING 2
 struct FmProbeWalk {
     size_t next, end, step;
 };

@@ -11,8 +11,8 @@
 
 namespace {
 
-constexpr int PROBE_WAVES = 8;
-constexpr int PROBE_RING = 4;
+constexpr int PROBE_WAVES = FM_PROBE_WAVES;
+constexpr int PROBE_RING = FM_PROBE_RING;
 constexpr int PROBE_SLOT = 4096;       // 4 loads of 64 lanes x 16 bytes
 
 extern __shared__ __attribute__((aligned(16))) uint8_t fm_probe_lds[];

@@ -126,8 +126,8 @@ FM_API int fm_release_graphs(fm_ctx *ctx);
 FM_API int fm_kernel_timing_read(fm_ctx *ctx, double *gate_up_ms, double *down_ms, int *calls);
 
 /* Streaming probe: reads nbytes (whole 4 KB slots) of the device buffer d_buf once, with the
- * access structure of the expert kernels (one workgroup of eight waves per CU, LDS-direct
- * 16-byte loads into a ring) and no arithmetic; asynchronous on the context's stream.
+ * access structure of the expert kernels (one workgroup of twelve waves per CU, LDS-direct
+ * 16-byte loads into a ring of two slots per wave) and no arithmetic; asynchronous on the context's stream.
  * pattern: 0 = slots dealt out over all waves of the chip (one dense window at any moment),
  * 1 = a contiguous share per workgroup, its waves interleaved (the decode kernels' order),
  * 2 = a contiguous share per wave (3..7: groups of workgroups in turn).  The loads carry the

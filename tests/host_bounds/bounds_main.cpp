@@ -103,13 +103,14 @@ static void walk_probe(size_t nbytes, int pattern) {
     g_case = "stream_probe pattern " + std::to_string(pattern) + " bytes " + std::to_string(nbytes);
     const size_t n_slots = nbytes / 4096;
     Region buf("probe buffer", nbytes, 4096);
-    const int G = N_CU, ring = 4, slot = 4096;
+    const int G = N_CU, ring = FM_PROBE_RING, slot = 4096;
+    CHECK((size_t)FM_PROBE_WAVES * ring * slot <= 160 * 1024, "LDS");
     for (int b = 0; b < G; b++)
-        for (int wave = 0; wave < 8; wave++) {
-            FmProbeWalk w = fm_probe_walk(pattern, n_slots, b, G, wave, 8);
+        for (int wave = 0; wave < FM_PROBE_WAVES; wave++) {
+            FmProbeWalk w = fm_probe_walk(pattern, n_slots, b, G, wave, FM_PROBE_WAVES);
             for (size_t s = w.next; s < w.end; s += w.step) buf.touch(s * 4096, 4096, "slot");
             // ring in LDS: wave * ring * slot + wpos * slot + 1024 j + 16 lane + 16
-            CHECK((size_t)wave * ring * slot + (ring - 1) * slot + 3 * 1024 + 63 * 16 + 16 <= (size_t)8 * ring * slot, "ring");
+            CHECK((size_t)wave * ring * slot + (ring - 1) * slot + 3 * 1024 + 63 * 16 + 16 <= (size_t)FM_PROBE_WAVES * ring * slot, "ring");
         }
     buf.expect_once(0, n_slots * 4096);
     std::printf("ok  %-58s %zu slots\n", g_case.c_str(), n_slots);
