@@ -882,11 +882,16 @@ def run_gguf(args):
         # experts of a chunk; per-position products stream every routed expert once per position
         uniq = float(np.mean([len(set(idx[:M, l].reshape(-1).tolist())) for l in range(n_layers)]))
         rbytes = uniq * (2 * gsl + dsl) if grouped else M * K * (2 * gsl + dsl)
+        # (per-position products: the library takes the one launch up to 8 positions and the three
+        # streaming launches beyond)
+        one = not grouped and not any(f in args.forms for f in ("gguf-phases", "plain-gguf")) and \
+            (M <= 8 or "gguf-one-launch" in args.forms)
         cres = {"event_ms_per_step": round(ev, 5),
                 "roofline": _roofline_hbm("fm_gq_gate_up + fm_gq_down + fm_pf_combine (grouped products; bytes of the "
                                           "chunk's distinct experts)" if grouped else
+                                          "fm_gguf_fused_rows (one launch, one group per position)" if one else
                                           "fm_gguf_stream<Q4_K gate/up> + fm_gguf_stream<Q6_K down> + fm_gguf_combine "
-                                          "(one group per position)", rbytes, ev * 1e3, 4 if grouped else 3)}
+                                          "(one group per position)", rbytes, ev * 1e3, 4 if grouped else 1 if one else 3)}
         if grouped:
             flops = 2.0 * M * K * 3 * H * I
             cres["tflops"] = round(flops / (ev * 1e-3) / 1e12, 2)
@@ -918,8 +923,8 @@ def run_gguf(args):
     k1, k2, n = ctx.kernel_timing_read()
     ctx.kernel_timing(0)
     assert torch.isfinite(d_out).all()
-    # (the library's own choice: one launch up to 32 layers, three streaming launches beyond)
-    phases = any(f in args.forms for f in ("gguf-phases", "plain-gguf")) or (n_layers > 32 and "gguf-one-launch" not in args.forms)
+    # (the library's own choice: one launch up to 13 layers, three streaming launches beyond)
+    phases = any(f in args.forms for f in ("gguf-phases", "plain-gguf")) or (n_layers > 13 and "gguf-one-launch" not in args.forms)
     res = {"kernels_us": {"fm_gguf_gate_up (as three launches)": round(k1 / n * 1e3, 2),
                           "fm_gguf_down+combine (as three launches)": round(k2 / n * 1e3, 2)},
            "event_ms_per_step": round(ev, 5), "us_per_layer": round(ms * 1e3 / n_layers, 3),

@@ -1503,12 +1503,14 @@ extern "C" int fm_launch_decode_gguf(const uint8_t *const *d_gate, const uint8_t
     // (the activation sets alternate between launches exactly as for the affine experts; a
     // captured launch would need the graph's set and a fill kernel in front, and takes the three
     // kernels instead).
-    // (With the non-temporal loads the three streaming launches are the faster form of a long step:
-    // 40 layers x 8 take 119.4 us as three and 121.3 us as one; up to 32 layers, for one layer and
-    // for the positions of a chunk the one launch wins, 98.0 / 56.3 / 16.9 against 98.5 / 58.4 /
-    // 19.7 us at 32 / 16 / 2 layers.)
+    // (The three streaming launches, twelve waves per workgroup, are the faster form of a longer
+    // call: layers of a step 116.7 / 95.5 / 75.9 / 55.7 / 50.9 us as three against 121.3 / 97.4 /
+    // 77.9 / 55.8 / 51.2 us as one at 40 / 32 / 24 / 16 / 14 layers, and 46.1 / 35.5 / 19.0 against
+    // 45.7 / 34.9 / 15.7 us at 12 / 8 / 1; positions of a chunk 76.0 / 48.6 / 41.3 / 38.7 / 32.9
+    // against 84.0 / 51.5 / 43.1 / 39.6 / 33.2 us at 32 / 16 / 12 / 10 / 8.)
     const bool phases = (fm_kernel_forms & (FM_FORM_PLAIN_GGUF | FM_FORM_GGUF_PHASES)) != 0 ||
-                        (n_layers > 32 && !(fm_kernel_forms & FM_FORM_GGUF_ONE_LAUNCH));
+                        (n_layers > fm_gg_one_launch_max(layer_stride) &&
+                         !(fm_kernel_forms & FM_FORM_GGUF_ONE_LAUNCH));
     const unsigned int act_need = (unsigned int)n_pairs * (unsigned int)g->inter;
     if (!phases && !kev && df && (flags & FM_INT_NO_EXPERT_OUT) && !(flags & FM_GUARD) && df->act_set[0] &&
         df->act_cap >= act_need && !df->always_graph_set) {

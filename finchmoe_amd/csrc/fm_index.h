@@ -617,6 +617,9 @@ FM_HD FmGgPlan fm_gg_plan(int n_pairs, int K, int in_dim, int rows, int q6, int 
 // one row block of one expert (Q6_K or Q4_K), weighed by their bytes.  LDS: eight rings (three
 // gate/up slots or ring_dn down slots each, whichever is larger) | two gate/up images or K down
 // images | segment tables | partial vectors.
+// groups (layers of a step: layer_stride != 0; positions of a chunk: 0) up to which a call without
+// per-expert vectors takes the one launch; beyond, the three streaming launches are faster
+FM_HD int fm_gg_one_launch_max(int layer_stride) { return layer_stride != 0 ? 13 : 8; }
 #define FM_GG2_RING_UP 3
 #define FM_GG2_SEG_BYTES 192
 struct FmGg2Plan {

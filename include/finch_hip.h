@@ -109,7 +109,7 @@ FM_API int fm_set_wait_limit(fm_ctx *ctx, unsigned int polls);
 #define FM_FORM_NO_DENSE_GEMM 4u   /* fm_matvec_prefill*: one GEMV per position for every M */
 #define FM_FORM_NO_GGUF_GROUP 8u   /* fm_gguf_moe_prefill*: the per-position kernels for every M */
 #define FM_FORM_GGUF_PHASES 16u    /* fm_gguf_moe_decode*: gate/up, down and combine as three launches */
-#define FM_FORM_GGUF_ONE_LAUNCH 32u /* fm_gguf_moe_decode*: the one launch also for more than 32 groups */
+#define FM_FORM_GGUF_ONE_LAUNCH 32u /* fm_gguf_moe_decode*: the one launch also for more than 13 layers / 8 positions */
 FM_API int fm_set_kernel_forms(unsigned int forms);
 /* sums in milliseconds since the last read, and the number of calls; resets */
 /* Calls captured into a HIP graph (hipStreamBeginCapture on fm_stream()).  A graph records the

@@ -283,7 +283,7 @@ def test_full_gguf_step_equals_layer_calls_and_oracle(orc):
         out, eo = d_out.cpu().numpy(), d_eo.cpu().numpy()
         assert np.isfinite(out).all() and np.abs(out).max() > 0
         # the same step without the per-expert vectors as one launch (the library's own choice for
-        # more than 32 layers is the three launches): the same bits, twice
+        # more than 13 layers is the three launches): the same bits, twice
         from finchmoe_amd import binding as fb
         try:
             ctx.set_kernel_forms(fb.FORM_GGUF_ONE_LAUNCH)

@@ -196,9 +196,13 @@ def test_gguf_one_launch_equals_three(orc, h, i, down_t, layers, K):
             dx, di, dw = (torch.from_numpy(a).cuda() for a in (x, idx, w))
             d_one, d_three = torch.from_numpy(base).cuda(), torch.from_numpy(base).cuda()
             torch.cuda.synchronize()
-            ctx.gguf_moe_decode_step_dev(0, layers, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K, d_one.data_ptr(),
-                                         None, flags)
-            ctx.sync()
+            try:
+                ctx.set_kernel_forms(fb.FORM_GGUF_ONE_LAUNCH)
+                ctx.gguf_moe_decode_step_dev(0, layers, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K,
+                                             d_one.data_ptr(), None, flags)
+                ctx.sync()
+            finally:
+                ctx.set_kernel_forms(0)
             try:
                 ctx.set_kernel_forms(fb.FORM_GGUF_PHASES)
                 ctx.gguf_moe_decode_step_dev(0, layers, dx.data_ptr(), di.data_ptr(), dw.data_ptr(), K,
