@@ -1049,7 +1049,7 @@ def run_copy_probe(args):
 
 def run_stream_probe(args):
     """The streaming ceiling: 2 GiB read once per step by the library's probe kernel (one
-    workgroup of eight waves per CU, LDS-direct 16-byte loads into a ring, no arithmetic) —
+    workgroup of twelve waves per CU, LDS-direct 16-byte loads into rings of two slots, no arithmetic) —
     what the memory system delivers to a kernel built like the expert kernels.  The headline
     is the dense order (pattern 0); the other two orders are reported beside it."""
     import torch

@@ -446,7 +446,7 @@ __global__ __launch_bounds__(256) void fm_gguf_matvec_rows_k(const uint8_t *W, c
 
 // ---------------------------------------------------------------- streaming kernels
 // The large launches take the form of the affine decode kernels: one workgroup of
-// eight waves per CU, each wave keeps a ring of slices in LDS filled by LDS-direct
+// twelve waves per CU (FM_GG_NW), each wave keeps a ring of two slices in LDS filled by LDS-direct
 // loads (a slice = the rows of one wave step exactly as they lie in memory, block
 // headers included), units are claimed from a counter in LDS, and the multiply
 // runs on the matrix cores with the codes placed in bf16 mantissas (fm_mfma.h).

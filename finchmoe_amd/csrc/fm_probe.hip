@@ -1,5 +1,5 @@
 // fm_probe.hip — the streaming ceiling of the memory system, measured the way the expert
-// kernels read: one workgroup of eight waves per CU, every wave a ring of 4 KB slots in LDS
+// kernels read: one workgroup of twelve waves per CU, every wave a ring of two 4 KB slots in LDS
 // filled with LDS-direct 16-byte loads, no arithmetic; three orders in which the waves walk
 // the buffer (the rate depends on it).
 // What this kernel reaches is what a bandwidth-bound kernel of that structure can reach at
@@ -20,7 +20,7 @@ extern __shared__ __attribute__((aligned(16))) uint8_t fm_probe_lds[];
 // PATTERN: which 4 KB slots a wave reads, in order
 //   0  dense: slot i of the buffer goes to wave i % (all waves of the grid) — at any moment the
 //      chip reads one contiguous window
-//   1  every workgroup a contiguous share, its eight waves interleaved over it (the order of
+//   1  every workgroup a contiguous share, its waves interleaved over it (the order of
 //      the expert decode kernels)
 //   2  every wave a contiguous share
 //   3, 4, 5  groups of 4 / 8 / 8 workgroups share a contiguous region whose slots go to the
