@@ -1,7 +1,8 @@
 // fm_probe.hip — the streaming ceiling of the memory system, measured the way the expert
 // kernels read: one workgroup of twelve waves per CU, every wave a ring of two 4 KB slots in LDS
 // filled with LDS-direct 16-byte loads, no arithmetic; three orders in which the waves walk
-// the buffer (the rate depends on it).
+// the buffer (with two waves per SIMD the rate depended on the order by up to 5 %; with three
+// it hardly does).
 // What this kernel reaches is what a bandwidth-bound kernel of that structure can reach at
 // best; the decode kernels are priced against the published peak and compared with this.
 // No counterpart in the reference (a measurement aid, like its --timing accumulators,
