@@ -37,6 +37,8 @@ FUSED_TRAFFIC_SOURCE = "offline constant from profiles/decode_step_3bit_hbm_traf
 # the same for the one-launch GGUF step (fm_gguf_fused_rows at 40 x 256, top-8)
 GGUF_FUSED_TRAFFIC_BYTES_40L = int((322575.7 * 2 + 2148.6) * 1024)
 GGUF_FUSED_TRAFFIC_SOURCE = "offline constant from profiles/gguf_step_and_gdn_kernel_trace.md (rocprofv3 --pmc), not measured in this run"
+# and for the first of the step's three streaming launches (fm_gguf_stream<Q4_K, 16, gate/up> at 40 x 256, top-8)
+GGUF_GATE_UP_TRAFFIC_BYTES_40L = int((185566.3 * 2 + 645.4) * 1024)
 
 H, I, E, K, L = 2048, 512, 256, 8, 40
 
@@ -933,6 +935,9 @@ def run_gguf(args):
         # the dominant kernel: the Q4_K gate/up stream (its own events, isolated launches)
         res["roofline"] = _roofline_hbm("fm_gguf_stream<Q4_K,16,gate/up> (first of the step's three launches)",
                                         n_layers * K * 2 * gsl, k1 / n * 1e3)
+        if (n_layers, E, K) == (40, 256, 8):
+            res["roofline"]["traffic"] = GGUF_GATE_UP_TRAFFIC_BYTES_40L
+            res["roofline"]["traffic_source"] = GGUF_FUSED_TRAFFIC_SOURCE
     else:
         # the step is one launch: HIP events around the timed region on the library's stream
         res["roofline"] = _roofline_hbm("fm_gguf_fused_rows<Q6_K,16,8> (the step's one launch)",
