@@ -88,6 +88,16 @@ def test_gguf_step_and_small_chunk(hip, orc, gstore):
     for m in range(8):
         single, _ = hip.gguf_moe_decode(2, x[0] * np.float32(m + 1), idx[0], w[0])
         assert np.array_equal(chunk[m], single)
+    # 20 positions with their own routing (beyond 8 positions the per-position products are the three
+    # streaming launches, up to 8 the one launch): still the per-position calls, bit for bit
+    M = 20
+    X = rng.standard_normal((M, H)).astype(np.float32)
+    cidx = np.stack([orc.route(rng.standard_normal(E).astype(np.float32), K)[0] for _ in range(M)])
+    cw = np.stack([orc.normalize_weights(rng.random(K).astype(np.float32)) for _ in range(M)])
+    chunk = hip.gguf_moe_prefill(1, X, cidx, cw)
+    for m in range(M):
+        single, _ = hip.gguf_moe_decode(1, X[m], cidx[m], cw[m])
+        assert np.array_equal(chunk[m], single), m
 
 
 @pytest.mark.parametrize("gtype,out_dim,in_dim", [(12, 64, 2048), (14, 96, 512), (14, 7, 1024),
