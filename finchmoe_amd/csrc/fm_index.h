@@ -122,6 +122,35 @@ FM_HD FmProbeWalk fm_probe_walk(int pattern, size_t n_slots, unsigned int b, uns
 }
 
 // ---------------------------------------------------------------------------------------------
+// row-tile products of a chunk (fm_pf_rows): a task = 32 weight rows of an item (gate/up: 16
+// gate rows and the same 16 rows of up; down: 32 rows) over the whole K dimension, a slab = 256
+// columns of them = one slot of a wave's ring, a round = eight consecutive tasks of an item
+// ---------------------------------------------------------------------------------------------
+// code bytes of a row inside a slab
+FM_HD int fm_pfr_slab_row_bytes(int bits) { return 8 * bits * 4; }
+// the rounds [lo, hi) of workgroup b out of RT (neighbouring shares behind one L2)
+FM_HD FmRange fm_pfr_rounds(long RT, unsigned int b, unsigned int G) { return fm_share(RT, fm_xcd_share(b, G), G); }
+// one workgroup per CU, more when a share could span more than the 64 items whose experts a
+// workgroup keeps one per lane
+FM_HD int fm_pfr_grid(int max_items, int n_cu) {
+    const int need = (max_items + 31) / 32;
+    return need > n_cu ? need : n_cu;
+}
+// 16-byte piece q (= 64 j + lane, the slot keeps the rows back to back) of a slot copy: its offset
+// in the expert's blob from (the task's first row, the slab's first byte).  first_w / second_w:
+// offsets of the gate and up (or down, unused) code matrices in the blob
+FM_HD uint32_t fm_pfr_piece_off(int gu, int bits, int q, uint32_t first_w, uint32_t second_w, int row_bytes) {
+    const int rp = fm_pfr_slab_row_bytes(bits) / 16, rr = q / rp, pc = q - rr * rp;
+    const uint32_t mat = gu ? (rr < 16 ? first_w : second_w) : first_w;
+    return mat + (uint32_t)((gu ? (rr & 15) : rr) * row_bytes + 16 * pc);
+}
+// scales (biases) fetched with the slot, 8 bytes per row and slab: the dword of lane `lane`
+FM_HD uint32_t fm_pfr_sb_off(int gu, int lane, uint32_t first, uint32_t second, int sb_bytes) {
+    const int rr = lane >> 1;
+    return (gu ? (rr < 16 ? first : second) : first) + (uint32_t)((gu ? (rr & 15) : rr) * sb_bytes + 4 * (lane & 1));
+}
+
+// ---------------------------------------------------------------------------------------------
 // dense GEMV, streaming form (fm_dense_stream): all wave steps of all tensors of a launch form
 // one sequence; unit_first[i] = first unit of tensor i (unit_first[n..] = total)
 // ---------------------------------------------------------------------------------------------

@@ -896,9 +896,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // turn and every XCD has an L2 of its own: workgroup b takes share (b % 8) * (grid / 8) +
     // b / 8, so that neighbouring shares — the rounds of one expert — run behind one L2.
     const long RT = (long)n_items * RPI;
-    const unsigned int share = gridDim.x % 8u == 0u ? (blockIdx.x % 8u) * (gridDim.x / 8u) + blockIdx.x / 8u
-                                                    : blockIdx.x;
-    const int R0 = (int)(RT * share / gridDim.x), R1 = (int)(RT * (share + 1) / gridDim.x);
+    const FmRange rounds = fm_pfr_rounds(RT, blockIdx.x, gridDim.x);
+    const int R0 = (int)rounds.lo, R1 = (int)rounds.hi;
     if (R0 >= R1) return;
     const int it0 = R0 / RPI;
     // the items the share touches, one per lane (the launcher sizes the grid so that a share
@@ -926,19 +925,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // rows back to back).  gate/up: slot rows 0-15 = gate rows, 16-31 = the same rows of up
     uint32_t coff[P::NQ];
 #pragma unroll
-    for (int j = 0; j < P::NQ; j++) {
-        const int q = 64 * j + lane, rr = q / P::RP, pc = q - rr * P::RP;
-        const uint32_t mat = GU ? (rr < 16 ? a.g.gate_w : a.g.up_w) : a.g.down_w;
-        coff[j] = mat + (uint32_t)((GU ? (rr & 15) : rr) * row_bytes + 16 * pc);
-    }
+    for (int j = 0; j < P::NQ; j++)
+        coff[j] = fm_pfr_piece_off(GU, BITS, 64 * j + lane, GU ? a.g.gate_w : a.g.down_w, a.g.up_w, row_bytes);
     // scales / biases fetched with the slot (down): 8 bytes per row and slab, one dword per lane
-    uint32_t soff, boff;
-    {
-        const int rr = lane >> 1;
-        const uint32_t r = (uint32_t)((GU ? (rr & 15) : rr) * sb_bytes + 4 * (lane & 1));
-        soff = (GU ? (rr < 16 ? a.g.gate_s : a.g.up_s) : a.g.down_s) + r;
-        boff = (GU ? (rr < 16 ? a.g.gate_b : a.g.up_b) : a.g.down_b) + r;
-    }
+    const uint32_t soff = fm_pfr_sb_off(GU, lane, GU ? a.g.gate_s : a.g.down_s, a.g.up_s, sb_bytes);
+    const uint32_t boff = fm_pfr_sb_off(GU, lane, GU ? a.g.gate_b : a.g.down_b, a.g.up_b, sb_bytes);
 
     // ---- loader: the slabs of this wave's tasks, in order
     int l_r = R0, l_s = 0, wpos = 0;
@@ -1419,20 +1410,13 @@ bool pf_supported(const FmExpertGeom *g) {
            g->inter == 512;
 }
 
-// grid of a row-tile launch: one workgroup per CU, more when a share could span more than the
-// 64 items whose experts a workgroup keeps one per lane
-int pfr_grid(int max_items, int n_cu) {
-    const int need = (max_items + 31) / 32;
-    return need > n_cu ? need : n_cu;
-}
-
 template <int BITS, bool FP16>
 int pf_launch(const PfArgs &a, const FmExpertGeom *g, int M, float *d_out, int flags, int n_cu,
               hipStream_t st) {
     const size_t n = (size_t)M * a.K;
     hipLaunchKernelGGL(fm_pf_group, dim3(1), dim3(1024), 0, st, a);
-    const int grid_up = pfr_grid(g->n_experts + (int)(n / a.tm_up), n_cu);
-    const int grid_dn = pfr_grid(g->n_experts + (int)(n / a.tm_dn), n_cu);
+    const int grid_up = fm_pfr_grid(g->n_experts + (int)(n / a.tm_up), n_cu);
+    const int grid_dn = fm_pfr_grid(g->n_experts + (int)(n / a.tm_dn), n_cu);
 #define PFR_LAUNCH(MODE, XB, GRID)                                                               \
     do {                                                                                         \
         auto kfn = fm_pf_rows<MODE, BITS, FP16, XB>;                                             \

@@ -13,8 +13,10 @@
 // What is NOT shared with the kernels and therefore restated here: the order in which a
 // workgroup's waves claim units (irrelevant for bounds: every unit of a share is claimed exactly
 // once, by fm_claim_unit's counter), the LDS-direct load helpers' fixed per-lane pattern
-// (lane * 16 + 1024 * j for codes, lane * 4 for scales and biases: fm_ring.h), and the activation
-// staging patterns (fm_mfma.h), which index inside one input vector.
+// (lane * 16 + 1024 * j for codes, lane * 4 for scales and biases: fm_ring.h), the activation
+// staging patterns (fm_mfma.h), which index inside one input vector, and — for the chunk's
+// row-tile kernels — fm_pf_group's counting sort and item cut, and which (group, position) a thread
+// stages.
 #include "../../finchmoe_amd/csrc/fm_index.h"
 
 #include <cstdio>
@@ -357,6 +359,135 @@ static Geom geom(int hidden, int inter, int bits) {
     g.down_w = o; o += d_w;  g.down_s = o; o += d_s;  g.down_b = o; o += d_s;
     g.expert_size = o;
     return g;
+}
+
+// fm_pf_group + fm_pf_rows (the grouped products of a chunk, config 3): M positions x K slots on E
+// experts, routing skewed like the benchmark's.  The items and the sorted pair list are built by
+// fm_pf_group's rule (restated: a counting sort); the workgroups' rounds, the per-lane pieces of a
+// slot copy and the scale / bias offsets come from fm_index.h, as in the kernel.  Checked: the shares
+// tile the rounds, a share's items fit its lane table, every item reads its expert's matrices
+// exactly once, every load stays inside the blob / X / act / sorted list, every output element is
+// written exactly once, the LDS of both kernels fits.
+static void walk_pf_rows(int M, int K, int E, int bits, bool x_bf16, unsigned seed) {
+    g_case = "chunk rows " + std::to_string(M) + " positions x " + std::to_string(K) + " on " + std::to_string(E) +
+             " experts, " + std::to_string(bits) + "-bit, " + (x_bf16 ? "bf16" : "fp32") + " positions";
+    const int hidden = 2048, inter = 512, n = M * K;
+    const Geom g = geom(hidden, inter, bits);
+    // routing: K distinct experts per position, low indices preferred
+    std::vector<int> idx((size_t)n);
+    uint64_t st = 0x9E3779B97F4A7C15ull * (seed + 1);
+    auto rnd = [&]() { st = st * 6364136223846793005ull + 1442695040888963407ull; return (double)(st >> 11) / 9007199254740992.0; };
+    for (int m = 0; m < M; m++)
+        for (int k = 0; k < K; k++) {
+            for (;;) {
+                const double u = rnd();
+                const int e = (int)(E * u * u * u);
+                bool dup = false;
+                for (int j = 0; j < k; j++) dup = dup || idx[(size_t)m * K + j] == e;
+                if (!dup && e < E) { idx[(size_t)m * K + k] = e; break; }
+            }
+        }
+    std::vector<int> cnt(E, 0), off(E + 1, 0);
+    for (int p = 0; p < n; p++) cnt[idx[p]]++;
+    for (int e = 0; e < E; e++) off[e + 1] = off[e] + cnt[e];
+    std::vector<int> sorted((size_t)n), cur(off.begin(), off.end() - 1);
+    for (int p = 0; p < n; p++) sorted[cur[idx[p]]++] = p;
+    struct Item { int expert, start, count; };
+    for (int mode = 0; mode < 2; mode++) {
+        const bool gu = mode == 0;
+        const int tm = gu ? (x_bf16 ? 16 : 8) : 16;
+        std::vector<Item> items;
+        for (int e = 0; e < E; e++)
+            for (int s0 = 0; s0 < cnt[e]; s0 += tm) items.push_back({e, off[e] + s0, cnt[e] - s0 < tm ? cnt[e] - s0 : tm});
+        const int n_items = (int)items.size();
+        CHECK(n_items <= E + n / tm + 1, "%d items in a list of %d", n_items, E + n / tm + 1);
+        const int in_dim = gu ? hidden : inter, out_rows = gu ? inter : hidden;
+        const int row_bytes = in_dim * bits / 8, sb_bytes = (in_dim / 64) * 2;
+        const int S = in_dim / 256, CB = fm_pfr_slab_row_bytes(bits), NQ = 32 * (CB / 16) / 64;
+        const int RPI = out_rows / (gu ? 16 : 32) / 8, TPI = RPI * 8;
+        CHECK(S * CB == row_bytes, "slabs of %d bytes in a row of %d", CB, row_bytes);
+        CHECK(NQ * 1024 == 32 * CB, "a slot copy is whole load instructions");
+        // LDS: rings | image | bias / offset operands (PfRows)
+        const int QK = gu ? 1 : 2, slot = 32 * CB + (gu ? 0 : 512), img = S * 4 * 2 * QK * 1024, side = S * 1024;
+        int ring = (160 * 1024 - 2048 - img - side) / (8 * slot);
+        if (ring > 4) ring = 4;
+        CHECK(ring >= 2 && 8 * ring * slot + img + side + 2048 <= 160 * 1024, "LDS: ring of %d", ring);
+        for (int j = 0; j < NQ; j++) CHECK(1024 * j + 63 * 16 + 16 <= 32 * CB, "codes of a slot");
+        const long RT = (long)n_items * RPI;
+        const int G = fm_pfr_grid(E + n / tm, N_CU);
+        std::vector<uint8_t> round_owner((size_t)RT, 0);
+        Region X("X", (size_t)M * hidden * (x_bf16 ? 2 : 4)), act("act", (size_t)n * inter * 4, 4);
+        Region eo("expert_out", (size_t)n * hidden * 4, 4), srt("sorted", (size_t)n * 4);
+        for (int b = 0; b < G; b++) {
+            const FmRange rr = fm_pfr_rounds(RT, (unsigned)b, (unsigned)G);
+            CHECK(rr.lo >= 0 && rr.hi <= RT && rr.lo <= rr.hi, "rounds [%ld, %ld) of %ld", rr.lo, rr.hi, RT);
+            if (rr.lo >= rr.hi) continue;
+            for (long r = rr.lo; r < rr.hi; r++) round_owner[(size_t)r]++;
+            const int it0 = (int)(rr.lo / RPI), it_last = (int)((rr.hi - 1) / RPI);
+            CHECK(it_last - it0 < 64 && it_last < n_items, "workgroup %d: items %d..%d of %d", b, it0, it_last, n_items);
+            // staging of every item of the share: its pair ids, then 64 activations per (group, position)
+            for (int it = it0; it <= it_last && it < n_items; it++) {
+                const Item &I = items[it];
+                for (int pos = 0; pos < I.count; pos++) {
+                    srt.touch((size_t)(I.start + pos) * 4, 4, "pair id");
+                    if (I.start + pos >= n) continue;
+                    const int pair = sorted[I.start + pos];
+                    for (int sg = 0; sg < S * 4; sg++) {
+                        if (gu) X.touch(((size_t)(pair / K) * hidden + 64 * (size_t)sg) * (x_bf16 ? 2 : 4), 64 * (x_bf16 ? 2 : 4), "X row");
+                        else act.touch(((size_t)(I.start + pos) * inter + 64 * (size_t)sg) * 4, 256, "act row");
+                    }
+                }
+            }
+        }
+        size_t bad = 0;
+        for (long r = 0; r < RT; r++) bad += round_owner[(size_t)r] != 1;
+        CHECK(bad == 0, "%zu of %ld rounds not owned by exactly one workgroup", bad, RT);
+        // every item: its tasks' loads tile the expert's matrices; outputs once
+        if (!gu) act = Region("act", (size_t)n * inter * 4);      // (read above; the output of the other mode)
+        Region out = gu ? Region("act", (size_t)n * inter * 4, 4) : Region("expert_out", (size_t)n * hidden * 4, 4);
+        for (int it = 0; it < n_items; it++) {
+            const Item &I = items[it];
+            CHECK(I.expert >= 0 && I.expert < E && I.count >= 1 && I.count <= tm && I.start + I.count <= n, "item %d", it);
+            Region blob("expert blob", g.expert_size, 4);
+            for (int t = 0; t < TPI; t++) {
+                const size_t r0 = (size_t)t * (gu ? 16 : 32);
+                for (int s0 = 0; s0 < S; s0++) {
+                    for (int q = 0; q < 64 * NQ; q++)
+                        blob.touch(r0 * row_bytes + (size_t)s0 * CB +
+                                       fm_pfr_piece_off(gu, bits, q, (uint32_t)(gu ? g.gate_w : g.down_w), (uint32_t)g.up_w, row_bytes),
+                                   16, "codes");
+                    if (!gu)
+                        for (int lane = 0; lane < 64; lane++) {
+                            blob.touch(r0 * sb_bytes + (size_t)s0 * 8 + fm_pfr_sb_off(0, lane, (uint32_t)g.down_s, 0u, sb_bytes), 4, "scales");
+                            blob.touch(r0 * sb_bytes + (size_t)s0 * 8 + fm_pfr_sb_off(0, lane, (uint32_t)g.down_b, 0u, sb_bytes), 4, "biases");
+                        }
+                }
+                if (gu)          // a task's scales and biases: four contiguous KB, 16 bytes per lane
+                    for (int lane = 0; lane < 64; lane++) {
+                        const size_t sc_lane = (size_t)(lane & 15) * sb_bytes + 16 * (size_t)(lane >> 4);
+                        for (size_t m0 : {g.gate_s, g.gate_b, g.up_s, g.up_b}) blob.touch(r0 * sb_bytes + m0 + sc_lane, 16, "scales of a task");
+                    }
+                for (int tok = 0; tok < I.count; tok++)
+                    for (int nn = 0; nn < 16; nn++) {
+                        if (gu) out.touch(((size_t)(I.start + tok) * inter + r0 + nn) * 4, 4, "act");
+                        else {
+                            const size_t pair = (size_t)sorted[I.start + tok];
+                            out.touch((pair * hidden + r0 + nn) * 4, 4, "expert_out");
+                            out.touch((pair * hidden + r0 + nn + 16) * 4, 4, "expert_out");
+                        }
+                    }
+            }
+            if (gu) {
+                blob.expect_once(g.gate_w, g.up_w + (g.up_s - g.up_w) + 2 * (g.up_b - g.up_s));      // gate and up: codes, scales, biases
+                blob.expect_untouched(g.down_w, g.expert_size);
+            } else {
+                blob.expect_once(g.down_w, g.expert_size);
+                blob.expect_untouched(0, g.down_w);
+            }
+        }
+        out.expect_once(0, out.size);
+        std::printf("ok  %-58s %s: %d items, %ld rounds over %d workgroups\n", g_case.c_str(), gu ? "gate/up" : "down", n_items, RT, G);
+    }
 }
 
 // fm_moe_fused_rows: n_groups layer groups (layers of a step / positions of a chunk) x K slots.
@@ -844,6 +975,14 @@ int main() {
     }
     walk_pf_dense(2048, 2048, 3, 512);
     walk_pf_dense(512, 512, 3, 64);
+    // ---- config 3: chunks of 32 positions and more on 256 experts (bench.py --workload prefill, the tests)
+    walk_pf_rows(512, 8, 256, 3, true, 1);
+    walk_pf_rows(512, 8, 256, 3, false, 2);
+    walk_pf_rows(512, 8, 256, 4, true, 3);
+    walk_pf_rows(2048, 8, 256, 3, true, 4);
+    walk_pf_rows(32, 8, 256, 3, true, 5);
+    walk_pf_rows(200, 5, 12, 4, false, 6);
+    walk_pf_rows(65535, 1, 3, 3, true, 7);
     // ---- routed experts: the decode step (config 2, and its 4-bit form), one layer per call
     // (config 0), chunks below 32 positions (config 3 at chunk 8)
     for (int bits : {3, 4}) {

@@ -43,7 +43,10 @@ def test_every_access_of_the_benchmark_launches_is_inside_its_buffer(walker):
                  "gguf stream down Q6_K 40 groups x 8", "gguf stream down Q6_K 8 groups x 8",
                  "fused rows, sweep of shapes", "fused rows + tail, LDS tables",
                  "gguf fused rows Q6_K down, 40 groups x 8, 2048x512", "gguf fused rows Q6_K down, 1 groups x 8, 2048x512",
-                 "gguf fused rows Q4_K down, 3 groups x 8, 1024x512"):
+                 "gguf fused rows Q4_K down, 3 groups x 8, 1024x512",
+                 "chunk rows 512 positions x 8 on 256 experts, 3-bit, bf16 positions",
+                 "chunk rows 512 positions x 8 on 256 experts, 4-bit, bf16 positions",
+                 "chunk rows 2048 positions x 8 on 256 experts, 3-bit, bf16 positions"):
         assert ("ok  " + case) in r.stdout or ("ok  dense " + case) in r.stdout, case
 
 
