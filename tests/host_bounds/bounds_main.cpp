@@ -982,7 +982,7 @@ int main() {
     walk_pf_rows(2048, 8, 256, 3, true, 4);
     walk_pf_rows(32, 8, 256, 3, true, 5);
     walk_pf_rows(200, 5, 12, 4, false, 6);
-    walk_pf_rows(65535, 1, 3, 3, true, 7);
+    walk_pf_rows(8192, 1, 3, 3, true, 7);
     // ---- routed experts: the decode step (config 2, and its 4-bit form), one layer per call
     // (config 0), chunks below 32 positions (config 3 at chunk 8)
     for (int bits : {3, 4}) {
