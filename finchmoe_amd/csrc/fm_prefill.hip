@@ -1541,10 +1541,9 @@ struct GqShare {
     int u0, u1;
 };
 __device__ __forceinline__ GqShare gq_share(int n_items, int per_item) {
-    const long total = (long)n_items * per_item;
+    const FmRange r = fm_share((long)n_items * per_item, blockIdx.x, gridDim.x);
     GqShare s;
-    s.u0 = (int)(total * blockIdx.x / gridDim.x);
-    s.u1 = (int)(total * (blockIdx.x + 1) / gridDim.x);
+    s.u0 = (int)r.lo, s.u1 = (int)r.hi;
     return s;
 }
 

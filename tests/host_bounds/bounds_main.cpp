@@ -361,6 +361,45 @@ static Geom geom(int hidden, int inter, int bits) {
     return g;
 }
 
+struct ChunkItem { int expert, start, count; };
+struct ChunkLists {
+    int n;
+    std::vector<int> idx, cnt, off, sorted;
+    // fm_pf_group: every expert's positions cut into items of at most tm
+    std::vector<ChunkItem> items(int tm) const {
+        std::vector<ChunkItem> v;
+        for (int e = 0; e < (int)cnt.size(); e++)
+            for (int s0 = 0; s0 < cnt[e]; s0 += tm) v.push_back({e, off[e] + s0, cnt[e] - s0 < tm ? cnt[e] - s0 : tm});
+        return v;
+    }
+};
+// routing of a chunk (K distinct experts per position, low indices preferred) and its counting sort
+static ChunkLists chunk_lists(int M, int K, int E, unsigned seed) {
+    ChunkLists c;
+    const int n = M * K;
+    c.n = n;
+    c.idx.assign((size_t)n, 0);
+    uint64_t st = 0x9E3779B97F4A7C15ull * (seed + 1);
+    auto rnd = [&]() { st = st * 6364136223846793005ull + 1442695040888963407ull; return (double)(st >> 11) / 9007199254740992.0; };
+    for (int m = 0; m < M; m++)
+        for (int k = 0; k < K; k++) {
+            for (;;) {
+                const double u = rnd();
+                const int e = (int)(E * u * u * u);
+                bool dup = false;
+                for (int j = 0; j < k; j++) dup = dup || c.idx[(size_t)m * K + j] == e;
+                if (!dup && e < E) { c.idx[(size_t)m * K + k] = e; break; }
+            }
+        }
+    c.cnt.assign(E, 0), c.off.assign(E + 1, 0);
+    for (int p = 0; p < n; p++) c.cnt[c.idx[p]]++;
+    for (int e = 0; e < E; e++) c.off[e + 1] = c.off[e] + c.cnt[e];
+    c.sorted.assign((size_t)n, 0);
+    std::vector<int> cur(c.off.begin(), c.off.end() - 1);
+    for (int p = 0; p < n; p++) c.sorted[cur[c.idx[p]]++] = p;
+    return c;
+}
+
 // fm_pf_group + fm_pf_rows (the grouped products of a chunk, config 3): M positions x K slots on E
 // experts, routing skewed like the benchmark's.  The items and the sorted pair list are built by
 // fm_pf_group's rule (restated: a counting sort); the workgroups' rounds, the per-lane pieces of a
@@ -373,32 +412,13 @@ static void walk_pf_rows(int M, int K, int E, int bits, bool x_bf16, unsigned se
              " experts, " + std::to_string(bits) + "-bit, " + (x_bf16 ? "bf16" : "fp32") + " positions";
     const int hidden = 2048, inter = 512, n = M * K;
     const Geom g = geom(hidden, inter, bits);
-    // routing: K distinct experts per position, low indices preferred
-    std::vector<int> idx((size_t)n);
-    uint64_t st = 0x9E3779B97F4A7C15ull * (seed + 1);
-    auto rnd = [&]() { st = st * 6364136223846793005ull + 1442695040888963407ull; return (double)(st >> 11) / 9007199254740992.0; };
-    for (int m = 0; m < M; m++)
-        for (int k = 0; k < K; k++) {
-            for (;;) {
-                const double u = rnd();
-                const int e = (int)(E * u * u * u);
-                bool dup = false;
-                for (int j = 0; j < k; j++) dup = dup || idx[(size_t)m * K + j] == e;
-                if (!dup && e < E) { idx[(size_t)m * K + k] = e; break; }
-            }
-        }
-    std::vector<int> cnt(E, 0), off(E + 1, 0);
-    for (int p = 0; p < n; p++) cnt[idx[p]]++;
-    for (int e = 0; e < E; e++) off[e + 1] = off[e] + cnt[e];
-    std::vector<int> sorted((size_t)n), cur(off.begin(), off.end() - 1);
-    for (int p = 0; p < n; p++) sorted[cur[idx[p]]++] = p;
-    struct Item { int expert, start, count; };
+    const ChunkLists cl = chunk_lists(M, K, E, seed);
+    const std::vector<int> &sorted = cl.sorted;
+    typedef ChunkItem Item;
     for (int mode = 0; mode < 2; mode++) {
         const bool gu = mode == 0;
         const int tm = gu ? (x_bf16 ? 16 : 8) : 16;
-        std::vector<Item> items;
-        for (int e = 0; e < E; e++)
-            for (int s0 = 0; s0 < cnt[e]; s0 += tm) items.push_back({e, off[e] + s0, cnt[e] - s0 < tm ? cnt[e] - s0 : tm});
+        const std::vector<Item> items = cl.items(tm);
         const int n_items = (int)items.size();
         CHECK(n_items <= E + n / tm + 1, "%d items in a list of %d", n_items, E + n / tm + 1);
         const int in_dim = gu ? hidden : inter, out_rows = gu ? inter : hidden;
@@ -487,6 +507,93 @@ static void walk_pf_rows(int M, int K, int E, int bits, bool x_bf16, unsigned se
         }
         out.expect_once(0, out.size);
         std::printf("ok  %-58s %s: %d items, %ld rounds over %d workgroups\n", g_case.c_str(), gu ? "gate/up" : "down", n_items, RT, G);
+    }
+}
+
+// fm_gq_gate_up / fm_gq_down (the grouped products of a chunk on a GGUF store, config 4's chunk
+// variant): the kernels' loops restated — a workgroup's share of the (item, eight tiles) units, the
+// staging of an item, a wave's tile, the blocks of its rows and the first block of its next tile
+// requested ahead (which may belong to the next item's expert).  Checked: every block read lies in
+// the expert's slab, every tile of every item is multiplied exactly once, the ahead-requests stay
+// inside the store, outputs are written exactly once, the images fit the LDS the launcher asks for.
+static void walk_gq(int M, int K, int E, int hidden, int inter, unsigned seed) {
+    g_case = "gguf chunk grouped " + std::to_string(M) + " positions x " + std::to_string(K) + " on " + std::to_string(E) +
+             " experts, " + std::to_string(hidden) + "x" + std::to_string(inter);
+    const ChunkLists cl = chunk_lists(M, K, E, seed);
+    const int n = cl.n;
+    for (int mode = 0; mode < 2; mode++) {
+        const bool gu = mode == 0;
+        const int tm = gu ? (hidden <= 2048 ? 16 : 8) : 16;
+        const std::vector<ChunkItem> items = cl.items(tm);
+        const int n_items = (int)items.size();
+        CHECK(n_items <= E + n / tm + 1, "%d items in a list of %d", n_items, E + n / tm + 1);
+        const int in_dim = gu ? hidden : inter, rows = gu ? inter : hidden;
+        const int NB = in_dim / 256, blk = gu ? 144 : 210, NW = 8;
+        const size_t row_bytes = (size_t)NB * blk, slab = (size_t)rows * row_bytes;
+        const int tiles = rows / 16, per_item = (tiles + NW - 1) / NW;
+        const size_t lds = gu ? (size_t)(hidden / 32) * ((tm == 16 ? 2048 : 1024) + 64)
+                              : (size_t)(inter / 16) * 1024 + (size_t)(inter / 256) * 1536;
+        CHECK(lds <= 160 * 1024 - 1024, "LDS %zu", lds);
+        const int G = gu ? N_CU : 2 * N_CU;
+        const long total = (long)n_items * per_item;
+        Region X("X", (size_t)M * hidden * 4), act_in("act", (size_t)n * inter * 4), srt("sorted", (size_t)n * 4);
+        Region out = gu ? Region("act", (size_t)n * inter * 4, 4) : Region("expert_out", (size_t)n * hidden * 4, 4);
+        // per (item, tile): how often it was multiplied
+        std::vector<uint8_t> done((size_t)n_items * tiles, 0);
+        Region store("expert slabs", (size_t)E * slab);       // gate (and, at the same offsets, up) or down
+        auto block = [&](size_t row_off, int b, const char *what) {     // a lane's words of block b of a row
+            store.touch(row_off + (size_t)b * blk, (size_t)blk, what);
+        };
+        for (int bq = 0; bq < G; bq++) {
+            const FmRange sh = fm_share(total, (unsigned)bq, (unsigned)G);
+            int cur_item = -1;
+            ChunkItem item{0, 0, 0}, item_next{0, 0, 0};
+            for (long u = sh.lo; u < sh.hi; u++) {
+                const int it = (int)(u / per_item), part = (int)(u - (long)it * per_item);
+                CHECK(it < n_items, "unit %ld -> item %d of %d", u, it, n_items);
+                if (it >= n_items) break;
+                if (it != cur_item) {
+                    cur_item = it;
+                    item = items[it];
+                    item_next = items[it + 1 < n_items ? it + 1 : it];
+                    for (int p = 0; p < item.count; p++) {
+                        srt.touch((size_t)(item.start + p) * 4, 4, "pair id");
+                        if (gu) X.touch((size_t)(cl.sorted[item.start + p] / K) * hidden * 4, (size_t)hidden * 4, "X row");
+                        else act_in.touch((size_t)(item.start + p) * inter * 4, (size_t)inter * 4, "act row");
+                    }
+                }
+                for (int wave = 0; wave < NW; wave++) {
+                    const int tile = part * NW + wave;
+                    if (tile >= tiles) continue;
+                    done[(size_t)it * tiles + tile]++;
+                    for (int nn = 0; nn < 16; nn++) {
+                        const size_t row_off = ((size_t)item.expert * rows + (size_t)tile * 16 + nn) * row_bytes;
+                        for (int b = 0; b < NB; b++) block(row_off, b, "block of the tile's row");
+                        for (int pos = 0; pos < item.count; pos++) {
+                            if (gu) out.touch(((size_t)(item.start + pos) * inter + (size_t)tile * 16 + nn) * 4, 4, "act");
+                            else out.touch(((size_t)cl.sorted[item.start + pos] * hidden + (size_t)tile * 16 + nn) * 4, 4, "expert_out");
+                        }
+                    }
+                    // the first block of the wave's tile of the next unit, requested ahead
+                    if (u + 1 < sh.hi) {
+                        const int it2 = (int)((u + 1) / per_item), tile2 = (int)(u + 1 - (long)it2 * per_item) * NW + wave;
+                        if (tile2 < tiles) {
+                            CHECK(it2 == cur_item || it2 == cur_item + 1, "next unit's item %d after %d", it2, cur_item);
+                            CHECK(it2 < n_items, "next unit's item %d of %d", it2, n_items);
+                            const int e2 = it2 == cur_item ? item.expert : item_next.expert;
+                            if (it2 < n_items) CHECK(e2 == items[it2].expert, "expert of the item ahead");
+                            for (int nn = 0; nn < 16; nn++)
+                                block(((size_t)e2 * rows + (size_t)tile2 * 16 + nn) * row_bytes, 0, "block requested ahead");
+                        }
+                    }
+                }
+            }
+        }
+        size_t bad = 0;
+        for (uint8_t d : done) bad += d != 1;
+        CHECK(bad == 0, "%zu (item, tile) combinations not multiplied exactly once", bad);
+        out.expect_once(0, out.size);
+        std::printf("ok  %-58s %s: %d items, %ld units over %d workgroups\n", g_case.c_str(), gu ? "gate/up" : "down", n_items, total, G);
     }
 }
 
@@ -983,6 +1090,12 @@ int main() {
     walk_pf_rows(32, 8, 256, 3, true, 5);
     walk_pf_rows(200, 5, 12, 4, false, 6);
     walk_pf_rows(8192, 1, 3, 3, true, 7);
+    // ---- config 4's chunk variant: grouped products on a GGUF store (bench.py --workload gguf_chunk, the tests)
+    walk_gq(512, 8, 256, 2048, 512, 11);
+    walk_gq(64, 8, 256, 2048, 512, 12);
+    walk_gq(97, 4, 12, 1024, 256, 13);
+    walk_gq(36, 4, 12, 4096, 256, 14);
+    walk_gq(2048, 8, 256, 2048, 512, 15);
     // ---- routed experts: the decode step (config 2, and its 4-bit form), one layer per call
     // (config 0), chunks below 32 positions (config 3 at chunk 8)
     for (int bits : {3, 4}) {

@@ -46,7 +46,9 @@ def test_every_access_of_the_benchmark_launches_is_inside_its_buffer(walker):
                  "gguf fused rows Q4_K down, 3 groups x 8, 1024x512",
                  "chunk rows 512 positions x 8 on 256 experts, 3-bit, bf16 positions",
                  "chunk rows 512 positions x 8 on 256 experts, 4-bit, bf16 positions",
-                 "chunk rows 2048 positions x 8 on 256 experts, 3-bit, bf16 positions"):
+                 "chunk rows 2048 positions x 8 on 256 experts, 3-bit, bf16 positions",
+                 "gguf chunk grouped 512 positions x 8 on 256 experts, 2048x512",
+                 "gguf chunk grouped 36 positions x 4 on 12 experts, 4096x256"):
         assert ("ok  " + case) in r.stdout or ("ok  dense " + case) in r.stdout, case
 
 
